@@ -1,0 +1,163 @@
+/*
+ * streamk.h -- C ABI of the MI355X (gfx950) Stream-K GEMM library (libstreamk.so).
+ *
+ * Plain C: pointers, sizes and PODs only.  Device pointers are ordinary HIP device addresses, the
+ * stream argument is a hipStream_t passed as void*.  Every function returns SK_OK (0) or a negative
+ * sk_status; nothing throws, nothing allocates or frees caller memory, all device work is enqueued
+ * on the caller's stream without a host synchronisation.
+ *
+ * Each entry point names the reference interface it replaces (paths relative to the
+ * LeiWang1999/Stream-k.tvm checkout).  In the reference the "operator" is a TVM-TL compiled callable
+ * `tl_mod(A, B, C)` (streamk_fp32.py:197-202) whose shapes, tiles and partition are compile-time
+ * constants; here they are run-time arguments.
+ */
+#ifndef STREAMK_H_
+#define STREAMK_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SK_VERSION 100
+
+typedef enum sk_status {
+  SK_OK = 0,
+  SK_ERR_NULL = -1,        /* a required pointer is NULL */
+  SK_ERR_SHAPE = -2,       /* M, N or K <= 0, or a leading dimension smaller than the row */
+  SK_ERR_ALIGN = -3,       /* pointer / leading dimension / K not aligned as the kernel needs */
+  SK_ERR_CONFIG = -4,      /* tile shape, grid, schedule or fix-up not supported */
+  SK_ERR_WORKSPACE = -5,   /* workspace missing or smaller than sk_workspace_bytes() */
+  SK_ERR_LAUNCH = -6,      /* HIP reported an error at launch */
+  SK_ERR_DEVICE = -7,      /* not a gfx950 device / device query failed */
+  SK_ERR_TIMEOUT = -8      /* a fix-up wait gave up (reported by sk_workspace_status) */
+} sk_status;
+
+/* B operand layout.  NT: B is [N,K] row-major, C = A * B^T (streamk_fp16.py:131-133).
+ *                    NN: B is [K,N] row-major, C = A * B   (streamk_fp32.py:65-76). */
+typedef enum sk_layout { SK_LAYOUT_NT = 0, SK_LAYOUT_NN = 1 } sk_layout;
+
+/* How output tiles are split over the persistent grid. */
+typedef enum sk_schedule {
+  SK_SCHED_AUTO = 0,       /* library heuristic */
+  SK_SCHED_DP = 1,         /* data-parallel only: one CTA per tile, ceil(tiles/grid) waves
+                              (dataparallel.fp16.breakdown/block_level_gemm.py:36-53) */
+  SK_SCHED_SK_TWO_TILE = 2,/* reference hybrid: (tiles % P) + P Stream-K tiles, rest data-parallel
+                              (streamk_fp32.py:37-43) */
+  SK_SCHED_SK_ONE_TILE = 3,/* tiles % P Stream-K tiles, rest data-parallel */
+  SK_SCHED_SK_BASIC = 4    /* every tile is a Stream-K tile (figures/image.png "basic Stream-K") */
+} sk_schedule;
+
+/* How partial tiles of the Stream-K wave are combined. */
+typedef enum sk_fixup {
+  SK_FIXUP_AUTO = 0,
+  SK_FIXUP_ATOMIC = 1,     /* fp32 atomicAdd of partial accumulators (streamk_fp32.py:127-134);
+                              summation order varies run to run */
+  SK_FIXUP_REDUCE = 2      /* per-CTA fp32 partial + flag; the tile's first CTA adds the others in
+                              ascending CTA order: bitwise reproducible */
+} sk_fixup;
+
+typedef enum sk_dtype { SK_F16 = 0, SK_F32 = 1, SK_Q4 = 2 } sk_dtype;
+
+/* Tunables; a zero field means "choose for me".  Replaces the module-level constants and
+ * bitblas Hint of the reference (streamk_fp32.py:24-28, streamk_fp16.py:32-59) and is what the
+ * autotuner enumerates (autotune/streamk_fp16_autotune.py:38-53). */
+typedef struct sk_config {
+  int32_t bm, bn, bk;     /* CTA tile */
+  int32_t grid;           /* persistent CTAs; the reference's total_sm (streamk_fp32.py:17) */
+  int32_t schedule;       /* sk_schedule */
+  int32_t fixup;          /* sk_fixup */
+  int32_t raster;         /* 0: row-major tile order (streamk_fp32.py:106-107); g>0: tiles walk g
+                             rows down before stepping one column (triton_impl.py:14-28) */
+  int32_t spin_limit;     /* REDUCE fix-up: polls of a peer flag before giving up; 0 = default */
+  int32_t reserved[4];
+} sk_config;
+
+/* Result of the host partitioner: the integers of streamk_fp32.py:30-54 for the chosen tile/grid. */
+typedef struct sk_plan {
+  int32_t bm, bn, bk, grid, schedule, fixup, raster, dtype, layout;
+  int32_t num_block_m, num_block_n, iters_per_tile, total_tiles;
+  int32_t streamk_tiles;         /* tile ids [0, streamk_tiles) are split along K */
+  int32_t blocking_tiles;        /* tile ids [streamk_tiles, total_tiles) are data-parallel */
+  int32_t streamk_iters;         /* streamk_tiles * iters_per_tile */
+  int32_t streamk_full_tiles;    /* K-iterations every CTA gets (reference's name kept) */
+  int32_t streamk_partial_tiles; /* the first this-many CTAs get one more */
+  int32_t dp_waves;              /* ceil(blocking_tiles / grid); the reference's
+                                    sm_patition_factor without its max(...,1) */
+  int32_t kernel_id;             /* which compiled kernel instance runs this plan */
+  int32_t threads;               /* workgroup size of that kernel */
+  int32_t lds_bytes;             /* static LDS of that kernel */
+  int64_t workspace_bytes;       /* what sk_gemm_* needs for this plan */
+  int64_t M, N, K;
+} sk_plan;
+
+int sk_version(void);
+const char *sk_strerror(int status);
+
+/* Number of compute units and max co-resident CTAs per CU are read from the current HIP device.
+ * Replaces `total_sm = 108` (streamk_fp32.py:17). */
+int sk_device_info(int *num_cus, int *clock_khz, int *lds_bytes_per_cu);
+
+/*
+ * Host partitioner (pure integer arithmetic, no GPU needed when num_cus > 0 is given).
+ * Replaces streamk_fp32.py:30-54 / streamk_fp16.py:92-113.
+ *   dtype/layout select the kernel family; cfg may be NULL (all heuristic).
+ */
+int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layout, const sk_config *cfg,
+                 int num_cus, sk_plan *out);
+
+/* K-iteration range [start, last) of CTA pid in the Stream-K wave (streamk_fp32.py:93-96). */
+int sk_plan_cta_range(const sk_plan *plan, int pid, int32_t *start, int32_t *last);
+
+/* Tile id -> (pid_m, pid_n) under the plan's raster (streamk_fp32.py:106-107). */
+int sk_plan_tile_coords(const sk_plan *plan, int tile, int32_t *pid_m, int32_t *pid_n);
+
+/* Workspace the plan needs (partials, flags / counters, status word).  0 is possible. */
+size_t sk_workspace_bytes(const sk_plan *plan);
+
+/* Must be run once on a freshly allocated workspace (and after an SK_ERR_TIMEOUT); kernels leave
+ * the workspace clean for the next launch.  Uses a fill kernel, so it may be graph-captured. */
+int sk_workspace_init(void *ws, size_t ws_bytes, void *stream);
+
+/* Reads the workspace status word (synchronises the stream): SK_OK or SK_ERR_TIMEOUT. */
+int sk_workspace_status(void *ws, void *stream);
+
+/*
+ * fp16 GEMM, fp32 accumulate, fp16 out.  C[M,N] (ldc) = A[M,K] (lda) * op(B).
+ * Replaces tl_mod(A, B, C) of streamk_fp16.py:382-387.  C need not be zeroed by the caller
+ * (the reference requires it, streamk_fp16.py:385).
+ * Requirements: K, lda, ldb multiples of 8 and 16-byte aligned A, B (vector loads).
+ */
+int sk_gemm_f16(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws, size_t ws_bytes,
+                void *stream);
+
+/* fp32 GEMM (fp32 MFMA, fp32 out).  Replaces tl_mod(A, B, C) of streamk_fp32.py:197-202. */
+int sk_gemm_f32(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws, size_t ws_bytes,
+                void *stream);
+
+/*
+ * Q4 weight-only GEMM: C[M,N] fp16 = A[M,K] fp16 * dequant(Wq)^T.
+ *   Wq      [N, K/2] bytes, element k of row n = (Wq[n][k/2] >> 4*(k&1)) & 0xF
+ *           (streamk.fp16.breakdown/streamk_fp16_ladder_block_reduce_q4.py:552)
+ *   scales  [N, K/group] fp16, w = fp16_rn((fp16(q) - zero) * scale)
+ * Replaces tl_mod(A, QLB, C) of streamk_fp16_ladder_block_reduce_q4.py:597-599; the weights stay in
+ * the natural byte order above (no LadderPermutate / LOP3Permutate step, :568-595).
+ * Requirements: K multiple of 256, group == 128, 0 <= zero <= 15.
+ */
+int sk_gemm_q4(const void *A, const void *Wq, const void *scales, void *C, int64_t M, int64_t N,
+               int64_t K, int64_t lda, int64_t ldc, int group, int zero, const sk_plan *plan,
+               void *ws, size_t ws_bytes, void *stream);
+
+/* Device dequantisation of Wq into fp16 W[N,K] with the very device function the GEMM uses
+ * (the closed form of streamk_fp16_ladder_block_reduce_q4.py:548-554 plus zero/scale). */
+int sk_dequant_q4(const void *Wq, const void *scales, void *W, int64_t N, int64_t K, int group,
+                  int zero, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* STREAMK_H_ */

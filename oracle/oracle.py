@@ -1,0 +1,188 @@
+"""CPU oracle for the Stream-K GEMM hot path.  TEST INFRASTRUCTURE ONLY.
+
+Two independent statements of the same arithmetic live here so each can pin the other:
+
+* ``liboracle.so`` (``streamk_oracle.c``): plain-C restatement of the reference partitioner, the
+  per-CTA segment loop with both fix-up flavours, and the Q4 dequantisation.
+* numpy / pure-Python twins in this file (``partition_py``, ``cta_segments_py``, ``dequant_q4_np``).
+
+Reference lines followed (relative to the LeiWang1999/Stream-k.tvm checkout):
+  partition       streamk_fp32.py:33-54
+  CTA range       streamk_fp32.py:93-96
+  segment loop    streamk_fp32.py:98-136, triton_impl.py:104-127
+  DP loop         streamk_fp32.py:149-158
+  Q4 order        streamk.fp16.breakdown/streamk_fp16_ladder_block_reduce_q4.py:552
+  host check      streamk_fp32.py:204-208 (dense matmul, rtol = atol = 1e-2)
+
+Nothing here is ever used by the product path; the product raises when its HIP library is missing.
+"""
+import ctypes
+import math
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+
+class _Partition(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int) for n in (
+        "num_block_m", "num_block_n", "iters_per_tile", "total_tiles", "streamk_tiles",
+        "blocking_tiles", "streamk_iters", "streamk_full_tiles", "streamk_partial_tiles",
+        "sm_partition_factor")]
+
+
+def build():
+    """Compile liboracle.so with gcc (a second or two)."""
+    subprocess.check_call(["make", "-s", "-C", _HERE, "liboracle.so"])
+
+
+def lib():
+    global _LIB
+    if _LIB is None:
+        path = os.path.join(_HERE, "liboracle.so")
+        if not os.path.exists(path):
+            build()
+        L = ctypes.CDLL(path)
+        L.ora_partition.argtypes = [ctypes.c_int] * 7 + [ctypes.POINTER(_Partition)]
+        L.ora_partition.restype = None
+        L.ora_cta_range.argtypes = [ctypes.POINTER(_Partition), ctypes.c_int,
+                                    ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]
+        L.ora_cta_range.restype = None
+        L.ora_streamk_gemm_f32.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int] * 8 + [
+            ctypes.c_void_p, ctypes.c_int]
+        L.ora_streamk_gemm_f32.restype = ctypes.c_int
+        L.ora_dequant_q4.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int] * 4
+        L.ora_dequant_q4.restype = None
+        L.ora_half_to_float.argtypes = [ctypes.c_uint16]
+        L.ora_half_to_float.restype = ctypes.c_float
+        L.ora_float_to_half.argtypes = [ctypes.c_float]
+        L.ora_float_to_half.restype = ctypes.c_uint16
+        _LIB = L
+    return _LIB
+
+
+# ------------------------------------------------------------------ partition (C and Python twins)
+def partition(M, N, K, BM, BN, BK, P):
+    """C restatement of streamk_fp32.py:33-54 -> dict."""
+    p = _Partition()
+    lib().ora_partition(M, N, K, BM, BN, BK, P, ctypes.byref(p))
+    return {n: getattr(p, n) for n, _ in _Partition._fields_}
+
+
+def partition_py(M, N, K, BM, BN, BK, P):
+    """Pure-Python twin of streamk_fp32.py:33-54 (factor = blocking_tiles // P, 0 allowed)."""
+    nbm, nbn, ipt = math.ceil(M / BM), math.ceil(N / BN), math.ceil(K / BK)
+    total = nbm * nbn
+    sk = total % P
+    if total - sk > P:
+        sk += P
+    dp = total - sk
+    it = sk * ipt
+    return dict(num_block_m=nbm, num_block_n=nbn, iters_per_tile=ipt, total_tiles=total,
+                streamk_tiles=sk, blocking_tiles=dp, streamk_iters=it, streamk_full_tiles=it // P,
+                streamk_partial_tiles=it % P, sm_partition_factor=dp // P)
+
+
+def cta_range(part, pid):
+    p = _Partition(**part)
+    s, e = ctypes.c_int(), ctypes.c_int()
+    lib().ora_cta_range(ctypes.byref(p), pid, ctypes.byref(s), ctypes.byref(e))
+    return s.value, e.value
+
+
+def cta_segments_py(part, pid):
+    """Segments (tile, k0, n_iters, whole) a CTA walks in its Stream-K wave
+    (streamk_fp32.py:93-136), pure Python."""
+    full, partial, ipt = (part["streamk_full_tiles"], part["streamk_partial_tiles"],
+                          part["iters_per_tile"])
+    start = pid * full + min(pid, partial)
+    last = (pid + 1) * full + min(pid + 1, partial)
+    out = []
+    while start < last:
+        end = min(start + (ipt - start % ipt), last)
+        k0 = start % ipt
+        out.append((start // ipt, k0, end - start, k0 == 0 and end % ipt == 0))
+        start = end
+    return out
+
+
+def dp_tiles_py(part, pid, P):
+    """Tiles of the data-parallel phase for one CTA (streamk_fp32.py:149-150)."""
+    return [pid + part["streamk_tiles"] + p * P for p in range(part["sm_partition_factor"])]
+
+
+# ------------------------------------------------------------------ Stream-K GEMM on the CPU
+def streamk_gemm_f32(A, B, BM, BN, BK, P, trans_b=False, cta_order=None, fixup="atomic"):
+    """Runs the reference's persistent kernel with P simulated CTAs (C restatement).
+    A [M,K] float32; B [K,N] (trans_b False) or [N,K] (trans_b True).  Returns C float32."""
+    A = np.ascontiguousarray(A, dtype=np.float32)
+    B = np.ascontiguousarray(B, dtype=np.float32)
+    M, K = A.shape
+    N = B.shape[0] if trans_b else B.shape[1]
+    assert (B.shape[1] if trans_b else B.shape[0]) == K
+    C = np.zeros((M, N), dtype=np.float32)  # pre-zero contract, streamk_fp32.py:200
+    order = None
+    if cta_order is not None:
+        order = np.ascontiguousarray(cta_order, dtype=np.int32)
+        assert sorted(order.tolist()) == list(range(P))
+    rc = lib().ora_streamk_gemm_f32(A.ctypes.data, B.ctypes.data, C.ctypes.data, M, N, K,
+                                    int(trans_b), BM, BN, BK, P,
+                                    order.ctypes.data if order is not None else None,
+                                    {"atomic": 0, "reduce": 1}[fixup])
+    if rc:
+        raise ValueError("ora_streamk_gemm_f32 rejected its arguments")
+    return C
+
+
+def matmul_fp32(A, B, trans_b=False):
+    """The reference's dense check (streamk_fp32.py:204, streamk_fp16.py:389) on the host in fp32:
+    inputs are widened to float32 first, as block_level_gemm.py:92-103 does."""
+    A = np.asarray(A, dtype=np.float32)
+    B = np.asarray(B, dtype=np.float32)
+    return A @ (B.T if trans_b else B)
+
+
+def max_abs_rel(got, ref):
+    """max |got - ref| / max |ref|  (the 'max-abs-rel' figure quoted for GEMM accuracy)."""
+    got = np.asarray(got, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    return float(np.max(np.abs(got - ref)) / max(float(np.max(np.abs(ref))), 1e-30))
+
+
+# ------------------------------------------------------------------ Q4
+def unpack_q4_np(Wq):
+    """[N, K/2] uint8 -> [N, K] uint8 nibbles; low nibble is the even k
+    (streamk_fp16_ladder_block_reduce_q4.py:552)."""
+    Wq = np.asarray(Wq, dtype=np.uint8)
+    out = np.empty((Wq.shape[0], Wq.shape[1] * 2), dtype=np.uint8)
+    out[:, 0::2] = Wq & 0xF
+    out[:, 1::2] = Wq >> 4
+    return out
+
+
+def dequant_q4_np(Wq, scales, group=128, zero=8):
+    """numpy float16 evaluation: w = fp16((fp16(q) - fp16(zero)) * scale[n, k // group])."""
+    q = unpack_q4_np(Wq).astype(np.float16)
+    d = q - np.float16(zero)
+    s = np.repeat(np.asarray(scales, dtype=np.float16), group, axis=1)[:, :q.shape[1]]
+    return (d * s).astype(np.float16)
+
+
+def dequant_q4(Wq, scales, group=128, zero=8):
+    """C restatement (software binary16 rounding), returns float16 [N, K]."""
+    Wq = np.ascontiguousarray(Wq, dtype=np.uint8)
+    N, K = Wq.shape[0], Wq.shape[1] * 2
+    sc = np.ascontiguousarray(scales, dtype=np.float16)
+    assert sc.shape == (N, math.ceil(K / group)), sc.shape
+    out = np.empty((N, K), dtype=np.float16)
+    lib().ora_dequant_q4(Wq.ctypes.data, sc.ctypes.data, out.ctypes.data, N, K, group, zero)
+    return out
+
+
+def q4_gemm_ref(A, Wq, scales, group=128, zero=8):
+    """fp32 host product of A [M,K] with the dequantised weights [N,K]^T."""
+    W = dequant_q4(Wq, scales, group, zero).astype(np.float32)
+    return np.asarray(A, dtype=np.float32) @ W.T

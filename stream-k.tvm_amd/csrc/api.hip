@@ -1,0 +1,261 @@
+// C ABI of libstreamk.so: argument checking, workspace carving, kernel launch.
+#include <hip/hip_runtime.h>
+
+#include <mutex>
+#include <unordered_map>
+
+#include "launch.h"
+#include "q4_dequant.h"
+#include "streamk.h"
+
+using namespace sk;
+
+namespace {
+
+struct DeviceInfo {
+  int ok = 0, cus = 0, clock_khz = 0, lds = 0;
+};
+DeviceInfo &device_info() {
+  static DeviceInfo d[16];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) { static DeviceInfo bad; return bad; }
+  if (!d[dev].ok) {
+    hipDeviceProp_t p;
+    if (hipGetDeviceProperties(&p, dev) == hipSuccess) {
+      d[dev].cus = p.multiProcessorCount;
+      d[dev].clock_khz = p.clockRate;
+      d[dev].lds = (int)p.maxSharedMemoryPerMultiProcessor;
+      d[dev].ok = 1;
+    }
+  }
+  return d[dev];
+}
+
+__global__ void fill_zero_kernel(uint32_t *p, size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) p[i] = 0;
+}
+
+// What the library knows about the contents of each workspace it has been handed.  Kernels leave
+// flags and counters at zero.  ATOMIC launches also leave the partial area zeroed (and need it
+// zeroed); REDUCE launches leave partial tiles behind.  An ATOMIC launch on a workspace whose partial
+// area is dirty is therefore preceded by a stream-ordered fill of that area.
+enum WsState { WS_CLEAN = 0, WS_PARTIALS_DIRTY = 1 };
+std::mutex g_ws_mutex;
+std::unordered_map<const void *, int> g_ws_state;
+
+int check_plan(const sk_plan *plan, int64_t M, int64_t N, int64_t K, int dtype, int layout) {
+  if (!plan) return SK_ERR_NULL;
+  if (plan->M != M || plan->N != N || plan->K != K || plan->dtype != dtype || plan->layout != layout)
+    return SK_ERR_CONFIG;
+  return SK_OK;
+}
+
+int make_dev_plan(const sk_plan *plan, const KernelInfo *k, void *ws, size_t ws_bytes, int occupancy,
+                  hipStream_t stream, DevPlan *dp, Workspace *w) {
+  if ((size_t)plan->workspace_bytes > ws_bytes) return SK_ERR_WORKSPACE;
+  if (plan->workspace_bytes > 0 && !ws) return SK_ERR_WORKSPACE;
+  if (plan->workspace_bytes > 0 && (reinterpret_cast<uintptr_t>(ws) & 255)) return SK_ERR_ALIGN;
+  DeviceInfo &d = device_info();
+  if (!d.ok) return SK_ERR_DEVICE;
+  // every CTA of the Stream-K wave may wait on another one: they must all be resident
+  if (plan->streamk_tiles > 0 && plan->fixup == SK_FIXUP_REDUCE &&
+      (occupancy <= 0 || plan->grid > d.cus * occupancy))
+    return SK_ERR_CONFIG;
+  if (plan->workspace_bytes > 0) {
+    const size_t part_off = (size_t)WS_PART_OFF;
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    auto it = g_ws_state.find(ws);
+    if (it == g_ws_state.end()) return SK_ERR_WORKSPACE;  // sk_workspace_init was never run on it
+    if (plan->fixup == SK_FIXUP_ATOMIC && it->second == WS_PARTIALS_DIRTY) {
+      const size_t n = (ws_bytes - part_off) / 4;
+      int blocks = (int)((n + 255) / 256);
+      if (blocks > 4096) blocks = 4096;
+      hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(256), 0, stream,
+                         reinterpret_cast<uint32_t *>(static_cast<char *>(ws) + part_off), n);
+      if (hipGetLastError() != hipSuccess) return SK_ERR_LAUNCH;
+      it->second = WS_CLEAN;
+    } else if (plan->fixup == SK_FIXUP_REDUCE) {
+      it->second = WS_PARTIALS_DIRTY;
+    }
+  }
+  dp->tiles_m = plan->num_block_m;
+  dp->tiles_n = plan->num_block_n;
+  dp->ipt = plan->iters_per_tile;
+  dp->total_tiles = plan->total_tiles;
+  dp->sk_tiles = plan->streamk_tiles;
+  dp->sk_full = plan->streamk_full_tiles;
+  dp->sk_extra = plan->streamk_partial_tiles;
+  dp->grid = plan->grid;
+  dp->fixup = plan->fixup == SK_FIXUP_ATOMIC ? FIXUP_ATOMIC : FIXUP_REDUCE;
+  dp->raster = plan->raster;
+  dp->spin_limit = 1 << 22;
+  dp->xcd_remap = (plan->grid % 8 == 0) ? 1 : 0;
+  w->status = nullptr; w->flags = nullptr; w->partials = nullptr;
+  if (plan->workspace_bytes > 0) {
+    char *base = static_cast<char *>(ws);
+    w->status = reinterpret_cast<int *>(base);
+    w->flags = reinterpret_cast<int *>(base + 256);
+    w->partials = reinterpret_cast<float *>(base + WS_PART_OFF);
+  }
+  (void)k;
+  return SK_OK;
+}
+
+int cached_occupancy(int id, bool skinny) {
+  static int cache[256];
+  static bool have[256];
+  int slot = id & 255;
+  if (!have[slot]) {
+    cache[slot] = skinny ? occupancy_skinny(id) : occupancy_tile(id);
+    have[slot] = true;
+  }
+  return cache[slot];
+}
+
+}  // namespace
+
+extern "C" int sk_version(void) { return SK_VERSION; }
+
+extern "C" const char *sk_strerror(int s) {
+  switch (s) {
+    case SK_OK: return "ok";
+    case SK_ERR_NULL: return "null pointer";
+    case SK_ERR_SHAPE: return "bad shape or leading dimension";
+    case SK_ERR_ALIGN: return "misaligned pointer, leading dimension or K";
+    case SK_ERR_CONFIG: return "unsupported tile / grid / schedule / fix-up, or plan does not match the call";
+    case SK_ERR_WORKSPACE: return "workspace missing or too small";
+    case SK_ERR_LAUNCH: return "HIP launch failed";
+    case SK_ERR_DEVICE: return "no usable gfx950 device";
+    case SK_ERR_TIMEOUT: return "fix-up wait timed out; re-initialise the workspace";
+  }
+  return "unknown status";
+}
+
+extern "C" int sk_device_info(int *num_cus, int *clock_khz, int *lds_bytes_per_cu) {
+  DeviceInfo &d = device_info();
+  if (!d.ok) return SK_ERR_DEVICE;
+  if (num_cus) *num_cus = d.cus;
+  if (clock_khz) *clock_khz = d.clock_khz;
+  if (lds_bytes_per_cu) *lds_bytes_per_cu = d.lds;
+  return SK_OK;
+}
+
+extern "C" int sk_workspace_init(void *ws, size_t ws_bytes, void *stream) {
+  if (ws_bytes == 0) return SK_OK;
+  if (!ws) return SK_ERR_NULL;
+  if ((reinterpret_cast<uintptr_t>(ws) & 3) || (ws_bytes & 3)) return SK_ERR_ALIGN;
+  const size_t n = ws_bytes / 4;
+  int blocks = (int)((n + 255) / 256);
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream,
+                     static_cast<uint32_t *>(ws), n);
+  if (hipGetLastError() != hipSuccess) return SK_ERR_LAUNCH;
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
+  g_ws_state[ws] = WS_CLEAN;
+  return SK_OK;
+}
+
+extern "C" int sk_workspace_status(void *ws, void *stream) {
+  if (!ws) return SK_ERR_NULL;
+  int v = 0;
+  if (hipMemcpyAsync(&v, ws, sizeof(int), hipMemcpyDeviceToHost, (hipStream_t)stream) != hipSuccess)
+    return SK_ERR_LAUNCH;
+  if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) return SK_ERR_LAUNCH;
+  return v == 0 ? SK_OK : SK_ERR_TIMEOUT;
+}
+
+extern "C" int sk_gemm_f16(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,
+                           int64_t lda, int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws,
+                           size_t ws_bytes, void *stream) {
+  if (!A || !B || !C) return SK_ERR_NULL;
+  int rc = check_plan(plan, M, N, K, SK_F16, plan ? plan->layout : 0);
+  if (rc) return rc;
+  if (plan->layout != SK_LAYOUT_NT) return SK_ERR_CONFIG;
+  if (lda < K || ldb < K || ldc < N) return SK_ERR_SHAPE;
+  if ((K % 8) || (lda % 8) || (ldb % 8)) return SK_ERR_ALIGN;
+  if ((reinterpret_cast<uintptr_t>(A) & 15) || (reinterpret_cast<uintptr_t>(B) & 15) ||
+      (reinterpret_cast<uintptr_t>(C) & 1))
+    return SK_ERR_ALIGN;
+  const KernelInfo *k = kernel_by_id(plan->kernel_id);
+  if (!k || k->dtype != SK_F16) return SK_ERR_CONFIG;
+  // a tile's rows must be addressable with 32-bit byte offsets
+  if (lda * 2 * k->bm >= (int64_t)1 << 31 || ldb * 2 * k->bn >= (int64_t)1 << 31) return SK_ERR_SHAPE;
+  DevPlan dp;
+  Workspace w;
+  const bool skinny = k->family == FAMILY_SKINNY;
+  rc = make_dev_plan(plan, k, ws, ws_bytes, cached_occupancy(k->id, skinny), (hipStream_t)stream, &dp, &w);
+  if (rc) return rc;
+  int herr;
+  if (skinny) {
+    SkinnyArgs a{(const half_t *)A, B, nullptr, (half_t *)C, (int)M, (int)N, (int)K, lda, ldb, ldc, 0, 0};
+    herr = launch_skinny(k->id, a, dp, w, (hipStream_t)stream);
+  } else {
+    GemmArgs a{(const half_t *)A, (const half_t *)B, (half_t *)C, (int)M, (int)N, (int)K, lda, ldb, ldc};
+    herr = launch_tile_f16(k->id, a, dp, w, (hipStream_t)stream);
+  }
+  return herr == 0 ? SK_OK : SK_ERR_LAUNCH;
+}
+
+extern "C" int sk_gemm_f32(const void *, const void *, void *, int64_t, int64_t, int64_t, int64_t, int64_t,
+                           int64_t, const sk_plan *, void *, size_t, void *) {
+  return SK_ERR_CONFIG;  // fp32 kernels are not built yet
+}
+
+extern "C" int sk_gemm_q4(const void *A, const void *Wq, const void *scales, void *C, int64_t M, int64_t N,
+                          int64_t K, int64_t lda, int64_t ldc, int group, int zero, const sk_plan *plan,
+                          void *ws, size_t ws_bytes, void *stream) {
+  if (!A || !Wq || !scales || !C) return SK_ERR_NULL;
+  int rc = check_plan(plan, M, N, K, SK_Q4, SK_LAYOUT_NT);
+  if (rc) return rc;
+  if (group != 128 || zero < 0 || zero > 15) return SK_ERR_CONFIG;
+  if (lda < K || ldc < N) return SK_ERR_SHAPE;
+  if ((K % 128) || (lda % 8)) return SK_ERR_ALIGN;
+  if ((reinterpret_cast<uintptr_t>(A) & 15) || (reinterpret_cast<uintptr_t>(Wq) & 15) ||
+      (reinterpret_cast<uintptr_t>(scales) & 1) || (reinterpret_cast<uintptr_t>(C) & 1))
+    return SK_ERR_ALIGN;
+  const KernelInfo *k = kernel_by_id(plan->kernel_id);
+  if (!k || k->dtype != SK_Q4 || k->family != FAMILY_SKINNY) return SK_ERR_CONFIG;
+  if (lda * 2 * k->bm >= (int64_t)1 << 31 || (K / 2) * k->bn >= (int64_t)1 << 31) return SK_ERR_SHAPE;
+  DevPlan dp;
+  Workspace w;
+  rc = make_dev_plan(plan, k, ws, ws_bytes, cached_occupancy(k->id, true), (hipStream_t)stream, &dp, &w);
+  if (rc) return rc;
+  SkinnyArgs a{(const half_t *)A, Wq, (const half_t *)scales, (half_t *)C, (int)M, (int)N, (int)K,
+               lda, K / 2, ldc, zero, (int)(K / group)};
+  int herr = launch_skinny(k->id, a, dp, w, (hipStream_t)stream);
+  return herr == 0 ? SK_OK : SK_ERR_LAUNCH;
+}
+
+namespace {
+// one thread per 32-bit word of packed nibbles: 8 weights, written in natural element order
+__global__ void dequant_q4_kernel(const uint32_t *wq, const half_t *scales, half_t *out, int64_t words,
+                                  int words_per_row, int groups, int group, int zero) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= words) return;
+  const int64_t row = i / words_per_row;
+  const int k = (int)(i % words_per_row) * 8;
+  const half_t s = scales[row * groups + k / group];
+  const half8v v = dequant_word_q4(wq[i], q4_bias(zero), half2v{s, s});
+  half8v o;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = v[q4_slot_of_element(e)];
+  *reinterpret_cast<half8v *>(out + i * 8) = o;
+}
+}  // namespace
+
+extern "C" int sk_dequant_q4(const void *Wq, const void *scales, void *W, int64_t N, int64_t K, int group,
+                             int zero, void *stream) {
+  if (!Wq || !scales || !W) return SK_ERR_NULL;
+  if (N <= 0 || K <= 0) return SK_ERR_SHAPE;
+  if (group <= 0 || (group % 8) || (K % group) || zero < 0 || zero > 15) return SK_ERR_CONFIG;
+  if ((reinterpret_cast<uintptr_t>(Wq) & 3) || (reinterpret_cast<uintptr_t>(W) & 15)) return SK_ERR_ALIGN;
+  const int64_t words = N * K / 8;
+  const int64_t blocks = (words + 255) / 256;
+  if (blocks > 0x7fffffff) return SK_ERR_SHAPE;
+  hipLaunchKernelGGL(dequant_q4_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                     (const uint32_t *)Wq, (const half_t *)scales, (half_t *)W, words, (int)(K / 8),
+                     (int)(K / group), group, zero);
+  return hipGetLastError() == hipSuccess ? SK_OK : SK_ERR_LAUNCH;
+}

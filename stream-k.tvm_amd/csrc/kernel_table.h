@@ -1,0 +1,60 @@
+// Registry of compiled kernel instances.  The host partitioner picks one by (dtype, layout, tile);
+// the launchers switch on its id.
+#pragma once
+#include <stddef.h>
+#include <stdint.h>
+
+namespace sk {
+
+// Workspace layout (bytes): [0,256) status word; [256, 256+WS_FLAG_BYTES) flags (REDUCE: one per
+// CTA) or arrival counters (ATOMIC: one per Stream-K tile); then the fp32 partial tiles.  The flag
+// area has a fixed size so that partial tiles of one plan never land where another plan keeps
+// its flags.
+constexpr int64_t WS_FLAG_BYTES = 262144;
+constexpr int64_t WS_PART_OFF = 256 + WS_FLAG_BYTES;
+constexpr int64_t WS_MAX_FLAGS = WS_FLAG_BYTES / 4;
+
+enum Family { FAMILY_TILE = 0, FAMILY_SKINNY = 1 };
+
+struct KernelInfo {
+  int id;
+  int family;
+  int dtype;    // sk_dtype
+  int layout;   // sk_layout
+  int bm, bn, bk;  // CTA tile; bk is the K extent of one CTA iteration
+  int threads;
+  int lds_bytes;
+  int ctas_per_cu;    // co-resident CTAs per CU the kernel is compiled for
+  int partial_elems;  // fp32 elements of one partial tile in the workspace
+  int max_ipt;        // largest iterations-per-tile the kernel supports (0 = unlimited)
+  int k_align;        // K must be a multiple of this
+  const char *name;
+};
+
+// fp16 LDS-tiled kernels, NT layout:  X(id, BM, BN, BK, WM, WN)
+#define SK_TILE_F16_NT_KERNELS(X) \
+  X(0, 256, 256, 64, 2, 4)        \
+  X(1, 128, 128, 64, 2, 2)        \
+  X(2, 128, 256, 64, 2, 4)        \
+  X(3, 256, 128, 64, 4, 2)        \
+  X(4, 64, 64, 64, 2, 2)          \
+  X(5, 256, 256, 32, 2, 4)        \
+  X(6, 128, 128, 32, 2, 2)
+
+// small-M kernels:  X(id, MB, NB, WN, RK, Q4, DEPTH)
+#define SK_SKINNY_KERNELS(X)  \
+  X(100, 1, 1, 4, 1, 0, 2)    \
+  X(101, 2, 1, 4, 1, 0, 2)    \
+  X(102, 4, 1, 4, 1, 0, 2)    \
+  X(103, 1, 1, 1, 4, 0, 2)    \
+  X(104, 1, 1, 2, 2, 0, 2)    \
+  X(120, 1, 1, 4, 1, 1, 4)    \
+  X(121, 2, 1, 4, 1, 1, 2)    \
+  X(122, 4, 1, 4, 1, 1, 2)    \
+  X(123, 1, 1, 1, 4, 1, 4)    \
+  X(124, 1, 1, 2, 2, 1, 4)
+
+const KernelInfo *kernel_table(int *count);
+const KernelInfo *kernel_by_id(int id);
+
+}  // namespace sk

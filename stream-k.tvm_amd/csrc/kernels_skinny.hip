@@ -1,0 +1,60 @@
+// Small-M Stream-K kernels, fp16 and Q4 weights (gfx950).
+#include "launch.h"
+#include "sk_persistent.h"
+
+namespace sk {
+
+template <class P>
+__global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_skinny_kernel(typename P::Args a, DevPlan plan, Workspace ws) {
+  __shared__ __attribute__((aligned(16))) char smem[P::LDS_BYTES];
+  run_persistent<P>(a, plan, ws, smem);
+}
+
+#define SK_POLICY(MB, NB, WN, RK, Q4, DEPTH) TileSkinny<MB, NB, WN, RK, (Q4) != 0, DEPTH>
+
+int skinny_kernel_infos(KernelInfo *out, int max) {
+  int n = 0;
+#define X(id, MB, NB, WN, RK, Q4, DEPTH)                                                           \
+  if (n < max) {                                                                                   \
+    typedef SK_POLICY(MB, NB, WN, RK, Q4, DEPTH) P;                                                \
+    out[n++] = KernelInfo{id, FAMILY_SKINNY, (Q4) ? 2 : 0, 0, P::BM, P::BN, P::BKC, P::NT,         \
+                          P::LDS_BYTES, P::CTAS_PER_CU, P::TILE_ELEMS, (Q4) ? P::SC_MAX_ITERS : 0, (Q4) ? 128 : 8, \
+                          (Q4) ? "skinny_q4_mb" #MB "_wn" #WN "_rk" #RK                            \
+                               : "skinny_f16_mb" #MB "_wn" #WN "_rk" #RK};                         \
+  }
+  SK_SKINNY_KERNELS(X)
+#undef X
+  return n;
+}
+
+int launch_skinny(int id, const SkinnyArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s) {
+  switch (id) {
+#define X(id_, MB, NB, WN, RK, Q4, DEPTH)                                                  \
+  case id_: {                                                                              \
+    typedef SK_POLICY(MB, NB, WN, RK, Q4, DEPTH) P;                                        \
+    hipLaunchKernelGGL(sk_skinny_kernel<P>, dim3(p.grid), dim3(P::NT), 0, s, a, p, ws);    \
+    return (int)hipGetLastError();                                                         \
+  }
+    SK_SKINNY_KERNELS(X)
+#undef X
+  }
+  return (int)hipErrorInvalidValue;
+}
+
+int occupancy_skinny(int id) {
+  int occ = 0;
+  switch (id) {
+#define X(id_, MB, NB, WN, RK, Q4, DEPTH)                                                             \
+  case id_: {                                                                                         \
+    typedef SK_POLICY(MB, NB, WN, RK, Q4, DEPTH) P;                                                   \
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_skinny_kernel<P>, P::NT, 0) != hipSuccess) \
+      return -1;                                                                                      \
+    return occ;                                                                                       \
+  }
+    SK_SKINNY_KERNELS(X)
+#undef X
+  }
+  return -1;
+}
+
+}  // namespace sk

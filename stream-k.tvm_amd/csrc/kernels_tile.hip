@@ -1,0 +1,58 @@
+// fp16 LDS-tiled Stream-K kernels (gfx950).
+#include "launch.h"
+#include "sk_persistent.h"
+
+namespace sk {
+
+template <class P>
+__global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_tile_kernel(typename P::Args a, DevPlan plan, Workspace ws) {
+  __shared__ __attribute__((aligned(16))) char smem[P::LDS_BYTES];
+  run_persistent<P>(a, plan, ws, smem);
+}
+
+#define SK_POLICY(id, BM, BN, BK, WM, WN) TileF16NT<BM, BN, BK, WM, WN>
+
+int tile_kernel_infos(KernelInfo *out, int max) {
+  int n = 0;
+#define X(id, BM, BN, BK, WM, WN)                                                                   \
+  if (n < max) {                                                                                    \
+    typedef SK_POLICY(id, BM, BN, BK, WM, WN) P;                                                    \
+    out[n++] = KernelInfo{id, FAMILY_TILE, 0, 0, BM, BN, BK, P::NT, P::LDS_BYTES, P::CTAS_PER_CU, P::TILE_ELEMS, 0, 8, \
+                          "tile_f16_nt_" #BM "x" #BN "x" #BK};                                      \
+  }
+  SK_TILE_F16_NT_KERNELS(X)
+#undef X
+  return n;
+}
+
+int launch_tile_f16(int id, const GemmArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s) {
+  switch (id) {
+#define X(id_, BM, BN, BK, WM, WN)                                                       \
+  case id_: {                                                                            \
+    typedef SK_POLICY(id_, BM, BN, BK, WM, WN) P;                                        \
+    hipLaunchKernelGGL(sk_tile_kernel<P>, dim3(p.grid), dim3(P::NT), 0, s, a, p, ws);    \
+    return (int)hipGetLastError();                                                       \
+  }
+    SK_TILE_F16_NT_KERNELS(X)
+#undef X
+  }
+  return (int)hipErrorInvalidValue;
+}
+
+int occupancy_tile(int id) {
+  int occ = 0;
+  switch (id) {
+#define X(id_, BM, BN, BK, WM, WN)                                                                  \
+  case id_: {                                                                                       \
+    typedef SK_POLICY(id_, BM, BN, BK, WM, WN) P;                                                   \
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_tile_kernel<P>, P::NT, 0) != hipSuccess) \
+      return -1;                                                                                    \
+    return occ;                                                                                     \
+  }
+    SK_TILE_F16_NT_KERNELS(X)
+#undef X
+  }
+  return -1;
+}
+
+}  // namespace sk

@@ -1,0 +1,21 @@
+// Internal launch interface between the C ABI and the kernel translation units.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "kernel_table.h"
+#include "sk_device.h"
+#include "tile_f16.h"
+#include "tile_skinny.h"
+
+namespace sk {
+
+int tile_kernel_infos(KernelInfo *out, int max);
+int skinny_kernel_infos(KernelInfo *out, int max);
+
+// return hipError_t as int; occupancy_* return co-resident CTAs per CU (<= 0 on error)
+int launch_tile_f16(int id, const GemmArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s);
+int launch_skinny(int id, const SkinnyArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s);
+int occupancy_tile(int id);
+int occupancy_skinny(int id);
+
+}  // namespace sk

@@ -1,0 +1,185 @@
+// Host-side Stream-K partitioner and kernel selection (pure integer code, no device access).
+//
+// The arithmetic restates streamk_fp32.py:30-54 of the reference for run-time shapes, with two
+// changes: the persistent grid is a parameter instead of `total_sm = 108`, and the number of
+// data-parallel waves is ceil(blocking_tiles / grid) with 0 allowed (the reference's
+// max(blocking_tiles // total_sm, 1) walks out of range when there are no data-parallel tiles).
+#include <string.h>
+
+#include "kernel_table.h"
+#include "streamk.h"
+
+namespace sk {
+
+static KernelInfo g_table[64];
+static int g_count = -1;
+
+int tile_kernel_infos(KernelInfo *out, int max);
+int skinny_kernel_infos(KernelInfo *out, int max);
+
+const KernelInfo *kernel_table(int *count) {
+  if (g_count < 0) {
+    int n = tile_kernel_infos(g_table, 64);
+    n += skinny_kernel_infos(g_table + n, 64 - n);
+    g_count = n;
+  }
+  if (count) *count = g_count;
+  return g_table;
+}
+
+const KernelInfo *kernel_by_id(int id) {
+  int n;
+  const KernelInfo *t = kernel_table(&n);
+  for (int i = 0; i < n; ++i)
+    if (t[i].id == id) return &t[i];
+  return nullptr;
+}
+
+static int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype, int layout,
+                                     const sk_config *cfg, int num_cus) {
+  int n;
+  const KernelInfo *t = kernel_table(&n);
+  const bool want_tile = cfg && cfg->bm > 0 && cfg->bn > 0;
+  if (want_tile) {
+    for (int i = 0; i < n; ++i)
+      if (t[i].dtype == dtype && t[i].layout == layout && t[i].bm == cfg->bm && t[i].bn == cfg->bn &&
+          (cfg->bk <= 0 || t[i].bk == cfg->bk))
+        return &t[i];
+    return nullptr;
+  }
+  // heuristic: small M -> weight-streaming kernels; otherwise the largest tile that still gives
+  // every CU something to do
+  const KernelInfo *best = nullptr;
+  if (M <= 64 || dtype == SK_Q4) {
+    int mb = M <= 16 ? 16 : (M <= 32 ? 32 : 64);
+    for (int i = 0; i < n; ++i)
+      if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].bm == mb && t[i].bn == 64) {
+        best = &t[i];
+        break;
+      }
+    if (best) return best;
+    if (dtype == SK_Q4) return nullptr;
+  }
+  static const int pref[][3] = {{256, 256, 64}, {128, 128, 64}, {64, 64, 64}};
+  for (auto &p : pref) {
+    for (int i = 0; i < n; ++i) {
+      if (t[i].family != FAMILY_TILE || t[i].dtype != dtype || t[i].layout != layout) continue;
+      if (t[i].bm != p[0] || t[i].bn != p[1] || t[i].bk != p[2]) continue;
+      int64_t tiles = cdiv(M, p[0]) * cdiv(N, p[1]);
+      int64_t iters = tiles * cdiv(K, p[2]);
+      // enough K-iterations per CU that a split tile still amortises its fix-up
+      if (best == nullptr && (tiles >= num_cus || iters >= (int64_t)num_cus * 16 || p[0] == 64)) best = &t[i];
+    }
+    if (best) break;
+  }
+  return best;
+}
+
+}  // namespace sk
+
+using namespace sk;
+
+extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layout, const sk_config *cfg,
+                            int num_cus, sk_plan *out) {
+  if (!out) return SK_ERR_NULL;
+  if (M <= 0 || N <= 0 || K <= 0 || M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return SK_ERR_SHAPE;
+  if (dtype != SK_F16 && dtype != SK_F32 && dtype != SK_Q4) return SK_ERR_CONFIG;
+  if (layout != SK_LAYOUT_NT && layout != SK_LAYOUT_NN) return SK_ERR_CONFIG;
+  if (num_cus <= 0) return SK_ERR_DEVICE;
+  const KernelInfo *k = pick_kernel(M, N, K, dtype, layout, cfg, num_cus);
+  if (!k) return SK_ERR_CONFIG;
+  if (K % k->k_align != 0) return SK_ERR_ALIGN;
+
+  memset(out, 0, sizeof(*out));
+  out->M = M; out->N = N; out->K = K;
+  out->dtype = dtype; out->layout = layout;
+  out->bm = k->bm; out->bn = k->bn; out->bk = k->bk;
+  out->kernel_id = k->id; out->threads = k->threads; out->lds_bytes = k->lds_bytes;
+  out->num_block_m = (int32_t)cdiv(M, k->bm);
+  out->num_block_n = (int32_t)cdiv(N, k->bn);
+  out->iters_per_tile = (int32_t)cdiv(K, k->bk);
+  if (k->max_ipt > 0 && out->iters_per_tile > k->max_ipt) return SK_ERR_CONFIG;
+  const int64_t total64 = (int64_t)out->num_block_m * out->num_block_n;
+  if (total64 * out->iters_per_tile > 0x7fffffff) return SK_ERR_SHAPE;
+  const int total = (int)total64;
+  out->total_tiles = total;
+
+  // every CTA of the Stream-K wave may wait for another one, so the grid is capped at what the
+  // device keeps resident; a small problem gets a smaller grid (at least 4 K-iterations per CTA)
+  const int occ = k->ctas_per_cu;
+  int grid = cfg && cfg->grid > 0 ? cfg->grid : num_cus * occ;
+  if (grid > num_cus * occ) return SK_ERR_CONFIG;
+  if (!(cfg && cfg->grid > 0)) {
+    const int64_t iters = total64 * out->iters_per_tile;
+    if (iters / 4 < grid) grid = (int)(iters / 4 > 8 ? (iters / 4) / 8 * 8 : (iters < 8 ? iters : 8));
+  }
+  int sched = cfg ? cfg->schedule : SK_SCHED_AUTO;
+  if (sched == SK_SCHED_AUTO) sched = (total % grid == 0) ? SK_SCHED_DP : SK_SCHED_SK_TWO_TILE;
+  // the grid never exceeds the work: with fewer K-iterations than CTAs the tail CTAs would idle
+  int sk_tiles;
+  switch (sched) {
+    case SK_SCHED_DP: sk_tiles = 0; break;
+    case SK_SCHED_SK_TWO_TILE:  // streamk_fp32.py:37-43
+      sk_tiles = total % grid;
+      if (total - sk_tiles > grid) sk_tiles += grid;
+      break;
+    case SK_SCHED_SK_ONE_TILE: sk_tiles = total % grid; break;
+    case SK_SCHED_SK_BASIC: sk_tiles = total; break;
+    default: return SK_ERR_CONFIG;
+  }
+  out->schedule = sched;
+  out->grid = grid;
+  out->streamk_tiles = sk_tiles;
+  out->blocking_tiles = total - sk_tiles;
+  out->streamk_iters = sk_tiles * out->iters_per_tile;
+  out->streamk_full_tiles = out->streamk_iters / grid;
+  out->streamk_partial_tiles = out->streamk_iters % grid;
+  out->dp_waves = (int32_t)cdiv(out->blocking_tiles, grid);
+  int fixup = cfg ? cfg->fixup : SK_FIXUP_AUTO;
+  if (fixup == SK_FIXUP_AUTO) fixup = SK_FIXUP_REDUCE;
+  if (fixup != SK_FIXUP_ATOMIC && fixup != SK_FIXUP_REDUCE) return SK_ERR_CONFIG;
+  out->fixup = fixup;
+  out->raster = cfg ? cfg->raster : 0;
+  if (out->raster < 0) return SK_ERR_CONFIG;
+
+  // workspace: status block, fixed-size flag area, fp32 partial tiles
+  int64_t ws = 0;
+  if (sk_tiles > 0) {
+    const int64_t nflags = fixup == SK_FIXUP_REDUCE ? grid : sk_tiles;
+    if (nflags > WS_MAX_FLAGS) return SK_ERR_CONFIG;
+    ws = WS_PART_OFF + nflags * (int64_t)k->partial_elems * 4;
+  }
+  out->workspace_bytes = ws;
+  return SK_OK;
+}
+
+extern "C" int sk_plan_cta_range(const sk_plan *p, int pid, int32_t *start, int32_t *last) {
+  if (!p || !start || !last) return SK_ERR_NULL;
+  if (pid < 0 || pid >= p->grid) return SK_ERR_CONFIG;
+  const int full = p->streamk_full_tiles, part = p->streamk_partial_tiles;
+  *start = pid * full + (pid < part ? pid : part);              // streamk_fp32.py:93
+  *last = (pid + 1) * full + (pid + 1 < part ? pid + 1 : part);  // streamk_fp32.py:94-96
+  return SK_OK;
+}
+
+extern "C" int sk_plan_tile_coords(const sk_plan *p, int tile, int32_t *pid_m, int32_t *pid_n) {
+  if (!p || !pid_m || !pid_n) return SK_ERR_NULL;
+  if (tile < 0 || tile >= p->total_tiles) return SK_ERR_CONFIG;
+  if (p->raster <= 0) {  // streamk_fp32.py:106-107
+    *pid_m = tile / p->num_block_n;
+    *pid_n = tile % p->num_block_n;
+  } else {  // triton_impl.py:14-28
+    const int width = p->raster * p->num_block_n;
+    const int group = tile / width;
+    const int first_m = group * p->raster;
+    const int gsize = p->num_block_m - first_m < p->raster ? p->num_block_m - first_m : p->raster;
+    const int r = tile - group * width;
+    *pid_m = first_m + r % gsize;
+    *pid_n = r / gsize;
+  }
+  return SK_OK;
+}
+
+extern "C" size_t sk_workspace_bytes(const sk_plan *p) { return p ? (size_t)p->workspace_bytes : 0; }

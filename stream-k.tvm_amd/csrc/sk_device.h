@@ -1,0 +1,121 @@
+// Device-side pieces shared by every Stream-K kernel: the plan as the kernels see it, the
+// CTA -> work mapping, and the two partial-tile fix-ups.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace sk {
+
+typedef _Float16 half_t;
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+typedef _Float16 half8v __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+
+enum { FIXUP_ATOMIC = 1, FIXUP_REDUCE = 2 };
+
+struct DevPlan {
+  int tiles_m, tiles_n, ipt;  // tile grid, K-iterations per tile
+  int total_tiles, sk_tiles;  // Stream-K tiles are ids [0, sk_tiles)
+  int sk_full, sk_extra;      // iterations per CTA / CTAs that get one more
+  int grid;                   // persistent CTAs
+  int fixup;                  // FIXUP_ATOMIC or FIXUP_REDUCE
+  int raster;                 // 0 row-major, g > 0 grouped by g tile rows
+  int spin_limit;             // polls before a waiting owner gives up
+  int xcd_remap;              // 1: spread logical CTA ids so each XCD owns a contiguous range
+};
+
+struct Workspace {
+  int *status;
+  int *flags;
+  float *partials;
+};
+
+// Workgroups are dealt round-robin to the 8 XCDs (each with its own L2).  Giving XCD x the logical
+// ids [x*grid/8, (x+1)*grid/8) makes neighbouring tiles share an L2.
+__device__ __forceinline__ int logical_pid(const DevPlan &p) {
+  int b = blockIdx.x;
+  if (p.xcd_remap) return (b & 7) * (p.grid >> 3) + (b >> 3);
+  return b;
+}
+
+__device__ __forceinline__ void sk_range(const DevPlan &p, int pid, int &start, int &last) {
+  start = pid * p.sk_full + min(pid, p.sk_extra);
+  last = (pid + 1) * p.sk_full + min(pid + 1, p.sk_extra);
+}
+
+__device__ __forceinline__ void tile_coords(const DevPlan &p, int tile, int &pm, int &pn) {
+  if (p.raster <= 0) {
+    pm = tile / p.tiles_n;
+    pn = tile - pm * p.tiles_n;
+  } else {
+    int width = p.raster * p.tiles_n;
+    int group = tile / width;
+    int first_m = group * p.raster;
+    int gsize = min(p.raster, p.tiles_m - first_m);
+    int r = tile - group * width;
+    pm = first_m + r % gsize;
+    pn = r / gsize;
+  }
+}
+
+// ---- REDUCE fix-up: flags ----
+// Contributor: all of the CTA's partial stores are made visible device-wide, then one thread
+// raises the flag.
+__device__ __forceinline__ void signal_partial_ready(int *flag) {
+  __threadfence();
+  __syncthreads();
+  if (threadIdx.x == 0) __hip_atomic_store(flag, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Owner: thread 0 polls, everybody then acquires.  Returns false if the poll limit ran out.
+__device__ __forceinline__ bool wait_partial_ready(int *flag, int spin_limit, int *lds_ok) {
+  if (threadIdx.x == 0) {
+    int ok = 0;
+    for (int i = 0; i < spin_limit; ++i) {
+      if (__hip_atomic_load(flag, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) != 0) { ok = 1; break; }
+      __builtin_amdgcn_s_sleep(2);
+    }
+    *lds_ok = ok;
+  }
+  __syncthreads();
+  bool ok = *lds_ok != 0;
+  __atomic_thread_fence(__ATOMIC_ACQUIRE);  // device scope is the default for HIP
+  return ok;
+}
+
+__device__ __forceinline__ void clear_flag_after_use(int *flag) {
+  __syncthreads();
+  if (threadIdx.x == 0) __hip_atomic_store(flag, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// ---- buffer addressing ----
+// A 128-bit buffer descriptor gives hardware range checking: a load whose byte offset is at or past
+// num_bytes returns zeros.  Tiles hanging over the matrix edge need no predication, and a K tail
+// is masked by pushing the per-lane offset out of range.
+typedef __amdgpu_buffer_rsrc_t BufferRsrc;
+__device__ __forceinline__ BufferRsrc make_rsrc(const void *base, uint32_t num_bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)num_bytes, 0x00020000);
+}
+__device__ __forceinline__ uint4v buffer_load_16(BufferRsrc r, uint32_t lane_off, uint32_t uniform_off) {
+  return __builtin_bit_cast(uint4v, __builtin_amdgcn_raw_buffer_load_b128(r, lane_off, uniform_off, 0));
+}
+constexpr uint32_t OOB_OFFSET = 0x80000000u;
+
+// Makes a pointer opaque to the optimiser at this program point.  The fix-up paths address dozens
+// of far-apart float4 slots per thread; without this the address arithmetic is hoisted out of the
+// persistent loop and kept in registers across the MFMA main loop.
+template <class T>
+__device__ __forceinline__ T *pin_here(T *p) {
+  asm volatile("" : "+v"(p));
+  return p;
+}
+
+__device__ __forceinline__ void atomic_add_f32(float *p, float v) {
+  // hardware global_atomic_add_f32, no return value, device scope
+  __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+}  // namespace sk

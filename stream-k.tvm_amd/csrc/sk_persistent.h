@@ -1,0 +1,100 @@
+// The persistent Stream-K + data-parallel loop every kernel family shares.
+//
+// A policy class P supplies the tile arithmetic:
+//   P::Args, P::Acc, P::TILE_ELEMS, P::NT
+//   P::mac(args, acc, pm, pn, k0, n, smem)      accumulate K-iterations [k0, k0+n) of tile (pm,pn)
+//   P::store_c(args, acc, pm, pn, smem)         write the finished tile to C
+//   P::store_partial / add_partial / atomic_partial / take_partial   fp32 partials in workspace
+//
+// Control flow follows the reference's persistent kernel: every CTA first walks its share of the
+// Stream-K iteration space (streamk_fp32.py:93-136), then its data-parallel tiles (:149-158).
+#pragma once
+#include "sk_device.h"
+
+namespace sk {
+
+template <class P>
+__device__ __forceinline__ void run_persistent(const typename P::Args &a, const DevPlan &plan,
+                                               const Workspace &ws, char *smem) {
+  __shared__ int s_word;
+  const int pid = logical_pid(plan);
+  const int ipt = plan.ipt;
+  typename P::Acc acc;
+
+  int start, last;
+  sk_range(plan, pid, start, last);
+  int dp_tile = plan.sk_tiles + pid;
+
+  // One loop body serves both phases so that the MAC loop and the epilogue exist once in the
+  // kernel: first the CTA's Stream-K segments, then its data-parallel tiles
+  // (tile = streamk_tiles + pid + wave * grid, streamk_fp32.py:149-158).
+  for (;;) {
+    int tile, k0, n;
+    if (start < last) {
+      tile = start / ipt;
+      k0 = start - tile * ipt;
+      n = min(ipt - k0, last - start);
+      start += n;
+    } else if (dp_tile < plan.total_tiles) {
+      tile = dp_tile;
+      k0 = 0;
+      n = ipt;
+      dp_tile += plan.grid;
+    } else {
+      break;
+    }
+    int pm, pn;
+    tile_coords(plan, tile, pm, pn);
+    P::mac(a, acc, pm, pn, k0, n, smem);
+
+    // a segment that is the whole tile is simply stored (streamk_fp32.py:128-129)
+    bool store = (n == ipt);
+    if (!store) {
+      if (plan.fixup == FIXUP_ATOMIC) {
+        // fp32 atomicAdd into the tile's accumulation buffer; whoever completes the K range
+        // converts and stores, then leaves buffer and counter zeroed for the next launch.
+        float *part = ws.partials + (size_t)tile * P::TILE_ELEMS;
+        P::atomic_partial(acc, part);
+        __threadfence();
+        __syncthreads();
+        if (threadIdx.x == 0) {
+          int old = __hip_atomic_fetch_add(&ws.flags[tile], n, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+          s_word = (old + n == ipt);
+        }
+        __syncthreads();
+        store = s_word != 0;
+        __syncthreads();
+        if (store) {
+          __atomic_thread_fence(__ATOMIC_ACQUIRE);
+          P::take_partial(acc, part);
+          if (threadIdx.x == 0)
+            __hip_atomic_store(&ws.flags[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      } else if (k0 != 0) {
+        // not the tile's first CTA: park the partial in this CTA's slot and raise its flag
+        P::store_partial(acc, ws.partials + (size_t)pid * P::TILE_ELEMS);
+        signal_partial_ready(&ws.flags[pid]);
+      } else {
+        // tile's first CTA: add the followers' partials in ascending CTA order, then store
+        const int tile_end = (tile + 1) * ipt;
+        int pos = last, p = pid + 1;
+        while (pos < tile_end) {
+          if (!wait_partial_ready(&ws.flags[p], plan.spin_limit, &s_word)) {
+            if (threadIdx.x == 0) *ws.status = -8;  // SK_ERR_TIMEOUT
+            break;
+          }
+          P::add_partial(acc, ws.partials + (size_t)p * P::TILE_ELEMS);
+          clear_flag_after_use(&ws.flags[p]);
+          int ps, pl;
+          sk_range(plan, p, ps, pl);
+          pos = pl;
+          ++p;
+        }
+        store = true;
+      }
+    }
+    if (store) P::store_c(a, acc, pm, pn, smem);
+  }
+}
+
+}  // namespace sk

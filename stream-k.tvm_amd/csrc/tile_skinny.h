@@ -1,0 +1,311 @@
+// Small-M ("skinny") tile arithmetic, fp16 and Q4 weights: M <= 64, the weight matrix streams from
+// HBM exactly once and never touches LDS.
+//
+// CTA tile: BM = 16*MB rows of A  x  BN = 16*NB*WN rows of W  x  BKC = RK*BK of K per iteration.
+// Waves are arranged WN (along N) x RK (along K): wave (wn, rk) multiplies its NB 16-row weight
+// blocks with the K sub-block rk of the iteration; the RK partial accumulators are summed through
+// LDS when the segment ends.  RK is the reference's intra-CTA K split ("block reduction",
+// streamk_fp16_block_reduce.py:45,235-306).
+//
+// Per v_mfma_f32_16x16x32_f16 a lane (row = lane%16, g = lane/16) supplies 8 K-values.  Which 8 is
+// free as long as both operands agree, so lane group g owns the contiguous K range
+// [g*KL, (g+1)*KL) of the wave's BK block (KL = BK/4): weights are loaded straight from global
+// memory as 16-byte pieces of one row, and the A tile is read from LDS at the same K offsets.
+// For Q4, A is written to LDS in the element order the nibble decode produces (0,4,1,5,2,6,3,7).
+#pragma once
+#include "q4_dequant.h"
+#include "sk_device.h"
+
+namespace sk {
+
+struct SkinnyArgs {
+  const half_t *A;
+  const void *W;          // fp16 [N,K] or packed nibbles [N,K/2]
+  const half_t *scales;   // Q4: [N, K/group]
+  half_t *C;
+  int M, N, K;
+  int64_t lda, ldw, ldc;  // ldw in elements (fp16) or bytes (Q4)
+  int zero;
+  int groups;             // Q4: scales per row
+};
+
+template <int MB_, int NB_, int WN_, int RK_, bool Q4_, int DEPTH_>
+struct TileSkinny {
+  typedef SkinnyArgs Args;
+  static constexpr int MB = MB_, NB = NB_, WN = WN_, RK = RK_, DEPTH = DEPTH_;
+  static constexpr bool Q4 = Q4_;
+  static constexpr int BM = 16 * MB, BN = 16 * NB * WN;
+  static constexpr int BK = Q4 ? 256 : 128;  // K per wave per iteration
+  static constexpr int BKC = BK * RK;        // K per CTA iteration
+  static constexpr int KL = BK / 4;          // K per lane group
+  static constexpr int NCH = KL / 8;         // MFMA K-chunks per iteration
+  static constexpr int WLOADS = Q4 ? KL / 32 : KL / 8;  // 16-byte weight loads per lane, block, iter
+  static constexpr int NT = WN * RK * 64;
+  static constexpr int LDA = BKC + 8;        // LDS row of A (halfs)
+  static constexpr int A_STAGE = BM * LDA;
+  static constexpr int A_CHUNKS = BM * BKC / 8;
+  static constexpr int A_LOADS = (A_CHUNKS + NT - 1) / NT;
+  static constexpr int QGROUP = 128;
+  static constexpr int SC_PER_ITER = BKC / QGROUP;  // Q4 scale groups per CTA iteration
+  static constexpr int SC_MAX_ITERS = 64;           // scale staging covers this many iterations
+  static constexpr int LDS_A = 2 * A_STAGE * 2;
+  static constexpr int LDS_SC = Q4 ? BN * SC_MAX_ITERS * SC_PER_ITER * 2 : 0;
+  static constexpr int LDS_RED = RK > 1 ? (RK - 1) * WN * 64 * MB * NB * 16 : 0;
+  static constexpr int LDS_BYTES = LDS_A + LDS_SC + LDS_RED;
+  // partials are held by the rk == 0 waves only
+  static constexpr int TILE_ELEMS = BM * BN;
+  static constexpr int NTP = WN * 64;
+  static constexpr int NV4 = MB * NB;
+  // co-resident CTAs per CU the kernel is compiled for: 16 waves per CU unless LDS says less
+  static constexpr int CTAS_PER_CU_WAVES = 16 / (NT / 64);
+  static constexpr int CTAS_PER_CU_LDS = (160 * 1024) / (LDS_BYTES + 64);
+  static constexpr int CTAS_PER_CU = CTAS_PER_CU_WAVES < CTAS_PER_CU_LDS ? CTAS_PER_CU_WAVES : CTAS_PER_CU_LDS;
+  static constexpr int WAVES_PER_EU = CTAS_PER_CU * (NT / 64) / 4 > 0 ? CTAS_PER_CU * (NT / 64) / 4 : 1;
+
+  struct Acc {
+    floatx4 c[MB][NB];
+  };
+
+  static __device__ __forceinline__ void mac(const Args &a, Acc &acc, int pm, int pn, int k0, int n,
+                                             char *smem) {
+    half_t *ldsA = reinterpret_cast<half_t *>(smem);
+    half_t *ldsS = reinterpret_cast<half_t *>(smem + LDS_A);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wn = wave % WN, rk = wave / WN;
+    const int lr = lane & 15, lg = lane >> 4;
+
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+      for (int j = 0; j < NB; ++j) acc.c[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    // ---- weights: one row per lane and block; the buffer descriptor covers the tile's rows, so
+    // rows past N read as zero ----
+    constexpr int WB = Q4 ? 1 : 4;  // bytes per 2 K-values... (Q4: 1 byte, fp16: 4 bytes)
+    const int rows_w = min(BN, a.N - pn * BN);
+    const uint32_t ldw_bytes = (uint32_t)a.ldw * (Q4 ? 1 : 2);
+    const BufferRsrc rsrc_w =
+        make_rsrc(reinterpret_cast<const char *>(a.W) + (int64_t)pn * BN * ldw_bytes, rows_w * ldw_bytes);
+    const int klane = rk * BK + lg * KL;  // K offset of this lane inside a CTA iteration
+    uint32_t voff_w[NB];
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+      voff_w[j] = (uint32_t)((wn * NB + j) * 16 + lr) * ldw_bytes + (uint32_t)(klane / 2) * WB;
+
+    // ---- A tile: all BM rows are staged; rows past M read as zero ----
+    const int a_rows = min(a.M - pm * BM, BM);
+    const BufferRsrc rsrc_a = make_rsrc(a.A + (int64_t)pm * BM * a.lda, (uint32_t)(a_rows * a.lda * 2));
+    int a_rd[MB];
+#pragma unroll
+    for (int i = 0; i < MB; ++i) a_rd[i] = (i * 16 + lr) * LDA + klane;
+    uint32_t voff_a[A_LOADS];
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+      const int idx = i * NT + tid;
+      const int row = idx / (BKC / 8), kc = idx % (BKC / 8);
+      voff_a[i] = (A_CHUNKS % NT == 0 || idx < A_CHUNKS) ? (uint32_t)(row * a.lda + kc * 8) * 2 : OOB_OFFSET;
+    }
+    // only the last K-iteration of a tile can hang over K
+    const int tail_kt = (a.K % BKC != 0) ? (a.K / BKC) : -1;
+
+    uint4v wreg[DEPTH][NB][WLOADS];
+    uint4v areg[DEPTH][A_LOADS];
+
+    auto issue_loads = [&](int slot, int kt) {
+      const int kbase = kt * BKC;
+      const uint32_t koff_w = (uint32_t)(kbase / 2) * WB, koff_a = (uint32_t)kbase * 2;
+      if (kt != tail_kt) {
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+#pragma unroll
+          for (int c = 0; c < WLOADS; ++c) wreg[slot][j][c] = buffer_load_16(rsrc_w, voff_w[j], koff_w + c * 16);
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) areg[slot][i] = buffer_load_16(rsrc_a, voff_a[i], koff_a);
+      } else {
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+#pragma unroll
+          for (int c = 0; c < WLOADS; ++c) {
+            const bool inside = kbase + klane + c * (Q4 ? 32 : 8) < a.K;
+            wreg[slot][j][c] = buffer_load_16(rsrc_w, inside ? voff_w[j] : OOB_OFFSET, koff_w + c * 16);
+          }
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) {
+          const int kc = (i * NT + tid) % (BKC / 8);
+          const bool inside = kbase + kc * 8 < a.K;
+          areg[slot][i] = buffer_load_16(rsrc_a, inside ? voff_a[i] : OOB_OFFSET, koff_a);
+        }
+      }
+    };
+    auto stage_a = [&](int slot, int buf) {
+      half_t *dst = ldsA + buf * A_STAGE;
+#pragma unroll
+      for (int i = 0; i < A_LOADS; ++i) {
+        const int idx = i * NT + tid;
+        const int row = idx / (BKC / 8), kc = idx % (BKC / 8);
+        if (A_CHUNKS % NT == 0 || idx < A_CHUNKS) {
+          uint4v v = areg[slot][i];
+          if (Q4) {
+            // element order 0,4,1,5,2,6,3,7 == interleave the low and high 8 bytes by halfs
+            uint4v p;
+            p[0] = __builtin_amdgcn_perm(v[2], v[0], 0x05040100u);
+            p[1] = __builtin_amdgcn_perm(v[2], v[0], 0x07060302u);
+            p[2] = __builtin_amdgcn_perm(v[3], v[1], 0x05040100u);
+            p[3] = __builtin_amdgcn_perm(v[3], v[1], 0x07060302u);
+            v = p;
+          }
+          *reinterpret_cast<uint4v *>(dst + row * LDA + kc * 8) = v;
+        }
+      }
+    };
+
+    // ---- Q4: stage the scales this segment needs: ldsS[row][iter][group-in-iter] ----
+    if (Q4) {
+      const int per_row = n * SC_PER_ITER;
+      for (int idx = tid; idx < BN * per_row; idx += NT) {
+        const int r = idx / per_row, c = idx % per_row;
+        const int row = min(pn * BN + r, a.N - 1);
+        const int g = min(k0 * SC_PER_ITER + c, a.groups - 1);
+        ldsS[r * (SC_MAX_ITERS * SC_PER_ITER) + c] = a.scales[(int64_t)row * a.groups + g];
+      }
+    }
+    const half2v bias = q4_bias(a.zero);
+
+    // ---- prologue: DEPTH iterations of loads in flight, A tile of the first one in LDS ----
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d)
+      if (d < n) issue_loads(d, k0 + d);
+    stage_a(0, 0);
+    __syncthreads();
+
+    for (int it0 = 0; it0 < n; it0 += DEPTH) {
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d) {
+        const int it = it0 + d;
+        if (it < n) {
+          const half_t *abuf = ldsA + (it & 1) * A_STAGE;
+          half2v sc[NB];
+          if (Q4) {
+#pragma unroll
+            for (int j = 0; j < NB; ++j) {
+              half_t s = ldsS[((wn * NB + j) * 16 + lr) * (SC_MAX_ITERS * SC_PER_ITER) +
+                              it * SC_PER_ITER + (klane / QGROUP)];
+              sc[j] = half2v{s, s};
+            }
+          }
+#pragma unroll
+          for (int ch = 0; ch < NCH; ++ch) {
+            half8v fa[MB];
+#pragma unroll
+            for (int i = 0; i < MB; ++i)
+              fa[i] = *reinterpret_cast<const half8v *>(abuf + a_rd[i] + ch * 8);
+#pragma unroll
+            for (int j = 0; j < NB; ++j) {
+              half8v fw;
+              if (Q4) {
+                fw = dequant_word_q4(wreg[d][j][ch / 4][ch % 4], bias, sc[j]);
+              } else {
+                union { uint4v u; half8v h; } cv;
+                cv.u = wreg[d][j][ch];
+                fw = cv.h;
+              }
+#pragma unroll
+              for (int i = 0; i < MB; ++i)
+                acc.c[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fw, fa[i], acc.c[i][j], 0, 0, 0);
+            }
+          }
+          // A tile of the next iteration into the other LDS buffer, then refill this ring slot
+          if (it + 1 < n) stage_a((d + 1) % DEPTH, (it + 1) & 1);
+          if (it + DEPTH < n) issue_loads(d, k0 + it + DEPTH);
+          __syncthreads();
+        }
+      }
+    }
+
+    // ---- sum the RK partial accumulators into the rk == 0 waves ----
+    if (RK > 1) {
+      float *red = reinterpret_cast<float *>(smem + LDS_A + LDS_SC);
+      if (rk > 0) {
+#pragma unroll
+        for (int i = 0; i < MB; ++i)
+#pragma unroll
+          for (int j = 0; j < NB; ++j)
+            *reinterpret_cast<floatx4 *>(red + ((((rk - 1) * WN + wn) * NV4 + i * NB + j) * 64 + lane) * 4) =
+                acc.c[i][j];
+      }
+      __syncthreads();
+      if (rk == 0) {
+#pragma unroll
+        for (int r = 1; r < RK; ++r)
+#pragma unroll
+          for (int i = 0; i < MB; ++i)
+#pragma unroll
+            for (int j = 0; j < NB; ++j)
+              acc.c[i][j] += *reinterpret_cast<const floatx4 *>(
+                  red + ((((r - 1) * WN + wn) * NV4 + i * NB + j) * 64 + lane) * 4);
+      }
+      __syncthreads();
+    }
+  }
+
+  // acc.c[i][j][r] = C[pm*BM + i*16 + lane%16][pn*BN + (wn*NB + j)*16 + 4*(lane/16) + r]
+  static __device__ __forceinline__ void store_c(const Args &a, const Acc &acc, int pm, int pn, char *) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (wave >= WN) return;
+    const int lr = lane & 15, lg = lane >> 4;
+    const bool vec_ok = (a.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(a.C) & 7) == 0);
+#pragma unroll
+    for (int i = 0; i < MB; ++i) {
+      const int row = pm * BM + i * 16 + lr;
+#pragma unroll
+      for (int j = 0; j < NB; ++j) {
+        const int col = pn * BN + (wave * NB + j) * 16 + lg * 4;
+        if (row < a.M && col < a.N) {
+          half4v h;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) h[e] = (half_t)acc.c[i][j][e];
+          half_t *dst = a.C + (int64_t)row * a.ldc + col;
+          if (vec_ok && col + 4 <= a.N) {
+            *reinterpret_cast<half4v *>(dst) = h;
+          } else {
+            for (int e = 0; e < 4 && col + e < a.N; ++e) dst[e] = h[e];
+          }
+        }
+      }
+    }
+  }
+
+  static __device__ __forceinline__ void store_partial(const Acc &acc, float *dst) {
+    if (threadIdx.x >= NTP) return;
+#pragma unroll
+    for (int v = 0; v < NV4; ++v)
+      *reinterpret_cast<floatx4 *>(dst + ((size_t)v * NTP + threadIdx.x) * 4) = acc.c[v / NB][v % NB];
+  }
+  static __device__ __forceinline__ void add_partial(Acc &acc, const float *src) {
+    if (threadIdx.x >= NTP) return;
+#pragma unroll
+    for (int v = 0; v < NV4; ++v)
+      acc.c[v / NB][v % NB] += *reinterpret_cast<const floatx4 *>(src + ((size_t)v * NTP + threadIdx.x) * 4);
+  }
+  static __device__ __forceinline__ void atomic_partial(const Acc &acc, float *dst) {
+    if (threadIdx.x >= NTP) return;
+#pragma unroll
+    for (int v = 0; v < NV4; ++v)
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        atomic_add_f32(dst + (size_t)(v * 4 + e) * NTP + threadIdx.x, acc.c[v / NB][v % NB][e]);
+  }
+  static __device__ __forceinline__ void take_partial(Acc &acc, float *src) {
+    if (threadIdx.x >= NTP) return;
+#pragma unroll
+    for (int v = 0; v < NV4; ++v)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float *p = src + (size_t)(v * 4 + e) * NTP + threadIdx.x;
+        acc.c[v / NB][v % NB][e] = *p;
+        *p = 0.f;
+      }
+  }
+};
+
+}  // namespace sk

@@ -1,0 +1,5 @@
+"""MI355X-native Stream-K GEMM: Python host layer over libstreamk.so."""
+from ._lib import LIB_PATH, StreamKError, lib, strerror  # noqa: F401
+from .ops import (StreamKKernel, bench_ms, dequant_q4, reset_workspaces, streamk_fp16,  # noqa: F401
+                  streamk_fp32, streamk_q4, tl_matmul_streamk, workspace_status)
+from .plan import cta_range, make_config, make_plan, num_cus, tile_coords  # noqa: F401

@@ -1,0 +1,89 @@
+"""ctypes binding of libstreamk.so (the C ABI declared in include/streamk.h).
+
+The library is mandatory: there is no Python or CPU fallback for any GEMM entry point.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libstreamk.so")
+
+SK_F16, SK_F32, SK_Q4 = 0, 1, 2
+LAYOUT_NT, LAYOUT_NN = 0, 1
+SCHEDULES = {"auto": 0, "dp": 1, "sk2": 2, "sk1": 3, "basic": 4}
+FIXUPS = {"auto": 0, "atomic": 1, "reduce": 2}
+
+
+class SkConfig(ctypes.Structure):
+    _fields_ = [("bm", ctypes.c_int32), ("bn", ctypes.c_int32), ("bk", ctypes.c_int32),
+                ("grid", ctypes.c_int32), ("schedule", ctypes.c_int32), ("fixup", ctypes.c_int32),
+                ("raster", ctypes.c_int32), ("spin_limit", ctypes.c_int32),
+                ("reserved", ctypes.c_int32 * 4)]
+
+
+class SkPlan(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in (
+        "bm", "bn", "bk", "grid", "schedule", "fixup", "raster", "dtype", "layout",
+        "num_block_m", "num_block_n", "iters_per_tile", "total_tiles", "streamk_tiles",
+        "blocking_tiles", "streamk_iters", "streamk_full_tiles", "streamk_partial_tiles",
+        "dp_waves", "kernel_id", "threads", "lds_bytes")] + [
+        ("workspace_bytes", ctypes.c_int64), ("M", ctypes.c_int64), ("N", ctypes.c_int64),
+        ("K", ctypes.c_int64)]
+
+    def as_dict(self):
+        return {n: getattr(self, n) for n, _ in self._fields_}
+
+
+class StreamKError(RuntimeError):
+    def __init__(self, status, where):
+        self.status = status
+        super().__init__(f"{where}: {strerror(status)} (status {status})")
+
+
+_lib = None
+
+
+def lib():
+    """Loads libstreamk.so.  torch is imported first so that the library binds to the HIP runtime
+    torch already carries (one runtime per process: streams and pointers are shared)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    import torch  # noqa: F401  (must precede the dlopen)
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `make -C stream-k.tvm_amd/csrc` "
+            "(or __graft_entry__.build()); there is no fallback path")
+    L = ctypes.CDLL(LIB_PATH)
+    i64, vp, ci, sz = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+    P = ctypes.POINTER
+    L.sk_version.restype = ci
+    L.sk_strerror.argtypes = [ci]
+    L.sk_strerror.restype = ctypes.c_char_p
+    L.sk_device_info.argtypes = [P(ci), P(ci), P(ci)]
+    L.sk_make_plan.argtypes = [i64, i64, i64, ci, ci, P(SkConfig), ci, P(SkPlan)]
+    L.sk_plan_cta_range.argtypes = [P(SkPlan), ci, P(ctypes.c_int32), P(ctypes.c_int32)]
+    L.sk_plan_tile_coords.argtypes = [P(SkPlan), ci, P(ctypes.c_int32), P(ctypes.c_int32)]
+    L.sk_workspace_bytes.argtypes = [P(SkPlan)]
+    L.sk_workspace_bytes.restype = sz
+    L.sk_workspace_init.argtypes = [vp, sz, vp]
+    L.sk_workspace_status.argtypes = [vp, vp]
+    L.sk_gemm_f16.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, P(SkPlan), vp, sz, vp]
+    L.sk_gemm_f32.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, P(SkPlan), vp, sz, vp]
+    L.sk_gemm_q4.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, ci, ci, P(SkPlan), vp, sz, vp]
+    L.sk_dequant_q4.argtypes = [vp, vp, vp, i64, i64, ci, ci, vp]
+    for f in ("sk_device_info", "sk_make_plan", "sk_plan_cta_range", "sk_plan_tile_coords",
+              "sk_workspace_init", "sk_workspace_status", "sk_gemm_f16", "sk_gemm_f32",
+              "sk_gemm_q4", "sk_dequant_q4"):
+        getattr(L, f).restype = ci
+    _lib = L
+    return L
+
+
+def strerror(status):
+    return lib().sk_strerror(status).decode()
+
+
+def check(status, where):
+    if status != 0:
+        raise StreamKError(status, where)

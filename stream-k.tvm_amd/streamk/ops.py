@@ -1,0 +1,197 @@
+"""Python-facing Stream-K GEMM entry points over the C ABI.
+
+Mirrors the reference's operator surface:
+  * `streamk_fp16(A, B)` / `streamk_fp32(A, B)`: what running streamk_fp16.py / streamk_fp32.py
+    computes (C = A @ B.T for the fp16 NT script, C = A @ B for the fp32 NN script);
+  * `tl_matmul_streamk(M, N, K, ...)` returns a callable `kernel(A, B, C)` that writes C in place,
+    the shape of the reference's `tl_mod = TL.Profiler(...)`; `tl_mod(A, B, b_c)`
+    (streamk_fp16.py:382-387), including `do_bench`.
+torch is used for device memory and streams only.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+from .plan import make_plan
+
+_workspaces = {}
+
+
+def _stream_ptr():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _workspace(nbytes, device):
+    """One self-cleaning workspace per (device, stream), grown on demand and zeroed once."""
+    if nbytes == 0:
+        return None
+    key = (device.index if device.index is not None else torch.cuda.current_device(),
+           torch.cuda.current_stream().cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _lib.check(_lib.lib().sk_workspace_init(ws.data_ptr(), ws.numel(), _stream_ptr()),
+                   "sk_workspace_init")
+        _workspaces[key] = ws
+    return ws
+
+
+def reset_workspaces():
+    """Drops cached workspaces (needed after a StreamKError with status SK_ERR_TIMEOUT)."""
+    _workspaces.clear()
+
+
+def workspace_status():
+    """SK_OK / raises if any fix-up wait on the current stream's workspace timed out."""
+    for (dev, stream), ws in _workspaces.items():
+        if stream == torch.cuda.current_stream().cuda_stream:
+            _lib.check(_lib.lib().sk_workspace_status(ws.data_ptr(), _stream_ptr()), "sk_workspace_status")
+
+
+def _check_matrix(t, name, dtype):
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise TypeError(f"{name} must be a CUDA/HIP tensor")
+    if t.dtype != dtype:
+        raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise ValueError(f"{name} must be 2-D with unit stride along its last dimension")
+
+
+def streamk_fp16(A, B, *, Wq=None, scales=None, layout="nt", out=None, plan=None, config=None,
+                 zero=8, group=128, **kw):
+    """C = A @ B.T (layout 'nt', B is [N,K]) in fp16 with fp32 accumulation.
+
+    With `Wq` (uint8 [N, K/2], low nibble = even k) and `scales` (fp16 [N, K/group]) the weights
+    are dequantised on the fly, w = fp16((q - zero) * scale), and B is ignored (pass None).
+    `config`/kwargs: bm, bn, bk, grid, schedule, fixup, raster (see plan.make_config).
+    """
+    if Wq is not None:
+        return streamk_q4(A, Wq, scales, out=out, plan=plan, config=config, zero=zero, group=group, **kw)
+    _check_matrix(A, "A", torch.float16)
+    _check_matrix(B, "B", torch.float16)
+    if layout != "nt":
+        raise NotImplementedError("fp16 layout 'nn' is not built yet")
+    M, K = A.shape
+    N, Kb = B.shape
+    if K != Kb:
+        raise ValueError(f"K mismatch: A is {tuple(A.shape)}, B is {tuple(B.shape)}")
+    if plan is None:
+        plan = make_plan(M, N, K, "float16", layout, config, **kw)
+    C = out if out is not None else torch.empty((M, N), dtype=torch.float16, device=A.device)
+    _check_matrix(C, "out", torch.float16)
+    if tuple(C.shape) != (M, N):
+        raise ValueError("out has the wrong shape")
+    ws = _workspace(plan.workspace_bytes, A.device)
+    rc = _lib.lib().sk_gemm_f16(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, A.stride(0),
+                                B.stride(0), C.stride(0), ctypes.byref(plan),
+                                ws.data_ptr() if ws is not None else None,
+                                ws.numel() if ws is not None else 0, _stream_ptr())
+    _lib.check(rc, "sk_gemm_f16")
+    return C
+
+
+def streamk_q4(A, Wq, scales, *, out=None, plan=None, config=None, zero=8, group=128, **kw):
+    """C[M,N] fp16 = A[M,K] fp16 @ dequant(Wq)[N,K].T, weights in natural nibble order
+    (streamk_fp16_ladder_block_reduce_q4.py:552)."""
+    _check_matrix(A, "A", torch.float16)
+    _check_matrix(Wq, "Wq", torch.uint8)
+    _check_matrix(scales, "scales", torch.float16)
+    M, K = A.shape
+    N = Wq.shape[0]
+    if Wq.shape[1] * 2 != K or not Wq.is_contiguous():
+        raise ValueError(f"Wq must be contiguous [N, K/2]; got {tuple(Wq.shape)} for K={K}")
+    if tuple(scales.shape) != (N, K // group) or not scales.is_contiguous():
+        raise ValueError(f"scales must be contiguous [N, K/group]; got {tuple(scales.shape)}")
+    if plan is None:
+        plan = make_plan(M, N, K, "q4", "nt", config, **kw)
+    C = out if out is not None else torch.empty((M, N), dtype=torch.float16, device=A.device)
+    _check_matrix(C, "out", torch.float16)
+    ws = _workspace(plan.workspace_bytes, A.device)
+    rc = _lib.lib().sk_gemm_q4(A.data_ptr(), Wq.data_ptr(), scales.data_ptr(), C.data_ptr(), M, N, K,
+                               A.stride(0), C.stride(0), group, zero, ctypes.byref(plan),
+                               ws.data_ptr() if ws is not None else None,
+                               ws.numel() if ws is not None else 0, _stream_ptr())
+    _lib.check(rc, "sk_gemm_q4")
+    return C
+
+
+def dequant_q4(Wq, scales, *, zero=8, group=128):
+    """fp16 W[N,K] from packed nibbles, by the same device function the Q4 GEMM uses."""
+    _check_matrix(Wq, "Wq", torch.uint8)
+    _check_matrix(scales, "scales", torch.float16)
+    N, K = Wq.shape[0], Wq.shape[1] * 2
+    if not Wq.is_contiguous() or not scales.is_contiguous():
+        raise ValueError("Wq and scales must be contiguous")
+    W = torch.empty((N, K), dtype=torch.float16, device=Wq.device)
+    rc = _lib.lib().sk_dequant_q4(Wq.data_ptr(), scales.data_ptr(), W.data_ptr(), N, K, group, zero,
+                                  _stream_ptr())
+    _lib.check(rc, "sk_dequant_q4")
+    return W
+
+
+def streamk_fp32(A, B, *, layout="nn", out=None, plan=None, config=None, **kw):
+    """C = A @ B in fp32 (layout 'nn', B is [K,N]: streamk_fp32.py:65-76)."""
+    _check_matrix(A, "A", torch.float32)
+    _check_matrix(B, "B", torch.float32)
+    M, K = A.shape
+    N = B.shape[1] if layout == "nn" else B.shape[0]
+    if plan is None:
+        plan = make_plan(M, N, K, "float32", layout, config, **kw)
+    C = out if out is not None else torch.empty((M, N), dtype=torch.float32, device=A.device)
+    ws = _workspace(plan.workspace_bytes, A.device)
+    rc = _lib.lib().sk_gemm_f32(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, A.stride(0),
+                                B.stride(0), C.stride(0), ctypes.byref(plan),
+                                ws.data_ptr() if ws is not None else None,
+                                ws.numel() if ws is not None else 0, _stream_ptr())
+    _lib.check(rc, "sk_gemm_f32")
+    return C
+
+
+class StreamKKernel:
+    """A planned GEMM, callable as `kernel(A, B, C)` (C written in place), the role of the
+    reference's compiled `tl_mod` (streamk_fp32.py:197-202)."""
+
+    def __init__(self, M, N, K, dtype, layout, plan):
+        self.M, self.N, self.K, self.dtype, self.layout, self.plan = M, N, K, dtype, layout, plan
+
+    def __call__(self, A, B, C):
+        if self.dtype == "float16":
+            return streamk_fp16(A, B, layout=self.layout, out=C, plan=self.plan)
+        return streamk_fp32(A, B, layout=self.layout, out=C, plan=self.plan)
+
+    def do_bench(self, fn=None, warmup=25, rep=100):
+        """Mean milliseconds per call over `rep` back-to-back launches after `warmup`
+        (streamk_fp16.py:394)."""
+        if fn is None:
+            dt = torch.float16 if self.dtype == "float16" else torch.float32
+            A = torch.randn(self.M, self.K, device="cuda", dtype=dt)
+            bshape = (self.N, self.K) if self.layout == "nt" else (self.K, self.N)
+            B = torch.randn(*bshape, device="cuda", dtype=dt)
+            C = torch.empty(self.M, self.N, device="cuda", dtype=dt)
+            fn = lambda: self(A, B, C)  # noqa: E731
+        return bench_ms(fn, warmup, rep)
+
+
+def bench_ms(fn, warmup=25, rep=100):
+    for _ in range(warmup):
+        fn()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(rep):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / rep
+
+
+def tl_matmul_streamk(M, N, K, *, dtypeAB="float16", layout=None, block_M=None, block_N=None,
+                      block_K=None, streamk_programs=None, schedule="auto", fixup="auto", raster=0):
+    """Factory with the reference's name and role (streamk_fp32.py:57-72, streamk_fp16.py:116-124):
+    fixes shape, tile and partition, returns the in-place kernel callable."""
+    if layout is None:
+        layout = "nt" if dtypeAB == "float16" else "nn"
+    plan = make_plan(M, N, K, dtypeAB, layout, bm=block_M, bn=block_N, bk=block_K,
+                     grid=streamk_programs, schedule=schedule, fixup=fixup, raster=raster)
+    return StreamKKernel(M, N, K, dtypeAB, layout, plan)

@@ -1,0 +1,64 @@
+"""Host partitioner front-end: the integers of streamk_fp32.py:30-54 for a run-time shape."""
+import ctypes
+
+from . import _lib
+from ._lib import SkConfig, SkPlan
+
+_DTYPES = {"float16": _lib.SK_F16, "float32": _lib.SK_F32, "q4": _lib.SK_Q4}
+_LAYOUTS = {"nt": _lib.LAYOUT_NT, "nn": _lib.LAYOUT_NN}
+_num_cus = None
+
+
+def num_cus():
+    """Compute units of the current device (the reference hard-codes total_sm = 108,
+    streamk_fp32.py:17)."""
+    global _num_cus
+    if _num_cus is None:
+        n = ctypes.c_int()
+        _lib.check(_lib.lib().sk_device_info(ctypes.byref(n), None, None), "sk_device_info")
+        _num_cus = n.value
+    return _num_cus
+
+
+def make_config(config=None, **kw):
+    """dict / kwargs -> SkConfig.  Keys: bm, bn, bk, grid, schedule ('auto'|'dp'|'sk2'|'sk1'|
+    'basic'), fixup ('auto'|'atomic'|'reduce'), raster, spin_limit."""
+    d = dict(config or {})
+    d.update(kw)
+    c = SkConfig()
+    for k, v in d.items():
+        if v is None:
+            continue
+        if k == "schedule":
+            v = _lib.SCHEDULES[v] if isinstance(v, str) else int(v)
+        elif k == "fixup":
+            v = _lib.FIXUPS[v] if isinstance(v, str) else int(v)
+        if k not in ("bm", "bn", "bk", "grid", "schedule", "fixup", "raster", "spin_limit"):
+            raise KeyError(f"unknown Stream-K config key {k!r}")
+        setattr(c, k, int(v))
+    return c
+
+
+def make_plan(M, N, K, dtype="float16", layout="nt", config=None, cus=None, **kw):
+    """Partition an M x N x K GEMM.  `cus` overrides the device's CU count (lets the partitioner
+    run without a GPU)."""
+    cfg = make_config(config, **kw)
+    plan = SkPlan()
+    rc = _lib.lib().sk_make_plan(M, N, K, _DTYPES[dtype], _LAYOUTS[layout], ctypes.byref(cfg),
+                                 cus if cus is not None else num_cus(), ctypes.byref(plan))
+    _lib.check(rc, f"sk_make_plan({M},{N},{K},{dtype},{layout},{kw or config})")
+    return plan
+
+
+def cta_range(plan, pid):
+    s, e = ctypes.c_int32(), ctypes.c_int32()
+    _lib.check(_lib.lib().sk_plan_cta_range(ctypes.byref(plan), pid, ctypes.byref(s), ctypes.byref(e)),
+               "sk_plan_cta_range")
+    return s.value, e.value
+
+
+def tile_coords(plan, tile):
+    m, n = ctypes.c_int32(), ctypes.c_int32()
+    _lib.check(_lib.lib().sk_plan_tile_coords(ctypes.byref(plan), tile, ctypes.byref(m), ctypes.byref(n)),
+               "sk_plan_tile_coords")
+    return m.value, n.value
