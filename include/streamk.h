@@ -89,6 +89,7 @@ typedef struct sk_plan {
   int32_t kernel_id;             /* which compiled kernel instance runs this plan */
   int32_t threads;               /* workgroup size of that kernel */
   int32_t lds_bytes;             /* static LDS of that kernel */
+  int32_t spin_limit;            /* REDUCE fix-up: polls of a peer's flag before giving up */
   int64_t workspace_bytes;       /* what sk_gemm_* needs for this plan */
   int64_t M, N, K;
 } sk_plan;

@@ -90,7 +90,7 @@ int make_dev_plan(const sk_plan *plan, const KernelInfo *k, void *ws, size_t ws_
   dp->grid = plan->grid;
   dp->fixup = plan->fixup == SK_FIXUP_ATOMIC ? FIXUP_ATOMIC : FIXUP_REDUCE;
   dp->raster = plan->raster;
-  dp->spin_limit = 1 << 22;
+  dp->spin_limit = plan->spin_limit > 0 ? plan->spin_limit : (1 << 22);
   dp->xcd_remap = (plan->grid % 8 == 0) ? 1 : 0;
   w->status = nullptr; w->flags = nullptr; w->partials = nullptr;
   if (plan->workspace_bytes > 0) {

@@ -141,6 +141,7 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
   if (fixup == SK_FIXUP_AUTO) fixup = SK_FIXUP_REDUCE;
   if (fixup != SK_FIXUP_ATOMIC && fixup != SK_FIXUP_REDUCE) return SK_ERR_CONFIG;
   out->fixup = fixup;
+  out->spin_limit = cfg && cfg->spin_limit > 0 ? cfg->spin_limit : (1 << 22);
   out->raster = cfg ? cfg->raster : 0;
   if (out->raster < 0) return SK_ERR_CONFIG;
 

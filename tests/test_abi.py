@@ -1,0 +1,118 @@
+"""CPU-side checks of the shipped library: it loads, exports what include/streamk.h declares, its
+partitioner agrees with the oracle's restatement of the reference, and bad calls are refused with
+error codes (no compute entry point is launched here)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def sk():
+    import streamk
+    streamk.lib()
+    return streamk
+
+
+def test_exports_every_declared_symbol(sk):
+    header = open(os.path.join(ROOT, "include", "streamk.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    names = set(re.findall(r"\b(sk_[a-z0-9_]+)\s*\(", header))
+    assert {"sk_make_plan", "sk_gemm_f16", "sk_gemm_f32", "sk_gemm_q4", "sk_dequant_q4",
+            "sk_workspace_init", "sk_workspace_bytes", "sk_strerror", "sk_version"} <= names
+    L = sk.lib()
+    for n in sorted(names):
+        assert hasattr(L, n), f"{n} is declared in streamk.h but not exported"
+    assert L.sk_version() == 100
+    assert sk.strerror(0) == "ok" and "workspace" in sk.strerror(-5)
+
+
+@pytest.mark.parametrize("shape,tile,P", [
+    ((1024, 1024, 8192), (128, 128, 64), 256),
+    ((3000, 5120, 12288), (128, 128, 64), 256),
+    ((8192, 8192, 8192), (256, 256, 64), 256),
+    ((256, 4096, 4096), (128, 128, 64), 200),
+    ((300, 700, 1000), (64, 64, 64), 24),
+])
+def test_plan_matches_oracle(sk, oracle, shape, tile, P):
+    """Two-tile hybrid schedule == the reference's partition (streamk_fp32.py:33-54) as the oracle
+    restates it, for the product's own tile shapes."""
+    M, N, K = shape
+    plan = sk.make_plan(M, N, K, "float16", "nt", cus=256, bm=tile[0], bn=tile[1], bk=tile[2],
+                        grid=P, schedule="sk2")
+    ref = oracle.partition(M, N, K, *tile, P)
+    for k in ("num_block_m", "num_block_n", "iters_per_tile", "total_tiles", "streamk_tiles",
+              "blocking_tiles", "streamk_iters", "streamk_full_tiles", "streamk_partial_tiles"):
+        assert getattr(plan, k) == ref[k], k
+    assert plan.dp_waves == ref["sm_partition_factor"]
+    for pid in (0, 1, P // 2, P - 1):
+        assert sk.cta_range(plan, pid) == oracle.cta_range(ref, pid)
+    nbn = ref["num_block_n"]
+    for t in (0, 1, nbn, ref["total_tiles"] - 1):
+        assert sk.tile_coords(plan, t) == (t // nbn, t % nbn)  # streamk_fp32.py:106-107
+
+
+def test_schedules(sk):
+    kw = dict(cus=256, bm=128, bn=128, bk=64, grid=256)
+    dp = sk.make_plan(1024, 8192, 8192, "float16", "nt", schedule="dp", **kw)
+    assert (dp.streamk_tiles, dp.blocking_tiles, dp.dp_waves, dp.workspace_bytes) == (0, 512, 2, 0)
+    basic = sk.make_plan(1024, 1024, 8192, "float16", "nt", schedule="basic", **kw)
+    assert (basic.streamk_tiles, basic.blocking_tiles) == (64, 0)
+    one = sk.make_plan(3000, 5120, 12288, "float16", "nt", schedule="sk1", **kw)
+    assert (one.total_tiles, one.streamk_tiles, one.blocking_tiles) == (960, 192, 768)
+    auto = sk.make_plan(8192, 8192, 8192, "float16", "nt", cus=256)
+    assert (auto.bm, auto.bn, auto.schedule, auto.streamk_tiles) == (256, 256, 1, 0)
+
+
+def test_raster_is_a_permutation(sk):
+    plan = sk.make_plan(3000, 5120, 4096, "float16", "nt", cus=256, bm=128, bn=128, bk=64, raster=8)
+    seen = {sk.tile_coords(plan, t) for t in range(plan.total_tiles)}
+    assert len(seen) == plan.total_tiles == plan.num_block_m * plan.num_block_n
+    # walks 8 tile rows down before stepping to the next column (triton_impl.py:14-28)
+    assert [sk.tile_coords(plan, t) for t in range(3)] == [(0, 0), (1, 0), (2, 0)]
+    assert sk.tile_coords(plan, 8) == (0, 1)
+
+
+def test_error_codes(sk):
+    L = sk.lib()
+    with pytest.raises(sk.StreamKError) as e:
+        sk.make_plan(0, 10, 10, cus=256)
+    assert e.value.status == -2
+    with pytest.raises(sk.StreamKError) as e:
+        sk.make_plan(128, 128, 100, cus=256)  # K not a multiple of 8
+    assert e.value.status == -3
+    with pytest.raises(sk.StreamKError) as e:
+        sk.make_plan(128, 128, 128, cus=256, bm=48, bn=48)  # no such kernel
+    assert e.value.status == -4
+    with pytest.raises(sk.StreamKError) as e:
+        sk.make_plan(4096, 4096, 4096, cus=256, bm=256, bn=256, grid=512)  # not co-resident
+    assert e.value.status == -4
+    plan = sk.make_plan(1024, 1024, 8192, cus=256, bm=128, bn=128, bk=64, grid=256)
+    assert L.sk_gemm_f16(None, None, None, 1024, 1024, 8192, 8192, 8192, 1024, ctypes.byref(plan),
+                         None, 0, None) == -1
+    fake = ctypes.c_void_p(4096)
+    # plan made for another shape
+    assert L.sk_gemm_f16(fake, fake, fake, 512, 1024, 8192, 8192, 8192, 1024, ctypes.byref(plan),
+                         None, 0, None) == -4
+    # leading dimension smaller than the row / misaligned
+    assert L.sk_gemm_f16(fake, fake, fake, 1024, 1024, 8192, 100, 8192, 1024, ctypes.byref(plan),
+                         None, 0, None) == -2
+    assert L.sk_gemm_f16(fake, fake, fake, 1024, 1024, 8192, 8196, 8192, 1024, ctypes.byref(plan),
+                         None, 0, None) == -3
+    assert L.sk_gemm_f16(ctypes.c_void_p(4098), fake, fake, 1024, 1024, 8192, 8192, 8192, 1024,
+                         ctypes.byref(plan), None, 0, None) == -3
+    assert L.sk_dequant_q4(fake, fake, fake, 16, 100, 128, 8, None) == -4
+    assert L.sk_workspace_init(None, 16, None) == -1
+
+
+def test_product_does_not_touch_the_oracle():
+    """The shipped package must never import or call the CPU checker."""
+    pkg = os.path.join(ROOT, "stream-k.tvm_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".h", ".hip", ".cpp", "Makefile")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text.lower(), os.path.join(dirpath, f)

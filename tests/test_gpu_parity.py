@@ -1,0 +1,258 @@
+"""GPU parity tests: the HIP path, called through the C ABI, against the CPU oracle on the same
+seeded inputs, against the committed fixtures, and through size-independent properties at the
+full benchmark sizes.
+
+Tolerance for fp16-out / fp32-accumulate GEMMs: max|C - ref| / max|ref| <= 1e-2 against an fp32 host
+matmul (the reference asserts rtol = atol = 1e-2, streamk_fp32.py:208).  Q4 dequantisation and the
+ordered-reduce fix-up are checked bit for bit.
+"""
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2
+
+
+@pytest.fixture(scope="module")
+def sk():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    import streamk
+    streamk.lib()
+    maps = open("/proc/self/maps").read()
+    assert "libstreamk.so" in maps, "native library not loaded"
+    return streamk
+
+
+def _t(x):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(x)).cuda()
+
+
+def _uniform16(shape, seed):
+    # uniform [-1, 1) rounded to fp16 (streamk_fp16.py:65-67 draws rand*2-1)
+    rng = np.random.default_rng(seed)
+    return (rng.random(shape, dtype=np.float32) * 2 - 1).astype(np.float16)
+
+
+def _rel(oracle, C, ref):
+    return oracle.max_abs_rel(C.float().cpu().numpy(), ref)
+
+
+TILE_CONFIGS = [
+    dict(bm=128, bn=128, bk=64), dict(bm=256, bn=256, bk=64), dict(bm=128, bn=256, bk=64),
+    dict(bm=256, bn=128, bk=64), dict(bm=64, bn=64, bk=64), dict(bm=256, bn=256, bk=32),
+    dict(bm=128, bn=128, bk=32),
+]
+SKINNY_CONFIGS = [
+    dict(bm=16, bn=64, bk=128), dict(bm=32, bn=64, bk=128), dict(bm=64, bn=64, bk=128),
+    dict(bm=16, bn=16, bk=512), dict(bm=16, bn=32, bk=256),
+]
+
+
+@pytest.mark.parametrize("cfg", TILE_CONFIGS + SKINNY_CONFIGS, ids=lambda c: f"{c['bm']}x{c['bn']}x{c['bk']}")
+@pytest.mark.parametrize("sched,fixup,grid", [("dp", "reduce", 8), ("basic", "reduce", 8),
+                                             ("basic", "atomic", 8), ("sk2", "reduce", 3),
+                                             ("sk2", "atomic", 5)])
+def test_fixture_ragged_f16(sk, oracle, golden_dir, cfg, sched, fixup, grid):
+    """200 x 136 x 328 (ragged in M, N and K for every tile shape) against the committed fixture;
+    small grids force tiles to be split over several CTAs."""
+    g = np.load(os.path.join(golden_dir, "gemm_f16_nt_200x136x328.npz"))
+    A, B, ref = g["A"], g["B"], g["C"]
+    if cfg["bm"] <= 64 and cfg["bn"] <= 64 and cfg["bk"] != 64:  # small-M kernels take M <= bm
+        A, ref = A[:cfg["bm"] - 3], ref[:cfg["bm"] - 3]
+    C = sk.streamk_fp16(_t(A), _t(B), schedule=sched, fixup=fixup, grid=grid, **cfg)
+    sk.workspace_status()
+    assert _rel(oracle, C, ref) <= 2e-3 <= TOL
+
+
+@pytest.mark.parametrize("fixup", ["atomic", "reduce"])
+@pytest.mark.parametrize("cfg", [dict(bm=128, bn=128, bk=64, grid=256), dict(bm=128, bn=128, bk=32, grid=256),
+                                 dict(bm=256, bn=256, bk=64)],
+                         ids=["128x128x64", "128x128x32", "256x256x64"])
+def test_cfg2_streamk_both_fixups(sk, oracle, cfg, fixup):
+    """M = N = 1024, K = 8192, NT, U[-1,1) seed 0: 64 tiles of 128x128 on 256 CUs, every tile split
+    along K over 4 CTAs; both fix-ups against the oracle's fp32 host matmul."""
+    A, B = _uniform16((1024, 8192), 0), _uniform16((1024, 8192), 1)
+    ref = oracle.matmul_fp32(A, B, trans_b=True)
+    plan = sk.make_plan(1024, 1024, 8192, "float16", "nt", schedule="sk2", fixup=fixup, **cfg)
+    assert plan.streamk_tiles == plan.total_tiles and plan.blocking_tiles == 0
+    C = sk.streamk_fp16(_t(A), _t(B), plan=plan)
+    sk.workspace_status()
+    assert _rel(oracle, C, ref) <= 1e-3 <= TOL
+
+
+def test_reduce_fixup_is_bitwise_reproducible(sk):
+    """The ordered reduce must give identical bits run to run (10 runs, two shapes); the schedule
+    splits every tile."""
+    import torch
+    for (M, N, K, cfg) in [(1024, 1024, 8192, dict(bm=128, bn=128, bk=64, grid=256)),
+                           (16, 4096, 11008, dict()), (300, 1000, 4096, dict(bm=64, bn=64, bk=64, grid=200))]:
+        A, B = _t(_uniform16((M, K), 2)), _t(_uniform16((N, K), 3))
+        first = sk.streamk_fp16(A, B, schedule="basic", fixup="reduce", **cfg).clone()
+        for _ in range(9):
+            again = sk.streamk_fp16(A, B, schedule="basic", fixup="reduce", **cfg)
+            assert torch.equal(first, again)
+    sk.workspace_status()
+
+
+@pytest.mark.parametrize("NK", [(4096, 4096), (11008, 4096), (4096, 11008), (28672, 8192)],
+                         ids=lambda nk: f"N{nk[0]}_K{nk[1]}")
+@pytest.mark.parametrize("M", [1, 16, 64, 256])
+def test_cfg3_small_m_sweep(sk, oracle, M, NK):
+    """Small-M sweep, inputs normal(0, 0.02); heuristic plan (weight-streaming kernels for M <= 64,
+    LDS-tiled kernel for M = 256)."""
+    N, K = NK
+    rng = np.random.default_rng(M * 7 + N)
+    A = (rng.standard_normal((M, K), dtype=np.float32) * 0.02).astype(np.float16)
+    B = (rng.standard_normal((N, K), dtype=np.float32) * 0.02).astype(np.float16)
+    ref = oracle.matmul_fp32(A, B, trans_b=True)
+    for fixup in ("reduce", "atomic"):
+        C = sk.streamk_fp16(_t(A), _t(B), fixup=fixup)
+        assert _rel(oracle, C, ref) <= 2e-3 <= TOL, fixup
+    sk.workspace_status()
+
+
+def test_q4_dequant_bit_exact(sk, oracle, golden_dir):
+    g = np.load(os.path.join(golden_dir, "q4_16x256.npz"))
+    W = sk.dequant_q4(_t(g["Wq"]), _t(g["scales"])).cpu().numpy()
+    assert np.array_equal(W.view(np.uint16), g["W"].view(np.uint16))
+    # every nibble x 4096 scales spread over all of fp16 (incl. subnormal results), zero points 0/8/15
+    bits = np.arange(0, 65536, 16, dtype=np.uint16)
+    sc = bits.view(np.float16)
+    sc = sc[np.isfinite(sc.astype(np.float32))].reshape(-1, 1)
+    nib = (np.arange(128) % 16).astype(np.uint8)
+    Wq = np.broadcast_to((nib[0::2] | (nib[1::2] << 4)).astype(np.uint8), (sc.shape[0], 64)).copy()
+    for zero in (8, 0, 15):
+        got = sk.dequant_q4(_t(Wq), _t(sc), zero=zero).cpu().numpy().view(np.uint16)
+        assert np.array_equal(got, oracle.dequant_q4(Wq, sc, 128, zero).view(np.uint16)), zero
+
+
+def test_q4_gemm_fixture(sk, oracle, golden_dir):
+    g = np.load(os.path.join(golden_dir, "q4_16x256.npz"))
+    for cfg in (dict(), dict(schedule="basic", grid=2), dict(schedule="basic", grid=2, fixup="atomic")):
+        C = sk.streamk_q4(_t(g["A"]), _t(g["Wq"]), _t(g["scales"]), **cfg)
+        assert _rel(oracle, C, g["C"]) <= 2e-3 <= TOL
+
+
+@pytest.mark.parametrize("M", [1, 16])
+def test_cfg4_q4_gemm(sk, oracle, M):
+    """Q4 weight-only GEMM at N = K = 8192: A normal(0,1), nibbles uniform 0..15, zero-point 8,
+    scales U[0.005, 0.02] per (row, 128-wide group); Stream-K with the ordered reduce (and atomic),
+    every kernel variant."""
+    N = K = 8192
+    rng = np.random.default_rng(40 + M)
+    A = rng.standard_normal((M, K), dtype=np.float32).astype(np.float16)
+    Wq = rng.integers(0, 256, (N, K // 2), dtype=np.uint8)
+    sc = rng.uniform(0.005, 0.02, (N, K // 128)).astype(np.float16)
+    ref = oracle.q4_gemm_ref(A, Wq, sc, 128, 8)
+    dA, dW, dS = _t(A), _t(Wq), _t(sc)
+    # the GEMM consumes exactly the weights the standalone dequant produces: check those first
+    W = sk.dequant_q4(dW, dS).cpu().numpy()
+    assert np.array_equal(W.view(np.uint16), oracle.dequant_q4(Wq, sc, 128, 8).view(np.uint16))
+    for cfg in (dict(fixup="reduce"), dict(fixup="atomic"), dict(schedule="dp"),
+                dict(bm=16, bn=16, bk=1024), dict(bm=16, bn=32, bk=512), dict(schedule="basic", grid=1000)):
+        C = sk.streamk_q4(dA, dW, dS, **cfg)
+        assert _rel(oracle, C, ref) <= 2e-3 <= TOL, cfg
+    sk.workspace_status()
+
+
+def test_cfg5_large_dense(sk, oracle):
+    """M = N = K = 8192 and the irregular 3000 x 5120 x 12288, U[-1,1): a random subset of rows is
+    checked against an fp64 host product; the Stream-K and data-parallel schedules of the same kernel
+    must agree within tolerance, and the GEMM must be linear in A."""
+    import torch
+    for (M, N, K) in [(8192, 8192, 8192), (3000, 5120, 12288)]:
+        A, B = _uniform16((M, K), 5), _uniform16((N, K), 6)
+        dA, dB = _t(A), _t(B)
+        rows = np.sort(np.random.default_rng(7).choice(M, 96, replace=False))
+        ref = A[rows].astype(np.float64) @ B.astype(np.float64).T
+        outs = {}
+        for name, cfg in [("auto", dict()), ("sk128", dict(bm=128, bn=128, bk=64, schedule="sk2")),
+                          ("dp128", dict(bm=128, bn=128, bk=64, schedule="dp")),
+                          ("sk256", dict(bm=256, bn=256, bk=64, schedule="sk2", raster=8))]:
+            C = sk.streamk_fp16(dA, dB, **cfg)
+            outs[name] = C
+            got = C[torch.from_numpy(rows).cuda()].float().cpu().numpy()
+            assert oracle.max_abs_rel(got, ref) <= 1e-3 <= TOL, (M, name)
+        scale = outs["auto"].float().abs().max().item()
+        assert (outs["sk128"].float() - outs["dp128"].float()).abs().max().item() <= 2e-3 * scale
+    sk.workspace_status()
+
+
+@pytest.mark.parametrize("shape", [(8192, 8192, 8192), (3000, 5120, 12288), (1024, 1024, 8192),
+                                   (16, 8192, 8192)], ids=lambda s: "x".join(map(str, s)))
+def test_full_size_exact_integer_checksums(sk, shape):
+    """With entries in {-1, 0, 1} every product and partial sum is an integer far below 2^24 and the
+    results stay below 2048, so fp32 accumulation and the fp16 store are exact: C must equal the
+    integer product bit for bit, whatever the tile shape, split or summation order.  Checked at the
+    full benchmark sizes through row and column checksums (C 1 = A (B^T 1), 1^T C = (1^T A) B^T) in
+    int64 on the host, plus a block of rows against the full integer product."""
+    import torch
+    M, N, K = shape
+    rng = np.random.default_rng(11)
+    A = rng.integers(-1, 2, (M, K)).astype(np.int8)
+    B = rng.integers(-1, 2, (N, K)).astype(np.int8)
+    row_sum = A.astype(np.int64) @ B.astype(np.int64).sum(axis=0)
+    col_sum = A.astype(np.int64).sum(axis=0) @ B.astype(np.int64).T
+    rows = slice(0, min(M, 64))
+    block = A[rows].astype(np.int32) @ B.astype(np.int32).T
+    assert np.abs(block).max() < 2048
+    dA, dB = _t(A.astype(np.float16)), _t(B.astype(np.float16))
+    cfgs = [dict(), dict(fixup="atomic"), dict(schedule="basic")]
+    if M > 64:
+        cfgs += [dict(bm=128, bn=128, bk=64, schedule="sk2", fixup="atomic"),
+                 dict(bm=256, bn=256, bk=64, schedule="sk2", raster=8), dict(bm=128, bn=256, bk=64)]
+    for cfg in cfgs:
+        C = sk.streamk_fp16(dA, dB, **cfg)
+        Cd = C.double()
+        assert np.array_equal(Cd.sum(dim=1).cpu().numpy().astype(np.int64), row_sum), cfg
+        assert np.array_equal(Cd.sum(dim=0).cpu().numpy().astype(np.int64), col_sum), cfg
+        assert np.array_equal(C[rows].cpu().numpy().astype(np.int32), block), cfg
+        # linearity under an exact scaling
+        assert torch.equal(sk.streamk_fp16(dA * 2, dB, **cfg), C * 2), cfg
+    sk.workspace_status()
+
+
+def test_strided_operands_and_out(sk, oracle):
+    """Leading dimensions larger than the rows, and writing into a caller-provided C."""
+    import torch
+    A_full, B_full = _t(_uniform16((300, 1024), 8)), _t(_uniform16((520, 1024), 9))
+    A, B = A_full[:, :512], B_full[:, 256:768]
+    out_full = torch.zeros(300, 1040, dtype=torch.float16, device="cuda")
+    out = out_full[:, 8:528]
+    sk.streamk_fp16(A, B, out=out, bm=128, bn=128, bk=64, schedule="basic", grid=40)
+    ref = oracle.matmul_fp32(A.cpu().numpy(), B.cpu().numpy(), trans_b=True)
+    assert _rel(oracle, out, ref) <= 2e-3
+    assert out_full[:, :8].abs().max().item() == 0 and out_full[:, 528:].abs().max().item() == 0
+
+
+def test_wait_gives_up_instead_of_hanging(sk):
+    """A fix-up wait that runs out of polls must end the kernel and report SK_ERR_TIMEOUT; the
+    condition is forced from the host with a poll limit of 1 on a schedule where the followers
+    cannot have finished yet."""
+    A, B = _t(_uniform16((1024, 8192), 10)), _t(_uniform16((1024, 8192), 11))
+    sk.streamk_fp16(A, B, bm=128, bn=128, bk=64, schedule="basic", fixup="reduce", grid=256, spin_limit=1)
+    with pytest.raises(sk.StreamKError) as e:
+        sk.workspace_status()
+    assert e.value.status == -8
+    sk.reset_workspaces()
+    # and the library is usable again afterwards
+    C = sk.streamk_fp16(A, B, bm=128, bn=128, bk=64, schedule="basic", fixup="reduce", grid=256)
+    C2 = sk.streamk_fp16(A, B, bm=128, bn=128, bk=64, schedule="dp")
+    sk.workspace_status()
+    assert (C.float() - C2.float()).abs().max().item() <= 2e-3 * C2.float().abs().max().item()
+
+
+def test_bad_calls_are_refused(sk):
+    import torch
+    A = torch.zeros(64, 128, dtype=torch.float16, device="cuda")
+    with pytest.raises(TypeError):
+        sk.streamk_fp16(A.float(), A)
+    with pytest.raises(ValueError):
+        sk.streamk_fp16(A, torch.zeros(64, 136, dtype=torch.float16, device="cuda"))
+    with pytest.raises(sk.StreamKError):
+        sk.streamk_fp16(A[:, :100], A[:, :100])  # K = 100 is not a multiple of 8

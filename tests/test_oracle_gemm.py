@@ -1,0 +1,75 @@
+"""Pins the oracle's CPU Stream-K GEMM (restating streamk_fp32.py:80-158) against dense matmul, and
+the committed golden fixture against both."""
+import os
+
+import numpy as np
+import pytest
+
+
+def _inputs(M, N, K, seed=0):
+    # uniform [-1, 1), the reference's distribution (streamk_fp32.py:19-22)
+    rng = np.random.default_rng(seed)
+    return (rng.random((M, K), dtype=np.float32) * 2 - 1, rng.random((K, N), dtype=np.float32) * 2 - 1)
+
+
+@pytest.mark.parametrize("P", [4, 3, 5, 7])
+@pytest.mark.parametrize("fixup", ["atomic", "reduce"])
+def test_cpu_config_256x256x1024(oracle, P, fixup):
+    """M=256, N=256, K=1024, 64x64 tiles, 16-wide K-iterations, 4 simulated CTAs (no tile is split at
+    P=4; P=3,5,7 split tiles and exercise the fix-up), checked against numpy matmul with the
+    reference's tolerance (streamk_fp32.py:208)."""
+    A, B = _inputs(256, 256, 1024)
+    C = oracle.streamk_gemm_f32(A, B, 64, 64, 16, P, fixup=fixup)
+    ref = A.astype(np.float64) @ B.astype(np.float64)
+    np.testing.assert_allclose(C, ref, rtol=1e-2, atol=1e-2)
+    assert oracle.max_abs_rel(C, ref) < 1e-5
+
+
+def test_exact_on_integers(oracle):
+    """Small-integer inputs make every partial sum exact in fp32, so Stream-K must equal numpy
+    bit for bit whatever the split: catches a dropped / doubled K-iteration or a wrong tile index."""
+    rng = np.random.default_rng(1)
+    A = rng.integers(-4, 5, (70, 90)).astype(np.float32)
+    B = rng.integers(-4, 5, (90, 50)).astype(np.float32)
+    ref = A @ B
+    for P in (1, 2, 3, 5, 8, 13):
+        for fixup in ("atomic", "reduce"):
+            for bm, bn, bk in ((16, 8, 8), (32, 32, 16), (8, 64, 32)):
+                C = oracle.streamk_gemm_f32(A, B, bm, bn, bk, P, fixup=fixup)
+                assert np.array_equal(C, ref), (P, fixup, bm, bn, bk)
+    Bt = np.ascontiguousarray(B.T)
+    assert np.array_equal(oracle.streamk_gemm_f32(A, Bt, 16, 8, 8, 5, trans_b=True), ref)
+
+
+def test_cta_order(oracle):
+    """The ordered reduce does not depend on the order CTAs run in; the atomic flavour may differ in
+    the last bits but stays within tolerance."""
+    A, B = _inputs(96, 80, 200, seed=2)
+    base = oracle.streamk_gemm_f32(A, B, 32, 16, 8, 7, fixup="reduce")
+    rng = np.random.default_rng(3)
+    for _ in range(5):
+        order = rng.permutation(7)
+        assert np.array_equal(oracle.streamk_gemm_f32(A, B, 32, 16, 8, 7, cta_order=order, fixup="reduce"), base)
+        C = oracle.streamk_gemm_f32(A, B, 32, 16, 8, 7, cta_order=order, fixup="atomic")
+        assert oracle.max_abs_rel(C, base) < 1e-5
+
+
+def test_golden_fixture(oracle, golden_dir):
+    g = np.load(os.path.join(golden_dir, "streamk_f32_48x40x72.npz"))
+    A, B = g["A"], g["B"]
+    assert np.array_equal(oracle.streamk_gemm_f32(A, B, 16, 8, 8, 7, fixup="atomic"), g["C_atomic"])
+    assert np.array_equal(oracle.streamk_gemm_f32(A, B, 16, 8, 8, 7, fixup="reduce"), g["C_reduce"])
+    ref = A.astype(np.float64) @ B.astype(np.float64)
+    assert oracle.max_abs_rel(g["C_atomic"], ref) < 1e-5 and oracle.max_abs_rel(g["C_reduce"], ref) < 1e-5
+    part = oracle.partition(48, 40, 72, 16, 8, 8, 7)
+    assert [part[k] for k in g["partition_keys"]] == g["partition"].tolist()
+    # 15 tiles of 9 iterations on 7 CTAs: 15 % 7 + 7 = 8 Stream-K tiles = 72 iterations,
+    # 10 per CTA and 2 left over; 7 data-parallel tiles
+    assert (part["total_tiles"], part["streamk_tiles"], part["blocking_tiles"]) == (15, 8, 7)
+    assert (part["streamk_full_tiles"], part["streamk_partial_tiles"]) == (10, 2)
+
+
+def test_bad_arguments(oracle):
+    A, B = _inputs(8, 8, 8)
+    with pytest.raises(ValueError):
+        oracle.streamk_gemm_f32(A, B, 0, 8, 8, 2)
