@@ -117,7 +117,9 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
   }
   int sched = cfg ? cfg->schedule : SK_SCHED_AUTO;
   if (sched == SK_SCHED_AUTO) sched = (total % grid == 0) ? SK_SCHED_DP : SK_SCHED_SK_TWO_TILE;
-  // the grid never exceeds the work: with fewer K-iterations than CTAs the tail CTAs would idle
+  // a data-parallel-only launch never has more CTAs than tiles (idle CTAs would also skew the
+  // CTA -> XCD mapping: the low logical ids sit on the first XCDs)
+  if (sched == SK_SCHED_DP && grid > total) grid = total;
   int sk_tiles;
   switch (sched) {
     case SK_SCHED_DP: sk_tiles = 0; break;

@@ -62,28 +62,28 @@ __device__ __forceinline__ void tile_coords(const DevPlan &p, int tile, int &pm,
 }
 
 // ---- REDUCE fix-up: flags ----
-// Contributor: all of the CTA's partial stores are made visible device-wide, then one thread
-// raises the flag.
+// Contributor: the barrier orders every thread's partial stores before thread 0, whose
+// device-scope release (one L2 write-back for the whole CTA) then publishes them with the flag.
 __device__ __forceinline__ void signal_partial_ready(int *flag) {
-  __threadfence();
   __syncthreads();
   if (threadIdx.x == 0) __hip_atomic_store(flag, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Owner: thread 0 polls, everybody then acquires.  Returns false if the poll limit ran out.
+// Owner: thread 0 polls with relaxed loads (a poll must not invalidate caches: other CTAs on the
+// same L2 are still streaming), acquires once when the flag is up, and the barrier hands the
+// visibility on to the rest of the CTA.  Returns false if the poll limit ran out.
 __device__ __forceinline__ bool wait_partial_ready(int *flag, int spin_limit, int *lds_ok) {
   if (threadIdx.x == 0) {
     int ok = 0;
     for (int i = 0; i < spin_limit; ++i) {
-      if (__hip_atomic_load(flag, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) != 0) { ok = 1; break; }
-      __builtin_amdgcn_s_sleep(2);
+      if (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) { ok = 1; break; }
+      __builtin_amdgcn_s_sleep(1);
     }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     *lds_ok = ok;
   }
   __syncthreads();
-  bool ok = *lds_ok != 0;
-  __atomic_thread_fence(__ATOMIC_ACQUIRE);  // device scope is the default for HIP
-  return ok;
+  return *lds_ok != 0;
 }
 
 __device__ __forceinline__ void clear_flag_after_use(int *flag) {

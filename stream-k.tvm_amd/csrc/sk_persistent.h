@@ -55,7 +55,6 @@ __device__ __forceinline__ void run_persistent(const typename P::Args &a, const 
         // converts and stores, then leaves buffer and counter zeroed for the next launch.
         float *part = ws.partials + (size_t)tile * P::TILE_ELEMS;
         P::atomic_partial(acc, part);
-        __threadfence();
         __syncthreads();
         if (threadIdx.x == 0) {
           int old = __hip_atomic_fetch_add(&ws.flags[tile], n, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
@@ -65,7 +64,6 @@ __device__ __forceinline__ void run_persistent(const typename P::Args &a, const 
         store = s_word != 0;
         __syncthreads();
         if (store) {
-          __atomic_thread_fence(__ATOMIC_ACQUIRE);
           P::take_partial(acc, part);
           if (threadIdx.x == 0)
             __hip_atomic_store(&ws.flags[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -49,7 +49,8 @@ struct TileSkinny {
   static constexpr int SC_PER_ITER = BKC / QGROUP;  // Q4 scale groups per CTA iteration
   static constexpr int SC_MAX_ITERS = 64;           // scale staging covers this many iterations
   static constexpr int LDS_A = 2 * A_STAGE * 2;
-  static constexpr int LDS_SC = Q4 ? BN * SC_MAX_ITERS * SC_PER_ITER * 2 : 0;
+  static constexpr int SC_ROW = SC_MAX_ITERS * SC_PER_ITER + 8;  // halfs per LDS scale row
+  static constexpr int LDS_SC = Q4 ? BN * SC_ROW * 2 : 0;
   static constexpr int LDS_RED = RK > 1 ? (RK - 1) * WN * 64 * MB * NB * 16 : 0;
   static constexpr int LDS_BYTES = LDS_A + LDS_SC + LDS_RED;
   // partials are held by the rk == 0 waves only
@@ -105,36 +106,28 @@ struct TileSkinny {
       const int row = idx / (BKC / 8), kc = idx % (BKC / 8);
       voff_a[i] = (A_CHUNKS % NT == 0 || idx < A_CHUNKS) ? (uint32_t)(row * a.lda + kc * 8) * 2 : OOB_OFFSET;
     }
-    // only the last K-iteration of a tile can hang over K
-    const int tail_kt = (a.K % BKC != 0) ? (a.K / BKC) : -1;
-
     uint4v wreg[DEPTH][NB][WLOADS];
     uint4v areg[DEPTH][A_LOADS];
 
-    auto issue_loads = [&](int slot, int kt) {
-      const int kbase = kt * BKC;
+    // Loads for iterations past the segment (or past K) are still issued -- every trip through
+    // the main loop then has the same loads in flight in the same order, which keeps the waits
+    // exact -- but with an out-of-range offset, which returns zeros without touching memory.
+    // klimit = K-values left in the tile row from this iteration's start (<= 0 past the segment).
+    auto issue_loads = [&](int slot, int rel_it) {
+      const int kbase = (k0 + rel_it) * BKC;
       const uint32_t koff_w = (uint32_t)(kbase / 2) * WB, koff_a = (uint32_t)kbase * 2;
-      if (kt != tail_kt) {
+      const int klimit = rel_it < n ? a.K - kbase : 0;
 #pragma unroll
-        for (int j = 0; j < NB; ++j)
+      for (int j = 0; j < NB; ++j)
 #pragma unroll
-          for (int c = 0; c < WLOADS; ++c) wreg[slot][j][c] = buffer_load_16(rsrc_w, voff_w[j], koff_w + c * 16);
-#pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) areg[slot][i] = buffer_load_16(rsrc_a, voff_a[i], koff_a);
-      } else {
-#pragma unroll
-        for (int j = 0; j < NB; ++j)
-#pragma unroll
-          for (int c = 0; c < WLOADS; ++c) {
-            const bool inside = kbase + klane + c * (Q4 ? 32 : 8) < a.K;
-            wreg[slot][j][c] = buffer_load_16(rsrc_w, inside ? voff_w[j] : OOB_OFFSET, koff_w + c * 16);
-          }
-#pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) {
-          const int kc = (i * NT + tid) % (BKC / 8);
-          const bool inside = kbase + kc * 8 < a.K;
-          areg[slot][i] = buffer_load_16(rsrc_a, inside ? voff_a[i] : OOB_OFFSET, koff_a);
+        for (int c = 0; c < WLOADS; ++c) {
+          const bool inside = klane + c * (Q4 ? 32 : 8) < klimit;
+          wreg[slot][j][c] = buffer_load_16(rsrc_w, inside ? voff_w[j] : OOB_OFFSET, koff_w + c * 16);
         }
+#pragma unroll
+      for (int i = 0; i < A_LOADS; ++i) {
+        const bool inside = ((i * NT + tid) % (BKC / 8)) * 8 < klimit;
+        areg[slot][i] = buffer_load_16(rsrc_a, inside ? voff_a[i] : OOB_OFFSET, koff_a);
       }
     };
     auto stage_a = [&](int slot, int buf) {
@@ -159,66 +152,71 @@ struct TileSkinny {
       }
     };
 
-    // ---- Q4: stage the scales this segment needs: ldsS[row][iter][group-in-iter] ----
-    if (Q4) {
-      const int per_row = n * SC_PER_ITER;
-      for (int idx = tid; idx < BN * per_row; idx += NT) {
-        const int r = idx / per_row, c = idx % per_row;
-        const int row = min(pn * BN + r, a.N - 1);
-        const int g = min(k0 * SC_PER_ITER + c, a.groups - 1);
-        ldsS[r * (SC_MAX_ITERS * SC_PER_ITER) + c] = a.scales[(int64_t)row * a.groups + g];
-      }
-    }
     const half2v bias = q4_bias(a.zero);
 
-    // ---- prologue: DEPTH iterations of loads in flight, A tile of the first one in LDS ----
+    // ---- prologue: DEPTH iterations of loads in flight ----
 #pragma unroll
-    for (int d = 0; d < DEPTH; ++d)
-      if (d < n) issue_loads(d, k0 + d);
+    for (int d = 0; d < DEPTH; ++d) issue_loads(d, d);
+
+    // ---- Q4: stage the scales of this segment, 16 bytes at a time.  Row r of the tile needs
+    // groups [k0*SC_PER_ITER, (k0+n)*SC_PER_ITER); the copy starts at the 8-aligned group below
+    // and ldsS[r][sc_shift + i] is group k0*SC_PER_ITER + i.
+    int sc_shift = 0;
+    if (Q4) {
+      const int g_first = k0 * SC_PER_ITER, g0 = g_first & ~7;
+      sc_shift = g_first - g0;
+      const int chunks = (sc_shift + n * SC_PER_ITER + 7) >> 3;
+      const BufferRsrc rsrc_s =
+          make_rsrc(a.scales + (int64_t)pn * BN * a.groups, (uint32_t)(rows_w * a.groups * 2));
+      for (int idx = tid; idx < BN * chunks; idx += NT) {
+        const int r = idx % BN, c = idx / BN;
+        const uint4v v = buffer_load_16(rsrc_s, (uint32_t)(r * a.groups + g0 + c * 8) * 2, 0);
+        *reinterpret_cast<uint4v *>(ldsS + r * SC_ROW + c * 8) = v;
+      }
+    }
     stage_a(0, 0);
     __syncthreads();
 
+    // ---- main loop: rounds of DEPTH iterations, no exit inside a round.  Iterations past the
+    // segment multiply zeros (their loads were pushed out of range), so n need not be a multiple
+    // of DEPTH. ----
     for (int it0 = 0; it0 < n; it0 += DEPTH) {
 #pragma unroll
       for (int d = 0; d < DEPTH; ++d) {
         const int it = it0 + d;
-        if (it < n) {
-          const half_t *abuf = ldsA + (it & 1) * A_STAGE;
-          half2v sc[NB];
-          if (Q4) {
+        const half_t *abuf = ldsA + (it & 1) * A_STAGE;
+        half2v sc[NB];
+        if (Q4) {
 #pragma unroll
-            for (int j = 0; j < NB; ++j) {
-              half_t s = ldsS[((wn * NB + j) * 16 + lr) * (SC_MAX_ITERS * SC_PER_ITER) +
-                              it * SC_PER_ITER + (klane / QGROUP)];
-              sc[j] = half2v{s, s};
-            }
+          for (int j = 0; j < NB; ++j) {
+            // iterations past the segment multiply zero weights; they must still see a finite scale
+            half_t s = ldsS[((wn * NB + j) * 16 + lr) * SC_ROW + sc_shift + min(it, n - 1) * SC_PER_ITER +
+                            (klane / QGROUP)];
+            sc[j] = half2v{s, s};
           }
+        }
 #pragma unroll
-          for (int ch = 0; ch < NCH; ++ch) {
-            half8v fa[MB];
+        for (int ch = 0; ch < NCH; ++ch) {
+          half8v fa[MB];
+#pragma unroll
+          for (int i = 0; i < MB; ++i) fa[i] = *reinterpret_cast<const half8v *>(abuf + a_rd[i] + ch * 8);
+#pragma unroll
+          for (int j = 0; j < NB; ++j) {
+            half8v fw;
+            if (Q4) {
+              fw = dequant_word_q4(wreg[d][j][ch / 4][ch % 4], bias, sc[j]);
+            } else {
+              fw = __builtin_bit_cast(half8v, wreg[d][j][ch]);
+            }
 #pragma unroll
             for (int i = 0; i < MB; ++i)
-              fa[i] = *reinterpret_cast<const half8v *>(abuf + a_rd[i] + ch * 8);
-#pragma unroll
-            for (int j = 0; j < NB; ++j) {
-              half8v fw;
-              if (Q4) {
-                fw = dequant_word_q4(wreg[d][j][ch / 4][ch % 4], bias, sc[j]);
-              } else {
-                union { uint4v u; half8v h; } cv;
-                cv.u = wreg[d][j][ch];
-                fw = cv.h;
-              }
-#pragma unroll
-              for (int i = 0; i < MB; ++i)
-                acc.c[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fw, fa[i], acc.c[i][j], 0, 0, 0);
-            }
+              acc.c[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fw, fa[i], acc.c[i][j], 0, 0, 0);
           }
-          // A tile of the next iteration into the other LDS buffer, then refill this ring slot
-          if (it + 1 < n) stage_a((d + 1) % DEPTH, (it + 1) & 1);
-          if (it + DEPTH < n) issue_loads(d, k0 + it + DEPTH);
-          __syncthreads();
         }
+        // A tile of the next iteration into the other LDS buffer, then refill this ring slot
+        stage_a((d + 1) % DEPTH, (it + 1) & 1);
+        issue_loads(d, it + DEPTH);
+        __syncthreads();
       }
     }
 
