@@ -21,6 +21,7 @@ struct KernelInfo {
   int family;
   int dtype;    // sk_dtype
   int layout;   // sk_layout
+  int variant;  // 0: registers -> padded LDS rows; 1: direct global -> LDS loads, swizzled rows
   int bm, bn, bk;  // CTA tile; bk is the K extent of one CTA iteration
   int threads;
   int lds_bytes;
@@ -40,6 +41,13 @@ struct KernelInfo {
   X(4, 64, 64, 64, 2, 2)          \
   X(5, 256, 256, 32, 2, 4)        \
   X(6, 128, 128, 32, 2, 2)
+
+// fp16 LDS-tiled kernels with direct-to-LDS loads (BK = 64), NT layout:  X(id, BM, BN, WM, WN)
+#define SK_TILE_F16_NT_DMA_KERNELS(X) \
+  X(10, 256, 256, 2, 4)               \
+  X(11, 128, 128, 2, 2)               \
+  X(12, 128, 256, 2, 4)               \
+  X(13, 256, 128, 4, 2)
 
 // small-M kernels:  X(id, MB, NB, WN, RK, Q4, DEPTH)
 #define SK_SKINNY_KERNELS(X)  \

@@ -17,7 +17,7 @@ int skinny_kernel_infos(KernelInfo *out, int max) {
 #define X(id, MB, NB, WN, RK, Q4, DEPTH)                                                           \
   if (n < max) {                                                                                   \
     typedef SK_POLICY(MB, NB, WN, RK, Q4, DEPTH) P;                                                \
-    out[n++] = KernelInfo{id, FAMILY_SKINNY, (Q4) ? 2 : 0, 0, P::BM, P::BN, P::BKC, P::NT,         \
+    out[n++] = KernelInfo{id, FAMILY_SKINNY, (Q4) ? 2 : 0, 0, 0, P::BM, P::BN, P::BKC, P::NT,         \
                           P::LDS_BYTES, P::CTAS_PER_CU, P::TILE_ELEMS, (Q4) ? P::SC_MAX_ITERS : 0, (Q4) ? 128 : 8, \
                           (Q4) ? "skinny_q4_mb" #MB "_wn" #WN "_rk" #RK                            \
                                : "skinny_f16_mb" #MB "_wn" #WN "_rk" #RK};                         \

@@ -5,6 +5,7 @@
 #include "kernel_table.h"
 #include "sk_device.h"
 #include "tile_f16.h"
+#include "tile_f16_dma.h"
 #include "tile_skinny.h"
 
 namespace sk {

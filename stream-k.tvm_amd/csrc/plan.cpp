@@ -42,12 +42,16 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
   int n;
   const KernelInfo *t = kernel_table(&n);
   const bool want_tile = cfg && cfg->bm > 0 && cfg->bn > 0;
+  // cfg->reserved[0]: 0 = newest variant of the tile, v > 0 = variant v - 1
+  const int want_variant = cfg ? cfg->reserved[0] - 1 : -1;
   if (want_tile) {
+    const KernelInfo *found = nullptr;
     for (int i = 0; i < n; ++i)
       if (t[i].dtype == dtype && t[i].layout == layout && t[i].bm == cfg->bm && t[i].bn == cfg->bn &&
-          (cfg->bk <= 0 || t[i].bk == cfg->bk))
-        return &t[i];
-    return nullptr;
+          (cfg->bk <= 0 || t[i].bk == cfg->bk) && (want_variant < 0 || t[i].variant == want_variant) &&
+          (found == nullptr || t[i].variant > found->variant))
+        found = &t[i];
+    return found;
   }
   // heuristic: small M -> weight-streaming kernels; otherwise the largest tile that still gives
   // every CU something to do
@@ -67,10 +71,11 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
     for (int i = 0; i < n; ++i) {
       if (t[i].family != FAMILY_TILE || t[i].dtype != dtype || t[i].layout != layout) continue;
       if (t[i].bm != p[0] || t[i].bn != p[1] || t[i].bk != p[2]) continue;
+      if (want_variant >= 0 ? t[i].variant != want_variant : (best != nullptr && t[i].variant < best->variant)) continue;
       int64_t tiles = cdiv(M, p[0]) * cdiv(N, p[1]);
       int64_t iters = tiles * cdiv(K, p[2]);
       // enough K-iterations per CU that a split tile still amortises its fix-up
-      if (best == nullptr && (tiles >= num_cus || iters >= (int64_t)num_cus * 16 || p[0] == 64)) best = &t[i];
+      if (tiles >= num_cus || iters >= (int64_t)num_cus * 16 || p[0] == 64) best = &t[i];
     }
     if (best) break;
   }

@@ -104,6 +104,26 @@ __device__ __forceinline__ uint4v buffer_load_16(BufferRsrc r, uint32_t lane_off
 }
 constexpr uint32_t OOB_OFFSET = 0x80000000u;
 
+// Direct global -> LDS load, 16 bytes per lane: lane l's data lands at lds_base + 16*l.  Issued as
+// inline assembly on purpose: the compiler's wait-count insertion cannot tell which LDS stage an
+// in-flight load writes and would otherwise stall every LDS read on all of them.  The kernels
+// that use this wait (vmcnt) and barrier by hand.  lds_base, rsrc and uniform_off are
+// wave-uniform.
+__device__ __forceinline__ uint4v make_rsrc_words(const void *base, uint32_t num_bytes) {
+  const uint64_t b = reinterpret_cast<uint64_t>(base);
+  return uint4v{(uint32_t)b, (uint32_t)(b >> 32) & 0xffffu, num_bytes, 0x00020000u};
+}
+__device__ __forceinline__ void dma_load_16(uint4v rsrc, uint32_t lds_base, uint32_t lane_off,
+                                            uint32_t uniform_off) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :
+               : "s"(lds_base), "v"(lane_off), "s"(rsrc), "s"(uniform_off)
+               : "memory", "m0");
+}
+__device__ __forceinline__ uint32_t lds_address(const void *p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)p;
+}
+
 // Makes a pointer opaque to the optimiser at this program point.  The fix-up paths address dozens
 // of far-apart float4 slots per thread; without this the address arithmetic is hoisted out of the
 // persistent loop and kept in registers across the MFMA main loop.

@@ -34,6 +34,7 @@ struct TileF16NT {
   static constexpr int LDS_STAGING = 2 * STAGE * 2;
   static constexpr int LDS_EPILOGUE = WM * WN * WTM * LDC * 2;
   static constexpr int LDS_BYTES = LDS_STAGING > LDS_EPILOGUE ? LDS_STAGING : LDS_EPILOGUE;
+  static constexpr int LDS_TOTAL = LDS_BYTES;
   static constexpr int TILE_ELEMS = BM * BN;
   static constexpr int NV4 = TM * TN * 4;  // float4 groups per thread
   // co-resident CTAs per CU the kernel is compiled for (register budget = 512 / waves per SIMD)
@@ -102,20 +103,34 @@ struct TileF16NT {
         *reinterpret_cast<uint4v *>(st + A_STAGE + lds_st + i * ROWS_PER_PASS * LDK) = rb[i];
       __syncthreads();
       if (it + 1 < n) load_global(k0 + it + 1);
-#pragma unroll
-      for (int kk = 0; kk < BK / 16; ++kk) {
-        half8v fa[TM], fb[TN];
+      // fragments are double-buffered in registers: the ds_reads of K-step kk+1 are issued before
+      // the MFMAs of step kk so that LDS latency hides behind the matrix pipe
+      half8v fa[2][TM], fb[2][TN];
+      auto read_frags = [&](int buf, int kk) {
 #pragma unroll
         for (int i = 0; i < TM; ++i)
-          fa[i] = *reinterpret_cast<const half8v *>(st + a_rd + i * 32 * LDK + kk * 16);
+          fa[buf][i] = *reinterpret_cast<const half8v *>(st + a_rd + i * 32 * LDK + kk * 16);
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-          fb[j] = *reinterpret_cast<const half8v *>(st + b_rd + j * 32 * LDK + kk * 16);
+          fb[buf][j] = *reinterpret_cast<const half8v *>(st + b_rd + j * 32 * LDK + kk * 16);
+      };
+      read_frags(0, 0);
+#pragma unroll
+      for (int kk = 0; kk < BK / 16; ++kk) {
+        if (kk + 1 < BK / 16) read_frags((kk + 1) & 1, kk + 1);
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
           for (int j = 0; j < TN; ++j)
-            acc.c[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[j], fa[i], acc.c[i][j], 0, 0, 0);
+            acc.c[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[kk & 1][j], fa[kk & 1][i], acc.c[i][j], 0, 0, 0);
+        // one DS read per MFMA keeps the order above through instruction scheduling
+        if (kk + 1 < BK / 16) {
+#pragma unroll
+          for (int g = 0; g < TM + TN; ++g) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          }
+        }
       }
     }
     __syncthreads();  // staging buffers are free again (next segment or the epilogue may write)

@@ -1,0 +1,233 @@
+// fp16 NT tile arithmetic with direct global->LDS loads (buffer_load ... lds, 16 bytes per lane),
+// XOR-swizzled LDS rows and a two-stage software pipeline.  BK is fixed at 64 (one LDS row = 128
+// bytes = 8 chunks of 16 bytes).
+//
+// LDS layout of one stage: BM rows of A then BN rows of B, 128 bytes each; chunk c of row r lives
+// at chunk position c ^ (r & 7) (the reference swizzles its 64-byte rows the same way,
+// streamk_fp16.py:72-80).  A wave-wide DMA instruction fills 1 KB = 8 consecutive rows: lane l
+// writes position (row l/8, chunk l%8) and therefore fetches global chunk (l%8) ^ (l/8) -- a
+// per-lane constant, so one VGPR offset per operand serves every load.
+//
+// Pipeline per K-iteration (stage `cur` holds the iteration's tiles, `nxt` the next one's):
+//   K-steps 0..2:  wait fragments(kk) | issue ds_reads(kk+1) | 8 MFMAs(kk)
+//   K-step 3:      wait fragments(3)  | wait own DMA(nxt), barrier
+//                  | issue DMA(cur <- iteration+2), ds_reads(nxt, 0) | 8 MFMAs(3)
+// so the barrier, the DMA issue and the first fragment reads of the next iteration all overlap
+// with the last MFMA block.
+#pragma once
+#include "sk_device.h"
+#include "tile_f16.h"
+
+namespace sk {
+
+// one LDS array per (size, id): distinct arrays let the compiler tell the stages apart when it
+// orders LDS reads against in-flight DMA writes
+template <int BYTES, int ID>
+struct LdsArray {
+  static __device__ __forceinline__ char *get() {
+    __shared__ __attribute__((aligned(1024))) char buf[BYTES];
+    return buf;
+  }
+};
+
+template <int BM_, int BN_, int WM_, int WN_>
+struct TileF16NTDma {
+  typedef GemmArgs Args;
+  static constexpr int BM = BM_, BN = BN_, BK = 64, WM = WM_, WN = WN_;
+  static constexpr int NW = WM * WN, NT = NW * 64;
+  static constexpr int TM = BM / (WM * 32), TN = BN / (WN * 32);
+  static constexpr int WTM = TM * 32, WTN = TN * 32;
+  static constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE_BYTES = A_BYTES + B_BYTES;
+  static constexpr int A_DMA = BM / 8 / NW, B_DMA = BN / 8 / NW, DMA_PER_WAVE = A_DMA + B_DMA;
+  static constexpr int LDC = WTN + 8;
+  // epilogue patches: waves [0, NW/2) use stage 0, the others stage 1; split the wave tile's rows
+  // into passes until the patches fit
+  static constexpr int patch_passes() {
+    int p = 1;
+    while ((NW / 2) * (WTM / p) * LDC * 2 > STAGE_BYTES) p *= 2;
+    return p;
+  }
+  static constexpr int PASSES = patch_passes();
+  static constexpr int PATCH_ROWS = WTM / PASSES;
+  static constexpr int LDS_BYTES = 16;  // the kernel's generic buffer is unused
+  static constexpr int LDS_TOTAL = 2 * STAGE_BYTES;
+  static constexpr int TILE_ELEMS = BM * BN;
+  static constexpr int NV4 = TM * TN * 4;
+  static constexpr int CTAS_PER_CU_REGS = NT >= 512 ? 1 : 2;
+  static constexpr int CTAS_PER_CU_LDS = (160 * 1024) / (LDS_TOTAL + 64);
+  static constexpr int CTAS_PER_CU = CTAS_PER_CU_REGS < CTAS_PER_CU_LDS ? CTAS_PER_CU_REGS : CTAS_PER_CU_LDS;
+  static constexpr int WAVES_PER_EU = CTAS_PER_CU * (NT / 64) / 4 > 0 ? CTAS_PER_CU * (NT / 64) / 4 : 1;
+  static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "tile shape");
+  static_assert((BM / 8) % NW == 0 && (BN / 8) % NW == 0, "DMA groups must divide over the waves");
+  static_assert(PATCH_ROWS % 32 == 0, "epilogue pass must hold whole 32-row blocks");
+
+  typedef TileF16NT<BM_, BN_, 64, WM_, WN_> Base;  // shares the accumulator type and the partials
+  typedef typename Base::Acc Acc;
+
+  static __device__ __forceinline__ char *stage(int s) {
+    return s == 0 ? LdsArray<STAGE_BYTES, 0>::get() : LdsArray<STAGE_BYTES, 1>::get();
+  }
+
+  template <int N>
+  static __device__ __forceinline__ void wait_dma_then_barrier() {
+    // own DMA writes of the awaited stage have landed (at most N younger loads still in flight),
+    // then everybody's have.  "memory": nothing may be moved across by the compiler.
+    if (N == 0)
+      asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
+  }
+
+  static __device__ __forceinline__ void mac(const Args &a, Acc &acc, int pm, int pn, int k0, int n,
+                                             char *) {
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc.c[i][j][r] = 0.f;
+
+    const int rows_a = min(BM, a.M - pm * BM), rows_b = min(BN, a.N - pn * BN);
+    const uint4v rsrc_a = make_rsrc_words(a.A + (int64_t)pm * BM * a.lda, (uint32_t)(rows_a * a.lda * 2));
+    const uint4v rsrc_b = make_rsrc_words(a.B + (int64_t)pn * BN * a.ldb, (uint32_t)(rows_b * a.ldb * 2));
+    const int my_chunk = (lane & 7) ^ (lane >> 3);  // global chunk this lane fetches
+    const uint32_t voff_a = (uint32_t)((lane >> 3) * a.lda + my_chunk * 8) * 2;
+    const uint32_t voff_b = (uint32_t)((lane >> 3) * a.ldb + my_chunk * 8) * 2;
+    const uint32_t grp_a = (uint32_t)(8 * a.lda * 2), grp_b = (uint32_t)(8 * a.ldb * 2);
+    const int tail_kt = (a.K % BK != 0) ? (a.K / BK) : -1;
+
+    auto issue_dma = [&](char *st, int kt) {
+      const uint32_t koff = (uint32_t)kt * (BK * 2);
+      uint32_t va = voff_a, vb = voff_b;
+      if (kt == tail_kt && kt * BK + my_chunk * 8 >= a.K) va = vb = OOB_OFFSET;
+#pragma unroll
+      for (int j = 0; j < A_DMA; ++j) {
+        const int g = wave + j * NW;
+        dma_load_16(rsrc_a, lds_address(st) + g * 1024, va, koff + g * grp_a);
+      }
+#pragma unroll
+      for (int j = 0; j < B_DMA; ++j) {
+        const int g = wave + j * NW;
+        dma_load_16(rsrc_b, lds_address(st) + A_BYTES + g * 1024, vb, koff + g * grp_b);
+      }
+    };
+
+    // fragment addressing: lane (r = lane%32, g = lane/32) reads row r of a 32-row block, logical
+    // chunk 2*kk + g, stored at chunk position (2*kk + g) ^ (r & 7)
+    int rd_a[4], rd_b[4];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      const int pos = ((2 * kk + (lane >> 5)) ^ (lane & 7)) * 16;
+      rd_a[kk] = (wm * WTM + (lane & 31)) * 128 + pos;
+      rd_b[kk] = A_BYTES + (wn * WTN + (lane & 31)) * 128 + pos;
+    }
+    half8v fa[2][TM], fb[2][TN];
+    auto read_frags = [&](const char *st, int buf, int kk) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i) fa[buf][i] = *reinterpret_cast<const half8v *>(st + rd_a[kk] + i * 4096);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) fb[buf][j] = *reinterpret_cast<const half8v *>(st + rd_b[kk] + j * 4096);
+    };
+    auto mfma_step = [&](int buf) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc.c[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[buf][j], fa[buf][i], acc.c[i][j], 0, 0, 0);
+    };
+    // one K-iteration on stage `cur`; `more1`/`more2`: iterations it+1 / it+2 exist
+    auto iteration = [&](char *cur, char *nxt, int it) {
+#pragma unroll
+      for (int kk = 0; kk < 3; ++kk) {
+        read_frags(cur, (kk + 1) & 1, kk + 1);
+        mfma_step(kk & 1);
+#pragma unroll
+        for (int g = 0; g < TM + TN; ++g) {
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        }
+      }
+      // every read of `cur` has been issued; they complete before the barrier below because the
+      // MFMAs of step 3 (which need them) follow it -- make that explicit for the hardware:
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      wait_dma_then_barrier<0>();
+      if (it + 2 < n) issue_dma(cur, k0 + it + 2);
+      if (it + 1 < n) read_frags(nxt, 0, 0);
+      mfma_step(1);
+    };
+
+    char *s0 = stage(0), *s1 = stage(1);
+    issue_dma(s0, k0);
+    wait_dma_then_barrier<0>();
+    if (n > 1) issue_dma(s1, k0 + 1);
+    read_frags(s0, 0, 0);
+    int it = 0;
+    for (; it + 1 < n; it += 2) {
+      iteration(s0, s1, it);
+      iteration(s1, s0, it + 1);
+    }
+    if (it < n) iteration(s0, s1, it);
+    // all LDS reads are complete and every wave has passed the last barrier only after finishing
+    // its reads of the other stage; one more barrier frees both stages for the epilogue / next tile
+    __syncthreads();
+  }
+
+  static __device__ __forceinline__ void store_c(const Args &a, const Acc &acc, int pm, int pn, char *) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    half_t *patch = reinterpret_cast<half_t *>(wave < NW / 2 ? stage(0) : stage(1)) +
+                    (wave % (NW / 2)) * (PATCH_ROWS * LDC);
+    const bool vec_ok = (a.ldc % 8 == 0) && ((reinterpret_cast<uintptr_t>(a.C) & 15) == 0);
+    constexpr int CPRC = WTN / 8;
+    constexpr int BLK = PATCH_ROWS / 32;  // 32-row blocks per pass
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+#pragma unroll
+      for (int ib = 0; ib < BLK; ++ib)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            half4v h;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) h[e] = (half_t)acc.c[p * BLK + ib][j][q * 4 + e];
+            *reinterpret_cast<half4v *>(patch + (ib * 32 + (lane & 31)) * LDC + j * 32 + q * 8 +
+                                        (lane >> 5) * 4) = h;
+          }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      const int row0 = pm * BM + wm * WTM + p * PATCH_ROWS, col0 = pn * BN + wn * WTN;
+#pragma unroll
+      for (int s = 0; s < PATCH_ROWS * CPRC / 64; ++s) {
+        const int idx = s * 64 + lane;
+        const int r = idx / CPRC, cc = idx % CPRC;
+        const int grow = row0 + r, gcol = col0 + cc * 8;
+        if (grow < a.M && gcol < a.N) {
+          const half_t *src = patch + r * LDC + cc * 8;
+          half_t *dst = a.C + (int64_t)grow * a.ldc + gcol;
+          if (vec_ok && gcol + 8 <= a.N) {
+            *reinterpret_cast<uint4v *>(dst) = *reinterpret_cast<const uint4v *>(src);
+          } else {
+            for (int e = 0; e < 8 && gcol + e < a.N; ++e) dst[e] = src[e];
+          }
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+    __syncthreads();  // patches overlap the stages of the next tile
+  }
+
+  static __device__ __forceinline__ void store_partial(const Acc &acc, float *dst) { Base::store_partial(acc, dst); }
+  static __device__ __forceinline__ void add_partial(Acc &acc, const float *src) { Base::add_partial(acc, src); }
+  static __device__ __forceinline__ void atomic_partial(const Acc &acc, float *dst) { Base::atomic_partial(acc, dst); }
+  static __device__ __forceinline__ void take_partial(Acc &acc, float *src) { Base::take_partial(acc, src); }
+};
+
+}  // namespace sk

@@ -53,6 +53,7 @@ struct TileSkinny {
   static constexpr int LDS_SC = Q4 ? BN * SC_ROW * 2 : 0;
   static constexpr int LDS_RED = RK > 1 ? (RK - 1) * WN * 64 * MB * NB * 16 : 0;
   static constexpr int LDS_BYTES = LDS_A + LDS_SC + LDS_RED;
+  static constexpr int LDS_TOTAL = LDS_BYTES;
   // partials are held by the rk == 0 waves only
   static constexpr int TILE_ELEMS = BM * BN;
   static constexpr int NTP = WN * 64;

@@ -33,6 +33,9 @@ def make_config(config=None, **kw):
             v = _lib.SCHEDULES[v] if isinstance(v, str) else int(v)
         elif k == "fixup":
             v = _lib.FIXUPS[v] if isinstance(v, str) else int(v)
+        if k == "variant":  # 0 = newest kernel variant of the tile, v > 0 = variant v - 1
+            c.reserved[0] = int(v)
+            continue
         if k not in ("bm", "bn", "bk", "grid", "schedule", "fixup", "raster", "spin_limit"):
             raise KeyError(f"unknown Stream-K config key {k!r}")
         setattr(c, k, int(v))
