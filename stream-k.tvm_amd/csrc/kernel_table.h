@@ -21,7 +21,8 @@ struct KernelInfo {
   int family;
   int dtype;    // sk_dtype
   int layout;   // sk_layout
-  int variant;  // 0: registers -> padded LDS rows; 1: direct global -> LDS loads, swizzled rows
+  int variant;  // 0: registers -> padded LDS rows; 1: direct global -> LDS loads, swizzled rows;
+                // 2: as 1 with four waves per CTA (one per SIMD, accumulators in AGPRs)
   int bm, bn, bk;  // CTA tile; bk is the K extent of one CTA iteration
   int threads;
   int lds_bytes;
@@ -47,7 +48,8 @@ struct KernelInfo {
   X(10, 256, 256, 2, 4)               \
   X(11, 128, 128, 2, 2)               \
   X(12, 128, 256, 2, 4)               \
-  X(13, 256, 128, 4, 2)
+  X(13, 256, 128, 4, 2)               \
+  X(14, 256, 256, 2, 2)
 
 // small-M kernels:  X(id, MB, NB, WN, RK, Q4, DEPTH)
 #define SK_SKINNY_KERNELS(X)  \

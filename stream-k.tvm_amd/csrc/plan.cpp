@@ -37,6 +37,9 @@ const KernelInfo *kernel_by_id(int id) {
 
 static int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// preference among kernel variants of one tile shape when the caller does not ask for one
+static int variant_rank(int v) { return v == 1 ? 2 : (v == 2 ? 1 : 0); }
+
 static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype, int layout,
                                      const sk_config *cfg, int num_cus) {
   int n;
@@ -49,7 +52,7 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
     for (int i = 0; i < n; ++i)
       if (t[i].dtype == dtype && t[i].layout == layout && t[i].bm == cfg->bm && t[i].bn == cfg->bn &&
           (cfg->bk <= 0 || t[i].bk == cfg->bk) && (want_variant < 0 || t[i].variant == want_variant) &&
-          (found == nullptr || t[i].variant > found->variant))
+          (found == nullptr || variant_rank(t[i].variant) > variant_rank(found->variant)))
         found = &t[i];
     return found;
   }
@@ -71,7 +74,7 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
     for (int i = 0; i < n; ++i) {
       if (t[i].family != FAMILY_TILE || t[i].dtype != dtype || t[i].layout != layout) continue;
       if (t[i].bm != p[0] || t[i].bn != p[1] || t[i].bk != p[2]) continue;
-      if (want_variant >= 0 ? t[i].variant != want_variant : (best != nullptr && t[i].variant < best->variant)) continue;
+      if (want_variant >= 0 ? t[i].variant != want_variant : (best != nullptr && variant_rank(t[i].variant) < variant_rank(best->variant))) continue;
       int64_t tiles = cdiv(M, p[0]) * cdiv(N, p[1]);
       int64_t iters = tiles * cdiv(K, p[2]);
       // enough K-iterations per CU that a split tile still amortises its fix-up

@@ -3,10 +3,14 @@
 // bytes = 8 chunks of 16 bytes).
 //
 // LDS layout of one stage: BM rows of A then BN rows of B, 128 bytes each; chunk c of row r lives
-// at chunk position c ^ (r & 7) (the reference swizzles its 64-byte rows the same way,
-// streamk_fp16.py:72-80).  A wave-wide DMA instruction fills 1 KB = 8 consecutive rows: lane l
-// writes position (row l/8, chunk l%8) and therefore fetches global chunk (l%8) ^ (l/8) -- a
-// per-lane constant, so one VGPR offset per operand serves every load.
+// at chunk position c ^ ((r >> 1) & 7) (XOR swizzle in the spirit of the reference's,
+// streamk_fp16.py:72-80).  With 64 four-byte banks and 16 lanes served per cycle, rows r and r+1
+// fall in different bank halves and (r >> 1) spreads the 8 row pairs over the 8 chunk positions:
+// measured conflict-free for the 32-row fragment reads (r & 7 is 2-way conflicted).
+// A wave-wide DMA instruction fills 1 KB = 8 consecutive rows: lane l writes position
+// (row 8*G + l/8, chunk l%8) of row group G and therefore fetches global chunk
+// (l%8) ^ (4*(G&1) + l/16).  A wave only ever loads groups of its own parity, so this is a
+// per-lane constant and one VGPR offset per operand serves every load.
 //
 // Pipeline per K-iteration (stage `cur` holds the iteration's tiles, `nxt` the next one's):
 //   K-steps 0..2:  wait fragments(kk) | issue ds_reads(kk+1) | 8 MFMAs(kk)
@@ -53,12 +57,13 @@ struct TileF16NTDma {
   static constexpr int LDS_TOTAL = 2 * STAGE_BYTES;
   static constexpr int TILE_ELEMS = BM * BN;
   static constexpr int NV4 = TM * TN * 4;
-  static constexpr int CTAS_PER_CU_REGS = NT >= 512 ? 1 : 2;
+  static constexpr int CTAS_PER_CU_REGS = (NT >= 512 || TM * TN > 4) ? 1 : 2;
   static constexpr int CTAS_PER_CU_LDS = (160 * 1024) / (LDS_TOTAL + 64);
   static constexpr int CTAS_PER_CU = CTAS_PER_CU_REGS < CTAS_PER_CU_LDS ? CTAS_PER_CU_REGS : CTAS_PER_CU_LDS;
   static constexpr int WAVES_PER_EU = CTAS_PER_CU * (NT / 64) / 4 > 0 ? CTAS_PER_CU * (NT / 64) / 4 : 1;
   static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "tile shape");
   static_assert((BM / 8) % NW == 0 && (BN / 8) % NW == 0, "DMA groups must divide over the waves");
+  static_assert(NW % 2 == 0, "a wave must keep to row groups of one parity");
   static_assert(PATCH_ROWS % 32 == 0, "epilogue pass must hold whole 32-row blocks");
 
   typedef TileF16NT<BM_, BN_, 64, WM_, WN_> Base;  // shares the accumulator type and the partials
@@ -94,7 +99,7 @@ struct TileF16NTDma {
     const int rows_a = min(BM, a.M - pm * BM), rows_b = min(BN, a.N - pn * BN);
     const uint4v rsrc_a = make_rsrc_words(a.A + (int64_t)pm * BM * a.lda, (uint32_t)(rows_a * a.lda * 2));
     const uint4v rsrc_b = make_rsrc_words(a.B + (int64_t)pn * BN * a.ldb, (uint32_t)(rows_b * a.ldb * 2));
-    const int my_chunk = (lane & 7) ^ (lane >> 3);  // global chunk this lane fetches
+    const int my_chunk = (lane & 7) ^ (((wave & 1) << 2) | (lane >> 4));  // global chunk this lane fetches
     const uint32_t voff_a = (uint32_t)((lane >> 3) * a.lda + my_chunk * 8) * 2;
     const uint32_t voff_b = (uint32_t)((lane >> 3) * a.ldb + my_chunk * 8) * 2;
     const uint32_t grp_a = (uint32_t)(8 * a.lda * 2), grp_b = (uint32_t)(8 * a.ldb * 2);
@@ -117,11 +122,11 @@ struct TileF16NTDma {
     };
 
     // fragment addressing: lane (r = lane%32, g = lane/32) reads row r of a 32-row block, logical
-    // chunk 2*kk + g, stored at chunk position (2*kk + g) ^ (r & 7)
+    // chunk 2*kk + g, stored at chunk position (2*kk + g) ^ ((r >> 1) & 7)
     int rd_a[4], rd_b[4];
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
-      const int pos = ((2 * kk + (lane >> 5)) ^ (lane & 7)) * 16;
+      const int pos = ((2 * kk + (lane >> 5)) ^ ((lane >> 1) & 7)) * 16;
       rd_a[kk] = (wm * WTM + (lane & 31)) * 128 + pos;
       rd_b[kk] = A_BYTES + (wn * WTN + (lane & 31)) * 128 + pos;
     }

@@ -42,10 +42,14 @@ def _rel(oracle, C, ref):
     return oracle.max_abs_rel(C.float().cpu().numpy(), ref)
 
 
+# variant 1: registers -> padded LDS rows; 2: direct-to-LDS, 8 (4) waves; 3: direct-to-LDS 256x256 on 4 waves
 TILE_CONFIGS = [
-    dict(bm=128, bn=128, bk=64), dict(bm=256, bn=256, bk=64), dict(bm=128, bn=256, bk=64),
-    dict(bm=256, bn=128, bk=64), dict(bm=64, bn=64, bk=64), dict(bm=256, bn=256, bk=32),
-    dict(bm=128, bn=128, bk=32),
+    dict(bm=128, bn=128, bk=64, variant=1), dict(bm=256, bn=256, bk=64, variant=1),
+    dict(bm=128, bn=256, bk=64, variant=1), dict(bm=256, bn=128, bk=64, variant=1),
+    dict(bm=64, bn=64, bk=64), dict(bm=256, bn=256, bk=32), dict(bm=128, bn=128, bk=32),
+    dict(bm=128, bn=128, bk=64, variant=2), dict(bm=256, bn=256, bk=64, variant=2),
+    dict(bm=128, bn=256, bk=64, variant=2), dict(bm=256, bn=128, bk=64, variant=2),
+    dict(bm=256, bn=256, bk=64, variant=3),
 ]
 SKINNY_CONFIGS = [
     dict(bm=16, bn=64, bk=128), dict(bm=32, bn=64, bk=128), dict(bm=64, bn=64, bk=128),
@@ -53,7 +57,7 @@ SKINNY_CONFIGS = [
 ]
 
 
-@pytest.mark.parametrize("cfg", TILE_CONFIGS + SKINNY_CONFIGS, ids=lambda c: f"{c['bm']}x{c['bn']}x{c['bk']}")
+@pytest.mark.parametrize("cfg", TILE_CONFIGS + SKINNY_CONFIGS, ids=lambda c: f"{c['bm']}x{c['bn']}x{c['bk']}v{c.get('variant', 0)}")
 @pytest.mark.parametrize("sched,fixup,grid", [("dp", "reduce", 8), ("basic", "reduce", 8),
                                              ("basic", "atomic", 8), ("sk2", "reduce", 3),
                                              ("sk2", "atomic", 5)])
