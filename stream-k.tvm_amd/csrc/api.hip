@@ -237,7 +237,7 @@ __global__ void dequant_q4_kernel(const uint32_t *wq, const half_t *scales, half
   const int64_t row = i / words_per_row;
   const int k = (int)(i % words_per_row) * 8;
   const half_t s = scales[row * groups + k / group];
-  const half8v v = dequant_word_q4(wq[i], q4_bias(zero), half2v{s, s});
+  const half8v v = dequant_word_q4(wq[i], q4_consts(zero), half2v{s, s});
   half8v o;
 #pragma unroll
   for (int e = 0; e < 8; ++e) o[e] = v[q4_slot_of_element(e)];

@@ -29,6 +29,7 @@ struct KernelInfo {
   int ctas_per_cu;    // co-resident CTAs per CU the kernel is compiled for
   int partial_elems;  // fp32 elements of one partial tile in the workspace
   int max_ipt;        // largest iterations-per-tile the kernel supports (0 = unlimited)
+  int max_m;          // small-M kernels: largest M the kernel accepts
   int k_align;        // K must be a multiple of this
   const char *name;
 };
@@ -51,18 +52,26 @@ struct KernelInfo {
   X(13, 256, 128, 4, 2)               \
   X(14, 256, 256, 2, 2)
 
-// small-M kernels:  X(id, MB, NB, WN, RK, Q4, DEPTH)
-#define SK_SKINNY_KERNELS(X)  \
-  X(100, 1, 1, 4, 1, 0, 2)    \
-  X(101, 2, 1, 4, 1, 0, 2)    \
-  X(102, 4, 1, 4, 1, 0, 2)    \
-  X(103, 1, 1, 1, 4, 0, 2)    \
-  X(104, 1, 1, 2, 2, 0, 2)    \
-  X(120, 1, 1, 4, 1, 1, 4)    \
-  X(121, 2, 1, 4, 1, 1, 2)    \
-  X(122, 4, 1, 4, 1, 1, 2)    \
-  X(123, 1, 1, 1, 4, 1, 4)    \
-  X(124, 1, 1, 2, 2, 1, 4)
+// small-M kernels:  X(id, MB, NB, WN, RK, Q4, DEPTH, ROW1)
+#define SK_SKINNY_KERNELS(X)     \
+  X(100, 1, 1, 4, 1, 0, 2, 0)    \
+  X(101, 2, 1, 4, 1, 0, 2, 0)    \
+  X(102, 4, 1, 4, 1, 0, 2, 0)    \
+  X(103, 1, 1, 1, 4, 0, 2, 0)    \
+  X(104, 1, 1, 2, 2, 0, 2, 0)    \
+  X(105, 1, 1, 1, 1, 0, 4, 1)    \
+  X(106, 1, 1, 4, 1, 0, 4, 1)    \
+  X(120, 1, 1, 4, 1, 1, 4, 0)    \
+  X(121, 2, 1, 4, 1, 1, 2, 0)    \
+  X(122, 4, 1, 4, 1, 1, 2, 0)    \
+  X(123, 1, 1, 1, 4, 1, 4, 0)    \
+  X(124, 1, 1, 2, 2, 1, 4, 0)    \
+  X(125, 1, 1, 1, 1, 1, 4, 1)    \
+  X(126, 1, 1, 4, 1, 1, 4, 1)    \
+  X(127, 1, 2, 1, 1, 1, 4, 1)    \
+  X(128, 1, 2, 2, 1, 1, 4, 1)    \
+  X(129, 1, 4, 1, 1, 1, 2, 1)    \
+  X(130, 1, 2, 1, 2, 1, 4, 1)
 
 const KernelInfo *kernel_table(int *count);
 const KernelInfo *kernel_by_id(int id);

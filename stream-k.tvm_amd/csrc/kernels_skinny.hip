@@ -10,17 +10,18 @@ __global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_skinny_kernel(typen
   run_persistent<P>(a, plan, ws, smem);
 }
 
-#define SK_POLICY(MB, NB, WN, RK, Q4, DEPTH) TileSkinny<MB, NB, WN, RK, (Q4) != 0, DEPTH>
+#define SK_POLICY(MB, NB, WN, RK, Q4, DEPTH, ROW1) TileSkinny<MB, NB, WN, RK, (Q4) != 0, DEPTH, (ROW1) != 0>
 
 int skinny_kernel_infos(KernelInfo *out, int max) {
   int n = 0;
-#define X(id, MB, NB, WN, RK, Q4, DEPTH)                                                           \
+#define X(id, MB, NB, WN, RK, Q4, DEPTH, ROW1)                                                         \
   if (n < max) {                                                                                   \
-    typedef SK_POLICY(MB, NB, WN, RK, Q4, DEPTH) P;                                                \
-    out[n++] = KernelInfo{id, FAMILY_SKINNY, (Q4) ? 2 : 0, 0, 0, P::BM, P::BN, P::BKC, P::NT,         \
-                          P::LDS_BYTES, P::CTAS_PER_CU, P::TILE_ELEMS, (Q4) ? P::SC_MAX_ITERS : 0, (Q4) ? 128 : 8, \
-                          (Q4) ? "skinny_q4_mb" #MB "_wn" #WN "_rk" #RK                            \
-                               : "skinny_f16_mb" #MB "_wn" #WN "_rk" #RK};                         \
+    typedef SK_POLICY(MB, NB, WN, RK, Q4, DEPTH, ROW1) P;                                                \
+    out[n++] = KernelInfo{id, FAMILY_SKINNY, (Q4) ? 2 : 0, 0, (ROW1) ? 1 : 0, P::BM, P::BN, P::BKC, P::NT, \
+                          P::LDS_BYTES, P::CTAS_PER_CU, P::TILE_ELEMS, (Q4) ? P::SC_MAX_ITERS : 0, \
+                          P::MAX_M, (Q4) ? 128 : 8,                                               \
+                          (Q4) ? "skinny_q4_mb" #MB "_wn" #WN "_rk" #RK "_row1_" #ROW1             \
+                               : "skinny_f16_mb" #MB "_wn" #WN "_rk" #RK "_row1_" #ROW1};          \
   }
   SK_SKINNY_KERNELS(X)
 #undef X
@@ -29,9 +30,9 @@ int skinny_kernel_infos(KernelInfo *out, int max) {
 
 int launch_skinny(int id, const SkinnyArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s) {
   switch (id) {
-#define X(id_, MB, NB, WN, RK, Q4, DEPTH)                                                  \
+#define X(id_, MB, NB, WN, RK, Q4, DEPTH, ROW1)                                                \
   case id_: {                                                                              \
-    typedef SK_POLICY(MB, NB, WN, RK, Q4, DEPTH) P;                                        \
+    typedef SK_POLICY(MB, NB, WN, RK, Q4, DEPTH, ROW1) P;                                        \
     hipLaunchKernelGGL(sk_skinny_kernel<P>, dim3(p.grid), dim3(P::NT), 0, s, a, p, ws);    \
     return (int)hipGetLastError();                                                         \
   }
@@ -44,9 +45,9 @@ int launch_skinny(int id, const SkinnyArgs &a, const DevPlan &p, const Workspace
 int occupancy_skinny(int id) {
   int occ = 0;
   switch (id) {
-#define X(id_, MB, NB, WN, RK, Q4, DEPTH)                                                             \
+#define X(id_, MB, NB, WN, RK, Q4, DEPTH, ROW1)                                                           \
   case id_: {                                                                                         \
-    typedef SK_POLICY(MB, NB, WN, RK, Q4, DEPTH) P;                                                   \
+    typedef SK_POLICY(MB, NB, WN, RK, Q4, DEPTH, ROW1) P;                                                   \
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_skinny_kernel<P>, P::NT, 0) != hipSuccess) \
       return -1;                                                                                      \
     return occ;                                                                                       \

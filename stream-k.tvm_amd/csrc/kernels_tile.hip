@@ -19,7 +19,7 @@ int tile_kernel_infos(KernelInfo *out, int max) {
   if (n < max) {                                                                                    \
     typedef SK_POLICY(id, BM, BN, BK, WM, WN) P;                                                    \
     out[n++] = KernelInfo{id, FAMILY_TILE, 0, 0, 0, BM, BN, BK, P::NT, P::LDS_TOTAL, P::CTAS_PER_CU,  \
-                          P::TILE_ELEMS, 0, 8, "tile_f16_nt_" #BM "x" #BN "x" #BK};                 \
+                          P::TILE_ELEMS, 0, 0, 8, "tile_f16_nt_" #BM "x" #BN "x" #BK};                 \
   }
   SK_TILE_F16_NT_KERNELS(X)
 #undef X
@@ -27,7 +27,7 @@ int tile_kernel_infos(KernelInfo *out, int max) {
   if (n < max) {                                                                                    \
     typedef SK_POLICY_DMA(id, BM, BN, WM, WN) P;                                                    \
     out[n++] = KernelInfo{id, FAMILY_TILE, 0, 0, (P::TM * P::TN > 8) ? 2 : 1, BM, BN, 64, P::NT, P::LDS_TOTAL, P::CTAS_PER_CU, \
-                          P::TILE_ELEMS, 0, 8, "tile_f16_nt_dma_" #BM "x" #BN "x64"};               \
+                          P::TILE_ELEMS, 0, 0, 8, "tile_f16_nt_dma_" #BM "x" #BN "x64"};               \
   }
   SK_TILE_F16_NT_DMA_KERNELS(X)
 #undef X

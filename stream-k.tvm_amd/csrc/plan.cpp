@@ -52,6 +52,7 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
     for (int i = 0; i < n; ++i)
       if (t[i].dtype == dtype && t[i].layout == layout && t[i].bm == cfg->bm && t[i].bn == cfg->bn &&
           (cfg->bk <= 0 || t[i].bk == cfg->bk) && (want_variant < 0 || t[i].variant == want_variant) &&
+          (t[i].max_m == 0 || M <= t[i].max_m) &&
           (found == nullptr || variant_rank(t[i].variant) > variant_rank(found->variant)))
         found = &t[i];
     return found;
@@ -62,10 +63,10 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
   if (M <= 64 || dtype == SK_Q4) {
     int mb = M <= 16 ? 16 : (M <= 32 ? 32 : 64);
     for (int i = 0; i < n; ++i)
-      if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].bm == mb && t[i].bn == 64) {
+      if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].bm == mb && t[i].bn == 64 &&
+          M <= t[i].max_m && (want_variant < 0 || t[i].variant == want_variant) &&
+          (best == nullptr || t[i].variant > best->variant))
         best = &t[i];
-        break;
-      }
     if (best) return best;
     if (dtype == SK_Q4) return nullptr;
   }

@@ -14,27 +14,49 @@ namespace sk {
 // One 32-bit word holds nibbles n0..n7 of elements k..k+7.  The four half2 results are
 // (n0,n4) (n1,n5) (n2,n6) (n3,n7): element order 0,4,1,5,2,6,3,7.  GEMM kernels feed the other
 // operand in the same order, so the weights never need re-packing on the host.
-__device__ __forceinline__ half8v dequant_word_q4(uint32_t w, half2v bias, half2v scale) {
+//
+// 13 VALU operations per word: one shift, four v_and_or_b32, two packed subtracts, two packed
+// FMAs, four packed multiplies.  Nibbles sitting at bits 4..7 of a half are OR-ed in place, which
+// yields 1024 + 16*q; fma(x, 1/16, -(64 + zero)) = q - zero exactly, saving the shift.
+struct Q4Consts {
+  uint32_t magic;  // 0x64006400 in a VGPR (v_and_or_b32 takes a single scalar operand)
+  half2v bias_lo;  // 1024 + zero
+  half2v bias_hi;  // -(64 + zero)
+  half2v sixteenth;
+};
+__device__ __forceinline__ Q4Consts q4_consts(int zero) {
+  Q4Consts c;
+  c.magic = 0x64006400u;
+  const half_t lo = (half_t)(float)(1024 + zero), hi = (half_t)(float)(-(64 + zero));
+  c.bias_lo = half2v{lo, lo};
+  c.bias_hi = half2v{hi, hi};
+  c.sixteenth = half2v{(half_t)0.0625f, (half_t)0.0625f};
+  return c;
+}
+__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t bits) {
+  uint32_t r;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "s"(mask), "v"(bits));
+  return r;
+}
+__device__ __forceinline__ half8v dequant_word_q4(uint32_t w, const Q4Consts &c, half2v scale) {
   union {
     uint32_t u[4];
     half2v h[4];
     half8v v;
   } r;
-  r.u[0] = (w & 0x000F000Fu) | 0x64006400u;
-  r.u[1] = ((w >> 4) & 0x000F000Fu) | 0x64006400u;
-  r.u[2] = ((w >> 8) & 0x000F000Fu) | 0x64006400u;
-  r.u[3] = ((w >> 12) & 0x000F000Fu) | 0x64006400u;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) r.h[i] = (r.h[i] - bias) * scale;
+  const uint32_t t = w >> 8;
+  r.u[0] = and_or(w, 0x000F000Fu, c.magic);
+  r.u[1] = and_or(w, 0x00F000F0u, c.magic);
+  r.u[2] = and_or(t, 0x000F000Fu, c.magic);
+  r.u[3] = and_or(t, 0x00F000F0u, c.magic);
+  r.h[0] = (r.h[0] - c.bias_lo) * scale;
+  r.h[1] = __builtin_elementwise_fma(r.h[1], c.sixteenth, c.bias_hi) * scale;
+  r.h[2] = (r.h[2] - c.bias_lo) * scale;
+  r.h[3] = __builtin_elementwise_fma(r.h[3], c.sixteenth, c.bias_hi) * scale;
   return r.v;
 }
 
 // position of logical element e (0..7) inside the vector dequant_word_q4 returns
 __device__ __forceinline__ constexpr int q4_slot_of_element(int e) { return (e & 3) * 2 + (e >> 2); }
-
-__device__ __forceinline__ half2v q4_bias(int zero) {
-  half_t b = (half_t)(float)(1024 + zero);
-  return half2v{b, b};
-}
 
 }  // namespace sk

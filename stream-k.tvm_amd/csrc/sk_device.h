@@ -61,34 +61,71 @@ __device__ __forceinline__ void tile_coords(const DevPlan &p, int tile, int &pm,
   }
 }
 
+// ---- coherent workspace access ----
+// Partial tiles and flags travel between CTAs on different XCDs, each with its own L2.  Every
+// access to them is a device-scope relaxed atomic (64 bits at most), which the hardware performs
+// coherently (write-through stores, loads that never return a stale L2 line).  That keeps the
+// fix-up free of whole-L2 write-back / invalidate operations, which cost far more than the few
+// kilobytes exchanged here and would be paid by every CTA.
+__device__ __forceinline__ void st_coherent(float *p, floatx4 v) {
+  union { floatx4 f; uint64_t u[2]; } c;
+  c.f = v;
+  __hip_atomic_store(reinterpret_cast<uint64_t *>(p), c.u[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(reinterpret_cast<uint64_t *>(p) + 1, c.u[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ floatx4 ld_coherent(const float *p) {
+  union { floatx4 f; uint64_t u[2]; } c;
+  c.u[0] = __hip_atomic_load(reinterpret_cast<const uint64_t *>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  c.u[1] = __hip_atomic_load(reinterpret_cast<const uint64_t *>(p) + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return c.f;
+}
+__device__ __forceinline__ void st_coherent(float *p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float ld_coherent_scalar(const float *p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// all of this thread's earlier memory operations have been performed (wait counters only)
+__device__ __forceinline__ void wait_own_memory_ops() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup"); }
+
 // ---- REDUCE fix-up: flags ----
-// Contributor: the barrier orders every thread's partial stores before thread 0, whose
-// device-scope release (one L2 write-back for the whole CTA) then publishes them with the flag.
+// Contributor: every thread waits for its own (write-through) partial stores, the barrier
+// collects the CTA, then thread 0 raises the flag.
 __device__ __forceinline__ void signal_partial_ready(int *flag) {
+  wait_own_memory_ops();
   __syncthreads();
-  if (threadIdx.x == 0) __hip_atomic_store(flag, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+  if (threadIdx.x == 0) __hip_atomic_store(flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Owner: thread 0 polls with relaxed loads (a poll must not invalidate caches: other CTAs on the
-// same L2 are still streaming), acquires once when the flag is up, and the barrier hands the
-// visibility on to the rest of the CTA.  Returns false if the poll limit ran out.
-__device__ __forceinline__ bool wait_partial_ready(int *flag, int spin_limit, int *lds_ok) {
-  if (threadIdx.x == 0) {
-    int ok = 0;
-    for (int i = 0; i < spin_limit; ++i) {
-      if (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) { ok = 1; break; }
-      __builtin_amdgcn_s_sleep(1);
+// CTA that owns K-iteration `iter` of the Stream-K wave (inverse of sk_range)
+__device__ __forceinline__ int sk_pid_of_iter(const DevPlan &p, int iter) {
+  const int boundary = p.sk_extra * (p.sk_full + 1);
+  if (iter < boundary) return iter / (p.sk_full + 1);
+  return p.sk_extra + (iter - boundary) / p.sk_full;
+}
+
+// Owner: the first wave polls all `npeers` follower flags at once, one flag per lane; the barrier
+// orders the CTA's (coherent) partial loads after the flags were seen.
+// Returns false if the poll limit ran out.
+__device__ __forceinline__ bool wait_partials_ready(int *flags, int npeers, int spin_limit) {
+  int ok = 1;
+  if (threadIdx.x < 64) {
+    for (int i = threadIdx.x; i < npeers; i += 64) {
+      int got = 0;
+      for (int s = 0; s < spin_limit; ++s) {
+        if (__hip_atomic_load(flags + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) { got = 1; break; }
+        __builtin_amdgcn_s_sleep(1);
+      }
+      ok &= got;
     }
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-    *lds_ok = ok;
   }
-  __syncthreads();
-  return *lds_ok != 0;
+  return __syncthreads_and(ok) != 0;
 }
 
-__device__ __forceinline__ void clear_flag_after_use(int *flag) {
+__device__ __forceinline__ void clear_flags_after_use(int *flags, int npeers) {
   __syncthreads();
-  if (threadIdx.x == 0) __hip_atomic_store(flag, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  for (int i = threadIdx.x; i < npeers; i += blockDim.x)
+    __hip_atomic_store(flags + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ---- buffer addressing ----

@@ -55,9 +55,10 @@ __device__ __forceinline__ void run_persistent(const typename P::Args &a, const 
         // converts and stores, then leaves buffer and counter zeroed for the next launch.
         float *part = ws.partials + (size_t)tile * P::TILE_ELEMS;
         P::atomic_partial(acc, part);
+        wait_own_memory_ops();
         __syncthreads();
         if (threadIdx.x == 0) {
-          int old = __hip_atomic_fetch_add(&ws.flags[tile], n, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+          int old = __hip_atomic_fetch_add(&ws.flags[tile], n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           s_word = (old + n == ipt);
         }
         __syncthreads();
@@ -73,20 +74,14 @@ __device__ __forceinline__ void run_persistent(const typename P::Args &a, const 
         P::store_partial(acc, ws.partials + (size_t)pid * P::TILE_ELEMS);
         signal_partial_ready(&ws.flags[pid]);
       } else {
-        // tile's first CTA: add the followers' partials in ascending CTA order, then store
-        const int tile_end = (tile + 1) * ipt;
-        int pos = last, p = pid + 1;
-        while (pos < tile_end) {
-          if (!wait_partial_ready(&ws.flags[p], plan.spin_limit, &s_word)) {
-            if (threadIdx.x == 0) *ws.status = -8;  // SK_ERR_TIMEOUT
-            break;
-          }
-          P::add_partial(acc, ws.partials + (size_t)p * P::TILE_ELEMS);
-          clear_flag_after_use(&ws.flags[p]);
-          int ps, pl;
-          sk_range(plan, p, ps, pl);
-          pos = pl;
-          ++p;
+        // tile's first CTA: wait for all followers at once, then add their partials in ascending
+        // CTA order and store
+        const int npeers = sk_pid_of_iter(plan, (tile + 1) * ipt - 1) - pid;
+        if (!wait_partials_ready(&ws.flags[pid + 1], npeers, plan.spin_limit)) {
+          if (threadIdx.x == 0) *ws.status = -8;  // SK_ERR_TIMEOUT
+        } else {
+          for (int p = 1; p <= npeers; ++p) P::add_partial(acc, ws.partials + (size_t)(pid + p) * P::TILE_ELEMS);
+          clear_flags_after_use(&ws.flags[pid + 1], npeers);
         }
         store = true;
       }

@@ -191,13 +191,13 @@ struct TileF16NT {
     dst = pin_here(dst);
 #pragma unroll
     for (int v = 0; v < NV4; ++v)
-      *reinterpret_cast<floatx4 *>(dst + ((size_t)v * NT + threadIdx.x) * 4) = grp(acc, v);
+      st_coherent(dst + ((size_t)v * NT + threadIdx.x) * 4, grp(acc, v));
   }
   static __device__ __forceinline__ void add_partial(Acc &acc, const float *src) {
     src = pin_here(src);
 #pragma unroll
     for (int v = 0; v < NV4; ++v) {
-      floatx4 x = *reinterpret_cast<const floatx4 *>(src + ((size_t)v * NT + threadIdx.x) * 4);
+      floatx4 x = ld_coherent(src + ((size_t)v * NT + threadIdx.x) * 4);
       floatx16 &c = acc.c[(v / 4) / TN][(v / 4) % TN];
       const int q = (v % 4) * 4;
 #pragma unroll
@@ -227,8 +227,8 @@ struct TileF16NT {
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         float *p = src + (size_t)(v * 4 + e) * NT + threadIdx.x;
-        c[q + e] = *p;
-        *p = 0.f;
+        c[q + e] = ld_coherent_scalar(p);
+        st_coherent(p, 0.f);
       }
       if (v % 4 == 3) asm volatile("" ::: "memory");
     }

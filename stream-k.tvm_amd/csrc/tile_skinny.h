@@ -8,10 +8,12 @@
 // streamk_fp16_block_reduce.py:45,235-306).
 //
 // Per v_mfma_f32_16x16x32_f16 a lane (row = lane%16, g = lane/16) supplies 8 K-values.  Which 8 is
-// free as long as both operands agree, so lane group g owns the contiguous K range
-// [g*KL, (g+1)*KL) of the wave's BK block (KL = BK/4): weights are loaded straight from global
-// memory as 16-byte pieces of one row, and the A tile is read from LDS at the same K offsets.
-// For Q4, A is written to LDS in the element order the nibble decode produces (0,4,1,5,2,6,3,7).
+// free as long as both operands agree.  Weights are loaded straight from global memory, 16 bytes
+// per lane: load c of an iteration covers E*4 consecutive K-values of each of the wave's 16 rows
+// (E = K-values per 16 bytes: 8 for fp16, 32 for Q4), lane group g taking piece g -- so one load
+// instruction reads 64 contiguous bytes from every row.  The A tile is read from LDS at the same
+// K offsets.  For Q4, A is written to LDS in the element order the nibble decode produces
+// (0,4,1,5,2,6,3,7).
 #pragma once
 #include "q4_dequant.h"
 #include "sk_device.h"
@@ -29,7 +31,9 @@ struct SkinnyArgs {
   int groups;             // Q4: scales per row
 };
 
-template <int MB_, int NB_, int WN_, int RK_, bool Q4_, int DEPTH_>
+// ROW1_: M == 1 only.  A single row of A is staged and every lane reads it (an LDS broadcast);
+// rows 1..15 of the MFMA result are then copies of row 0 and are never stored.
+template <int MB_, int NB_, int WN_, int RK_, bool Q4_, int DEPTH_, bool ROW1_ = false>
 struct TileSkinny {
   typedef SkinnyArgs Args;
   static constexpr int MB = MB_, NB = NB_, WN = WN_, RK = RK_, DEPTH = DEPTH_;
@@ -42,8 +46,12 @@ struct TileSkinny {
   static constexpr int WLOADS = Q4 ? KL / 32 : KL / 8;  // 16-byte weight loads per lane, block, iter
   static constexpr int NT = WN * RK * 64;
   static constexpr int LDA = BKC + 8;        // LDS row of A (halfs)
-  static constexpr int A_STAGE = BM * LDA;
-  static constexpr int A_CHUNKS = BM * BKC / 8;
+  static constexpr bool ROW1 = ROW1_;
+  static constexpr int A_ROWS = ROW1 ? 1 : BM;  // rows of A staged in LDS
+  static constexpr int MAX_M = ROW1 ? 1 : BM;
+  static constexpr int A_STAGE = A_ROWS * LDA;
+  static constexpr int A_CHUNKS = A_ROWS * BKC / 8;
+  static_assert(!ROW1 || MB_ == 1, "the single-row variant has one 16-row block");
   static constexpr int A_LOADS = (A_CHUNKS + NT - 1) / NT;
   static constexpr int QGROUP = 128;
   static constexpr int SC_PER_ITER = BKC / QGROUP;  // Q4 scale groups per CTA iteration
@@ -88,18 +96,19 @@ struct TileSkinny {
     const uint32_t ldw_bytes = (uint32_t)a.ldw * (Q4 ? 1 : 2);
     const BufferRsrc rsrc_w =
         make_rsrc(reinterpret_cast<const char *>(a.W) + (int64_t)pn * BN * ldw_bytes, rows_w * ldw_bytes);
-    const int klane = rk * BK + lg * KL;  // K offset of this lane inside a CTA iteration
+    constexpr int E = Q4 ? 32 : 8;               // K-values in one 16-byte load
+    const int klane = rk * BK + lg * E;          // K offset of this lane's piece of load 0
     uint32_t voff_w[NB];
 #pragma unroll
     for (int j = 0; j < NB; ++j)
       voff_w[j] = (uint32_t)((wn * NB + j) * 16 + lr) * ldw_bytes + (uint32_t)(klane / 2) * WB;
 
     // ---- A tile: all BM rows are staged; rows past M read as zero ----
-    const int a_rows = min(a.M - pm * BM, BM);
+    const int a_rows = min(a.M - pm * BM, A_ROWS);
     const BufferRsrc rsrc_a = make_rsrc(a.A + (int64_t)pm * BM * a.lda, (uint32_t)(a_rows * a.lda * 2));
     int a_rd[MB];
 #pragma unroll
-    for (int i = 0; i < MB; ++i) a_rd[i] = (i * 16 + lr) * LDA + klane;
+    for (int i = 0; i < MB; ++i) a_rd[i] = (ROW1 ? 0 : (i * 16 + lr) * LDA) + klane;
     uint32_t voff_a[A_LOADS];
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) {
@@ -122,8 +131,8 @@ struct TileSkinny {
       for (int j = 0; j < NB; ++j)
 #pragma unroll
         for (int c = 0; c < WLOADS; ++c) {
-          const bool inside = klane + c * (Q4 ? 32 : 8) < klimit;
-          wreg[slot][j][c] = buffer_load_16(rsrc_w, inside ? voff_w[j] : OOB_OFFSET, koff_w + c * 16);
+          const bool inside = klane + c * (4 * E) < klimit;
+          wreg[slot][j][c] = buffer_load_16(rsrc_w, inside ? voff_w[j] : OOB_OFFSET, koff_w + c * 64);
         }
 #pragma unroll
       for (int i = 0; i < A_LOADS; ++i) {
@@ -153,7 +162,7 @@ struct TileSkinny {
       }
     };
 
-    const half2v bias = q4_bias(a.zero);
+    const Q4Consts qc = q4_consts(a.zero);
 
     // ---- prologue: DEPTH iterations of loads in flight ----
 #pragma unroll
@@ -186,26 +195,30 @@ struct TileSkinny {
       for (int d = 0; d < DEPTH; ++d) {
         const int it = it0 + d;
         const half_t *abuf = ldsA + (it & 1) * A_STAGE;
-        half2v sc[NB];
+        half2v sc[NB][WLOADS];
         if (Q4) {
 #pragma unroll
           for (int j = 0; j < NB; ++j) {
             // iterations past the segment multiply zero weights; they must still see a finite scale
-            half_t s = ldsS[((wn * NB + j) * 16 + lr) * SC_ROW + sc_shift + min(it, n - 1) * SC_PER_ITER +
-                            (klane / QGROUP)];
-            sc[j] = half2v{s, s};
+            // load c of a Q4 iteration spans exactly one 128-wide scale group: group rk*2 + c
+            const half_t *sp = ldsS + ((wn * NB + j) * 16 + lr) * SC_ROW + sc_shift + min(it, n - 1) * SC_PER_ITER + rk * 2;
+#pragma unroll
+            for (int c = 0; c < WLOADS; ++c) sc[j][c] = half2v{sp[c], sp[c]};
           }
         }
 #pragma unroll
         for (int ch = 0; ch < NCH; ++ch) {
           half8v fa[MB];
+          // K offset of chunk ch relative to the lane's piece of load 0
+          constexpr int CH_PER_LOAD = E / 8;
+          const int koff_ch = (ch / CH_PER_LOAD) * (4 * E) + (ch % CH_PER_LOAD) * 8;
 #pragma unroll
-          for (int i = 0; i < MB; ++i) fa[i] = *reinterpret_cast<const half8v *>(abuf + a_rd[i] + ch * 8);
+          for (int i = 0; i < MB; ++i) fa[i] = *reinterpret_cast<const half8v *>(abuf + a_rd[i] + koff_ch);
 #pragma unroll
           for (int j = 0; j < NB; ++j) {
             half8v fw;
             if (Q4) {
-              fw = dequant_word_q4(wreg[d][j][ch / 4][ch % 4], bias, sc[j]);
+              fw = dequant_word_q4(wreg[d][j][ch / 4][ch % 4], qc, sc[j][ch / 4]);
             } else {
               fw = __builtin_bit_cast(half8v, wreg[d][j][ch]);
             }
@@ -278,13 +291,13 @@ struct TileSkinny {
     if (threadIdx.x >= NTP) return;
 #pragma unroll
     for (int v = 0; v < NV4; ++v)
-      *reinterpret_cast<floatx4 *>(dst + ((size_t)v * NTP + threadIdx.x) * 4) = acc.c[v / NB][v % NB];
+      st_coherent(dst + ((size_t)v * NTP + threadIdx.x) * 4, acc.c[v / NB][v % NB]);
   }
   static __device__ __forceinline__ void add_partial(Acc &acc, const float *src) {
     if (threadIdx.x >= NTP) return;
 #pragma unroll
     for (int v = 0; v < NV4; ++v)
-      acc.c[v / NB][v % NB] += *reinterpret_cast<const floatx4 *>(src + ((size_t)v * NTP + threadIdx.x) * 4);
+      acc.c[v / NB][v % NB] += ld_coherent(src + ((size_t)v * NTP + threadIdx.x) * 4);
   }
   static __device__ __forceinline__ void atomic_partial(const Acc &acc, float *dst) {
     if (threadIdx.x >= NTP) return;
@@ -301,8 +314,8 @@ struct TileSkinny {
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         float *p = src + (size_t)(v * 4 + e) * NTP + threadIdx.x;
-        acc.c[v / NB][v % NB][e] = *p;
-        *p = 0.f;
+        acc.c[v / NB][v % NB][e] = ld_coherent_scalar(p);
+        st_coherent(p, 0.f);
       }
   }
 };

@@ -2,4 +2,5 @@
 from ._lib import LIB_PATH, StreamKError, lib, strerror  # noqa: F401
 from .ops import (StreamKKernel, bench_ms, dequant_q4, reset_workspaces, streamk_fp16,  # noqa: F401
                   streamk_fp32, streamk_q4, tl_matmul_streamk, workspace_status)
-from .plan import cta_range, make_config, make_plan, num_cus, tile_coords  # noqa: F401
+from .autotune import autotune, candidate_configs  # noqa: F401
+from .plan import cta_range, make_config, make_plan, num_cus, tile_coords, tuned_config  # noqa: F401

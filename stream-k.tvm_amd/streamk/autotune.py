@@ -1,0 +1,158 @@
+"""Per-shape autotuner over tile / kernel variant / schedule / grid / fix-up.
+
+Plays the role of the reference's `@autotune(configs=...) @jit(...)` loop
+(autotune/streamk_fp16_autotune.py:38-53, 88-95, 373-386): enumerate configurations, time each,
+keep the fastest and return `(best_latency, best_config, ref_latency)`.  Here no code is
+generated per configuration: every candidate is a (kernel instance, partition) pair of the already
+built library, so a search costs milliseconds per candidate.
+
+Results are kept in a JSON cache keyed by (arch, dtype, layout, M, N, K); `plan.make_plan` consults
+the cache when the caller gives no configuration.
+"""
+import itertools
+import json
+import os
+
+import torch
+
+from . import ops, plan as _plan
+from ._lib import StreamKError
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+DEFAULT_CACHE = os.path.join(_HERE, "tuned", "gfx950.json")
+USER_CACHE_ENV = "STREAMK_TUNE_CACHE"
+
+_TILES_F16 = [(256, 256, 64), (128, 128, 64), (128, 256, 64), (256, 128, 64), (64, 64, 64)]
+_SKINNY_F16 = [(16, 64, 128), (32, 64, 128), (64, 64, 128), (16, 16, 512), (16, 32, 256), (16, 16, 128)]
+_SKINNY_Q4 = [(16, 64, 256), (32, 64, 256), (64, 64, 256), (16, 16, 1024), (16, 32, 512), (16, 16, 256),
+              (16, 32, 256)]
+
+
+def _key(dtype, layout, M, N, K):
+    return f"gfx950/{dtype}/{layout}/{M}x{N}x{K}"
+
+
+def load_cache(path=None):
+    path = path or os.environ.get(USER_CACHE_ENV) or DEFAULT_CACHE
+    try:
+        with open(path) as f:
+            return json.load(f)
+    except (OSError, ValueError):
+        return {}
+
+
+def save_cache(cache, path=None):
+    path = path or os.environ.get(USER_CACHE_ENV) or DEFAULT_CACHE
+    os.makedirs(os.path.dirname(path), exist_ok=True)
+    with open(path, "w") as f:
+        json.dump(cache, f, indent=1, sort_keys=True)
+
+
+def candidate_configs(M, N, K, dtype="float16", cus=None):
+    """The search space.  The reference multiplies out warp/chunk/stage lists
+    (autotune/streamk_fp16_autotune.py:38-53); here the axes are tile shape, kernel variant,
+    schedule, grid and fix-up."""
+    cus = cus or _plan.num_cus()
+    out = []
+    if dtype == "q4" or M <= 64:
+        tiles = _SKINNY_Q4 if dtype == "q4" else _SKINNY_F16
+        for (bm, bn, bk) in tiles:
+            if bm < M and not (bm == 16 and M <= 16):
+                continue
+            if bm >= 2 * M and bm > 16:
+                continue
+            out.append(dict(bm=bm, bn=bn, bk=bk, schedule="dp"))
+            for grid, fixup in itertools.product((cus, 2 * cus, 4 * cus), ("reduce", "atomic")):
+                out.append(dict(bm=bm, bn=bn, bk=bk, schedule="sk2", grid=grid, fixup=fixup))
+    if dtype == "float16" and M > 16:
+        for (bm, bn, bk) in _TILES_F16:
+            variants = (2, 1) if (bm, bn) != (64, 64) else (0,)
+            for variant, raster in itertools.product(variants, (0, 8)):
+                base = dict(bm=bm, bn=bn, bk=bk, variant=variant, raster=raster)
+                out.append(dict(base, schedule="dp"))
+                for sched, fixup in itertools.product(("sk2", "sk1", "basic"), ("reduce", "atomic")):
+                    out.append(dict(base, schedule=sched, fixup=fixup))
+    return out
+
+
+def _time_ms(fn, warmup, rep, graph):
+    if not graph:
+        return ops.bench_ms(fn, warmup, rep)
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        for _ in range(max(1, warmup)):
+            fn()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=s):
+            for _ in range(rep):
+                fn()
+        g.replay()
+        torch.cuda.synchronize()
+        st, en = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        st.record()
+        for _ in range(3):
+            g.replay()
+        en.record()
+        torch.cuda.synchronize()
+    return st.elapsed_time(en) / (3 * rep)
+
+
+def autotune(M, N, K, dtype="float16", layout="nt", *, configs=None, warmup=5, rep=20, check=True,
+             cache=True, cache_path=None, verbose=False):
+    """Searches `configs` (default: candidate_configs) for the fastest plan.
+
+    Returns (best_latency_ms, best_config, ref_latency_ms); ref is torch.matmul on the same GPU, the
+    reference's comparator (streamk_fp16.py:396) -- None for Q4.  Every candidate is checked against
+    the first valid one (max-abs-rel 1e-2) unless check=False, mirroring `skip_check` of the
+    reference's jit decorator."""
+    dev = "cuda"
+    g = torch.Generator(device="cpu").manual_seed(0)
+    A = (torch.rand(M, K, generator=g) * 2 - 1).half().to(dev)
+    C = torch.empty(M, N, dtype=torch.float16, device=dev)
+    if dtype == "q4":
+        Wq = torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8).to(dev)
+        sc = (torch.rand(N, K // 128, generator=g) * 0.015 + 0.005).half().to(dev)
+        run = lambda p: ops.streamk_q4(A, Wq, sc, out=C, plan=p)  # noqa: E731
+        ref_ms = None
+    else:
+        bshape = (N, K) if layout == "nt" else (K, N)
+        B = (torch.rand(*bshape, generator=g) * 2 - 1).half().to(dev)
+        run = lambda p: ops.streamk_fp16(A, B, layout=layout, out=C, plan=p)  # noqa: E731
+        Bt = B.T if layout == "nt" else B
+        small = 2.0 * M * N * K < 5e10
+        ref_ms = _time_ms(lambda: torch.matmul(A, Bt, out=C), warmup, rep, small)
+    small = 2.0 * M * N * K < 5e10  # microsecond kernels: time graph-captured batches
+    configs = configs if configs is not None else candidate_configs(M, N, K, dtype)
+    best, golden, results = None, None, []
+    for cfg in configs:
+        try:
+            p = _plan.make_plan(M, N, K, dtype, layout, cfg)
+            run(p)
+            torch.cuda.synchronize()
+            ops.workspace_status()
+        except StreamKError as e:
+            if e.status == -8:
+                ops.reset_workspaces()
+            continue
+        if check:
+            if golden is None:
+                golden = C.float().clone()
+            else:
+                err = (C.float() - golden).abs().max().item() / max(golden.abs().max().item(), 1e-30)
+                if err > 1e-2:
+                    raise AssertionError(f"config {cfg} disagrees with the first candidate: {err}")
+        ms = _time_ms(lambda: run(p), warmup, rep, small)
+        results.append((ms, cfg))
+        if verbose:
+            print(f"  {ms * 1e3:9.2f} us  {cfg}")
+        if best is None or ms < best[0]:
+            best = (ms, cfg)
+    if best is None:
+        raise RuntimeError(f"no valid configuration for {M}x{N}x{K} {dtype}/{layout}")
+    if cache:
+        c = load_cache(cache_path)
+        c[_key(dtype, layout, M, N, K)] = {"config": best[1], "latency_ms": best[0], "ref_latency_ms": ref_ms}
+        save_cache(c, cache_path)
+        _plan.invalidate_tuned_cache()
+    return best[0], best[1], ref_ms

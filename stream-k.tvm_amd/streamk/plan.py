@@ -42,9 +42,31 @@ def make_config(config=None, **kw):
     return c
 
 
-def make_plan(M, N, K, dtype="float16", layout="nt", config=None, cus=None, **kw):
+_tuned = None
+
+
+def invalidate_tuned_cache():
+    global _tuned
+    _tuned = None
+
+
+def tuned_config(M, N, K, dtype="float16", layout="nt"):
+    """Configuration the autotuner recorded for exactly this problem, or None."""
+    global _tuned
+    if _tuned is None:
+        from .autotune import load_cache
+        _tuned = load_cache()
+    hit = _tuned.get(f"gfx950/{dtype}/{layout}/{M}x{N}x{K}")
+    return dict(hit["config"]) if hit else None
+
+
+def make_plan(M, N, K, dtype="float16", layout="nt", config=None, cus=None, use_tuned=True, **kw):
     """Partition an M x N x K GEMM.  `cus` overrides the device's CU count (lets the partitioner
-    run without a GPU)."""
+    run without a GPU).  With no configuration given, a tuned one from the autotune cache is used
+    when there is one for this exact problem, else the library heuristic."""
+    kw = {k: v for k, v in kw.items() if v is not None}
+    if use_tuned and not config and not kw and cus is None:
+        config = tuned_config(M, N, K, dtype, layout)
     cfg = make_config(config, **kw)
     plan = SkPlan()
     rc = _lib.lib().sk_make_plan(M, N, K, _DTYPES[dtype], _LAYOUTS[layout], ctypes.byref(cfg),
