@@ -172,16 +172,16 @@ extern "C" int sk_gemm_f16(const void *A, const void *B, void *C, int64_t M, int
   if (!A || !B || !C) return SK_ERR_NULL;
   int rc = check_plan(plan, M, N, K, SK_F16, plan ? plan->layout : 0);
   if (rc) return rc;
-  if (plan->layout != SK_LAYOUT_NT) return SK_ERR_CONFIG;
-  if (lda < K || ldb < K || ldc < N) return SK_ERR_SHAPE;
-  if ((K % 8) || (lda % 8) || (ldb % 8)) return SK_ERR_ALIGN;
+  const bool nn = plan->layout == SK_LAYOUT_NN;
+  if (lda < K || ldb < (nn ? N : K) || ldc < N) return SK_ERR_SHAPE;
+  if ((K % 8) || (lda % 8) || (ldb % 8) || (nn && (N % 8))) return SK_ERR_ALIGN;
   if ((reinterpret_cast<uintptr_t>(A) & 15) || (reinterpret_cast<uintptr_t>(B) & 15) ||
       (reinterpret_cast<uintptr_t>(C) & 1))
     return SK_ERR_ALIGN;
   const KernelInfo *k = kernel_by_id(plan->kernel_id);
-  if (!k || k->dtype != SK_F16) return SK_ERR_CONFIG;
-  // a tile's rows must be addressable with 32-bit byte offsets
-  if (lda * 2 * k->bm >= (int64_t)1 << 31 || ldb * 2 * k->bn >= (int64_t)1 << 31) return SK_ERR_SHAPE;
+  if (!k || k->dtype != SK_F16 || k->layout != plan->layout) return SK_ERR_CONFIG;
+  // a tile's rows (NN: all K rows of B) must be addressable with 32-bit byte offsets
+  if (lda * 2 * k->bm >= (int64_t)1 << 31 || ldb * 2 * (nn ? K : k->bn) >= (int64_t)1 << 31) return SK_ERR_SHAPE;
   DevPlan dp;
   Workspace w;
   const bool skinny = k->family == FAMILY_SKINNY;

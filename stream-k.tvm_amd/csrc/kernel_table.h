@@ -29,7 +29,14 @@ struct KernelInfo {
   int ctas_per_cu;    // co-resident CTAs per CU the kernel is compiled for
   int partial_elems;  // fp32 elements of one partial tile in the workspace
   int max_ipt;        // largest iterations-per-tile the kernel supports (0 = unlimited)
-  int max_m;          // small-M kernels: largest M the kernel accepts
+  int max_m;          // the same for the NN layout (B is [K,N]), fragments through transposing LDS reads:  X(id, BM, BN, WM, WN)
+#define SK_TILE_F16_NN_DMA_KERNELS(X) \
+  X(20, 256, 256, 2, 4)               \
+  X(21, 128, 128, 2, 2)               \
+  X(22, 128, 256, 2, 4)               \
+  X(23, 256, 128, 4, 2)
+
+// small-M kernels: largest M the kernel accepts
   int k_align;        // K must be a multiple of this
   const char *name;
 };
@@ -51,6 +58,13 @@ struct KernelInfo {
   X(12, 128, 256, 2, 4)               \
   X(13, 256, 128, 4, 2)               \
   X(14, 256, 256, 2, 2)
+
+// the same for the NN layout (B is [K,N]), fragments through transposing LDS reads:  X(id, BM, BN, WM, WN)
+#define SK_TILE_F16_NN_DMA_KERNELS(X) \
+  X(20, 256, 256, 2, 4)               \
+  X(21, 128, 128, 2, 2)               \
+  X(22, 128, 256, 2, 4)               \
+  X(23, 256, 128, 4, 2)
 
 // small-M kernels:  X(id, MB, NB, WN, RK, Q4, DEPTH, ROW1)
 #define SK_SKINNY_KERNELS(X)     \

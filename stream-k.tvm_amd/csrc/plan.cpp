@@ -60,7 +60,7 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
   // heuristic: small M -> weight-streaming kernels; otherwise the largest tile that still gives
   // every CU something to do
   const KernelInfo *best = nullptr;
-  if (M <= 64 || dtype == SK_Q4) {
+  if ((M <= 64 && layout == SK_LAYOUT_NT) || dtype == SK_Q4) {
     int mb = M <= 16 ? 16 : (M <= 32 ? 32 : 64);
     for (int i = 0; i < n; ++i)
       if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].bm == mb && t[i].bn == 64 &&

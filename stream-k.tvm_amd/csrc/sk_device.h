@@ -91,10 +91,19 @@ __device__ __forceinline__ void wait_own_memory_ops() { __builtin_amdgcn_fence(_
 // ---- REDUCE fix-up: flags ----
 // Contributor: every thread waits for its own (write-through) partial stores, the barrier
 // collects the CTA, then thread 0 raises the flag.
+// COHERENT = false: the partial went through the L2 with ordinary stores; thread 0's device-scope
+// release (one L2 write-back for the whole CTA, after the barrier has collected everybody's
+// stores) publishes it together with the flag.
+template <bool COHERENT>
 __device__ __forceinline__ void signal_partial_ready(int *flag) {
   wait_own_memory_ops();
   __syncthreads();
-  if (threadIdx.x == 0) __hip_atomic_store(flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (threadIdx.x == 0) {
+    if (COHERENT)
+      __hip_atomic_store(flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else
+      __hip_atomic_store(flag, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+  }
 }
 
 // CTA that owns K-iteration `iter` of the Stream-K wave (inverse of sk_range)
@@ -107,6 +116,9 @@ __device__ __forceinline__ int sk_pid_of_iter(const DevPlan &p, int iter) {
 // Owner: the first wave polls all `npeers` follower flags at once, one flag per lane; the barrier
 // orders the CTA's (coherent) partial loads after the flags were seen.
 // Returns false if the poll limit ran out.
+// COHERENT = false: one device-scope acquire (L2 invalidate) by the polling wave before the
+// barrier, so that the ordinary loads that follow cannot hit stale lines.
+template <bool COHERENT>
 __device__ __forceinline__ bool wait_partials_ready(int *flags, int npeers, int spin_limit) {
   int ok = 1;
   if (threadIdx.x < 64) {
@@ -118,6 +130,7 @@ __device__ __forceinline__ bool wait_partials_ready(int *flags, int npeers, int 
       }
       ok &= got;
     }
+    if (!COHERENT) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
   }
   return __syncthreads_and(ok) != 0;
 }

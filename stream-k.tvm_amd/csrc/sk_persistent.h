@@ -60,6 +60,8 @@ __device__ __forceinline__ void run_persistent(const typename P::Args &a, const 
         if (threadIdx.x == 0) {
           int old = __hip_atomic_fetch_add(&ws.flags[tile], n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           s_word = (old + n == ipt);
+          // the last arriver reads the sum with ordinary loads: drop stale L2 lines first
+          if (!P::COHERENT_PARTIALS && s_word) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
         }
         __syncthreads();
         store = s_word != 0;
@@ -72,12 +74,12 @@ __device__ __forceinline__ void run_persistent(const typename P::Args &a, const 
       } else if (k0 != 0) {
         // not the tile's first CTA: park the partial in this CTA's slot and raise its flag
         P::store_partial(acc, ws.partials + (size_t)pid * P::TILE_ELEMS);
-        signal_partial_ready(&ws.flags[pid]);
+        signal_partial_ready<P::COHERENT_PARTIALS>(&ws.flags[pid]);
       } else {
         // tile's first CTA: wait for all followers at once, then add their partials in ascending
         // CTA order and store
         const int npeers = sk_pid_of_iter(plan, (tile + 1) * ipt - 1) - pid;
-        if (!wait_partials_ready(&ws.flags[pid + 1], npeers, plan.spin_limit)) {
+        if (!wait_partials_ready<P::COHERENT_PARTIALS>(&ws.flags[pid + 1], npeers, plan.spin_limit)) {
           if (threadIdx.x == 0) *ws.status = -8;  // SK_ERR_TIMEOUT
         } else {
           for (int p = 1; p <= npeers; ++p) P::add_partial(acc, ws.partials + (size_t)(pid + p) * P::TILE_ELEMS);

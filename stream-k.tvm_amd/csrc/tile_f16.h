@@ -180,6 +180,10 @@ struct TileF16NT {
     __syncthreads();  // patches overlap the staging buffers of the next tile
   }
 
+  // Partial tiles are large (BM*BN*4 bytes) and few: they go through the L2 with ordinary 16-byte
+  // accesses, and each CTA pays one L2 write-back (contributor) or invalidate (owner) per fix-up.
+  static constexpr bool COHERENT_PARTIALS = false;
+
   // Partials live in the workspace in "fragment order": float4 group v of thread t sits at
   // (v * NT + t) * 4, so every access is a fully coalesced 16 bytes per lane.
   static __device__ __forceinline__ floatx4 grp(const Acc &acc, int v) {
@@ -191,13 +195,13 @@ struct TileF16NT {
     dst = pin_here(dst);
 #pragma unroll
     for (int v = 0; v < NV4; ++v)
-      st_coherent(dst + ((size_t)v * NT + threadIdx.x) * 4, grp(acc, v));
+      *reinterpret_cast<floatx4 *>(dst + ((size_t)v * NT + threadIdx.x) * 4) = grp(acc, v);
   }
   static __device__ __forceinline__ void add_partial(Acc &acc, const float *src) {
     src = pin_here(src);
 #pragma unroll
     for (int v = 0; v < NV4; ++v) {
-      floatx4 x = ld_coherent(src + ((size_t)v * NT + threadIdx.x) * 4);
+      floatx4 x = *reinterpret_cast<const floatx4 *>(src + ((size_t)v * NT + threadIdx.x) * 4);
       floatx16 &c = acc.c[(v / 4) / TN][(v / 4) % TN];
       const int q = (v % 4) * 4;
 #pragma unroll
@@ -227,8 +231,8 @@ struct TileF16NT {
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         float *p = src + (size_t)(v * 4 + e) * NT + threadIdx.x;
-        c[q + e] = ld_coherent_scalar(p);
-        st_coherent(p, 0.f);
+        c[q + e] = *p;
+        *p = 0.f;
       }
       if (v % 4 == 3) asm volatile("" ::: "memory");
     }

@@ -34,8 +34,18 @@ struct LdsArray {
   }
 };
 
-template <int BM_, int BN_, int WM_, int WN_>
+// B_KN_: B is [K,N] row-major (NN GEMM).  Its stage is then 64 rows (K) of BN halfs.  Fragments
+// are read with ds_read_b64_tr_b16, which hands lane L of each 16-lane group the element (L & 3) of
+// the 8 bytes addressed by lane (L >> 2) + 4*j of that group, j = 0..3: a 16-lane group pointing at
+// a 4 (K) x 16 (N) patch receives, per lane, 4 consecutive K of one column -- half an MFMA operand.
+// 16-byte chunk c of K-row k is stored at position c ^ (4 * (k & 3)), which keeps the 32 lanes
+// served in one cycle (2 groups x 4 rows x 32 bytes) on distinct banks.
+template <int BM_, int BN_, int WM_, int WN_, bool B_KN_ = false>
 struct TileF16NTDma {
+  static constexpr bool B_KN = B_KN_;
+  static constexpr int B_ROW_BYTES = B_KN_ ? BN_ * 2 : 128;    // bytes of one LDS row of the B stage
+  static constexpr int B_ROWS_PER_DMA = 1024 / B_ROW_BYTES;    // rows one wave-wide load fills
+  static_assert(!B_KN_ || (BN_ >= 128 && BN_ <= 512), "NN layout: 16..64 chunks per LDS row");
   typedef GemmArgs Args;
   static constexpr int BM = BM_, BN = BN_, BK = 64, WM = WM_, WN = WN_;
   static constexpr int NW = WM * WN, NT = NW * 64;
@@ -98,17 +108,37 @@ struct TileF16NTDma {
 
     const int rows_a = min(BM, a.M - pm * BM), rows_b = min(BN, a.N - pn * BN);
     const uint4v rsrc_a = make_rsrc_words(a.A + (int64_t)pm * BM * a.lda, (uint32_t)(rows_a * a.lda * 2));
-    const uint4v rsrc_b = make_rsrc_words(a.B + (int64_t)pn * BN * a.ldb, (uint32_t)(rows_b * a.ldb * 2));
     const int my_chunk = (lane & 7) ^ (((wave & 1) << 2) | (lane >> 4));  // global chunk this lane fetches
     const uint32_t voff_a = (uint32_t)((lane >> 3) * a.lda + my_chunk * 8) * 2;
-    const uint32_t voff_b = (uint32_t)((lane >> 3) * a.ldb + my_chunk * 8) * 2;
-    const uint32_t grp_a = (uint32_t)(8 * a.lda * 2), grp_b = (uint32_t)(8 * a.ldb * 2);
+    const uint32_t grp_a = (uint32_t)(8 * a.lda * 2);
     const int tail_kt = (a.K % BK != 0) ? (a.K / BK) : -1;
+    // B operand.  NT: rows are N, same scheme as A.  NN: rows are K; the descriptor starts at the
+    // tile's first column and ends with the last valid element of row K-1, so K-rows past the
+    // matrix read as zero; columns past N are masked per lane (N % 8 == 0).
+    uint4v rsrc_b;
+    uint32_t voff_b, grp_b, kstep_b;
+    if (!B_KN) {
+      rsrc_b = make_rsrc_words(a.B + (int64_t)pn * BN * a.ldb, (uint32_t)(rows_b * a.ldb * 2));
+      voff_b = (uint32_t)((lane >> 3) * a.ldb + my_chunk * 8) * 2;
+      grp_b = (uint32_t)(8 * a.ldb * 2);
+      kstep_b = BK * 2;
+    } else {
+      rsrc_b = make_rsrc_words(a.B + (int64_t)pn * BN, (uint32_t)(((int64_t)(a.K - 1) * a.ldb + rows_b) * 2));
+      const int row_in = (lane * 16) / B_ROW_BYTES, pos = ((lane * 16) % B_ROW_BYTES) / 16;
+      const int k_low = (B_ROWS_PER_DMA == 2 ? 2 * (wave & 1) + row_in : row_in) & 3;  // (K-row & 3)
+      const int chunk = pos ^ (4 * k_low);
+      voff_b = (chunk * 8 < rows_b) ? (uint32_t)(row_in * a.ldb + chunk * 8) * 2 : OOB_OFFSET;
+      grp_b = (uint32_t)(B_ROWS_PER_DMA * a.ldb * 2);
+      kstep_b = (uint32_t)(BK * a.ldb * 2);
+    }
 
     auto issue_dma = [&](char *st, int kt) {
       const uint32_t koff = (uint32_t)kt * (BK * 2);
       uint32_t va = voff_a, vb = voff_b;
-      if (kt == tail_kt && kt * BK + my_chunk * 8 >= a.K) va = vb = OOB_OFFSET;
+      if (kt == tail_kt && kt * BK + my_chunk * 8 >= a.K) {
+        va = OOB_OFFSET;
+        if (!B_KN) vb = OOB_OFFSET;
+      }
 #pragma unroll
       for (int j = 0; j < A_DMA; ++j) {
         const int g = wave + j * NW;
@@ -117,7 +147,7 @@ struct TileF16NTDma {
 #pragma unroll
       for (int j = 0; j < B_DMA; ++j) {
         const int g = wave + j * NW;
-        dma_load_16(rsrc_b, lds_address(st) + A_BYTES + g * 1024, vb, koff + g * grp_b);
+        dma_load_16(rsrc_b, lds_address(st) + A_BYTES + g * 1024, vb, (uint32_t)kt * kstep_b + g * grp_b);
       }
     };
 
@@ -130,12 +160,35 @@ struct TileF16NTDma {
       rd_a[kk] = (wm * WTM + (lane & 31)) * 128 + pos;
       rd_b[kk] = A_BYTES + (wn * WTN + (lane & 31)) * 128 + pos;
     }
+    // NN: per 32-column block j, the byte address of this lane's 8-byte piece in K-row
+    // 8*(lane/32) + (lane%16)/4 of the stage; K-steps and the second half add row multiples
+    int rd_bt[TN];
+    if (B_KN) {
+      const int k_lane = 8 * (lane >> 5) + ((lane & 15) >> 2);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int col = wn * WTN + j * 32 + 16 * ((lane & 31) >> 4) + 4 * (lane & 3);
+        const int chunk = (col >> 3) ^ (4 * (k_lane & 3));
+        rd_bt[j] = A_BYTES + k_lane * B_ROW_BYTES + chunk * 16 + (col & 7) * 2;
+      }
+    }
     half8v fa[2][TM], fb[2][TN];
     auto read_frags = [&](const char *st, int buf, int kk) {
 #pragma unroll
       for (int i = 0; i < TM; ++i) fa[buf][i] = *reinterpret_cast<const half8v *>(st + rd_a[kk] + i * 4096);
 #pragma unroll
-      for (int j = 0; j < TN; ++j) fb[buf][j] = *reinterpret_cast<const half8v *>(st + rd_b[kk] + j * 4096);
+      for (int j = 0; j < TN; ++j) {
+        if (!B_KN) {
+          fb[buf][j] = *reinterpret_cast<const half8v *>(st + rd_b[kk] + j * 4096);
+        } else {
+          typedef short short4v __attribute__((ext_vector_type(4)));
+          typedef __attribute__((address_space(3))) short4v *lds_s4;
+          union { short4v s[2]; half8v h; } u;
+          u.s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4)(st + rd_bt[j] + (kk * 16) * B_ROW_BYTES));
+          u.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4)(st + rd_bt[j] + (kk * 16 + 4) * B_ROW_BYTES));
+          fb[buf][j] = u.h;
+        }
+      }
     };
     auto mfma_step = [&](int buf) {
 #pragma unroll
@@ -229,6 +282,7 @@ struct TileF16NTDma {
     __syncthreads();  // patches overlap the stages of the next tile
   }
 
+  static constexpr bool COHERENT_PARTIALS = false;
   static __device__ __forceinline__ void store_partial(const Acc &acc, float *dst) { Base::store_partial(acc, dst); }
   static __device__ __forceinline__ void add_partial(Acc &acc, const float *src) { Base::add_partial(acc, src); }
   static __device__ __forceinline__ void atomic_partial(const Acc &acc, float *dst) { Base::atomic_partial(acc, dst); }

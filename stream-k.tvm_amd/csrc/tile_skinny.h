@@ -287,6 +287,10 @@ struct TileSkinny {
     }
   }
 
+  // Partial tiles are a few KB and there can be thousands of CTAs: every access is a coherent
+  // (write-through / L2-bypassing) one, so no CTA ever flushes or invalidates a whole L2.
+  static constexpr bool COHERENT_PARTIALS = true;
+
   static __device__ __forceinline__ void store_partial(const Acc &acc, float *dst) {
     if (threadIdx.x >= NTP) return;
 #pragma unroll

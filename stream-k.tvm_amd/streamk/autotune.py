@@ -70,8 +70,9 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
             for variant, raster in itertools.product(variants, (0, 8)):
                 base = dict(bm=bm, bn=bn, bk=bk, variant=variant, raster=raster)
                 out.append(dict(base, schedule="dp"))
-                for sched, fixup in itertools.product(("sk2", "sk1", "basic"), ("reduce", "atomic")):
-                    out.append(dict(base, schedule=sched, fixup=fixup))
+                grids = (None,) if bm * bn >= 256 * 256 or (bm, bn) == (64, 64) else (None, cus)
+                for sched, fixup, grid in itertools.product(("sk2", "sk1", "basic"), ("reduce", "atomic"), grids):
+                    out.append(dict(base, schedule=sched, fixup=fixup, **({"grid": grid} if grid else {})))
     return out
 
 

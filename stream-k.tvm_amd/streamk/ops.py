@@ -60,7 +60,8 @@ def _check_matrix(t, name, dtype):
 
 def streamk_fp16(A, B, *, Wq=None, scales=None, layout="nt", out=None, plan=None, config=None,
                  zero=8, group=128, **kw):
-    """C = A @ B.T (layout 'nt', B is [N,K]) in fp16 with fp32 accumulation.
+    """C = A @ B.T (layout 'nt', B is [N,K]) or A @ B (layout 'nn', B is [K,N]) in fp16 with fp32
+    accumulation.
 
     With `Wq` (uint8 [N, K/2], low nibble = even k) and `scales` (fp16 [N, K/group]) the weights
     are dequantised on the fly, w = fp16((q - zero) * scale), and B is ignored (pass None).
@@ -70,10 +71,10 @@ def streamk_fp16(A, B, *, Wq=None, scales=None, layout="nt", out=None, plan=None
         return streamk_q4(A, Wq, scales, out=out, plan=plan, config=config, zero=zero, group=group, **kw)
     _check_matrix(A, "A", torch.float16)
     _check_matrix(B, "B", torch.float16)
-    if layout != "nt":
-        raise NotImplementedError("fp16 layout 'nn' is not built yet")
+    if layout not in ("nt", "nn"):
+        raise ValueError("layout must be 'nt' (B is [N,K]) or 'nn' (B is [K,N])")
     M, K = A.shape
-    N, Kb = B.shape
+    N, Kb = B.shape if layout == "nt" else (B.shape[1], B.shape[0])
     if K != Kb:
         raise ValueError(f"K mismatch: A is {tuple(A.shape)}, B is {tuple(B.shape)}")
     if plan is None:

@@ -221,6 +221,32 @@ def test_full_size_exact_integer_checksums(sk, shape):
     sk.workspace_status()
 
 
+@pytest.mark.parametrize("cfg", [dict(bm=256, bn=256), dict(bm=128, bn=128), dict(bm=128, bn=256), dict(bm=256, bn=128)],
+                         ids=lambda c: f"{c['bm']}x{c['bn']}")
+def test_nn_layout(sk, oracle, cfg):
+    """B given as [K,N] (the layout of the reference's fp32 script and of the large dense
+    configuration): ragged shapes against the oracle, all schedules; then exact integer data at
+    3000 x 5120 x 12288."""
+    rng = np.random.default_rng(21)
+    for (M, N, K) in [(200, 136, 328), (1000, 1096, 4104), (520, 264, 64)]:
+        A = (rng.random((M, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+        B = (rng.random((K, N), dtype=np.float32) * 2 - 1).astype(np.float16)
+        ref = oracle.matmul_fp32(A, B)
+        for sch in (dict(schedule="dp"), dict(schedule="basic", fixup="reduce", grid=24),
+                    dict(schedule="sk2", fixup="atomic", grid=16)):
+            C = sk.streamk_fp16(_t(A), _t(B), layout="nn", bk=64, **cfg, **sch)
+            assert _rel(oracle, C, ref) <= 2e-3 <= TOL, (M, N, K, sch)
+    M, N, K = 3000, 5120, 12288
+    A = rng.integers(-1, 2, (M, K)).astype(np.int8)
+    B = rng.integers(-1, 2, (K, N)).astype(np.int8)
+    row_sum = A.astype(np.int64) @ B.astype(np.int64).sum(axis=1)
+    col_sum = A.astype(np.int64).sum(axis=0) @ B.astype(np.int64)
+    C = sk.streamk_fp16(_t(A.astype(np.float16)), _t(B.astype(np.float16)), layout="nn", bk=64, **cfg).double()
+    assert np.array_equal(C.sum(dim=1).cpu().numpy().astype(np.int64), row_sum)
+    assert np.array_equal(C.sum(dim=0).cpu().numpy().astype(np.int64), col_sum)
+    sk.workspace_status()
+
+
 def test_strided_operands_and_out(sk, oracle):
     """Leading dimensions larger than the rows, and writing into a caller-provided C."""
     import torch
