@@ -198,9 +198,30 @@ extern "C" int sk_gemm_f16(const void *A, const void *B, void *C, int64_t M, int
   return herr == 0 ? SK_OK : SK_ERR_LAUNCH;
 }
 
-extern "C" int sk_gemm_f32(const void *, const void *, void *, int64_t, int64_t, int64_t, int64_t, int64_t,
-                           int64_t, const sk_plan *, void *, size_t, void *) {
-  return SK_ERR_CONFIG;  // fp32 kernels are not built yet
+extern "C" int sk_gemm_f32(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,
+                           int64_t lda, int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws,
+                           size_t ws_bytes, void *stream) {
+  if (!A || !B || !C) return SK_ERR_NULL;
+  int rc = check_plan(plan, M, N, K, SK_F32, plan ? plan->layout : 0);
+  if (rc) return rc;
+  const bool nn = plan->layout == SK_LAYOUT_NN;
+  if (lda < K || ldb < (nn ? N : K) || ldc < N) return SK_ERR_SHAPE;
+  if ((K % 4) || (lda % 4) || (ldb % 4) || (nn && (N % 4))) return SK_ERR_ALIGN;
+  if ((reinterpret_cast<uintptr_t>(A) & 15) || (reinterpret_cast<uintptr_t>(B) & 15) ||
+      (reinterpret_cast<uintptr_t>(C) & 3))
+    return SK_ERR_ALIGN;
+  const KernelInfo *k = kernel_by_id(plan->kernel_id);
+  if (!k || k->dtype != SK_F32 || k->layout != plan->layout) return SK_ERR_CONFIG;
+  if (lda * 4 * k->bm >= (int64_t)1 << 31 || ldb * 4 * (nn ? K : k->bn) >= (int64_t)1 << 31) return SK_ERR_SHAPE;
+  DevPlan dp;
+  Workspace w;
+  static int occ[2] = {0, 0};
+  int &o = occ[k->id == 200 ? 0 : 1];
+  if (o == 0) o = occupancy_f32(k->id);
+  rc = make_dev_plan(plan, k, ws, ws_bytes, o, (hipStream_t)stream, &dp, &w);
+  if (rc) return rc;
+  GemmArgsF32 a{(const float *)A, (const float *)B, (float *)C, (int)M, (int)N, (int)K, lda, ldb, ldc};
+  return launch_f32(k->id, a, dp, w, (hipStream_t)stream) == 0 ? SK_OK : SK_ERR_LAUNCH;
 }
 
 extern "C" int sk_gemm_q4(const void *A, const void *Wq, const void *scales, void *C, int64_t M, int64_t N,

@@ -6,6 +6,7 @@
 #include "sk_device.h"
 #include "tile_f16.h"
 #include "tile_f16_dma.h"
+#include "tile_f32.h"
 #include "tile_skinny.h"
 
 namespace sk {
@@ -16,6 +17,9 @@ int skinny_kernel_infos(KernelInfo *out, int max);
 // return hipError_t as int; occupancy_* return co-resident CTAs per CU (<= 0 on error)
 int launch_tile_f16(int id, const GemmArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s);
 int launch_skinny(int id, const SkinnyArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s);
+int f32_kernel_infos(KernelInfo *out, int max);
+int launch_f32(int id, const GemmArgsF32 &a, const DevPlan &p, const Workspace &ws, hipStream_t s);
+int occupancy_f32(int id);
 int occupancy_tile(int id);
 int occupancy_skinny(int id);
 

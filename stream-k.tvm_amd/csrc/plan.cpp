@@ -16,11 +16,13 @@ static int g_count = -1;
 
 int tile_kernel_infos(KernelInfo *out, int max);
 int skinny_kernel_infos(KernelInfo *out, int max);
+int f32_kernel_infos(KernelInfo *out, int max);
 
 const KernelInfo *kernel_table(int *count) {
   if (g_count < 0) {
     int n = tile_kernel_infos(g_table, 64);
     n += skinny_kernel_infos(g_table + n, 64 - n);
+    n += f32_kernel_infos(g_table + n, 64 - n);
     g_count = n;
   }
   if (count) *count = g_count;
@@ -69,6 +71,11 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
         best = &t[i];
     if (best) return best;
     if (dtype == SK_Q4) return nullptr;
+  }
+  if (dtype == SK_F32) {
+    for (int i = 0; i < n; ++i)
+      if (t[i].dtype == SK_F32 && t[i].layout == layout) return &t[i];
+    return nullptr;
   }
   static const int pref[][3] = {{256, 256, 64}, {128, 128, 64}, {64, 64, 64}};
   for (auto &p : pref) {

@@ -135,11 +135,16 @@ def streamk_fp32(A, B, *, layout="nn", out=None, plan=None, config=None, **kw):
     """C = A @ B in fp32 (layout 'nn', B is [K,N]: streamk_fp32.py:65-76)."""
     _check_matrix(A, "A", torch.float32)
     _check_matrix(B, "B", torch.float32)
+    if layout not in ("nt", "nn"):
+        raise ValueError("layout must be 'nn' (B is [K,N]) or 'nt' (B is [N,K])")
     M, K = A.shape
-    N = B.shape[1] if layout == "nn" else B.shape[0]
+    N, Kb = (B.shape[1], B.shape[0]) if layout == "nn" else B.shape
+    if K != Kb:
+        raise ValueError(f"K mismatch: A is {tuple(A.shape)}, B is {tuple(B.shape)}")
     if plan is None:
         plan = make_plan(M, N, K, "float32", layout, config, **kw)
     C = out if out is not None else torch.empty((M, N), dtype=torch.float32, device=A.device)
+    _check_matrix(C, "out", torch.float32)
     ws = _workspace(plan.workspace_bytes, A.device)
     rc = _lib.lib().sk_gemm_f32(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, A.stride(0),
                                 B.stride(0), C.stride(0), ctypes.byref(plan),

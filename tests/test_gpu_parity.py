@@ -247,6 +247,50 @@ def test_nn_layout(sk, oracle, cfg):
     sk.workspace_status()
 
 
+@pytest.mark.parametrize("fixup", ["atomic", "reduce"])
+def test_fp32_cfg1_and_fixture(sk, oracle, golden_dir, fixup):
+    """fp32 Stream-K GEMM: the 256 x 256 x 1024 U[-1,1) seed-0 problem of the CPU configuration
+    (there simulated with 64x64x16 tiles on 4 CTAs) on the GPU's 128x128x16 fp32-MFMA tiles, split
+    over 3 / 5 / 7 CTAs, against the oracle's CPU Stream-K run and numpy; plus the committed
+    48 x 40 x 72 fixture, the [N,K] layout and exact integer data."""
+    rng = np.random.default_rng(0)
+    A = rng.random((256, 1024), dtype=np.float32) * 2 - 1
+    B = rng.random((1024, 256), dtype=np.float32) * 2 - 1
+    ref_sim = oracle.streamk_gemm_f32(A, B, 64, 64, 16, 4, fixup=fixup)
+    ref = A.astype(np.float64) @ B.astype(np.float64)
+    for grid in (3, 5, 7, 4):
+        C = sk.streamk_fp32(_t(A), _t(B), schedule="basic", fixup=fixup, grid=grid).cpu().numpy()
+        assert oracle.max_abs_rel(C, ref) <= 1e-5
+        assert oracle.max_abs_rel(C, ref_sim) <= 1e-5
+    g = np.load(os.path.join(golden_dir, "streamk_f32_48x40x72.npz"))
+    C = sk.streamk_fp32(_t(g["A"]), _t(g["B"]), schedule="basic", fixup=fixup, grid=2).cpu().numpy()
+    assert oracle.max_abs_rel(C, g["C_reduce"]) <= 1e-5
+    # [N,K] layout and ragged shapes
+    A2 = rng.random((300, 520), dtype=np.float32) * 2 - 1
+    B2 = rng.random((200, 520), dtype=np.float32) * 2 - 1
+    C = sk.streamk_fp32(_t(A2), _t(B2), layout="nt", schedule="sk2", fixup=fixup, grid=5).cpu().numpy()
+    assert oracle.max_abs_rel(C, A2.astype(np.float64) @ B2.astype(np.float64).T) <= 1e-5
+    # exact: integer entries keep every fp32 partial sum exact
+    Ai = rng.integers(-4, 5, (260, 1032)).astype(np.float32)
+    Bi = rng.integers(-4, 5, (1032, 388)).astype(np.float32)
+    C = sk.streamk_fp32(_t(Ai), _t(Bi), schedule="basic", fixup=fixup, grid=9).cpu().numpy()
+    assert np.array_equal(C, Ai @ Bi)
+    sk.workspace_status()
+
+
+def test_fp32_reference_shape(sk, oracle):
+    """The shape the reference's fp32 script runs (16 x 16384 x 8192, streamk_fp32.py:15), B as
+    [K,N]: checked against an fp64 host product on a slice of columns."""
+    rng = np.random.default_rng(3)
+    A = rng.random((16, 8192), dtype=np.float32) * 2 - 1
+    B = rng.random((8192, 16384), dtype=np.float32) * 2 - 1
+    C = sk.streamk_fp32(_t(A), _t(B)).cpu().numpy()
+    cols = slice(4000, 4512)
+    ref = A.astype(np.float64) @ B[:, cols].astype(np.float64)
+    assert oracle.max_abs_rel(C[:, cols], ref) <= 1e-5
+    sk.workspace_status()
+
+
 def test_strided_operands_and_out(sk, oracle):
     """Leading dimensions larger than the rows, and writing into a caller-provided C."""
     import torch
