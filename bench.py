@@ -35,6 +35,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-extra", action="store_true", help="skip the sweep / Q4 section")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a 1 GiB device-to-device copy (reference point for rocprofv3 byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this library runs on one GPU; --gpus must be 1 "
@@ -93,6 +95,14 @@ def main():
             torch.cuda.synchronize()
         return st.elapsed_time(en) / (launches * replays)
 
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     # ---------------------------------------------------------------- headline: 8192^3
     M = N = K = 8192
     A, B = inputs(M, N, K)
@@ -109,6 +119,13 @@ def main():
     err = oracle.max_abs_rel(C[:64].float().cpu().numpy(), ref)
     assert err <= 1e-2, err
 
+    # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/)
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic_tile_f16_nt_dma_256x256x64_8192.json")
+    if os.path.exists(tpath):
+        with open(tpath) as f:
+            traffic = json.load(f).get("hbm_bytes_per_launch")
+
     out = {
         "metric": "fp16 Stream-K GEMM TFLOP/s (M=N=K=8192; sweep and Q4 GB/s in extra)",
         "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
@@ -120,7 +137,7 @@ def main():
                    "compute_units": cus, "check_max_abs_rel": err},
         "roofline": {"bound": "mfma", "achieved": round(kernel_tflops, 2), "peak": PEAK_FP16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(kernel_tflops / PEAK_FP16_TFLOPS, 4),
-                     "traffic": None, "kernel": f"tile_f16_nt_{plan.bm}x{plan.bn}x{plan.bk}",
+                     "traffic": traffic, "kernel": f"tile_f16_nt_dma_{plan.bm}x{plan.bn}x{plan.bk}",
                      "avg_launch_ms": round(ev_ms, 5)},
     }
 

@@ -1,0 +1,54 @@
+// Microbenchmark: time to stream 32 MB once with the small-M kernels' access pattern (a wave reads
+// 64 contiguous bytes from each of 16 rows per load) against fully contiguous 1 KB-per-wave loads.
+#include <hip/hip_runtime.h>
+#include <cstdio>
+#include <cstdint>
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+// Pattern A ("rows"): wave handles 16 rows (pitch bytes apart); lane (r=l%16,g=l/16) reads 16B at row r, byte off it*128 + c*64 + g*16.
+// Pattern B ("contig"): wave reads 1KB contiguous per load.
+template <int PATTERN, int ROT>
+__global__ __launch_bounds__(64) void stream(const char* base, uint32_t* out, int pitch, int iters_per_wave, int waves_per_rowblock) {
+  int wave = blockIdx.x, lane = threadIdx.x;
+  uint4v acc = {0, 0, 0, 0};
+  if (PATTERN == 0) {
+    int rb = wave / waves_per_rowblock, seg = wave % waves_per_rowblock;
+    const char* p = base + (size_t)(rb * 16 + (lane & 15)) * pitch + (size_t)seg * iters_per_wave * 128 + (lane >> 4) * 16;
+    int rot = ROT ? (wave * 5) % iters_per_wave : 0;
+#pragma unroll 4
+    for (int it = 0; it < iters_per_wave; ++it) {
+      int i2 = it + rot; if (i2 >= iters_per_wave) i2 -= iters_per_wave;
+      acc += *(const uint4v*)(p + i2 * 128);
+      acc += *(const uint4v*)(p + i2 * 128 + 64);
+    }
+  } else {
+    const char* p = base + (size_t)wave * iters_per_wave * 2048 + lane * 16;
+#pragma unroll 4
+    for (int it = 0; it < iters_per_wave; ++it) {
+      acc += *(const uint4v*)(p + it * 2048);
+      acc += *(const uint4v*)(p + it * 2048 + 1024);
+    }
+  }
+  out[blockIdx.x * 64 + lane] = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
+}
+template <int PATTERN, int ROT> void run(const char* name, const char* buf, uint32_t* out, int waves, int iters, int wprb) {
+  hipEvent_t a, b; hipEventCreate(&a); hipEventCreate(&b);
+  for (int i = 0; i < 3; ++i) stream<PATTERN, ROT><<<waves, 64>>>(buf, out, 4096, iters, wprb);
+  hipDeviceSynchronize();
+  hipEventRecord(a);
+  for (int i = 0; i < 20; ++i) stream<PATTERN, ROT><<<waves, 64>>>(buf, out, 4096, iters, wprb);
+  hipEventRecord(b); hipDeviceSynchronize();
+  float ms; hipEventElapsedTime(&ms, a, b); ms /= 20;
+  double bytes = (double)waves * iters * 2048;
+  printf("%-28s waves=%5d iters=%3d  %.2f us  %.0f GB/s\n", name, waves, iters, ms * 1e3, bytes / ms / 1e6);
+}
+int main() {
+  char* buf; uint32_t* out; hipMalloc(&buf, 64 << 20); hipMalloc(&out, 1 << 22); hipMemset(buf, 1, 64 << 20);
+  // 32 MB = 8192 rows x 4096 B.  rowblocks = 512; each row = 32 iterations of 128B.
+  for (int wprb : {1, 2, 4, 8}) {
+    int waves = 512 * wprb, iters = 32 / wprb;
+    run<0, 0>("rows", buf, out, waves, iters, wprb);
+    run<0, 1>("rows+rot", buf, out, waves, iters, wprb);
+    run<1, 0>("contig", buf, out, waves, iters, wprb);
+  }
+  return 0;
+}

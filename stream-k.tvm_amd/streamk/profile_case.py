@@ -1,0 +1,49 @@
+"""Runs one GEMM case a few times so that a profiler sees nothing else.
+
+    rocprofv3 --kernel-trace --stats -- python3 stream-k.tvm_amd/streamk/profile_case.py 8192x8192x8192
+    python3 stream-k.tvm_amd/streamk/profile_case.py 1x8192x8192 --dtype q4 --config "dict(grid=256)"
+"""
+import argparse
+import os
+import sys
+
+sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("shape", help="MxNxK")
+    ap.add_argument("--dtype", default="float16", choices=["float16", "float32", "q4"])
+    ap.add_argument("--layout", default="nt", choices=["nt", "nn"])
+    ap.add_argument("--config", default="{}", help="python dict of plan options, e.g. \"dict(bm=256,bn=256,raster=8)\"")
+    ap.add_argument("--reps", type=int, default=5)
+    args = ap.parse_args()
+    import torch
+    import streamk
+
+    M, N, K = (int(x) for x in args.shape.split("x"))
+    cfg = eval(args.config, {"dict": dict})  # noqa: S307 (developer tool)
+    g = torch.Generator(device="cpu").manual_seed(0)
+    plan = streamk.make_plan(M, N, K, args.dtype, args.layout, cfg)
+    if args.dtype == "q4":
+        A = torch.randn(M, K, generator=g).half().cuda()
+        Wq = torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8).cuda()
+        sc = (torch.rand(N, K // 128, generator=g) * 0.015 + 0.005).half().cuda()
+        run = lambda: streamk.streamk_q4(A, Wq, sc, plan=plan)  # noqa: E731
+    else:
+        dt = torch.float16 if args.dtype == "float16" else torch.float32
+        A = (torch.rand(M, K, generator=g) * 2 - 1).to(dt).cuda()
+        bshape = (N, K) if args.layout == "nt" else (K, N)
+        B = (torch.rand(*bshape, generator=g) * 2 - 1).to(dt).cuda()
+        fn = streamk.streamk_fp16 if args.dtype == "float16" else streamk.streamk_fp32
+        run = lambda: fn(A, B, layout=args.layout, plan=plan)  # noqa: E731
+    for _ in range(args.reps):
+        run()
+    torch.cuda.synchronize()
+    streamk.workspace_status()
+    print(f"ran {args.reps} x {args.dtype} {args.layout} {M}x{N}x{K} kernel {plan.kernel_id} grid {plan.grid} "
+          f"streamk_tiles {plan.streamk_tiles}")
+
+
+if __name__ == "__main__":
+    main()
