@@ -132,23 +132,22 @@ struct TileF16NTDma {
       kstep_b = (uint32_t)(BK * a.ldb * 2);
     }
 
+    // one wave-wide load of stage `st` for K-iteration kt: x < A_DMA loads rows of A, the rest B
+    auto dma_one = [&](char *st, int kt, int x) {
+      const bool tail_oob = (kt == tail_kt) && (kt * BK + my_chunk * 8 >= a.K);
+      if (x < A_DMA) {
+        const int g = wave + x * NW;
+        dma_load_16(rsrc_a, lds_address(st) + g * 1024, tail_oob ? OOB_OFFSET : voff_a,
+                    (uint32_t)kt * (BK * 2) + g * grp_a);
+      } else {
+        const int g = wave + (x - A_DMA) * NW;
+        dma_load_16(rsrc_b, lds_address(st) + A_BYTES + g * 1024, (tail_oob && !B_KN) ? OOB_OFFSET : voff_b,
+                    (uint32_t)kt * kstep_b + g * grp_b);
+      }
+    };
     auto issue_dma = [&](char *st, int kt) {
-      const uint32_t koff = (uint32_t)kt * (BK * 2);
-      uint32_t va = voff_a, vb = voff_b;
-      if (kt == tail_kt && kt * BK + my_chunk * 8 >= a.K) {
-        va = OOB_OFFSET;
-        if (!B_KN) vb = OOB_OFFSET;
-      }
 #pragma unroll
-      for (int j = 0; j < A_DMA; ++j) {
-        const int g = wave + j * NW;
-        dma_load_16(rsrc_a, lds_address(st) + g * 1024, va, koff + g * grp_a);
-      }
-#pragma unroll
-      for (int j = 0; j < B_DMA; ++j) {
-        const int g = wave + j * NW;
-        dma_load_16(rsrc_b, lds_address(st) + A_BYTES + g * 1024, vb, (uint32_t)kt * kstep_b + g * grp_b);
-      }
+      for (int x = 0; x < DMA_PER_WAVE; ++x) dma_one(st, kt, x);
     };
 
     // fragment addressing: lane (r = lane%32, g = lane/32) reads row r of a 32-row block, logical
