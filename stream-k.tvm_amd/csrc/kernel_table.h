@@ -21,22 +21,16 @@ struct KernelInfo {
   int family;
   int dtype;    // sk_dtype
   int layout;   // sk_layout
-  int variant;  // 0: registers -> padded LDS rows; 1: direct global -> LDS loads, swizzled rows;
-                // 2: as 1 with four waves per CTA (one per SIMD, accumulators in AGPRs)
+  int variant;  // tile kernels -- 0: registers -> padded LDS rows; 1: direct global -> LDS loads,
+                // swizzled rows; 2: as 1 with four waves per CTA (one per SIMD, accumulators in AGPRs)
+                // small-M kernels -- 0: up to 16*MB rows of A; 1: M == 1; 2: M == 1, Q4 matrix-vector
   int bm, bn, bk;  // CTA tile; bk is the K extent of one CTA iteration
   int threads;
   int lds_bytes;
   int ctas_per_cu;    // co-resident CTAs per CU the kernel is compiled for
   int partial_elems;  // fp32 elements of one partial tile in the workspace
   int max_ipt;        // largest iterations-per-tile the kernel supports (0 = unlimited)
-  int max_m;          // the same for the NN layout (B is [K,N]), fragments through transposing LDS reads:  X(id, BM, BN, WM, WN)
-#define SK_TILE_F16_NN_DMA_KERNELS(X) \
-  X(20, 256, 256, 2, 4)               \
-  X(21, 128, 128, 2, 2)               \
-  X(22, 128, 256, 2, 4)               \
-  X(23, 256, 128, 4, 2)
-
-// small-M kernels: largest M the kernel accepts
+  int max_m;          // small-M kernels: largest M the kernel accepts (0 = unlimited)
   int k_align;        // K must be a multiple of this
   const char *name;
 };
@@ -86,6 +80,17 @@ struct KernelInfo {
   X(128, 1, 2, 2, 1, 1, 4, 1)    \
   X(129, 1, 4, 1, 1, 1, 2, 1)    \
   X(130, 1, 2, 1, 2, 1, 4, 1)
+
+// M == 1 Q4 matrix-vector kernels (variant 2):  X(id, NB, WN, RK, DEPTH)
+#define SK_GEMV_Q4_KERNELS(X) \
+  X(140, 1, 4, 1, 4)          \
+  X(141, 1, 2, 2, 4)          \
+  X(142, 1, 1, 4, 4)          \
+  X(143, 2, 4, 1, 2)          \
+  X(144, 2, 2, 2, 2)          \
+  X(145, 1, 2, 1, 4)          \
+  X(146, 1, 1, 2, 4)          \
+  X(147, 1, 1, 1, 4)
 
 const KernelInfo *kernel_table(int *count);
 const KernelInfo *kernel_by_id(int id);

@@ -25,6 +25,15 @@ int skinny_kernel_infos(KernelInfo *out, int max) {
   }
   SK_SKINNY_KERNELS(X)
 #undef X
+#define X(id, NB, WN, RK, DEPTH)                                                                          \
+  if (n < max) {                                                                                         \
+    typedef TileGemvQ4<NB, WN, RK, DEPTH> P;                                                             \
+    out[n++] = KernelInfo{id, FAMILY_SKINNY, 2, 0, 2, P::BM, P::BN, P::BKC, P::NT, P::LDS_BYTES,         \
+                          P::CTAS_PER_CU, P::TILE_ELEMS, P::MAX_ITERS, P::MAX_M, 128,                    \
+                          "gemv_q4_nb" #NB "_wn" #WN "_rk" #RK};                                         \
+  }
+  SK_GEMV_Q4_KERNELS(X)
+#undef X
   return n;
 }
 
@@ -37,6 +46,14 @@ int launch_skinny(int id, const SkinnyArgs &a, const DevPlan &p, const Workspace
     return (int)hipGetLastError();                                                         \
   }
     SK_SKINNY_KERNELS(X)
+#undef X
+#define X(id_, NB, WN, RK, DEPTH)                                                          \
+  case id_: {                                                                              \
+    typedef TileGemvQ4<NB, WN, RK, DEPTH> P;                                               \
+    hipLaunchKernelGGL(sk_skinny_kernel<P>, dim3(p.grid), dim3(P::NT), 0, s, a, p, ws);    \
+    return (int)hipGetLastError();                                                         \
+  }
+    SK_GEMV_Q4_KERNELS(X)
 #undef X
   }
   return (int)hipErrorInvalidValue;
@@ -53,6 +70,15 @@ int occupancy_skinny(int id) {
     return occ;                                                                                       \
   }
     SK_SKINNY_KERNELS(X)
+#undef X
+#define X(id_, NB, WN, RK, DEPTH)                                                                        \
+  case id_: {                                                                                            \
+    typedef TileGemvQ4<NB, WN, RK, DEPTH> P;                                                             \
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_skinny_kernel<P>, P::NT, 0) != hipSuccess) \
+      return -1;                                                                                         \
+    return occ;                                                                                          \
+  }
+    SK_GEMV_Q4_KERNELS(X)
 #undef X
   }
   return -1;

@@ -11,7 +11,7 @@
 
 namespace sk {
 
-static KernelInfo g_table[64];
+static KernelInfo g_table[128];
 static int g_count = -1;
 
 int tile_kernel_infos(KernelInfo *out, int max);
@@ -20,9 +20,9 @@ int f32_kernel_infos(KernelInfo *out, int max);
 
 const KernelInfo *kernel_table(int *count) {
   if (g_count < 0) {
-    int n = tile_kernel_infos(g_table, 64);
-    n += skinny_kernel_infos(g_table + n, 64 - n);
-    n += f32_kernel_infos(g_table + n, 64 - n);
+    int n = tile_kernel_infos(g_table, 128);
+    n += skinny_kernel_infos(g_table + n, 128 - n);
+    n += f32_kernel_infos(g_table + n, 128 - n);
     g_count = n;
   }
   if (count) *count = g_count;
@@ -39,8 +39,15 @@ const KernelInfo *kernel_by_id(int id) {
 
 static int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
-// preference among kernel variants of one tile shape when the caller does not ask for one
-static int variant_rank(int v) { return v == 1 ? 2 : (v == 2 ? 1 : 0); }
+// preference among kernel variants of one tile shape when the caller does not ask for one: the
+// eight-wave direct-to-LDS tile kernels; the most specialised small-M kernel that accepts the shape
+static int variant_rank(const KernelInfo &k) {
+  if (k.family == FAMILY_SKINNY) return k.variant;
+  return k.variant == 1 ? 2 : (k.variant == 2 ? 1 : 0);
+}
+static bool accepts_shape(const KernelInfo &k, int64_t M, int64_t K) {
+  return (k.max_m == 0 || M <= k.max_m) && (k.max_ipt == 0 || (K + k.bk - 1) / k.bk <= k.max_ipt);
+}
 
 static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype, int layout,
                                      const sk_config *cfg, int num_cus) {
@@ -54,8 +61,7 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
     for (int i = 0; i < n; ++i)
       if (t[i].dtype == dtype && t[i].layout == layout && t[i].bm == cfg->bm && t[i].bn == cfg->bn &&
           (cfg->bk <= 0 || t[i].bk == cfg->bk) && (want_variant < 0 || t[i].variant == want_variant) &&
-          (t[i].max_m == 0 || M <= t[i].max_m) &&
-          (found == nullptr || variant_rank(t[i].variant) > variant_rank(found->variant)))
+          accepts_shape(t[i], M, K) && (found == nullptr || variant_rank(t[i]) > variant_rank(*found)))
         found = &t[i];
     return found;
   }
@@ -66,7 +72,7 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
     int mb = M <= 16 ? 16 : (M <= 32 ? 32 : 64);
     for (int i = 0; i < n; ++i)
       if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].bm == mb && t[i].bn == 64 &&
-          M <= t[i].max_m && (want_variant < 0 || t[i].variant == want_variant) &&
+          accepts_shape(t[i], M, K) && (want_variant < 0 || t[i].variant == want_variant) &&
           (best == nullptr || t[i].variant > best->variant))
         best = &t[i];
     if (best) return best;
@@ -82,7 +88,7 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
     for (int i = 0; i < n; ++i) {
       if (t[i].family != FAMILY_TILE || t[i].dtype != dtype || t[i].layout != layout) continue;
       if (t[i].bm != p[0] || t[i].bn != p[1] || t[i].bk != p[2]) continue;
-      if (want_variant >= 0 ? t[i].variant != want_variant : (best != nullptr && variant_rank(t[i].variant) < variant_rank(best->variant))) continue;
+      if (want_variant >= 0 ? t[i].variant != want_variant : (best != nullptr && variant_rank(t[i]) < variant_rank(*best))) continue;
       int64_t tiles = cdiv(M, p[0]) * cdiv(N, p[1]);
       int64_t iters = tiles * cdiv(K, p[2]);
       // enough K-iterations per CU that a split tile still amortises its fix-up

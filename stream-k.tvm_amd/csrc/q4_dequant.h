@@ -19,25 +19,35 @@ namespace sk {
 // FMAs, four packed multiplies.  Nibbles sitting at bits 4..7 of a half are OR-ed in place, which
 // yields 1024 + 16*q; fma(x, 1/16, -(64 + zero)) = q - zero exactly, saving the shift.
 struct Q4Consts {
-  uint32_t magic;  // 0x64006400 in a VGPR (v_and_or_b32 takes a single scalar operand)
-  half2v bias_lo;  // 1024 + zero
-  half2v bias_hi;  // -(64 + zero)
+  uint32_t magic;    // 0x64006400 in a VGPR (v_and_or_b32 takes a single scalar operand)
+  uint32_t mask_lo;  // 0x000F000F: nibbles at bits 0..3 of each half
+  uint32_t mask_hi;  // 0x00F000F0: nibbles at bits 4..7 of each half
+  half2v bias_lo;    // 1024 + zero
+  half2v bias_hi;    // -(64 + zero)
   half2v sixteenth;
 };
+// The three bit patterns are made opaque to the optimiser (empty asm statements that only pin the
+// register class), so that (x & mask) | magic is selected as one v_and_or_b32 with the mask in an
+// SGPR and the magic in a VGPR instead of being split around literal constants.  The operation
+// itself stays ordinary code: the compiler must see it to keep MFMA hazards covered.
+__device__ __forceinline__ void q4_pin_patterns(Q4Consts &c) {
+  c.magic = 0x64006400u;
+  c.mask_lo = 0x000F000Fu;
+  c.mask_hi = 0x00F000F0u;
+  asm volatile("" : "+v"(c.magic));
+  asm volatile("" : "+s"(c.mask_lo));
+  asm volatile("" : "+s"(c.mask_hi));
+}
 __device__ __forceinline__ Q4Consts q4_consts(int zero) {
   Q4Consts c;
-  c.magic = 0x64006400u;
+  q4_pin_patterns(c);
   const half_t lo = (half_t)(float)(1024 + zero), hi = (half_t)(float)(-(64 + zero));
   c.bias_lo = half2v{lo, lo};
   c.bias_hi = half2v{hi, hi};
   c.sixteenth = half2v{(half_t)0.0625f, (half_t)0.0625f};
   return c;
 }
-__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t bits) {
-  uint32_t r;
-  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "s"(mask), "v"(bits));
-  return r;
-}
+__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t bits) { return (x & mask) | bits; }
 __device__ __forceinline__ half8v dequant_word_q4(uint32_t w, const Q4Consts &c, half2v scale) {
   union {
     uint32_t u[4];
@@ -45,10 +55,10 @@ __device__ __forceinline__ half8v dequant_word_q4(uint32_t w, const Q4Consts &c,
     half8v v;
   } r;
   const uint32_t t = w >> 8;
-  r.u[0] = and_or(w, 0x000F000Fu, c.magic);
-  r.u[1] = and_or(w, 0x00F000F0u, c.magic);
-  r.u[2] = and_or(t, 0x000F000Fu, c.magic);
-  r.u[3] = and_or(t, 0x00F000F0u, c.magic);
+  r.u[0] = and_or(w, c.mask_lo, c.magic);
+  r.u[1] = and_or(w, c.mask_hi, c.magic);
+  r.u[2] = and_or(t, c.mask_lo, c.magic);
+  r.u[3] = and_or(t, c.mask_hi, c.magic);
   r.h[0] = (r.h[0] - c.bias_lo) * scale;
   r.h[1] = __builtin_elementwise_fma(r.h[1], c.sixteenth, c.bias_hi) * scale;
   r.h[2] = (r.h[2] - c.bias_lo) * scale;

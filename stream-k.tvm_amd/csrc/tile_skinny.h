@@ -31,6 +31,29 @@ struct SkinnyArgs {
   int groups;             // Q4: scales per row
 };
 
+// Copies the scales of groups [g0, g0 + 8*chunks) of the tile's BN weight rows to LDS rows of SC_ROW
+// halfs, 16 bytes at a time.  A 16-byte piece that would run past the end of its row (K / group
+// not a multiple of 8) is fetched half by half instead: on the tile's last row a vector load would
+// cross the end of the buffer, and the hardware then zeroes the straddling dword.
+template <int BN, int SC_ROW, int NT>
+__device__ __forceinline__ void stage_scales(half_t *ldsS, const half_t *scales_tile, int rows, int groups, int g0,
+                                             int chunks) {
+  const BufferRsrc rsrc_s = make_rsrc(scales_tile, (uint32_t)(rows * groups * 2));
+  for (int idx = threadIdx.x; idx < BN * chunks; idx += NT) {
+    const int r = idx % BN, c = idx / BN, g = g0 + c * 8;
+    half_t *dst = ldsS + r * SC_ROW + c * 8;
+    if (g + 8 <= groups) {
+      *reinterpret_cast<uint4v *>(dst) = buffer_load_16(rsrc_s, (uint32_t)(r * groups + g) * 2, 0);
+    } else {
+      for (int e = 0; e < 8; ++e) {
+        const uint16_t v =
+            g + e < groups ? __builtin_amdgcn_raw_buffer_load_b16(rsrc_s, (uint32_t)(r * groups + g + e) * 2, 0, 0) : 0;
+        dst[e] = __builtin_bit_cast(half_t, v);
+      }
+    }
+  }
+}
+
 // ROW1_: M == 1 only.  A single row of A is staged and every lane reads it (an LDS broadcast);
 // rows 1..15 of the MFMA result are then copies of row 0 and are never stored.
 template <int MB_, int NB_, int WN_, int RK_, bool Q4_, int DEPTH_, bool ROW1_ = false>
@@ -176,13 +199,7 @@ struct TileSkinny {
       const int g_first = k0 * SC_PER_ITER, g0 = g_first & ~7;
       sc_shift = g_first - g0;
       const int chunks = (sc_shift + n * SC_PER_ITER + 7) >> 3;
-      const BufferRsrc rsrc_s =
-          make_rsrc(a.scales + (int64_t)pn * BN * a.groups, (uint32_t)(rows_w * a.groups * 2));
-      for (int idx = tid; idx < BN * chunks; idx += NT) {
-        const int r = idx % BN, c = idx / BN;
-        const uint4v v = buffer_load_16(rsrc_s, (uint32_t)(r * a.groups + g0 + c * 8) * 2, 0);
-        *reinterpret_cast<uint4v *>(ldsS + r * SC_ROW + c * 8) = v;
-      }
+      stage_scales<BN, SC_ROW, NT>(ldsS, a.scales + (int64_t)pn * BN * a.groups, rows_w, a.groups, g0, chunks);
     }
     stage_a(0, 0);
     __syncthreads();

@@ -158,9 +158,76 @@ def test_cfg4_q4_gemm(sk, oracle, M):
     W = sk.dequant_q4(dW, dS).cpu().numpy()
     assert np.array_equal(W.view(np.uint16), oracle.dequant_q4(Wq, sc, 128, 8).view(np.uint16))
     for cfg in (dict(fixup="reduce"), dict(fixup="atomic"), dict(schedule="dp"),
-                dict(bm=16, bn=16, bk=1024), dict(bm=16, bn=32, bk=512), dict(schedule="basic", grid=1000)):
+                dict(bm=16, bn=16, bk=1024), dict(bm=16, bn=32, bk=512), dict(schedule="basic", grid=700)):
         C = sk.streamk_q4(dA, dW, dS, **cfg)
         assert _rel(oracle, C, ref) <= 2e-3 <= TOL, cfg
+    sk.workspace_status()
+
+
+Q4_TILES = [(16, 64, 256), (16, 32, 512), (16, 16, 1024), (16, 128, 256), (16, 64, 512), (16, 32, 256),
+            (16, 16, 512), (16, 16, 256), (32, 64, 256), (64, 64, 256)]
+
+
+@pytest.mark.parametrize("variant", [1, 2, 3], ids=["general", "row1", "gemv"])
+def test_q4_ragged_shapes_every_kernel(sk, oracle, variant):
+    """Every Q4 kernel instance (general small-M, single-row, matrix-vector) on ragged shapes: N not
+    a multiple of the tile, K a multiple of 128 only (a scale row shorter than one 16-byte piece, a
+    last iteration hanging over K), zero points 0 / 5 / 8 / 15, all three schedules.  The
+    matrix-vector kernels accumulate unrounded (q - zero) * scale products in fp32, the others
+    multiply fp16-rounded weights; both stay within 2e-3 of the fp32 host product of the
+    dequantised weights."""
+    rng = np.random.default_rng(50 + variant)
+    shapes = [(1, 1000, 1152, 8), (1, 520, 384, 15), (1, 72, 4096, 0), (1, 2048, 16384, 5)]
+    if variant == 1:
+        shapes += [(5, 1000, 1152, 8), (16, 520, 384, 15), (33, 200, 640, 8), (64, 136, 2048, 3)]
+    ran = 0
+    for (M, N, K, zero) in shapes:
+        A = (rng.random((M, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+        Wq = rng.integers(0, 256, (N, K // 2), dtype=np.uint8)
+        sc = rng.uniform(0.005, 0.02, (N, K // 128)).astype(np.float16)
+        ref = oracle.q4_gemm_ref(A, Wq, sc, 128, zero)
+        dA, dW, dS = _t(A), _t(Wq), _t(sc)
+        for (bm, bn, bk) in Q4_TILES:
+            for sch in (dict(schedule="dp"), dict(schedule="sk2", fixup="reduce", grid=48),
+                        dict(schedule="sk2", fixup="atomic", grid=40)):
+                try:
+                    plan = sk.make_plan(M, N, K, "q4", "nt", dict(bm=bm, bn=bn, bk=bk, variant=variant, **sch))
+                except sk.StreamKError:
+                    continue  # no such instance of this variant, or it does not take this M / K
+                C = sk.streamk_q4(dA, dW, dS, zero=zero, plan=plan)
+                assert _rel(oracle, C, ref) <= 2e-3 <= TOL, (M, N, K, zero, bm, bn, bk, sch, plan.kernel_id)
+                ran += 1
+    assert ran >= 40
+    sk.workspace_status()
+
+
+def test_q4_matrix_vector_exact_on_integer_data(sk):
+    """M = 1, N = K = 8192, A in {-1, 0, 1}, scales 1 (and 0.5): every group sum is an integer
+    below 2^24, so the fp32 arithmetic of the matrix-vector kernels is exact and C must equal the
+    integer product bit for bit, for every kernel instance, schedule and fix-up."""
+    import torch
+    N = K = 8192
+    rng = np.random.default_rng(61)
+    A = rng.integers(-1, 2, (1, K)).astype(np.int64)
+    Wq = rng.integers(0, 256, (N, K // 2), dtype=np.uint8)
+    q = np.empty((N, K), dtype=np.int64)
+    q[:, 0::2], q[:, 1::2] = Wq & 15, Wq >> 4
+    exact = (q - 8) @ A[0]
+    assert np.abs(exact).max() < 2048
+    dA, dW = _t(A.astype(np.float16)), _t(Wq)
+    ones = torch.ones(N, K // 128, dtype=torch.float16, device="cuda")
+    for (bm, bn, bk) in Q4_TILES[:8]:
+        for sch in (dict(schedule="dp"), dict(schedule="sk2", fixup="reduce"), dict(schedule="sk2", fixup="atomic"),
+                    dict(schedule="basic", fixup="reduce", grid=1000)):
+            try:
+                plan = sk.make_plan(1, N, K, "q4", "nt", dict(bm=bm, bn=bn, bk=bk, variant=3, **sch))
+            except sk.StreamKError:
+                assert "grid" in sch  # more CTAs than this instance keeps resident
+                continue
+            C = sk.streamk_q4(dA, dW, ones, zero=8, plan=plan)
+            assert np.array_equal(C.cpu().numpy()[0].astype(np.int64), exact), (bm, bn, bk, sch)
+            C = sk.streamk_q4(dA, dW, ones * 0.5, zero=8, plan=plan)
+            assert np.array_equal((C.double() * 2).cpu().numpy()[0].astype(np.int64), exact), (bm, bn, bk, sch)
     sk.workspace_status()
 
 
