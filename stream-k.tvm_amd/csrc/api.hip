@@ -92,6 +92,15 @@ int make_dev_plan(const sk_plan *plan, const KernelInfo *k, void *ws, size_t ws_
   dp->raster = plan->raster;
   dp->spin_limit = plan->spin_limit > 0 ? plan->spin_limit : (1 << 22);
   dp->xcd_remap = (plan->grid % 8 == 0) ? 1 : 0;
+  const int raster = plan->raster > 0 ? plan->raster : 1;
+  dp->raster_tail = plan->num_block_m % raster ? plan->num_block_m % raster : raster;
+  dp->by_ipt = FastDiv::make(plan->iters_per_tile);
+  dp->by_tiles_n = FastDiv::make(plan->num_block_n);
+  dp->by_width = FastDiv::make((uint32_t)raster * plan->num_block_n);
+  dp->by_raster = FastDiv::make(raster);
+  dp->by_tail = FastDiv::make(dp->raster_tail);
+  dp->by_full1 = FastDiv::make(plan->streamk_full_tiles + 1);
+  dp->by_full = FastDiv::make(plan->streamk_full_tiles > 0 ? plan->streamk_full_tiles : 1);
   w->status = nullptr; w->flags = nullptr; w->partials = nullptr;
   if (plan->workspace_bytes > 0) {
     char *base = static_cast<char *>(ws);

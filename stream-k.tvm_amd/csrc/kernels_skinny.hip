@@ -3,6 +3,9 @@
 #include "sk_persistent.h"
 
 namespace sk {
+#ifdef SK_PHASE_TRACE
+__device__ long long g_trace_buf[2048 * 16];
+#endif
 
 template <class P>
 __global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_skinny_kernel(typename P::Args a, DevPlan plan, Workspace ws) {
@@ -28,7 +31,7 @@ int skinny_kernel_infos(KernelInfo *out, int max) {
 #define X(id, NB, WN, RK, DEPTH)                                                                          \
   if (n < max) {                                                                                         \
     typedef TileGemvQ4<NB, WN, RK, DEPTH> P;                                                             \
-    out[n++] = KernelInfo{id, FAMILY_SKINNY, 2, 0, 2, P::BM, P::BN, P::BKC, P::NT, P::LDS_BYTES,         \
+    out[n++] = KernelInfo{id, FAMILY_SKINNY, 2, 0, (DEPTH) == 8 ? 3 : 2, P::BM, P::BN, P::BKC, P::NT, P::LDS_BYTES,         \
                           P::CTAS_PER_CU, P::TILE_ELEMS, P::MAX_ITERS, P::MAX_M, 128,                    \
                           "gemv_q4_nb" #NB "_wn" #WN "_rk" #RK};                                         \
   }
@@ -85,3 +88,9 @@ int occupancy_skinny(int id) {
 }
 
 }  // namespace sk
+
+#ifdef SK_PHASE_TRACE
+extern "C" int sk_debug_trace_read(long long *out) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(sk::g_trace_buf), sizeof(long long) * 2048 * 16);
+}
+#endif

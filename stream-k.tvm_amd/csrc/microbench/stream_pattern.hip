@@ -20,6 +20,23 @@ __global__ __launch_bounds__(64) void stream(const char* base, uint32_t* out, in
       acc += *(const uint4v*)(p + i2 * 128);
       acc += *(const uint4v*)(p + i2 * 128 + 64);
     }
+  } else if (PATTERN >= 2) {
+    // PATTERN 2: 4 rows x 256 contiguous bytes per load (lane l: row l/16, piece l%16)
+    // PATTERN 3: 8 rows x 128 bytes (row l/8, piece l%8); PATTERN 4: 16 rows x 64 bytes with the four
+    // lanes of a row adjacent (row l/4, piece l%4).  A wave still owns 16 rows x (iters*128) bytes.
+    constexpr int LPR = PATTERN == 2 ? 16 : (PATTERN == 3 ? 8 : 4);   // lanes per row
+    constexpr int RPL = 64 / LPR;                                     // rows per load
+    constexpr int LOADS = 16 / RPL;                                   // loads to cover 16 rows
+    int rb = wave / waves_per_rowblock, seg = wave % waves_per_rowblock;
+    const char* p = base + (size_t)(rb * 16 + lane / LPR) * pitch + (size_t)seg * iters_per_wave * 128 + (lane % LPR) * 16;
+    // per "iteration" the wave consumes 2 KB: LOADS row groups x (2048 / LOADS / RPL) bytes per row
+    constexpr int BYTES_PER_ROW = LPR * 16;
+    const int steps = iters_per_wave * 128 / BYTES_PER_ROW;  // steps along K
+#pragma unroll(8 / LOADS)
+    for (int st = 0; st < steps; ++st) {
+#pragma unroll
+      for (int g = 0; g < LOADS; ++g) acc += *(const uint4v*)(p + (size_t)g * RPL * pitch + st * BYTES_PER_ROW);
+    }
   } else {
     const char* p = base + (size_t)wave * iters_per_wave * 2048 + lane * 16;
 #pragma unroll 4
@@ -49,6 +66,9 @@ int main() {
     run<0, 0>("rows", buf, out, waves, iters, wprb);
     run<0, 1>("rows+rot", buf, out, waves, iters, wprb);
     run<1, 0>("contig", buf, out, waves, iters, wprb);
+    if (iters * 128 >= 256) run<2, 0>("4rows x 256B", buf, out, waves, iters, wprb);
+    run<3, 0>("8rows x 128B", buf, out, waves, iters, wprb);
+    run<4, 0>("16rows x 64B, quads", buf, out, waves, iters, wprb);
   }
   return 0;
 }

@@ -69,11 +69,18 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
   // every CU something to do
   const KernelInfo *best = nullptr;
   if ((M <= 64 && layout == SK_LAYOUT_NT) || dtype == SK_Q4) {
+    // M == 1 with Q4 weights: the matrix-vector kernel with four waves splitting K (data-parallel
+    // over 16-row tiles), the fastest instance at LLM-sized N and K
+    if (dtype == SK_Q4 && M == 1 && want_variant < 0)
+      for (int i = 0; i < n; ++i)
+        if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].variant == 2 && t[i].bn == 16 &&
+            t[i].bk == 1024 && accepts_shape(t[i], M, K))
+          return &t[i];
     int mb = M <= 16 ? 16 : (M <= 32 ? 32 : 64);
     for (int i = 0; i < n; ++i)
       if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].bm == mb && t[i].bn == 64 &&
           accepts_shape(t[i], M, K) && (want_variant < 0 || t[i].variant == want_variant) &&
-          (best == nullptr || t[i].variant > best->variant))
+          t[i].variant <= 2 && (best == nullptr || t[i].variant > best->variant))
         best = &t[i];
     if (best) return best;
     if (dtype == SK_Q4) return nullptr;
@@ -129,16 +136,27 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
   out->total_tiles = total;
 
   // every CTA of the Stream-K wave may wait for another one, so the grid is capped at what the
-  // device keeps resident; a small problem gets a smaller grid (at least 4 K-iterations per CTA)
+  // device keeps resident.  A small problem gets a smaller grid: a split tile keeps at least 4
+  // K-iterations per CTA, but there are never fewer CTAs than tiles (as far as they fit).
   const int occ = k->ctas_per_cu;
-  int grid = cfg && cfg->grid > 0 ? cfg->grid : num_cus * occ;
-  if (grid > num_cus * occ) return SK_ERR_CONFIG;
+  const int max_grid = num_cus * occ;
+  int grid = cfg && cfg->grid > 0 ? cfg->grid : max_grid;
+  if (grid > max_grid) return SK_ERR_CONFIG;
   if (!(cfg && cfg->grid > 0)) {
     const int64_t iters = total64 * out->iters_per_tile;
-    if (iters / 4 < grid) grid = (int)(iters / 4 > 8 ? (iters / 4) / 8 * 8 : (iters < 8 ? iters : 8));
+    const int64_t tiles_fit = total64 < max_grid ? total64 : max_grid;
+    int64_t want = iters / 4 > tiles_fit ? iters / 4 : tiles_fit;
+    if (want < grid) grid = (int)(want > 8 && want != total64 ? want / 8 * 8 : want);
   }
   int sched = cfg ? cfg->schedule : SK_SCHED_AUTO;
-  if (sched == SK_SCHED_AUTO) sched = (total % grid == 0) ? SK_SCHED_DP : SK_SCHED_SK_TWO_TILE;
+  if (sched == SK_SCHED_AUTO) {
+    // data-parallel when the last wave of tiles is (nearly) full: Stream-K's fix-up and the L2
+    // reuse it gives up cost more than a tail of under 10 %.  Otherwise Stream-K, splitting only
+    // the remainder tiles when there are at least two full waves beside them.
+    const int64_t waves = (total64 + grid - 1) / grid;
+    if (total64 * 10 >= waves * grid * 9) sched = SK_SCHED_DP;
+    else sched = total64 >= 2 * (int64_t)grid ? SK_SCHED_SK_ONE_TILE : SK_SCHED_SK_TWO_TILE;
+  }
   // a data-parallel-only launch never has more CTAs than tiles (idle CTAs would also skew the
   // CTA -> XCD mapping: the low logical ids sit on the first XCDs)
   if (sched == SK_SCHED_DP && grid > total) grid = total;

@@ -16,6 +16,39 @@ typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 
 enum { FIXUP_ATOMIC = 1, FIXUP_REDUCE = 2 };
 
+// Phase tracing (off unless the small-M translation unit is built with -DSK_PHASE_TRACE): thread 0
+// of every CTA stores the 100 MHz wall clock into slot `slot` of its row of g_trace_buf; the host
+// reads the table back with sk_debug_trace_read.  Slots: 0 kernel entry, 1-7 inside the
+// matrix-vector kernel's segment (loads issued, A staged, scales staged, barrier, loop start,
+// loop end), 8/9 before/after the store of C, 10/11 after the CTA's range / tile coordinates.
+#ifdef SK_PHASE_TRACE
+extern __device__ long long g_trace_buf[2048 * 16];
+#define SK_TRACE(slot)                                                              \
+  do {                                                                              \
+    if (threadIdx.x == 0) g_trace_buf[blockIdx.x * 16 + (slot)] = wall_clock64();  \
+  } while (0)
+#else
+#define SK_TRACE(slot)
+#endif
+
+// Division of a non-negative 32-bit integer by a divisor known on the host: the host stores
+// mul = floor(2^32 (2^shift - d) / d) + 1 with shift = ceil(log2 d), and
+// n / d == (umulhi(n, mul) + n) >> shift for every 0 <= n < 2^31.  The kernels divide wave-uniform
+// values only, so this is a handful of scalar instructions instead of a reciprocal sequence.
+struct FastDiv {
+  uint32_t mul, shift;
+#if defined(__HIPCC__)
+  __device__ __forceinline__ int div(int n) const { return (int)((__umulhi((uint32_t)n, mul) + (uint32_t)n) >> shift); }
+#endif
+  static FastDiv make(uint32_t d) {
+    FastDiv f{1u, 0u};
+    if (d <= 1) return f;
+    while ((1ull << f.shift) < d) ++f.shift;
+    f.mul = (uint32_t)((((1ull << f.shift) - d) << 32) / d + 1);
+    return f;
+  }
+};
+
 struct DevPlan {
   int tiles_m, tiles_n, ipt;  // tile grid, K-iterations per tile
   int total_tiles, sk_tiles;  // Stream-K tiles are ids [0, sk_tiles)
@@ -25,6 +58,8 @@ struct DevPlan {
   int raster;                 // 0 row-major, g > 0 grouped by g tile rows
   int spin_limit;             // polls before a waiting owner gives up
   int xcd_remap;              // 1: spread logical CTA ids so each XCD owns a contiguous range
+  int raster_tail;            // tile rows in the last raster group (tiles_m % raster, or raster)
+  FastDiv by_ipt, by_tiles_n, by_width, by_raster, by_tail, by_full1, by_full;
 };
 
 struct Workspace {
@@ -47,17 +82,21 @@ __device__ __forceinline__ void sk_range(const DevPlan &p, int pid, int &start, 
 }
 
 __device__ __forceinline__ void tile_coords(const DevPlan &p, int tile, int &pm, int &pn) {
-  if (p.raster <= 0) {
-    pm = tile / p.tiles_n;
+  if (p.tiles_m == 1) {
+    pm = 0;
+    pn = tile;
+  } else if (p.raster <= 0) {
+    pm = p.by_tiles_n.div(tile);
     pn = tile - pm * p.tiles_n;
   } else {
-    int width = p.raster * p.tiles_n;
-    int group = tile / width;
-    int first_m = group * p.raster;
-    int gsize = min(p.raster, p.tiles_m - first_m);
-    int r = tile - group * width;
-    pm = first_m + r % gsize;
-    pn = r / gsize;
+    const int width = p.raster * p.tiles_n;
+    const int group = p.by_width.div(tile);
+    const int first_m = group * p.raster;
+    const int r = tile - group * width;
+    const bool tail = first_m + p.raster > p.tiles_m;
+    const int gsize = tail ? p.raster_tail : p.raster;
+    pn = tail ? p.by_tail.div(r) : p.by_raster.div(r);
+    pm = first_m + r - pn * gsize;
   }
 }
 
@@ -109,8 +148,8 @@ __device__ __forceinline__ void signal_partial_ready(int *flag) {
 // CTA that owns K-iteration `iter` of the Stream-K wave (inverse of sk_range)
 __device__ __forceinline__ int sk_pid_of_iter(const DevPlan &p, int iter) {
   const int boundary = p.sk_extra * (p.sk_full + 1);
-  if (iter < boundary) return iter / (p.sk_full + 1);
-  return p.sk_extra + (iter - boundary) / p.sk_full;
+  if (iter < boundary) return p.by_full1.div(iter);
+  return p.sk_extra + p.by_full.div(iter - boundary);
 }
 
 // Owner: the first wave polls all `npeers` follower flags at once, one flag per lane; the barrier

@@ -17,12 +17,14 @@ template <class P>
 __device__ __forceinline__ void run_persistent(const typename P::Args &a, const DevPlan &plan,
                                                const Workspace &ws, char *smem) {
   __shared__ int s_word;
+  SK_TRACE(0);
   const int pid = logical_pid(plan);
   const int ipt = plan.ipt;
   typename P::Acc acc;
 
   int start, last;
   sk_range(plan, pid, start, last);
+  SK_TRACE(10);
   int dp_tile = plan.sk_tiles + pid;
 
   // One loop body serves both phases so that the MAC loop and the epilogue exist once in the
@@ -31,7 +33,7 @@ __device__ __forceinline__ void run_persistent(const typename P::Args &a, const 
   for (;;) {
     int tile, k0, n;
     if (start < last) {
-      tile = start / ipt;
+      tile = plan.by_ipt.div(start);
       k0 = start - tile * ipt;
       n = min(ipt - k0, last - start);
       start += n;
@@ -45,6 +47,7 @@ __device__ __forceinline__ void run_persistent(const typename P::Args &a, const 
     }
     int pm, pn;
     tile_coords(plan, tile, pm, pn);
+    SK_TRACE(11);
     P::mac(a, acc, pm, pn, k0, n, smem);
 
     // a segment that is the whole tile is simply stored (streamk_fp32.py:128-129)
@@ -88,7 +91,9 @@ __device__ __forceinline__ void run_persistent(const typename P::Args &a, const 
         store = true;
       }
     }
+    SK_TRACE(8);
     if (store) P::store_c(a, acc, pm, pn, smem);
+    SK_TRACE(9);
   }
 }
 

@@ -35,23 +35,56 @@ struct SkinnyArgs {
 // halfs, 16 bytes at a time.  A 16-byte piece that would run past the end of its row (K / group
 // not a multiple of 8) is fetched half by half instead: on the tile's last row a vector load would
 // cross the end of the buffer, and the hardware then zeroes the straddling dword.
+// begin() issues the first piece of every thread and returns; finish() stores it and copies the
+// rest, so a caller can put its other loads in flight between the two.
 template <int BN, int SC_ROW, int NT>
-__device__ __forceinline__ void stage_scales(half_t *ldsS, const half_t *scales_tile, int rows, int groups, int g0,
-                                             int chunks) {
-  const BufferRsrc rsrc_s = make_rsrc(scales_tile, (uint32_t)(rows * groups * 2));
-  for (int idx = threadIdx.x; idx < BN * chunks; idx += NT) {
+struct ScaleStager {
+  BufferRsrc rsrc;
+  half_t *lds;
+  int groups, g0, chunks;
+  uint4v first;
+
+  __device__ __forceinline__ bool whole_piece(int idx) const { return g0 + (idx / BN) * 8 + 8 <= groups; }
+  __device__ __forceinline__ uint4v load_piece(int idx) const {
+    const int r = idx % BN, g = g0 + (idx / BN) * 8;
+    return buffer_load_16(rsrc, (uint32_t)(r * groups + g) * 2, 0);
+  }
+  __device__ __forceinline__ void store_piece(int idx, uint4v v) const {
     const int r = idx % BN, c = idx / BN, g = g0 + c * 8;
-    half_t *dst = ldsS + r * SC_ROW + c * 8;
-    if (g + 8 <= groups) {
-      *reinterpret_cast<uint4v *>(dst) = buffer_load_16(rsrc_s, (uint32_t)(r * groups + g) * 2, 0);
+    half_t *dst = lds + r * SC_ROW + c * 8;
+    if (whole_piece(idx)) {
+      *reinterpret_cast<uint4v *>(dst) = v;
     } else {
       for (int e = 0; e < 8; ++e) {
-        const uint16_t v =
-            g + e < groups ? __builtin_amdgcn_raw_buffer_load_b16(rsrc_s, (uint32_t)(r * groups + g + e) * 2, 0, 0) : 0;
-        dst[e] = __builtin_bit_cast(half_t, v);
+        const uint16_t h =
+            g + e < groups ? __builtin_amdgcn_raw_buffer_load_b16(rsrc, (uint32_t)(r * groups + g + e) * 2, 0, 0) : 0;
+        dst[e] = __builtin_bit_cast(half_t, h);
       }
     }
   }
+  __device__ __forceinline__ void begin(half_t *ldsS, const half_t *scales_tile, int rows, int groups_, int g0_,
+                                        int chunks_) {
+    rsrc = make_rsrc(scales_tile, (uint32_t)(rows * groups_ * 2));
+    lds = ldsS;
+    groups = groups_;
+    g0 = g0_;
+    chunks = chunks_;
+    const int idx = threadIdx.x;
+    // a piece that is out of range or not whole is loaded from an out-of-range offset (zeros)
+    first = buffer_load_16(rsrc, idx < BN * chunks && whole_piece(idx) ? (uint32_t)((idx % BN) * groups + g0 + (idx / BN) * 8) * 2
+                                                                       : OOB_OFFSET, 0);
+  }
+  __device__ __forceinline__ void finish() const {
+    if ((int)threadIdx.x < BN * chunks) store_piece(threadIdx.x, first);
+    for (int idx = threadIdx.x + NT; idx < BN * chunks; idx += NT) store_piece(idx, whole_piece(idx) ? load_piece(idx) : first);
+  }
+};
+template <int BN, int SC_ROW, int NT>
+__device__ __forceinline__ void stage_scales(half_t *ldsS, const half_t *scales_tile, int rows, int groups, int g0,
+                                             int chunks) {
+  ScaleStager<BN, SC_ROW, NT> st;
+  st.begin(ldsS, scales_tile, rows, groups, g0, chunks);
+  st.finish();
 }
 
 // ROW1_: M == 1 only.  A single row of A is staged and every lane reads it (an LDS broadcast);
