@@ -81,22 +81,21 @@ struct KernelInfo {
   X(129, 1, 4, 1, 1, 1, 2, 1)    \
   X(130, 1, 2, 1, 2, 1, 4, 1)
 
-// M == 1 Q4 matrix-vector kernels (variant 2; variant 3: eight iterations of loads in flight):
-//   X(id, NB, WN, RK, DEPTH)
-#define SK_GEMV_Q4_KERNELS(X) \
-  X(140, 1, 4, 1, 4)          \
-  X(141, 1, 2, 2, 4)          \
-  X(142, 1, 1, 4, 4)          \
-  X(143, 2, 4, 1, 2)          \
-  X(144, 1, 4, 2, 4)          \
-  X(145, 1, 2, 1, 4)          \
-  X(146, 1, 1, 2, 4)          \
-  X(147, 1, 1, 1, 4)          \
-  X(148, 1, 2, 4, 4)          \
-  X(149, 1, 1, 8, 4)          \
-  X(150, 1, 4, 1, 8)          \
-  X(151, 1, 2, 2, 8)          \
-  X(152, 1, 1, 4, 8)
+// M == 1 Q4 matrix-vector kernels (variant 2):  X(id, NB, WN, RK, DEPTH, KMAX)
+// KMAX is the largest K range one segment may span (A is kept in LDS for the whole segment).
+#define SK_GEMV_Q4_KERNELS(X)  \
+  X(140, 1, 4, 1, 4, 16384)    \
+  X(141, 1, 2, 2, 4, 16384)    \
+  X(142, 1, 1, 4, 4, 16384)    \
+  X(143, 2, 4, 1, 2, 16384)    \
+  X(144, 1, 4, 2, 4, 16384)    \
+  X(145, 1, 2, 1, 4, 16384)    \
+  X(146, 1, 1, 2, 4, 16384)    \
+  X(147, 1, 1, 1, 4, 16384)    \
+  X(148, 1, 2, 4, 4, 16384)    \
+  X(149, 1, 1, 8, 4, 16384)    \
+  X(150, 1, 1, 4, 4, 32768)    \
+  X(151, 1, 2, 4, 4, 32768)
 
 const KernelInfo *kernel_table(int *count);
 const KernelInfo *kernel_by_id(int id);

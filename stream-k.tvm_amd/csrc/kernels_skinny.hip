@@ -28,12 +28,12 @@ int skinny_kernel_infos(KernelInfo *out, int max) {
   }
   SK_SKINNY_KERNELS(X)
 #undef X
-#define X(id, NB, WN, RK, DEPTH)                                                                          \
+#define X(id, NB, WN, RK, DEPTH, KMAX)                                                                        \
   if (n < max) {                                                                                         \
-    typedef TileGemvQ4<NB, WN, RK, DEPTH> P;                                                             \
-    out[n++] = KernelInfo{id, FAMILY_SKINNY, 2, 0, (DEPTH) == 8 ? 3 : 2, P::BM, P::BN, P::BKC, P::NT, P::LDS_BYTES,         \
+    typedef TileGemvQ4<NB, WN, RK, DEPTH, KMAX> P;                                                        \
+    out[n++] = KernelInfo{id, FAMILY_SKINNY, 2, 0, 2, P::BM, P::BN, P::BKC, P::NT, P::LDS_BYTES,         \
                           P::CTAS_PER_CU, P::TILE_ELEMS, P::MAX_ITERS, P::MAX_M, 128,                    \
-                          "gemv_q4_nb" #NB "_wn" #WN "_rk" #RK};                                         \
+                          "gemv_q4_nb" #NB "_wn" #WN "_rk" #RK "_k" #KMAX};                                     \
   }
   SK_GEMV_Q4_KERNELS(X)
 #undef X
@@ -50,9 +50,9 @@ int launch_skinny(int id, const SkinnyArgs &a, const DevPlan &p, const Workspace
   }
     SK_SKINNY_KERNELS(X)
 #undef X
-#define X(id_, NB, WN, RK, DEPTH)                                                          \
+#define X(id_, NB, WN, RK, DEPTH, KMAX)                                                        \
   case id_: {                                                                              \
-    typedef TileGemvQ4<NB, WN, RK, DEPTH> P;                                               \
+    typedef TileGemvQ4<NB, WN, RK, DEPTH, KMAX> P;                                          \
     hipLaunchKernelGGL(sk_skinny_kernel<P>, dim3(p.grid), dim3(P::NT), 0, s, a, p, ws);    \
     return (int)hipGetLastError();                                                         \
   }
@@ -74,9 +74,9 @@ int occupancy_skinny(int id) {
   }
     SK_SKINNY_KERNELS(X)
 #undef X
-#define X(id_, NB, WN, RK, DEPTH)                                                                        \
+#define X(id_, NB, WN, RK, DEPTH, KMAX)                                                                      \
   case id_: {                                                                                            \
-    typedef TileGemvQ4<NB, WN, RK, DEPTH> P;                                                             \
+    typedef TileGemvQ4<NB, WN, RK, DEPTH, KMAX> P;                                                        \
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_skinny_kernel<P>, P::NT, 0) != hipSuccess) \
       return -1;                                                                                         \
     return occ;                                                                                          \

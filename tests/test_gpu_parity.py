@@ -177,7 +177,7 @@ def test_q4_ragged_shapes_every_kernel(sk, oracle, variant):
     multiply fp16-rounded weights; both stay within 2e-3 of the fp32 host product of the
     dequantised weights."""
     rng = np.random.default_rng(50 + variant)
-    shapes = [(1, 1000, 1152, 8), (1, 520, 384, 15), (1, 72, 4096, 0), (1, 2048, 16384, 5)]
+    shapes = [(1, 1000, 1152, 8), (1, 520, 384, 15), (1, 72, 4096, 0), (1, 2048, 16384, 5), (1, 264, 28672, 8)]
     if variant == 1:
         shapes += [(5, 1000, 1152, 8), (16, 520, 384, 15), (33, 200, 640, 8), (64, 136, 2048, 3)]
     ran = 0
