@@ -22,7 +22,8 @@ struct KernelInfo {
   int dtype;    // sk_dtype
   int layout;   // sk_layout
   int variant;  // tile kernels -- 0: registers -> padded LDS rows; 1: direct global -> LDS loads,
-                // swizzled rows; 2: as 1 with four waves per CTA (one per SIMD, accumulators in AGPRs)
+                // swizzled rows; 2: as 1 with four waves per CTA (one per SIMD, accumulators in AGPRs);
+                // 3: as 1 with BK = 32 and four LDS stages (loads three iterations ahead)
                 // small-M kernels -- 0: up to 16*MB rows of A; 1: M == 1; 2: M == 1, Q4 matrix-vector
   int bm, bn, bk;  // CTA tile; bk is the K extent of one CTA iteration
   int threads;
@@ -52,6 +53,13 @@ struct KernelInfo {
   X(12, 128, 256, 2, 4)               \
   X(13, 256, 128, 4, 2)               \
   X(14, 256, 256, 2, 2)
+
+// direct-to-LDS loads, BK = 32, four stages (variant 3), NT layout:  X(id, BM, BN, WM, WN)
+#define SK_TILE_F16_NT_DMA32_KERNELS(X) \
+  X(15, 256, 256, 2, 4)                 \
+  X(16, 128, 128, 2, 2)                 \
+  X(17, 128, 256, 2, 4)                 \
+  X(18, 256, 128, 4, 2)
 
 // the same for the NN layout (B is [K,N]), fragments through transposing LDS reads:  X(id, BM, BN, WM, WN)
 #define SK_TILE_F16_NN_DMA_KERNELS(X) \

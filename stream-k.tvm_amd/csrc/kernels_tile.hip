@@ -13,6 +13,7 @@ __global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_tile_kernel(typenam
 #define SK_POLICY(id, BM, BN, BK, WM, WN) TileF16NT<BM, BN, BK, WM, WN>
 #define SK_POLICY_DMA(id, BM, BN, WM, WN) TileF16NTDma<BM, BN, WM, WN>
 #define SK_POLICY_NN(id, BM, BN, WM, WN) TileF16NTDma<BM, BN, WM, WN, true>
+#define SK_POLICY_DMA32(id, BM, BN, WM, WN) TileF16NTDma<BM, BN, WM, WN, false, 32>
 
 int tile_kernel_infos(KernelInfo *out, int max) {
   int n = 0;
@@ -39,6 +40,14 @@ int tile_kernel_infos(KernelInfo *out, int max) {
                           P::TILE_ELEMS, 0, 0, 8, "tile_f16_nn_dma_" #BM "x" #BN "x64"};            \
   }
   SK_TILE_F16_NN_DMA_KERNELS(X)
+#undef X
+#define X(id, BM, BN, WM, WN)                                                                       \
+  if (n < max) {                                                                                    \
+    typedef SK_POLICY_DMA32(id, BM, BN, WM, WN) P;                                                  \
+    out[n++] = KernelInfo{id, FAMILY_TILE, 0, 0, 3, BM, BN, 32, P::NT, P::LDS_TOTAL, P::CTAS_PER_CU, \
+                          P::TILE_ELEMS, 0, 0, 8, "tile_f16_nt_dma_" #BM "x" #BN "x32"};            \
+  }
+  SK_TILE_F16_NT_DMA32_KERNELS(X)
 #undef X
   return n;
 }
@@ -68,6 +77,14 @@ int launch_tile_f16(int id, const GemmArgs &a, const DevPlan &p, const Workspace
     return (int)hipGetLastError();                                                       \
   }
     SK_TILE_F16_NN_DMA_KERNELS(X)
+#undef X
+#define X(id_, BM, BN, WM, WN)                                                           \
+  case id_: {                                                                            \
+    typedef SK_POLICY_DMA32(id_, BM, BN, WM, WN) P;                                      \
+    hipLaunchKernelGGL(sk_tile_kernel<P>, dim3(p.grid), dim3(P::NT), 0, s, a, p, ws);    \
+    return (int)hipGetLastError();                                                       \
+  }
+    SK_TILE_F16_NT_DMA32_KERNELS(X)
 #undef X
   }
   return (int)hipErrorInvalidValue;
@@ -102,6 +119,15 @@ int occupancy_tile(int id) {
     return occ;                                                                                     \
   }
     SK_TILE_F16_NN_DMA_KERNELS(X)
+#undef X
+#define X(id_, BM, BN, WM, WN)                                                                      \
+  case id_: {                                                                                       \
+    typedef SK_POLICY_DMA32(id_, BM, BN, WM, WN) P;                                                 \
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_tile_kernel<P>, P::NT, 0) != hipSuccess) \
+      return -1;                                                                                    \
+    return occ;                                                                                     \
+  }
+    SK_TILE_F16_NT_DMA32_KERNELS(X)
 #undef X
   }
   return -1;

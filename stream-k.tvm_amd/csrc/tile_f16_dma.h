@@ -40,31 +40,42 @@ struct LdsArray {
 // a 4 (K) x 16 (N) patch receives, per lane, 4 consecutive K of one column -- half an MFMA operand.
 // 16-byte chunk c of K-row k is stored at position c ^ (4 * (k & 3)), which keeps the 32 lanes
 // served in one cycle (2 groups x 4 rows x 32 bytes) on distinct banks.
-template <int BM_, int BN_, int WM_, int WN_, bool B_KN_ = false>
+//
+// BK_ = 32: four stages of half the depth (LDS rows of 64 bytes, 4 chunks, chunk c of row r at
+// position c ^ ((r >> 2) & 3); a wave-wide load fills 16 rows).  The tiles of iteration it+4 are
+// requested when iteration it has been read, three iterations (about 1.5 iterations of the
+// two-stage pipeline) before they are needed: a load that misses the L2 takes longer than one
+// iteration of MFMAs, which the two-stage pipeline exposes as a stall at every barrier.
+template <int BM_, int BN_, int WM_, int WN_, bool B_KN_ = false, int BK_ = 64>
 struct TileF16NTDma {
   static constexpr bool B_KN = B_KN_;
-  static constexpr int B_ROW_BYTES = B_KN_ ? BN_ * 2 : 128;    // bytes of one LDS row of the B stage
+  static constexpr int ROW_BYTES = BK_ * 2;                    // bytes of one LDS row of A (and of B, NT)
+  static constexpr int ROWS_PER_DMA = 1024 / ROW_BYTES;        // rows one wave-wide load fills
+  static constexpr int NSTAGE = 128 / BK_, KSTEPS = BK_ / 16;
+  static_assert(BK_ == 64 || (BK_ == 32 && !B_KN_), "BK is 64, or 32 for the NT layout");
+  static constexpr int B_ROW_BYTES = B_KN_ ? BN_ * 2 : ROW_BYTES;  // bytes of one LDS row of the B stage
   static constexpr int B_ROWS_PER_DMA = 1024 / B_ROW_BYTES;    // rows one wave-wide load fills
   static_assert(!B_KN_ || (BN_ >= 128 && BN_ <= 512), "NN layout: 16..64 chunks per LDS row");
   typedef GemmArgs Args;
-  static constexpr int BM = BM_, BN = BN_, BK = 64, WM = WM_, WN = WN_;
+  static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
   static constexpr int NW = WM * WN, NT = NW * 64;
   static constexpr int TM = BM / (WM * 32), TN = BN / (WN * 32);
   static constexpr int WTM = TM * 32, WTN = TN * 32;
-  static constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE_BYTES = A_BYTES + B_BYTES;
-  static constexpr int A_DMA = BM / 8 / NW, B_DMA = BN / 8 / NW, DMA_PER_WAVE = A_DMA + B_DMA;
+  static constexpr int A_BYTES = BM * ROW_BYTES, B_BYTES = BN * ROW_BYTES, STAGE_BYTES = A_BYTES + B_BYTES;
+  static constexpr int A_DMA = A_BYTES / 1024 / NW, B_DMA = B_BYTES / 1024 / NW, DMA_PER_WAVE = A_DMA + B_DMA;
   static constexpr int LDC = WTN + 8;
-  // epilogue patches: waves [0, NW/2) use stage 0, the others stage 1; split the wave tile's rows
-  // into passes until the patches fit
+  // epilogue patches: the waves share out the stages evenly; split the wave tile's rows into
+  // passes until the patches fit
+  static constexpr int WAVES_PER_STAGE = NW / NSTAGE;
   static constexpr int patch_passes() {
     int p = 1;
-    while ((NW / 2) * (WTM / p) * LDC * 2 > STAGE_BYTES) p *= 2;
+    while (WAVES_PER_STAGE * (WTM / p) * LDC * 2 > STAGE_BYTES) p *= 2;
     return p;
   }
   static constexpr int PASSES = patch_passes();
   static constexpr int PATCH_ROWS = WTM / PASSES;
   static constexpr int LDS_BYTES = 16;  // the kernel's generic buffer is unused
-  static constexpr int LDS_TOTAL = 2 * STAGE_BYTES;
+  static constexpr int LDS_TOTAL = NSTAGE * STAGE_BYTES;
   static constexpr int TILE_ELEMS = BM * BN;
   static constexpr int NV4 = TM * TN * 4;
   static constexpr int CTAS_PER_CU_REGS = (NT >= 512 || TM * TN > 4) ? 1 : 2;
@@ -72,15 +83,18 @@ struct TileF16NTDma {
   static constexpr int CTAS_PER_CU = CTAS_PER_CU_REGS < CTAS_PER_CU_LDS ? CTAS_PER_CU_REGS : CTAS_PER_CU_LDS;
   static constexpr int WAVES_PER_EU = CTAS_PER_CU * (NT / 64) / 4 > 0 ? CTAS_PER_CU * (NT / 64) / 4 : 1;
   static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "tile shape");
-  static_assert((BM / 8) % NW == 0 && (BN / 8) % NW == 0, "DMA groups must divide over the waves");
-  static_assert(NW % 2 == 0, "a wave must keep to row groups of one parity");
+  static_assert((A_BYTES / 1024) % NW == 0 && (B_BYTES / 1024) % NW == 0, "DMA groups must divide over the waves");
+  static_assert(NW % NSTAGE == 0, "a wave must keep to row groups of one parity; patches per stage");
   static_assert(PATCH_ROWS % 32 == 0, "epilogue pass must hold whole 32-row blocks");
 
   typedef TileF16NT<BM_, BN_, 64, WM_, WN_> Base;  // shares the accumulator type and the partials
   typedef typename Base::Acc Acc;
 
   static __device__ __forceinline__ char *stage(int s) {
-    return s == 0 ? LdsArray<STAGE_BYTES, 0>::get() : LdsArray<STAGE_BYTES, 1>::get();
+    if (NSTAGE == 2) return s == 0 ? LdsArray<STAGE_BYTES, 0>::get() : LdsArray<STAGE_BYTES, 1>::get();
+    return s == 0 ? LdsArray<STAGE_BYTES, 0>::get()
+                  : (s == 1 ? LdsArray<STAGE_BYTES, 1>::get()
+                            : (s == 2 ? LdsArray<STAGE_BYTES, 2>::get() : LdsArray<STAGE_BYTES, 3>::get()));
   }
 
   template <int N>
@@ -108,9 +122,11 @@ struct TileF16NTDma {
 
     const int rows_a = min(BM, a.M - pm * BM), rows_b = min(BN, a.N - pn * BN);
     const uint4v rsrc_a = make_rsrc_words(a.A + (int64_t)pm * BM * a.lda, (uint32_t)(rows_a * a.lda * 2));
-    const int my_chunk = (lane & 7) ^ (((wave & 1) << 2) | (lane >> 4));  // global chunk this lane fetches
-    const uint32_t voff_a = (uint32_t)((lane >> 3) * a.lda + my_chunk * 8) * 2;
-    const uint32_t grp_a = (uint32_t)(8 * a.lda * 2);
+    // global chunk this lane fetches: its LDS position XOR the swizzle of its row
+    const int my_chunk = BK == 64 ? (lane & 7) ^ (((wave & 1) << 2) | (lane >> 4)) : (lane & 3) ^ (lane >> 4);
+    const int my_row = BK == 64 ? lane >> 3 : lane >> 2;  // row within the load's group
+    const uint32_t voff_a = (uint32_t)(my_row * a.lda + my_chunk * 8) * 2;
+    const uint32_t grp_a = (uint32_t)(ROWS_PER_DMA * a.lda * 2);
     const int tail_kt = (a.K % BK != 0) ? (a.K / BK) : -1;
     // B operand.  NT: rows are N, same scheme as A.  NN: rows are K; the descriptor starts at the
     // tile's first column and ends with the last valid element of row K-1, so K-rows past the
@@ -119,8 +135,8 @@ struct TileF16NTDma {
     uint32_t voff_b, grp_b, kstep_b;
     if (!B_KN) {
       rsrc_b = make_rsrc_words(a.B + (int64_t)pn * BN * a.ldb, (uint32_t)(rows_b * a.ldb * 2));
-      voff_b = (uint32_t)((lane >> 3) * a.ldb + my_chunk * 8) * 2;
-      grp_b = (uint32_t)(8 * a.ldb * 2);
+      voff_b = (uint32_t)(my_row * a.ldb + my_chunk * 8) * 2;
+      grp_b = (uint32_t)(ROWS_PER_DMA * a.ldb * 2);
       kstep_b = BK * 2;
     } else {
       rsrc_b = make_rsrc_words(a.B + (int64_t)pn * BN, (uint32_t)(((int64_t)(a.K - 1) * a.ldb + rows_b) * 2));
@@ -134,7 +150,9 @@ struct TileF16NTDma {
 
     // one wave-wide load of stage `st` for K-iteration kt: x < A_DMA loads rows of A, the rest B
     auto dma_one = [&](char *st, int kt, int x) {
-      const bool tail_oob = (kt == tail_kt) && (kt * BK + my_chunk * 8 >= a.K);
+      // the four-stage pipeline also issues the loads of iterations past the segment (the wait
+      // counts stay uniform): they fetch nothing and fill a stage nobody reads with zeros
+      const bool tail_oob = ((kt == tail_kt) && (kt * BK + my_chunk * 8 >= a.K)) || (NSTAGE == 4 && kt >= k0 + n);
       if (x < A_DMA) {
         const int g = wave + x * NW;
         dma_load_16(rsrc_a, lds_address(st) + g * 1024, tail_oob ? OOB_OFFSET : voff_a,
@@ -152,12 +170,13 @@ struct TileF16NTDma {
 
     // fragment addressing: lane (r = lane%32, g = lane/32) reads row r of a 32-row block, logical
     // chunk 2*kk + g, stored at chunk position (2*kk + g) ^ ((r >> 1) & 7)
-    int rd_a[4], rd_b[4];
+    // (BK = 32: swizzle (r >> 2) & 3)
+    int rd_a[KSTEPS], rd_b[KSTEPS];
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      const int pos = ((2 * kk + (lane >> 5)) ^ ((lane >> 1) & 7)) * 16;
-      rd_a[kk] = (wm * WTM + (lane & 31)) * 128 + pos;
-      rd_b[kk] = A_BYTES + (wn * WTN + (lane & 31)) * 128 + pos;
+    for (int kk = 0; kk < KSTEPS; ++kk) {
+      const int pos = ((2 * kk + (lane >> 5)) ^ (BK == 64 ? (lane >> 1) & 7 : (lane >> 2) & 3)) * 16;
+      rd_a[kk] = (wm * WTM + (lane & 31)) * ROW_BYTES + pos;
+      rd_b[kk] = A_BYTES + (wn * WTN + (lane & 31)) * ROW_BYTES + pos;
     }
     // NN: per 32-column block j, the byte address of this lane's 8-byte piece in K-row
     // 8*(lane/32) + (lane%16)/4 of the stage; K-steps and the second half add row multiples
@@ -174,11 +193,11 @@ struct TileF16NTDma {
     half8v fa[2][TM], fb[2][TN];
     auto read_frags = [&](const char *st, int buf, int kk) {
 #pragma unroll
-      for (int i = 0; i < TM; ++i) fa[buf][i] = *reinterpret_cast<const half8v *>(st + rd_a[kk] + i * 4096);
+      for (int i = 0; i < TM; ++i) fa[buf][i] = *reinterpret_cast<const half8v *>(st + rd_a[kk] + i * 32 * ROW_BYTES);
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
         if (!B_KN) {
-          fb[buf][j] = *reinterpret_cast<const half8v *>(st + rd_b[kk] + j * 4096);
+          fb[buf][j] = *reinterpret_cast<const half8v *>(st + rd_b[kk] + j * 32 * ROW_BYTES);
         } else {
           typedef short short4v __attribute__((ext_vector_type(4)));
           typedef __attribute__((address_space(3))) short4v *lds_s4;
@@ -196,48 +215,88 @@ struct TileF16NTDma {
         for (int j = 0; j < TN; ++j)
           acc.c[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[buf][j], fa[buf][i], acc.c[i][j], 0, 0, 0);
     };
-    // one K-iteration on stage `cur`; `more1`/`more2`: iterations it+1 / it+2 exist
-    auto iteration = [&](char *cur, char *nxt, int it) {
-#pragma unroll
-      for (int kk = 0; kk < 3; ++kk) {
-        read_frags(cur, (kk + 1) & 1, kk + 1);
-        mfma_step(kk & 1);
+    if constexpr (NSTAGE == 4) {
+      // one K-iteration (two K-steps) on stage `cur`: the barrier in the middle retires the reads
+      // of `cur` (it is refilled for iteration it+4 right away) and publishes stage `nxt`, whose
+      // loads were issued three iterations ago -- two younger groups may still be in flight
+      auto iteration4 = [&](char *cur, char *nxt, int it) {
+        read_frags(cur, 1, 1);
+        mfma_step(0);
 #pragma unroll
         for (int g = 0; g < TM + TN; ++g) {
           __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        wait_dma_then_barrier<2 * DMA_PER_WAVE>();
+        issue_dma(cur, k0 + it + 4);
+        read_frags(nxt, 0, 0);
+        mfma_step(1);
+      };
+      char *s0 = stage(0), *s1 = stage(1), *s2 = stage(2), *s3 = stage(3);
+      issue_dma(s0, k0);
+      issue_dma(s1, k0 + 1);
+      issue_dma(s2, k0 + 2);
+      wait_dma_then_barrier<2 * DMA_PER_WAVE>();
+      issue_dma(s3, k0 + 3);
+      read_frags(s0, 0, 0);
+      int it = 0;
+      for (; it + 3 < n; it += 4) {
+        iteration4(s0, s1, it);
+        iteration4(s1, s2, it + 1);
+        iteration4(s2, s3, it + 2);
+        iteration4(s3, s0, it + 3);
       }
-      // every read of `cur` has been issued; they complete before the barrier below because the
-      // MFMAs of step 3 (which need them) follow it -- make that explicit for the hardware:
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-      wait_dma_then_barrier<0>();
-      if (it + 2 < n) issue_dma(cur, k0 + it + 2);
-      if (it + 1 < n) read_frags(nxt, 0, 0);
-      mfma_step(1);
-    };
+      if (it < n) iteration4(s0, s1, it);
+      if (it + 1 < n) iteration4(s1, s2, it + 1);
+      if (it + 2 < n) iteration4(s2, s3, it + 2);
+      // the (empty) loads of the iterations past the segment still write LDS: drain them before
+      // the stages are handed to the epilogue / the next tile
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    } else {
+      // one K-iteration on stage `cur`; `more1`/`more2`: iterations it+1 / it+2 exist
+      auto iteration = [&](char *cur, char *nxt, int it) {
+#pragma unroll
+        for (int kk = 0; kk < 3; ++kk) {
+          read_frags(cur, (kk + 1) & 1, kk + 1);
+          mfma_step(kk & 1);
+#pragma unroll
+          for (int g = 0; g < TM + TN; ++g) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          }
+        }
+        // every read of `cur` has been issued; they complete before the barrier below because the
+        // MFMAs of step 3 (which need them) follow it -- make that explicit for the hardware:
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        wait_dma_then_barrier<0>();
+        if (it + 2 < n) issue_dma(cur, k0 + it + 2);
+        if (it + 1 < n) read_frags(nxt, 0, 0);
+        mfma_step(1);
+      };
 
-    char *s0 = stage(0), *s1 = stage(1);
-    issue_dma(s0, k0);
-    wait_dma_then_barrier<0>();
-    if (n > 1) issue_dma(s1, k0 + 1);
-    read_frags(s0, 0, 0);
-    int it = 0;
-    for (; it + 1 < n; it += 2) {
-      iteration(s0, s1, it);
-      iteration(s1, s0, it + 1);
+      char *s0 = stage(0), *s1 = stage(1);
+      issue_dma(s0, k0);
+      wait_dma_then_barrier<0>();
+      if (n > 1) issue_dma(s1, k0 + 1);
+      read_frags(s0, 0, 0);
+      int it = 0;
+      for (; it + 1 < n; it += 2) {
+        iteration(s0, s1, it);
+        iteration(s1, s0, it + 1);
+      }
+      if (it < n) iteration(s0, s1, it);
+      // all LDS reads are complete and every wave has passed the last barrier only after finishing
+      // its reads of the other stage; one more barrier frees both stages for the epilogue / next tile
     }
-    if (it < n) iteration(s0, s1, it);
-    // all LDS reads are complete and every wave has passed the last barrier only after finishing
-    // its reads of the other stage; one more barrier frees both stages for the epilogue / next tile
     __syncthreads();
   }
 
   static __device__ __forceinline__ void store_c(const Args &a, const Acc &acc, int pm, int pn, char *) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
-    half_t *patch = reinterpret_cast<half_t *>(wave < NW / 2 ? stage(0) : stage(1)) +
-                    (wave % (NW / 2)) * (PATCH_ROWS * LDC);
+    half_t *patch = reinterpret_cast<half_t *>(stage(wave / WAVES_PER_STAGE)) +
+                    (wave % WAVES_PER_STAGE) * (PATCH_ROWS * LDC);
     const bool vec_ok = (a.ldc % 8 == 0) && ((reinterpret_cast<uintptr_t>(a.C) & 15) == 0);
     constexpr int CPRC = WTN / 8;
     constexpr int BLK = PATCH_ROWS / 32;  // 32-row blocks per pass

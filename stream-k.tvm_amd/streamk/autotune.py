@@ -66,9 +66,10 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
                 out.append(dict(bm=bm, bn=bn, bk=bk, schedule="sk2", grid=grid, fixup=fixup))
     if dtype == "float16" and M > 16:
         for (bm, bn, bk) in _TILES_F16:
-            variants = (2, 1) if (bm, bn) != (64, 64) else (0,)
-            for variant, raster in itertools.product(variants, (0, 8)):
-                base = dict(bm=bm, bn=bn, bk=bk, variant=variant, raster=raster)
+            # (variant, bk): direct-to-LDS two-stage, register-staged, direct-to-LDS four-stage
+            variants = ((2, bk), (1, bk), (4, 32)) if (bm, bn) != (64, 64) else ((0, bk),)
+            for (variant, vbk), raster in itertools.product(variants, (0, 8)):
+                base = dict(bm=bm, bn=bn, bk=vbk, variant=variant, raster=raster)
                 out.append(dict(base, schedule="dp"))
                 grids = (None,) if bm * bn >= 256 * 256 or (bm, bn) == (64, 64) else (None, cus)
                 for sched, fixup, grid in itertools.product(("sk2", "sk1", "basic"), ("reduce", "atomic"), grids):

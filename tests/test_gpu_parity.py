@@ -42,7 +42,8 @@ def _rel(oracle, C, ref):
     return oracle.max_abs_rel(C.float().cpu().numpy(), ref)
 
 
-# variant 1: registers -> padded LDS rows; 2: direct-to-LDS, 8 (4) waves; 3: direct-to-LDS 256x256 on 4 waves
+# variant 1: registers -> padded LDS rows; 2: direct-to-LDS, 8 (4) waves; 3: direct-to-LDS 256x256 on 4 waves;
+# 4: direct-to-LDS with BK = 32 and four stages
 TILE_CONFIGS = [
     dict(bm=128, bn=128, bk=64, variant=1), dict(bm=256, bn=256, bk=64, variant=1),
     dict(bm=128, bn=256, bk=64, variant=1), dict(bm=256, bn=128, bk=64, variant=1),
@@ -50,6 +51,8 @@ TILE_CONFIGS = [
     dict(bm=128, bn=128, bk=64, variant=2), dict(bm=256, bn=256, bk=64, variant=2),
     dict(bm=128, bn=256, bk=64, variant=2), dict(bm=256, bn=128, bk=64, variant=2),
     dict(bm=256, bn=256, bk=64, variant=3),
+    dict(bm=128, bn=128, bk=32, variant=4), dict(bm=256, bn=256, bk=32, variant=4),
+    dict(bm=128, bn=256, bk=32, variant=4), dict(bm=256, bn=128, bk=32, variant=4),
 ]
 SKINNY_CONFIGS = [
     dict(bm=16, bn=64, bk=128), dict(bm=32, bn=64, bk=128), dict(bm=64, bn=64, bk=128),
