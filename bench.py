@@ -209,7 +209,8 @@ def main():
             c = torch.empty(m, N, dtype=torch.float16, device="cuda")
             nbytes = 2 * m * K + N * K // 2 + 2 * N * (K // 128) + 2 * m * N
             row = {"M": m, "bytes": nbytes}
-            for name, cfg in {"streamk_reduce": dict(schedule="sk2", fixup="reduce", grid=256),
+            for name, cfg in {"tuned": dict(),
+                              "streamk_reduce": dict(schedule="sk2", fixup="reduce", grid=256),
                               "streamk_atomic": dict(schedule="sk2", fixup="atomic", grid=256),
                               "dp": dict(schedule="dp")}.items():
                 p = streamk.make_plan(m, N, K, "q4", "nt", **cfg)

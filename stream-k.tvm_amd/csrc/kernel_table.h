@@ -52,14 +52,20 @@ struct KernelInfo {
   X(11, 128, 128, 2, 2)               \
   X(12, 128, 256, 2, 4)               \
   X(13, 256, 128, 4, 2)               \
-  X(14, 256, 256, 2, 2)
+  X(14, 256, 256, 2, 2)               \
+  X(24, 64, 64, 2, 2)                 \
+  X(25, 128, 64, 2, 2)                \
+  X(26, 64, 128, 2, 2)
 
 // direct-to-LDS loads, BK = 32, four stages (variant 3), NT layout:  X(id, BM, BN, WM, WN)
 #define SK_TILE_F16_NT_DMA32_KERNELS(X) \
   X(15, 256, 256, 2, 4)                 \
   X(16, 128, 128, 2, 2)                 \
   X(17, 128, 256, 2, 4)                 \
-  X(18, 256, 128, 4, 2)
+  X(18, 256, 128, 4, 2)                 \
+  X(27, 64, 64, 2, 2)                   \
+  X(28, 128, 64, 2, 2)                  \
+  X(29, 64, 128, 2, 2)
 
 // the same for the NN layout (B is [K,N]), fragments through transposing LDS reads:  X(id, BM, BN, WM, WN)
 #define SK_TILE_F16_NN_DMA_KERNELS(X) \

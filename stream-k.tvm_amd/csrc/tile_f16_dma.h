@@ -78,7 +78,7 @@ struct TileF16NTDma {
   static constexpr int LDS_TOTAL = NSTAGE * STAGE_BYTES;
   static constexpr int TILE_ELEMS = BM * BN;
   static constexpr int NV4 = TM * TN * 4;
-  static constexpr int CTAS_PER_CU_REGS = (NT >= 512 || TM * TN > 4) ? 1 : 2;
+  static constexpr int CTAS_PER_CU_REGS = (NT >= 512 || TM * TN > 4) ? 1 : (TM * TN <= 2 ? 4 : 2);
   static constexpr int CTAS_PER_CU_LDS = (160 * 1024) / (LDS_TOTAL + 64);
   static constexpr int CTAS_PER_CU = CTAS_PER_CU_REGS < CTAS_PER_CU_LDS ? CTAS_PER_CU_REGS : CTAS_PER_CU_LDS;
   static constexpr int WAVES_PER_EU = CTAS_PER_CU * (NT / 64) / 4 > 0 ? CTAS_PER_CU * (NT / 64) / 4 : 1;

@@ -22,7 +22,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 DEFAULT_CACHE = os.path.join(_HERE, "tuned", "gfx950.json")
 USER_CACHE_ENV = "STREAMK_TUNE_CACHE"
 
-_TILES_F16 = [(256, 256, 64), (128, 128, 64), (128, 256, 64), (256, 128, 64), (64, 64, 64)]
+_TILES_F16 = [(256, 256, 64), (128, 128, 64), (128, 256, 64), (256, 128, 64), (64, 64, 64), (128, 64, 64),
+              (64, 128, 64)]
 _SKINNY_F16 = [(16, 64, 128), (32, 64, 128), (64, 64, 128), (16, 16, 512), (16, 32, 256), (16, 16, 128)]
 _SKINNY_Q4 = [(16, 64, 256), (32, 64, 256), (64, 64, 256), (16, 16, 1024), (16, 32, 512), (16, 16, 256),
               (16, 32, 256), (16, 32, 1024), (16, 16, 2048), (16, 64, 512), (16, 16, 512)]
@@ -67,11 +68,13 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
     if dtype == "float16" and M > 16:
         for (bm, bn, bk) in _TILES_F16:
             # (variant, bk): direct-to-LDS two-stage, register-staged, direct-to-LDS four-stage
-            variants = ((2, bk), (1, bk), (4, 32)) if (bm, bn) != (64, 64) else ((0, bk),)
+            variants = ((2, bk), (1, bk), (4, 32)) if bm * bn > 64 * 128 else ((2, bk), (4, 32))
+            if (bm, bn) == (64, 64):
+                variants += ((1, bk),)
             for (variant, vbk), raster in itertools.product(variants, (0, 8)):
                 base = dict(bm=bm, bn=bn, bk=vbk, variant=variant, raster=raster)
                 out.append(dict(base, schedule="dp"))
-                grids = (None,) if bm * bn >= 256 * 256 or (bm, bn) == (64, 64) else (None, cus)
+                grids = (None,) if bm * bn >= 256 * 256 else (None, cus)
                 for sched, fixup, grid in itertools.product(("sk2", "sk1", "basic"), ("reduce", "atomic"), grids):
                     out.append(dict(base, schedule=sched, fixup=fixup, **({"grid": grid} if grid else {})))
     return out

@@ -2,6 +2,11 @@
 
     rocprofv3 --kernel-trace --stats -- python3 stream-k.tvm_amd/streamk/profile_case.py 8192x8192x8192
     python3 stream-k.tvm_amd/streamk/profile_case.py 1x8192x8192 --dtype q4 --config "dict(grid=256)"
+    python3 stream-k.tvm_amd/streamk/profile_case.py 8192x8192x8192 --data zeros --time --vendor
+
+--data chooses the operand values (the clock the part sustains depends on how many bits toggle);
+--time prints the average time of --reps launches; --vendor also times torch.matmul (hipBLASLt) on the
+same operands.
 """
 import argparse
 import os
@@ -17,6 +22,9 @@ def main():
     ap.add_argument("--layout", default="nt", choices=["nt", "nn"])
     ap.add_argument("--config", default="{}", help="python dict of plan options, e.g. \"dict(bm=256,bn=256,raster=8)\"")
     ap.add_argument("--reps", type=int, default=5)
+    ap.add_argument("--data", default="rand", choices=["rand", "zeros", "ones"])
+    ap.add_argument("--time", action="store_true")
+    ap.add_argument("--vendor", action="store_true")
     args = ap.parse_args()
     import torch
     import streamk
@@ -32,15 +40,27 @@ def main():
         run = lambda: streamk.streamk_q4(A, Wq, sc, plan=plan)  # noqa: E731
     else:
         dt = torch.float16 if args.dtype == "float16" else torch.float32
-        A = (torch.rand(M, K, generator=g) * 2 - 1).to(dt).cuda()
         bshape = (N, K) if args.layout == "nt" else (K, N)
-        B = (torch.rand(*bshape, generator=g) * 2 - 1).to(dt).cuda()
+        if args.data == "rand":
+            A = (torch.rand(M, K, generator=g) * 2 - 1).to(dt).cuda()
+            B = (torch.rand(*bshape, generator=g) * 2 - 1).to(dt).cuda()
+        else:
+            fill = torch.zeros if args.data == "zeros" else torch.ones
+            A, B = fill(M, K, dtype=dt, device="cuda"), fill(*bshape, dtype=dt, device="cuda")
+        C = torch.empty(M, N, dtype=dt, device="cuda")
         fn = streamk.streamk_fp16 if args.dtype == "float16" else streamk.streamk_fp32
-        run = lambda: fn(A, B, layout=args.layout, plan=plan)  # noqa: E731
+        run = lambda: fn(A, B, layout=args.layout, out=C, plan=plan)  # noqa: E731
     for _ in range(args.reps):
         run()
     torch.cuda.synchronize()
     streamk.workspace_status()
+    if args.time:
+        ms = streamk.bench_ms(run, 3, args.reps)
+        print(f"{args.data}: {ms * 1e3:.2f} us, {2.0 * M * N * K / ms / 1e9:.0f} TFLOP/s")
+        if args.vendor and args.dtype != "q4":
+            Bt = B.T if args.layout == "nt" else B
+            ms = streamk.bench_ms(lambda: torch.matmul(A, Bt, out=C), 3, args.reps)
+            print(f"{args.data}: torch.matmul {ms * 1e3:.2f} us, {2.0 * M * N * K / ms / 1e9:.0f} TFLOP/s")
     print(f"ran {args.reps} x {args.dtype} {args.layout} {M}x{N}x{K} kernel {plan.kernel_id} grid {plan.grid} "
           f"streamk_tiles {plan.streamk_tiles}")
 

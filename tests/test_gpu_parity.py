@@ -47,12 +47,14 @@ def _rel(oracle, C, ref):
 TILE_CONFIGS = [
     dict(bm=128, bn=128, bk=64, variant=1), dict(bm=256, bn=256, bk=64, variant=1),
     dict(bm=128, bn=256, bk=64, variant=1), dict(bm=256, bn=128, bk=64, variant=1),
-    dict(bm=64, bn=64, bk=64), dict(bm=256, bn=256, bk=32), dict(bm=128, bn=128, bk=32),
+    dict(bm=64, bn=64, bk=64, variant=1), dict(bm=256, bn=256, bk=32), dict(bm=128, bn=128, bk=32),
     dict(bm=128, bn=128, bk=64, variant=2), dict(bm=256, bn=256, bk=64, variant=2),
     dict(bm=128, bn=256, bk=64, variant=2), dict(bm=256, bn=128, bk=64, variant=2),
     dict(bm=256, bn=256, bk=64, variant=3),
     dict(bm=128, bn=128, bk=32, variant=4), dict(bm=256, bn=256, bk=32, variant=4),
     dict(bm=128, bn=256, bk=32, variant=4), dict(bm=256, bn=128, bk=32, variant=4),
+    dict(bm=64, bn=64, bk=64, variant=2), dict(bm=128, bn=64, bk=64, variant=2), dict(bm=64, bn=128, bk=64, variant=2),
+    dict(bm=64, bn=64, bk=32, variant=4), dict(bm=128, bn=64, bk=32, variant=4), dict(bm=64, bn=128, bk=32, variant=4),
 ]
 SKINNY_CONFIGS = [
     dict(bm=16, bn=64, bk=128), dict(bm=32, bn=64, bk=128), dict(bm=64, bn=64, bk=128),
