@@ -68,7 +68,8 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
   // heuristic: small M -> weight-streaming kernels; otherwise the largest tile that still gives
   // every CU something to do
   const KernelInfo *best = nullptr;
-  if ((M <= 64 && layout == SK_LAYOUT_NT) || dtype == SK_Q4) {
+  // (for 32 < M <= 64 the 64x64 LDS tile below is faster than streaming the weights past 64 rows)
+  if ((M <= 32 && layout == SK_LAYOUT_NT) || dtype == SK_Q4) {
     // M == 1 with Q4 weights: the matrix-vector kernel with four waves splitting K (data-parallel
     // over 16-row tiles), the fastest instance at LLM-sized N and K
     if (dtype == SK_Q4 && M == 1 && want_variant < 0)
@@ -90,18 +91,24 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
       if (t[i].dtype == SK_F32 && t[i].layout == layout) return &t[i];
     return nullptr;
   }
-  static const int pref[][3] = {{256, 256, 64}, {128, 128, 64}, {64, 64, 64}};
-  for (auto &p : pref) {
-    for (int i = 0; i < n; ++i) {
-      if (t[i].family != FAMILY_TILE || t[i].dtype != dtype || t[i].layout != layout) continue;
-      if (t[i].bm != p[0] || t[i].bn != p[1] || t[i].bk != p[2]) continue;
-      if (want_variant >= 0 ? t[i].variant != want_variant : (best != nullptr && variant_rank(t[i]) < variant_rank(*best))) continue;
-      int64_t tiles = cdiv(M, p[0]) * cdiv(N, p[1]);
-      int64_t iters = tiles * cdiv(K, p[2]);
-      // enough K-iterations per CU that a split tile still amortises its fix-up
-      if (tiles >= num_cus || iters >= (int64_t)num_cus * 16 || p[0] == 64) best = &t[i];
+  // 256x256 tiles when they fill the device; else 128x128, else 64x64.  The smaller tiles run one
+  // or two waves per SIMD, where the four-stage (BK = 32) pipeline hides the load latency better;
+  // it exists for the NT layout only.
+  const int64_t tiles256 = cdiv(M, 256) * cdiv(N, 256), tiles128 = cdiv(M, 128) * cdiv(N, 128);
+  int pref[3][4] = {{256, 256, 64, 1}, {128, 128, 32, 3}, {64, 64, 32, 3}};  // bm, bn, bk, variant
+  const int first = tiles256 * 4 >= (int64_t)num_cus * 3 ? 0 : (tiles128 * 2 >= num_cus ? 1 : 2);
+  const int order[3][3] = {{0, 1, 2}, {1, 2, 0}, {2, 1, 0}};  // smaller tiles first, then larger ones
+  for (int oi = 0; oi < 3 && !best; ++oi) {
+    const int pi = order[first][oi];
+    for (int pass = 0; pass < 2 && !best; ++pass) {  // pass 1: any variant / BK of the tile shape
+      for (int i = 0; i < n; ++i) {
+        if (t[i].family != FAMILY_TILE || t[i].dtype != dtype || t[i].layout != layout) continue;
+        if (t[i].bm != pref[pi][0] || t[i].bn != pref[pi][1]) continue;
+        if (want_variant >= 0 && t[i].variant != want_variant) continue;
+        if (pass == 0 && want_variant < 0 && (t[i].bk != pref[pi][2] || t[i].variant != pref[pi][3])) continue;
+        if (best == nullptr || variant_rank(t[i]) > variant_rank(*best)) best = &t[i];
+      }
     }
-    if (best) break;
   }
   return best;
 }
@@ -136,19 +143,25 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
   out->total_tiles = total;
 
   // every CTA of the Stream-K wave may wait for another one, so the grid is capped at what the
-  // device keeps resident.  A small problem gets a smaller grid: a split tile keeps at least 4
-  // K-iterations per CTA, but there are never fewer CTAs than tiles (as far as they fit).
+  // device keeps resident
   const int occ = k->ctas_per_cu;
   const int max_grid = num_cus * occ;
   int grid = cfg && cfg->grid > 0 ? cfg->grid : max_grid;
   if (grid > max_grid) return SK_ERR_CONFIG;
+  int sched = cfg ? cfg->schedule : SK_SCHED_AUTO;
   if (!(cfg && cfg->grid > 0)) {
     const int64_t iters = total64 * out->iters_per_tile;
-    const int64_t tiles_fit = total64 < max_grid ? total64 : max_grid;
-    int64_t want = iters / 4 > tiles_fit ? iters / 4 : tiles_fit;
-    if (want < grid) grid = (int)(want > 8 && want != total64 ? want / 8 * 8 : want);
+    if (total64 >= num_cus && total64 <= max_grid) {
+      grid = (int)total64;  // one tile per CTA, all resident: a single data-parallel wave
+    } else if (total64 < num_cus) {
+      // fewer tiles than CUs: one CTA per CU, but a split tile keeps at least 4 K-iterations per CTA
+      // and there are never fewer CTAs than tiles
+      int64_t want = iters / 4 < num_cus ? iters / 4 : num_cus;
+      if (want < total64) want = total64;
+      grid = (int)(want > 8 && want != total64 ? want / 8 * 8 : want);
+      if (grid > max_grid) grid = max_grid;
+    }
   }
-  int sched = cfg ? cfg->schedule : SK_SCHED_AUTO;
   if (sched == SK_SCHED_AUTO) {
     // data-parallel when the last wave of tiles is (nearly) full: Stream-K's fix-up and the L2
     // reuse it gives up cost more than a tail of under 10 %.  Otherwise Stream-K, splitting only
