@@ -17,7 +17,7 @@ typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 enum { FIXUP_ATOMIC = 1, FIXUP_REDUCE = 2 };
 
 // Phase tracing (off unless the small-M translation unit is built with -DSK_PHASE_TRACE): thread 0
-// of every CTA stores the 100 MHz wall clock into slot `slot` of its row of g_trace_buf; the host
+// of every CTA stores the shader clock counter into slot `slot` of its row of g_trace_buf; the host
 // reads the table back with sk_debug_trace_read.  Slots: 0 kernel entry, 1-7 inside the
 // matrix-vector kernel's segment (loads issued, A staged, scales staged, barrier, loop start,
 // loop end), 8/9 before/after the store of C, 10/11 after the CTA's range / tile coordinates.
@@ -25,7 +25,7 @@ enum { FIXUP_ATOMIC = 1, FIXUP_REDUCE = 2 };
 extern __device__ long long g_trace_buf[2048 * 16];
 #define SK_TRACE(slot)                                                              \
   do {                                                                              \
-    if (threadIdx.x == 0) g_trace_buf[blockIdx.x * 16 + (slot)] = wall_clock64();  \
+    if (threadIdx.x == 0) g_trace_buf[blockIdx.x * 16 + (slot)] = (long long)__builtin_readcyclecounter();  \
   } while (0)
 #else
 #define SK_TRACE(slot)
