@@ -363,6 +363,55 @@ def test_fp32_reference_shape(sk, oracle):
     sk.workspace_status()
 
 
+def test_graph_capture_replays_match_eager(sk, oracle):
+    """The launches are capturable (no host synchronisation, no allocation; the workspace is cleared
+    by a fill kernel, not by a memset node): a captured sequence reduce fix-up -> atomic fix-up ->
+    Q4 matrix-vector is replayed several times, with eager launches and synchronisations in
+    between, and every replay must reproduce the eager results bit for bit (reduce, Q4) or within
+    tolerance (atomic: summation order varies)."""
+    import torch
+    rng = np.random.default_rng(77)
+    M, N, K = 512, 1024, 2048
+    A = _t((rng.random((M, K), dtype=np.float32) * 2 - 1).astype(np.float16))
+    B = _t((rng.random((N, K), dtype=np.float32) * 2 - 1).astype(np.float16))
+    a1 = _t((rng.random((1, K), dtype=np.float32) * 2 - 1).astype(np.float16))
+    Wq = _t(rng.integers(0, 256, (N, K // 2), dtype=np.uint8))
+    sc = _t(rng.uniform(0.005, 0.02, (N, K // 128)).astype(np.float16))
+    red = dict(bm=128, bn=128, bk=64, schedule="basic", fixup="reduce", grid=40)
+    atm = dict(bm=128, bn=128, bk=64, schedule="basic", fixup="atomic", grid=40)
+    eager_red = sk.streamk_fp16(A, B, **red)
+    eager_q4 = sk.streamk_q4(a1, Wq, sc, schedule="sk2", grid=48, fixup="reduce")
+    ref = oracle.matmul_fp32(A.cpu().numpy(), B.cpu().numpy(), trans_b=True)
+    side = torch.cuda.Stream()
+    c_red = torch.empty(M, N, dtype=torch.float16, device="cuda")
+    c_atm = torch.empty(M, N, dtype=torch.float16, device="cuda")
+    c_q4 = torch.empty(1, N, dtype=torch.float16, device="cuda")
+    with torch.cuda.stream(side):
+        p_red = sk.make_plan(M, N, K, "float16", "nt", red)
+        p_atm = sk.make_plan(M, N, K, "float16", "nt", atm)
+        p_q4 = sk.make_plan(1, N, K, "q4", "nt", dict(schedule="sk2", grid=48, fixup="reduce"))
+        for _ in range(2):  # warm up on the capture stream: its workspace is created and initialised here
+            sk.streamk_fp16(A, B, out=c_red, plan=p_red)
+            sk.streamk_fp16(A, B, out=c_atm, plan=p_atm)
+            sk.streamk_q4(a1, Wq, sc, out=c_q4, plan=p_q4)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            sk.streamk_fp16(A, B, out=c_red, plan=p_red)
+            sk.streamk_fp16(A, B, out=c_atm, plan=p_atm)
+            sk.streamk_q4(a1, Wq, sc, out=c_q4, plan=p_q4)
+    for replay in range(4):
+        c_red.zero_(); c_atm.zero_(); c_q4.zero_()
+        sk.streamk_fp16(A, B, **atm)  # eager work on the default stream between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(c_red, eager_red), replay
+        assert torch.equal(c_q4, eager_q4), replay
+        assert _rel(oracle, c_atm, ref) <= 2e-3 <= TOL, replay
+    sk.workspace_status()
+
+
 def test_strided_operands_and_out(sk, oracle):
     """Leading dimensions larger than the rows, and writing into a caller-provided C."""
     import torch
