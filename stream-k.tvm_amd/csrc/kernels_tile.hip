@@ -4,10 +4,20 @@
 
 namespace sk {
 
-template <class P>
+template <class P, bool FIXUP = true>
 __global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_tile_kernel(typename P::Args a, DevPlan plan, Workspace ws) {
   __shared__ __attribute__((aligned(16))) char smem[P::LDS_BYTES];  // policies with their own LDS arrays keep this at 16 bytes
-  run_persistent<P>(a, plan, ws, smem);
+  run_persistent<P, FIXUP>(a, plan, ws, smem);
+}
+
+// data-parallel launches of the direct-to-LDS kernels use the instance without fix-up code
+template <class P>
+static int launch_dma(const GemmArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s) {
+  if (p.sk_tiles == 0)
+    hipLaunchKernelGGL((sk_tile_kernel<P, false>), dim3(p.grid), dim3(P::NT), 0, s, a, p, ws);
+  else
+    hipLaunchKernelGGL((sk_tile_kernel<P, true>), dim3(p.grid), dim3(P::NT), 0, s, a, p, ws);
+  return (int)hipGetLastError();
 }
 
 #define SK_POLICY(id, BM, BN, BK, WM, WN) TileF16NT<BM, BN, BK, WM, WN>
@@ -64,25 +74,22 @@ int launch_tile_f16(int id, const GemmArgs &a, const DevPlan &p, const Workspace
 #undef X
 #define X(id_, BM, BN, WM, WN)                                                           \
   case id_: {                                                                            \
-    typedef SK_POLICY_DMA(id_, BM, BN, WM, WN) P;                                        \
-    hipLaunchKernelGGL(sk_tile_kernel<P>, dim3(p.grid), dim3(P::NT), 0, s, a, p, ws);    \
-    return (int)hipGetLastError();                                                       \
+    typedef SK_POLICY_DMA(id_, BM, BN, WM, WN) P;                                      \
+    return launch_dma<P>(a, p, ws, s);                                                       \
   }
     SK_TILE_F16_NT_DMA_KERNELS(X)
 #undef X
 #define X(id_, BM, BN, WM, WN)                                                           \
   case id_: {                                                                            \
-    typedef SK_POLICY_NN(id_, BM, BN, WM, WN) P;                                         \
-    hipLaunchKernelGGL(sk_tile_kernel<P>, dim3(p.grid), dim3(P::NT), 0, s, a, p, ws);    \
-    return (int)hipGetLastError();                                                       \
+    typedef SK_POLICY_NN(id_, BM, BN, WM, WN) P;                                      \
+    return launch_dma<P>(a, p, ws, s);                                                       \
   }
     SK_TILE_F16_NN_DMA_KERNELS(X)
 #undef X
 #define X(id_, BM, BN, WM, WN)                                                           \
   case id_: {                                                                            \
     typedef SK_POLICY_DMA32(id_, BM, BN, WM, WN) P;                                      \
-    hipLaunchKernelGGL(sk_tile_kernel<P>, dim3(p.grid), dim3(P::NT), 0, s, a, p, ws);    \
-    return (int)hipGetLastError();                                                       \
+    return launch_dma<P>(a, p, ws, s);                                                       \
   }
     SK_TILE_F16_NT_DMA32_KERNELS(X)
 #undef X

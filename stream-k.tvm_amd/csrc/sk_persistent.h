@@ -13,7 +13,10 @@
 
 namespace sk {
 
-template <class P>
+// FIXUP = false: an instance for launches without Stream-K tiles.  Every segment is a whole tile
+// and the fix-up code is not compiled in -- its hundreds of partial-tile addresses otherwise
+// shape the register allocation of the main loop (spills in the 256x256 kernels).
+template <class P, bool FIXUP = true>
 __device__ __forceinline__ void run_persistent(const typename P::Args &a, const DevPlan &plan,
                                                const Workspace &ws, char *smem) {
   __shared__ int s_word;
@@ -51,8 +54,8 @@ __device__ __forceinline__ void run_persistent(const typename P::Args &a, const 
     P::mac(a, acc, pm, pn, k0, n, smem);
 
     // a segment that is the whole tile is simply stored (streamk_fp32.py:128-129)
-    bool store = (n == ipt);
-    if (!store) {
+    bool store = (n == ipt) || !FIXUP;
+    if (FIXUP && !store) {
       if (plan.fixup == FIXUP_ATOMIC) {
         // fp32 atomicAdd into the tile's accumulation buffer; whoever completes the K range
         // converts and stores, then leaves buffer and counter zeroed for the next launch.
