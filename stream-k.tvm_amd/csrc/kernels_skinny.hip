@@ -7,10 +7,21 @@ namespace sk {
 __device__ long long g_trace_buf[2048 * 16];
 #endif
 
-template <class P>
+template <class P, bool FIXUP = true>
 __global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_skinny_kernel(typename P::Args a, DevPlan plan, Workspace ws) {
   __shared__ __attribute__((aligned(16))) char smem[P::LDS_BYTES];
-  run_persistent<P>(a, plan, ws, smem);
+  run_persistent<P, FIXUP>(a, plan, ws, smem);
+}
+
+// launches without Stream-K tiles use the instance without fix-up code: these kernels run for a
+// few microseconds, most of which is set-up executed from a cold instruction cache
+template <class P>
+static int launch_policy(const SkinnyArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s) {
+  if (p.sk_tiles == 0)
+    hipLaunchKernelGGL((sk_skinny_kernel<P, false>), dim3(p.grid), dim3(P::NT), 0, s, a, p, ws);
+  else
+    hipLaunchKernelGGL((sk_skinny_kernel<P, true>), dim3(p.grid), dim3(P::NT), 0, s, a, p, ws);
+  return (int)hipGetLastError();
 }
 
 #define SK_POLICY(MB, NB, WN, RK, Q4, DEPTH, ROW1) TileSkinny<MB, NB, WN, RK, (Q4) != 0, DEPTH, (ROW1) != 0>
@@ -45,16 +56,14 @@ int launch_skinny(int id, const SkinnyArgs &a, const DevPlan &p, const Workspace
 #define X(id_, MB, NB, WN, RK, Q4, DEPTH, ROW1)                                                \
   case id_: {                                                                              \
     typedef SK_POLICY(MB, NB, WN, RK, Q4, DEPTH, ROW1) P;                                        \
-    hipLaunchKernelGGL(sk_skinny_kernel<P>, dim3(p.grid), dim3(P::NT), 0, s, a, p, ws);    \
-    return (int)hipGetLastError();                                                         \
+    return launch_policy<P>(a, p, ws, s);                                                         \
   }
     SK_SKINNY_KERNELS(X)
 #undef X
 #define X(id_, NB, WN, RK, DEPTH, KMAX)                                                        \
   case id_: {                                                                              \
     typedef TileGemvQ4<NB, WN, RK, DEPTH, KMAX> P;                                          \
-    hipLaunchKernelGGL(sk_skinny_kernel<P>, dim3(p.grid), dim3(P::NT), 0, s, a, p, ws);    \
-    return (int)hipGetLastError();                                                         \
+    return launch_policy<P>(a, p, ws, s);                                                         \
   }
     SK_GEMV_Q4_KERNELS(X)
 #undef X
