@@ -72,7 +72,8 @@ typedef struct sk_config {
   int32_t raster;         /* 0: row-major tile order (streamk_fp32.py:106-107); g>0: tiles walk g
                              rows down before stepping one column (triton_impl.py:14-28) */
   int32_t spin_limit;     /* REDUCE fix-up: polls of a peer flag before giving up; 0 = default */
-  int32_t reserved[4];
+  int32_t reserved[4];    /* reserved[0]: 0 = preferred kernel variant of the tile, v > 0 = variant v - 1
+                             (implementation alternatives of one tile shape, for the autotuner) */
 } sk_config;
 
 /* Result of the host partitioner: the integers of streamk_fp32.py:30-54 for the chosen tile/grid. */
@@ -147,13 +148,17 @@ int sk_gemm_f32(const void *A, const void *B, void *C, int64_t M, int64_t N, int
  *   scales  [N, K/group] fp16, w = fp16_rn((fp16(q) - zero) * scale)
  * Replaces tl_mod(A, QLB, C) of streamk_fp16_ladder_block_reduce_q4.py:597-599; the weights stay in
  * the natural byte order above (no LadderPermutate / LOP3Permutate step, :568-595).
- * Requirements: K multiple of 256, group == 128, 0 <= zero <= 15.
+ * Requirements: K multiple of 128, group == 128, 0 <= zero <= 15.
+ * For M == 1 the matrix-vector kernels multiply the nibbles undecoded and apply zero point and
+ * scale to fp32 group sums, i.e. they use the unrounded (q - zero) * scale: at least as close to
+ * the exact product as the rounded-weight form (within 2^-11 relative per weight of it).
+ * sk_dequant_q4 and the M > 1 kernels produce the rounded weights bit for bit.
  */
 int sk_gemm_q4(const void *A, const void *Wq, const void *scales, void *C, int64_t M, int64_t N,
                int64_t K, int64_t lda, int64_t ldc, int group, int zero, const sk_plan *plan,
                void *ws, size_t ws_bytes, void *stream);
 
-/* Device dequantisation of Wq into fp16 W[N,K] with the very device function the GEMM uses
+/* Device dequantisation of Wq into fp16 W[N,K] with the device function the M > 1 GEMM uses
  * (the closed form of streamk_fp16_ladder_block_reduce_q4.py:548-554 plus zero/scale). */
 int sk_dequant_q4(const void *Wq, const void *scales, void *W, int64_t N, int64_t K, int group,
                   int zero, void *stream);
