@@ -24,7 +24,7 @@ struct KernelInfo {
   int variant;  // tile kernels -- 0: registers -> padded LDS rows; 1: direct global -> LDS loads,
                 // swizzled rows; 2: as 1 with four waves per CTA (one per SIMD, accumulators in AGPRs);
                 // 3: as 1 with BK = 32 and four LDS stages (loads three iterations ahead)
-                // small-M kernels -- 0: up to 16*MB rows of A; 1: M == 1; 2: M == 1, Q4 matrix-vector
+                // small-M kernels -- 0: up to 16*MB rows of A; 1: M == 1; 2: M == 1, matrix-vector on 4x4x4 MFMA
   int bm, bn, bk;  // CTA tile; bk is the K extent of one CTA iteration
   int threads;
   int lds_bytes;
@@ -110,6 +110,17 @@ struct KernelInfo {
   X(149, 1, 1, 8, 4, 16384)    \
   X(150, 1, 1, 4, 4, 32768)    \
   X(151, 1, 2, 4, 4, 32768)
+
+// M == 1 fp16 (NT) matrix-vector kernels (variant 2):  X(id, NB, WN, RK, DEPTH, KMAX)
+#define SK_GEMV_F16_KERNELS(X) \
+  X(160, 1, 1, 4, 4, 8192)     \
+  X(161, 1, 1, 8, 4, 8192)     \
+  X(162, 2, 1, 4, 2, 8192)     \
+  X(163, 1, 4, 1, 4, 8192)     \
+  X(164, 1, 2, 2, 4, 8192)     \
+  X(165, 1, 1, 2, 4, 8192)     \
+  X(166, 1, 1, 4, 4, 32768)    \
+  X(167, 2, 1, 4, 2, 32768)
 
 const KernelInfo *kernel_table(int *count);
 const KernelInfo *kernel_by_id(int id);

@@ -48,6 +48,15 @@ int skinny_kernel_infos(KernelInfo *out, int max) {
   }
   SK_GEMV_Q4_KERNELS(X)
 #undef X
+#define X(id, NB, WN, RK, DEPTH, KMAX)                                                                        \
+  if (n < max) {                                                                                         \
+    typedef TileGemvF16<NB, WN, RK, DEPTH, KMAX> P;                                                       \
+    out[n++] = KernelInfo{id, FAMILY_SKINNY, 0, 0, 2, P::BM, P::BN, P::BKC, P::NT, P::LDS_BYTES,         \
+                          P::CTAS_PER_CU, P::TILE_ELEMS, P::MAX_ITERS, P::MAX_M, 8,                      \
+                          "gemv_f16_nb" #NB "_wn" #WN "_rk" #RK "_k" #KMAX};                                    \
+  }
+  SK_GEMV_F16_KERNELS(X)
+#undef X
   return n;
 }
 
@@ -66,6 +75,13 @@ int launch_skinny(int id, const SkinnyArgs &a, const DevPlan &p, const Workspace
     return launch_policy<P>(a, p, ws, s);                                                         \
   }
     SK_GEMV_Q4_KERNELS(X)
+#undef X
+#define X(id_, NB, WN, RK, DEPTH, KMAX)                                                        \
+  case id_: {                                                                              \
+    typedef TileGemvF16<NB, WN, RK, DEPTH, KMAX> P;                                         \
+    return launch_policy<P>(a, p, ws, s);                                                         \
+  }
+    SK_GEMV_F16_KERNELS(X)
 #undef X
   }
   return (int)hipErrorInvalidValue;
@@ -91,6 +107,15 @@ int occupancy_skinny(int id) {
     return occ;                                                                                          \
   }
     SK_GEMV_Q4_KERNELS(X)
+#undef X
+#define X(id_, NB, WN, RK, DEPTH, KMAX)                                                                      \
+  case id_: {                                                                                            \
+    typedef TileGemvF16<NB, WN, RK, DEPTH, KMAX> P;                                                       \
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_skinny_kernel<P>, P::NT, 0) != hipSuccess) \
+      return -1;                                                                                         \
+    return occ;                                                                                          \
+  }
+    SK_GEMV_F16_KERNELS(X)
 #undef X
   }
   return -1;

@@ -7,6 +7,7 @@
 #include "tile_f16.h"
 #include "tile_f16_dma.h"
 #include "tile_f32.h"
+#include "tile_gemv_f16.h"
 #include "tile_gemv_q4.h"
 #include "tile_skinny.h"
 

@@ -77,6 +77,12 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
         if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].variant == 2 && t[i].bn == 16 &&
             t[i].bk == 1024 && accepts_shape(t[i], M, K))
           return &t[i];
+    // M == 1 with fp16 weights: the same structure, K split over four waves
+    if (dtype == SK_F16 && M == 1 && want_variant < 0)
+      for (int i = 0; i < n; ++i)
+        if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].layout == layout && t[i].variant == 2 &&
+            t[i].bn == 16 && t[i].bk == 512 && accepts_shape(t[i], M, K))
+          return &t[i];
     int mb = M <= 16 ? 16 : (M <= 32 ? 32 : 64);
     for (int i = 0; i < n; ++i)
       if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].bm == mb && t[i].bn == 64 &&

@@ -236,6 +236,46 @@ def test_q4_matrix_vector_exact_on_integer_data(sk):
     sk.workspace_status()
 
 
+F16_GEMV_TILES = [(16, 16, 512), (16, 16, 1024), (16, 32, 512), (16, 64, 128), (16, 32, 256), (16, 16, 256)]
+
+
+def test_f16_matrix_vector_every_kernel(sk, oracle):
+    """Every fp16 matrix-vector instance (M = 1, NT) on ragged shapes: N not a multiple of 16, K a
+    multiple of 8 only, a strided W, K beyond 8192 (the instances that keep a longer A in LDS), all
+    schedules and both fix-ups, against the fp32 host product.  On integer data (|sums| < 2048) the
+    result must be exact."""
+    import torch
+    rng = np.random.default_rng(71)
+    ran = 0
+    for (N, K, pad) in [(1000, 1160, 0), (520, 392, 8), (72, 4096, 0), (2048, 8192, 64), (264, 28672, 0), (4099, 11008, 0)]:
+        A = (rng.random((1, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+        W = (rng.random((N, K + pad), dtype=np.float32) * 2 - 1).astype(np.float16)
+        Ai = rng.integers(-1, 2, (1, K)).astype(np.float16)
+        Wi = rng.integers(-2, 3, (N, K + pad)).astype(np.float16)
+        ref = oracle.matmul_fp32(A, W[:, :K], trans_b=True)
+        exact = Wi[:, :K].astype(np.int64) @ Ai[0].astype(np.int64)
+        assert np.abs(exact).max() < 2048
+        dA, dW, dAi, dWi = _t(A), _t(W)[:, :K], _t(Ai), _t(Wi)[:, :K]
+        for (bm, bn, bk) in F16_GEMV_TILES:
+            for sch in (dict(schedule="dp"), dict(schedule="sk2", fixup="reduce", grid=48),
+                        dict(schedule="sk2", fixup="atomic", grid=40), dict(schedule="basic", fixup="reduce", grid=56)):
+                try:
+                    plan = sk.make_plan(1, N, K, "float16", "nt", dict(bm=bm, bn=bn, bk=bk, variant=3, **sch))
+                except sk.StreamKError:
+                    assert K > 8192  # only some instances take a long K
+                    continue
+                C = sk.streamk_fp16(dA, dW, plan=plan)
+                assert _rel(oracle, C, ref) <= 2e-3 <= TOL, (N, K, bm, bn, bk, sch, plan.kernel_id)
+                C = sk.streamk_fp16(dAi, dWi, plan=plan)
+                assert np.array_equal(C.cpu().numpy()[0].astype(np.int64), exact), (N, K, bm, bn, bk, sch)
+                ran += 1
+    assert ran >= 100
+    # the heuristic plan for M = 1 is one of these kernels
+    plan = sk.make_plan(1, 4096, 4096, "float16", "nt", {})
+    assert (plan.bm, plan.bn, plan.bk) == (16, 16, 512) and 160 <= plan.kernel_id < 170
+    sk.workspace_status()
+
+
 def test_cfg5_large_dense(sk, oracle):
     """M = N = K = 8192 and the irregular 3000 x 5120 x 12288, U[-1,1): a random subset of rows is
     checked against an fp64 host product; the Stream-K and data-parallel schedules of the same kernel
