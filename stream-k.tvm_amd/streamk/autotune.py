@@ -105,8 +105,13 @@ def _time_ms(fn, warmup, rep, graph):
 
 
 def autotune(M, N, K, dtype="float16", layout="nt", *, configs=None, warmup=5, rep=20, check=True,
-             cache=True, cache_path=None, verbose=False):
+             cache=True, cache_path=None, verbose=False, weights=None):
     """Searches `configs` (default: candidate_configs) for the fastest plan.
+
+    weights="hbm" times every candidate on a rotation of copies of the weight operand (more than
+    512 MB in total), so that each launch reads its weights from HBM as a layer of a model larger
+    than the 256 MB Infinity Cache does; weights="warm" reuses one copy.  Default: "hbm" for
+    M <= 64, where the launch is a stream over the weights, "warm" otherwise.
 
     Returns (best_latency_ms, best_config, ref_latency_ms); ref is torch.matmul on the same GPU, the
     reference's comparator (streamk_fp16.py:396) -- None for Q4.  Every candidate is checked against
@@ -116,18 +121,28 @@ def autotune(M, N, K, dtype="float16", layout="nt", *, configs=None, warmup=5, r
     g = torch.Generator(device="cpu").manual_seed(0)
     A = (torch.rand(M, K, generator=g) * 2 - 1).half().to(dev)
     C = torch.empty(M, N, dtype=torch.float16, device=dev)
+    weights = weights or ("hbm" if M <= 64 else "warm")
+    wbytes = N * K // 2 if dtype == "q4" else N * K * 2
+    copies = 1 if weights == "warm" else max(2, min(rep, -(-(512 << 20) // wbytes)))
+    turn = [0]
+
+    def rotate(items):
+        turn[0] += 1
+        return items[turn[0] % len(items)]
     if dtype == "q4":
         Wq = torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8).to(dev)
         sc = (torch.rand(N, K // 128, generator=g) * 0.015 + 0.005).half().to(dev)
-        run = lambda p: ops.streamk_q4(A, Wq, sc, out=C, plan=p)  # noqa: E731
+        Ws = [(Wq, sc)] + [(Wq.clone(), sc.clone()) for _ in range(copies - 1)]
+        run = lambda p: ops.streamk_q4(A, *rotate(Ws), out=C, plan=p)  # noqa: E731
         ref_ms = None
     else:
         bshape = (N, K) if layout == "nt" else (K, N)
         B = (torch.rand(*bshape, generator=g) * 2 - 1).half().to(dev)
-        run = lambda p: ops.streamk_fp16(A, B, layout=layout, out=C, plan=p)  # noqa: E731
-        Bt = B.T if layout == "nt" else B
+        Bs = [B] + [B.clone() for _ in range(copies - 1)]
+        run = lambda p: ops.streamk_fp16(A, rotate(Bs), layout=layout, out=C, plan=p)  # noqa: E731
         small = 2.0 * M * N * K < 5e10
-        ref_ms = _time_ms(lambda: torch.matmul(A, Bt, out=C), warmup, rep, small)
+        as_b = (lambda b: b.T) if layout == "nt" else (lambda b: b)
+        ref_ms = _time_ms(lambda: torch.matmul(A, as_b(rotate(Bs)), out=C), warmup, rep, small)
     small = 2.0 * M * N * K < 5e10  # microsecond kernels: time graph-captured batches
     configs = configs if configs is not None else candidate_configs(M, N, K, dtype)
     best, golden, results = None, None, []
