@@ -163,6 +163,28 @@ int sk_gemm_q4(const void *A, const void *Wq, const void *scales, void *C, int64
 int sk_dequant_q4(const void *Wq, const void *scales, void *W, int64_t N, int64_t K, int group,
                   int zero, void *stream);
 
+/*
+ * Offline side of the Q4 path: what produces Wq and scales.  The reference packs two nibbles per
+ * byte (streamk_fp16_ladder_block_reduce_q4.py:545,552) and then runs BitBLAS LadderPermutate and
+ * LOP3Permutate over the array on the CPU (:568-595); this library reads the packed array as it is,
+ * so these calls replace that whole step.
+ *
+ * sk_q4_pack_host / sk_q4_unpack_host: q[N,K] bytes with values 0..15 <-> Wq[N,K/2] (host memory).
+ * sk_q4_quantize_host (host memory, W as fp16 bit patterns, row pitch ldw elements) and
+ * sk_q4_quantize (device memory, stream-ordered; group must be 128, ldw a multiple of 8, W 16-byte
+ * aligned) quantise fp16 weights group by group:
+ *   levels = min(zero, 15 - zero), or 15 if that is 0;  scale = fp16_rn(max|w| / levels);
+ *   q = clamp(rint(w / scale) + zero, 0, 15), divisions in fp32, ties to even; q = zero if scale is 0.
+ * Both produce the same bytes.  Weights must be finite (the host call returns SK_ERR_CONFIG otherwise,
+ * the device call does not look).
+ */
+int sk_q4_pack_host(const uint8_t *q, int64_t N, int64_t K, uint8_t *Wq);
+int sk_q4_unpack_host(const uint8_t *Wq, int64_t N, int64_t K, uint8_t *q);
+int sk_q4_quantize_host(const uint16_t *W, int64_t N, int64_t K, int64_t ldw, int group, int zero,
+                        uint8_t *Wq, uint16_t *scales);
+int sk_q4_quantize(const void *W, int64_t N, int64_t K, int64_t ldw, int group, int zero, void *Wq,
+                   void *scales, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

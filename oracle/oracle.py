@@ -163,6 +163,32 @@ def unpack_q4_np(Wq):
     return out
 
 
+def pack_q4_np(q):
+    """[N, K] nibbles -> [N, K/2] bytes, the array streamk_fp16_ladder_block_reduce_q4.py:552 expands
+    (element k in bits 4*(k&1).. of byte k/2)."""
+    q = np.asarray(q, dtype=np.uint8)
+    assert q.max(initial=0) <= 15
+    return (q[:, 0::2] | (q[:, 1::2] << 4)).astype(np.uint8)
+
+
+def quantize_q4_np(W, group=128, zero=8):
+    """Group-wise quantisation rule of this build (the reference draws random nibbles and has no
+    quantiser): scale = fp16(max|w| / levels), q = clamp(rint(w / scale) + zero, 0, 15), fp32
+    divisions; levels = min(zero, 15 - zero) or 15 if that is 0; q = zero where scale is 0.
+    Returns (Wq [N, K/2] uint8, scales [N, K/group] float16)."""
+    W = np.asarray(W, dtype=np.float16)
+    N, K = W.shape
+    levels = min(zero, 15 - zero) or 15
+    w = W.astype(np.float32).reshape(N, K // group, group)
+    amax = np.abs(w).max(axis=2)
+    sc = (amax / np.float32(levels)).astype(np.float16)
+    s = sc.astype(np.float32)[:, :, None]
+    with np.errstate(divide="ignore", invalid="ignore"):
+        q = np.rint(w / s) + np.float32(zero)
+    q = np.where(s == 0, np.float32(zero), np.clip(q, 0, 15)).astype(np.uint8).reshape(N, K)
+    return pack_q4_np(q), sc
+
+
 def dequant_q4_np(Wq, scales, group=128, zero=8):
     """numpy float16 evaluation: w = fp16((fp16(q) - fp16(zero)) * scale[n, k // group])."""
     q = unpack_q4_np(Wq).astype(np.float16)

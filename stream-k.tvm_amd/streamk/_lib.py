@@ -72,6 +72,12 @@ def lib():
     L.sk_gemm_f32.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, P(SkPlan), vp, sz, vp]
     L.sk_gemm_q4.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, ci, ci, P(SkPlan), vp, sz, vp]
     L.sk_dequant_q4.argtypes = [vp, vp, vp, i64, i64, ci, ci, vp]
+    L.sk_q4_pack_host.argtypes = [vp, i64, i64, vp]
+    L.sk_q4_unpack_host.argtypes = [vp, i64, i64, vp]
+    L.sk_q4_quantize_host.argtypes = [vp, i64, i64, i64, ci, ci, vp, vp]
+    L.sk_q4_quantize.argtypes = [vp, i64, i64, i64, ci, ci, vp, vp, vp]
+    for f in ("sk_q4_pack_host", "sk_q4_unpack_host", "sk_q4_quantize_host", "sk_q4_quantize"):
+        getattr(L, f).restype = ci
     for f in ("sk_device_info", "sk_make_plan", "sk_plan_cta_range", "sk_plan_tile_coords",
               "sk_workspace_init", "sk_workspace_status", "sk_gemm_f16", "sk_gemm_f32",
               "sk_gemm_q4", "sk_dequant_q4"):

@@ -1,0 +1,84 @@
+"""`torch.nn.Linear`-shaped caller of the Stream-K GEMMs: the step above `streamk_fp16`.
+
+The reference stops at kernel scripts; wrapping them as an operator of a model is its open item
+("integrate with BitBLAS", README.md:21).  This module is that wrapper for this library: it owns
+the weight in the layout the kernels read ([N, K] fp16, or packed nibbles + scales), flattens the
+leading dimensions of the input into M, and keeps one plan per M it has seen (a decode step calls
+with M = batch, a prefill with M = batch * tokens), each taken from the tuned cache when the shape
+is in it.  Inference only: the GEMM is not recorded by autograd.
+"""
+import torch
+
+from . import ops
+from .plan import make_plan
+
+
+class StreamKLinear(torch.nn.Module):
+    def __init__(self, in_features, out_features, bias=False, *, weight_format="float16", group=128, zero=8,
+                 device=None):
+        super().__init__()
+        if weight_format not in ("float16", "q4"):
+            raise ValueError("weight_format must be 'float16' or 'q4'")
+        if weight_format == "q4" and (group != 128 or in_features % 128):
+            raise ValueError("Q4 weights need group == 128 and in_features a multiple of 128")
+        if in_features % 8:
+            raise ValueError("in_features must be a multiple of 8")
+        self.in_features, self.out_features = in_features, out_features
+        self.weight_format, self.group, self.zero = weight_format, group, zero
+        N, K = out_features, in_features
+        if weight_format == "float16":
+            self.register_buffer("weight", torch.zeros(N, K, dtype=torch.float16, device=device))
+        else:
+            self.register_buffer("qweight", torch.zeros(N, K // 2, dtype=torch.uint8, device=device))
+            self.register_buffer("scales", torch.zeros(N, K // group, dtype=torch.float16, device=device))
+        self.register_buffer("bias", torch.zeros(N, dtype=torch.float16, device=device) if bias else None)
+        self._plans = {}
+
+    @classmethod
+    def from_linear(cls, linear, *, weight_format="float16", group=128, zero=8):
+        """Takes over the weight (and bias) of a torch.nn.Linear; weight_format='q4' quantises it
+        with `quantize_q4` on the device it lives on."""
+        w = linear.weight.detach().to(torch.float16).contiguous()
+        m = cls(linear.in_features, linear.out_features, linear.bias is not None, weight_format=weight_format,
+                group=group, zero=zero, device=w.device)
+        if weight_format == "float16":
+            m.weight.copy_(w)
+        else:
+            q, s = ops.quantize_q4(w, group=group, zero=zero)
+            m.qweight.copy_(q)
+            m.scales.copy_(s)
+        if linear.bias is not None:
+            m.bias.copy_(linear.bias.detach().to(torch.float16))
+        return m
+
+    def plan_for(self, M):
+        p = self._plans.get(M)
+        if p is None:
+            dtype = "float16" if self.weight_format == "float16" else "q4"
+            p = self._plans[M] = make_plan(M, self.out_features, self.in_features, dtype, "nt")
+        return p
+
+    @torch.no_grad()
+    def forward(self, x):
+        if x.dtype != torch.float16 or x.shape[-1] != self.in_features:
+            raise ValueError(f"input must be fp16 [..., {self.in_features}], got {x.dtype} {tuple(x.shape)}")
+        lead = x.shape[:-1]
+        a = x.reshape(-1, self.in_features)
+        if a.stride(-1) != 1 or (a.shape[0] > 1 and a.stride(0) % 8) or a.data_ptr() % 16:
+            a = a.contiguous()
+        M = a.shape[0]
+        if M == 0:
+            return x.new_zeros(*lead, self.out_features)
+        if self.weight_format == "float16":
+            c = ops.streamk_fp16(a, self.weight, plan=self.plan_for(M))
+        else:
+            # (more rows than one Q4 launch takes: streamk_q4 splits the call itself)
+            c = ops.streamk_q4(a, self.qweight, self.scales, plan=self.plan_for(M) if M <= ops.Q4_MAX_M else None,
+                               zero=self.zero, group=self.group)
+        if self.bias is not None:
+            c += self.bias
+        return c.view(*lead, self.out_features)
+
+    def extra_repr(self):
+        return (f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}, "
+                f"weight_format={self.weight_format}")

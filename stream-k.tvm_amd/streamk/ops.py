@@ -92,6 +92,9 @@ def streamk_fp16(A, B, *, Wq=None, scales=None, layout="nt", out=None, plan=None
     return C
 
 
+Q4_MAX_M = 64  # rows of A the Q4 kernels take in one launch
+
+
 def streamk_q4(A, Wq, scales, *, out=None, plan=None, config=None, zero=8, group=128, **kw):
     """C[M,N] fp16 = A[M,K] fp16 @ dequant(Wq)[N,K].T, weights in natural nibble order
     (streamk_fp16_ladder_block_reduce_q4.py:552)."""
@@ -104,10 +107,22 @@ def streamk_q4(A, Wq, scales, *, out=None, plan=None, config=None, zero=8, group
         raise ValueError(f"Wq must be contiguous [N, K/2]; got {tuple(Wq.shape)} for K={K}")
     if tuple(scales.shape) != (N, K // group) or not scales.is_contiguous():
         raise ValueError(f"scales must be contiguous [N, K/group]; got {tuple(scales.shape)}")
-    if plan is None:
-        plan = make_plan(M, N, K, "q4", "nt", config, **kw)
     C = out if out is not None else torch.empty((M, N), dtype=torch.float16, device=A.device)
     _check_matrix(C, "out", torch.float16)
+    if tuple(C.shape) != (M, N):
+        raise ValueError("out has the wrong shape")
+    if plan is None and M > Q4_MAX_M:
+        # the Q4 kernels stream the weights past at most 64 rows of A.  Up to 256 rows: one launch
+        # per block of 64 rows.  Beyond: dequantise once (bit-exact device function) and run the
+        # fp16 tile kernels, whose time then dwarfs the extra pass over the weights.
+        if M <= 4 * Q4_MAX_M:
+            for m0 in range(0, M, Q4_MAX_M):
+                streamk_q4(A[m0:m0 + Q4_MAX_M], Wq, scales, out=C[m0:m0 + Q4_MAX_M], config=config, zero=zero,
+                           group=group, **kw)
+            return C
+        return streamk_fp16(A, dequant_q4(Wq, scales, zero=zero, group=group), out=C)
+    if plan is None:
+        plan = make_plan(M, N, K, "q4", "nt", config, **kw)
     ws = _workspace(plan.workspace_bytes, A.device)
     rc = _lib.lib().sk_gemm_q4(A.data_ptr(), Wq.data_ptr(), scales.data_ptr(), C.data_ptr(), M, N, K,
                                A.stride(0), C.stride(0), group, zero, ctypes.byref(plan),
@@ -129,6 +144,48 @@ def dequant_q4(Wq, scales, *, zero=8, group=128):
                                   _stream_ptr())
     _lib.check(rc, "sk_dequant_q4")
     return W
+
+
+def pack_q4(q):
+    """Wq[N, K/2] from q[N, K] (uint8 values 0..15, host memory): element k of a row goes to nibble
+    k & 1 of byte k / 2, the order streamk_fp16_ladder_block_reduce_q4.py:552 expands.  This is the
+    array the kernels read: there is no further permutation step (the reference's :568-595)."""
+    if q.dtype != torch.uint8 or q.dim() != 2 or q.is_cuda or not q.is_contiguous():
+        raise ValueError("q must be a contiguous 2-D uint8 tensor in host memory")
+    N, K = q.shape
+    Wq = torch.empty((N, K // 2), dtype=torch.uint8)
+    _lib.check(_lib.lib().sk_q4_pack_host(q.data_ptr(), N, K, Wq.data_ptr()), "sk_q4_pack_host")
+    return Wq
+
+
+def unpack_q4(Wq):
+    """Inverse of pack_q4 (host memory)."""
+    if Wq.dtype != torch.uint8 or Wq.dim() != 2 or Wq.is_cuda or not Wq.is_contiguous():
+        raise ValueError("Wq must be a contiguous 2-D uint8 tensor in host memory")
+    N, K = Wq.shape[0], Wq.shape[1] * 2
+    q = torch.empty((N, K), dtype=torch.uint8)
+    _lib.check(_lib.lib().sk_q4_unpack_host(Wq.data_ptr(), N, K, q.data_ptr()), "sk_q4_unpack_host")
+    return q
+
+
+def quantize_q4(W, *, group=128, zero=8):
+    """(Wq[N, K/2] uint8, scales[N, K/group] fp16) from fp16 W[N, K], on the device W lives on.
+    scale = fp16(max|w| / levels) per group, q = clamp(rint(w / scale) + zero, 0, 15)."""
+    if W.dtype != torch.float16 or W.dim() != 2 or W.stride(1) != 1:
+        raise ValueError("W must be a 2-D fp16 tensor with unit stride along K")
+    N, K = W.shape
+    ldw = W.stride(0) if N > 1 else K  # the stride of a single row is arbitrary
+    Wq = torch.empty((N, K // 2), dtype=torch.uint8, device=W.device)
+    sc = torch.empty((N, K // max(group, 1)), dtype=torch.float16, device=W.device)
+    if W.is_cuda:
+        rc = _lib.lib().sk_q4_quantize(W.data_ptr(), N, K, ldw, group, zero, Wq.data_ptr(), sc.data_ptr(),
+                                       _stream_ptr())
+        _lib.check(rc, "sk_q4_quantize")
+    else:
+        rc = _lib.lib().sk_q4_quantize_host(W.data_ptr(), N, K, ldw, group, zero, Wq.data_ptr(),
+                                            sc.data_ptr())
+        _lib.check(rc, "sk_q4_quantize_host")
+    return Wq, sc
 
 
 def streamk_fp32(A, B, *, layout="nn", out=None, plan=None, config=None, **kw):

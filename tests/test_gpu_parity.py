@@ -276,6 +276,70 @@ def test_f16_matrix_vector_every_kernel(sk, oracle):
     sk.workspace_status()
 
 
+def test_device_quantiser_matches_host_and_feeds_the_gemm(sk, oracle):
+    """sk_q4_quantize on the device writes the bytes sk_q4_quantize_host and the numpy restatement
+    write (special groups included), and a Q4 GEMM on the result agrees with the fp32 product of
+    the dequantised weights; against the unquantised weights the error is that of 4-bit rounding."""
+    import torch
+    rng = np.random.default_rng(81)
+    for zero in (8, 0, 5, 15):
+        N, K, pad = 1000, 4096, 8
+        W = (rng.standard_normal((N, K + pad), dtype=np.float32) * 0.02).astype(np.float16)
+        W[0, :128] = 0
+        W[1, :128] = np.float16(6e-8) * rng.integers(-3, 4, 128)
+        W[2, :128] = 65504 * rng.choice([-1, 1], 128)
+        W[3, :128] = rng.integers(-40, 41, 128) * 0.25
+        dW = _t(W)[:, :K]
+        Wq, sc = sk.quantize_q4(dW, zero=zero)
+        hWq, hsc = sk.quantize_q4(torch.from_numpy(W)[:, :K], zero=zero)
+        nWq, nsc = oracle.quantize_q4_np(W[:, :K], zero=zero)
+        assert torch.equal(Wq.cpu(), hWq) and np.array_equal(hWq.numpy(), nWq)
+        assert torch.equal(sc.cpu().view(torch.int16), hsc.view(torch.int16))
+        assert np.array_equal(hsc.numpy().view(np.uint16), nsc.view(np.uint16))
+    W = (rng.standard_normal((2048, 4096), dtype=np.float32) * 0.02).astype(np.float16)
+    Wq, sc = sk.quantize_q4(_t(W))
+    for M in (1, 16):
+        A = rng.standard_normal((M, 4096), dtype=np.float32).astype(np.float16)
+        C = sk.streamk_q4(_t(A), Wq, sc)
+        ref_q = oracle.q4_gemm_ref(A, Wq.cpu().numpy(), sc.cpu().numpy())
+        assert _rel(oracle, C, ref_q) <= 2e-3 <= TOL
+        ref = oracle.matmul_fp32(A, W, trans_b=True)
+        assert _rel(oracle, C, ref) <= 0.12  # 4-bit weights: ~7 % rms per weight at 7 levels
+    sk.workspace_status()
+
+
+def test_linear_module_matches_functional_linear(sk, oracle):
+    """StreamKLinear (fp16 and Q4 weights, with bias) against the fp32 host product for the shapes
+    a model sends: one token, a decode batch, a [batch, tokens, K] prefill, an unaligned slice."""
+    import torch
+    torch.manual_seed(5)
+    lin = torch.nn.Linear(1024, 1536, bias=True).half().cuda()
+    lin.weight.data.mul_(2.0)
+    fp = sk.StreamKLinear.from_linear(lin)
+    q4 = sk.StreamKLinear.from_linear(lin, weight_format="q4")
+    Wd = oracle.dequant_q4(q4.qweight.cpu().numpy(), q4.scales.cpu().numpy()).astype(np.float32)
+    Wf, b = lin.weight.detach().float().cpu().numpy(), lin.bias.detach().float().cpu().numpy()
+    big = torch.randn(40, 1032, device="cuda").half()
+    for x in (torch.randn(1, 1024, device="cuda").half(), torch.randn(16, 1024, device="cuda").half(),
+              torch.randn(3, 50, 1024, device="cuda").half(), big[:, 1:1025], torch.randn(1024, device="cuda").half(),
+              torch.randn(2, 300, 1024, device="cuda").half()):
+        xf = x.float().cpu().numpy().reshape(-1, 1024)
+        for mod, W in ((fp, Wf), (q4, Wd)):
+            y = mod(x)
+            assert y.shape == x.shape[:-1] + (1536,) and y.dtype == torch.float16
+            ref = xf @ W.T + b
+            assert oracle.max_abs_rel(y.float().cpu().numpy().reshape(-1, 1536), ref) <= 2e-3 <= TOL
+    assert set(fp._plans) == {1, 16, 150, 40, 600} and set(q4._plans) == {1, 16, 40} and set(q4.state_dict()) == {"qweight", "scales", "bias"}
+    # state round trip into a freshly constructed module
+    fresh = sk.StreamKLinear(1024, 1536, bias=True, weight_format="q4", device="cuda")
+    fresh.load_state_dict(q4.state_dict())
+    x = torch.randn(4, 1024, device="cuda").half()
+    assert torch.equal(fresh(x), q4(x))
+    with pytest.raises(ValueError):
+        fp(torch.randn(4, 1000, device="cuda").half())
+    sk.workspace_status()
+
+
 def test_cfg5_large_dense(sk, oracle):
     """M = N = K = 8192 and the irregular 3000 x 5120 x 12288, U[-1,1): a random subset of rows is
     checked against an fp64 host product; the Stream-K and data-parallel schedules of the same kernel
