@@ -47,7 +47,13 @@ typedef enum sk_schedule {
   SK_SCHED_SK_TWO_TILE = 2,/* reference hybrid: (tiles % P) + P Stream-K tiles, rest data-parallel
                               (streamk_fp32.py:37-43) */
   SK_SCHED_SK_ONE_TILE = 3,/* tiles % P Stream-K tiles, rest data-parallel */
-  SK_SCHED_SK_BASIC = 4    /* every tile is a Stream-K tile (figures/image.png "basic Stream-K") */
+  SK_SCHED_SK_BASIC = 4,   /* every tile is a Stream-K tile (figures/image.png "basic Stream-K") */
+  SK_SCHED_SPLIT_K = 5     /* fixed split: every tile is cut into `split` equal K ranges, one CTA each, grid =
+                              tiles * split (the comparator of dataparallel.fp16.breakdown/
+                              thread_level_gemm_with_macro_ladder_atomic_reduce.py:129-131,153-154).  split
+                              comes from sk_config.reserved[1]; 0 picks the largest factor that divides the
+                              K-iterations of a tile, leaves at least 4 of them per CTA and keeps the grid
+                              resident.  Both fix-ups apply (the reference's atomicAdd into C is ATOMIC). */
 } sk_schedule;
 
 /* How partial tiles of the Stream-K wave are combined. */
@@ -73,7 +79,8 @@ typedef struct sk_config {
                              rows down before stepping one column (triton_impl.py:14-28) */
   int32_t spin_limit;     /* REDUCE fix-up: polls of a peer flag before giving up; 0 = default */
   int32_t reserved[4];    /* reserved[0]: 0 = preferred kernel variant of the tile, v > 0 = variant v - 1
-                             (implementation alternatives of one tile shape, for the autotuner) */
+                             (implementation alternatives of one tile shape, for the autotuner);
+                             reserved[1]: split factor of SK_SCHED_SPLIT_K, 0 = choose */
 } sk_config;
 
 /* Result of the host partitioner: the integers of streamk_fp32.py:30-54 for the chosen tile/grid. */

@@ -168,6 +168,19 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
       if (grid > max_grid) grid = max_grid;
     }
   }
+  if (sched == SK_SCHED_SPLIT_K) {
+    // fixed split: the grid follows from the split factor, a caller's grid is not consulted
+    const int ipt = out->iters_per_tile;
+    int split = cfg ? cfg->reserved[1] : 0;
+    if (split < 0) return SK_ERR_CONFIG;
+    if (split == 0) {
+      split = 1;
+      for (int s = 2; s <= ipt / 4 && total64 * s <= max_grid; ++s)
+        if (ipt % s == 0) split = s;
+    }
+    if (ipt % split != 0 || total64 * split > max_grid) return SK_ERR_CONFIG;
+    grid = (int)(total64 * split);
+  }
   if (sched == SK_SCHED_AUTO) {
     // data-parallel when the last wave of tiles is (nearly) full: Stream-K's fix-up and the L2
     // reuse it gives up cost more than a tail of under 10 %.  Otherwise Stream-K, splitting only
@@ -188,6 +201,7 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
       break;
     case SK_SCHED_SK_ONE_TILE: sk_tiles = total % grid; break;
     case SK_SCHED_SK_BASIC: sk_tiles = total; break;
+    case SK_SCHED_SPLIT_K: sk_tiles = grid == total ? 0 : total; break;  // split 1 is data-parallel
     default: return SK_ERR_CONFIG;
   }
   out->schedule = sched;

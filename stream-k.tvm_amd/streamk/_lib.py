@@ -10,7 +10,7 @@ LIB_PATH = os.path.join(_HERE, "libstreamk.so")
 
 SK_F16, SK_F32, SK_Q4 = 0, 1, 2
 LAYOUT_NT, LAYOUT_NN = 0, 1
-SCHEDULES = {"auto": 0, "dp": 1, "sk2": 2, "sk1": 3, "basic": 4}
+SCHEDULES = {"auto": 0, "dp": 1, "sk2": 2, "sk1": 3, "basic": 4, "splitk": 5}
 FIXUPS = {"auto": 0, "atomic": 1, "reduce": 2}
 
 

@@ -78,6 +78,9 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
                 grids = (None,) if bm * bn >= 256 * 256 else (None, cus)
                 for sched, fixup, grid in itertools.product(("sk2", "sk1", "basic"), ("reduce", "atomic"), grids):
                     out.append(dict(base, schedule=sched, fixup=fixup, **({"grid": grid} if grid else {})))
+                # fixed split-K, the fallback when there are fewer tiles than CUs
+                if -(-M // bm) * -(-N // bn) < cus:
+                    out.extend(dict(base, schedule="splitk", fixup=fixup) for fixup in ("reduce", "atomic"))
     return out
 
 

@@ -22,7 +22,7 @@ def num_cus():
 
 def make_config(config=None, **kw):
     """dict / kwargs -> SkConfig.  Keys: bm, bn, bk, grid, schedule ('auto'|'dp'|'sk2'|'sk1'|
-    'basic'), fixup ('auto'|'atomic'|'reduce'), raster, spin_limit."""
+    'basic'|'splitk'), split, fixup ('auto'|'atomic'|'reduce'), raster, spin_limit, variant."""
     d = dict(config or {})
     d.update(kw)
     c = SkConfig()
@@ -35,6 +35,9 @@ def make_config(config=None, **kw):
             v = _lib.FIXUPS[v] if isinstance(v, str) else int(v)
         if k == "variant":  # 0 = newest kernel variant of the tile, v > 0 = variant v - 1
             c.reserved[0] = int(v)
+            continue
+        if k == "split":  # factor of schedule 'splitk'; 0 = choose
+            c.reserved[1] = int(v)
             continue
         if k not in ("bm", "bn", "bk", "grid", "schedule", "fixup", "raster", "spin_limit"):
             raise KeyError(f"unknown Stream-K config key {k!r}")

@@ -69,6 +69,28 @@ def test_schedules(sk):
     assert (auto.bm, auto.bn, auto.schedule, auto.streamk_tiles) == (256, 256, 1, 0)
 
 
+def test_fixed_split_k_schedule(sk):
+    """Every tile is cut into `split` equal K ranges, CTA g owning range g % split of tile g // split:
+    the grid of thread_level_gemm_with_macro_ladder_atomic_reduce.py:129-131 flattened, K range of
+    :153-154."""
+    kw = dict(cus=256, bm=128, bn=128, bk=64)
+    p = sk.make_plan(1024, 1024, 8192, "float16", "nt", schedule="splitk", split=4, **kw)
+    assert (p.grid, p.streamk_tiles, p.blocking_tiles, p.iters_per_tile) == (256, 64, 0, 128)
+    for g in range(p.grid):
+        tile, part = divmod(g, 4)
+        assert sk.cta_range(p, g) == (tile * 128 + part * 32, tile * 128 + (part + 1) * 32)
+    # split 0: the largest factor of 128 that keeps 64 * split CTAs resident (2 per CU here)
+    p = sk.make_plan(1024, 1024, 8192, "float16", "nt", schedule="splitk", **kw)
+    assert p.grid == 64 * 8 and sk.cta_range(p, 9) == (128 + 16, 128 + 32)
+    # split 1 is the data-parallel schedule; a factor that does not divide the K-iterations, or a
+    # grid beyond what stays resident, is refused
+    p = sk.make_plan(1024, 1024, 8192, "float16", "nt", schedule="splitk", split=1, **kw)
+    assert (p.grid, p.streamk_tiles, p.workspace_bytes) == (64, 0, 0)
+    for bad in (3, 16):
+        with pytest.raises(sk.StreamKError):
+            sk.make_plan(1024, 1024, 8192, "float16", "nt", schedule="splitk", split=bad, **kw)
+
+
 def test_raster_is_a_permutation(sk):
     plan = sk.make_plan(3000, 5120, 4096, "float16", "nt", cus=256, bm=128, bn=128, bk=64, raster=8)
     seen = {sk.tile_coords(plan, t) for t in range(plan.total_tiles)}

@@ -94,6 +94,36 @@ def test_cfg2_streamk_both_fixups(sk, oracle, cfg, fixup):
     assert _rel(oracle, C, ref) <= 1e-3 <= TOL
 
 
+def test_fixed_split_k(sk, oracle):
+    """Fixed split-K (the reference's data-parallel comparator with splitk_factor,
+    thread_level_gemm_with_macro_ladder_atomic_reduce.py:129-199) on tile and small-M kernels, both
+    fix-ups; with the ordered reduce it is the same partition as basic Stream-K on tiles * split CTAs,
+    so the two agree bit for bit."""
+    import torch
+    A, B = _uniform16((1024, 8192), 0), _uniform16((1024, 8192), 1)
+    ref = oracle.matmul_fp32(A, B, trans_b=True)
+    dA, dB = _t(A), _t(B)
+    for cfg in (dict(bm=128, bn=128, bk=64, split=4), dict(bm=128, bn=128, bk=32, variant=4, split=8),
+                dict(bm=256, bn=256, bk=64, split=16), dict(bm=64, bn=64, bk=64, split=2), dict(bm=128, bn=128, bk=64)):
+        for fixup in ("atomic", "reduce"):
+            plan = sk.make_plan(1024, 1024, 8192, "float16", "nt", schedule="splitk", fixup=fixup, **cfg)
+            assert plan.grid == plan.total_tiles * cfg.get("split", 8)
+            C = sk.streamk_fp16(dA, dB, plan=plan)
+            assert _rel(oracle, C, ref) <= 1e-3 <= TOL, (cfg, fixup)
+        same = dict(cfg)
+        same.pop("split", None)
+        basic = sk.streamk_fp16(dA, dB, schedule="basic", fixup="reduce", grid=plan.grid, **same)
+        assert torch.equal(C, basic), cfg
+    # small-M kernels: 16 x 4096 x 11008 with 16 x 64 x 128 tiles, 86 K-iterations = 2 * 43
+    A, B = _uniform16((16, 11008), 2), _uniform16((4096, 11008), 3)
+    ref = oracle.matmul_fp32(A, B, trans_b=True)
+    for fixup in ("atomic", "reduce"):
+        plan = sk.make_plan(16, 4096, 11008, "float16", "nt", bm=16, bn=64, bk=128, schedule="splitk", split=2, fixup=fixup)
+        assert plan.grid == 128 and plan.iters_per_tile == 86
+        assert _rel(oracle, sk.streamk_fp16(_t(A), _t(B), plan=plan), ref) <= 1e-3
+    sk.workspace_status()
+
+
 def test_reduce_fixup_is_bitwise_reproducible(sk):
     """The ordered reduce must give identical bits run to run (10 runs, two shapes); the schedule
     splits every tile."""
