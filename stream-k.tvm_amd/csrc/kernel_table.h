@@ -23,7 +23,8 @@ struct KernelInfo {
   int layout;   // sk_layout
   int variant;  // tile kernels -- 0: registers -> padded LDS rows; 1: direct global -> LDS loads,
                 // swizzled rows; 2: as 1 with four waves per CTA (one per SIMD, accumulators in AGPRs);
-                // 3: as 1 with BK = 32 and four LDS stages (loads three iterations ahead)
+                // 3: as 1 with BK = 32 and four LDS stages (loads three iterations ahead);
+                // 4: as 1 with 16x16x32 MFMAs
                 // small-M kernels -- 0: up to 16*MB rows of A; 1: M == 1; 2: M == 1, matrix-vector on 4x4x4 MFMA
   int bm, bn, bk;  // CTA tile; bk is the K extent of one CTA iteration
   int threads;
@@ -66,6 +67,13 @@ struct KernelInfo {
   X(27, 64, 64, 2, 2)                   \
   X(28, 128, 64, 2, 2)                  \
   X(29, 64, 128, 2, 2)
+
+// direct-to-LDS loads, BK = 64, arithmetic on v_mfma_f32_16x16x32_f16 (variant 4), NT layout:  X(id, BM, BN, WM, WN)
+#define SK_TILE_F16_NT_DMA16_KERNELS(X) \
+  X(30, 256, 256, 2, 4)                 \
+  X(31, 128, 128, 2, 2)                 \
+  X(32, 128, 256, 2, 4)                 \
+  X(33, 256, 128, 4, 2)
 
 // the same for the NN layout (B is [K,N]), fragments through transposing LDS reads:  X(id, BM, BN, WM, WN)
 #define SK_TILE_F16_NN_DMA_KERNELS(X) \

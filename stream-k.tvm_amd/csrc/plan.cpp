@@ -43,7 +43,7 @@ static int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // eight-wave direct-to-LDS tile kernels; the most specialised small-M kernel that accepts the shape
 static int variant_rank(const KernelInfo &k) {
   if (k.family == FAMILY_SKINNY) return k.variant;
-  return k.variant == 1 ? 2 : (k.variant == 2 ? 1 : 0);
+  return k.variant == 4 ? 3 : (k.variant == 1 ? 2 : (k.variant == 2 ? 1 : 0));
 }
 static bool accepts_shape(const KernelInfo &k, int64_t M, int64_t K) {
   return (k.max_m == 0 || M <= k.max_m) && (k.max_ipt == 0 || (K + k.bk - 1) / k.bk <= k.max_ipt);
@@ -101,7 +101,8 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
   // or two waves per SIMD, where the four-stage (BK = 32) pipeline hides the load latency better;
   // it exists for the NT layout only.
   const int64_t tiles256 = cdiv(M, 256) * cdiv(N, 256), tiles128 = cdiv(M, 128) * cdiv(N, 128);
-  int pref[3][4] = {{256, 256, 64, 1}, {128, 128, 32, 3}, {64, 64, 32, 3}};  // bm, bn, bk, variant
+  // (256x256: the 16x16x32-MFMA form, NT only; the NN layout falls through to its variant 1)
+  int pref[3][4] = {{256, 256, 64, 4}, {128, 128, 32, 3}, {64, 64, 32, 3}};  // bm, bn, bk, variant
   const int first = tiles256 * 4 >= (int64_t)num_cus * 3 ? 0 : (tiles128 * 2 >= num_cus ? 1 : 2);
   const int order[3][3] = {{0, 1, 2}, {1, 2, 0}, {2, 1, 0}};  // smaller tiles first, then larger ones
   for (int oi = 0; oi < 3 && !best; ++oi) {

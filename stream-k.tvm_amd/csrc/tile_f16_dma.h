@@ -46,12 +46,20 @@ struct LdsArray {
 // requested when iteration it has been read, three iterations (about 1.5 iterations of the
 // two-stage pipeline) before they are needed: a load that misses the L2 takes longer than one
 // iteration of MFMAs, which the two-stage pipeline exposes as a stall at every barrier.
-template <int BM_, int BN_, int WM_, int WN_, bool B_KN_ = false, int BK_ = 64>
+//
+// MFMA16_: the arithmetic uses v_mfma_f32_16x16x32_f16 instead of v_mfma_f32_32x32x16_f16.  Both
+// run at the same FLOP per cycle, but the 16x16x32 form reads and writes half as many accumulator
+// registers per FLOP, and on random operands the part sustains a ~12 % higher clock with it under
+// its power limit.  Each 32x32 block of the accumulator is then four 16x16 blocks (block (si, sj)
+// in elements 4*(2*si+sj) .. +3): lane l holds C[16*si + l%16][16*sj + 4*(l/16) + e].  A K-step
+// covers 32 K-values: lane group g = l/16 takes 16-byte chunk 4*kk + g of its row.
+template <int BM_, int BN_, int WM_, int WN_, bool B_KN_ = false, int BK_ = 64, bool MFMA16_ = false>
 struct TileF16NTDma {
-  static constexpr bool B_KN = B_KN_;
+  static constexpr bool B_KN = B_KN_, MFMA16 = MFMA16_;
+  static_assert(!MFMA16_ || (BK_ == 64 && !B_KN_), "the 16x16x32 form exists for NT, BK = 64");
   static constexpr int ROW_BYTES = BK_ * 2;                    // bytes of one LDS row of A (and of B, NT)
   static constexpr int ROWS_PER_DMA = 1024 / ROW_BYTES;        // rows one wave-wide load fills
-  static constexpr int NSTAGE = 128 / BK_, KSTEPS = BK_ / 16;
+  static constexpr int NSTAGE = 128 / BK_, KSTEPS = BK_ / (MFMA16_ ? 32 : 16);
   static_assert(BK_ == 64 || (BK_ == 32 && !B_KN_), "BK is 64, or 32 for the NT layout");
   static constexpr int B_ROW_BYTES = B_KN_ ? BN_ * 2 : ROW_BYTES;  // bytes of one LDS row of the B stage
   static constexpr int B_ROWS_PER_DMA = 1024 / B_ROW_BYTES;    // rows one wave-wide load fills
@@ -61,6 +69,8 @@ struct TileF16NTDma {
   static constexpr int NW = WM * WN, NT = NW * 64;
   static constexpr int TM = BM / (WM * 32), TN = BN / (WN * 32);
   static constexpr int WTM = TM * 32, WTN = TN * 32;
+  static constexpr int FROWS = MFMA16_ ? 16 : 32;              // rows of one operand fragment
+  static constexpr int FM = WTM / FROWS, FN = WTN / FROWS;     // fragments per K-step
   static constexpr int A_BYTES = BM * ROW_BYTES, B_BYTES = BN * ROW_BYTES, STAGE_BYTES = A_BYTES + B_BYTES;
   static constexpr int A_DMA = A_BYTES / 1024 / NW, B_DMA = B_BYTES / 1024 / NW, DMA_PER_WAVE = A_DMA + B_DMA;
   static constexpr int LDC = WTN + 8;
@@ -105,6 +115,16 @@ struct TileF16NTDma {
       asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
     else
       asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
+  }
+
+  // scheduling hint: one LDS read, then PER MFMAs, READS times
+  template <int READS, int PER>
+  static __device__ __forceinline__ void interleave16() {
+#pragma unroll
+    for (int g = 0; g < READS; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);
+    }
   }
 
   static __device__ __forceinline__ void mac(const Args &a, Acc &acc, int pm, int pn, int k0, int n,
@@ -171,12 +191,14 @@ struct TileF16NTDma {
     // fragment addressing: lane (r = lane%32, g = lane/32) reads row r of a 32-row block, logical
     // chunk 2*kk + g, stored at chunk position (2*kk + g) ^ ((r >> 1) & 7)
     // (BK = 32: swizzle (r >> 2) & 3)
+    // (16x16x32: row lane%16, logical chunk 4*kk + lane/16, same swizzle)
     int rd_a[KSTEPS], rd_b[KSTEPS];
 #pragma unroll
     for (int kk = 0; kk < KSTEPS; ++kk) {
-      const int pos = ((2 * kk + (lane >> 5)) ^ (BK == 64 ? (lane >> 1) & 7 : (lane >> 2) & 3)) * 16;
-      rd_a[kk] = (wm * WTM + (lane & 31)) * ROW_BYTES + pos;
-      rd_b[kk] = A_BYTES + (wn * WTN + (lane & 31)) * ROW_BYTES + pos;
+      const int chunk = MFMA16 ? 4 * kk + (lane >> 4) : 2 * kk + (lane >> 5);
+      const int pos = (chunk ^ (BK == 64 ? (lane >> 1) & 7 : (lane >> 2) & 3)) * 16;
+      rd_a[kk] = (wm * WTM + (lane & (FROWS - 1))) * ROW_BYTES + pos;
+      rd_b[kk] = A_BYTES + (wn * WTN + (lane & (FROWS - 1))) * ROW_BYTES + pos;
     }
     // NN: per 32-column block j, the byte address of this lane's 8-byte piece in K-row
     // 8*(lane/32) + (lane%16)/4 of the stage; K-steps and the second half add row multiples
@@ -190,14 +212,38 @@ struct TileF16NTDma {
         rd_bt[j] = A_BYTES + k_lane * B_ROW_BYTES + chunk * 16 + (col & 7) * 2;
       }
     }
-    half8v fa[2][TM], fb[2][TN];
+    // 16x16x32: A fragments are double-buffered per half of the wave tile's rows (two half-steps per
+    // K-step), which keeps accumulators + fragments + addresses within 256 registers
+    constexpr int FA = MFMA16 ? FM / 2 : FM;
+    half8v fa[2][FA], fb[2][FN];
+    auto read_a16 = [&](const char *st, int buf, int kk, int mh) {
+#pragma unroll
+      for (int i = 0; i < FA; ++i)
+        fa[buf][i] = *reinterpret_cast<const half8v *>(st + rd_a[kk] + (mh * FA + i) * FROWS * ROW_BYTES);
+    };
+    auto read_b16 = [&](const char *st, int buf, int kk) {
+#pragma unroll
+      for (int j = 0; j < FN; ++j) fb[buf][j] = *reinterpret_cast<const half8v *>(st + rd_b[kk] + j * FROWS * ROW_BYTES);
+    };
+    auto mfma_one16 = [&](int abuf, int bbuf, int mh, int idx) {
+      const int i = idx / FN, j = idx % FN, ii = mh * FA + i;
+      floatx16 &c = acc.c[ii / 2][j / 2];
+      const int q = 4 * (2 * (ii & 1) + (j & 1));
+      floatx4 t = floatx4{c[q], c[q + 1], c[q + 2], c[q + 3]};
+      t = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[bbuf][j], fa[abuf][i], t, 0, 0, 0);
+      c[q] = t[0], c[q + 1] = t[1], c[q + 2] = t[2], c[q + 3] = t[3];
+    };
+    auto mfma_half16 = [&](int abuf, int bbuf, int mh) {
+#pragma unroll
+      for (int idx = 0; idx < FA * FN; ++idx) mfma_one16(abuf, bbuf, mh, idx);
+    };
     auto read_frags = [&](const char *st, int buf, int kk) {
 #pragma unroll
-      for (int i = 0; i < TM; ++i) fa[buf][i] = *reinterpret_cast<const half8v *>(st + rd_a[kk] + i * 32 * ROW_BYTES);
+      for (int i = 0; i < FM; ++i) fa[buf][i] = *reinterpret_cast<const half8v *>(st + rd_a[kk] + i * FROWS * ROW_BYTES);
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
+      for (int j = 0; j < FN; ++j) {
         if (!B_KN) {
-          fb[buf][j] = *reinterpret_cast<const half8v *>(st + rd_b[kk] + j * 32 * ROW_BYTES);
+          fb[buf][j] = *reinterpret_cast<const half8v *>(st + rd_b[kk] + j * FROWS * ROW_BYTES);
         } else {
           typedef short short4v __attribute__((ext_vector_type(4)));
           typedef __attribute__((address_space(3))) short4v *lds_s4;
@@ -252,6 +298,71 @@ struct TileF16NTDma {
       if (it + 2 < n) iteration4(s2, s3, it + 2);
       // the (empty) loads of the iterations past the segment still write LDS: drain them before
       // the stages are handed to the epilogue / the next tile
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    } else if constexpr (MFMA16) {
+      // one K-iteration on stage `cur`: two K-steps of 32, each in two halves of the wave tile's
+      // rows.  Entering, fa[0] / fb[0] hold the fragments of (K-step 0, first half).
+      auto iteration16 = [&](char *cur, char *nxt, int it) {
+        // (hints: the reads are spread evenly over the MFMAs of a half-step.  Issuing them all at
+        // its start is faster on all-zero operands and slower on random ones, where the power
+        // limit sets the clock.)
+        read_a16(cur, 1, 0, 1);
+        read_b16(cur, 1, 1);
+        mfma_half16(0, 0, 0);
+        interleave16<FA + FN, FA * FN / (FA + FN)>();
+        read_a16(cur, 0, 1, 0);
+        mfma_half16(1, 0, 1);
+        interleave16<FA, FN>();
+        read_a16(cur, 1, 1, 1);
+        mfma_half16(0, 1, 0);
+        interleave16<FA, FN>();
+        // every read of `cur` has been issued and has completed behind the MFMAs above
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        wait_dma_then_barrier<0>();
+        // last half-step in DMA_PER_WAVE slices: each issues one load of iteration it+2 into `cur`,
+        // its share of the first fragment reads of `nxt` and its share of the MFMAs, so the matrix
+        // pipe does not run dry behind a block of load instructions.  No branches: past the segment
+        // the loads get an out-of-range offset (they fetch nothing and zero a stage nobody reads;
+        // drained below) and the reads fetch fragments nobody uses.
+        const int kt2 = k0 + it + 2;
+        const bool oob2 = it + 2 >= n || (kt2 == tail_kt && kt2 * BK + my_chunk * 8 >= a.K);
+        const uint32_t va2 = oob2 ? OOB_OFFSET : voff_a, vb2 = oob2 ? OOB_OFFSET : voff_b;
+        constexpr int CH = DMA_PER_WAVE, NRD = FA + FN, NMF = FA * FN;
+#pragma unroll
+        for (int x = 0; x < CH; ++x) {
+#pragma unroll
+          for (int r = 0; r < NRD; ++r)
+            if (r * CH / NRD == x) {
+              if (r < FA)
+                fa[0][r] = *reinterpret_cast<const half8v *>(nxt + rd_a[0] + r * FROWS * ROW_BYTES);
+              else
+                fb[0][r - FA] = *reinterpret_cast<const half8v *>(nxt + rd_b[0] + (r - FA) * FROWS * ROW_BYTES);
+            }
+          if (x < A_DMA) {
+            const int g = wave + x * NW;
+            dma_load_16(rsrc_a, lds_address(cur) + g * 1024, va2, (uint32_t)kt2 * (BK * 2) + g * grp_a);
+          } else {
+            const int g = wave + (x - A_DMA) * NW;
+            dma_load_16(rsrc_b, lds_address(cur) + A_BYTES + g * 1024, vb2, (uint32_t)kt2 * kstep_b + g * grp_b);
+          }
+#pragma unroll
+          for (int m = 0; m < NMF; ++m)
+            if (m * CH / NMF == x) mfma_one16(1, 1, 1, m);
+        }
+      };
+      char *s0 = stage(0), *s1 = stage(1);
+      issue_dma(s0, k0);
+      wait_dma_then_barrier<0>();
+      if (n > 1) issue_dma(s1, k0 + 1);
+      read_a16(s0, 0, 0, 0);
+      read_b16(s0, 0, 0);
+      int it = 0;
+      for (; it + 1 < n; it += 2) {
+        iteration16(s0, s1, it);
+        iteration16(s1, s0, it + 1);
+      }
+      if (it < n) iteration16(s0, s1, it);
+      // the empty loads of the last two iterations still write LDS
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     } else {
       // one K-iteration on stage `cur`; `more1`/`more2`: iterations it+1 / it+2 exist
@@ -311,8 +422,12 @@ struct TileF16NTDma {
             half4v h;
 #pragma unroll
             for (int e = 0; e < 4; ++e) h[e] = (half_t)acc.c[p * BLK + ib][j][q * 4 + e];
-            *reinterpret_cast<half4v *>(patch + (ib * 32 + (lane & 31)) * LDC + j * 32 + q * 8 +
-                                        (lane >> 5) * 4) = h;
+            if (MFMA16)  // q = 2*si + sj: rows 16*si + lane%16, columns 16*sj + 4*(lane/16) + e
+              *reinterpret_cast<half4v *>(patch + (ib * 32 + (q >> 1) * 16 + (lane & 15)) * LDC + j * 32 +
+                                          (q & 1) * 16 + (lane >> 4) * 4) = h;
+            else
+              *reinterpret_cast<half4v *>(patch + (ib * 32 + (lane & 31)) * LDC + j * 32 + q * 8 +
+                                          (lane >> 5) * 4) = h;
           }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
