@@ -24,7 +24,7 @@ struct KernelInfo {
   int variant;  // tile kernels -- 0: registers -> padded LDS rows; 1: direct global -> LDS loads,
                 // swizzled rows; 2: as 1 with four waves per CTA (one per SIMD, accumulators in AGPRs);
                 // 3: as 1 with BK = 32 and four LDS stages (loads three iterations ahead);
-                // 4: as 1 with 16x16x32 MFMAs
+                // 4: as 1 with 16x16x32 MFMAs; 5: as 3 with 16x16x32 MFMAs
                 // small-M kernels -- 0: up to 16*MB rows of A; 1: M == 1; 2: M == 1, matrix-vector on 4x4x4 MFMA
   int bm, bn, bk;  // CTA tile; bk is the K extent of one CTA iteration
   int threads;
@@ -74,6 +74,16 @@ struct KernelInfo {
   X(31, 128, 128, 2, 2)                 \
   X(32, 128, 256, 2, 4)                 \
   X(33, 256, 128, 4, 2)
+
+// BK = 32, four stages, 16x16x32 MFMAs (variant 5), NT layout:  X(id, BM, BN, WM, WN)
+#define SK_TILE_F16_NT_DMA32_16_KERNELS(X) \
+  X(35, 256, 256, 2, 4)                    \
+  X(36, 128, 128, 2, 2)                    \
+  X(37, 128, 256, 2, 4)                    \
+  X(38, 256, 128, 4, 2)                    \
+  X(39, 64, 64, 2, 2)                      \
+  X(40, 128, 64, 2, 2)                     \
+  X(41, 64, 128, 2, 2)
 
 // the same for the NN layout (B is [K,N]), fragments through transposing LDS reads:  X(id, BM, BN, WM, WN)
 #define SK_TILE_F16_NN_DMA_KERNELS(X) \

@@ -56,7 +56,7 @@ struct LdsArray {
 template <int BM_, int BN_, int WM_, int WN_, bool B_KN_ = false, int BK_ = 64, bool MFMA16_ = false>
 struct TileF16NTDma {
   static constexpr bool B_KN = B_KN_, MFMA16 = MFMA16_;
-  static_assert(!MFMA16_ || (BK_ == 64 && !B_KN_), "the 16x16x32 form exists for NT, BK = 64");
+  static_assert(!MFMA16_ || !B_KN_, "the 16x16x32 form exists for the NT layout");
   static constexpr int ROW_BYTES = BK_ * 2;                    // bytes of one LDS row of A (and of B, NT)
   static constexpr int ROWS_PER_DMA = 1024 / ROW_BYTES;        // rows one wave-wide load fills
   static constexpr int NSTAGE = 128 / BK_, KSTEPS = BK_ / (MFMA16_ ? 32 : 16);
@@ -261,7 +261,69 @@ struct TileF16NTDma {
         for (int j = 0; j < TN; ++j)
           acc.c[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[buf][j], fa[buf][i], acc.c[i][j], 0, 0, 0);
     };
-    if constexpr (NSTAGE == 4) {
+    // 16x16x32, the half-step behind the barrier, in DMA_PER_WAVE slices: each issues one load of
+    // K-iteration kt_next into `cur`, its share of the first fragment reads of `nxt` (A into
+    // fa[0], B into fb[bnext]) and its share of the MFMAs of the second half of the rows (fa[1],
+    // fb[bcur]), so the matrix pipe does not run dry behind a block of load instructions.  No
+    // branches: past the segment the loads get an out-of-range offset (they fetch nothing and zero
+    // a stage nobody reads; drained after the loop) and the reads fetch fragments nobody uses.
+    auto tail16 = [&](char *cur, const char *nxt, int kt_next, bool dead, int bcur, int bnext) {
+      const bool oob = dead || (kt_next == tail_kt && kt_next * BK + my_chunk * 8 >= a.K);
+      const uint32_t va = oob ? OOB_OFFSET : voff_a, vb = oob ? OOB_OFFSET : voff_b;
+      constexpr int CH = DMA_PER_WAVE, NRD = FA + FN, NMF = FA * FN;
+#pragma unroll
+      for (int x = 0; x < CH; ++x) {
+#pragma unroll
+        for (int r = 0; r < NRD; ++r)
+          if (r * CH / NRD == x) {
+            if (r < FA)
+              fa[0][r] = *reinterpret_cast<const half8v *>(nxt + rd_a[0] + r * FROWS * ROW_BYTES);
+            else
+              fb[bnext][r - FA] = *reinterpret_cast<const half8v *>(nxt + rd_b[0] + (r - FA) * FROWS * ROW_BYTES);
+          }
+        if (x < A_DMA) {
+          const int g = wave + x * NW;
+          dma_load_16(rsrc_a, lds_address(cur) + g * 1024, va, (uint32_t)kt_next * (BK * 2) + g * grp_a);
+        } else {
+          const int g = wave + (x - A_DMA) * NW;
+          dma_load_16(rsrc_b, lds_address(cur) + A_BYTES + g * 1024, vb, (uint32_t)kt_next * kstep_b + g * grp_b);
+        }
+#pragma unroll
+        for (int m = 0; m < NMF; ++m)
+          if (m * CH / NMF == x) mfma_one16(1, bcur, 1, m);
+      }
+    };
+    if constexpr (NSTAGE == 4 && MFMA16) {
+      // BK = 32 is one K-step: two half-steps per iteration.  Entering, fa[0] holds the first half
+      // of the A rows and fb[par] the B fragments of stage `cur` (par = iteration parity).
+      auto iteration4 = [&](char *cur, char *nxt, int it, int par) {
+        read_a16(cur, 1, 0, 1);
+        mfma_half16(0, par, 0);
+        interleave16<FA, FN>();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        wait_dma_then_barrier<2 * DMA_PER_WAVE>();
+        tail16(cur, nxt, k0 + it + 4, it + 4 >= n, par, par ^ 1);
+      };
+      char *s0 = stage(0), *s1 = stage(1), *s2 = stage(2), *s3 = stage(3);
+      issue_dma(s0, k0);
+      issue_dma(s1, k0 + 1);
+      issue_dma(s2, k0 + 2);
+      wait_dma_then_barrier<2 * DMA_PER_WAVE>();
+      issue_dma(s3, k0 + 3);
+      read_a16(s0, 0, 0, 0);
+      read_b16(s0, 0, 0);
+      int it = 0;
+      for (; it + 3 < n; it += 4) {
+        iteration4(s0, s1, it, 0);
+        iteration4(s1, s2, it + 1, 1);
+        iteration4(s2, s3, it + 2, 0);
+        iteration4(s3, s0, it + 3, 1);
+      }
+      if (it < n) iteration4(s0, s1, it, 0);
+      if (it + 1 < n) iteration4(s1, s2, it + 1, 1);
+      if (it + 2 < n) iteration4(s2, s3, it + 2, 0);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    } else if constexpr (NSTAGE == 4) {
       // one K-iteration (two K-steps) on stage `cur`: the barrier in the middle retires the reads
       // of `cur` (it is refilled for iteration it+4 right away) and publishes stage `nxt`, whose
       // loads were issued three iterations ago -- two younger groups may still be in flight
@@ -319,36 +381,7 @@ struct TileF16NTDma {
         // every read of `cur` has been issued and has completed behind the MFMAs above
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         wait_dma_then_barrier<0>();
-        // last half-step in DMA_PER_WAVE slices: each issues one load of iteration it+2 into `cur`,
-        // its share of the first fragment reads of `nxt` and its share of the MFMAs, so the matrix
-        // pipe does not run dry behind a block of load instructions.  No branches: past the segment
-        // the loads get an out-of-range offset (they fetch nothing and zero a stage nobody reads;
-        // drained below) and the reads fetch fragments nobody uses.
-        const int kt2 = k0 + it + 2;
-        const bool oob2 = it + 2 >= n || (kt2 == tail_kt && kt2 * BK + my_chunk * 8 >= a.K);
-        const uint32_t va2 = oob2 ? OOB_OFFSET : voff_a, vb2 = oob2 ? OOB_OFFSET : voff_b;
-        constexpr int CH = DMA_PER_WAVE, NRD = FA + FN, NMF = FA * FN;
-#pragma unroll
-        for (int x = 0; x < CH; ++x) {
-#pragma unroll
-          for (int r = 0; r < NRD; ++r)
-            if (r * CH / NRD == x) {
-              if (r < FA)
-                fa[0][r] = *reinterpret_cast<const half8v *>(nxt + rd_a[0] + r * FROWS * ROW_BYTES);
-              else
-                fb[0][r - FA] = *reinterpret_cast<const half8v *>(nxt + rd_b[0] + (r - FA) * FROWS * ROW_BYTES);
-            }
-          if (x < A_DMA) {
-            const int g = wave + x * NW;
-            dma_load_16(rsrc_a, lds_address(cur) + g * 1024, va2, (uint32_t)kt2 * (BK * 2) + g * grp_a);
-          } else {
-            const int g = wave + (x - A_DMA) * NW;
-            dma_load_16(rsrc_b, lds_address(cur) + A_BYTES + g * 1024, vb2, (uint32_t)kt2 * kstep_b + g * grp_b);
-          }
-#pragma unroll
-          for (int m = 0; m < NMF; ++m)
-            if (m * CH / NMF == x) mfma_one16(1, 1, 1, m);
-        }
+        tail16(cur, nxt, k0 + it + 2, it + 2 >= n, 1, 0);
       };
       char *s0 = stage(0), *s1 = stage(1);
       issue_dma(s0, k0);

@@ -70,8 +70,9 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
         for (bm, bn, bk) in _TILES_F16:
             # (variant, bk): direct-to-LDS two-stage, register-staged, direct-to-LDS four-stage, 16x16x32 form
             variants = ((2, bk), (1, bk), (4, 32)) if bm * bn > 64 * 128 else ((2, bk), (4, 32))
+            variants += ((6, 32),)  # four-stage with 16x16x32 MFMAs
             if bm >= 128 and bn >= 128:
-                variants += ((5, bk),)  # 16x16x32 MFMAs
+                variants += ((5, bk),)  # two-stage with 16x16x32 MFMAs
             if (bm, bn) == (64, 64):
                 variants += ((1, bk),)
             for (variant, vbk), raster in itertools.product(variants, (0, 8)):

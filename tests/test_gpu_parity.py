@@ -43,7 +43,7 @@ def _rel(oracle, C, ref):
 
 
 # variant 1: registers -> padded LDS rows; 2: direct-to-LDS, 8 (4) waves; 3: direct-to-LDS 256x256 on 4 waves;
-# 4: direct-to-LDS with BK = 32 and four stages; 5: direct-to-LDS, 16x16x32 MFMAs
+# 4: direct-to-LDS with BK = 32 and four stages; 5: direct-to-LDS, 16x16x32 MFMAs; 6: as 4 with 16x16x32 MFMAs
 TILE_CONFIGS = [
     dict(bm=128, bn=128, bk=64, variant=1), dict(bm=256, bn=256, bk=64, variant=1),
     dict(bm=128, bn=256, bk=64, variant=1), dict(bm=256, bn=128, bk=64, variant=1),
@@ -57,6 +57,9 @@ TILE_CONFIGS = [
     dict(bm=64, bn=64, bk=32, variant=4), dict(bm=128, bn=64, bk=32, variant=4), dict(bm=64, bn=128, bk=32, variant=4),
     dict(bm=128, bn=128, bk=64, variant=5), dict(bm=256, bn=256, bk=64, variant=5),
     dict(bm=128, bn=256, bk=64, variant=5), dict(bm=256, bn=128, bk=64, variant=5),
+    dict(bm=128, bn=128, bk=32, variant=6), dict(bm=256, bn=256, bk=32, variant=6),
+    dict(bm=128, bn=256, bk=32, variant=6), dict(bm=256, bn=128, bk=32, variant=6),
+    dict(bm=64, bn=64, bk=32, variant=6), dict(bm=128, bn=64, bk=32, variant=6), dict(bm=64, bn=128, bk=32, variant=6),
 ]
 SKINNY_CONFIGS = [
     dict(bm=16, bn=64, bk=128), dict(bm=32, bn=64, bk=128), dict(bm=64, bn=64, bk=128),
