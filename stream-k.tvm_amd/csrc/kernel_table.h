@@ -140,6 +140,13 @@ struct KernelInfo {
   X(166, 1, 1, 4, 4, 32768)    \
   X(167, 2, 1, 4, 2, 32768)
 
+// NN layout, 16x16x32 MFMAs (variant 4):  X(id, BM, BN, WM, WN)
+#define SK_TILE_F16_NN_DMA16_KERNELS(X) \
+  X(42, 256, 256, 2, 4)                 \
+  X(43, 128, 128, 2, 2)                 \
+  X(44, 128, 256, 2, 4)                 \
+  X(45, 256, 128, 4, 2)
+
 const KernelInfo *kernel_table(int *count);
 const KernelInfo *kernel_by_id(int id);
 

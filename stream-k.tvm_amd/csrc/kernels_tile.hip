@@ -26,6 +26,7 @@ static int launch_dma(const GemmArgs &a, const DevPlan &p, const Workspace &ws, 
 #define SK_POLICY_DMA32(id, BM, BN, WM, WN) TileF16NTDma<BM, BN, WM, WN, false, 32>
 #define SK_POLICY_DMA16(id, BM, BN, WM, WN) TileF16NTDma<BM, BN, WM, WN, false, 64, true>
 #define SK_POLICY_DMA32_16(id, BM, BN, WM, WN) TileF16NTDma<BM, BN, WM, WN, false, 32, true>
+#define SK_POLICY_NN16(id, BM, BN, WM, WN) TileF16NTDma<BM, BN, WM, WN, true, 64, true>
 
 int tile_kernel_infos(KernelInfo *out, int max) {
   int n = 0;
@@ -77,6 +78,14 @@ int tile_kernel_infos(KernelInfo *out, int max) {
   }
   SK_TILE_F16_NT_DMA32_16_KERNELS(X)
 #undef X
+#define X(id, BM, BN, WM, WN)                                                                       \
+  if (n < max) {                                                                                    \
+    typedef SK_POLICY_NN16(id, BM, BN, WM, WN) P;                                                   \
+    out[n++] = KernelInfo{id, FAMILY_TILE, 0, 1, 4, BM, BN, 64, P::NT, P::LDS_TOTAL, P::CTAS_PER_CU, \
+                          P::TILE_ELEMS, 0, 0, 8, "tile_f16_nn_dma16_" #BM "x" #BN "x64"};          \
+  }
+  SK_TILE_F16_NN_DMA16_KERNELS(X)
+#undef X
   return n;
 }
 
@@ -124,6 +133,13 @@ int launch_tile_f16(int id, const GemmArgs &a, const DevPlan &p, const Workspace
     return launch_dma<P>(a, p, ws, s);                                                       \
   }
     SK_TILE_F16_NT_DMA32_16_KERNELS(X)
+#undef X
+#define X(id_, BM, BN, WM, WN)                                                           \
+  case id_: {                                                                            \
+    typedef SK_POLICY_NN16(id_, BM, BN, WM, WN) P;                                       \
+    return launch_dma<P>(a, p, ws, s);                                                       \
+  }
+    SK_TILE_F16_NN_DMA16_KERNELS(X)
 #undef X
   }
   return (int)hipErrorInvalidValue;
@@ -185,6 +201,15 @@ int occupancy_tile(int id) {
     return occ;                                                                                     \
   }
     SK_TILE_F16_NT_DMA32_16_KERNELS(X)
+#undef X
+#define X(id_, BM, BN, WM, WN)                                                                      \
+  case id_: {                                                                                       \
+    typedef SK_POLICY_NN16(id_, BM, BN, WM, WN) P;                                                  \
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_tile_kernel<P>, P::NT, 0) != hipSuccess) \
+      return -1;                                                                                    \
+    return occ;                                                                                     \
+  }
+    SK_TILE_F16_NN_DMA16_KERNELS(X)
 #undef X
   }
   return -1;

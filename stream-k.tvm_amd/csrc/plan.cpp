@@ -101,7 +101,7 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
   // or two waves per SIMD, where the four-stage (BK = 32) pipeline hides the load latency better;
   // it exists for the NT layout only.
   const int64_t tiles256 = cdiv(M, 256) * cdiv(N, 256), tiles128 = cdiv(M, 128) * cdiv(N, 128);
-  // (256x256: the 16x16x32-MFMA form, NT only; the NN layout falls through to its variant 1)
+  // (256x256: the 16x16x32-MFMA form)
   int pref[3][4] = {{256, 256, 64, 4}, {128, 128, 32, 3}, {64, 64, 32, 3}};  // bm, bn, bk, variant
   const int first = tiles256 * 4 >= (int64_t)num_cus * 3 ? 0 : (tiles128 * 2 >= num_cus ? 1 : 2);
   const int order[3][3] = {{0, 1, 2}, {1, 2, 0}, {2, 1, 0}};  // smaller tiles first, then larger ones

@@ -56,7 +56,6 @@ struct LdsArray {
 template <int BM_, int BN_, int WM_, int WN_, bool B_KN_ = false, int BK_ = 64, bool MFMA16_ = false>
 struct TileF16NTDma {
   static constexpr bool B_KN = B_KN_, MFMA16 = MFMA16_;
-  static_assert(!MFMA16_ || !B_KN_, "the 16x16x32 form exists for the NT layout");
   static constexpr int ROW_BYTES = BK_ * 2;                    // bytes of one LDS row of A (and of B, NT)
   static constexpr int ROWS_PER_DMA = 1024 / ROW_BYTES;        // rows one wave-wide load fills
   static constexpr int NSTAGE = 128 / BK_, KSTEPS = BK_ / (MFMA16_ ? 32 : 16);
@@ -160,9 +159,12 @@ struct TileF16NTDma {
       kstep_b = BK * 2;
     } else {
       rsrc_b = make_rsrc_words(a.B + (int64_t)pn * BN, (uint32_t)(((int64_t)(a.K - 1) * a.ldb + rows_b) * 2));
+      // this lane's K-row within the stage is B_ROWS_PER_DMA * (wave + x * NW) + row_in; its bits
+      // 0..3 do not depend on x
+      static_assert((B_ROWS_PER_DMA * NW) % 16 == 0, "swizzle bits of a lane's K-row must not depend on the load");
       const int row_in = (lane * 16) / B_ROW_BYTES, pos = ((lane * 16) % B_ROW_BYTES) / 16;
-      const int k_low = (B_ROWS_PER_DMA == 2 ? 2 * (wave & 1) + row_in : row_in) & 3;  // (K-row & 3)
-      const int chunk = pos ^ (4 * k_low);
+      const int k_bits = B_ROWS_PER_DMA * wave + row_in;
+      const int chunk = pos ^ (4 * (k_bits & 3)) ^ (MFMA16 ? 2 * ((k_bits >> 3) & 1) : 0);
       voff_b = (chunk * 8 < rows_b) ? (uint32_t)(row_in * a.ldb + chunk * 8) * 2 : OOB_OFFSET;
       grp_b = (uint32_t)(B_ROWS_PER_DMA * a.ldb * 2);
       kstep_b = (uint32_t)(BK * a.ldb * 2);
@@ -202,13 +204,17 @@ struct TileF16NTDma {
     }
     // NN: per 32-column block j, the byte address of this lane's 8-byte piece in K-row
     // 8*(lane/32) + (lane%16)/4 of the stage; K-steps and the second half add row multiples
-    int rd_bt[TN];
+    // (16x16x32: lane group g = lane/16 reads K-rows 8g..8g+7 of a 16-column block.  Groups 0 and
+    // 1 are served in the same cycle and read the same columns of K-rows 8 apart, so the swizzle
+    // also flips chunk bit 1 with bit 3 of the K-row.)
+    int rd_bt[FN];
     if (B_KN) {
-      const int k_lane = 8 * (lane >> 5) + ((lane & 15) >> 2);
+      const int k_lane = MFMA16 ? 8 * (lane >> 4) + ((lane & 15) >> 2) : 8 * (lane >> 5) + ((lane & 15) >> 2);
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int col = wn * WTN + j * 32 + 16 * ((lane & 31) >> 4) + 4 * (lane & 3);
-        const int chunk = (col >> 3) ^ (4 * (k_lane & 3));
+      for (int j = 0; j < FN; ++j) {
+        const int col = MFMA16 ? wn * WTN + j * 16 + 4 * (lane & 3)
+                               : wn * WTN + j * 32 + 16 * ((lane & 31) >> 4) + 4 * (lane & 3);
+        const int chunk = (col >> 3) ^ (4 * (k_lane & 3)) ^ (MFMA16 ? 2 * ((k_lane >> 3) & 1) : 0);
         rd_bt[j] = A_BYTES + k_lane * B_ROW_BYTES + chunk * 16 + (col & 7) * 2;
       }
     }
@@ -221,9 +227,21 @@ struct TileF16NTDma {
       for (int i = 0; i < FA; ++i)
         fa[buf][i] = *reinterpret_cast<const half8v *>(st + rd_a[kk] + (mh * FA + i) * FROWS * ROW_BYTES);
     };
+    auto read_b16_one = [&](const char *st, int buf, int kk, int j) {
+      if (!B_KN) {
+        fb[buf][j] = *reinterpret_cast<const half8v *>(st + rd_b[kk] + j * FROWS * ROW_BYTES);
+      } else {
+        typedef short short4v __attribute__((ext_vector_type(4)));
+        typedef __attribute__((address_space(3))) short4v *lds_s4;
+        union { short4v s[2]; half8v h; } u;
+        u.s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4)(st + rd_bt[j] + (kk * 32) * B_ROW_BYTES));
+        u.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4)(st + rd_bt[j] + (kk * 32 + 4) * B_ROW_BYTES));
+        fb[buf][j] = u.h;
+      }
+    };
     auto read_b16 = [&](const char *st, int buf, int kk) {
 #pragma unroll
-      for (int j = 0; j < FN; ++j) fb[buf][j] = *reinterpret_cast<const half8v *>(st + rd_b[kk] + j * FROWS * ROW_BYTES);
+      for (int j = 0; j < FN; ++j) read_b16_one(st, buf, kk, j);
     };
     auto mfma_one16 = [&](int abuf, int bbuf, int mh, int idx) {
       const int i = idx / FN, j = idx % FN, ii = mh * FA + i;
@@ -269,7 +287,8 @@ struct TileF16NTDma {
     // a stage nobody reads; drained after the loop) and the reads fetch fragments nobody uses.
     auto tail16 = [&](char *cur, const char *nxt, int kt_next, bool dead, int bcur, int bnext) {
       const bool oob = dead || (kt_next == tail_kt && kt_next * BK + my_chunk * 8 >= a.K);
-      const uint32_t va = oob ? OOB_OFFSET : voff_a, vb = oob ? OOB_OFFSET : voff_b;
+      // (NN: the K tail of B is cut off by its descriptor, not per lane)
+      const uint32_t va = oob ? OOB_OFFSET : voff_a, vb = (B_KN ? dead : oob) ? OOB_OFFSET : voff_b;
       constexpr int CH = DMA_PER_WAVE, NRD = FA + FN, NMF = FA * FN;
 #pragma unroll
       for (int x = 0; x < CH; ++x) {
@@ -279,7 +298,7 @@ struct TileF16NTDma {
             if (r < FA)
               fa[0][r] = *reinterpret_cast<const half8v *>(nxt + rd_a[0] + r * FROWS * ROW_BYTES);
             else
-              fb[bnext][r - FA] = *reinterpret_cast<const half8v *>(nxt + rd_b[0] + (r - FA) * FROWS * ROW_BYTES);
+              read_b16_one(nxt, bnext, 0, r - FA);
           }
         if (x < A_DMA) {
           const int g = wave + x * NW;

@@ -432,12 +432,14 @@ def test_full_size_exact_integer_checksums(sk, shape):
     sk.workspace_status()
 
 
+@pytest.mark.parametrize("variant", [2, 5], ids=["mfma32", "mfma16"])
 @pytest.mark.parametrize("cfg", [dict(bm=256, bn=256), dict(bm=128, bn=128), dict(bm=128, bn=256), dict(bm=256, bn=128)],
                          ids=lambda c: f"{c['bm']}x{c['bn']}")
-def test_nn_layout(sk, oracle, cfg):
+def test_nn_layout(sk, oracle, cfg, variant):
     """B given as [K,N] (the layout of the reference's fp32 script and of the large dense
-    configuration): ragged shapes against the oracle, all schedules; then exact integer data at
-    3000 x 5120 x 12288."""
+    configuration), both MFMA forms: ragged shapes against the oracle, all schedules; then exact
+    integer data at 3000 x 5120 x 12288."""
+    cfg = dict(cfg, variant=variant)
     rng = np.random.default_rng(21)
     for (M, N, K) in [(200, 136, 328), (1000, 1096, 4104), (520, 264, 64)]:
         A = (rng.random((M, K), dtype=np.float32) * 2 - 1).astype(np.float16)
