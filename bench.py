@@ -121,7 +121,7 @@ def main():
 
     # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/)
     traffic = None
-    tpath = os.path.join(ROOT, "profiles", "traffic_tile_f16_nt_dma_256x256x64_8192.json")
+    tpath = os.path.join(ROOT, "profiles", f"traffic_{streamk.kernel_name(plan.kernel_id)}_8192.json")
     if os.path.exists(tpath):
         with open(tpath) as f:
             traffic = json.load(f).get("hbm_bytes_per_launch")
@@ -137,7 +137,7 @@ def main():
                    "compute_units": cus, "check_max_abs_rel": err},
         "roofline": {"bound": "mfma", "achieved": round(kernel_tflops, 2), "peak": PEAK_FP16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(kernel_tflops / PEAK_FP16_TFLOPS, 4),
-                     "traffic": traffic, "kernel": f"tile_f16_nt_dma_{plan.bm}x{plan.bn}x{plan.bk}",
+                     "traffic": traffic, "kernel": streamk.kernel_name(plan.kernel_id),
                      "avg_launch_ms": round(ev_ms, 5)},
     }
 
@@ -199,6 +199,27 @@ def main():
             ms = time_graph(lambda: streamk.streamk_fp16(a, b, out=c, plan=p))
             cfg2[name] = {"us": round(ms * 1e3, 2), "tflops": round(2.0 * 1024 * 1024 * 8192 / ms / 1e9, 1)}
         extra["cfg_1024x1024x8192_128x128"] = cfg2
+
+        # the large dense configuration in both layouts: tuned plan against the data-parallel-only
+        # schedule of the same tile, and torch.matmul (hipBLASLt) on the same operands
+        dense = []
+        for (m, n, k) in ((8192, 8192, 8192), (3000, 5120, 12288)):
+            a, b = inputs(m, n, k, seed=5)
+            bt = b.T.contiguous()
+            c = torch.empty(m, n, dtype=torch.float16, device="cuda")
+            for layout, bmat in (("nt", b), ("nn", bt)):
+                p = streamk.make_plan(m, n, k, "float16", layout)
+                pd = streamk.make_plan(m, n, k, "float16", layout, bm=p.bm, bn=p.bn, bk=p.bk, schedule="dp", raster=8)
+                row = {"shape": [m, n, k], "layout": layout, "tile": [p.bm, p.bn, p.bk],
+                       "kernel": streamk.kernel_name(p.kernel_id), "streamk_tiles": p.streamk_tiles}
+                for name, fn in (("tuned", lambda: streamk.streamk_fp16(a, bmat, layout=layout, out=c, plan=p)),
+                                 ("dp_only", lambda: streamk.streamk_fp16(a, bmat, layout=layout, out=c, plan=pd)),
+                                 ("torch_matmul", lambda: torch.matmul(a, bmat.T if layout == "nt" else bmat, out=c))):
+                    ms = min(time_eager(fn, 3, 10)[0] for _ in range(2))
+                    row[name] = {"us": round(ms * 1e3, 1), "tflops": round(2.0 * m * n * k / ms / 1e9, 1)}
+                dense.append(row)
+            del a, b, bt, c
+        extra["large_dense"] = dense
 
         q4 = []
         g = torch.Generator(device="cpu").manual_seed(4)

@@ -104,6 +104,9 @@ typedef struct sk_plan {
 
 int sk_version(void);
 const char *sk_strerror(int status);
+/* Name of the compiled kernel instance a plan runs (sk_plan.kernel_id), e.g. for reading profiler
+ * output; NULL for an unknown id.  The reference names its generated kernel after the script. */
+const char *sk_kernel_name(int kernel_id);
 
 /* Number of compute units and max co-resident CTAs per CU are read from the current HIP device.
  * Replaces `total_sm = 108` (streamk_fp32.py:17). */

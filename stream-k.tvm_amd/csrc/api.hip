@@ -127,6 +127,11 @@ int cached_occupancy(int id, bool skinny) {
 
 extern "C" int sk_version(void) { return SK_VERSION; }
 
+extern "C" const char *sk_kernel_name(int kernel_id) {
+  const KernelInfo *k = kernel_by_id(kernel_id);
+  return k ? k->name : nullptr;
+}
+
 extern "C" const char *sk_strerror(int s) {
   switch (s) {
     case SK_OK: return "ok";

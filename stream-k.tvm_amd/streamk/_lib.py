@@ -60,6 +60,8 @@ def lib():
     L.sk_version.restype = ci
     L.sk_strerror.argtypes = [ci]
     L.sk_strerror.restype = ctypes.c_char_p
+    L.sk_kernel_name.argtypes = [ci]
+    L.sk_kernel_name.restype = ctypes.c_char_p
     L.sk_device_info.argtypes = [P(ci), P(ci), P(ci)]
     L.sk_make_plan.argtypes = [i64, i64, i64, ci, ci, P(SkConfig), ci, P(SkPlan)]
     L.sk_plan_cta_range.argtypes = [P(SkPlan), ci, P(ctypes.c_int32), P(ctypes.c_int32)]
@@ -84,6 +86,11 @@ def lib():
         getattr(L, f).restype = ci
     _lib = L
     return L
+
+
+def kernel_name(kernel_id):
+    name = lib().sk_kernel_name(kernel_id)
+    return name.decode() if name else None
 
 
 def strerror(status):
