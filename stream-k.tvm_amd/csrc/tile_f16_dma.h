@@ -19,6 +19,8 @@
 // so the barrier, the DMA issue and the first fragment reads of the next iteration all overlap
 // with the last MFMA block.
 #pragma once
+#include <type_traits>
+
 #include "sk_device.h"
 #include "tile_f16.h"
 
@@ -50,9 +52,9 @@ struct LdsArray {
 // MFMA16_: the arithmetic uses v_mfma_f32_16x16x32_f16 instead of v_mfma_f32_32x32x16_f16.  Both
 // run at the same FLOP per cycle, but the 16x16x32 form reads and writes half as many accumulator
 // registers per FLOP, and on random operands the part sustains a ~12 % higher clock with it under
-// its power limit.  Each 32x32 block of the accumulator is then four 16x16 blocks (block (si, sj)
-// in elements 4*(2*si+sj) .. +3): lane l holds C[16*si + l%16][16*sj + 4*(l/16) + e].  A K-step
-// covers 32 K-values: lane group g = l/16 takes 16-byte chunk 4*kk + g of its row.
+// its power limit.  The accumulator is then kept as 16x16 blocks of four registers: lane l holds
+// C[16*ii + l%16][16*jj + 4*(l/16) + e] of block (ii, jj).  A K-step covers 32 K-values: lane
+// group g = l/16 takes 16-byte chunk 4*kk + g of its row.
 template <int BM_, int BN_, int WM_, int WN_, bool B_KN_ = false, int BK_ = 64, bool MFMA16_ = false>
 struct TileF16NTDma {
   static constexpr bool B_KN = B_KN_, MFMA16 = MFMA16_;
@@ -97,7 +99,12 @@ struct TileF16NTDma {
   static_assert(PATCH_ROWS % 32 == 0, "epilogue pass must hold whole 32-row blocks");
 
   typedef TileF16NT<BM_, BN_, 64, WM_, WN_> Base;  // shares the accumulator type and the partials
-  typedef typename Base::Acc Acc;
+  // 16x16x32: the accumulator is kept as 16x16 blocks of four registers (block (ii, jj): lane l holds
+  // C[16*ii + l%16][16*jj + 4*(l/16) + e]), each updated in place by its MFMA
+  struct Acc16 {
+    floatx4 v[FM][FN];
+  };
+  typedef typename std::conditional<MFMA16_, Acc16, typename Base::Acc>::type Acc;
 
   static __device__ __forceinline__ char *stage(int s) {
     if (NSTAGE == 2) return s == 0 ? LdsArray<STAGE_BYTES, 0>::get() : LdsArray<STAGE_BYTES, 1>::get();
@@ -132,12 +139,19 @@ struct TileF16NTDma {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
 
+    if constexpr (MFMA16) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+      for (int i = 0; i < FM; ++i)
 #pragma unroll
-      for (int j = 0; j < TN; ++j)
+        for (int j = 0; j < FN; ++j) acc.v[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+    } else {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc.c[i][j][r] = 0.f;
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc.c[i][j][r] = 0.f;
+    }
 
     const int rows_a = min(BM, a.M - pm * BM), rows_b = min(BN, a.N - pn * BN);
     const uint4v rsrc_a = make_rsrc_words(a.A + (int64_t)pm * BM * a.lda, (uint32_t)(rows_a * a.lda * 2));
@@ -244,12 +258,10 @@ struct TileF16NTDma {
       for (int j = 0; j < FN; ++j) read_b16_one(st, buf, kk, j);
     };
     auto mfma_one16 = [&](int abuf, int bbuf, int mh, int idx) {
-      const int i = idx / FN, j = idx % FN, ii = mh * FA + i;
-      floatx16 &c = acc.c[ii / 2][j / 2];
-      const int q = 4 * (2 * (ii & 1) + (j & 1));
-      floatx4 t = floatx4{c[q], c[q + 1], c[q + 2], c[q + 3]};
-      t = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[bbuf][j], fa[abuf][i], t, 0, 0, 0);
-      c[q] = t[0], c[q + 1] = t[1], c[q + 2] = t[2], c[q + 3] = t[3];
+      if constexpr (MFMA16) {
+        const int i = idx / FN, j = idx % FN, ii = mh * FA + i;
+        acc.v[ii][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[bbuf][j], fa[abuf][i], acc.v[ii][j], 0, 0, 0);
+      }
     };
     auto mfma_half16 = [&](int abuf, int bbuf, int mh) {
 #pragma unroll
@@ -273,11 +285,13 @@ struct TileF16NTDma {
       }
     };
     auto mfma_step = [&](int buf) {
+      if constexpr (!MFMA16) {
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc.c[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[buf][j], fa[buf][i], acc.c[i][j], 0, 0, 0);
+          for (int j = 0; j < TN; ++j)
+            acc.c[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[buf][j], fa[buf][i], acc.c[i][j], 0, 0, 0);
+      }
     };
     // 16x16x32, the half-step behind the barrier, in DMA_PER_WAVE slices: each issues one load of
     // K-iteration kt_next into `cur`, its share of the first fragment reads of `nxt` (A into
@@ -465,22 +479,30 @@ struct TileF16NTDma {
     constexpr int BLK = PATCH_ROWS / 32;  // 32-row blocks per pass
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
+      if constexpr (MFMA16) {
 #pragma unroll
-      for (int ib = 0; ib < BLK; ++ib)
+        for (int ib = 0; ib < PATCH_ROWS / 16; ++ib)
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
+          for (int j = 0; j < FN; ++j) {
             half4v h;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) h[e] = (half_t)acc.c[p * BLK + ib][j][q * 4 + e];
-            if (MFMA16)  // q = 2*si + sj: rows 16*si + lane%16, columns 16*sj + 4*(lane/16) + e
-              *reinterpret_cast<half4v *>(patch + (ib * 32 + (q >> 1) * 16 + (lane & 15)) * LDC + j * 32 +
-                                          (q & 1) * 16 + (lane >> 4) * 4) = h;
-            else
+            for (int e = 0; e < 4; ++e) h[e] = (half_t)acc.v[p * (PATCH_ROWS / 16) + ib][j][e];
+            *reinterpret_cast<half4v *>(patch + (ib * 16 + (lane & 15)) * LDC + j * 16 + (lane >> 4) * 4) = h;
+          }
+      } else {
+#pragma unroll
+        for (int ib = 0; ib < BLK; ++ib)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              half4v h;
+#pragma unroll
+              for (int e = 0; e < 4; ++e) h[e] = (half_t)acc.c[p * BLK + ib][j][q * 4 + e];
               *reinterpret_cast<half4v *>(patch + (ib * 32 + (lane & 31)) * LDC + j * 32 + q * 8 +
                                           (lane >> 5) * 4) = h;
-          }
+            }
+      }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -508,10 +530,59 @@ struct TileF16NTDma {
   }
 
   static constexpr bool COHERENT_PARTIALS = false;
-  static __device__ __forceinline__ void store_partial(const Acc &acc, float *dst) { Base::store_partial(acc, dst); }
-  static __device__ __forceinline__ void add_partial(Acc &acc, const float *src) { Base::add_partial(acc, src); }
-  static __device__ __forceinline__ void atomic_partial(const Acc &acc, float *dst) { Base::atomic_partial(acc, dst); }
-  static __device__ __forceinline__ void take_partial(Acc &acc, float *src) { Base::take_partial(acc, src); }
+  // partials in the workspace: float4 group v of thread t at (v * NT + t) * 4 (ordered reduce),
+  // element s of thread t at s * NT + t (atomic accumulation buffer); see tile_f16.h
+  static __device__ __forceinline__ void store_partial(const Acc &acc, float *dst) {
+    if constexpr (MFMA16) {
+      dst = pin_here(dst);
+#pragma unroll
+      for (int v = 0; v < NV4; ++v)
+        *reinterpret_cast<floatx4 *>(dst + ((size_t)v * NT + threadIdx.x) * 4) = acc.v[v / FN][v % FN];
+    } else {
+      Base::store_partial(acc, dst);
+    }
+  }
+  static __device__ __forceinline__ void add_partial(Acc &acc, const float *src) {
+    if constexpr (MFMA16) {
+      src = pin_here(src);
+#pragma unroll
+      for (int v = 0; v < NV4; ++v) {
+        acc.v[v / FN][v % FN] += *reinterpret_cast<const floatx4 *>(src + ((size_t)v * NT + threadIdx.x) * 4);
+        if (v % 8 == 7) asm volatile("" ::: "memory");  // at most 8 loads in flight
+      }
+    } else {
+      Base::add_partial(acc, src);
+    }
+  }
+  static __device__ __forceinline__ void atomic_partial(const Acc &acc, float *dst) {
+    if constexpr (MFMA16) {
+      dst = pin_here(dst);
+#pragma unroll
+      for (int v = 0; v < NV4; ++v)
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          atomic_add_f32(dst + (size_t)(v * 4 + e) * NT + threadIdx.x, acc.v[v / FN][v % FN][e]);
+    } else {
+      Base::atomic_partial(acc, dst);
+    }
+  }
+  static __device__ __forceinline__ void take_partial(Acc &acc, float *src) {
+    if constexpr (MFMA16) {
+      src = pin_here(src);
+#pragma unroll
+      for (int v = 0; v < NV4; ++v) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float *p = src + (size_t)(v * 4 + e) * NT + threadIdx.x;
+          acc.v[v / FN][v % FN][e] = *p;
+          *p = 0.f;
+        }
+        if (v % 4 == 3) asm volatile("" ::: "memory");
+      }
+    } else {
+      Base::take_partial(acc, src);
+    }
+  }
 };
 
 }  // namespace sk
