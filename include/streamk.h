@@ -65,7 +65,7 @@ typedef enum sk_fixup {
                               ascending CTA order: bitwise reproducible */
 } sk_fixup;
 
-typedef enum sk_dtype { SK_F16 = 0, SK_F32 = 1, SK_Q4 = 2 } sk_dtype;
+typedef enum sk_dtype { SK_F16 = 0, SK_F32 = 1, SK_Q4 = 2, SK_BF16 = 3 } sk_dtype;
 
 /* Tunables; a zero field means "choose for me".  Replaces the module-level constants and
  * bitblas Hint of the reference (streamk_fp32.py:24-28, streamk_fp16.py:32-59) and is what the
@@ -147,6 +147,12 @@ int sk_gemm_f16(const void *A, const void *B, void *C, int64_t M, int64_t N, int
                 void *stream);
 
 /* fp32 GEMM (fp32 MFMA, fp32 out).  Replaces tl_mod(A, B, C) of streamk_fp32.py:197-202. */
+/* The same call for bfloat16 operands and output (fp32 accumulate, C rounded to nearest even); the
+ * plan is made with dtype SK_BF16.  No counterpart in the reference, whose scripts are fp16 / fp32:
+ * the tile kernels with the bfloat16 form of the MFMA.  Requirements as for sk_gemm_f16. */
+int sk_gemm_bf16(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                 int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws, size_t ws_bytes, void *stream);
+
 int sk_gemm_f32(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
                 int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws, size_t ws_bytes,
                 void *stream);

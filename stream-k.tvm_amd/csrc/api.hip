@@ -180,11 +180,11 @@ extern "C" int sk_workspace_status(void *ws, void *stream) {
   return v == 0 ? SK_OK : SK_ERR_TIMEOUT;
 }
 
-extern "C" int sk_gemm_f16(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,
-                           int64_t lda, int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws,
-                           size_t ws_bytes, void *stream) {
+static int gemm_16bit(int dtype, const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,
+                      int64_t lda, int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws,
+                      size_t ws_bytes, void *stream) {
   if (!A || !B || !C) return SK_ERR_NULL;
-  int rc = check_plan(plan, M, N, K, SK_F16, plan ? plan->layout : 0);
+  int rc = check_plan(plan, M, N, K, dtype, plan ? plan->layout : 0);
   if (rc) return rc;
   const bool nn = plan->layout == SK_LAYOUT_NN;
   if (lda < K || ldb < (nn ? N : K) || ldc < N) return SK_ERR_SHAPE;
@@ -193,7 +193,7 @@ extern "C" int sk_gemm_f16(const void *A, const void *B, void *C, int64_t M, int
       (reinterpret_cast<uintptr_t>(C) & 1))
     return SK_ERR_ALIGN;
   const KernelInfo *k = kernel_by_id(plan->kernel_id);
-  if (!k || k->dtype != SK_F16 || k->layout != plan->layout) return SK_ERR_CONFIG;
+  if (!k || k->dtype != dtype || k->layout != plan->layout) return SK_ERR_CONFIG;
   // a tile's rows (NN: all K rows of B) must be addressable with 32-bit byte offsets
   if (lda * 2 * k->bm >= (int64_t)1 << 31 || ldb * 2 * (nn ? K : k->bn) >= (int64_t)1 << 31) return SK_ERR_SHAPE;
   DevPlan dp;
@@ -210,6 +210,19 @@ extern "C" int sk_gemm_f16(const void *A, const void *B, void *C, int64_t M, int
     herr = launch_tile_f16(k->id, a, dp, w, (hipStream_t)stream);
   }
   return herr == 0 ? SK_OK : SK_ERR_LAUNCH;
+}
+
+extern "C" int sk_gemm_f16(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,
+                           int64_t lda, int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws,
+                           size_t ws_bytes, void *stream) {
+  return gemm_16bit(SK_F16, A, B, C, M, N, K, lda, ldb, ldc, plan, ws, ws_bytes, stream);
+}
+
+// bfloat16 kernels take the same 16-bit containers; only the MFMA and the rounding of C differ
+extern "C" int sk_gemm_bf16(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,
+                            int64_t lda, int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws,
+                            size_t ws_bytes, void *stream) {
+  return gemm_16bit(SK_BF16, A, B, C, M, N, K, lda, ldb, ldc, plan, ws, ws_bytes, stream);
 }
 
 extern "C" int sk_gemm_f32(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,

@@ -147,6 +147,15 @@ struct KernelInfo {
   X(44, 128, 256, 2, 4)                 \
   X(45, 256, 128, 4, 2)
 
+// bfloat16 instances of the direct-to-LDS tile kernels (16x16x32 MFMAs):  X(id, BM, BN, WM, WN, BK, NN)
+#define SK_TILE_BF16_KERNELS(X)    \
+  X(60, 256, 256, 2, 4, 64, false) \
+  X(61, 128, 128, 2, 2, 64, false) \
+  X(62, 128, 128, 2, 2, 32, false) \
+  X(63, 64, 64, 2, 2, 32, false)   \
+  X(64, 256, 256, 2, 4, 64, true)  \
+  X(65, 128, 128, 2, 2, 64, true)
+
 const KernelInfo *kernel_table(int *count);
 const KernelInfo *kernel_by_id(int id);
 

@@ -27,6 +27,7 @@ static int launch_dma(const GemmArgs &a, const DevPlan &p, const Workspace &ws, 
 #define SK_POLICY_DMA16(id, BM, BN, WM, WN) TileF16NTDma<BM, BN, WM, WN, false, 64, true>
 #define SK_POLICY_DMA32_16(id, BM, BN, WM, WN) TileF16NTDma<BM, BN, WM, WN, false, 32, true>
 #define SK_POLICY_NN16(id, BM, BN, WM, WN) TileF16NTDma<BM, BN, WM, WN, true, 64, true>
+#define SK_POLICY_BF16(id, BM, BN, WM, WN, BK, NN) TileF16NTDma<BM, BN, WM, WN, NN, BK, true, true>
 
 int tile_kernel_infos(KernelInfo *out, int max) {
   int n = 0;
@@ -86,6 +87,15 @@ int tile_kernel_infos(KernelInfo *out, int max) {
   }
   SK_TILE_F16_NN_DMA16_KERNELS(X)
 #undef X
+#define X(id, BM, BN, WM, WN, BK, NN)                                                               \
+  if (n < max) {                                                                                    \
+    typedef SK_POLICY_BF16(id, BM, BN, WM, WN, BK, NN) P;                                           \
+    out[n++] = KernelInfo{id, FAMILY_TILE, 3 /* SK_BF16 */, (NN) ? 1 : 0, (BK) == 32 ? 5 : 4, BM, BN, BK, P::NT, P::LDS_TOTAL, \
+                          P::CTAS_PER_CU, P::TILE_ELEMS, 0, 0, 8,                                    \
+                          (NN) ? "tile_bf16_nn_dma16_" #BM "x" #BN "x" #BK : "tile_bf16_nt_dma16_" #BM "x" #BN "x" #BK}; \
+  }
+  SK_TILE_BF16_KERNELS(X)
+#undef X
   return n;
 }
 
@@ -140,6 +150,13 @@ int launch_tile_f16(int id, const GemmArgs &a, const DevPlan &p, const Workspace
     return launch_dma<P>(a, p, ws, s);                                                       \
   }
     SK_TILE_F16_NN_DMA16_KERNELS(X)
+#undef X
+#define X(id_, BM, BN, WM, WN, BK, NN)                                                   \
+  case id_: {                                                                            \
+    typedef SK_POLICY_BF16(id_, BM, BN, WM, WN, BK, NN) P;                               \
+    return launch_dma<P>(a, p, ws, s);                                                       \
+  }
+    SK_TILE_BF16_KERNELS(X)
 #undef X
   }
   return (int)hipErrorInvalidValue;
@@ -210,6 +227,15 @@ int occupancy_tile(int id) {
     return occ;                                                                                     \
   }
     SK_TILE_F16_NN_DMA16_KERNELS(X)
+#undef X
+#define X(id_, BM, BN, WM, WN, BK, NN)                                                              \
+  case id_: {                                                                                       \
+    typedef SK_POLICY_BF16(id_, BM, BN, WM, WN, BK, NN) P;                                          \
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_tile_kernel<P>, P::NT, 0) != hipSuccess) \
+      return -1;                                                                                    \
+    return occ;                                                                                     \
+  }
+    SK_TILE_BF16_KERNELS(X)
 #undef X
   }
   return -1;

@@ -55,9 +55,12 @@ struct LdsArray {
 // its power limit.  The accumulator is then kept as 16x16 blocks of four registers: lane l holds
 // C[16*ii + l%16][16*jj + 4*(l/16) + e] of block (ii, jj).  A K-step covers 32 K-values: lane
 // group g = l/16 takes 16-byte chunk 4*kk + g of its row.
-template <int BM_, int BN_, int WM_, int WN_, bool B_KN_ = false, int BK_ = 64, bool MFMA16_ = false>
+template <int BM_, int BN_, int WM_, int WN_, bool B_KN_ = false, int BK_ = 64, bool MFMA16_ = false, bool BF16_ = false>
 struct TileF16NTDma {
   static constexpr bool B_KN = B_KN_, MFMA16 = MFMA16_;
+  // BF16_: operands and C are bfloat16 (same 16-bit data movement; v_mfma_f32_16x16x32_bf16; C rounded to
+  // nearest even with v_cvt_pk_bf16_f32)
+  static_assert(!BF16_ || MFMA16_, "bfloat16 exists in the 16x16x32 form");
   static constexpr int ROW_BYTES = BK_ * 2;                    // bytes of one LDS row of A (and of B, NT)
   static constexpr int ROWS_PER_DMA = 1024 / ROW_BYTES;        // rows one wave-wide load fills
   static constexpr int NSTAGE = 128 / BK_, KSTEPS = BK_ / (MFMA16_ ? 32 : 16);
@@ -260,7 +263,13 @@ struct TileF16NTDma {
     auto mfma_one16 = [&](int abuf, int bbuf, int mh, int idx) {
       if constexpr (MFMA16) {
         const int i = idx / FN, j = idx % FN, ii = mh * FA + i;
-        acc.v[ii][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[bbuf][j], fa[abuf][i], acc.v[ii][j], 0, 0, 0);
+        if constexpr (BF16_) {
+          typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+          acc.v[ii][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, fb[bbuf][j]),
+                                                                 __builtin_bit_cast(bf16x8, fa[abuf][i]), acc.v[ii][j], 0, 0, 0);
+        } else {
+          acc.v[ii][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[bbuf][j], fa[abuf][i], acc.v[ii][j], 0, 0, 0);
+        }
       }
     };
     auto mfma_half16 = [&](int abuf, int bbuf, int mh) {
@@ -486,7 +495,15 @@ struct TileF16NTDma {
           for (int j = 0; j < FN; ++j) {
             half4v h;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) h[e] = (half_t)acc.v[p * (PATCH_ROWS / 16) + ib][j][e];
+            for (int e = 0; e < 4; ++e) {
+              const float x = acc.v[p * (PATCH_ROWS / 16) + ib][j][e];
+              if constexpr (BF16_) {
+                const __bf16 b = (__bf16)x;
+                h[e] = __builtin_bit_cast(half_t, b);  // the patch only carries 16-bit patterns
+              } else {
+                h[e] = (half_t)x;
+              }
+            }
             *reinterpret_cast<half4v *>(patch + (ib * 16 + (lane & 15)) * LDC + j * 16 + (lane >> 4) * 4) = h;
           }
       } else {

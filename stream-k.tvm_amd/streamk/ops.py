@@ -92,6 +92,33 @@ def streamk_fp16(A, B, *, Wq=None, scales=None, layout="nt", out=None, plan=None
     return C
 
 
+def streamk_bf16(A, B, *, layout="nt", out=None, plan=None, config=None, **kw):
+    """streamk_fp16 for bfloat16 operands and output (fp32 accumulation, C rounded to nearest even).
+    The reference's scripts are fp16 / fp32 only; this is the bfloat16 instance of the same tile
+    kernels."""
+    _check_matrix(A, "A", torch.bfloat16)
+    _check_matrix(B, "B", torch.bfloat16)
+    if layout not in ("nt", "nn"):
+        raise ValueError("layout must be 'nt' (B is [N,K]) or 'nn' (B is [K,N])")
+    M, K = A.shape
+    N, Kb = B.shape if layout == "nt" else (B.shape[1], B.shape[0])
+    if K != Kb:
+        raise ValueError(f"K mismatch: A is {tuple(A.shape)}, B is {tuple(B.shape)}")
+    if plan is None:
+        plan = make_plan(M, N, K, "bfloat16", layout, config, **kw)
+    C = out if out is not None else torch.empty((M, N), dtype=torch.bfloat16, device=A.device)
+    _check_matrix(C, "out", torch.bfloat16)
+    if tuple(C.shape) != (M, N):
+        raise ValueError("out has the wrong shape")
+    ws = _workspace(plan.workspace_bytes, A.device)
+    rc = _lib.lib().sk_gemm_bf16(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, A.stride(0),
+                                 B.stride(0), C.stride(0), ctypes.byref(plan),
+                                 ws.data_ptr() if ws is not None else None,
+                                 ws.numel() if ws is not None else 0, _stream_ptr())
+    _lib.check(rc, "sk_gemm_bf16")
+    return C
+
+
 Q4_MAX_M = 64  # rows of A the Q4 kernels take in one launch
 
 

@@ -375,6 +375,44 @@ def test_linear_module_matches_functional_linear(sk, oracle):
     sk.workspace_status()
 
 
+def test_bf16_tile_kernels(sk, oracle):
+    """bfloat16 instances of the tile kernels, NT and NN: ragged shapes, every instance, all schedules
+    and both fix-ups against the fp32 host product of the same (bfloat16-valued) operands; tolerance
+    1e-2 (bfloat16 rounds C to 8 bits: 2^-9 relative).  On {-1, 0, 1} data with |sums| <= 256 the
+    result must be exact, and the ordered reduce bitwise repeatable."""
+    import torch
+    torch.manual_seed(7)
+    tiles = {"nt": [(256, 256, 64), (128, 128, 64), (128, 128, 32), (64, 64, 32)], "nn": [(256, 256, 64), (128, 128, 64)]}
+    for (M, N, K) in [(200, 136, 328), (1000, 1096, 1032), (520, 264, 64), (64, 512, 2048)]:
+        A = (torch.rand(M, K) * 2 - 1).bfloat16()
+        Ai = torch.randint(-1, 2, (M, K)).bfloat16()
+        for layout in ("nt", "nn"):
+            B = (torch.rand(*((N, K) if layout == "nt" else (K, N))) * 2 - 1).bfloat16()
+            Bi = torch.randint(-1, 2, tuple(B.shape)).bfloat16()
+            ref = oracle.matmul_fp32(A.float().numpy(), B.float().numpy(), trans_b=layout == "nt")
+            exact = (Ai.double() @ (Bi.double().T if layout == "nt" else Bi.double())).numpy()
+            dA, dB, dAi, dBi = A.cuda(), B.cuda(), Ai.cuda(), Bi.cuda()
+            for (bm, bn, bk) in tiles[layout]:
+                for sch in (dict(schedule="dp"), dict(schedule="basic", fixup="reduce", grid=24),
+                            dict(schedule="sk2", fixup="atomic", grid=16)):
+                    plan = sk.make_plan(M, N, K, "bfloat16", layout, dict(bm=bm, bn=bn, bk=bk, **sch))
+                    C = sk.streamk_bf16(dA, dB, layout=layout, plan=plan)
+                    assert C.dtype == torch.bfloat16 and _rel(oracle, C, ref) <= 4e-3 <= TOL, (M, N, K, layout, bm, bn, bk, sch)
+                    Ci = sk.streamk_bf16(dAi, dBi, layout=layout, plan=plan)
+                    if np.abs(exact).max() <= 256:
+                        assert np.array_equal(Ci.double().cpu().numpy(), exact), (M, N, K, layout, bm, bn, bk, sch)
+                    if sch.get("fixup") == "reduce":
+                        assert torch.equal(C, sk.streamk_bf16(dA, dB, layout=layout, plan=plan))
+    # heuristic plans, from one row to a large tile count; a float16 tensor is refused
+    for (M, N, K) in [(1, 512, 1024), (16, 4096, 4096), (2048, 2048, 2048)]:
+        A, B = (torch.rand(M, K) * 2 - 1).bfloat16(), (torch.rand(N, K) * 2 - 1).bfloat16()
+        ref = oracle.matmul_fp32(A.float().numpy(), B.float().numpy(), trans_b=True)
+        assert _rel(oracle, sk.streamk_bf16(A.cuda(), B.cuda()), ref) <= 4e-3
+    with pytest.raises(TypeError):
+        sk.streamk_bf16(torch.zeros(8, 64, dtype=torch.float16, device="cuda"), torch.zeros(8, 64, dtype=torch.bfloat16, device="cuda"))
+    sk.workspace_status()
+
+
 def test_cfg5_large_dense(sk, oracle):
     """M = N = K = 8192 and the irregular 3000 x 5120 x 12288, U[-1,1): a random subset of rows is
     checked against an fp64 host product; the Stream-K and data-parallel schedules of the same kernel
