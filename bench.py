@@ -263,7 +263,19 @@ def main():
                 ms = time_graph(cold)
                 row["tuned_weights_from_hbm"] = {"us": round(ms * 1e3, 2), "gbs": round(nbytes / ms / 1e6, 1),
                                                  "frac_hbm": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
+                # the same with the weights in the tiled layout (one contiguous KB per load instruction)
+                tiles = [(streamk.tile_q4(w), s_) for (w, s_) in copies]
                 del copies
+                p_tiled = streamk.make_plan(m, N, K, "q4_tiled", "nt")
+
+                def cold_tiled():
+                    w, s_ = tiles[turn[0] % len(tiles)]
+                    turn[0] += 1
+                    streamk.streamk_q4(a, w, s_, out=c, plan=p_tiled, tiled=True)
+                ms = time_graph(cold_tiled)
+                row["tiled_weights_from_hbm"] = {"us": round(ms * 1e3, 2), "gbs": round(nbytes / ms / 1e6, 1),
+                                                 "frac_hbm": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
+                del tiles
             q4.append(row)
         extra["q4_N8192_K8192"] = q4
         extra["q4_note"] = ("34.6 MB of weights stay in the 256 MB Infinity Cache between launches of one weight "

@@ -65,7 +65,13 @@ typedef enum sk_fixup {
                               ascending CTA order: bitwise reproducible */
 } sk_fixup;
 
-typedef enum sk_dtype { SK_F16 = 0, SK_F32 = 1, SK_Q4 = 2, SK_BF16 = 3 } sk_dtype;
+typedef enum sk_dtype {
+  SK_F16 = 0,
+  SK_F32 = 1,
+  SK_Q4 = 2,       /* fp16 A, packed nibbles [N, K/2] row-major */
+  SK_BF16 = 3,
+  SK_Q4_TILED = 4  /* fp16 A, packed nibbles in 16-row x 64-byte tiles (sk_q4_tile_host / sk_q4_tile) */
+} sk_dtype;
 
 /* Tunables; a zero field means "choose for me".  Replaces the module-level constants and
  * bitblas Hint of the reference (streamk_fp32.py:24-28, streamk_fp16.py:32-59) and is what the
@@ -146,13 +152,13 @@ int sk_gemm_f16(const void *A, const void *B, void *C, int64_t M, int64_t N, int
                 int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws, size_t ws_bytes,
                 void *stream);
 
-/* fp32 GEMM (fp32 MFMA, fp32 out).  Replaces tl_mod(A, B, C) of streamk_fp32.py:197-202. */
 /* The same call for bfloat16 operands and output (fp32 accumulate, C rounded to nearest even); the
  * plan is made with dtype SK_BF16.  No counterpart in the reference, whose scripts are fp16 / fp32:
  * the tile kernels with the bfloat16 form of the MFMA.  Requirements as for sk_gemm_f16. */
 int sk_gemm_bf16(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
                  int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws, size_t ws_bytes, void *stream);
 
+/* fp32 GEMM (fp32 MFMA, fp32 out).  Replaces tl_mod(A, B, C) of streamk_fp32.py:197-202. */
 int sk_gemm_f32(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
                 int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws, size_t ws_bytes,
                 void *stream);
@@ -169,6 +175,8 @@ int sk_gemm_f32(const void *A, const void *B, void *C, int64_t M, int64_t N, int
  * scale to fp32 group sums, i.e. they use the unrounded (q - zero) * scale: at least as close to
  * the exact product as the rounded-weight form (within 2^-11 relative per weight of it).
  * sk_dequant_q4 and the M > 1 kernels produce the rounded weights bit for bit.
+ * A plan made with dtype SK_Q4_TILED takes Wq in the tiled layout instead (see sk_q4_tile_host): same
+ * results bit for bit, the weights stream faster.
  */
 int sk_gemm_q4(const void *A, const void *Wq, const void *scales, void *C, int64_t M, int64_t N,
                int64_t K, int64_t lda, int64_t ldc, int group, int zero, const sk_plan *plan,
@@ -195,6 +203,15 @@ int sk_dequant_q4(const void *Wq, const void *scales, void *W, int64_t N, int64_
  * the device call does not look).
  */
 int sk_q4_pack_host(const uint8_t *q, int64_t N, int64_t K, uint8_t *Wq);
+/* Tiled layout of the packed weights, the MI355X-side counterpart of the reference's weight
+ * pre-transformation (LadderPermutate, streamk_fp16_ladder_block_reduce_q4.py:568-580): byte b of row
+ * n of Wq[N, K/2] moves to ((n/16) * (K/128) + b/64) * 1024 + (n%16) * 64 + b%64, i.e. tiles of 16 rows
+ * x 64 bytes (one scale group), row by row inside a tile.  N is padded to a multiple of 16 with zero
+ * rows: the tiled array has ceil(N/16)*16 * K/2 bytes.  K must be a multiple of 128.
+ * sk_q4_tile_host / sk_q4_untile_host work on host memory, sk_q4_tile on device memory (stream-ordered). */
+int sk_q4_tile_host(const uint8_t *Wq, int64_t N, int64_t K, uint8_t *tiled);
+int sk_q4_untile_host(const uint8_t *tiled, int64_t N, int64_t K, uint8_t *Wq);
+int sk_q4_tile(const void *Wq, int64_t N, int64_t K, void *tiled, void *stream);
 int sk_q4_unpack_host(const uint8_t *Wq, int64_t N, int64_t K, uint8_t *q);
 int sk_q4_quantize_host(const uint16_t *W, int64_t N, int64_t K, int64_t ldw, int group, int zero,
                         uint8_t *Wq, uint16_t *scales);

@@ -255,7 +255,8 @@ extern "C" int sk_gemm_q4(const void *A, const void *Wq, const void *scales, voi
                           int64_t K, int64_t lda, int64_t ldc, int group, int zero, const sk_plan *plan,
                           void *ws, size_t ws_bytes, void *stream) {
   if (!A || !Wq || !scales || !C) return SK_ERR_NULL;
-  int rc = check_plan(plan, M, N, K, SK_Q4, SK_LAYOUT_NT);
+  const int dtype = plan && plan->dtype == SK_Q4_TILED ? SK_Q4_TILED : SK_Q4;  // which layout Wq is in
+  int rc = check_plan(plan, M, N, K, dtype, SK_LAYOUT_NT);
   if (rc) return rc;
   if (group != 128 || zero < 0 || zero > 15) return SK_ERR_CONFIG;
   if (lda < K || ldc < N) return SK_ERR_SHAPE;
@@ -264,7 +265,7 @@ extern "C" int sk_gemm_q4(const void *A, const void *Wq, const void *scales, voi
       (reinterpret_cast<uintptr_t>(scales) & 1) || (reinterpret_cast<uintptr_t>(C) & 1))
     return SK_ERR_ALIGN;
   const KernelInfo *k = kernel_by_id(plan->kernel_id);
-  if (!k || k->dtype != SK_Q4 || k->family != FAMILY_SKINNY) return SK_ERR_CONFIG;
+  if (!k || k->dtype != dtype || k->family != FAMILY_SKINNY) return SK_ERR_CONFIG;
   if (lda * 2 * k->bm >= (int64_t)1 << 31 || (K / 2) * k->bn >= (int64_t)1 << 31) return SK_ERR_SHAPE;
   DevPlan dp;
   Workspace w;

@@ -129,6 +129,21 @@ struct KernelInfo {
   X(150, 1, 1, 4, 4, 32768)    \
   X(151, 1, 2, 4, 4, 32768)
 
+// Q4 kernels reading tiled weights (dtype SK_Q4_TILED), same variants as their row-major twins.
+// general small-M:  X(id, MB, NB, WN, RK, DEPTH);  matrix-vector:  X(id, NB, WN, RK, DEPTH, KMAX)
+#define SK_SKINNY_Q4T_KERNELS(X) \
+  X(180, 1, 1, 4, 1, 4)          \
+  X(181, 2, 1, 4, 1, 2)          \
+  X(182, 4, 1, 4, 1, 2)          \
+  X(183, 1, 1, 1, 4, 4)          \
+  X(184, 1, 1, 2, 2, 4)
+#define SK_GEMV_Q4T_KERNELS(X) \
+  X(190, 1, 4, 1, 4, 16384)    \
+  X(191, 1, 2, 2, 4, 16384)    \
+  X(192, 1, 1, 4, 4, 16384)    \
+  X(193, 1, 2, 4, 4, 16384)    \
+  X(194, 1, 1, 4, 4, 32768)
+
 // M == 1 fp16 (NT) matrix-vector kernels (variant 2):  X(id, NB, WN, RK, DEPTH, KMAX)
 #define SK_GEMV_F16_KERNELS(X) \
   X(160, 1, 1, 4, 4, 8192)     \

@@ -57,6 +57,24 @@ int skinny_kernel_infos(KernelInfo *out, int max) {
   }
   SK_GEMV_F16_KERNELS(X)
 #undef X
+#define X(id, MB, NB, WN, RK, DEPTH)                                                                     \
+  if (n < max) {                                                                                     \
+    typedef TileSkinny<MB, NB, WN, RK, true, DEPTH, false, true> P;                                  \
+    out[n++] = KernelInfo{id, FAMILY_SKINNY, 4 /* SK_Q4_TILED */, 0, 0, P::BM, P::BN, P::BKC, P::NT, \
+                          P::LDS_BYTES, P::CTAS_PER_CU, P::TILE_ELEMS, P::SC_MAX_ITERS, P::MAX_M, 128, \
+                          "skinny_q4t_mb" #MB "_wn" #WN "_rk" #RK};                                   \
+  }
+  SK_SKINNY_Q4T_KERNELS(X)
+#undef X
+#define X(id, NB, WN, RK, DEPTH, KMAX)                                                                   \
+  if (n < max) {                                                                                     \
+    typedef TileGemvQ4<NB, WN, RK, DEPTH, KMAX, true> P;                                              \
+    out[n++] = KernelInfo{id, FAMILY_SKINNY, 4 /* SK_Q4_TILED */, 0, 2, P::BM, P::BN, P::BKC, P::NT, \
+                          P::LDS_BYTES, P::CTAS_PER_CU, P::TILE_ELEMS, P::MAX_ITERS, P::MAX_M, 128,   \
+                          "gemv_q4t_nb" #NB "_wn" #WN "_rk" #RK "_k" #KMAX};                          \
+  }
+  SK_GEMV_Q4T_KERNELS(X)
+#undef X
   return n;
 }
 
@@ -82,6 +100,20 @@ int launch_skinny(int id, const SkinnyArgs &a, const DevPlan &p, const Workspace
     return launch_policy<P>(a, p, ws, s);                                                         \
   }
     SK_GEMV_F16_KERNELS(X)
+#undef X
+#define X(id_, MB, NB, WN, RK, DEPTH)                                                       \
+  case id_: {                                                                              \
+    typedef TileSkinny<MB, NB, WN, RK, true, DEPTH, false, true> P;                        \
+    return launch_policy<P>(a, p, ws, s);                                                         \
+  }
+    SK_SKINNY_Q4T_KERNELS(X)
+#undef X
+#define X(id_, NB, WN, RK, DEPTH, KMAX)                                                     \
+  case id_: {                                                                              \
+    typedef TileGemvQ4<NB, WN, RK, DEPTH, KMAX, true> P;                                    \
+    return launch_policy<P>(a, p, ws, s);                                                         \
+  }
+    SK_GEMV_Q4T_KERNELS(X)
 #undef X
   }
   return (int)hipErrorInvalidValue;
@@ -116,6 +148,24 @@ int occupancy_skinny(int id) {
     return occ;                                                                                          \
   }
     SK_GEMV_F16_KERNELS(X)
+#undef X
+#define X(id_, MB, NB, WN, RK, DEPTH)                                                                     \
+  case id_: {                                                                                            \
+    typedef TileSkinny<MB, NB, WN, RK, true, DEPTH, false, true> P;                                      \
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_skinny_kernel<P>, P::NT, 0) != hipSuccess) \
+      return -1;                                                                                         \
+    return occ;                                                                                          \
+  }
+    SK_SKINNY_Q4T_KERNELS(X)
+#undef X
+#define X(id_, NB, WN, RK, DEPTH, KMAX)                                                                   \
+  case id_: {                                                                                            \
+    typedef TileGemvQ4<NB, WN, RK, DEPTH, KMAX, true> P;                                                  \
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_skinny_kernel<P>, P::NT, 0) != hipSuccess) \
+      return -1;                                                                                         \
+    return occ;                                                                                          \
+  }
+    SK_GEMV_Q4T_KERNELS(X)
 #undef X
   }
   return -1;

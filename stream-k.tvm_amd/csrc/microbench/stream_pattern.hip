@@ -20,7 +20,7 @@ __global__ __launch_bounds__(64) void stream(const char* base, uint32_t* out, in
       acc += *(const uint4v*)(p + i2 * 128);
       acc += *(const uint4v*)(p + i2 * 128 + 64);
     }
-  } else if (PATTERN >= 2) {
+  } else if (PATTERN >= 2 && PATTERN <= 4) {
     // PATTERN 2: 4 rows x 256 contiguous bytes per load (lane l: row l/16, piece l%16)
     // PATTERN 3: 8 rows x 128 bytes (row l/8, piece l%8); PATTERN 4: 16 rows x 64 bytes with the four
     // lanes of a row adjacent (row l/4, piece l%4).  A wave still owns 16 rows x (iters*128) bytes.
@@ -36,6 +36,15 @@ __global__ __launch_bounds__(64) void stream(const char* base, uint32_t* out, in
     for (int st = 0; st < steps; ++st) {
 #pragma unroll
       for (int g = 0; g < LOADS; ++g) acc += *(const uint4v*)(p + (size_t)g * RPL * pitch + st * BYTES_PER_ROW);
+    }
+  } else if (PATTERN == 5) {
+    // 1 KB contiguous per load, but lane l reads the piece a 16x16 MFMA operand layout takes from
+    // a 16-row x 64-byte tile stored row by row: offset (l%16)*64 + (l/16)*16
+    const char* p = base + (size_t)wave * iters_per_wave * 2048 + (lane & 15) * 64 + (lane >> 4) * 16;
+#pragma unroll 4
+    for (int it = 0; it < iters_per_wave; ++it) {
+      acc += *(const uint4v*)(p + it * 2048);
+      acc += *(const uint4v*)(p + it * 2048 + 1024);
     }
   } else {
     const char* p = base + (size_t)wave * iters_per_wave * 2048 + lane * 16;
@@ -69,6 +78,7 @@ int main() {
     if (iters * 128 >= 256) run<2, 0>("4rows x 256B", buf, out, waves, iters, wprb);
     run<3, 0>("8rows x 128B", buf, out, waves, iters, wprb);
     run<4, 0>("16rows x 64B, quads", buf, out, waves, iters, wprb);
+    run<5, 0>("1KB tile, MFMA16 lane order", buf, out, waves, iters, wprb);
   }
   return 0;
 }

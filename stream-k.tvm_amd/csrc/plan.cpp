@@ -69,10 +69,11 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
   // every CU something to do
   const KernelInfo *best = nullptr;
   // (for 32 < M <= 64 the 64x64 LDS tile below is faster than streaming the weights past 64 rows)
-  if ((M <= 32 && layout == SK_LAYOUT_NT) || dtype == SK_Q4) {
+  const bool q4 = dtype == SK_Q4 || dtype == SK_Q4_TILED;
+  if ((M <= 32 && layout == SK_LAYOUT_NT) || q4) {
     // M == 1 with Q4 weights: the matrix-vector kernel with four waves splitting K (data-parallel
     // over 16-row tiles), the fastest instance at LLM-sized N and K
-    if (dtype == SK_Q4 && M == 1 && want_variant < 0)
+    if (q4 && M == 1 && want_variant < 0)
       for (int i = 0; i < n; ++i)
         if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].variant == 2 && t[i].bn == 16 &&
             t[i].bk == 1024 && accepts_shape(t[i], M, K))
@@ -90,7 +91,7 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
           t[i].variant <= 2 && (best == nullptr || t[i].variant > best->variant))
         best = &t[i];
     if (best) return best;
-    if (dtype == SK_Q4) return nullptr;
+    if (q4) return nullptr;
   }
   if (dtype == SK_F32) {
     for (int i = 0; i < n; ++i)
@@ -128,7 +129,8 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
                             int num_cus, sk_plan *out) {
   if (!out) return SK_ERR_NULL;
   if (M <= 0 || N <= 0 || K <= 0 || M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return SK_ERR_SHAPE;
-  if (dtype != SK_F16 && dtype != SK_F32 && dtype != SK_Q4 && dtype != SK_BF16) return SK_ERR_CONFIG;
+  if (dtype != SK_F16 && dtype != SK_F32 && dtype != SK_Q4 && dtype != SK_BF16 && dtype != SK_Q4_TILED)
+    return SK_ERR_CONFIG;
   if (layout != SK_LAYOUT_NT && layout != SK_LAYOUT_NN) return SK_ERR_CONFIG;
   if (num_cus <= 0) return SK_ERR_DEVICE;
   const KernelInfo *k = pick_kernel(M, N, K, dtype, layout, cfg, num_cus);

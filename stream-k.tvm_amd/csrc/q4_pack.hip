@@ -87,10 +87,56 @@ __global__ __launch_bounds__(256) void quantize_q4_kernel(const half_t *W, uint3
   }
 }
 
+// tiled position of byte b of row n (runs = K / 128 tiles per row block)
+__host__ __device__ inline int64_t q4_tiled_offset(int64_t n, int64_t b, int64_t runs) {
+  return ((n / 16) * runs + b / 64) * 1024 + (n % 16) * 64 + b % 64;
+}
+
+// one thread per 16 bytes of the tiled array (rows past N are written as zeros)
+__global__ __launch_bounds__(256) void tile_q4_kernel(const uint4v *wq, uint4v *tiled, int64_t pieces, int64_t N,
+                                                      int64_t runs) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= pieces) return;
+  const int64_t tile = i / 64, in = i % 64;           // 64 pieces of 16 bytes per tile
+  const int64_t n = (tile / runs) * 16 + in / 4, b = (tile % runs) * 64 + (in % 4) * 16;
+  tiled[i] = n < N ? wq[(n * runs * 64 + b) / 16] : uint4v{0, 0, 0, 0};
+}
+
 }  // namespace
 }  // namespace sk
 
 using namespace sk;
+
+extern "C" int sk_q4_tile_host(const uint8_t *Wq, int64_t N, int64_t K, uint8_t *tiled) {
+  if (!Wq || !tiled) return SK_ERR_NULL;
+  if (N <= 0 || K <= 0 || (K % 128)) return SK_ERR_SHAPE;
+  const int64_t runs = K / 128, n16 = (N + 15) / 16 * 16;
+  memset(tiled, 0, (size_t)(n16 * (K / 2)));
+  for (int64_t n = 0; n < N; ++n)
+    for (int64_t b = 0; b < K / 2; b += 64) memcpy(tiled + q4_tiled_offset(n, b, runs), Wq + n * (K / 2) + b, 64);
+  return SK_OK;
+}
+
+extern "C" int sk_q4_untile_host(const uint8_t *tiled, int64_t N, int64_t K, uint8_t *Wq) {
+  if (!Wq || !tiled) return SK_ERR_NULL;
+  if (N <= 0 || K <= 0 || (K % 128)) return SK_ERR_SHAPE;
+  const int64_t runs = K / 128;
+  for (int64_t n = 0; n < N; ++n)
+    for (int64_t b = 0; b < K / 2; b += 64) memcpy(Wq + n * (K / 2) + b, tiled + q4_tiled_offset(n, b, runs), 64);
+  return SK_OK;
+}
+
+extern "C" int sk_q4_tile(const void *Wq, int64_t N, int64_t K, void *tiled, void *stream) {
+  if (!Wq || !tiled) return SK_ERR_NULL;
+  if (N <= 0 || K <= 0 || (K % 128)) return SK_ERR_SHAPE;
+  if ((reinterpret_cast<uintptr_t>(Wq) & 15) || (reinterpret_cast<uintptr_t>(tiled) & 15)) return SK_ERR_ALIGN;
+  const int64_t runs = K / 128, pieces = (N + 15) / 16 * runs * 64;
+  const int64_t blocks = (pieces + 255) / 256;
+  if (blocks > 0x7fffffff) return SK_ERR_SHAPE;
+  hipLaunchKernelGGL(tile_q4_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const uint4v *)Wq,
+                     (uint4v *)tiled, pieces, N, runs);
+  return hipGetLastError() == hipSuccess ? SK_OK : SK_ERR_LAUNCH;
+}
 
 extern "C" int sk_q4_pack_host(const uint8_t *q, int64_t N, int64_t K, uint8_t *Wq) {
   if (!q || !Wq) return SK_ERR_NULL;

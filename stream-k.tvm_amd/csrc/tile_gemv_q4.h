@@ -38,7 +38,10 @@
 
 namespace sk {
 
-template <int NB_, int WN_, int RK_, int DEPTH_, int KMAX_ = 16384>
+//
+// TILED_: the weights come in 16-row x 64-byte tiles (see tile_skinny.h); the lane order of the
+// loads, row = lane/4, piece = lane%4, is then the byte order of a tile: one contiguous KB per load.
+template <int NB_, int WN_, int RK_, int DEPTH_, int KMAX_ = 16384, bool TILED_ = false>
 struct TileGemvQ4 {
   typedef SkinnyArgs Args;
   static constexpr int NB = NB_, WN = WN_, RK = RK_, DEPTH = DEPTH_, KMAX = KMAX_;
@@ -86,11 +89,17 @@ struct TileGemvQ4 {
     // group of its row; rows past N read as zero ----
     const int rows_w = min(BN, a.N - pn * BN);
     const uint32_t ldw = (uint32_t)a.ldw;
-    const BufferRsrc rsrc_w = make_rsrc(reinterpret_cast<const char *>(a.W) + (int64_t)pn * BN * ldw, rows_w * ldw);
+    const uint32_t block_bytes = (uint32_t)a.groups * 1024;  // tiled: one 16-row block of W
+    const BufferRsrc rsrc_w =
+        TILED_ ? make_rsrc(reinterpret_cast<const char *>(a.W) + (int64_t)pn * (BN / 16) * block_bytes,
+                           (uint32_t)((rows_w + 15) / 16) * block_bytes)
+               : make_rsrc(reinterpret_cast<const char *>(a.W) + (int64_t)pn * BN * ldw, rows_w * ldw);
     const int klane = rk * BK + piece * 32;
     uint32_t voff_w[NB];
 #pragma unroll
-    for (int j = 0; j < NB; ++j) voff_w[j] = (uint32_t)((wn * NB + j) * 16 + row) * ldw + (uint32_t)(klane / 2);
+    for (int j = 0; j < NB; ++j)
+      voff_w[j] = TILED_ ? (uint32_t)(wn * NB + j) * block_bytes + (uint32_t)lane * 16
+                         : (uint32_t)((wn * NB + j) * 16 + row) * ldw + (uint32_t)(klane / 2);
     uint4v wreg[DEPTH][NB][2];
     // loads of iterations past the segment or past K get an out-of-range offset: they return
     // zeros without touching memory, and every round of the main loop has the same loads in flight
@@ -102,7 +111,10 @@ struct TileGemvQ4 {
 #pragma unroll
         for (int c = 0; c < 2; ++c)
           wreg[slot][j][c] =
-              buffer_load_16(rsrc_w, klane + c * 128 < klimit ? voff_w[j] : OOB_OFFSET, (uint32_t)(kbase / 2) + c * 64);
+              TILED_ ? buffer_load_16(rsrc_w, rk * BK + c * 128 < klimit ? voff_w[j] : OOB_OFFSET,
+                                      (uint32_t)((kbase + rk * BK) / QGROUP + c) * 1024)
+                     : buffer_load_16(rsrc_w, klane + c * 128 < klimit ? voff_w[j] : OOB_OFFSET,
+                                      (uint32_t)(kbase / 2) + c * 64);
     };
     SK_TRACE(1);
 

@@ -89,8 +89,16 @@ __device__ __forceinline__ void stage_scales(half_t *ldsS, const half_t *scales_
 
 // ROW1_: M == 1 only.  A single row of A is staged and every lane reads it (an LDS broadcast);
 // rows 1..15 of the MFMA result are then copies of row 0 and are never stored.
-template <int MB_, int NB_, int WN_, int RK_, bool Q4_, int DEPTH_, bool ROW1_ = false>
+//
+// TILED_ (Q4 only): the packed weights are stored in tiles of 16 rows x 64 bytes (one 128-wide scale
+// group of 16 weight rows), row by row inside a tile, tiles ordered [row block][group]
+// (sk_q4_tile_host / sk_q4_tile).  A wave's load instruction then reads one contiguous KB instead
+// of 64 bytes from each of 16 rows 4 KB apart, which streams 1.5x faster (profiles/
+// gemv_q4_M1_N8192_K8192.md, access pattern table); each lane receives the same bytes as from the
+// row-major array.
+template <int MB_, int NB_, int WN_, int RK_, bool Q4_, int DEPTH_, bool ROW1_ = false, bool TILED_ = false>
 struct TileSkinny {
+  static_assert(!TILED_ || Q4_, "tiled weights exist for Q4");
   typedef SkinnyArgs Args;
   static constexpr int MB = MB_, NB = NB_, WN = WN_, RK = RK_, DEPTH = DEPTH_;
   static constexpr bool Q4 = Q4_;
@@ -150,14 +158,19 @@ struct TileSkinny {
     constexpr int WB = Q4 ? 1 : 4;  // bytes per 2 K-values... (Q4: 1 byte, fp16: 4 bytes)
     const int rows_w = min(BN, a.N - pn * BN);
     const uint32_t ldw_bytes = (uint32_t)a.ldw * (Q4 ? 1 : 2);
+    // tiled: a 16-row block of the tile is a.groups consecutive KB; blocks past N are out of range
+    const uint32_t block_bytes = (uint32_t)a.groups * 1024;
     const BufferRsrc rsrc_w =
-        make_rsrc(reinterpret_cast<const char *>(a.W) + (int64_t)pn * BN * ldw_bytes, rows_w * ldw_bytes);
+        TILED_ ? make_rsrc(reinterpret_cast<const char *>(a.W) + (int64_t)pn * (BN / 16) * block_bytes,
+                           (uint32_t)((rows_w + 15) / 16) * block_bytes)
+               : make_rsrc(reinterpret_cast<const char *>(a.W) + (int64_t)pn * BN * ldw_bytes, rows_w * ldw_bytes);
     constexpr int E = Q4 ? 32 : 8;               // K-values in one 16-byte load
     const int klane = rk * BK + lg * E;          // K offset of this lane's piece of load 0
     uint32_t voff_w[NB];
 #pragma unroll
     for (int j = 0; j < NB; ++j)
-      voff_w[j] = (uint32_t)((wn * NB + j) * 16 + lr) * ldw_bytes + (uint32_t)(klane / 2) * WB;
+      voff_w[j] = TILED_ ? (uint32_t)(wn * NB + j) * block_bytes + (uint32_t)(lr * 64 + lg * 16)
+                         : (uint32_t)((wn * NB + j) * 16 + lr) * ldw_bytes + (uint32_t)(klane / 2) * WB;
 
     // ---- A tile: all BM rows are staged; rows past M read as zero ----
     const int a_rows = min(a.M - pm * BM, A_ROWS);
@@ -181,14 +194,15 @@ struct TileSkinny {
     // klimit = K-values left in the tile row from this iteration's start (<= 0 past the segment).
     auto issue_loads = [&](int slot, int rel_it) {
       const int kbase = (k0 + rel_it) * BKC;
-      const uint32_t koff_w = (uint32_t)(kbase / 2) * WB, koff_a = (uint32_t)kbase * 2;
+      const uint32_t koff_w = TILED_ ? (uint32_t)((kbase + rk * BK) / QGROUP) * 1024 : (uint32_t)(kbase / 2) * WB;
+      const uint32_t koff_a = (uint32_t)kbase * 2;
       const int klimit = rel_it < n ? a.K - kbase : 0;
 #pragma unroll
       for (int j = 0; j < NB; ++j)
 #pragma unroll
         for (int c = 0; c < WLOADS; ++c) {
-          const bool inside = klane + c * (4 * E) < klimit;
-          wreg[slot][j][c] = buffer_load_16(rsrc_w, inside ? voff_w[j] : OOB_OFFSET, koff_w + c * 64);
+          const bool inside = (TILED_ ? rk * BK : klane) + c * (4 * E) < klimit;
+          wreg[slot][j][c] = buffer_load_16(rsrc_w, inside ? voff_w[j] : OOB_OFFSET, koff_w + c * (TILED_ ? 1024 : 64));
         }
 #pragma unroll
       for (int i = 0; i < A_LOADS; ++i) {

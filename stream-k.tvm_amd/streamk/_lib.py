@@ -8,7 +8,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libstreamk.so")
 
-SK_F16, SK_F32, SK_Q4, SK_BF16 = 0, 1, 2, 3
+SK_F16, SK_F32, SK_Q4, SK_BF16, SK_Q4_TILED = 0, 1, 2, 3, 4
 LAYOUT_NT, LAYOUT_NN = 0, 1
 SCHEDULES = {"auto": 0, "dp": 1, "sk2": 2, "sk1": 3, "basic": 4, "splitk": 5}
 FIXUPS = {"auto": 0, "atomic": 1, "reduce": 2}
@@ -80,7 +80,11 @@ def lib():
     L.sk_q4_unpack_host.argtypes = [vp, i64, i64, vp]
     L.sk_q4_quantize_host.argtypes = [vp, i64, i64, i64, ci, ci, vp, vp]
     L.sk_q4_quantize.argtypes = [vp, i64, i64, i64, ci, ci, vp, vp, vp]
-    for f in ("sk_q4_pack_host", "sk_q4_unpack_host", "sk_q4_quantize_host", "sk_q4_quantize"):
+    L.sk_q4_tile_host.argtypes = [vp, i64, i64, vp]
+    L.sk_q4_untile_host.argtypes = [vp, i64, i64, vp]
+    L.sk_q4_tile.argtypes = [vp, i64, i64, vp, vp]
+    for f in ("sk_q4_pack_host", "sk_q4_unpack_host", "sk_q4_quantize_host", "sk_q4_quantize", "sk_q4_tile_host",
+              "sk_q4_untile_host", "sk_q4_tile"):
         getattr(L, f).restype = ci
     for f in ("sk_device_info", "sk_make_plan", "sk_plan_cta_range", "sk_plan_tile_coords",
               "sk_workspace_init", "sk_workspace_status", "sk_gemm_f16", "sk_gemm_f32",

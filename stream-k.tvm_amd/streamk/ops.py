@@ -122,18 +122,50 @@ def streamk_bf16(A, B, *, layout="nt", out=None, plan=None, config=None, **kw):
 Q4_MAX_M = 64  # rows of A the Q4 kernels take in one launch
 
 
-def streamk_q4(A, Wq, scales, *, out=None, plan=None, config=None, zero=8, group=128, **kw):
+def tile_q4(Wq):
+    """Packed weights Wq[N, K/2] -> the tiled layout (16 rows x 64 bytes per tile, [row block][group]),
+    on the device Wq lives on.  Returns a [ceil(N/16)*16, K/2] array (rows past N are zero) to pass to
+    streamk_q4(..., tiled=True); the weights then stream faster and the results are the same bit
+    for bit.  The counterpart of the reference's offline weight transformation
+    (streamk_fp16_ladder_block_reduce_q4.py:568-580)."""
+    if Wq.dtype != torch.uint8 or Wq.dim() != 2 or not Wq.is_contiguous():
+        raise ValueError("Wq must be a contiguous 2-D uint8 tensor")
+    N, K = Wq.shape[0], Wq.shape[1] * 2
+    out = torch.empty(((N + 15) // 16 * 16, K // 2), dtype=torch.uint8, device=Wq.device)
+    if Wq.is_cuda:
+        _lib.check(_lib.lib().sk_q4_tile(Wq.data_ptr(), N, K, out.data_ptr(), _stream_ptr()), "sk_q4_tile")
+    else:
+        _lib.check(_lib.lib().sk_q4_tile_host(Wq.data_ptr(), N, K, out.data_ptr()), "sk_q4_tile_host")
+    return out
+
+
+def untile_q4(tiled, N):
+    """Inverse of tile_q4 for host tensors: the row-major Wq[N, K/2]."""
+    if tiled.dtype != torch.uint8 or tiled.dim() != 2 or tiled.is_cuda or not tiled.is_contiguous():
+        raise ValueError("tiled must be a contiguous 2-D uint8 tensor in host memory")
+    K = tiled.shape[1] * 2
+    if tiled.shape[0] != (N + 15) // 16 * 16:
+        raise ValueError("tiled has ceil(N/16)*16 rows")
+    Wq = torch.empty((N, K // 2), dtype=torch.uint8)
+    _lib.check(_lib.lib().sk_q4_untile_host(tiled.data_ptr(), N, K, Wq.data_ptr()), "sk_q4_untile_host")
+    return Wq
+
+
+def streamk_q4(A, Wq, scales, *, out=None, plan=None, config=None, zero=8, group=128, tiled=False, **kw):
     """C[M,N] fp16 = A[M,K] fp16 @ dequant(Wq)[N,K].T, weights in natural nibble order
-    (streamk_fp16_ladder_block_reduce_q4.py:552)."""
+    (streamk_fp16_ladder_block_reduce_q4.py:552).  tiled=True: Wq is the output of tile_q4 (N is
+    then taken from scales)."""
     _check_matrix(A, "A", torch.float16)
     _check_matrix(Wq, "Wq", torch.uint8)
     _check_matrix(scales, "scales", torch.float16)
     M, K = A.shape
-    N = Wq.shape[0]
-    if Wq.shape[1] * 2 != K or not Wq.is_contiguous():
-        raise ValueError(f"Wq must be contiguous [N, K/2]; got {tuple(Wq.shape)} for K={K}")
+    N = scales.shape[0] if tiled else Wq.shape[0]
+    if Wq.shape[1] * 2 != K or not Wq.is_contiguous() or (tiled and Wq.shape[0] != (N + 15) // 16 * 16):
+        raise ValueError(f"Wq must be contiguous [N, K/2] (tiled: ceil(N/16)*16 rows); got {tuple(Wq.shape)} for K={K}")
     if tuple(scales.shape) != (N, K // group) or not scales.is_contiguous():
         raise ValueError(f"scales must be contiguous [N, K/group]; got {tuple(scales.shape)}")
+    if plan is not None and (plan.dtype == _lib.SK_Q4_TILED) != bool(tiled):
+        raise ValueError("the plan was made for the other weight layout")
     C = out if out is not None else torch.empty((M, N), dtype=torch.float16, device=A.device)
     _check_matrix(C, "out", torch.float16)
     if tuple(C.shape) != (M, N):
@@ -145,11 +177,13 @@ def streamk_q4(A, Wq, scales, *, out=None, plan=None, config=None, zero=8, group
         if M <= 4 * Q4_MAX_M:
             for m0 in range(0, M, Q4_MAX_M):
                 streamk_q4(A[m0:m0 + Q4_MAX_M], Wq, scales, out=C[m0:m0 + Q4_MAX_M], config=config, zero=zero,
-                           group=group, **kw)
+                           group=group, tiled=tiled, **kw)
             return C
+        if tiled:
+            raise ValueError("more than 256 rows of A need the row-major weights (they are dequantised once)")
         return streamk_fp16(A, dequant_q4(Wq, scales, zero=zero, group=group), out=C)
     if plan is None:
-        plan = make_plan(M, N, K, "q4", "nt", config, **kw)
+        plan = make_plan(M, N, K, "q4_tiled" if tiled else "q4", "nt", config, **kw)
     ws = _workspace(plan.workspace_bytes, A.device)
     rc = _lib.lib().sk_gemm_q4(A.data_ptr(), Wq.data_ptr(), scales.data_ptr(), C.data_ptr(), M, N, K,
                                A.stride(0), C.stride(0), group, zero, ctypes.byref(plan),

@@ -4,7 +4,8 @@ import ctypes
 from . import _lib
 from ._lib import SkConfig, SkPlan
 
-_DTYPES = {"float16": _lib.SK_F16, "float32": _lib.SK_F32, "q4": _lib.SK_Q4, "bfloat16": _lib.SK_BF16}
+_DTYPES = {"float16": _lib.SK_F16, "float32": _lib.SK_F32, "q4": _lib.SK_Q4, "bfloat16": _lib.SK_BF16,
+           "q4_tiled": _lib.SK_Q4_TILED}
 _LAYOUTS = {"nt": _lib.LAYOUT_NT, "nn": _lib.LAYOUT_NN}
 _num_cus = None
 

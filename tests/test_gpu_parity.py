@@ -241,6 +241,43 @@ def test_q4_ragged_shapes_every_kernel(sk, oracle, variant):
     sk.workspace_status()
 
 
+def test_q4_tiled_weights_give_identical_results(sk, oracle):
+    """The tiled weight layout (16-row x 64-byte tiles) hands every lane the bytes it gets from the
+    row-major array, so each tiled kernel must reproduce its row-major twin bit for bit (ordered
+    reduce and data-parallel schedules); the device tiler must write what the host one writes."""
+    import torch
+    rng = np.random.default_rng(91)
+    ran = 0
+    for (M, N, K, zero) in [(1, 1000, 1152, 8), (1, 264, 28672, 8), (1, 2048, 4096, 5), (5, 1000, 1152, 8),
+                            (16, 520, 384, 15), (33, 200, 640, 8), (64, 136, 2048, 3), (16, 4096, 4096, 8)]:
+        A = (rng.random((M, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+        Wq = rng.integers(0, 256, (N, K // 2), dtype=np.uint8)
+        sc = rng.uniform(0.005, 0.02, (N, K // 128)).astype(np.float16)
+        dA, dW, dS = _t(A), _t(Wq), _t(sc)
+        dT = sk.tile_q4(dW)
+        assert torch.equal(dT.cpu(), sk.tile_q4(torch.from_numpy(Wq)))
+        ref = oracle.q4_gemm_ref(A, Wq, sc, 128, zero)
+        C = sk.streamk_q4(dA, dT, dS, zero=zero, tiled=True)           # heuristic plan
+        assert _rel(oracle, C, ref) <= 2e-3 <= TOL
+        for (bm, bn, bk) in Q4_TILES:
+            for variant in (1, 3):
+                for sch in (dict(schedule="dp"), dict(schedule="sk2", fixup="reduce", grid=48)):
+                    cfg = dict(bm=bm, bn=bn, bk=bk, variant=variant, **sch)
+                    try:
+                        pt = sk.make_plan(M, N, K, "q4_tiled", "nt", cfg)
+                        pr = sk.make_plan(M, N, K, "q4", "nt", cfg)
+                    except sk.StreamKError:
+                        continue
+                    Ct = sk.streamk_q4(dA, dT, dS, zero=zero, plan=pt, tiled=True)
+                    Cr = sk.streamk_q4(dA, dW, dS, zero=zero, plan=pr)
+                    assert torch.equal(Ct, Cr), (M, N, K, cfg)
+                    ran += 1
+    assert ran >= 40
+    with pytest.raises(ValueError):
+        sk.streamk_q4(dA, dW, dS, plan=pt)  # a tiled plan with row-major weights
+    sk.workspace_status()
+
+
 def test_q4_matrix_vector_exact_on_integer_data(sk):
     """M = 1, N = K = 8192, A in {-1, 0, 1}, scales 1 (and 0.5): every group sum is an integer
     below 2^24, so the fp32 arithmetic of the matrix-vector kernels is exact and C must equal the

@@ -83,6 +83,29 @@ def test_quantisation_error_is_half_a_step(sk, oracle):
     assert sk.unpack_q4(Wq).numpy().min() >= 1  # -8 is never used
 
 
+def test_tiled_layout_round_trip_and_offsets(sk):
+    """Byte b of row n goes to ((n/16) * (K/128) + b/64) * 1024 + (n%16) * 64 + b%64; rows are padded
+    to a multiple of 16 with zeros; untile is the inverse."""
+    rng = np.random.default_rng(9)
+    for (N, K) in [(16, 128), (40, 384), (1000, 1152), (8, 256)]:
+        Wq = rng.integers(0, 256, (N, K // 2), dtype=np.uint8)
+        T = sk.tile_q4(torch.from_numpy(Wq))
+        n16 = (N + 15) // 16 * 16
+        assert T.shape == (n16, K // 2)
+        flat = T.numpy().reshape(-1)
+        runs = K // 128
+        for (n, b) in [(0, 0), (N - 1, K // 2 - 1), (N // 2, 67 % (K // 2)), (min(17, N - 1), 64 % (K // 2))]:
+            assert flat[((n // 16) * runs + b // 64) * 1024 + (n % 16) * 64 + b % 64] == Wq[n, b]
+        # a tile holds 16 rows x 64 bytes, row by row
+        tiles = flat.reshape(n16 // 16, runs, 16, 64)
+        padded = np.zeros((n16, K // 2), dtype=np.uint8)
+        padded[:N] = Wq
+        assert np.array_equal(tiles, padded.reshape(n16 // 16, 16, runs, 64).transpose(0, 2, 1, 3))
+        assert np.array_equal(sk.untile_q4(T, N).numpy(), Wq)
+    with pytest.raises(sk.StreamKError):
+        sk.tile_q4(torch.zeros(4, 100, dtype=torch.uint8))  # K not a multiple of 128
+
+
 def test_bad_arguments(sk):
     with pytest.raises(sk.StreamKError):
         sk.pack_q4(torch.full((2, 4), 16, dtype=torch.uint8))       # not a nibble
