@@ -658,6 +658,31 @@ def test_wait_gives_up_instead_of_hanging(sk):
     assert (C.float() - C2.float()).abs().max().item() <= 2e-3 * C2.float().abs().max().item()
 
 
+def test_extreme_aspect_ratios(sk, oracle):
+    """Very long and very wide problems: tile bases are 64-bit, offsets inside a tile 32-bit.  Rows
+    and columns sampled from both ends are checked against the fp32 host product; exact {-1,0,1}
+    data gives bit-exact row and column checksums over the whole result."""
+    import torch
+    rng = np.random.default_rng(33)
+    for (M, N, K) in [(300000, 136, 64), (24, 1000000, 128), (1, 2000000, 64), (70000, 70000, 8)]:
+        A = rng.integers(-1, 2, (M, K)).astype(np.float16)
+        B = rng.integers(-1, 2, (N, K)).astype(np.float16)
+        dA, dB = _t(A), _t(B)
+        C = sk.streamk_fp16(dA, dB)
+        rows = np.unique(np.concatenate([np.arange(min(M, 40)), np.arange(max(M - 40, 0), M)]))
+        cols = np.unique(np.concatenate([np.arange(min(N, 40)), np.arange(max(N - 40, 0), N)]))
+        got_r = C[torch.from_numpy(rows).cuda()].cpu().numpy().astype(np.int32)
+        assert np.array_equal(got_r, (A[rows].astype(np.int32) @ B.astype(np.int32).T))
+        got_c = C[:, torch.from_numpy(cols).cuda()].cpu().numpy().astype(np.int32)
+        assert np.array_equal(got_c, (A.astype(np.int32) @ B[cols].astype(np.int32).T))
+        # whole-result checksums: sum_j C[i][j] = A[i] . sum_j B[j]
+        Cd = C.double()
+        assert np.array_equal(Cd.sum(dim=1).cpu().numpy().astype(np.int64), A.astype(np.int64) @ B.astype(np.int64).sum(axis=0))
+        assert np.array_equal(Cd.sum(dim=0).cpu().numpy().astype(np.int64), B.astype(np.int64) @ A.astype(np.int64).sum(axis=0))
+        del C, Cd, dA, dB
+    sk.workspace_status()
+
+
 def test_bad_calls_are_refused(sk):
     import torch
     A = torch.zeros(64, 128, dtype=torch.float16, device="cuda")
