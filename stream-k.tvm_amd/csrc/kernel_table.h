@@ -101,6 +101,10 @@ struct KernelInfo {
   X(104, 1, 1, 2, 2, 0, 2, 0)    \
   X(105, 1, 1, 1, 1, 0, 4, 1)    \
   X(106, 1, 1, 4, 1, 0, 4, 1)    \
+  X(107, 1, 1, 2, 4, 0, 2, 0)    \
+  X(108, 1, 1, 4, 2, 0, 2, 0)    \
+  X(109, 2, 1, 4, 2, 0, 2, 0)    \
+  X(110, 4, 1, 4, 2, 0, 2, 0)    \
   X(120, 1, 1, 4, 1, 1, 4, 0)    \
   X(121, 2, 1, 4, 1, 1, 2, 0)    \
   X(122, 4, 1, 4, 1, 1, 2, 0)    \
@@ -111,7 +115,9 @@ struct KernelInfo {
   X(127, 1, 2, 1, 1, 1, 4, 1)    \
   X(128, 1, 2, 2, 1, 1, 4, 1)    \
   X(129, 1, 4, 1, 1, 1, 2, 1)    \
-  X(130, 1, 2, 1, 2, 1, 4, 1)
+  X(130, 1, 2, 1, 2, 1, 4, 1)    \
+  X(131, 1, 1, 2, 4, 1, 2, 0)    \
+  X(132, 1, 1, 4, 2, 1, 2, 0)
 
 // M == 1 Q4 matrix-vector kernels (variant 2):  X(id, NB, WN, RK, DEPTH, KMAX)
 // KMAX is the largest K range one segment may span (A is kept in LDS for the whole segment).

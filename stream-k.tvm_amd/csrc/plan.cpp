@@ -78,6 +78,13 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
         if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].variant == 2 && t[i].bn == 16 &&
             t[i].bk == 1024 && accepts_shape(t[i], M, K))
           return &t[i];
+    // 2 <= M <= 16 with Q4 weights: eight waves per CTA (two per SIMD cover each other's waits),
+    // 32 weight rows, K split over four waves
+    if (dtype == SK_Q4 && M > 1 && M <= 16 && want_variant < 0)
+      for (int i = 0; i < n; ++i)
+        if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].variant == 0 && t[i].bm == 16 &&
+            t[i].bn == 32 && t[i].bk == 1024 && accepts_shape(t[i], M, K))
+          return &t[i];
     // M == 1 with fp16 weights: the same structure, K split over four waves
     if (dtype == SK_F16 && M == 1 && want_variant < 0)
       for (int i = 0; i < n; ++i)

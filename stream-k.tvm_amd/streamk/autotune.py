@@ -25,7 +25,7 @@ USER_CACHE_ENV = "STREAMK_TUNE_CACHE"
 _TILES_F16 = [(256, 256, 64), (128, 128, 64), (128, 256, 64), (256, 128, 64), (64, 64, 64), (128, 64, 64),
               (64, 128, 64)]
 _SKINNY_F16 = [(16, 64, 128), (32, 64, 128), (64, 64, 128), (16, 16, 512), (16, 32, 256), (16, 16, 128),
-               (16, 16, 1024), (16, 32, 512), (16, 16, 256)]
+               (16, 16, 1024), (16, 32, 512), (16, 16, 256), (16, 64, 256), (32, 64, 256), (64, 64, 256)]
 _SKINNY_Q4 = [(16, 64, 256), (32, 64, 256), (64, 64, 256), (16, 16, 1024), (16, 32, 512), (16, 16, 256),
               (16, 32, 256), (16, 32, 1024), (16, 16, 2048), (16, 64, 512), (16, 16, 512)]
 

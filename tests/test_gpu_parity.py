@@ -64,6 +64,7 @@ TILE_CONFIGS = [
 SKINNY_CONFIGS = [
     dict(bm=16, bn=64, bk=128), dict(bm=32, bn=64, bk=128), dict(bm=64, bn=64, bk=128),
     dict(bm=16, bn=16, bk=512), dict(bm=16, bn=32, bk=256),
+    dict(bm=16, bn=32, bk=512, variant=1), dict(bm=16, bn=64, bk=256), dict(bm=32, bn=64, bk=256), dict(bm=64, bn=64, bk=256),
 ]
 
 
@@ -198,14 +199,14 @@ def test_cfg4_q4_gemm(sk, oracle, M):
     W = sk.dequant_q4(dW, dS).cpu().numpy()
     assert np.array_equal(W.view(np.uint16), oracle.dequant_q4(Wq, sc, 128, 8).view(np.uint16))
     for cfg in (dict(fixup="reduce"), dict(fixup="atomic"), dict(schedule="dp"),
-                dict(bm=16, bn=16, bk=1024), dict(bm=16, bn=32, bk=512), dict(schedule="basic", grid=700)):
+                dict(bm=16, bn=16, bk=1024), dict(bm=16, bn=32, bk=512), dict(schedule="basic", grid=256)):
         C = sk.streamk_q4(dA, dW, dS, **cfg)
         assert _rel(oracle, C, ref) <= 2e-3 <= TOL, cfg
     sk.workspace_status()
 
 
 Q4_TILES = [(16, 64, 256), (16, 32, 512), (16, 16, 1024), (16, 128, 256), (16, 64, 512), (16, 32, 256),
-            (16, 16, 512), (16, 16, 256), (32, 64, 256), (64, 64, 256)]
+            (16, 16, 512), (16, 16, 256), (32, 64, 256), (64, 64, 256), (16, 32, 1024)]
 
 
 @pytest.mark.parametrize("variant", [1, 2, 3], ids=["general", "row1", "gemv"])
