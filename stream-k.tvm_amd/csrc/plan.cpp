@@ -101,9 +101,15 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
     if (q4) return nullptr;
   }
   if (dtype == SK_F32) {
+    // 32 x 256 tiles for M <= 32 (a quarter of the wasted rows of a 128-row tile), else 128 x 128
+    const int want_bm = M <= 32 ? 32 : 128;
+    const KernelInfo *any = nullptr;
     for (int i = 0; i < n; ++i)
-      if (t[i].dtype == SK_F32 && t[i].layout == layout) return &t[i];
-    return nullptr;
+      if (t[i].dtype == SK_F32 && t[i].layout == layout) {
+        if (t[i].bm == want_bm) return &t[i];
+        if (!any) any = &t[i];
+      }
+    return any;
   }
   // 256x256 tiles when they fill the device; else 128x128, else 64x64.  The smaller tiles run one
   // or two waves per SIMD, where the four-stage (BK = 32) pipeline hides the load latency better;

@@ -1,4 +1,5 @@
-// fp32 tile arithmetic: 128 x 128 x 16 CTA tile, 2 x 2 waves, v_mfma_f32_32x32x2_f32.
+// fp32 tile arithmetic: BM x BN x 16 CTA tile (128 x 128 on 2 x 2 waves; 32 x 256 on 1 x 4 waves for small M),
+// v_mfma_f32_32x32x2_f32.
 //
 // Replaces the T.gemm of the reference's fp32 kernel (streamk_fp32.py:109-125).  B may be [K,N]
 // (the reference's layout, streamk_fp32.py:74) or [N,K].
@@ -19,12 +20,13 @@ struct GemmArgsF32 {
   int64_t lda, ldb, ldc;
 };
 
-template <bool B_KN_>
+template <bool B_KN_, int BM_ = 128, int BN_ = 128, int WM_ = 2, int WN_ = 2>
 struct TileF32 {
   typedef GemmArgsF32 Args;
   static constexpr bool B_KN = B_KN_;
-  static constexpr int BM = 128, BN = 128, BK = 16, WM = 2, WN = 2;
-  static constexpr int NT = 256, TM = 2, TN = 2, WTM = 64, WTN = 64;
+  static constexpr int BM = BM_, BN = BN_, BK = 16, WM = WM_, WN = WN_;
+  static constexpr int NT = 256, TM = BM / (WM * 32), TN = BN / (WN * 32), WTM = TM * 32, WTN = TN * 32;
+  static_assert(WM * WN == 4 && BM % (WM * 32) == 0 && BN % (WN * 32) == 0 && BN % 64 == 0, "tile shape");
   static constexpr int LDA = BK + 4;                 // floats per LDS row of A (and of B when [N,K])
   static constexpr int LDB = B_KN ? BN + 8 : BK + 4; // floats per LDS row of B
   static constexpr int A_STAGE = BM * LDA, B_STAGE = B_KN ? BK * LDB : BN * LDB, STAGE = A_STAGE + B_STAGE;
@@ -32,7 +34,10 @@ struct TileF32 {
   static constexpr int TILE_ELEMS = BM * BN, NV4 = TM * TN * 4;
   static constexpr int CTAS_PER_CU = 2, WAVES_PER_EU = 2;
   static constexpr bool COHERENT_PARTIALS = false;
-  static constexpr int A_LOADS = BM * BK / 4 / NT, B_LOADS = BN * BK / 4 / NT;  // 16-byte loads per thread
+  // 16-byte loads per thread: a pass of the 256 threads covers 64 rows of 16 K-values (A, and B as
+  // [N,K]) or 1024 / BN K-rows of BN values (B as [K,N])
+  static constexpr int A_LOADS = (BM + 63) / 64, B_LOADS = BN * BK / 4 / NT;
+  static constexpr int B_CPR = BN / 4, B_RPP = NT / B_CPR;  // [K,N]: chunks per K-row, K-rows per pass
 
   struct Acc {
     floatx16 c[TM][TN];
@@ -53,7 +58,7 @@ struct TileF32 {
     const int rows_a = min(BM, a.M - pm * BM), cols_b = min(BN, a.N - pn * BN);
     const BufferRsrc rsrc_a = make_rsrc(a.A + (int64_t)pm * BM * a.lda, (uint32_t)(rows_a * a.lda * 4));
     const int a_row = tid / 4, a_c = tid % 4;  // 4 chunks of 4 floats per K-row of 16
-    const uint32_t voff_a = (uint32_t)(a_row * a.lda + a_c * 4) * 4;
+    const uint32_t voff_a = (BM % 64 == 0 || a_row < BM) ? (uint32_t)(a_row * a.lda + a_c * 4) * 4 : OOB_OFFSET;
     const uint32_t pass_a = (uint32_t)(64 * a.lda * 4);
     BufferRsrc rsrc_b;
     uint32_t voff_b, pass_b, kstep_b;
@@ -66,9 +71,9 @@ struct TileF32 {
       b_st = a_row * LDB + a_c * 4;
     } else {
       rsrc_b = make_rsrc(a.B + (int64_t)pn * BN, (uint32_t)(((int64_t)(a.K - 1) * a.ldb + cols_b) * 4));
-      const int k_row = tid / 32, c = tid % 32;  // 32 chunks per K-row of 128 floats, 8 rows per pass
+      const int k_row = tid / B_CPR, c = tid % B_CPR;
       voff_b = (c * 4 < cols_b) ? (uint32_t)(k_row * a.ldb + c * 4) * 4 : OOB_OFFSET;
-      pass_b = (uint32_t)(8 * a.ldb * 4);
+      pass_b = (uint32_t)(B_RPP * a.ldb * 4);
       kstep_b = (uint32_t)(BK * a.ldb * 4);
       b_st = k_row * LDB + c * 4;
     }
@@ -96,10 +101,11 @@ struct TileF32 {
     for (int it = 0; it < n; ++it) {
       float *st = lds + (it & 1) * STAGE;
 #pragma unroll
-      for (int i = 0; i < A_LOADS; ++i) *reinterpret_cast<uint4v *>(st + a_st + i * 64 * LDA) = ra[i];
+      for (int i = 0; i < A_LOADS; ++i)
+        if (BM % 64 == 0 || a_row + i * 64 < BM) *reinterpret_cast<uint4v *>(st + a_st + i * 64 * LDA) = ra[i];
 #pragma unroll
       for (int i = 0; i < B_LOADS; ++i)
-        *reinterpret_cast<uint4v *>(st + A_STAGE + b_st + i * (B_KN ? 8 * LDB : 64 * LDB)) = rb[i];
+        *reinterpret_cast<uint4v *>(st + A_STAGE + b_st + i * (B_KN ? B_RPP * LDB : 64 * LDB)) = rb[i];
       __syncthreads();
       if (it + 1 < n) load_global(k0 + it + 1);
 #pragma unroll
@@ -128,7 +134,7 @@ struct TileF32 {
     __syncthreads();
   }
 
-  // acc.c[i][j][r] = C[pm*BM + wm*64 + i*32 + 8*(r/4) + 4*(lane/32) + r%4][pn*BN + wn*64 + j*32 + lane%32]
+  // acc.c[i][j][r] = C[pm*BM + wm*WTM + i*32 + 8*(r/4) + 4*(lane/32) + r%4][pn*BN + wn*WTN + j*32 + lane%32]
   static __device__ __forceinline__ void store_c(const Args &a, const Acc &acc, int pm, int pn, char *) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;

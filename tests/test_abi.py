@@ -64,6 +64,8 @@ def test_schedules(sk):
     one = sk.make_plan(3000, 5120, 12288, "float16", "nt", schedule="sk1", **kw)
     assert (one.total_tiles, one.streamk_tiles, one.blocking_tiles) == (960, 192, 768)
     f32 = sk.make_plan(16, 16384, 8192, "float32", "nn", cus=256)
+    assert (f32.bm, f32.bn, f32.bk, f32.kernel_id) == (32, 256, 16, 202)  # M <= 32: the 32-row tile
+    f32 = sk.make_plan(256, 256, 1024, "float32", "nn", cus=256)
     assert (f32.bm, f32.bn, f32.bk, f32.kernel_id) == (128, 128, 16, 200)
     auto = sk.make_plan(8192, 8192, 8192, "float16", "nt", cus=256)
     assert (auto.bm, auto.bn, auto.schedule, auto.streamk_tiles) == (256, 256, 1, 0)

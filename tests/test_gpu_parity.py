@@ -564,6 +564,19 @@ def test_fp32_cfg1_and_fixture(sk, oracle, golden_dir, fixup):
     Bi = rng.integers(-4, 5, (1032, 388)).astype(np.float32)
     C = sk.streamk_fp32(_t(Ai), _t(Bi), schedule="basic", fixup=fixup, grid=9).cpu().numpy()
     assert np.array_equal(C, Ai @ Bi)
+    # the 32 x 256 tile (the plan for M <= 32) and the 128 x 128 one on the same ragged problems, both layouts
+    for (M, N, K) in [(16, 1000, 1032), (40, 388, 260), (1, 264, 72), (260, 520, 1032)]:
+        Ai = rng.integers(-4, 5, (M, K)).astype(np.float32)
+        Bi = rng.integers(-4, 5, (K, N)).astype(np.float32)
+        Ar = rng.random((M, K), dtype=np.float32) * 2 - 1
+        for (bm, bn) in ((32, 256), (128, 128)):
+            for sch in (dict(schedule="dp"), dict(schedule="basic", fixup=fixup, grid=7), dict(schedule="sk2", fixup=fixup, grid=3)):
+                C = sk.streamk_fp32(_t(Ai), _t(Bi), bm=bm, bn=bn, **sch).cpu().numpy()
+                assert np.array_equal(C, Ai @ Bi), (M, N, K, bm, bn, sch)
+                C = sk.streamk_fp32(_t(Ai), _t(np.ascontiguousarray(Bi.T)), layout="nt", bm=bm, bn=bn, **sch).cpu().numpy()
+                assert np.array_equal(C, Ai @ Bi), (M, N, K, bm, bn, sch, "nt")
+                C = sk.streamk_fp32(_t(Ar), _t(Bi), bm=bm, bn=bn, **sch).cpu().numpy()
+                assert oracle.max_abs_rel(C, Ar.astype(np.float64) @ Bi.astype(np.float64)) <= 1e-5
     sk.workspace_status()
 
 
@@ -573,9 +586,13 @@ def test_fp32_reference_shape(sk, oracle):
     rng = np.random.default_rng(3)
     A = rng.random((16, 8192), dtype=np.float32) * 2 - 1
     B = rng.random((8192, 16384), dtype=np.float32) * 2 - 1
-    C = sk.streamk_fp32(_t(A), _t(B)).cpu().numpy()
+    plan = sk.make_plan(16, 16384, 8192, "float32", "nn")
+    assert (plan.bm, plan.bn) == (32, 256)
+    C = sk.streamk_fp32(_t(A), _t(B), plan=plan).cpu().numpy()
     cols = slice(4000, 4512)
     ref = A.astype(np.float64) @ B[:, cols].astype(np.float64)
+    assert oracle.max_abs_rel(C[:, cols], ref) <= 1e-5
+    C = sk.streamk_fp32(_t(A), _t(B), bm=128, bn=128).cpu().numpy()
     assert oracle.max_abs_rel(C[:, cols], ref) <= 1e-5
     sk.workspace_status()
 
