@@ -70,7 +70,8 @@ typedef enum sk_dtype {
   SK_F32 = 1,
   SK_Q4 = 2,       /* fp16 A, packed nibbles [N, K/2] row-major */
   SK_BF16 = 3,
-  SK_Q4_TILED = 4  /* fp16 A, packed nibbles in 16-row x 64-byte tiles (sk_q4_tile_host / sk_q4_tile) */
+  SK_Q4_TILED = 4, /* fp16 A, packed nibbles in 16-row x 64-byte tiles (sk_q4_tile_host / sk_q4_tile) */
+  SK_F8E4M3 = 5    /* A and B one byte per element, OCP e4m3 (bias 7, no infinities, NaN = S.1111.111); C fp16 */
 } sk_dtype;
 
 /* Tunables; a zero field means "choose for me".  Replaces the module-level constants and
@@ -81,8 +82,9 @@ typedef struct sk_config {
   int32_t grid;           /* persistent CTAs; the reference's total_sm (streamk_fp32.py:17) */
   int32_t schedule;       /* sk_schedule */
   int32_t fixup;          /* sk_fixup */
-  int32_t raster;         /* 0: row-major tile order (streamk_fp32.py:106-107); g>0: tiles walk g
-                             rows down before stepping one column (triton_impl.py:14-28) */
+  int32_t raster;         /* g>0: tiles walk g rows down before stepping one column (triton_impl.py:14-28);
+                             1 is the reference's row-major order (streamk_fp32.py:106-107); 0: choose
+                             (8 for the 16-bit and fp8 tile kernels, row-major otherwise) */
   int32_t spin_limit;     /* REDUCE fix-up: polls of a peer flag before giving up; 0 = default */
   int32_t reserved[4];    /* reserved[0]: 0 = preferred kernel variant of the tile, v > 0 = variant v - 1
                              (implementation alternatives of one tile shape, for the autotuner);
@@ -157,6 +159,15 @@ int sk_gemm_f16(const void *A, const void *B, void *C, int64_t M, int64_t N, int
  * the tile kernels with the bfloat16 form of the MFMA.  Requirements as for sk_gemm_f16. */
 int sk_gemm_bf16(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
                  int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws, size_t ws_bytes, void *stream);
+
+/* fp8 operands: A [M,K] and B [N,K] (NT only) hold OCP e4m3 bytes, C is fp16, accumulation fp32;
+ * the plan is made with dtype SK_F8E4M3 (its bk counts fp8 elements).  No counterpart in the
+ * reference's scripts; its Triton comparator takes whatever dtype its inputs have
+ * (triton.streamk/first_wave.py:123 picks the accumulator type from them).  Same partitioner,
+ * fix-ups and workspace rules as sk_gemm_f16.  K, lda and ldb multiples of 16; A and B 16-byte
+ * aligned.  Values are not scaled: a caller that keeps per-tensor scales applies them to C. */
+int sk_gemm_f8(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
+               int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws, size_t ws_bytes, void *stream);
 
 /* fp32 GEMM (fp32 MFMA, fp32 out).  Replaces tl_mod(A, B, C) of streamk_fp32.py:197-202. */
 int sk_gemm_f32(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,

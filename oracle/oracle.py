@@ -212,3 +212,23 @@ def q4_gemm_ref(A, Wq, scales, group=128, zero=8):
     """fp32 host product of A [M,K] with the dequantised weights [N,K]^T."""
     W = dequant_q4(Wq, scales, group, zero).astype(np.float32)
     return np.asarray(A, dtype=np.float32) @ W.T
+
+
+# ------------------------------------------------------------------ fp8 (OCP e4m3)
+def f8e4m3_decode(u8):
+    """Bytes -> float32 values of the OCP 8-bit floating point format E4M3 (OCP 8-bit Floating Point
+    Specification (OFP8) rev 1.0, section 5: sign, 4 exponent bits with bias 7, 3 mantissa bits; no
+    infinities; S.1111.111 is NaN; exponent 0 is subnormal, m * 2^-9).  Not in the reference's scripts,
+    which stop at fp16; its Triton comparator takes the dtype of its inputs (triton.streamk/first_wave.py:123)."""
+    u8 = np.asarray(u8, dtype=np.uint8)
+    e = ((u8 >> 3) & 15).astype(np.int32)
+    m = (u8 & 7).astype(np.float32)
+    mag = np.where(e == 0, np.ldexp(m, -9), np.ldexp(8.0 + m, e - 10)).astype(np.float32)
+    mag = np.where((e == 15) & ((u8 & 7) == 7), np.float32(np.nan), mag)
+    return np.where(u8 >> 7 == 1, -mag, mag).astype(np.float32)
+
+
+def f8_gemm_ref(A_u8, B_u8):
+    """float64 host product A [M,K] x B [N,K]^T of e4m3 bytes (each product of two e4m3 values is exact in
+    float32; the sum is taken in float64)."""
+    return f8e4m3_decode(A_u8).astype(np.float64) @ f8e4m3_decode(B_u8).astype(np.float64).T

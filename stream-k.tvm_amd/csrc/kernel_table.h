@@ -24,7 +24,7 @@ struct KernelInfo {
   int variant;  // tile kernels -- 0: registers -> padded LDS rows; 1: direct global -> LDS loads,
                 // swizzled rows; 2: as 1 with four waves per CTA (one per SIMD, accumulators in AGPRs);
                 // 3: as 1 with BK = 32 and four LDS stages (loads three iterations ahead);
-                // 4: as 1 with 16x16x32 MFMAs; 5: as 3 with 16x16x32 MFMAs
+                // 4: as 1 with 16x16x32 MFMAs; 5: as 3 with 16x16x32 MFMAs; 6: as 1 for fp8 operands (32x32x64 MFMAs)
                 // small-M kernels -- 0: up to 16*MB rows of A; 1: M == 1; 2: M == 1, matrix-vector on 4x4x4 MFMA
   int bm, bn, bk;  // CTA tile; bk is the K extent of one CTA iteration
   int threads;
@@ -176,6 +176,13 @@ struct KernelInfo {
   X(63, 64, 64, 2, 2, 32, false)   \
   X(64, 256, 256, 2, 4, 64, true)  \
   X(65, 128, 128, 2, 2, 64, true)
+
+// fp8 (OCP e4m3) operands, fp16 C, NT layout; bk counts fp8 elements (variant 6):  X(id, BM, BN, WM, WN)
+#define SK_TILE_F8_KERNELS(X) \
+  X(70, 256, 256, 2, 4)       \
+  X(71, 128, 128, 2, 2)       \
+  X(72, 128, 256, 2, 4)       \
+  X(73, 256, 128, 4, 2)
 
 const KernelInfo *kernel_table(int *count);
 const KernelInfo *kernel_by_id(int id);

@@ -11,7 +11,7 @@
 
 namespace sk {
 
-static KernelInfo g_table[128];
+static KernelInfo g_table[192];
 static int g_count = -1;
 
 int tile_kernel_infos(KernelInfo *out, int max);
@@ -20,9 +20,9 @@ int f32_kernel_infos(KernelInfo *out, int max);
 
 const KernelInfo *kernel_table(int *count) {
   if (g_count < 0) {
-    int n = tile_kernel_infos(g_table, 128);
-    n += skinny_kernel_infos(g_table + n, 128 - n);
-    n += f32_kernel_infos(g_table + n, 128 - n);
+    int n = tile_kernel_infos(g_table, 192);
+    n += skinny_kernel_infos(g_table + n, 192 - n);
+    n += f32_kernel_infos(g_table + n, 192 - n);
     g_count = n;
   }
   if (count) *count = g_count;
@@ -142,8 +142,10 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
                             int num_cus, sk_plan *out) {
   if (!out) return SK_ERR_NULL;
   if (M <= 0 || N <= 0 || K <= 0 || M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return SK_ERR_SHAPE;
-  if (dtype != SK_F16 && dtype != SK_F32 && dtype != SK_Q4 && dtype != SK_BF16 && dtype != SK_Q4_TILED)
+  if (dtype != SK_F16 && dtype != SK_F32 && dtype != SK_Q4 && dtype != SK_BF16 && dtype != SK_Q4_TILED &&
+      dtype != SK_F8E4M3)
     return SK_ERR_CONFIG;
+  if (dtype == SK_F8E4M3 && layout != SK_LAYOUT_NT) return SK_ERR_CONFIG;
   if (layout != SK_LAYOUT_NT && layout != SK_LAYOUT_NN) return SK_ERR_CONFIG;
   if (num_cus <= 0) return SK_ERR_DEVICE;
   const KernelInfo *k = pick_kernel(M, N, K, dtype, layout, cfg, num_cus);
@@ -235,6 +237,10 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
   out->spin_limit = cfg && cfg->spin_limit > 0 ? cfg->spin_limit : (1 << 22);
   out->raster = cfg ? cfg->raster : 0;
   if (out->raster < 0) return SK_ERR_CONFIG;
+  // default tile order of the LDS-tiled 16-bit and fp8 kernels: groups of 8 tile rows.  Concurrent CTAs
+  // then share B tiles as well as A tiles in the L2s: 0-20 % faster than row-major order on every shape
+  // measured (no effect on the fp32 kernels, which keep the reference's order).
+  if (out->raster == 0 && k->family == FAMILY_TILE && dtype != SK_F32 && out->num_block_m > 1) out->raster = 8;
 
   // workspace: status block, fixed-size flag area, fp32 partial tiles
   int64_t ws = 0;

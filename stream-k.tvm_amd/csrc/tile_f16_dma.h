@@ -55,9 +55,21 @@ struct LdsArray {
 // its power limit.  The accumulator is then kept as 16x16 blocks of four registers: lane l holds
 // C[16*ii + l%16][16*jj + 4*(l/16) + e] of block (ii, jj).  A K-step covers 32 K-values: lane
 // group g = l/16 takes 16-byte chunk 4*kk + g of its row.
-template <int BM_, int BN_, int WM_, int WN_, bool B_KN_ = false, int BK_ = 64, bool MFMA16_ = false, bool BF16_ = false>
+//
+// F8_ (1: e4m3, 2: e5m2, both OCP): A and B hold one byte per element and C is fp16.  The launcher
+// passes K and the leading dimensions of A and B in 16-bit units (half the element counts), so the
+// data movement is that of the fp16 kernel: an LDS row of 128 bytes is 128 K-values, one iteration.
+// The arithmetic is v_mfma_f32_32x32x64_f8f6f4 (twice the FLOP of the 16-bit forms per byte of
+// operand) into the 32x32 accumulator blocks of the fp16 kernel.  Lane (r = l%32, g = l/32) hands
+// the instruction, for K-step s of 64 bytes, chunks 4s + g and 4s + 2 + g of row r as its 32-byte
+// operand.  Which K-values a lane's bytes stand for does not matter as long as A and B agree: the
+// instruction pairs byte b of lane group g of one operand with the same byte of the other.
+template <int BM_, int BN_, int WM_, int WN_, bool B_KN_ = false, int BK_ = 64, bool MFMA16_ = false, bool BF16_ = false,
+          int F8_ = 0>
 struct TileF16NTDma {
   static constexpr bool B_KN = B_KN_, MFMA16 = MFMA16_;
+  static constexpr int F8 = F8_;
+  static_assert(F8_ == 0 || (!MFMA16_ && !B_KN_ && BK_ == 64 && !BF16_), "fp8: NT layout, two stages");
   // BF16_: operands and C are bfloat16 (same 16-bit data movement; v_mfma_f32_16x16x32_bf16; C rounded to
   // nearest even with v_cvt_pk_bf16_f32)
   static_assert(!BF16_ || MFMA16_, "bfloat16 exists in the 16x16x32 form");
@@ -100,6 +112,7 @@ struct TileF16NTDma {
   static_assert((A_BYTES / 1024) % NW == 0 && (B_BYTES / 1024) % NW == 0, "DMA groups must divide over the waves");
   static_assert(NW % NSTAGE == 0, "a wave must keep to row groups of one parity; patches per stage");
   static_assert(PATCH_ROWS % 32 == 0, "epilogue pass must hold whole 32-row blocks");
+  static_assert(F8_ == 0 || TM % 2 == 0, "fp8: the wave tile's rows are processed in two halves");
 
   typedef TileF16NT<BM_, BN_, 64, WM_, WN_> Base;  // shares the accumulator type and the partials
   // 16x16x32: the accumulator is kept as 16x16 blocks of four registers (block (ii, jj): lane l holds
@@ -133,6 +146,17 @@ struct TileF16NTDma {
     for (int g = 0; g < READS; ++g) {
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);
+    }
+  }
+
+  // scheduling hint for MFMAS matrix instructions with READS LDS reads spread over them
+  template <int MFMAS, int READS>
+  static __device__ __forceinline__ void interleave8() {
+    if (READS % MFMAS) __builtin_amdgcn_sched_group_barrier(0x100, READS % MFMAS, 0);
+#pragma unroll
+    for (int g = 0; g < MFMAS; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x100, READS / MFMAS, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
     }
   }
 
@@ -335,7 +359,105 @@ struct TileF16NTDma {
           if (m * CH / NMF == x) mfma_one16(1, bcur, 1, m);
       }
     };
-    if constexpr (NSTAGE == 4 && MFMA16) {
+    // fp8: 32-byte fragments, A double-buffered per half of the wave tile's rows, B per K-step
+    typedef int intx8 __attribute__((ext_vector_type(8)));
+    constexpr int FA8 = TM / 2 > 0 ? TM / 2 : 1;
+    intx8 fa8[2][FA8], fb8[2][TN];
+    auto read8 = [&](const char *p0, const char *p1) {
+      union { uint4v q[2]; intx8 v; } u;
+      u.q[0] = *reinterpret_cast<const uint4v *>(p0);
+      u.q[1] = *reinterpret_cast<const uint4v *>(p1);
+      return u.v;
+    };
+    auto read_a8_one = [&](const char *st, int buf, int s, int mh, int i) {
+      const int off = (mh * FA8 + i) * 32 * ROW_BYTES;
+      fa8[buf][i] = read8(st + rd_a[(2 * s) % KSTEPS] + off, st + rd_a[(2 * s + 1) % KSTEPS] + off);
+    };
+    auto read_b8_one = [&](const char *st, int buf, int s, int j) {
+      const int off = j * 32 * ROW_BYTES;
+      fb8[buf][j] = read8(st + rd_b[(2 * s) % KSTEPS] + off, st + rd_b[(2 * s + 1) % KSTEPS] + off);
+    };
+    auto read_a8 = [&](const char *st, int buf, int s, int mh) {
+#pragma unroll
+      for (int i = 0; i < FA8; ++i) read_a8_one(st, buf, s, mh, i);
+    };
+    auto read_b8 = [&](const char *st, int buf, int s) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j) read_b8_one(st, buf, s, j);
+    };
+    auto mfma_one8 = [&](int abuf, int bbuf, int mh, int idx) {
+      if constexpr (F8_ != 0) {
+        const int i = idx / TN, j = idx % TN, ii = mh * FA8 + i;
+        acc.c[ii][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb8[bbuf][j], fa8[abuf][i], acc.c[ii][j], F8_ - 1,
+                                                                       F8_ - 1, 0, 0, 0, 0);
+      }
+    };
+    auto mfma_half8 = [&](int abuf, int bbuf, int mh) {
+#pragma unroll
+      for (int idx = 0; idx < FA8 * TN; ++idx) mfma_one8(abuf, bbuf, mh, idx);
+    };
+    // the half-step behind the barrier, sliced like tail16: loads of K-iteration kt_next into `cur`,
+    // the first fragments of `nxt` (A into fa8[0], B into fb8[0]) and the MFMAs of (K-step 1, second
+    // half of the rows)
+    auto tail8 = [&](char *cur, const char *nxt, int kt_next, bool dead) {
+      const bool oob = dead || (kt_next == tail_kt && kt_next * BK + my_chunk * 8 >= a.K);
+      const uint32_t va = oob ? OOB_OFFSET : voff_a, vb = oob ? OOB_OFFSET : voff_b;
+      constexpr int CH = DMA_PER_WAVE, NRD = FA8 + TN, NMF = FA8 * TN;
+#pragma unroll
+      for (int x = 0; x < CH; ++x) {
+#pragma unroll
+        for (int r = 0; r < NRD; ++r)
+          if (r * CH / NRD == x) {
+            if (r < FA8)
+              read_a8_one(nxt, 0, 0, 0, r);
+            else
+              read_b8_one(nxt, 0, 0, r - FA8);
+          }
+        if (x < A_DMA) {
+          const int g = wave + x * NW;
+          dma_load_16(rsrc_a, lds_address(cur) + g * 1024, va, (uint32_t)kt_next * (BK * 2) + g * grp_a);
+        } else {
+          const int g = wave + (x - A_DMA) * NW;
+          dma_load_16(rsrc_b, lds_address(cur) + A_BYTES + g * 1024, vb, (uint32_t)kt_next * kstep_b + g * grp_b);
+        }
+#pragma unroll
+        for (int m = 0; m < NMF; ++m)
+          if (m * CH / NMF == x) mfma_one8(1, 1, 1, m);
+      }
+    };
+    if constexpr (F8_ != 0) {
+      // one K-iteration (128 K-values) on stage `cur`: two K-steps of 64, each in two halves of the
+      // wave tile's rows.  Entering, fa8[0] / fb8[0] hold the fragments of (K-step 0, first half).
+      auto iteration8 = [&](char *cur, char *nxt, int it) {
+        read_a8(cur, 1, 0, 1);
+        read_b8(cur, 1, 1);
+        mfma_half8(0, 0, 0);
+        interleave8<FA8 * TN, 2 * (FA8 + TN)>();
+        read_a8(cur, 0, 1, 0);
+        mfma_half8(1, 0, 1);
+        interleave8<FA8 * TN, 2 * FA8>();
+        read_a8(cur, 1, 1, 1);
+        mfma_half8(0, 1, 0);
+        interleave8<FA8 * TN, 2 * FA8>();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        wait_dma_then_barrier<0>();
+        tail8(cur, nxt, k0 + it + 2, it + 2 >= n);
+      };
+      char *s0 = stage(0), *s1 = stage(1);
+      issue_dma(s0, k0);
+      wait_dma_then_barrier<0>();
+      if (n > 1) issue_dma(s1, k0 + 1);
+      read_a8(s0, 0, 0, 0);
+      read_b8(s0, 0, 0);
+      int it = 0;
+      for (; it + 1 < n; it += 2) {
+        iteration8(s0, s1, it);
+        iteration8(s1, s0, it + 1);
+      }
+      if (it < n) iteration8(s0, s1, it);
+      // the empty loads of the last two iterations still write LDS
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    } else if constexpr (NSTAGE == 4 && MFMA16) {
       // BK = 32 is one K-step: two half-steps per iteration.  Entering, fa[0] holds the first half
       // of the A rows and fb[par] the B fragments of stage `cur` (par = iteration parity).
       auto iteration4 = [&](char *cur, char *nxt, int it, int par) {

@@ -56,7 +56,7 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
     schedule, grid and fix-up."""
     cus = cus or _plan.num_cus()
     out = []
-    if dtype == "q4" or M <= 64:
+    if dtype == "q4" or (M <= 64 and dtype != "float8_e4m3"):
         tiles = _SKINNY_Q4 if dtype == "q4" else _SKINNY_F16
         for (bm, bn, bk) in tiles:
             if bm < M and not (bm == 16 and M <= 16):
@@ -75,7 +75,7 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
                 variants += ((5, bk),)  # two-stage with 16x16x32 MFMAs
             if (bm, bn) == (64, 64):
                 variants += ((1, bk),)
-            for (variant, vbk), raster in itertools.product(variants, (0, 8)):
+            for (variant, vbk), raster in itertools.product(variants, (1, 8)):
                 base = dict(bm=bm, bn=bn, bk=vbk, variant=variant, raster=raster)
                 out.append(dict(base, schedule="dp"))
                 grids = (None,) if bm * bn >= 256 * 256 else (None, cus)
@@ -84,6 +84,14 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
                 # fixed split-K, the fallback when there are fewer tiles than CUs
                 if -(-M // bm) * -(-N // bn) < cus:
                     out.extend(dict(base, schedule="splitk", fixup=fixup) for fixup in ("reduce", "atomic"))
+    if dtype == "float8_e4m3":
+        for (bm, bn), raster in itertools.product(((256, 256), (256, 128), (128, 256), (128, 128)), (1, 8)):
+            base = dict(bm=bm, bn=bn, raster=raster)
+            out.append(dict(base, schedule="dp"))
+            for sched, fixup in itertools.product(("sk2", "sk1", "basic"), ("reduce", "atomic")):
+                out.append(dict(base, schedule=sched, fixup=fixup))
+            if -(-M // bm) * -(-N // bn) < cus:
+                out.extend(dict(base, schedule="splitk", fixup=fixup) for fixup in ("reduce", "atomic"))
     return out
 
 
@@ -128,7 +136,7 @@ def autotune(M, N, K, dtype="float16", layout="nt", *, configs=None, warmup=5, r
     A = (torch.rand(M, K, generator=g) * 2 - 1).half().to(dev)
     C = torch.empty(M, N, dtype=torch.float16, device=dev)
     weights = weights or ("hbm" if M <= 64 else "warm")
-    wbytes = N * K // 2 if dtype == "q4" else N * K * 2
+    wbytes = N * K // 2 if dtype == "q4" else (N * K if dtype == "float8_e4m3" else N * K * 2)
     copies = 1 if weights == "warm" else max(2, min(rep, -(-(512 << 20) // wbytes)))
     turn = [0]
 
@@ -141,6 +149,17 @@ def autotune(M, N, K, dtype="float16", layout="nt", *, configs=None, warmup=5, r
         Ws = [(Wq, sc)] + [(Wq.clone(), sc.clone()) for _ in range(copies - 1)]
         run = lambda p: ops.streamk_q4(A, *rotate(Ws), out=C, plan=p)  # noqa: E731
         ref_ms = None
+    elif dtype == "float8_e4m3":
+        A8 = A.to(torch.float8_e4m3fn)
+        B8 = (torch.rand(N, K, generator=g) * 2 - 1).to(dev).to(torch.float8_e4m3fn)
+        Bs = [B8] + [B8.clone() for _ in range(copies - 1)]
+        run = lambda p: ops.streamk_fp8(A8, rotate(Bs), out=C, plan=p)  # noqa: E731
+        one = torch.ones(1, device=dev)
+        try:   # hipBLASLt's fp8 GEMM, where this torch build has it
+            ref_ms = _time_ms(lambda: torch._scaled_mm(A8, rotate(Bs).T, scale_a=one, scale_b=one, out_dtype=torch.float16),
+                              warmup, rep, 2.0 * M * N * K < 5e10)
+        except Exception:
+            ref_ms = None
     else:
         bshape = (N, K) if layout == "nt" else (K, N)
         B = (torch.rand(*bshape, generator=g) * 2 - 1).half().to(dev)

@@ -119,6 +119,35 @@ def streamk_bf16(A, B, *, layout="nt", out=None, plan=None, config=None, **kw):
     return C
 
 
+def streamk_fp8(A, B, *, out=None, plan=None, config=None, **kw):
+    """C = A @ B.T for fp8 operands (OCP e4m3: torch.float8_e4m3fn, or the same bytes as uint8),
+    A [M,K], B [N,K]; fp32 accumulation, fp16 C.  Values are taken as they are (no scales).  The
+    reference's scripts stop at fp16; this is the same partitioner and fix-ups over the fp8 form of
+    the tile kernel."""
+    f8 = getattr(torch, "float8_e4m3fn", None)
+    for t, name in ((A, "A"), (B, "B")):
+        if not isinstance(t, torch.Tensor) or t.dtype not in (torch.uint8, f8):
+            raise TypeError(f"{name} must be a float8_e4m3fn (or uint8) tensor")
+        _check_matrix(t, name, t.dtype)
+    M, K = A.shape
+    N, Kb = B.shape
+    if K != Kb:
+        raise ValueError(f"K mismatch: A is {tuple(A.shape)}, B is {tuple(B.shape)}")
+    if plan is None:
+        plan = make_plan(M, N, K, "float8_e4m3", "nt", config, **kw)
+    C = out if out is not None else torch.empty((M, N), dtype=torch.float16, device=A.device)
+    _check_matrix(C, "out", torch.float16)
+    if tuple(C.shape) != (M, N):
+        raise ValueError("out has the wrong shape")
+    ws = _workspace(plan.workspace_bytes, A.device)
+    rc = _lib.lib().sk_gemm_f8(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, A.stride(0),
+                               B.stride(0), C.stride(0), ctypes.byref(plan),
+                               ws.data_ptr() if ws is not None else None,
+                               ws.numel() if ws is not None else 0, _stream_ptr())
+    _lib.check(rc, "sk_gemm_f8")
+    return C
+
+
 Q4_MAX_M = 64  # rows of A the Q4 kernels take in one launch
 
 

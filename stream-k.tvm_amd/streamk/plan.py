@@ -5,7 +5,7 @@ from . import _lib
 from ._lib import SkConfig, SkPlan
 
 _DTYPES = {"float16": _lib.SK_F16, "float32": _lib.SK_F32, "q4": _lib.SK_Q4, "bfloat16": _lib.SK_BF16,
-           "q4_tiled": _lib.SK_Q4_TILED}
+           "q4_tiled": _lib.SK_Q4_TILED, "float8_e4m3": _lib.SK_F8E4M3}
 _LAYOUTS = {"nt": _lib.LAYOUT_NT, "nn": _lib.LAYOUT_NN}
 _num_cus = None
 
@@ -61,7 +61,12 @@ def tuned_config(M, N, K, dtype="float16", layout="nt"):
         from .autotune import load_cache
         _tuned = load_cache()
     hit = _tuned.get(f"gfx950/{dtype}/{layout}/{M}x{N}x{K}")
-    return dict(hit["config"]) if hit else None
+    if not hit:
+        return None
+    cfg = dict(hit["config"])
+    if cfg.get("raster") == 0:   # recorded as "row-major was fastest"; 0 now means "library default"
+        cfg["raster"] = 1
+    return cfg
 
 
 def make_plan(M, N, K, dtype="float16", layout="nt", config=None, cus=None, use_tuned=True, **kw):

@@ -42,7 +42,8 @@ def test_plan_matches_oracle(sk, oracle, shape, tile, P):
     restates it, for the product's own tile shapes."""
     M, N, K = shape
     plan = sk.make_plan(M, N, K, "float16", "nt", cus=256, bm=tile[0], bn=tile[1], bk=tile[2],
-                        grid=P, schedule="sk2")
+                        grid=P, schedule="sk2", raster=1)
+    assert sk.make_plan(M, N, K, "float16", "nt", cus=256, bm=tile[0], bn=tile[1], bk=tile[2]).raster == 8  # default
     ref = oracle.partition(M, N, K, *tile, P)
     for k in ("num_block_m", "num_block_n", "iters_per_tile", "total_tiles", "streamk_tiles",
               "blocking_tiles", "streamk_iters", "streamk_full_tiles", "streamk_partial_tiles"):
@@ -91,6 +92,18 @@ def test_fixed_split_k_schedule(sk):
     for bad in (3, 16):
         with pytest.raises(sk.StreamKError):
             sk.make_plan(1024, 1024, 8192, "float16", "nt", schedule="splitk", split=bad, **kw)
+
+
+def test_fp8_plans(sk):
+    """fp8 plans: tile kernels only (also for one row), bk counts fp8 elements, NT only."""
+    for (M, N, K, bm) in [(8192, 8192, 8192, 256), (512, 512, 4096, 128), (1, 4096, 4096, 128)]:
+        p = sk.make_plan(M, N, K, "float8_e4m3", "nt", cus=256)
+        assert (p.bm, p.bn, p.bk) == (bm, bm, 128) and p.iters_per_tile == K // 128
+        assert sk.kernel_name(p.kernel_id) == f"tile_f8e4m3_nt_dma_{bm}x{bm}x128"
+    with pytest.raises(sk.StreamKError):
+        sk.make_plan(256, 256, 256, "float8_e4m3", "nn", cus=256)
+    with pytest.raises(sk.StreamKError):
+        sk.make_plan(256, 256, 264, "float8_e4m3", "nt", cus=256)   # K not a multiple of 16
 
 
 def test_raster_is_a_permutation(sk):

@@ -451,6 +451,60 @@ def test_bf16_tile_kernels(sk, oracle):
     sk.workspace_status()
 
 
+def test_fp8_tile_kernels(sk, oracle):
+    """fp8 (OCP e4m3) operands, fp16 C: every instance, ragged shapes, K tails (K a multiple of 16 but not
+    of the 128-value iteration), all schedules and both fix-ups against the float64 host product of the
+    decoded bytes; tolerance 1e-2 (measured <= 1e-3: fp16 rounding of C).  On {-1, 0, 1} data with
+    |sums| <= 2048 the result must equal the host product exactly -- any mispairing of A and B bytes along
+    K would show -- and the ordered reduce must be bitwise repeatable."""
+    import torch
+    torch.manual_seed(11)
+    f8 = torch.float8_e4m3fn
+    tiles = [(256, 256), (128, 128), (128, 256), (256, 128)]
+    for (M, N, K) in [(200, 136, 336), (1000, 1096, 1040), (520, 264, 128), (64, 512, 2048), (300, 300, 16)]:
+        A, B = torch.randn(M, K).to(f8), torch.randn(N, K).to(f8)
+        Ai, Bi = torch.randint(-1, 2, (M, K)).float().to(f8), torch.randint(-1, 2, (N, K)).float().to(f8)
+        ref = oracle.f8_gemm_ref(A.view(torch.uint8).numpy(), B.view(torch.uint8).numpy())
+        exact = oracle.f8_gemm_ref(Ai.view(torch.uint8).numpy(), Bi.view(torch.uint8).numpy())
+        assert np.abs(exact).max() <= 2048
+        dA, dB, dAi, dBi = A.cuda(), B.cuda(), Ai.cuda(), Bi.cuda()
+        for (bm, bn) in tiles:
+            for sch in (dict(schedule="dp"), dict(schedule="basic", fixup="reduce", grid=24),
+                        dict(schedule="sk2", fixup="atomic", grid=16), dict(schedule="sk1", fixup="reduce", grid=7)):
+                plan = sk.make_plan(M, N, K, "float8_e4m3", "nt", dict(bm=bm, bn=bn, **sch))
+                assert plan.bk == 128 and plan.iters_per_tile == -(-K // 128)
+                C = sk.streamk_fp8(dA, dB, plan=plan)
+                assert C.dtype == torch.float16 and _rel(oracle, C, ref) <= 1e-3 <= TOL, (M, N, K, bm, bn, sch)
+                Ci = sk.streamk_fp8(dAi.view(torch.uint8), dBi.view(torch.uint8), plan=plan)   # raw bytes are accepted too
+                assert np.array_equal(Ci.double().cpu().numpy(), exact), (M, N, K, bm, bn, sch)
+                if sch.get("fixup") == "reduce":
+                    assert torch.equal(C, sk.streamk_fp8(dA, dB, plan=plan))
+    # heuristic plans from one row to many tiles; strided operands (leading dimension a multiple of 16)
+    for (M, N, K) in [(1, 512, 1024), (16, 4096, 4096), (2048, 2048, 2048), (1024, 8192, 8192)]:
+        A, B = torch.randn(M, K).to(f8), torch.randn(N, K).to(f8)
+        rows = np.random.RandomState(M).choice(M, size=min(M, 64), replace=False)
+        ref = oracle.f8_gemm_ref(A.view(torch.uint8).numpy()[rows], B.view(torch.uint8).numpy())
+        C = sk.streamk_fp8(A.cuda(), B.cuda())
+        assert oracle.max_abs_rel(C.float().cpu().numpy()[rows], ref) <= 1e-3
+    big = torch.randn(300, 1024).to(f8).cuda()
+    A, B = big[:200, 16:16 + 640], big[40:, 256:256 + 640]
+    ref = oracle.f8_gemm_ref(A.cpu().view(torch.uint8).numpy(), B.cpu().view(torch.uint8).numpy())
+    assert _rel(oracle, sk.streamk_fp8(A, B), ref) <= 1e-3
+    # every byte value except the NaN patterns (subnormals, +-0, +-448), against partners 0 and +-2^-6
+    allv = torch.tensor([b for b in range(256) if b & 127 != 127], dtype=torch.uint8)
+    A = torch.stack([allv.repeat(4)[torch.randperm(1016)[:1008]] for _ in range(40)])
+    B = torch.tensor([0x00, 0x08, 0x88], dtype=torch.uint8)[torch.randint(0, 3, (24, 1008))]
+    ref = oracle.f8_gemm_ref(A.numpy(), B.numpy())
+    assert _rel(oracle, sk.streamk_fp8(A.cuda(), B.cuda()), ref) <= 1e-3
+    with pytest.raises(TypeError):
+        sk.streamk_fp8(torch.zeros(8, 64, dtype=torch.float16, device="cuda"), torch.zeros(8, 64, dtype=torch.uint8, device="cuda"))
+    with pytest.raises(sk.StreamKError):
+        sk.streamk_fp8(torch.zeros(8, 72, dtype=torch.uint8, device="cuda"), torch.zeros(8, 72, dtype=torch.uint8, device="cuda"))
+    with pytest.raises(sk.StreamKError):
+        sk.make_plan(64, 64, 128, "float8_e4m3", "nn")
+    sk.workspace_status()
+
+
 def test_cfg5_large_dense(sk, oracle):
     """M = N = K = 8192 and the irregular 3000 x 5120 x 12288, U[-1,1): a random subset of rows is
     checked against an fp64 host product; the Stream-K and data-parallel schedules of the same kernel

@@ -73,3 +73,22 @@ def test_bad_arguments(oracle):
     A, B = _inputs(8, 8, 8)
     with pytest.raises(ValueError):
         oracle.streamk_gemm_f32(A, B, 0, 8, 8, 2)
+
+
+def test_f8e4m3_decode(oracle):
+    """The e4m3 decoder of the fp8 oracle against the format's definition (known values: 1.0, the largest
+    finite value 448, the smallest subnormal 2^-9 and normal 2^-6, the two NaN patterns, signed zero;
+    strictly increasing over the positive bytes) and against torch's own CPU conversion of all 256 bytes."""
+    import torch
+    d = oracle.f8e4m3_decode(np.arange(256, dtype=np.uint8))
+    assert d.dtype == np.float32
+    assert d[0x38] == 1.0 and d[0x7E] == 448.0 and d[0x01] == 2.0 ** -9 and d[0x08] == 2.0 ** -6 and d[0x07] == 7 * 2.0 ** -9
+    assert d[0x00] == 0 and d[0x80] == 0 and np.signbit(d[0x80]) and not np.signbit(d[0x00])
+    assert np.isnan(d[0x7F]) and np.isnan(d[0xFF]) and np.isnan(d).sum() == 2
+    assert np.all(np.diff(d[:0x7F]) > 0) and np.array_equal(d[0x80:0xFF], -d[:0x7F])
+    t = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn).float().numpy()
+    assert np.array_equal(np.isnan(d), np.isnan(t)) and np.array_equal(d[~np.isnan(d)], t[~np.isnan(t)])
+    # the host product is the plain sum of products
+    A = np.array([[0x38, 0x40, 0xB8, 0x01]], dtype=np.uint8)   # 1, 2, -1, 2^-9
+    B = np.array([[0x38, 0x38, 0x40, 0x7E], [0, 0, 0, 0]], dtype=np.uint8)   # 1, 1, 2, 448
+    assert np.array_equal(oracle.f8_gemm_ref(A, B), [[1 + 2 - 2 + 448 * 2.0 ** -9, 0.0]])
