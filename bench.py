@@ -239,33 +239,44 @@ def main():
             del a, b, bt, c
         extra["large_dense"] = dense
 
-        # the same kernel structure on fp8 (e4m3) operands: against the 5.0 PFLOP/s dense fp8 peak, with
-        # torch._scaled_mm (hipBLASLt) on the same operands where this torch build provides it
-        f8 = []
-        for (m, n, k) in ((8192, 8192, 8192), (1024, 8192, 8192)):
-            a, b = inputs(m, n, k, seed=6)
-            a8, b8 = a.to(torch.float8_e4m3fn), b.to(torch.float8_e4m3fn)
-            c = torch.empty(m, n, dtype=torch.float16, device="cuda")
-            one = torch.ones(1, device="cuda")
-            p = streamk.make_plan(m, n, k, "float8_e4m3", "nt")
-            row = {"shape": [m, n, k], "tile": [p.bm, p.bn, p.bk], "kernel": streamk.kernel_name(p.kernel_id),
-                   "streamk_tiles": p.streamk_tiles}
-            fns = {"tuned": lambda: streamk.streamk_fp8(a8, b8, out=c, plan=p),
-                   "torch_scaled_mm": lambda: torch._scaled_mm(a8, b8.T, scale_a=one, scale_b=one, out_dtype=torch.float16)}
-            best = {}
-            for _ in range(3):
-                for name, fn in fns.items():
-                    try:
-                        best[name] = min(best.get(name, 1e9), time_eager(fn, 3, 10)[0])
-                    except Exception:   # no fp8 GEMM in this torch build
-                        best[name] = None
-                        break
-            for name, ms in best.items():
-                row[name] = None if ms is None else {"us": round(ms * 1e3, 1), "tflops": round(2.0 * m * n * k / ms / 1e9, 1),
-                                                     "frac_fp8_peak": round(2.0 * m * n * k / ms / 1e9 / 5000.0, 4)}
-            f8.append(row)
-            del a, b, a8, b8, c
-        extra["fp8_e4m3_dense"] = f8
+        # the same kernel structure on one-byte operands, against the 5.0 PFLOP/s (POP/s) dense fp8 / int8 peak, with
+        # hipBLASLt (torch._scaled_mm / torch._int_mm) on the same operands where this torch build provides it
+        for key, dt in (("fp8_e4m3_dense", "float8_e4m3"), ("int8_dense", "int8")):
+            rows8 = []
+            for (m, n, k) in ((8192, 8192, 8192), (1024, 8192, 8192)):
+                if dt == "int8":
+                    g8 = torch.Generator(device="cpu").manual_seed(6)
+                    a8 = torch.randint(-128, 128, (m, k), generator=g8, dtype=torch.int8).cuda()
+                    b8 = torch.randint(-128, 128, (n, k), generator=g8, dtype=torch.int8).cuda()
+                    c = torch.empty(m, n, dtype=torch.int32, device="cuda")
+                    ours, vendor, vname = streamk.streamk_int8, (lambda: torch._int_mm(a8, b8.T)), "torch_int_mm"
+                else:
+                    a, b = inputs(m, n, k, seed=6)
+                    a8, b8 = a.to(torch.float8_e4m3fn), b.to(torch.float8_e4m3fn)
+                    del a, b
+                    c = torch.empty(m, n, dtype=torch.float16, device="cuda")
+                    one = torch.ones(1, device="cuda")
+                    ours, vname = streamk.streamk_fp8, "torch_scaled_mm"
+                    vendor = lambda: torch._scaled_mm(a8, b8.T, scale_a=one, scale_b=one, out_dtype=torch.float16)  # noqa: E731
+                p = streamk.make_plan(m, n, k, dt, "nt")
+                row = {"shape": [m, n, k], "tile": [p.bm, p.bn, p.bk], "kernel": streamk.kernel_name(p.kernel_id),
+                       "streamk_tiles": p.streamk_tiles}
+                fns = {"tuned": lambda: ours(a8, b8, out=c, plan=p), vname: vendor}
+                best = {}
+                for _ in range(3):
+                    for name, fn in fns.items():
+                        if best.get(name, 0) is None:
+                            continue
+                        try:
+                            best[name] = min(best.get(name, 1e9), time_eager(fn, 3, 10)[0])
+                        except Exception:   # no such GEMM in this torch build
+                            best[name] = None
+                for name, ms in best.items():
+                    row[name] = None if ms is None else {"us": round(ms * 1e3, 1), "tops": round(2.0 * m * n * k / ms / 1e9, 1),
+                                                         "frac_peak": round(2.0 * m * n * k / ms / 1e9 / 5000.0, 4)}
+                rows8.append(row)
+                del a8, b8, c
+            extra[key] = rows8
 
         q4 = []
         g = torch.Generator(device="cpu").manual_seed(4)

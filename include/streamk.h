@@ -71,7 +71,8 @@ typedef enum sk_dtype {
   SK_Q4 = 2,       /* fp16 A, packed nibbles [N, K/2] row-major */
   SK_BF16 = 3,
   SK_Q4_TILED = 4, /* fp16 A, packed nibbles in 16-row x 64-byte tiles (sk_q4_tile_host / sk_q4_tile) */
-  SK_F8E4M3 = 5    /* A and B one byte per element, OCP e4m3 (bias 7, no infinities, NaN = S.1111.111); C fp16 */
+  SK_F8E4M3 = 5,   /* A and B one byte per element, OCP e4m3 (bias 7, no infinities, NaN = S.1111.111); C fp16 */
+  SK_I8 = 6        /* A and B int8, C int32 */
 } sk_dtype;
 
 /* Tunables; a zero field means "choose for me".  Replaces the module-level constants and
@@ -167,6 +168,15 @@ int sk_gemm_bf16(const void *A, const void *B, void *C, int64_t M, int64_t N, in
  * fix-ups and workspace rules as sk_gemm_f16.  K, lda and ldb multiples of 16; A and B 16-byte
  * aligned.  Values are not scaled: a caller that keeps per-tensor scales applies them to C. */
 int sk_gemm_f8(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
+               int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws, size_t ws_bytes, void *stream);
+
+/* int8 operands: A [M,K] and B [N,K] (NT only) int8, C int32 (ldc in int32 elements), exact int32
+ * accumulation (wraps beyond 2^31, i.e. not below K = 133 000); the plan is made with dtype SK_I8.  The
+ * reference's Triton comparator accumulates integer inputs in int32 (triton.streamk/first_wave.py:123).
+ * Partial tiles are int32 too, so every schedule and both fix-ups give the same bits.  K, lda and ldb
+ * multiples of 16; A and B 16-byte aligned; C 4-byte aligned (16 bytes and ldc a multiple of 4 for
+ * vector stores). */
+int sk_gemm_i8(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
                int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws, size_t ws_bytes, void *stream);
 
 /* fp32 GEMM (fp32 MFMA, fp32 out).  Replaces tl_mod(A, B, C) of streamk_fp32.py:197-202. */

@@ -232,3 +232,13 @@ def f8_gemm_ref(A_u8, B_u8):
     """float64 host product A [M,K] x B [N,K]^T of e4m3 bytes (each product of two e4m3 values is exact in
     float32; the sum is taken in float64)."""
     return f8e4m3_decode(A_u8).astype(np.float64) @ f8e4m3_decode(B_u8).astype(np.float64).T
+
+
+def i8_gemm_ref(A_i8, B_i8):
+    """Exact integer product A [M,K] x B [N,K]^T of int8 operands (int64 on the host; the device accumulates
+    in int32 like the reference's Triton comparator, triton.streamk/first_wave.py:123, which is the same
+    number while |sum| < 2^31)."""
+    A = np.asarray(A_i8)
+    B = np.asarray(B_i8)
+    assert A.dtype == np.int8 and B.dtype == np.int8
+    return A.astype(np.int64) @ B.astype(np.int64).T

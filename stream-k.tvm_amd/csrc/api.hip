@@ -225,21 +225,21 @@ extern "C" int sk_gemm_bf16(const void *A, const void *B, void *C, int64_t M, in
   return gemm_16bit(SK_BF16, A, B, C, M, N, K, lda, ldb, ldc, plan, ws, ws_bytes, stream);
 }
 
-// fp8 operands travel through the fp16 tile machinery as pairs: K and the leading dimensions of A
-// and B are handed to the kernel in 16-bit units
-extern "C" int sk_gemm_f8(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,
-                          int64_t lda, int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws,
-                          size_t ws_bytes, void *stream) {
+// one-byte operands (fp8, int8) travel through the fp16 tile machinery as pairs: K and the leading
+// dimensions of A and B are handed to the kernel in 16-bit units
+static int gemm_8bit(int dtype, const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,
+                     int64_t lda, int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws,
+                     size_t ws_bytes, void *stream) {
   if (!A || !B || !C) return SK_ERR_NULL;
-  int rc = check_plan(plan, M, N, K, SK_F8E4M3, SK_LAYOUT_NT);
+  int rc = check_plan(plan, M, N, K, dtype, SK_LAYOUT_NT);
   if (rc) return rc;
   if (lda < K || ldb < K || ldc < N) return SK_ERR_SHAPE;
   if ((K % 16) || (lda % 16) || (ldb % 16)) return SK_ERR_ALIGN;
   if ((reinterpret_cast<uintptr_t>(A) & 15) || (reinterpret_cast<uintptr_t>(B) & 15) ||
-      (reinterpret_cast<uintptr_t>(C) & 1))
+      (reinterpret_cast<uintptr_t>(C) & (dtype == SK_I8 ? 3 : 1)))
     return SK_ERR_ALIGN;
   const KernelInfo *k = kernel_by_id(plan->kernel_id);
-  if (!k || k->dtype != SK_F8E4M3 || k->family != FAMILY_TILE) return SK_ERR_CONFIG;
+  if (!k || k->dtype != dtype || k->family != FAMILY_TILE) return SK_ERR_CONFIG;
   if (lda * k->bm >= (int64_t)1 << 31 || ldb * k->bn >= (int64_t)1 << 31) return SK_ERR_SHAPE;
   DevPlan dp;
   Workspace w;
@@ -247,6 +247,19 @@ extern "C" int sk_gemm_f8(const void *A, const void *B, void *C, int64_t M, int6
   if (rc) return rc;
   GemmArgs a{(const half_t *)A, (const half_t *)B, (half_t *)C, (int)M, (int)N, (int)(K / 2), lda / 2, ldb / 2, ldc};
   return launch_tile_f16(k->id, a, dp, w, (hipStream_t)stream) == 0 ? SK_OK : SK_ERR_LAUNCH;
+}
+
+extern "C" int sk_gemm_f8(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,
+                          int64_t lda, int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws,
+                          size_t ws_bytes, void *stream) {
+  return gemm_8bit(SK_F8E4M3, A, B, C, M, N, K, lda, ldb, ldc, plan, ws, ws_bytes, stream);
+}
+
+// (C and ldc are int32 here; the kernel casts)
+extern "C" int sk_gemm_i8(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,
+                          int64_t lda, int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws,
+                          size_t ws_bytes, void *stream) {
+  return gemm_8bit(SK_I8, A, B, C, M, N, K, lda, ldb, ldc, plan, ws, ws_bytes, stream);
 }
 
 extern "C" int sk_gemm_f32(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,

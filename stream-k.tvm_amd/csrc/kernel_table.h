@@ -184,6 +184,13 @@ struct KernelInfo {
   X(72, 128, 256, 2, 4)       \
   X(73, 256, 128, 4, 2)
 
+// int8 operands, int32 C, NT layout; bk counts int8 elements (variant 4: 16x16 accumulator blocks):  X(id, BM, BN, WM, WN)
+#define SK_TILE_I8_KERNELS(X) \
+  X(80, 256, 256, 2, 4)       \
+  X(81, 128, 128, 2, 2)       \
+  X(82, 128, 256, 2, 4)       \
+  X(83, 256, 128, 4, 2)
+
 const KernelInfo *kernel_table(int *count);
 const KernelInfo *kernel_by_id(int id);
 

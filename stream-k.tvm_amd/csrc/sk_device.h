@@ -226,5 +226,8 @@ __device__ __forceinline__ void atomic_add_f32(float *p, float v) {
   // hardware global_atomic_add_f32, no return value, device scope
   __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+__device__ __forceinline__ void atomic_add_i32(int *p, int v) {
+  __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 }  // namespace sk

@@ -64,12 +64,20 @@ struct LdsArray {
 // the instruction, for K-step s of 64 bytes, chunks 4s + g and 4s + 2 + g of row r as its 32-byte
 // operand.  Which K-values a lane's bytes stand for does not matter as long as A and B agree: the
 // instruction pairs byte b of lane group g of one operand with the same byte of the other.
+//
+// F8_ = 3: int8 operands, int32 accumulators and C.  The 16x16x32 pipeline as it is, with
+// v_mfma_i32_16x16x64_i8 on the same 16-byte fragments (64 K-values per K-step, same cycles as the fp16
+// form); partial tiles travel through the workspace as int32 in the fp32 slots, so both fix-ups are
+// exact and independent of the order of the additions.  C is stored from registers (a lane holds four
+// consecutive int32 of a row).
 template <int BM_, int BN_, int WM_, int WN_, bool B_KN_ = false, int BK_ = 64, bool MFMA16_ = false, bool BF16_ = false,
           int F8_ = 0>
 struct TileF16NTDma {
   static constexpr bool B_KN = B_KN_, MFMA16 = MFMA16_;
-  static constexpr int F8 = F8_;
-  static_assert(F8_ == 0 || (!MFMA16_ && !B_KN_ && BK_ == 64 && !BF16_), "fp8: NT layout, two stages");
+  static constexpr bool I8 = F8_ == 3;
+  static constexpr int F8 = I8 ? 0 : F8_;
+  static_assert(F8 == 0 || (!MFMA16_ && !B_KN_ && BK_ == 64 && !BF16_), "fp8: NT layout, two stages");
+  static_assert(!I8 || (MFMA16_ && !B_KN_ && !BF16_), "int8: NT layout, 16x16 accumulator blocks");
   // BF16_: operands and C are bfloat16 (same 16-bit data movement; v_mfma_f32_16x16x32_bf16; C rounded to
   // nearest even with v_cvt_pk_bf16_f32)
   static_assert(!BF16_ || MFMA16_, "bfloat16 exists in the 16x16x32 form");
@@ -112,13 +120,15 @@ struct TileF16NTDma {
   static_assert((A_BYTES / 1024) % NW == 0 && (B_BYTES / 1024) % NW == 0, "DMA groups must divide over the waves");
   static_assert(NW % NSTAGE == 0, "a wave must keep to row groups of one parity; patches per stage");
   static_assert(PATCH_ROWS % 32 == 0, "epilogue pass must hold whole 32-row blocks");
-  static_assert(F8_ == 0 || TM % 2 == 0, "fp8: the wave tile's rows are processed in two halves");
+  static_assert(F8 == 0 || TM % 2 == 0, "fp8: the wave tile's rows are processed in two halves");
 
   typedef TileF16NT<BM_, BN_, 64, WM_, WN_> Base;  // shares the accumulator type and the partials
   // 16x16x32: the accumulator is kept as 16x16 blocks of four registers (block (ii, jj): lane l holds
   // C[16*ii + l%16][16*jj + 4*(l/16) + e]), each updated in place by its MFMA
+  typedef int intx4 __attribute__((ext_vector_type(4)));
+  typedef typename std::conditional<I8, intx4, floatx4>::type AccV;
   struct Acc16 {
-    floatx4 v[FM][FN];
+    AccV v[FM][FN];
   };
   typedef typename std::conditional<MFMA16_, Acc16, typename Base::Acc>::type Acc;
 
@@ -170,7 +180,7 @@ struct TileF16NTDma {
 #pragma unroll
       for (int i = 0; i < FM; ++i)
 #pragma unroll
-        for (int j = 0; j < FN; ++j) acc.v[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < FN; ++j) acc.v[i][j] = AccV{0, 0, 0, 0};
     } else {
 #pragma unroll
       for (int i = 0; i < TM; ++i)
@@ -287,7 +297,10 @@ struct TileF16NTDma {
     auto mfma_one16 = [&](int abuf, int bbuf, int mh, int idx) {
       if constexpr (MFMA16) {
         const int i = idx / FN, j = idx % FN, ii = mh * FA + i;
-        if constexpr (BF16_) {
+        if constexpr (I8) {
+          acc.v[ii][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(intx4, fb[bbuf][j]),
+                                                               __builtin_bit_cast(intx4, fa[abuf][i]), acc.v[ii][j], 0, 0, 0);
+        } else if constexpr (BF16_) {
           typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
           acc.v[ii][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, fb[bbuf][j]),
                                                                  __builtin_bit_cast(bf16x8, fa[abuf][i]), acc.v[ii][j], 0, 0, 0);
@@ -386,10 +399,10 @@ struct TileF16NTDma {
       for (int j = 0; j < TN; ++j) read_b8_one(st, buf, s, j);
     };
     auto mfma_one8 = [&](int abuf, int bbuf, int mh, int idx) {
-      if constexpr (F8_ != 0) {
+      if constexpr (F8 != 0) {
         const int i = idx / TN, j = idx % TN, ii = mh * FA8 + i;
-        acc.c[ii][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb8[bbuf][j], fa8[abuf][i], acc.c[ii][j], F8_ - 1,
-                                                                       F8_ - 1, 0, 0, 0, 0);
+        acc.c[ii][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb8[bbuf][j], fa8[abuf][i], acc.c[ii][j], F8 - 1,
+                                                                       F8 - 1, 0, 0, 0, 0);
       }
     };
     auto mfma_half8 = [&](int abuf, int bbuf, int mh) {
@@ -425,7 +438,7 @@ struct TileF16NTDma {
           if (m * CH / NMF == x) mfma_one8(1, 1, 1, m);
       }
     };
-    if constexpr (F8_ != 0) {
+    if constexpr (F8 != 0) {
       // one K-iteration (128 K-values) on stage `cur`: two K-steps of 64, each in two halves of the
       // wave tile's rows.  Entering, fa8[0] / fb8[0] hold the fragments of (K-step 0, first half).
       auto iteration8 = [&](char *cur, char *nxt, int it) {
@@ -603,6 +616,28 @@ struct TileF16NTDma {
   static __device__ __forceinline__ void store_c(const Args &a, const Acc &acc, int pm, int pn, char *) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
+    if constexpr (I8) {
+      // int32 C straight from the accumulators: lane l of block (ii, jj) holds row 16*ii + l%16, columns
+      // 16*jj + 4*(l/16) .. +3
+      int *C = reinterpret_cast<int *>(a.C);
+      const bool vec_ok = (a.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(a.C) & 15) == 0);
+      const int row0 = pm * BM + wm * WTM + (lane & 15), col0 = pn * BN + wn * WTN + 4 * (lane >> 4);
+#pragma unroll
+      for (int ii = 0; ii < FM; ++ii)
+#pragma unroll
+        for (int jj = 0; jj < FN; ++jj) {
+          const int grow = row0 + 16 * ii, gcol = col0 + 16 * jj;
+          if (grow < a.M && gcol < a.N) {
+            int *dst = C + (int64_t)grow * a.ldc + gcol;
+            if (vec_ok && gcol + 4 <= a.N) {
+              *reinterpret_cast<intx4 *>(dst) = acc.v[ii][jj];
+            } else {
+              for (int e = 0; e < 4 && gcol + e < a.N; ++e) dst[e] = acc.v[ii][jj][e];
+            }
+          }
+        }
+      return;
+    }
     half_t *patch = reinterpret_cast<half_t *>(stage(wave / WAVES_PER_STAGE)) +
                     (wave % WAVES_PER_STAGE) * (PATCH_ROWS * LDC);
     const bool vec_ok = (a.ldc % 8 == 0) && ((reinterpret_cast<uintptr_t>(a.C) & 15) == 0);
@@ -610,7 +645,8 @@ struct TileF16NTDma {
     constexpr int BLK = PATCH_ROWS / 32;  // 32-row blocks per pass
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
-      if constexpr (MFMA16) {
+      if constexpr (I8) {
+      } else if constexpr (MFMA16) {
 #pragma unroll
         for (int ib = 0; ib < PATCH_ROWS / 16; ++ib)
 #pragma unroll
@@ -676,7 +712,7 @@ struct TileF16NTDma {
       dst = pin_here(dst);
 #pragma unroll
       for (int v = 0; v < NV4; ++v)
-        *reinterpret_cast<floatx4 *>(dst + ((size_t)v * NT + threadIdx.x) * 4) = acc.v[v / FN][v % FN];
+        *reinterpret_cast<AccV *>(dst + ((size_t)v * NT + threadIdx.x) * 4) = acc.v[v / FN][v % FN];
     } else {
       Base::store_partial(acc, dst);
     }
@@ -686,7 +722,7 @@ struct TileF16NTDma {
       src = pin_here(src);
 #pragma unroll
       for (int v = 0; v < NV4; ++v) {
-        acc.v[v / FN][v % FN] += *reinterpret_cast<const floatx4 *>(src + ((size_t)v * NT + threadIdx.x) * 4);
+        acc.v[v / FN][v % FN] += *reinterpret_cast<const AccV *>(src + ((size_t)v * NT + threadIdx.x) * 4);
         if (v % 8 == 7) asm volatile("" ::: "memory");  // at most 8 loads in flight
       }
     } else {
@@ -699,8 +735,12 @@ struct TileF16NTDma {
 #pragma unroll
       for (int v = 0; v < NV4; ++v)
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
-          atomic_add_f32(dst + (size_t)(v * 4 + e) * NT + threadIdx.x, acc.v[v / FN][v % FN][e]);
+        for (int e = 0; e < 4; ++e) {
+          if constexpr (I8)
+            atomic_add_i32(reinterpret_cast<int *>(dst) + (size_t)(v * 4 + e) * NT + threadIdx.x, acc.v[v / FN][v % FN][e]);
+          else
+            atomic_add_f32(dst + (size_t)(v * 4 + e) * NT + threadIdx.x, acc.v[v / FN][v % FN][e]);
+        }
     } else {
       Base::atomic_partial(acc, dst);
     }
@@ -713,7 +753,10 @@ struct TileF16NTDma {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           float *p = src + (size_t)(v * 4 + e) * NT + threadIdx.x;
-          acc.v[v / FN][v % FN][e] = *p;
+          if constexpr (I8)
+            acc.v[v / FN][v % FN][e] = *reinterpret_cast<int *>(p);
+          else
+            acc.v[v / FN][v % FN][e] = *p;
           *p = 0.f;
         }
         if (v % 4 == 3) asm volatile("" ::: "memory");

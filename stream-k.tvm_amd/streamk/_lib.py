@@ -8,7 +8,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libstreamk.so")
 
-SK_F16, SK_F32, SK_Q4, SK_BF16, SK_Q4_TILED, SK_F8E4M3 = 0, 1, 2, 3, 4, 5
+SK_F16, SK_F32, SK_Q4, SK_BF16, SK_Q4_TILED, SK_F8E4M3, SK_I8 = 0, 1, 2, 3, 4, 5, 6
 LAYOUT_NT, LAYOUT_NN = 0, 1
 SCHEDULES = {"auto": 0, "dp": 1, "sk2": 2, "sk1": 3, "basic": 4, "splitk": 5}
 FIXUPS = {"auto": 0, "atomic": 1, "reduce": 2}
@@ -76,6 +76,8 @@ def lib():
     L.sk_gemm_bf16.restype = ci
     L.sk_gemm_f8.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, P(SkPlan), vp, sz, vp]
     L.sk_gemm_f8.restype = ci
+    L.sk_gemm_i8.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, P(SkPlan), vp, sz, vp]
+    L.sk_gemm_i8.restype = ci
     L.sk_gemm_q4.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, ci, ci, P(SkPlan), vp, sz, vp]
     L.sk_dequant_q4.argtypes = [vp, vp, vp, i64, i64, ci, ci, vp]
     L.sk_q4_pack_host.argtypes = [vp, i64, i64, vp]

@@ -56,7 +56,7 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
     schedule, grid and fix-up."""
     cus = cus or _plan.num_cus()
     out = []
-    if dtype == "q4" or (M <= 64 and dtype != "float8_e4m3"):
+    if dtype == "q4" or (M <= 64 and dtype not in ("float8_e4m3", "int8")):
         tiles = _SKINNY_Q4 if dtype == "q4" else _SKINNY_F16
         for (bm, bn, bk) in tiles:
             if bm < M and not (bm == 16 and M <= 16):
@@ -84,7 +84,7 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
                 # fixed split-K, the fallback when there are fewer tiles than CUs
                 if -(-M // bm) * -(-N // bn) < cus:
                     out.extend(dict(base, schedule="splitk", fixup=fixup) for fixup in ("reduce", "atomic"))
-    if dtype == "float8_e4m3":
+    if dtype in ("float8_e4m3", "int8"):
         for (bm, bn), raster in itertools.product(((256, 256), (256, 128), (128, 256), (128, 128)), (1, 8)):
             base = dict(bm=bm, bn=bn, raster=raster)
             out.append(dict(base, schedule="dp"))
@@ -136,7 +136,7 @@ def autotune(M, N, K, dtype="float16", layout="nt", *, configs=None, warmup=5, r
     A = (torch.rand(M, K, generator=g) * 2 - 1).half().to(dev)
     C = torch.empty(M, N, dtype=torch.float16, device=dev)
     weights = weights or ("hbm" if M <= 64 else "warm")
-    wbytes = N * K // 2 if dtype == "q4" else (N * K if dtype == "float8_e4m3" else N * K * 2)
+    wbytes = N * K // 2 if dtype == "q4" else (N * K if dtype in ("float8_e4m3", "int8") else N * K * 2)
     copies = 1 if weights == "warm" else max(2, min(rep, -(-(512 << 20) // wbytes)))
     turn = [0]
 
@@ -158,6 +158,16 @@ def autotune(M, N, K, dtype="float16", layout="nt", *, configs=None, warmup=5, r
         try:   # hipBLASLt's fp8 GEMM, where this torch build has it
             ref_ms = _time_ms(lambda: torch._scaled_mm(A8, rotate(Bs).T, scale_a=one, scale_b=one, out_dtype=torch.float16),
                               warmup, rep, 2.0 * M * N * K < 5e10)
+        except Exception:
+            ref_ms = None
+    elif dtype == "int8":
+        Ai = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int8).to(dev)
+        Bi = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int8).to(dev)
+        Bs = [Bi] + [Bi.clone() for _ in range(copies - 1)]
+        C = torch.empty(M, N, dtype=torch.int32, device=dev)
+        run = lambda p: ops.streamk_int8(Ai, rotate(Bs), out=C, plan=p)  # noqa: E731
+        try:   # the vendor's int8 GEMM, where this torch build has it
+            ref_ms = _time_ms(lambda: torch._int_mm(Ai, rotate(Bs).T), warmup, rep, 2.0 * M * N * K < 5e10)
         except Exception:
             ref_ms = None
     else:

@@ -148,6 +148,31 @@ def streamk_fp8(A, B, *, out=None, plan=None, config=None, **kw):
     return C
 
 
+def streamk_int8(A, B, *, out=None, plan=None, config=None, **kw):
+    """C = A @ B.T for int8 operands, A [M,K], B [N,K]; exact int32 accumulation, int32 C (the accumulator
+    type the reference's Triton comparator picks for integer inputs, triton.streamk/first_wave.py:123).
+    Every schedule and fix-up returns the same bits."""
+    _check_matrix(A, "A", torch.int8)
+    _check_matrix(B, "B", torch.int8)
+    M, K = A.shape
+    N, Kb = B.shape
+    if K != Kb:
+        raise ValueError(f"K mismatch: A is {tuple(A.shape)}, B is {tuple(B.shape)}")
+    if plan is None:
+        plan = make_plan(M, N, K, "int8", "nt", config, **kw)
+    C = out if out is not None else torch.empty((M, N), dtype=torch.int32, device=A.device)
+    _check_matrix(C, "out", torch.int32)
+    if tuple(C.shape) != (M, N):
+        raise ValueError("out has the wrong shape")
+    ws = _workspace(plan.workspace_bytes, A.device)
+    rc = _lib.lib().sk_gemm_i8(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, A.stride(0),
+                               B.stride(0), C.stride(0), ctypes.byref(plan),
+                               ws.data_ptr() if ws is not None else None,
+                               ws.numel() if ws is not None else 0, _stream_ptr())
+    _lib.check(rc, "sk_gemm_i8")
+    return C
+
+
 Q4_MAX_M = 64  # rows of A the Q4 kernels take in one launch
 
 

@@ -18,7 +18,7 @@ sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("shape", help="MxNxK")
-    ap.add_argument("--dtype", default="float16", choices=["float16", "float32", "q4", "float8_e4m3"])
+    ap.add_argument("--dtype", default="float16", choices=["float16", "float32", "q4", "float8_e4m3", "int8"])
     ap.add_argument("--layout", default="nt", choices=["nt", "nn"])
     ap.add_argument("--config", default="{}", help="python dict of plan options, e.g. \"dict(bm=256,bn=256,raster=8)\"")
     ap.add_argument("--reps", type=int, default=5)
@@ -38,6 +38,15 @@ def main():
         Wq = torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8).cuda()
         sc = (torch.rand(N, K // 128, generator=g) * 0.015 + 0.005).half().cuda()
         run = lambda: streamk.streamk_q4(A, Wq, sc, plan=plan)  # noqa: E731
+    elif args.dtype == "int8":
+        if args.data == "rand":
+            A = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int8).cuda()
+            B = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int8).cuda()
+        else:
+            fill = torch.zeros if args.data == "zeros" else torch.ones
+            A, B = fill(M, K, dtype=torch.int8, device="cuda"), fill(N, K, dtype=torch.int8, device="cuda")
+        C = torch.empty(M, N, dtype=torch.int32, device="cuda")
+        run = lambda: streamk.streamk_int8(A, B, out=C, plan=plan)  # noqa: E731
     elif args.dtype == "float8_e4m3":
         f8 = torch.float8_e4m3fn
         if args.data == "rand":
@@ -71,6 +80,9 @@ def main():
             one = torch.ones(1, device="cuda")
             ms = streamk.bench_ms(lambda: torch._scaled_mm(A, B.T, scale_a=one, scale_b=one, out_dtype=torch.float16), 3, args.reps)
             print(f"{args.data}: torch._scaled_mm {ms * 1e3:.2f} us, {2.0 * M * N * K / ms / 1e9:.0f} TFLOP/s")
+        elif args.vendor and args.dtype == "int8":
+            ms = streamk.bench_ms(lambda: torch._int_mm(A, B.T), 3, args.reps)
+            print(f"{args.data}: torch._int_mm {ms * 1e3:.2f} us, {2.0 * M * N * K / ms / 1e9:.0f} TOP/s")
         elif args.vendor and args.dtype != "q4":
             Bt = B.T if args.layout == "nt" else B
             ms = streamk.bench_ms(lambda: torch.matmul(A, Bt, out=C), 3, args.reps)

@@ -100,6 +100,11 @@ def test_fp8_plans(sk):
         p = sk.make_plan(M, N, K, "float8_e4m3", "nt", cus=256)
         assert (p.bm, p.bn, p.bk) == (bm, bm, 128) and p.iters_per_tile == K // 128
         assert sk.kernel_name(p.kernel_id) == f"tile_f8e4m3_nt_dma_{bm}x{bm}x128"
+        q = sk.make_plan(M, N, K, "int8", "nt", cus=256)
+        assert (q.bm, q.bn, q.bk, q.grid) == (p.bm, p.bn, 128, p.grid)
+        assert sk.kernel_name(q.kernel_id) == f"tile_i8_nt_dma16_{bm}x{bm}x128"
+    with pytest.raises(sk.StreamKError):
+        sk.make_plan(256, 256, 256, "int8", "nn", cus=256)
     with pytest.raises(sk.StreamKError):
         sk.make_plan(256, 256, 256, "float8_e4m3", "nn", cus=256)
     with pytest.raises(sk.StreamKError):

@@ -505,6 +505,51 @@ def test_fp8_tile_kernels(sk, oracle):
     sk.workspace_status()
 
 
+def test_int8_tile_kernels(sk, oracle):
+    """int8 operands, int32 C: integer arithmetic, so every instance, schedule and fix-up (the atomic one
+    included) must return the host's exact product, on the full range -128..127, ragged shapes, K tails,
+    strided operands and an output whose rows are not 16-byte aligned."""
+    import torch
+    torch.manual_seed(12)
+    tiles = [(256, 256), (128, 128), (128, 256), (256, 128)]
+    for (M, N, K) in [(200, 136, 336), (1000, 1096, 1040), (520, 264, 128), (64, 512, 2048), (300, 300, 16)]:
+        A = torch.randint(-128, 128, (M, K), dtype=torch.int8)
+        B = torch.randint(-128, 128, (N, K), dtype=torch.int8)
+        ref = torch.from_numpy(oracle.i8_gemm_ref(A.numpy(), B.numpy()))
+        dA, dB = A.cuda(), B.cuda()
+        for (bm, bn) in tiles:
+            for sch in (dict(schedule="dp"), dict(schedule="basic", fixup="reduce", grid=24),
+                        dict(schedule="sk2", fixup="atomic", grid=16), dict(schedule="sk1", fixup="reduce", grid=7),
+                        dict(schedule="basic", fixup="atomic", grid=40, raster=1)):
+                plan = sk.make_plan(M, N, K, "int8", "nt", dict(bm=bm, bn=bn, **sch))
+                assert plan.bk == 128 and plan.iters_per_tile == -(-K // 128)
+                C = sk.streamk_int8(dA, dB, plan=plan)
+                assert C.dtype == torch.int32 and torch.equal(C.cpu().long(), ref), (M, N, K, bm, bn, sch)
+    # heuristic plans; extreme values (K * 128 * 128 stays below 2^31)
+    for (M, N, K) in [(1, 512, 1024), (16, 4096, 4096), (2048, 2048, 2048), (1024, 8192, 8192)]:
+        A = torch.randint(-128, 128, (M, K), dtype=torch.int8)
+        B = torch.randint(-128, 128, (N, K), dtype=torch.int8)
+        rows = np.random.RandomState(M).choice(M, size=min(M, 64), replace=False)
+        ref = torch.from_numpy(oracle.i8_gemm_ref(A.numpy()[rows], B.numpy()))
+        assert torch.equal(sk.streamk_int8(A.cuda(), B.cuda()).cpu().long()[rows], ref)
+    A = torch.full((130, 4096), -128, dtype=torch.int8)
+    B = torch.full((70, 4096), -128, dtype=torch.int8)
+    B[::2] = 127
+    assert torch.equal(sk.streamk_int8(A.cuda(), B.cuda()).cpu().long(), torch.from_numpy(oracle.i8_gemm_ref(A.numpy(), B.numpy())))
+    big = torch.randint(-128, 128, (300, 1024), dtype=torch.int8).cuda()
+    A, B = big[:200, 16:16 + 640], big[40:, 256:256 + 640]
+    ref = torch.from_numpy(oracle.i8_gemm_ref(A.cpu().numpy(), B.cpu().numpy()))
+    out = torch.zeros(200, 263, dtype=torch.int32, device="cuda")[:, 1:261]     # ldc 263, first column misaligned
+    assert torch.equal(sk.streamk_int8(A, B, out=out).cpu().long(), ref)
+    with pytest.raises(TypeError):
+        sk.streamk_int8(torch.zeros(8, 64, dtype=torch.uint8, device="cuda"), torch.zeros(8, 64, dtype=torch.int8, device="cuda"))
+    with pytest.raises(sk.StreamKError):
+        sk.streamk_int8(torch.zeros(8, 72, dtype=torch.int8, device="cuda"), torch.zeros(8, 72, dtype=torch.int8, device="cuda"))
+    with pytest.raises(sk.StreamKError):
+        sk.make_plan(64, 64, 128, "int8", "nn")
+    sk.workspace_status()
+
+
 def test_cfg5_large_dense(sk, oracle):
     """M = N = K = 8192 and the irregular 3000 x 5120 x 12288, U[-1,1): a random subset of rows is
     checked against an fp64 host product; the Stream-K and data-parallel schedules of the same kernel

@@ -92,3 +92,14 @@ def test_f8e4m3_decode(oracle):
     A = np.array([[0x38, 0x40, 0xB8, 0x01]], dtype=np.uint8)   # 1, 2, -1, 2^-9
     B = np.array([[0x38, 0x38, 0x40, 0x7E], [0, 0, 0, 0]], dtype=np.uint8)   # 1, 1, 2, 448
     assert np.array_equal(oracle.f8_gemm_ref(A, B), [[1 + 2 - 2 + 448 * 2.0 ** -9, 0.0]])
+
+
+def test_i8_gemm_ref(oracle):
+    """The int8 host product: hand-worked values at the ends of the range and agreement with a Python-int loop."""
+    A = np.array([[-128, 127, 1, 0], [1, 1, 1, 1]], dtype=np.int8)
+    B = np.array([[-128, 127, -1, 5], [127, -128, 0, 0], [0, 0, 0, 0]], dtype=np.int8)
+    assert np.array_equal(oracle.i8_gemm_ref(A, B), [[16384 + 16129 - 1, -16256 - 16256, 0], [3, -1, 0]])
+    rs = np.random.RandomState(0)
+    A, B = rs.randint(-128, 128, (5, 37)).astype(np.int8), rs.randint(-128, 128, (4, 37)).astype(np.int8)
+    want = [[sum(int(a) * int(b) for a, b in zip(ra, rb)) for rb in B] for ra in A]
+    assert np.array_equal(oracle.i8_gemm_ref(A, B), want)
