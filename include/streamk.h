@@ -72,7 +72,8 @@ typedef enum sk_dtype {
   SK_BF16 = 3,
   SK_Q4_TILED = 4, /* fp16 A, packed nibbles in 16-row x 64-byte tiles (sk_q4_tile_host / sk_q4_tile) */
   SK_F8E4M3 = 5,   /* A and B one byte per element, OCP e4m3 (bias 7, no infinities, NaN = S.1111.111); C fp16 */
-  SK_I8 = 6        /* A and B int8, C int32 */
+  SK_I8 = 6,       /* A and B int8, C int32 */
+  SK_Q4_ZP = 7     /* as SK_Q4 with one zero point per scale group and row (sk_gemm_q4_zp) */
 } sk_dtype;
 
 /* Tunables; a zero field means "choose for me".  Replaces the module-level constants and
@@ -202,6 +203,25 @@ int sk_gemm_f32(const void *A, const void *B, void *C, int64_t M, int64_t N, int
 int sk_gemm_q4(const void *A, const void *Wq, const void *scales, void *C, int64_t M, int64_t N,
                int64_t K, int64_t lda, int64_t ldc, int group, int zero, const sk_plan *plan,
                void *ws, size_t ws_bytes, void *stream);
+
+/* The same with one zero point per scale group and row: zeros [N, K/group] fp16 holding integers 0..15,
+ * w = fp16_rn((fp16(q) - zeros[n][k/group]) * scales[n][k/group]) -- the asymmetric formats of weight-only
+ * quantisers (min/max per group), which the reference's unsigned nibbles with one implied zero point do
+ * not cover.  The plan is made with dtype SK_Q4_ZP; every M goes through the general small-M kernels
+ * (bit-exact rounded weights; there is no matrix-vector specialisation), at most 64 rows per call. */
+int sk_gemm_q4_zp(const void *A, const void *Wq, const void *scales, const void *zeros, void *C, int64_t M,
+                  int64_t N, int64_t K, int64_t lda, int64_t ldc, int group, const sk_plan *plan, void *ws,
+                  size_t ws_bytes, void *stream);
+int sk_dequant_q4_zp(const void *Wq, const void *scales, const void *zeros, void *W, int64_t N, int64_t K,
+                     int group, void *stream);
+/* Asymmetric group-wise quantiser producing that format (host memory / device memory, same bytes):
+ *   lo = min(min w, 0), hi = max(max w, 0) over the group;  scale = fp16_rn((hi - lo) / 15)
+ *   z = clamp(rint(-lo / scale), 0, 15);  q = clamp(rint(w / scale) + z, 0, 15);  scale 0: z = q = 0
+ * (fp32 arithmetic, ties to even).  zeros is written as fp16 (uint16_t bit patterns on the host). */
+int sk_q4_quantize_zp_host(const uint16_t *W, int64_t N, int64_t K, int64_t ldw, int group, uint8_t *Wq,
+                           uint16_t *scales, uint16_t *zeros);
+int sk_q4_quantize_zp(const void *W, int64_t N, int64_t K, int64_t ldw, int group, void *Wq, void *scales,
+                      void *zeros, void *stream);
 
 /* Device dequantisation of Wq into fp16 W[N,K] with the device function the M > 1 GEMM uses
  * (the closed form of streamk_fp16_ladder_block_reduce_q4.py:548-554 plus zero/scale). */

@@ -242,3 +242,39 @@ def i8_gemm_ref(A_i8, B_i8):
     B = np.asarray(B_i8)
     assert A.dtype == np.int8 and B.dtype == np.int8
     return A.astype(np.int64) @ B.astype(np.int64).T
+
+
+# ------------------------------------------------------------------ Q4 with one zero point per group and row
+def dequant_q4_zp_np(Wq, scales, zeros, group=128):
+    """w = fp16((fp16(q) - z[n, k // group]) * scale[n, k // group]) in numpy float16 arithmetic; z holds
+    integers 0..15.  With a constant z this is dequant_q4_np / ora_dequant_q4 at that zero point (tested),
+    which follow streamk.fp16.breakdown/streamk_fp16_ladder_block_reduce_q4_atomic.py:280-282."""
+    q = unpack_q4_np(Wq).astype(np.float16)
+    z = np.repeat(np.asarray(zeros, dtype=np.float16), group, axis=1)[:, :q.shape[1]]
+    s = np.repeat(np.asarray(scales, dtype=np.float16), group, axis=1)[:, :q.shape[1]]
+    return ((q - z) * s).astype(np.float16)
+
+
+def quantize_q4_zp_np(W, group=128):
+    """Asymmetric group-wise rule of this build (the reference has no quantiser): lo = min(min w, 0),
+    hi = max(max w, 0); scale = fp16((hi - lo) / 15); z = clip(rint(-lo / scale), 0, 15);
+    q = clip(rint(w / scale) + z, 0, 15); scale 0: z = q = 0.  fp32 arithmetic.
+    Returns (Wq [N, K/2] uint8, scales, zeros [N, K/group] float16)."""
+    W = np.asarray(W, dtype=np.float16)
+    N, K = W.shape
+    w = W.astype(np.float32).reshape(N, K // group, group)
+    lo = np.minimum(w.min(axis=2), np.float32(0))
+    hi = np.maximum(w.max(axis=2), np.float32(0))
+    sc = ((hi - lo) / np.float32(15)).astype(np.float16)
+    s = sc.astype(np.float32)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        z = np.where(s == 0, np.float32(0), np.clip(np.rint(-lo / s), 0, 15)).astype(np.float32)
+        q = np.rint(w / s[:, :, None]) + z[:, :, None]
+    q = np.where(s[:, :, None] == 0, np.float32(0), np.clip(q, 0, 15)).astype(np.uint8).reshape(N, K)
+    return pack_q4_np(q), sc, z.astype(np.float16)
+
+
+def q4_zp_gemm_ref(A, Wq, scales, zeros, group=128):
+    """fp32 host product of A [M,K] with the dequantised weights [N,K]^T."""
+    W = dequant_q4_zp_np(Wq, scales, zeros, group).astype(np.float32)
+    return np.asarray(A, dtype=np.float32) @ W.T

@@ -288,18 +288,18 @@ extern "C" int sk_gemm_f32(const void *A, const void *B, void *C, int64_t M, int
   return launch_f32(k->id, a, dp, w, (hipStream_t)stream) == 0 ? SK_OK : SK_ERR_LAUNCH;
 }
 
-extern "C" int sk_gemm_q4(const void *A, const void *Wq, const void *scales, void *C, int64_t M, int64_t N,
-                          int64_t K, int64_t lda, int64_t ldc, int group, int zero, const sk_plan *plan,
-                          void *ws, size_t ws_bytes, void *stream) {
-  if (!A || !Wq || !scales || !C) return SK_ERR_NULL;
-  const int dtype = plan && plan->dtype == SK_Q4_TILED ? SK_Q4_TILED : SK_Q4;  // which layout Wq is in
+static int gemm_q4_any(const void *A, const void *Wq, const void *scales, const void *zeros, void *C, int64_t M,
+                       int64_t N, int64_t K, int64_t lda, int64_t ldc, int group, int zero, int dtype,
+                       const sk_plan *plan, void *ws, size_t ws_bytes, void *stream) {
+  if (!A || !Wq || !scales || !C || (dtype == SK_Q4_ZP && !zeros)) return SK_ERR_NULL;
   int rc = check_plan(plan, M, N, K, dtype, SK_LAYOUT_NT);
   if (rc) return rc;
   if (group != 128 || zero < 0 || zero > 15) return SK_ERR_CONFIG;
   if (lda < K || ldc < N) return SK_ERR_SHAPE;
   if ((K % 128) || (lda % 8)) return SK_ERR_ALIGN;
   if ((reinterpret_cast<uintptr_t>(A) & 15) || (reinterpret_cast<uintptr_t>(Wq) & 15) ||
-      (reinterpret_cast<uintptr_t>(scales) & 1) || (reinterpret_cast<uintptr_t>(C) & 1))
+      (reinterpret_cast<uintptr_t>(scales) & 1) || (reinterpret_cast<uintptr_t>(zeros) & 1) ||
+      (reinterpret_cast<uintptr_t>(C) & 1))
     return SK_ERR_ALIGN;
   const KernelInfo *k = kernel_by_id(plan->kernel_id);
   if (!k || k->dtype != dtype || k->family != FAMILY_SKINNY) return SK_ERR_CONFIG;
@@ -309,21 +309,41 @@ extern "C" int sk_gemm_q4(const void *A, const void *Wq, const void *scales, voi
   rc = make_dev_plan(plan, k, ws, ws_bytes, cached_occupancy(k->id, true), (hipStream_t)stream, &dp, &w);
   if (rc) return rc;
   SkinnyArgs a{(const half_t *)A, Wq, (const half_t *)scales, (half_t *)C, (int)M, (int)N, (int)K,
-               lda, K / 2, ldc, zero, (int)(K / group)};
+               lda, K / 2, ldc, zero, (int)(K / group), (const half_t *)zeros};
   int herr = launch_skinny(k->id, a, dp, w, (hipStream_t)stream);
   return herr == 0 ? SK_OK : SK_ERR_LAUNCH;
 }
 
+extern "C" int sk_gemm_q4(const void *A, const void *Wq, const void *scales, void *C, int64_t M, int64_t N,
+                          int64_t K, int64_t lda, int64_t ldc, int group, int zero, const sk_plan *plan,
+                          void *ws, size_t ws_bytes, void *stream) {
+  const int dtype = plan && plan->dtype == SK_Q4_TILED ? SK_Q4_TILED : SK_Q4;  // which layout Wq is in
+  return gemm_q4_any(A, Wq, scales, nullptr, C, M, N, K, lda, ldc, group, zero, dtype, plan, ws, ws_bytes, stream);
+}
+
+extern "C" int sk_gemm_q4_zp(const void *A, const void *Wq, const void *scales, const void *zeros, void *C,
+                             int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc, int group,
+                             const sk_plan *plan, void *ws, size_t ws_bytes, void *stream) {
+  return gemm_q4_any(A, Wq, scales, zeros, C, M, N, K, lda, ldc, group, 0, SK_Q4_ZP, plan, ws, ws_bytes, stream);
+}
+
 namespace {
 // one thread per 32-bit word of packed nibbles: 8 weights, written in natural element order
-__global__ void dequant_q4_kernel(const uint32_t *wq, const half_t *scales, half_t *out, int64_t words,
-                                  int words_per_row, int groups, int group, int zero) {
+__global__ void dequant_q4_kernel(const uint32_t *wq, const half_t *scales, const half_t *zeros, half_t *out,
+                                  int64_t words, int words_per_row, int groups, int group, int zero) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= words) return;
   const int64_t row = i / words_per_row;
   const int k = (int)(i % words_per_row) * 8;
   const half_t s = scales[row * groups + k / group];
-  const half8v v = dequant_word_q4(wq[i], q4_consts(zero), half2v{s, s});
+  half8v v;
+  if (zeros) {  // one zero point per group and row
+    const half_t z = zeros[row * groups + k / group];
+    const half_t lo = (half_t)1024.f + z, hi = (half_t)-64.f - z;
+    v = dequant_word_q4(wq[i], q4_consts(0), half2v{s, s}, half2v{lo, lo}, half2v{hi, hi});
+  } else {
+    v = dequant_word_q4(wq[i], q4_consts(zero), half2v{s, s});
+  }
   half8v o;
 #pragma unroll
   for (int e = 0; e < 8; ++e) o[e] = v[q4_slot_of_element(e)];
@@ -331,8 +351,19 @@ __global__ void dequant_q4_kernel(const uint32_t *wq, const half_t *scales, half
 }
 }  // namespace
 
+static int dequant_q4_any(const void *Wq, const void *scales, const void *zeros, void *W, int64_t N, int64_t K,
+                          int group, int zero, void *stream);
 extern "C" int sk_dequant_q4(const void *Wq, const void *scales, void *W, int64_t N, int64_t K, int group,
                              int zero, void *stream) {
+  return dequant_q4_any(Wq, scales, nullptr, W, N, K, group, zero, stream);
+}
+extern "C" int sk_dequant_q4_zp(const void *Wq, const void *scales, const void *zeros, void *W, int64_t N,
+                                int64_t K, int group, void *stream) {
+  if (!zeros) return SK_ERR_NULL;
+  return dequant_q4_any(Wq, scales, zeros, W, N, K, group, 0, stream);
+}
+static int dequant_q4_any(const void *Wq, const void *scales, const void *zeros, void *W, int64_t N, int64_t K,
+                          int group, int zero, void *stream) {
   if (!Wq || !scales || !W) return SK_ERR_NULL;
   if (N <= 0 || K <= 0) return SK_ERR_SHAPE;
   if (group <= 0 || (group % 8) || (K % group) || zero < 0 || zero > 15) return SK_ERR_CONFIG;
@@ -341,7 +372,7 @@ extern "C" int sk_dequant_q4(const void *Wq, const void *scales, void *W, int64_
   const int64_t blocks = (words + 255) / 256;
   if (blocks > 0x7fffffff) return SK_ERR_SHAPE;
   hipLaunchKernelGGL(dequant_q4_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
-                     (const uint32_t *)Wq, (const half_t *)scales, (half_t *)W, words, (int)(K / 8),
-                     (int)(K / group), group, zero);
+                     (const uint32_t *)Wq, (const half_t *)scales, (const half_t *)zeros, (half_t *)W, words,
+                     (int)(K / 8), (int)(K / group), group, zero);
   return hipGetLastError() == hipSuccess ? SK_OK : SK_ERR_LAUNCH;
 }

@@ -150,6 +150,15 @@ struct KernelInfo {
   X(193, 1, 2, 4, 4, 16384)    \
   X(194, 1, 1, 4, 4, 32768)
 
+// Q4 with one zero point per group and row (dtype SK_Q4_ZP), general small-M kernels:  X(id, MB, NB, WN, RK, DEPTH)
+#define SK_SKINNY_Q4ZP_KERNELS(X) \
+  X(220, 1, 1, 4, 1, 4)           \
+  X(221, 2, 1, 4, 1, 2)           \
+  X(222, 4, 1, 4, 1, 2)           \
+  X(223, 1, 1, 2, 4, 2)           \
+  X(224, 1, 1, 4, 2, 2)           \
+  X(225, 1, 1, 1, 4, 4)
+
 // M == 1 fp16 (NT) matrix-vector kernels (variant 2):  X(id, NB, WN, RK, DEPTH, KMAX)
 #define SK_GEMV_F16_KERNELS(X) \
   X(160, 1, 1, 4, 4, 8192)     \

@@ -66,6 +66,15 @@ int skinny_kernel_infos(KernelInfo *out, int max) {
   }
   SK_SKINNY_Q4T_KERNELS(X)
 #undef X
+#define X(id, MB, NB, WN, RK, DEPTH)                                                                     \
+  if (n < max) {                                                                                     \
+    typedef TileSkinny<MB, NB, WN, RK, true, DEPTH, false, false, true> P;                           \
+    out[n++] = KernelInfo{id, FAMILY_SKINNY, 7 /* SK_Q4_ZP */, 0, 0, P::BM, P::BN, P::BKC, P::NT,    \
+                          P::LDS_BYTES, P::CTAS_PER_CU, P::TILE_ELEMS, P::SC_MAX_ITERS, P::MAX_M, 128, \
+                          "skinny_q4zp_mb" #MB "_wn" #WN "_rk" #RK};                                  \
+  }
+  SK_SKINNY_Q4ZP_KERNELS(X)
+#undef X
 #define X(id, NB, WN, RK, DEPTH, KMAX)                                                                   \
   if (n < max) {                                                                                     \
     typedef TileGemvQ4<NB, WN, RK, DEPTH, KMAX, true> P;                                              \
@@ -107,6 +116,13 @@ int launch_skinny(int id, const SkinnyArgs &a, const DevPlan &p, const Workspace
     return launch_policy<P>(a, p, ws, s);                                                         \
   }
     SK_SKINNY_Q4T_KERNELS(X)
+#undef X
+#define X(id_, MB, NB, WN, RK, DEPTH)                                                       \
+  case id_: {                                                                              \
+    typedef TileSkinny<MB, NB, WN, RK, true, DEPTH, false, false, true> P;                 \
+    return launch_policy<P>(a, p, ws, s);                                                         \
+  }
+    SK_SKINNY_Q4ZP_KERNELS(X)
 #undef X
 #define X(id_, NB, WN, RK, DEPTH, KMAX)                                                     \
   case id_: {                                                                              \
@@ -157,6 +173,15 @@ int occupancy_skinny(int id) {
     return occ;                                                                                          \
   }
     SK_SKINNY_Q4T_KERNELS(X)
+#undef X
+#define X(id_, MB, NB, WN, RK, DEPTH)                                                                     \
+  case id_: {                                                                                            \
+    typedef TileSkinny<MB, NB, WN, RK, true, DEPTH, false, false, true> P;                               \
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_skinny_kernel<P>, P::NT, 0) != hipSuccess) \
+      return -1;                                                                                         \
+    return occ;                                                                                          \
+  }
+    SK_SKINNY_Q4ZP_KERNELS(X)
 #undef X
 #define X(id_, NB, WN, RK, DEPTH, KMAX)                                                                   \
   case id_: {                                                                                            \

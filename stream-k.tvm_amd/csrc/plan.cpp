@@ -69,7 +69,7 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
   // every CU something to do
   const KernelInfo *best = nullptr;
   // (for 32 < M <= 64 the 64x64 LDS tile below is faster than streaming the weights past 64 rows)
-  const bool q4 = dtype == SK_Q4 || dtype == SK_Q4_TILED;
+  const bool q4 = dtype == SK_Q4 || dtype == SK_Q4_TILED || dtype == SK_Q4_ZP;
   if ((M <= 32 && layout == SK_LAYOUT_NT) || q4) {
     // M == 1 with Q4 weights: the matrix-vector kernel with four waves splitting K (data-parallel
     // over 16-row tiles), the fastest instance at LLM-sized N and K
@@ -80,7 +80,8 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
           return &t[i];
     // 2 <= M <= 16 with Q4 weights: eight waves per CTA (two per SIMD cover each other's waits),
     // 32 weight rows, K split over four waves
-    if (dtype == SK_Q4 && M > 1 && M <= 16 && want_variant < 0)
+    // (per-group zero points: also for M == 1, which has no matrix-vector kernel of its own)
+    if (((dtype == SK_Q4 && M > 1) || dtype == SK_Q4_ZP) && M <= 16 && want_variant < 0)
       for (int i = 0; i < n; ++i)
         if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].variant == 0 && t[i].bm == 16 &&
             t[i].bn == 32 && t[i].bk == 1024 && accepts_shape(t[i], M, K))
@@ -143,7 +144,7 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
   if (!out) return SK_ERR_NULL;
   if (M <= 0 || N <= 0 || K <= 0 || M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return SK_ERR_SHAPE;
   if (dtype != SK_F16 && dtype != SK_F32 && dtype != SK_Q4 && dtype != SK_BF16 && dtype != SK_Q4_TILED &&
-      dtype != SK_F8E4M3 && dtype != SK_I8)
+      dtype != SK_F8E4M3 && dtype != SK_I8 && dtype != SK_Q4_ZP)
     return SK_ERR_CONFIG;
   if ((dtype == SK_F8E4M3 || dtype == SK_I8) && layout != SK_LAYOUT_NT) return SK_ERR_CONFIG;
   if (layout != SK_LAYOUT_NT && layout != SK_LAYOUT_NN) return SK_ERR_CONFIG;

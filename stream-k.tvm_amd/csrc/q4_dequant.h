@@ -66,6 +66,26 @@ __device__ __forceinline__ half8v dequant_word_q4(uint32_t w, const Q4Consts &c,
   return r.v;
 }
 
+// the same with the zero point given per call: bias_lo = 1024 + z, bias_hi = -(64 + z), z an integer in
+// 0..15 (both exact in fp16), for weights quantised with one zero point per group
+__device__ __forceinline__ half8v dequant_word_q4(uint32_t w, const Q4Consts &c, half2v scale, half2v bias_lo, half2v bias_hi) {
+  union {
+    uint32_t u[4];
+    half2v h[4];
+    half8v v;
+  } r;
+  const uint32_t t = w >> 8;
+  r.u[0] = and_or(w, c.mask_lo, c.magic);
+  r.u[1] = and_or(w, c.mask_hi, c.magic);
+  r.u[2] = and_or(t, c.mask_lo, c.magic);
+  r.u[3] = and_or(t, c.mask_hi, c.magic);
+  r.h[0] = (r.h[0] - bias_lo) * scale;
+  r.h[1] = __builtin_elementwise_fma(r.h[1], c.sixteenth, bias_hi) * scale;
+  r.h[2] = (r.h[2] - bias_lo) * scale;
+  r.h[3] = __builtin_elementwise_fma(r.h[3], c.sixteenth, bias_hi) * scale;
+  return r.v;
+}
+
 // position of logical element e (0..7) inside the vector dequant_word_q4 returns
 __device__ __forceinline__ constexpr int q4_slot_of_element(int e) { return (e & 3) * 2 + (e >> 2); }
 

@@ -87,6 +87,48 @@ __global__ __launch_bounds__(256) void quantize_q4_kernel(const half_t *W, uint3
   }
 }
 
+// asymmetric rule: the group's range [lo, hi] (widened to contain 0) is mapped onto 0..15
+__host__ __device__ inline float q4_zp_of(float lo, float scale) {
+  if (scale == 0.f) return 0.f;
+  float z = rintf(-lo / scale);
+  return z < 0.f ? 0.f : (z > 15.f ? 15.f : z);
+}
+
+// 16 lanes per group of 128, as quantize_q4_kernel
+__global__ __launch_bounds__(256) void quantize_q4_zp_kernel(const half_t *W, uint32_t *wq, half_t *scales, half_t *zeros,
+                                                             int64_t chunks, int chunks_per_row, int64_t ldw) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const bool live = i < chunks;
+  const int64_t ic = live ? i : 0;
+  const int64_t row = ic / chunks_per_row;
+  const int c = (int)(ic % chunks_per_row);
+  const half8v v = *reinterpret_cast<const half8v *>(W + row * ldw + (int64_t)c * 8);
+  float lo = 0.f, hi = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    lo = fminf(lo, (float)v[e]);
+    hi = fmaxf(hi, (float)v[e]);
+  }
+#pragma unroll
+  for (int m = 1; m < 16; m <<= 1) {
+    lo = fminf(lo, __shfl_xor(lo, m));
+    hi = fmaxf(hi, __shfl_xor(hi, m));
+  }
+  const half_t sh = (half_t)((hi - lo) / 15.f);
+  const float s = (float)sh;
+  const float z = q4_zp_of(lo, s);
+  uint32_t word = 0;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) word |= q4_quantize_one((float)v[e], s, (int)z) << (4 * e);
+  if (live) {
+    wq[i] = word;
+    if ((c & 15) == 0) {
+      scales[row * (chunks_per_row / 16) + c / 16] = sh;
+      zeros[row * (chunks_per_row / 16) + c / 16] = (half_t)z;
+    }
+  }
+}
+
 // tiled position of byte b of row n (runs = K / 128 tiles per row block)
 __host__ __device__ inline int64_t q4_tiled_offset(int64_t n, int64_t b, int64_t runs) {
   return ((n / 16) * runs + b / 64) * 1024 + (n % 16) * 64 + b % 64;
@@ -196,5 +238,50 @@ extern "C" int sk_q4_quantize(const void *W, int64_t N, int64_t K, int64_t ldw, 
   if (blocks > 0x7fffffff) return SK_ERR_SHAPE;
   hipLaunchKernelGGL(quantize_q4_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const half_t *)W,
                      (uint32_t *)Wq, (half_t *)scales, chunks, (int)(K / 8), ldw, zero);
+  return hipGetLastError() == hipSuccess ? SK_OK : SK_ERR_LAUNCH;
+}
+
+extern "C" int sk_q4_quantize_zp_host(const uint16_t *W, int64_t N, int64_t K, int64_t ldw, int group, uint8_t *Wq,
+                                      uint16_t *scales, uint16_t *zeros) {
+  if (!W || !Wq || !scales || !zeros) return SK_ERR_NULL;
+  if (N <= 0 || K <= 0 || ldw < K) return SK_ERR_SHAPE;
+  if (group <= 0 || (group % 8) || (K % group)) return SK_ERR_CONFIG;
+  const int64_t groups = K / group;
+  for (int64_t n = 0; n < N; ++n)
+    for (int64_t g = 0; g < groups; ++g) {
+      const uint16_t *w = W + n * ldw + g * group;
+      float lo = 0.f, hi = 0.f;
+      for (int k = 0; k < group; ++k) {
+        const float f = half_bits_to_float(w[k]);
+        if (!(fabsf(f) <= 65504.f)) return SK_ERR_CONFIG;  // NaN or infinity
+        lo = f < lo ? f : lo;
+        hi = f > hi ? f : hi;
+      }
+      const uint16_t sh = float_to_half_bits((hi - lo) / 15.f);
+      const float s = half_bits_to_float(sh);
+      const float z = q4_zp_of(lo, s);
+      scales[n * groups + g] = sh;
+      zeros[n * groups + g] = float_to_half_bits(z);
+      uint8_t *out = Wq + (n * K + g * group) / 2;
+      for (int k = 0; k < group; k += 2)
+        out[k / 2] = (uint8_t)(q4_quantize_one(half_bits_to_float(w[k]), s, (int)z) |
+                               (q4_quantize_one(half_bits_to_float(w[k + 1]), s, (int)z) << 4));
+    }
+  return SK_OK;
+}
+
+extern "C" int sk_q4_quantize_zp(const void *W, int64_t N, int64_t K, int64_t ldw, int group, void *Wq, void *scales,
+                                 void *zeros, void *stream) {
+  if (!W || !Wq || !scales || !zeros) return SK_ERR_NULL;
+  if (N <= 0 || K <= 0 || ldw < K || (ldw % 8)) return SK_ERR_SHAPE;
+  if (group != 128 || (K % group)) return SK_ERR_CONFIG;
+  if ((reinterpret_cast<uintptr_t>(W) & 15) || (reinterpret_cast<uintptr_t>(Wq) & 3) ||
+      (reinterpret_cast<uintptr_t>(scales) & 1) || (reinterpret_cast<uintptr_t>(zeros) & 1))
+    return SK_ERR_ALIGN;
+  const int64_t chunks = N * K / 8;
+  const int64_t blocks = (chunks + 255) / 256;
+  if (blocks > 0x7fffffff) return SK_ERR_SHAPE;
+  hipLaunchKernelGGL(quantize_q4_zp_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const half_t *)W,
+                     (uint32_t *)Wq, (half_t *)scales, (half_t *)zeros, chunks, (int)(K / 8), ldw);
   return hipGetLastError() == hipSuccess ? SK_OK : SK_ERR_LAUNCH;
 }

@@ -29,6 +29,7 @@ struct SkinnyArgs {
   int64_t lda, ldw, ldc;  // ldw in elements (fp16) or bytes (Q4)
   int zero;
   int groups;             // Q4: scales per row
+  const half_t *zeros;    // Q4 with per-group zero points: [N, K/group], integer values 0..15 (else unused)
 };
 
 // Copies the scales of groups [g0, g0 + 8*chunks) of the tile's BN weight rows to LDS rows of SC_ROW
@@ -96,9 +97,14 @@ __device__ __forceinline__ void stage_scales(half_t *ldsS, const half_t *scales_
 // of 64 bytes from each of 16 rows 4 KB apart, which streams 1.5x faster (profiles/
 // gemv_q4_M1_N8192_K8192.md, access pattern table); each lane receives the same bytes as from the
 // row-major array.
-template <int MB_, int NB_, int WN_, int RK_, bool Q4_, int DEPTH_, bool ROW1_ = false, bool TILED_ = false>
+//
+// ZP_ (Q4 only): one zero point per scale group and row (a.zeros, same shape as the scales) instead of
+// one for the whole matrix; staged in LDS beside the scales.
+template <int MB_, int NB_, int WN_, int RK_, bool Q4_, int DEPTH_, bool ROW1_ = false, bool TILED_ = false,
+          bool ZP_ = false>
 struct TileSkinny {
   static_assert(!TILED_ || Q4_, "tiled weights exist for Q4");
+  static_assert(!ZP_ || Q4_, "zero points exist for Q4");
   typedef SkinnyArgs Args;
   static constexpr int MB = MB_, NB = NB_, WN = WN_, RK = RK_, DEPTH = DEPTH_;
   static constexpr bool Q4 = Q4_;
@@ -122,7 +128,8 @@ struct TileSkinny {
   static constexpr int SC_MAX_ITERS = 64;           // scale staging covers this many iterations
   static constexpr int LDS_A = 2 * A_STAGE * 2;
   static constexpr int SC_ROW = SC_MAX_ITERS * SC_PER_ITER + 8;  // halfs per LDS scale row
-  static constexpr int LDS_SC = Q4 ? BN * SC_ROW * 2 : 0;
+  static constexpr int LDS_SC1 = Q4 ? BN * SC_ROW * 2 : 0;       // scales
+  static constexpr int LDS_SC = ZP_ ? 2 * LDS_SC1 : LDS_SC1;     // scales, then zero points
   static constexpr int LDS_RED = RK > 1 ? (RK - 1) * WN * 64 * MB * NB * 16 : 0;
   static constexpr int LDS_BYTES = LDS_A + LDS_SC + LDS_RED;
   static constexpr int LDS_TOTAL = LDS_BYTES;
@@ -249,6 +256,8 @@ struct TileSkinny {
       sc_shift = g_first - g0;
       const int chunks = (sc_shift + n * SC_PER_ITER + 7) >> 3;
       stage_scales<BN, SC_ROW, NT>(ldsS, a.scales + (int64_t)pn * BN * a.groups, rows_w, a.groups, g0, chunks);
+      if (ZP_)
+        stage_scales<BN, SC_ROW, NT>(ldsS + BN * SC_ROW, a.zeros + (int64_t)pn * BN * a.groups, rows_w, a.groups, g0, chunks);
     }
     SK_TRACE(4);
     stage_a(0, 0);
@@ -264,7 +273,7 @@ struct TileSkinny {
       for (int d = 0; d < DEPTH; ++d) {
         const int it = it0 + d;
         const half_t *abuf = ldsA + (it & 1) * A_STAGE;
-        half2v sc[NB][WLOADS];
+        half2v sc[NB][WLOADS], zlo[NB][WLOADS], zhi[NB][WLOADS];
         if (Q4) {
 #pragma unroll
           for (int j = 0; j < NB; ++j) {
@@ -272,7 +281,15 @@ struct TileSkinny {
             // load c of a Q4 iteration spans exactly one 128-wide scale group: group rk*2 + c
             const half_t *sp = ldsS + ((wn * NB + j) * 16 + lr) * SC_ROW + sc_shift + min(it, n - 1) * SC_PER_ITER + rk * 2;
 #pragma unroll
-            for (int c = 0; c < WLOADS; ++c) sc[j][c] = half2v{sp[c], sp[c]};
+            for (int c = 0; c < WLOADS; ++c) {
+              sc[j][c] = half2v{sp[c], sp[c]};
+              if (ZP_) {
+                const half_t z = sp[BN * SC_ROW + c];
+                const half_t lo = (half_t)1024.f + z, hi = (half_t)-64.f - z;   // exact: integers below 2048
+                zlo[j][c] = half2v{lo, lo};
+                zhi[j][c] = half2v{hi, hi};
+              }
+            }
           }
         }
 #pragma unroll
@@ -287,7 +304,10 @@ struct TileSkinny {
           for (int j = 0; j < NB; ++j) {
             half8v fw;
             if (Q4) {
-              fw = dequant_word_q4(wreg[d][j][ch / 4][ch % 4], qc, sc[j][ch / 4]);
+              if (ZP_)
+                fw = dequant_word_q4(wreg[d][j][ch / 4][ch % 4], qc, sc[j][ch / 4], zlo[j][ch / 4], zhi[j][ch / 4]);
+              else
+                fw = dequant_word_q4(wreg[d][j][ch / 4][ch % 4], qc, sc[j][ch / 4]);
             } else {
               fw = __builtin_bit_cast(half8v, wreg[d][j][ch]);
             }

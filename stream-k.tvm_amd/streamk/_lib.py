@@ -8,7 +8,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libstreamk.so")
 
-SK_F16, SK_F32, SK_Q4, SK_BF16, SK_Q4_TILED, SK_F8E4M3, SK_I8 = 0, 1, 2, 3, 4, 5, 6
+SK_F16, SK_F32, SK_Q4, SK_BF16, SK_Q4_TILED, SK_F8E4M3, SK_I8, SK_Q4_ZP = 0, 1, 2, 3, 4, 5, 6, 7
 LAYOUT_NT, LAYOUT_NN = 0, 1
 SCHEDULES = {"auto": 0, "dp": 1, "sk2": 2, "sk1": 3, "basic": 4, "splitk": 5}
 FIXUPS = {"auto": 0, "atomic": 1, "reduce": 2}
@@ -74,6 +74,14 @@ def lib():
     L.sk_gemm_f32.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, P(SkPlan), vp, sz, vp]
     L.sk_gemm_bf16.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, P(SkPlan), vp, sz, vp]
     L.sk_gemm_bf16.restype = ci
+    L.sk_gemm_q4_zp.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, ci, P(SkPlan), vp, sz, vp]
+    L.sk_gemm_q4_zp.restype = ci
+    L.sk_dequant_q4_zp.argtypes = [vp, vp, vp, vp, i64, i64, ci, vp]
+    L.sk_dequant_q4_zp.restype = ci
+    L.sk_q4_quantize_zp_host.argtypes = [vp, i64, i64, i64, ci, vp, vp, vp]
+    L.sk_q4_quantize_zp_host.restype = ci
+    L.sk_q4_quantize_zp.argtypes = [vp, i64, i64, i64, ci, vp, vp, vp, vp]
+    L.sk_q4_quantize_zp.restype = ci
     L.sk_gemm_f8.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, P(SkPlan), vp, sz, vp]
     L.sk_gemm_f8.restype = ci
     L.sk_gemm_i8.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, P(SkPlan), vp, sz, vp]

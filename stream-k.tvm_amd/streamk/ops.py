@@ -205,10 +205,26 @@ def untile_q4(tiled, N):
     return Wq
 
 
-def streamk_q4(A, Wq, scales, *, out=None, plan=None, config=None, zero=8, group=128, tiled=False, **kw):
+def _zero_points(zeros, scales):
+    """Per-group zero points as the library takes them: fp16 [N, K/group] holding integers 0..15.  Integer
+    tensors are converted (an allocation per call: keep them as fp16 to avoid it)."""
+    if zeros.dtype != torch.float16:
+        zeros = zeros.to(torch.float16)
+    _check_matrix(zeros, "zeros", torch.float16)
+    if tuple(zeros.shape) != tuple(scales.shape) or not zeros.is_contiguous():
+        raise ValueError(f"zeros must be contiguous and shaped like scales; got {tuple(zeros.shape)}")
+    return zeros
+
+
+def streamk_q4(A, Wq, scales, *, out=None, plan=None, config=None, zero=8, group=128, tiled=False, zeros=None, **kw):
     """C[M,N] fp16 = A[M,K] fp16 @ dequant(Wq)[N,K].T, weights in natural nibble order
     (streamk_fp16_ladder_block_reduce_q4.py:552).  tiled=True: Wq is the output of tile_q4 (N is
-    then taken from scales)."""
+    then taken from scales).  zeros: one zero point per scale group and row ([N, K/group], integers
+    0..15) instead of the scalar `zero`."""
+    if zeros is not None:
+        if tiled:
+            raise ValueError("per-group zero points need the row-major weights")
+        zeros = _zero_points(zeros, scales)
     _check_matrix(A, "A", torch.float16)
     _check_matrix(Wq, "Wq", torch.uint8)
     _check_matrix(scales, "scales", torch.float16)
@@ -220,6 +236,8 @@ def streamk_q4(A, Wq, scales, *, out=None, plan=None, config=None, zero=8, group
         raise ValueError(f"scales must be contiguous [N, K/group]; got {tuple(scales.shape)}")
     if plan is not None and (plan.dtype == _lib.SK_Q4_TILED) != bool(tiled):
         raise ValueError("the plan was made for the other weight layout")
+    if plan is not None and (plan.dtype == _lib.SK_Q4_ZP) != (zeros is not None):
+        raise ValueError("the plan was made with / without per-group zero points")
     C = out if out is not None else torch.empty((M, N), dtype=torch.float16, device=A.device)
     _check_matrix(C, "out", torch.float16)
     if tuple(C.shape) != (M, N):
@@ -231,14 +249,21 @@ def streamk_q4(A, Wq, scales, *, out=None, plan=None, config=None, zero=8, group
         if M <= 4 * Q4_MAX_M:
             for m0 in range(0, M, Q4_MAX_M):
                 streamk_q4(A[m0:m0 + Q4_MAX_M], Wq, scales, out=C[m0:m0 + Q4_MAX_M], config=config, zero=zero,
-                           group=group, tiled=tiled, **kw)
+                           group=group, tiled=tiled, zeros=zeros, **kw)
             return C
         if tiled:
             raise ValueError("more than 256 rows of A need the row-major weights (they are dequantised once)")
-        return streamk_fp16(A, dequant_q4(Wq, scales, zero=zero, group=group), out=C)
+        return streamk_fp16(A, dequant_q4(Wq, scales, zero=zero, group=group, zeros=zeros), out=C)
     if plan is None:
-        plan = make_plan(M, N, K, "q4_tiled" if tiled else "q4", "nt", config, **kw)
+        plan = make_plan(M, N, K, "q4_zp" if zeros is not None else ("q4_tiled" if tiled else "q4"), "nt", config, **kw)
     ws = _workspace(plan.workspace_bytes, A.device)
+    if zeros is not None:
+        rc = _lib.lib().sk_gemm_q4_zp(A.data_ptr(), Wq.data_ptr(), scales.data_ptr(), zeros.data_ptr(), C.data_ptr(),
+                                      M, N, K, A.stride(0), C.stride(0), group, ctypes.byref(plan),
+                                      ws.data_ptr() if ws is not None else None,
+                                      ws.numel() if ws is not None else 0, _stream_ptr())
+        _lib.check(rc, "sk_gemm_q4_zp")
+        return C
     rc = _lib.lib().sk_gemm_q4(A.data_ptr(), Wq.data_ptr(), scales.data_ptr(), C.data_ptr(), M, N, K,
                                A.stride(0), C.stride(0), group, zero, ctypes.byref(plan),
                                ws.data_ptr() if ws is not None else None,
@@ -247,7 +272,7 @@ def streamk_q4(A, Wq, scales, *, out=None, plan=None, config=None, zero=8, group
     return C
 
 
-def dequant_q4(Wq, scales, *, zero=8, group=128):
+def dequant_q4(Wq, scales, *, zero=8, group=128, zeros=None):
     """fp16 W[N,K] from packed nibbles, by the same device function the Q4 GEMM uses."""
     _check_matrix(Wq, "Wq", torch.uint8)
     _check_matrix(scales, "scales", torch.float16)
@@ -255,6 +280,12 @@ def dequant_q4(Wq, scales, *, zero=8, group=128):
     if not Wq.is_contiguous() or not scales.is_contiguous():
         raise ValueError("Wq and scales must be contiguous")
     W = torch.empty((N, K), dtype=torch.float16, device=Wq.device)
+    if zeros is not None:
+        zeros = _zero_points(zeros, scales)
+        rc = _lib.lib().sk_dequant_q4_zp(Wq.data_ptr(), scales.data_ptr(), zeros.data_ptr(), W.data_ptr(), N, K,
+                                         group, _stream_ptr())
+        _lib.check(rc, "sk_dequant_q4_zp")
+        return W
     rc = _lib.lib().sk_dequant_q4(Wq.data_ptr(), scales.data_ptr(), W.data_ptr(), N, K, group, zero,
                                   _stream_ptr())
     _lib.check(rc, "sk_dequant_q4")
@@ -283,15 +314,27 @@ def unpack_q4(Wq):
     return q
 
 
-def quantize_q4(W, *, group=128, zero=8):
+def quantize_q4(W, *, group=128, zero=8, asymmetric=False):
     """(Wq[N, K/2] uint8, scales[N, K/group] fp16) from fp16 W[N, K], on the device W lives on.
-    scale = fp16(max|w| / levels) per group, q = clamp(rint(w / scale) + zero, 0, 15)."""
+    scale = fp16(max|w| / levels) per group, q = clamp(rint(w / scale) + zero, 0, 15).
+    asymmetric=True: each group's range [min(w, 0), max(w, 0)] is mapped onto 0..15 with its own zero
+    point; returns (Wq, scales, zeros[N, K/group] fp16) for streamk_q4(..., zeros=zeros)."""
     if W.dtype != torch.float16 or W.dim() != 2 or W.stride(1) != 1:
         raise ValueError("W must be a 2-D fp16 tensor with unit stride along K")
     N, K = W.shape
     ldw = W.stride(0) if N > 1 else K  # the stride of a single row is arbitrary
     Wq = torch.empty((N, K // 2), dtype=torch.uint8, device=W.device)
     sc = torch.empty((N, K // max(group, 1)), dtype=torch.float16, device=W.device)
+    if asymmetric:
+        zp = torch.empty_like(sc)
+        if W.is_cuda:
+            rc = _lib.lib().sk_q4_quantize_zp(W.data_ptr(), N, K, ldw, group, Wq.data_ptr(), sc.data_ptr(),
+                                              zp.data_ptr(), _stream_ptr())
+        else:
+            rc = _lib.lib().sk_q4_quantize_zp_host(W.data_ptr(), N, K, ldw, group, Wq.data_ptr(), sc.data_ptr(),
+                                                   zp.data_ptr())
+        _lib.check(rc, "sk_q4_quantize_zp")
+        return Wq, sc, zp
     if W.is_cuda:
         rc = _lib.lib().sk_q4_quantize(W.data_ptr(), N, K, ldw, group, zero, Wq.data_ptr(), sc.data_ptr(),
                                        _stream_ptr())

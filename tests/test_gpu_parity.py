@@ -242,6 +242,62 @@ def test_q4_ragged_shapes_every_kernel(sk, oracle, variant):
     sk.workspace_status()
 
 
+def test_q4_per_group_zero_points(sk, oracle):
+    """Q4 with one zero point per scale group and row: device dequantisation bit for bit against the
+    oracle; the GEMM on every kernel instance, ragged shapes, all schedules, within 2e-3 of the fp32 host
+    product of the dequantised weights; with a constant zero point the result equals the scalar-zero
+    kernel's bit for bit; more than 64 rows through the split / dequantise paths; device quantiser equal to
+    the host one."""
+    import torch
+    rng = np.random.default_rng(77)
+    tiles = [(16, 64, 256), (32, 64, 256), (64, 64, 256), (16, 32, 1024), (16, 64, 512), (16, 16, 1024)]
+    ran = 0
+    for (M, N, K) in [(1, 1000, 1152), (5, 520, 384), (16, 264, 4096), (33, 200, 640), (64, 136, 2048), (1, 72, 16384)]:
+        A = (rng.random((M, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+        Wq = rng.integers(0, 256, (N, K // 2), dtype=np.uint8)
+        sc = rng.uniform(0.005, 0.02, (N, K // 128)).astype(np.float16)
+        zp = rng.integers(0, 16, (N, K // 128)).astype(np.float16)
+        dA, dW, dS, dZ = _t(A), _t(Wq), _t(sc), _t(zp)
+        W = sk.dequant_q4(dW, dS, zeros=dZ)
+        assert np.array_equal(W.cpu().numpy().view(np.uint16), oracle.dequant_q4_zp_np(Wq, sc, zp).view(np.uint16))
+        ref = oracle.q4_zp_gemm_ref(A, Wq, sc, zp)
+        z7 = torch.full_like(dZ, 7.0)
+        for (bm, bn, bk) in tiles:
+            for sch in (dict(schedule="dp"), dict(schedule="sk2", fixup="reduce", grid=48),
+                        dict(schedule="sk2", fixup="atomic", grid=40)):
+                try:
+                    plan = sk.make_plan(M, N, K, "q4_zp", "nt", dict(bm=bm, bn=bn, bk=bk, **sch))
+                except sk.StreamKError:
+                    continue  # the instance does not take this M / K
+                C = sk.streamk_q4(dA, dW, dS, zeros=dZ, plan=plan)
+                assert _rel(oracle, C, ref) <= 2e-3 <= TOL, (M, N, K, bm, bn, bk, sch, plan.kernel_id)
+                if sch.get("fixup") != "atomic":
+                    same = sk.make_plan(M, N, K, "q4", "nt", dict(bm=bm, bn=bn, bk=bk, variant=1, **sch))
+                    assert torch.equal(sk.streamk_q4(dA, dW, dS, zeros=z7, plan=plan), sk.streamk_q4(dA, dW, dS, zero=7, plan=same))
+                ran += 1
+        C = sk.streamk_q4(dA, dW, dS, zeros=_t(zp.astype(np.uint8)))      # heuristic plan; integer zero points are converted
+        assert _rel(oracle, C, ref) <= 2e-3
+    assert ran >= 60
+    # more rows than one launch takes: blocks of 64 rows, then dequantise + fp16 GEMM
+    N, K = 520, 1024
+    Wf = torch.randn(N, K, device="cuda").half() * 0.05 + 0.02
+    Wq, sc, zp = sk.quantize_q4(Wf, asymmetric=True)
+    hq, hs, hz = sk.quantize_q4(Wf.cpu(), asymmetric=True)
+    assert torch.equal(Wq.cpu(), hq) and torch.equal(sc.cpu(), hs) and torch.equal(zp.cpu(), hz)
+    for M in (150, 300):
+        A = torch.randn(M, K, device="cuda").half()
+        ref = oracle.q4_zp_gemm_ref(A.cpu().numpy(), hq.numpy(), hs.numpy(), hz.numpy())
+        assert _rel(oracle, sk.streamk_q4(A, Wq, sc, zeros=zp), ref) <= 2e-3
+    # quantisation error of the asymmetric rule on shifted weights is below the symmetric rule's
+    back_a = sk.dequant_q4(Wq, sc, zeros=zp).float()
+    sq, ss = sk.quantize_q4(Wf)
+    back_s = sk.dequant_q4(sq, ss).float()
+    assert (back_a - Wf.float()).abs().mean() < (back_s - Wf.float()).abs().mean()
+    with pytest.raises(ValueError):
+        sk.streamk_q4(A, Wq, sc, zeros=zp[:, :4])
+    sk.workspace_status()
+
+
 def test_q4_tiled_weights_give_identical_results(sk, oracle):
     """The tiled weight layout (16-row x 64-byte tiles) hands every lane the bytes it gets from the
     row-major array, so each tiled kernel must reproduce its row-major twin bit for bit (ordered

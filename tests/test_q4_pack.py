@@ -119,3 +119,56 @@ def test_bad_arguments(sk):
         sk.quantize_q4(torch.zeros(2, 100, dtype=torch.float16))    # K not a multiple of the group
     with pytest.raises(sk.StreamKError):
         sk.quantize_q4(torch.zeros(2, 128, dtype=torch.float16), zero=16)
+
+
+def test_asymmetric_quantiser_hand_worked_groups(sk, oracle):
+    """One zero point per group: hand-worked groups, then the host entry point against the oracle's numpy
+    restatement, and the round trip error bound of one step."""
+    # range [-5, 10]: scale = 1, z = 5, q = w + 5
+    w = np.resize(np.arange(-5, 11), 128).astype(np.float16)[None, :]
+    Wq, sc, zp = sk.quantize_q4(torch.from_numpy(w), asymmetric=True)
+    assert sc.tolist() == [[1.0]] and zp.tolist() == [[5.0]] and zp.dtype == torch.float16
+    assert np.array_equal(sk.unpack_q4(Wq).numpy()[0], (w[0] + 5).astype(np.uint8))
+    # all positive [0.5 .. 7.5]: the range is widened to contain 0: scale 0.5, z = 0; ties to even (1.25 / 0.5 = 2.5 -> 2)
+    w = np.zeros((1, 128), dtype=np.float16)
+    w[0, :4] = [7.5, 0.5, 1.25, 1.75]
+    Wq, sc, zp = sk.quantize_q4(torch.from_numpy(w), asymmetric=True)
+    assert sc.tolist() == [[0.5]] and zp.tolist() == [[0.0]]
+    assert sk.unpack_q4(Wq).numpy()[0, :5].tolist() == [15, 1, 2, 4, 0]
+    # all negative: z = 15
+    Wq, sc, zp = sk.quantize_q4(torch.from_numpy(-w), asymmetric=True)
+    assert zp.tolist() == [[15.0]] and sk.unpack_q4(Wq).numpy()[0, :5].tolist() == [0, 14, 13, 11, 15]   # rint(-2.5) + 15 = 13
+    # an all-zero group: scale 0, zero point 0, nibbles 0
+    Wq, sc, zp = sk.quantize_q4(torch.zeros(2, 256, dtype=torch.float16), asymmetric=True)
+    assert sc.abs().max().item() == 0 and zp.abs().max().item() == 0 and Wq.abs().max().item() == 0
+    # two groups of one row get their own zero points
+    w = np.concatenate([np.resize(np.arange(-5, 11), 128), np.resize(np.arange(-12, 4), 128)]).astype(np.float16)[None, :]
+    Wq, sc, zp = sk.quantize_q4(torch.from_numpy(w), asymmetric=True)
+    assert sc.tolist() == [[1.0, 1.0]] and zp.tolist() == [[5.0, 12.0]]
+    rng = np.random.default_rng(3)
+    for (N, K, group) in [(5, 256, 128), (33, 1024, 128), (4, 256, 32)]:
+        W = (rng.standard_normal((N, K)) * rng.uniform(0.01, 4.0, (N, 1)) + rng.uniform(-2, 2, (N, 1))).astype(np.float16)
+        Wq, sc, zp = sk.quantize_q4(torch.from_numpy(W), group=group, asymmetric=True)
+        rq, rs, rz = oracle.quantize_q4_zp_np(W, group)
+        assert np.array_equal(Wq.numpy(), rq) and np.array_equal(sc.numpy(), rs) and np.array_equal(zp.numpy(), rz)
+        assert set(np.unique(rz)) <= set(np.arange(16, dtype=np.float16))
+        back = oracle.dequant_q4_zp_np(rq, rs, rz, group).astype(np.float32)
+        step = np.repeat(rs.astype(np.float32), group, axis=1)
+        # half a step from rounding q, up to another half where the rounded zero point pushes the end of the range out
+        assert np.all(np.abs(back - W.astype(np.float32)) <= step * 1.002 + 1e-6)
+    with pytest.raises(sk.StreamKError):
+        sk.quantize_q4(torch.full((1, 128), float("inf"), dtype=torch.float16), asymmetric=True)
+
+
+def test_per_group_zero_point_dequant_reduces_to_the_scalar_form(oracle):
+    """The oracle's per-group form with a constant zero point is the pinned scalar form (numpy and C), and a
+    hand-worked row shows each group using its own zero point."""
+    rng = np.random.default_rng(5)
+    Wq = rng.integers(0, 256, (7, 192), dtype=np.uint8)
+    sc = rng.uniform(0.01, 0.5, (7, 3)).astype(np.float16)
+    for z in (0, 3, 8, 15):
+        zs = np.full((7, 3), z, dtype=np.float16)
+        assert np.array_equal(oracle.dequant_q4_zp_np(Wq, sc, zs).view(np.uint16), oracle.dequant_q4(Wq, sc, 128, z).view(np.uint16))
+    Wq = np.tile(np.array([0x10, 0xF7], dtype=np.uint8), 64)[None, :]      # nibbles 0, 1, 7, 15 repeating; two groups
+    out = oracle.dequant_q4_zp_np(Wq, np.array([[0.5, 2.0]], np.float16), np.array([[1, 7]], np.float16))
+    assert out[0, :4].tolist() == [-0.5, 0.0, 3.0, 7.0] and out[0, 128:132].tolist() == [-14.0, -12.0, 0.0, 16.0]
