@@ -56,8 +56,8 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
     schedule, grid and fix-up."""
     cus = cus or _plan.num_cus()
     out = []
-    if dtype == "q4" or (M <= 64 and dtype not in ("float8_e4m3", "int8")):
-        tiles = _SKINNY_Q4 if dtype == "q4" else _SKINNY_F16
+    if dtype in ("q4", "q4_zp") or (M <= 64 and dtype not in ("float8_e4m3", "int8")):
+        tiles = _SKINNY_Q4 if dtype in ("q4", "q4_zp") else _SKINNY_F16
         for (bm, bn, bk) in tiles:
             if bm < M and not (bm == 16 and M <= 16):
                 continue
@@ -136,18 +136,22 @@ def autotune(M, N, K, dtype="float16", layout="nt", *, configs=None, warmup=5, r
     A = (torch.rand(M, K, generator=g) * 2 - 1).half().to(dev)
     C = torch.empty(M, N, dtype=torch.float16, device=dev)
     weights = weights or ("hbm" if M <= 64 else "warm")
-    wbytes = N * K // 2 if dtype == "q4" else (N * K if dtype in ("float8_e4m3", "int8") else N * K * 2)
+    wbytes = N * K // 2 if dtype in ("q4", "q4_zp") else (N * K if dtype in ("float8_e4m3", "int8") else N * K * 2)
     copies = 1 if weights == "warm" else max(2, min(rep, -(-(512 << 20) // wbytes)))
     turn = [0]
 
     def rotate(items):
         turn[0] += 1
         return items[turn[0] % len(items)]
-    if dtype == "q4":
+    if dtype in ("q4", "q4_zp"):
         Wq = torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8).to(dev)
         sc = (torch.rand(N, K // 128, generator=g) * 0.015 + 0.005).half().to(dev)
         Ws = [(Wq, sc)] + [(Wq.clone(), sc.clone()) for _ in range(copies - 1)]
-        run = lambda p: ops.streamk_q4(A, *rotate(Ws), out=C, plan=p)  # noqa: E731
+        if dtype == "q4_zp":
+            zp = torch.randint(0, 16, (N, K // 128), generator=g).half().to(dev)
+            run = lambda p: ops.streamk_q4(A, *rotate(Ws), zeros=zp, out=C, plan=p)  # noqa: E731
+        else:
+            run = lambda p: ops.streamk_q4(A, *rotate(Ws), out=C, plan=p)  # noqa: E731
         ref_ms = None
     elif dtype == "float8_e4m3":
         A8 = A.to(torch.float8_e4m3fn)

@@ -17,9 +17,9 @@ class StreamKLinear(torch.nn.Module):
     def __init__(self, in_features, out_features, bias=False, *, weight_format="float16", group=128, zero=8,
                  device=None):
         super().__init__()
-        if weight_format not in ("float16", "q4"):
-            raise ValueError("weight_format must be 'float16' or 'q4'")
-        if weight_format == "q4" and (group != 128 or in_features % 128):
+        if weight_format not in ("float16", "q4", "q4_zp"):
+            raise ValueError("weight_format must be 'float16', 'q4' or 'q4_zp' (one zero point per group)")
+        if weight_format != "float16" and (group != 128 or in_features % 128):
             raise ValueError("Q4 weights need group == 128 and in_features a multiple of 128")
         if in_features % 8:
             raise ValueError("in_features must be a multiple of 8")
@@ -31,18 +31,26 @@ class StreamKLinear(torch.nn.Module):
         else:
             self.register_buffer("qweight", torch.zeros(N, K // 2, dtype=torch.uint8, device=device))
             self.register_buffer("scales", torch.zeros(N, K // group, dtype=torch.float16, device=device))
+            if weight_format == "q4_zp":
+                self.register_buffer("zeros", torch.zeros(N, K // group, dtype=torch.float16, device=device))
         self.register_buffer("bias", torch.zeros(N, dtype=torch.float16, device=device) if bias else None)
         self._plans = {}
 
     @classmethod
     def from_linear(cls, linear, *, weight_format="float16", group=128, zero=8):
-        """Takes over the weight (and bias) of a torch.nn.Linear; weight_format='q4' quantises it
-        with `quantize_q4` on the device it lives on."""
+        """Takes over the weight (and bias) of a torch.nn.Linear; weight_format='q4' / 'q4_zp' quantises
+        it with `quantize_q4` (symmetric around `zero` / asymmetric with a zero point per group) on the
+        device it lives on."""
         w = linear.weight.detach().to(torch.float16).contiguous()
         m = cls(linear.in_features, linear.out_features, linear.bias is not None, weight_format=weight_format,
                 group=group, zero=zero, device=w.device)
         if weight_format == "float16":
             m.weight.copy_(w)
+        elif weight_format == "q4_zp":
+            q, s, z = ops.quantize_q4(w, group=group, asymmetric=True)
+            m.qweight.copy_(q)
+            m.scales.copy_(s)
+            m.zeros.copy_(z)
         else:
             q, s = ops.quantize_q4(w, group=group, zero=zero)
             m.qweight.copy_(q)
@@ -54,7 +62,7 @@ class StreamKLinear(torch.nn.Module):
     def plan_for(self, M):
         p = self._plans.get(M)
         if p is None:
-            dtype = "float16" if self.weight_format == "float16" else "q4"
+            dtype = self.weight_format
             p = self._plans[M] = make_plan(M, self.out_features, self.in_features, dtype, "nt")
         return p
 
@@ -74,7 +82,7 @@ class StreamKLinear(torch.nn.Module):
         else:
             # (more rows than one Q4 launch takes: streamk_q4 splits the call itself)
             c = ops.streamk_q4(a, self.qweight, self.scales, plan=self.plan_for(M) if M <= ops.Q4_MAX_M else None,
-                               zero=self.zero, group=self.group)
+                               zero=self.zero, group=self.group, zeros=getattr(self, "zeros", None))
         if self.bias is not None:
             c += self.bias
         return c.view(*lead, self.out_features)

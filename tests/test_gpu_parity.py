@@ -295,6 +295,17 @@ def test_q4_per_group_zero_points(sk, oracle):
     assert (back_a - Wf.float()).abs().mean() < (back_s - Wf.float()).abs().mean()
     with pytest.raises(ValueError):
         sk.streamk_q4(A, Wq, sc, zeros=zp[:, :4])
+    # as a layer: asymmetric weights, plans per M, state round trip
+    lin = torch.nn.Linear(K, N, bias=True).cuda().half()
+    with torch.no_grad():
+        lin.weight.add_(0.03)
+    layer = sk.StreamKLinear.from_linear(lin, weight_format="q4_zp")
+    assert set(layer.state_dict()) == {"qweight", "scales", "zeros", "bias"}
+    for shape in ((1, K), (2, 8, K), (150, K)):
+        x = torch.randn(*shape, device="cuda").half()
+        W = oracle.dequant_q4_zp_np(layer.qweight.cpu().numpy(), layer.scales.cpu().numpy(), layer.zeros.cpu().numpy())
+        ref = x.float().cpu().numpy().reshape(-1, K) @ W.astype(np.float32).T + lin.bias.detach().float().cpu().numpy()
+        assert oracle.max_abs_rel(layer(x).float().cpu().numpy().reshape(-1, N), ref) <= 2e-3
     sk.workspace_status()
 
 
