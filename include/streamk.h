@@ -167,9 +167,12 @@ int sk_gemm_bf16(const void *A, const void *B, void *C, int64_t M, int64_t N, in
  * reference's scripts; its Triton comparator takes whatever dtype its inputs have
  * (triton.streamk/first_wave.py:123 picks the accumulator type from them).  Same partitioner,
  * fix-ups and workspace rules as sk_gemm_f16.  K, lda and ldb multiples of 16; A and B 16-byte
- * aligned.  Values are not scaled: a caller that keeps per-tensor scales applies them to C. */
+ * aligned.  C = fp16_rn(alpha * (A B^T)): alpha (finite; the product of the two per-tensor scales of
+ * a scaled-fp8 caller, 1 for none) multiplies the fp32 sums before they are rounded, so sums beyond
+ * fp16's range can be brought back into it. */
 int sk_gemm_f8(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
-               int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws, size_t ws_bytes, void *stream);
+               int64_t ldb, int64_t ldc, float alpha, const sk_plan *plan, void *ws, size_t ws_bytes,
+               void *stream);
 
 /* int8 operands: A [M,K] and B [N,K] (NT only) int8, C int32 (ldc in int32 elements), exact int32
  * accumulation (wraps beyond 2^31, i.e. not below K = 133 000); the plan is made with dtype SK_I8.  The

@@ -206,7 +206,7 @@ static int gemm_16bit(int dtype, const void *A, const void *B, void *C, int64_t 
     SkinnyArgs a{(const half_t *)A, B, nullptr, (half_t *)C, (int)M, (int)N, (int)K, lda, ldb, ldc, 0, 0};
     herr = launch_skinny(k->id, a, dp, w, (hipStream_t)stream);
   } else {
-    GemmArgs a{(const half_t *)A, (const half_t *)B, (half_t *)C, (int)M, (int)N, (int)K, lda, ldb, ldc};
+    GemmArgs a{(const half_t *)A, (const half_t *)B, (half_t *)C, (int)M, (int)N, (int)K, lda, ldb, ldc, 1.f};
     herr = launch_tile_f16(k->id, a, dp, w, (hipStream_t)stream);
   }
   return herr == 0 ? SK_OK : SK_ERR_LAUNCH;
@@ -228,7 +228,7 @@ extern "C" int sk_gemm_bf16(const void *A, const void *B, void *C, int64_t M, in
 // one-byte operands (fp8, int8) travel through the fp16 tile machinery as pairs: K and the leading
 // dimensions of A and B are handed to the kernel in 16-bit units
 static int gemm_8bit(int dtype, const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,
-                     int64_t lda, int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws,
+                     int64_t lda, int64_t ldb, int64_t ldc, float alpha, const sk_plan *plan, void *ws,
                      size_t ws_bytes, void *stream) {
   if (!A || !B || !C) return SK_ERR_NULL;
   int rc = check_plan(plan, M, N, K, dtype, SK_LAYOUT_NT);
@@ -245,21 +245,22 @@ static int gemm_8bit(int dtype, const void *A, const void *B, void *C, int64_t M
   Workspace w;
   rc = make_dev_plan(plan, k, ws, ws_bytes, cached_occupancy(k->id, false), (hipStream_t)stream, &dp, &w);
   if (rc) return rc;
-  GemmArgs a{(const half_t *)A, (const half_t *)B, (half_t *)C, (int)M, (int)N, (int)(K / 2), lda / 2, ldb / 2, ldc};
+  GemmArgs a{(const half_t *)A, (const half_t *)B, (half_t *)C, (int)M, (int)N, (int)(K / 2), lda / 2, ldb / 2, ldc, alpha};
   return launch_tile_f16(k->id, a, dp, w, (hipStream_t)stream) == 0 ? SK_OK : SK_ERR_LAUNCH;
 }
 
 extern "C" int sk_gemm_f8(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,
-                          int64_t lda, int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws,
+                          int64_t lda, int64_t ldb, int64_t ldc, float alpha, const sk_plan *plan, void *ws,
                           size_t ws_bytes, void *stream) {
-  return gemm_8bit(SK_F8E4M3, A, B, C, M, N, K, lda, ldb, ldc, plan, ws, ws_bytes, stream);
+  if (!(alpha == alpha) || alpha - alpha != 0.f) return SK_ERR_CONFIG;  // NaN or infinite
+  return gemm_8bit(SK_F8E4M3, A, B, C, M, N, K, lda, ldb, ldc, alpha, plan, ws, ws_bytes, stream);
 }
 
 // (C and ldc are int32 here; the kernel casts)
 extern "C" int sk_gemm_i8(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,
                           int64_t lda, int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws,
                           size_t ws_bytes, void *stream) {
-  return gemm_8bit(SK_I8, A, B, C, M, N, K, lda, ldb, ldc, plan, ws, ws_bytes, stream);
+  return gemm_8bit(SK_I8, A, B, C, M, N, K, lda, ldb, ldc, 1.f, plan, ws, ws_bytes, stream);
 }
 
 extern "C" int sk_gemm_f32(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,

@@ -16,6 +16,7 @@ struct GemmArgs {
   half_t *C;
   int M, N, K;
   int64_t lda, ldb, ldc;
+  float alpha;  // fp8 kernels: C = fp16(alpha * A B^T); unused elsewhere
 };
 
 template <int BM_, int BN_, int BK_, int WM_, int WN_>

@@ -673,7 +673,12 @@ struct TileF16NTDma {
             for (int q = 0; q < 4; ++q) {
               half4v h;
 #pragma unroll
-              for (int e = 0; e < 4; ++e) h[e] = (half_t)acc.c[p * BLK + ib][j][q * 4 + e];
+              for (int e = 0; e < 4; ++e) {
+                if constexpr (F8 != 0)  // the product of fp8 operands is scaled before it is rounded to fp16
+                  h[e] = (half_t)(a.alpha * (float)acc.c[p * BLK + ib][j][q * 4 + e]);
+                else
+                  h[e] = (half_t)acc.c[p * BLK + ib][j][q * 4 + e];
+              }
               *reinterpret_cast<half4v *>(patch + (ib * 32 + (lane & 31)) * LDC + j * 32 + q * 8 +
                                           (lane >> 5) * 4) = h;
             }

@@ -82,7 +82,7 @@ def lib():
     L.sk_q4_quantize_zp_host.restype = ci
     L.sk_q4_quantize_zp.argtypes = [vp, i64, i64, i64, ci, vp, vp, vp, vp]
     L.sk_q4_quantize_zp.restype = ci
-    L.sk_gemm_f8.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, P(SkPlan), vp, sz, vp]
+    L.sk_gemm_f8.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, ctypes.c_float, P(SkPlan), vp, sz, vp]
     L.sk_gemm_f8.restype = ci
     L.sk_gemm_i8.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, P(SkPlan), vp, sz, vp]
     L.sk_gemm_i8.restype = ci

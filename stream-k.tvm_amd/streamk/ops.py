@@ -119,11 +119,11 @@ def streamk_bf16(A, B, *, layout="nt", out=None, plan=None, config=None, **kw):
     return C
 
 
-def streamk_fp8(A, B, *, out=None, plan=None, config=None, **kw):
-    """C = A @ B.T for fp8 operands (OCP e4m3: torch.float8_e4m3fn, or the same bytes as uint8),
-    A [M,K], B [N,K]; fp32 accumulation, fp16 C.  Values are taken as they are (no scales).  The
-    reference's scripts stop at fp16; this is the same partitioner and fix-ups over the fp8 form of
-    the tile kernel."""
+def streamk_fp8(A, B, *, alpha=1.0, out=None, plan=None, config=None, **kw):
+    """C = alpha * (A @ B.T) for fp8 operands (OCP e4m3: torch.float8_e4m3fn, or the same bytes as
+    uint8), A [M,K], B [N,K]; fp32 accumulation, alpha applied to the fp32 sums, fp16 C.  alpha is
+    the product of the per-tensor scales of a scaled-fp8 caller.  The reference's scripts stop at
+    fp16; this is the same partitioner and fix-ups over the fp8 form of the tile kernel."""
     f8 = getattr(torch, "float8_e4m3fn", None)
     for t, name in ((A, "A"), (B, "B")):
         if not isinstance(t, torch.Tensor) or t.dtype not in (torch.uint8, f8):
@@ -141,7 +141,7 @@ def streamk_fp8(A, B, *, out=None, plan=None, config=None, **kw):
         raise ValueError("out has the wrong shape")
     ws = _workspace(plan.workspace_bytes, A.device)
     rc = _lib.lib().sk_gemm_f8(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, A.stride(0),
-                               B.stride(0), C.stride(0), ctypes.byref(plan),
+                               B.stride(0), C.stride(0), float(alpha), ctypes.byref(plan),
                                ws.data_ptr() if ws is not None else None,
                                ws.numel() if ws is not None else 0, _stream_ptr())
     _lib.check(rc, "sk_gemm_f8")

@@ -563,6 +563,20 @@ def test_fp8_tile_kernels(sk, oracle):
     B = torch.tensor([0x00, 0x08, 0x88], dtype=torch.uint8)[torch.randint(0, 3, (24, 1008))]
     ref = oracle.f8_gemm_ref(A.numpy(), B.numpy())
     assert _rel(oracle, sk.streamk_fp8(A.cuda(), B.cuda()), ref) <= 1e-3
+    # alpha scales the fp32 sums before the rounding to fp16: operands near the top of the range, whose plain
+    # product overflows fp16 (448 * 448 * K), come back finite and accurate with alpha = 2^-14
+    A = (torch.rand(130, 512) * 200 + 200).to(f8)
+    B = (torch.rand(70, 512) * 200 + 200).to(f8)
+    ref = oracle.f8_gemm_ref(A.view(torch.uint8).numpy(), B.view(torch.uint8).numpy())
+    assert torch.isinf(sk.streamk_fp8(A.cuda(), B.cuda())).all() and ref.min() > 65504
+    for cfg in (dict(schedule="dp"), dict(schedule="basic", fixup="reduce", grid=8), dict(schedule="basic", fixup="atomic", grid=8)):
+        C = sk.streamk_fp8(A.cuda(), B.cuda(), alpha=2.0 ** -14, bm=128, bn=128, **cfg)
+        assert _rel(oracle, C, ref * 2.0 ** -14) <= 1e-3, cfg
+    Cp = sk.streamk_fp8(A.cuda(), B.cuda(), alpha=2.0 ** -14, bm=128, bn=128, schedule="dp")
+    Cn = sk.streamk_fp8(A.cuda(), B.cuda(), alpha=-2.0 ** -15, bm=128, bn=128, schedule="dp")
+    assert torch.equal(Cn * -2, Cp)     # sign and power of two: exact
+    with pytest.raises(sk.StreamKError):
+        sk.streamk_fp8(A.cuda(), B.cuda(), alpha=float("nan"))
     with pytest.raises(TypeError):
         sk.streamk_fp8(torch.zeros(8, 64, dtype=torch.float16, device="cuda"), torch.zeros(8, 64, dtype=torch.uint8, device="cuda"))
     with pytest.raises(sk.StreamKError):
