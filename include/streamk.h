@@ -156,6 +156,27 @@ int sk_gemm_f16(const void *A, const void *B, void *C, int64_t M, int64_t N, int
                 int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws, size_t ws_bytes,
                 void *stream);
 
+/* Optional epilogue of the *_ex entry points (NULL = none): bias points at N device values of C's type
+ * (fp16, or bfloat16 for sk_gemm_bf16_ex) that are added to every row of C in fp32 before the rounding --
+ * the bias of a linear layer, which the reference leaves to a separate kernel.  Fix-ups are unaffected
+ * (partials stay unbiased; the CTA that stores a tile adds the bias).  reserved must be zero. */
+typedef struct sk_epilogue {
+  const void *bias;
+  int64_t reserved[3];
+} sk_epilogue;
+
+int sk_gemm_f16_ex(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                   int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws, size_t ws_bytes, void *stream,
+                   const sk_epilogue *epi);
+int sk_gemm_bf16_ex(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                    int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws, size_t ws_bytes, void *stream,
+                    const sk_epilogue *epi);
+/* Q4 with the epilogue: zeros == NULL is sk_gemm_q4 (plan dtype SK_Q4 or SK_Q4_TILED, scalar `zero`),
+ * otherwise sk_gemm_q4_zp (plan dtype SK_Q4_ZP, `zero` ignored). */
+int sk_gemm_q4_ex(const void *A, const void *Wq, const void *scales, const void *zeros, void *C, int64_t M,
+                  int64_t N, int64_t K, int64_t lda, int64_t ldc, int group, int zero, const sk_plan *plan,
+                  void *ws, size_t ws_bytes, void *stream, const sk_epilogue *epi);
+
 /* The same call for bfloat16 operands and output (fp32 accumulate, C rounded to nearest even); the
  * plan is made with dtype SK_BF16.  No counterpart in the reference, whose scripts are fp16 / fp32:
  * the tile kernels with the bfloat16 form of the MFMA.  Requirements as for sk_gemm_f16. */

@@ -182,7 +182,9 @@ extern "C" int sk_workspace_status(void *ws, void *stream) {
 
 static int gemm_16bit(int dtype, const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,
                       int64_t lda, int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws,
-                      size_t ws_bytes, void *stream) {
+                      size_t ws_bytes, void *stream, const sk_epilogue *epi = nullptr) {
+  const half_t *bias = epi ? (const half_t *)epi->bias : nullptr;
+  if (reinterpret_cast<uintptr_t>(bias) & 1) return SK_ERR_ALIGN;
   if (!A || !B || !C) return SK_ERR_NULL;
   int rc = check_plan(plan, M, N, K, dtype, plan ? plan->layout : 0);
   if (rc) return rc;
@@ -203,11 +205,11 @@ static int gemm_16bit(int dtype, const void *A, const void *B, void *C, int64_t 
   if (rc) return rc;
   int herr;
   if (skinny) {
-    SkinnyArgs a{(const half_t *)A, B, nullptr, (half_t *)C, (int)M, (int)N, (int)K, lda, ldb, ldc, 0, 0};
-    herr = launch_skinny(k->id, a, dp, w, (hipStream_t)stream);
+    SkinnyArgs a{(const half_t *)A, B, nullptr, (half_t *)C, (int)M, (int)N, (int)K, lda, ldb, ldc, 0, 0, nullptr};
+    herr = launch_skinny(k->id, a, dp, w, (hipStream_t)stream, bias);
   } else {
     GemmArgs a{(const half_t *)A, (const half_t *)B, (half_t *)C, (int)M, (int)N, (int)K, lda, ldb, ldc, 1.f};
-    herr = launch_tile_f16(k->id, a, dp, w, (hipStream_t)stream);
+    herr = launch_tile_f16(k->id, a, dp, w, (hipStream_t)stream, bias);
   }
   return herr == 0 ? SK_OK : SK_ERR_LAUNCH;
 }
@@ -216,6 +218,17 @@ extern "C" int sk_gemm_f16(const void *A, const void *B, void *C, int64_t M, int
                            int64_t lda, int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws,
                            size_t ws_bytes, void *stream) {
   return gemm_16bit(SK_F16, A, B, C, M, N, K, lda, ldb, ldc, plan, ws, ws_bytes, stream);
+}
+
+extern "C" int sk_gemm_f16_ex(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,
+                              int64_t lda, int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws,
+                              size_t ws_bytes, void *stream, const sk_epilogue *epi) {
+  return gemm_16bit(SK_F16, A, B, C, M, N, K, lda, ldb, ldc, plan, ws, ws_bytes, stream, epi);
+}
+extern "C" int sk_gemm_bf16_ex(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,
+                               int64_t lda, int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws,
+                               size_t ws_bytes, void *stream, const sk_epilogue *epi) {
+  return gemm_16bit(SK_BF16, A, B, C, M, N, K, lda, ldb, ldc, plan, ws, ws_bytes, stream, epi);
 }
 
 // bfloat16 kernels take the same 16-bit containers; only the MFMA and the rounding of C differ
@@ -246,7 +259,7 @@ static int gemm_8bit(int dtype, const void *A, const void *B, void *C, int64_t M
   rc = make_dev_plan(plan, k, ws, ws_bytes, cached_occupancy(k->id, false), (hipStream_t)stream, &dp, &w);
   if (rc) return rc;
   GemmArgs a{(const half_t *)A, (const half_t *)B, (half_t *)C, (int)M, (int)N, (int)(K / 2), lda / 2, ldb / 2, ldc, alpha};
-  return launch_tile_f16(k->id, a, dp, w, (hipStream_t)stream) == 0 ? SK_OK : SK_ERR_LAUNCH;
+  return launch_tile_f16(k->id, a, dp, w, (hipStream_t)stream, nullptr) == 0 ? SK_OK : SK_ERR_LAUNCH;
 }
 
 extern "C" int sk_gemm_f8(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,
@@ -291,7 +304,10 @@ extern "C" int sk_gemm_f32(const void *A, const void *B, void *C, int64_t M, int
 
 static int gemm_q4_any(const void *A, const void *Wq, const void *scales, const void *zeros, void *C, int64_t M,
                        int64_t N, int64_t K, int64_t lda, int64_t ldc, int group, int zero, int dtype,
-                       const sk_plan *plan, void *ws, size_t ws_bytes, void *stream) {
+                       const sk_plan *plan, void *ws, size_t ws_bytes, void *stream,
+                       const sk_epilogue *epi = nullptr) {
+  const half_t *bias = epi ? (const half_t *)epi->bias : nullptr;
+  if (reinterpret_cast<uintptr_t>(bias) & 1) return SK_ERR_ALIGN;
   if (!A || !Wq || !scales || !C || (dtype == SK_Q4_ZP && !zeros)) return SK_ERR_NULL;
   int rc = check_plan(plan, M, N, K, dtype, SK_LAYOUT_NT);
   if (rc) return rc;
@@ -311,7 +327,7 @@ static int gemm_q4_any(const void *A, const void *Wq, const void *scales, const 
   if (rc) return rc;
   SkinnyArgs a{(const half_t *)A, Wq, (const half_t *)scales, (half_t *)C, (int)M, (int)N, (int)K,
                lda, K / 2, ldc, zero, (int)(K / group), (const half_t *)zeros};
-  int herr = launch_skinny(k->id, a, dp, w, (hipStream_t)stream);
+  int herr = launch_skinny(k->id, a, dp, w, (hipStream_t)stream, bias);
   return herr == 0 ? SK_OK : SK_ERR_LAUNCH;
 }
 
@@ -320,6 +336,14 @@ extern "C" int sk_gemm_q4(const void *A, const void *Wq, const void *scales, voi
                           void *ws, size_t ws_bytes, void *stream) {
   const int dtype = plan && plan->dtype == SK_Q4_TILED ? SK_Q4_TILED : SK_Q4;  // which layout Wq is in
   return gemm_q4_any(A, Wq, scales, nullptr, C, M, N, K, lda, ldc, group, zero, dtype, plan, ws, ws_bytes, stream);
+}
+
+extern "C" int sk_gemm_q4_ex(const void *A, const void *Wq, const void *scales, const void *zeros, void *C,
+                             int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc, int group, int zero,
+                             const sk_plan *plan, void *ws, size_t ws_bytes, void *stream, const sk_epilogue *epi) {
+  const int dtype = zeros ? SK_Q4_ZP : (plan && plan->dtype == SK_Q4_TILED ? SK_Q4_TILED : SK_Q4);
+  return gemm_q4_any(A, Wq, scales, zeros, C, M, N, K, lda, ldc, group, zeros ? 0 : zero, dtype, plan, ws, ws_bytes,
+                     stream, epi);
 }
 
 extern "C" int sk_gemm_q4_zp(const void *A, const void *Wq, const void *scales, const void *zeros, void *C,

@@ -12,15 +12,28 @@ __global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_skinny_kernel(typen
   __shared__ __attribute__((aligned(16))) char smem[P::LDS_BYTES];
   run_persistent<P, FIXUP>(a, plan, ws, smem);
 }
+// the same with a bias row added in the epilogue (a second instance: see run_persistent)
+template <class P, bool FIXUP = true>
+__global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_skinny_kernel_bias(typename P::Args a, DevPlan plan, Workspace ws,
+                                                                               const void *bias) {
+  __shared__ __attribute__((aligned(16))) char smem[P::LDS_BYTES];
+  run_persistent<P, FIXUP, true>(a, plan, ws, smem, bias);
+}
 
 // launches without Stream-K tiles use the instance without fix-up code: these kernels run for a
 // few microseconds, most of which is set-up executed from a cold instruction cache
 template <class P>
-static int launch_policy(const SkinnyArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s) {
-  if (p.sk_tiles == 0)
+static int launch_policy(const SkinnyArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s, const void *bias) {
+  if (bias != nullptr) {
+    if (p.sk_tiles == 0)
+      hipLaunchKernelGGL((sk_skinny_kernel_bias<P, false>), dim3(p.grid), dim3(P::NT), 0, s, a, p, ws, bias);
+    else
+      hipLaunchKernelGGL((sk_skinny_kernel_bias<P, true>), dim3(p.grid), dim3(P::NT), 0, s, a, p, ws, bias);
+  } else if (p.sk_tiles == 0) {
     hipLaunchKernelGGL((sk_skinny_kernel<P, false>), dim3(p.grid), dim3(P::NT), 0, s, a, p, ws);
-  else
+  } else {
     hipLaunchKernelGGL((sk_skinny_kernel<P, true>), dim3(p.grid), dim3(P::NT), 0, s, a, p, ws);
+  }
   return (int)hipGetLastError();
 }
 
@@ -87,47 +100,47 @@ int skinny_kernel_infos(KernelInfo *out, int max) {
   return n;
 }
 
-int launch_skinny(int id, const SkinnyArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s) {
+int launch_skinny(int id, const SkinnyArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s, const void *bias) {
   switch (id) {
 #define X(id_, MB, NB, WN, RK, Q4, DEPTH, ROW1)                                                \
   case id_: {                                                                              \
     typedef SK_POLICY(MB, NB, WN, RK, Q4, DEPTH, ROW1) P;                                        \
-    return launch_policy<P>(a, p, ws, s);                                                         \
+    return launch_policy<P>(a, p, ws, s, bias);                                                         \
   }
     SK_SKINNY_KERNELS(X)
 #undef X
 #define X(id_, NB, WN, RK, DEPTH, KMAX)                                                        \
   case id_: {                                                                              \
     typedef TileGemvQ4<NB, WN, RK, DEPTH, KMAX> P;                                          \
-    return launch_policy<P>(a, p, ws, s);                                                         \
+    return launch_policy<P>(a, p, ws, s, bias);                                                         \
   }
     SK_GEMV_Q4_KERNELS(X)
 #undef X
 #define X(id_, NB, WN, RK, DEPTH, KMAX)                                                        \
   case id_: {                                                                              \
     typedef TileGemvF16<NB, WN, RK, DEPTH, KMAX> P;                                         \
-    return launch_policy<P>(a, p, ws, s);                                                         \
+    return launch_policy<P>(a, p, ws, s, bias);                                                         \
   }
     SK_GEMV_F16_KERNELS(X)
 #undef X
 #define X(id_, MB, NB, WN, RK, DEPTH)                                                       \
   case id_: {                                                                              \
     typedef TileSkinny<MB, NB, WN, RK, true, DEPTH, false, true> P;                        \
-    return launch_policy<P>(a, p, ws, s);                                                         \
+    return launch_policy<P>(a, p, ws, s, bias);                                                         \
   }
     SK_SKINNY_Q4T_KERNELS(X)
 #undef X
 #define X(id_, MB, NB, WN, RK, DEPTH)                                                       \
   case id_: {                                                                              \
     typedef TileSkinny<MB, NB, WN, RK, true, DEPTH, false, false, true> P;                 \
-    return launch_policy<P>(a, p, ws, s);                                                         \
+    return launch_policy<P>(a, p, ws, s, bias);                                                         \
   }
     SK_SKINNY_Q4ZP_KERNELS(X)
 #undef X
 #define X(id_, NB, WN, RK, DEPTH, KMAX)                                                     \
   case id_: {                                                                              \
     typedef TileGemvQ4<NB, WN, RK, DEPTH, KMAX, true> P;                                    \
-    return launch_policy<P>(a, p, ws, s);                                                         \
+    return launch_policy<P>(a, p, ws, s, bias);                                                         \
   }
     SK_GEMV_Q4T_KERNELS(X)
 #undef X

@@ -4,19 +4,21 @@
 
 namespace sk {
 
+// bias: optional row added in the epilogue (null: none); one instance serves both cases, the epilogue branches
 template <class P, bool FIXUP = true>
-__global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_tile_kernel(typename P::Args a, DevPlan plan, Workspace ws) {
+__global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_tile_kernel(typename P::Args a, DevPlan plan, Workspace ws,
+                                                                        const void *bias) {
   __shared__ __attribute__((aligned(16))) char smem[P::LDS_BYTES];  // policies with their own LDS arrays keep this at 16 bytes
-  run_persistent<P, FIXUP>(a, plan, ws, smem);
+  run_persistent<P, FIXUP, true>(a, plan, ws, smem, bias);
 }
 
 // data-parallel launches of the direct-to-LDS kernels use the instance without fix-up code
 template <class P>
-static int launch_dma(const GemmArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s) {
+static int launch_dma(const GemmArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s, const void *bias) {
   if (p.sk_tiles == 0)
-    hipLaunchKernelGGL((sk_tile_kernel<P, false>), dim3(p.grid), dim3(P::NT), 0, s, a, p, ws);
+    hipLaunchKernelGGL((sk_tile_kernel<P, false>), dim3(p.grid), dim3(P::NT), 0, s, a, p, ws, bias);
   else
-    hipLaunchKernelGGL((sk_tile_kernel<P, true>), dim3(p.grid), dim3(P::NT), 0, s, a, p, ws);
+    hipLaunchKernelGGL((sk_tile_kernel<P, true>), dim3(p.grid), dim3(P::NT), 0, s, a, p, ws, bias);
   return (int)hipGetLastError();
 }
 
@@ -117,12 +119,12 @@ int tile_kernel_infos(KernelInfo *out, int max) {
   return n;
 }
 
-int launch_tile_f16(int id, const GemmArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s) {
+int launch_tile_f16(int id, const GemmArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s, const void *bias) {
   switch (id) {
 #define X(id_, BM, BN, BK, WM, WN)                                                       \
   case id_: {                                                                            \
     typedef SK_POLICY(id_, BM, BN, BK, WM, WN) P;                                        \
-    hipLaunchKernelGGL(sk_tile_kernel<P>, dim3(p.grid), dim3(P::NT), 0, s, a, p, ws);    \
+    hipLaunchKernelGGL(sk_tile_kernel<P>, dim3(p.grid), dim3(P::NT), 0, s, a, p, ws, bias);    \
     return (int)hipGetLastError();                                                       \
   }
     SK_TILE_F16_NT_KERNELS(X)
@@ -130,63 +132,63 @@ int launch_tile_f16(int id, const GemmArgs &a, const DevPlan &p, const Workspace
 #define X(id_, BM, BN, WM, WN)                                                           \
   case id_: {                                                                            \
     typedef SK_POLICY_DMA(id_, BM, BN, WM, WN) P;                                      \
-    return launch_dma<P>(a, p, ws, s);                                                       \
+    return launch_dma<P>(a, p, ws, s, bias);                                                       \
   }
     SK_TILE_F16_NT_DMA_KERNELS(X)
 #undef X
 #define X(id_, BM, BN, WM, WN)                                                           \
   case id_: {                                                                            \
     typedef SK_POLICY_NN(id_, BM, BN, WM, WN) P;                                      \
-    return launch_dma<P>(a, p, ws, s);                                                       \
+    return launch_dma<P>(a, p, ws, s, bias);                                                       \
   }
     SK_TILE_F16_NN_DMA_KERNELS(X)
 #undef X
 #define X(id_, BM, BN, WM, WN)                                                           \
   case id_: {                                                                            \
     typedef SK_POLICY_DMA32(id_, BM, BN, WM, WN) P;                                      \
-    return launch_dma<P>(a, p, ws, s);                                                       \
+    return launch_dma<P>(a, p, ws, s, bias);                                                       \
   }
     SK_TILE_F16_NT_DMA32_KERNELS(X)
 #undef X
 #define X(id_, BM, BN, WM, WN)                                                           \
   case id_: {                                                                            \
     typedef SK_POLICY_DMA16(id_, BM, BN, WM, WN) P;                                      \
-    return launch_dma<P>(a, p, ws, s);                                                       \
+    return launch_dma<P>(a, p, ws, s, bias);                                                       \
   }
     SK_TILE_F16_NT_DMA16_KERNELS(X)
 #undef X
 #define X(id_, BM, BN, WM, WN)                                                           \
   case id_: {                                                                            \
     typedef SK_POLICY_DMA32_16(id_, BM, BN, WM, WN) P;                                   \
-    return launch_dma<P>(a, p, ws, s);                                                       \
+    return launch_dma<P>(a, p, ws, s, bias);                                                       \
   }
     SK_TILE_F16_NT_DMA32_16_KERNELS(X)
 #undef X
 #define X(id_, BM, BN, WM, WN)                                                           \
   case id_: {                                                                            \
     typedef SK_POLICY_NN16(id_, BM, BN, WM, WN) P;                                       \
-    return launch_dma<P>(a, p, ws, s);                                                       \
+    return launch_dma<P>(a, p, ws, s, bias);                                                       \
   }
     SK_TILE_F16_NN_DMA16_KERNELS(X)
 #undef X
 #define X(id_, BM, BN, WM, WN, BK, NN)                                                   \
   case id_: {                                                                            \
     typedef SK_POLICY_BF16(id_, BM, BN, WM, WN, BK, NN) P;                               \
-    return launch_dma<P>(a, p, ws, s);                                                       \
+    return launch_dma<P>(a, p, ws, s, bias);                                                       \
   }
     SK_TILE_BF16_KERNELS(X)
 #undef X
 #define X(id_, BM, BN, WM, WN)                                                           \
   case id_: {                                                                            \
     typedef SK_POLICY_F8(id_, BM, BN, WM, WN) P;                                         \
-    return launch_dma<P>(a, p, ws, s);                                                   \
+    return launch_dma<P>(a, p, ws, s, bias);                                                   \
   }
     SK_TILE_F8_KERNELS(X)
 #undef X
 #define X(id_, BM, BN, WM, WN)                                                           \
   case id_: {                                                                            \
     typedef SK_POLICY_I8(id_, BM, BN, WM, WN) P;                                         \
-    return launch_dma<P>(a, p, ws, s);                                                   \
+    return launch_dma<P>(a, p, ws, s, bias);                                                   \
   }
     SK_TILE_I8_KERNELS(X)
 #undef X

@@ -17,8 +17,9 @@ int tile_kernel_infos(KernelInfo *out, int max);
 int skinny_kernel_infos(KernelInfo *out, int max);
 
 // return hipError_t as int; occupancy_* return co-resident CTAs per CU (<= 0 on error)
-int launch_tile_f16(int id, const GemmArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s);
-int launch_skinny(int id, const SkinnyArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s);
+// bias: optional row of N values of C's type added in the epilogue (null: none)
+int launch_tile_f16(int id, const GemmArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s, const void *bias);
+int launch_skinny(int id, const SkinnyArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s, const void *bias);
 int f32_kernel_infos(KernelInfo *out, int max);
 int launch_f32(int id, const GemmArgsF32 &a, const DevPlan &p, const Workspace &ws, hipStream_t s);
 int occupancy_f32(int id);

@@ -222,6 +222,45 @@ __device__ __forceinline__ T *pin_here(T *p) {
   return p;
 }
 
+// the same for a lane-dependent integer (column arithmetic of an epilogue operand)
+__device__ __forceinline__ int pin_here(int x) {
+  asm volatile("" : "+v"(x));
+  return x;
+}
+
+// optional epilogue operand: a row vector added to every row of C in fp32, before the rounding to C's type
+// (fp16 bits, or bfloat16 bits when BF16).  Returns 0 without a bias or past the last column.
+template <bool BF16 = false>
+__device__ __forceinline__ float bias_at(const half_t *bias, int col, int N) {
+  if (bias == nullptr || col >= N) return 0.f;
+  if constexpr (BF16) {
+    const uint32_t bits = (uint32_t)__builtin_bit_cast(uint16_t, bias[col]) << 16;
+    return __builtin_bit_cast(float, bits);
+  } else {
+    return (float)bias[col];
+  }
+}
+
+// four consecutive bias values starting at column col (a multiple of 4): one 8-byte load where the row allows it
+template <bool BF16 = false>
+__device__ __forceinline__ floatx4 bias4_at(const half_t *bias, int col, int N) {
+  floatx4 r;
+  if (col + 4 <= N && (reinterpret_cast<uintptr_t>(bias) & 7) == 0) {
+    const half4v h = *reinterpret_cast<const half4v *>(bias + col);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if constexpr (BF16)
+        r[e] = __builtin_bit_cast(float, (uint32_t)__builtin_bit_cast(uint16_t, (half_t)h[e]) << 16);
+      else
+        r[e] = (float)h[e];
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) r[e] = bias_at<BF16>(bias, col + e, N);
+  }
+  return r;
+}
+
 __device__ __forceinline__ void atomic_add_f32(float *p, float v) {
   // hardware global_atomic_add_f32, no return value, device scope
   __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -3,7 +3,7 @@
 // A policy class P supplies the tile arithmetic:
 //   P::Args, P::Acc, P::TILE_ELEMS, P::NT
 //   P::mac(args, acc, pm, pn, k0, n, smem)      accumulate K-iterations [k0, k0+n) of tile (pm,pn)
-//   P::store_c(args, acc, pm, pn, smem)         write the finished tile to C
+//   P::store_c(args, acc, pm, pn, smem, bias)   write the finished tile to C (+ optional bias row)
 //   P::store_partial / add_partial / atomic_partial / take_partial   fp32 partials in workspace
 //
 // Control flow follows the reference's persistent kernel: every CTA first walks its share of the
@@ -16,19 +16,33 @@ namespace sk {
 // FIXUP = false: an instance for launches without Stream-K tiles.  Every segment is a whole tile
 // and the fix-up code is not compiled in -- its hundreds of partial-tile addresses otherwise
 // shape the register allocation of the main loop (spills in the 256x256 kernels).
-template <class P, bool FIXUP = true>
+// BIAS: the kernel has the optional bias row among its arguments (bias_arg, may still be null); without it the
+// epilogue's bias code is not compiled in.  The small-M kernels exist in both forms, because even an unused
+// bias argument costs them 0.2-0.3 us of their 7-12 us (argument loads and waits at kernel entry move).
+template <class P, bool FIXUP = true, bool BIAS = false>
 __device__ __forceinline__ void run_persistent(const typename P::Args &a, const DevPlan &plan,
-                                               const Workspace &ws, char *smem) {
+                                               const Workspace &ws, char *smem, const void *bias_arg = nullptr) {
   __shared__ int s_word;
+  // Fetch the bias pointer with the other kernel arguments: left to the compiler it is read from the argument
+  // buffer right before the first store, a dependent scalar load (~0.3 us) at the end of every CTA.
+  const void *bias = nullptr;
+  if constexpr (BIAS) {
+    bias = bias_arg;
+    asm volatile("" ::"s"(bias));
+  }
   SK_TRACE(0);
   const int pid = logical_pid(plan);
   const int ipt = plan.ipt;
   typename P::Acc acc;
 
-  int start, last;
-  sk_range(plan, pid, start, last);
+  // The instance without fix-up code is only launched for plans without Stream-K tiles, whose range is empty.
+  // P::LEAN_ENTRY: leave its computation out there.  Worth 0.8 % to the 256x256 tile kernels at 8192^3; the
+  // small-M kernels start 0.2-0.3 us later without it (their argument loads get ordered differently), so they
+  // keep it.
+  int start = 0, last = 0;
+  if constexpr (FIXUP || !P::LEAN_ENTRY) sk_range(plan, pid, start, last);
   SK_TRACE(10);
-  int dp_tile = plan.sk_tiles + pid;
+  int dp_tile = (FIXUP || !P::LEAN_ENTRY) ? plan.sk_tiles + pid : pid;
 
   // One loop body serves both phases so that the MAC loop and the epilogue exist once in the
   // kernel: first the CTA's Stream-K segments, then its data-parallel tiles
@@ -95,7 +109,7 @@ __device__ __forceinline__ void run_persistent(const typename P::Args &a, const 
       }
     }
     SK_TRACE(8);
-    if (store) P::store_c(a, acc, pm, pn, smem);
+    if (store) P::store_c(a, acc, pm, pn, smem, bias);
     SK_TRACE(9);
   }
 }

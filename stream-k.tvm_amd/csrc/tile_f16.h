@@ -22,6 +22,7 @@ struct GemmArgs {
 template <int BM_, int BN_, int BK_, int WM_, int WN_>
 struct TileF16NT {
   typedef GemmArgs Args;
+  static constexpr bool LEAN_ENTRY = true;  // see run_persistent
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
   static constexpr int NT = WM * WN * 64;
   static constexpr int TM = BM / (WM * 32), TN = BN / (WN * 32);
@@ -139,11 +140,21 @@ struct TileF16NT {
 
   // fp32 -> fp16, through a per-wave LDS patch so that global stores are 16 bytes per lane and
   // 128 bytes contiguous per row.
-  static __device__ __forceinline__ void store_c(const Args &a, const Acc &acc, int pm, int pn,
-                                                 char *smem) {
+  // (two copies behind one uniform branch, so that the epilogue without a bias carries none of its code)
+  static __device__ __forceinline__ void store_c(const Args &a, const Acc &acc, int pm, int pn, char *smem,
+                                                 const void *bias) {
+    if (bias == nullptr)
+      store_c_impl<false>(a, acc, pm, pn, smem, nullptr);
+    else
+      store_c_impl<true>(a, acc, pm, pn, smem, static_cast<const half_t *>(bias));
+  }
+  template <bool BIAS>
+  static __device__ __forceinline__ void store_c_impl(const Args &a, const Acc &acc, int pm, int pn, char *smem,
+                                                      const half_t *bias) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
     half_t *patch = reinterpret_cast<half_t *>(smem) + wave * (WTM * LDC);
+    const int bias_col0 = BIAS ? pn * BN + wn * WTN + pin_here(lane >> 5) * 4 : 0;  // not hoisted out of the persistent loop
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -152,7 +163,11 @@ struct TileF16NT {
         for (int q = 0; q < 4; ++q) {
           half4v h;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) h[e] = (half_t)acc.c[i][j][q * 4 + e];
+          for (int e = 0; e < 4; ++e) {
+            float x = acc.c[i][j][q * 4 + e];
+            if constexpr (BIAS) x += bias_at(bias, bias_col0 + j * 32 + q * 8 + e, a.N);
+            h[e] = (half_t)x;
+          }
           *reinterpret_cast<half4v *>(patch + (i * 32 + (lane & 31)) * LDC + j * 32 + q * 8 +
                                       (lane >> 5) * 4) = h;
         }

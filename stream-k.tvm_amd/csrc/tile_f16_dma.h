@@ -89,6 +89,7 @@ struct TileF16NTDma {
   static constexpr int B_ROWS_PER_DMA = 1024 / B_ROW_BYTES;    // rows one wave-wide load fills
   static_assert(!B_KN_ || (BN_ >= 128 && BN_ <= 512), "NN layout: 16..64 chunks per LDS row");
   typedef GemmArgs Args;
+  static constexpr bool LEAN_ENTRY = true;  // see run_persistent
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
   static constexpr int NW = WM * WN, NT = NW * 64;
   static constexpr int TM = BM / (WM * 32), TN = BN / (WN * 32);
@@ -613,7 +614,18 @@ struct TileF16NTDma {
     __syncthreads();
   }
 
-  static __device__ __forceinline__ void store_c(const Args &a, const Acc &acc, int pm, int pn, char *) {
+  // two copies of the epilogue behind one uniform branch: the one without a bias is the code the kernel had
+  // before the bias existed (bias loads inside a single epilogue cost the 256x256 kernel 6 % at 8192^3)
+  static __device__ __forceinline__ void store_c(const Args &a, const Acc &acc, int pm, int pn, char *smem,
+                                                 const void *bias) {
+    if (bias == nullptr)
+      store_c_impl<false>(a, acc, pm, pn, smem, nullptr);
+    else
+      store_c_impl<true>(a, acc, pm, pn, smem, static_cast<const half_t *>(bias));
+  }
+  template <bool BIAS>
+  static __device__ __forceinline__ void store_c_impl(const Args &a, const Acc &acc, int pm, int pn, char *,
+                                                      const half_t *bias) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
     if constexpr (I8) {
@@ -638,6 +650,9 @@ struct TileF16NTDma {
         }
       return;
     }
+    // first column of this lane's accumulator groups, for the bias; computed here, from a value the compiler cannot
+    // see through, so that it is not hoisted out of the persistent loop and kept in a register across the main loop
+    const int bias_col0 = BIAS ? pn * BN + wn * WTN + pin_here(lane >> (MFMA16 ? 4 : 5)) * 4 : 0;
     half_t *patch = reinterpret_cast<half_t *>(stage(wave / WAVES_PER_STAGE)) +
                     (wave % WAVES_PER_STAGE) * (PATCH_ROWS * LDC);
     const bool vec_ok = (a.ldc % 8 == 0) && ((reinterpret_cast<uintptr_t>(a.C) & 15) == 0);
@@ -652,9 +667,12 @@ struct TileF16NTDma {
 #pragma unroll
           for (int j = 0; j < FN; ++j) {
             half4v h;
+            floatx4 bv = {0.f, 0.f, 0.f, 0.f};
+            if constexpr (BIAS) bv = bias4_at<BF16_>(bias, bias_col0 + j * 16, a.N);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-              const float x = acc.v[p * (PATCH_ROWS / 16) + ib][j][e];
+              float x = acc.v[p * (PATCH_ROWS / 16) + ib][j][e];
+              if constexpr (BIAS) x += bv[e];
               if constexpr (BF16_) {
                 const __bf16 b = (__bf16)x;
                 h[e] = __builtin_bit_cast(half_t, b);  // the patch only carries 16-bit patterns
@@ -672,12 +690,14 @@ struct TileF16NTDma {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
               half4v h;
+              floatx4 bv = {0.f, 0.f, 0.f, 0.f};
+              if constexpr (BIAS) bv = bias4_at(bias, bias_col0 + j * 32 + q * 8, a.N);
 #pragma unroll
               for (int e = 0; e < 4; ++e) {
-                if constexpr (F8 != 0)  // the product of fp8 operands is scaled before it is rounded to fp16
-                  h[e] = (half_t)(a.alpha * (float)acc.c[p * BLK + ib][j][q * 4 + e]);
-                else
-                  h[e] = (half_t)acc.c[p * BLK + ib][j][q * 4 + e];
+                float x = acc.c[p * BLK + ib][j][q * 4 + e];
+                if constexpr (F8 != 0) x *= a.alpha;  // the product of fp8 operands is scaled before it is rounded to fp16
+                if constexpr (BIAS) x += bv[e];
+                h[e] = (half_t)x;
               }
               *reinterpret_cast<half4v *>(patch + (ib * 32 + (lane & 31)) * LDC + j * 32 + q * 8 +
                                           (lane >> 5) * 4) = h;

@@ -23,6 +23,7 @@ struct GemmArgsF32 {
 template <bool B_KN_, int BM_ = 128, int BN_ = 128, int WM_ = 2, int WN_ = 2>
 struct TileF32 {
   typedef GemmArgsF32 Args;
+  static constexpr bool LEAN_ENTRY = true;  // see run_persistent
   static constexpr bool B_KN = B_KN_;
   static constexpr int BM = BM_, BN = BN_, BK = 16, WM = WM_, WN = WN_;
   static constexpr int NT = 256, TM = BM / (WM * 32), TN = BN / (WN * 32), WTM = TM * 32, WTN = TN * 32;
@@ -135,7 +136,8 @@ struct TileF32 {
   }
 
   // acc.c[i][j][r] = C[pm*BM + wm*WTM + i*32 + 8*(r/4) + 4*(lane/32) + r%4][pn*BN + wn*WTN + j*32 + lane%32]
-  static __device__ __forceinline__ void store_c(const Args &a, const Acc &acc, int pm, int pn, char *) {
+  static __device__ __forceinline__ void store_c(const Args &a, const Acc &acc, int pm, int pn, char *,
+                                                 const void * /*bias: not offered for fp32*/) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
 #pragma unroll

@@ -44,6 +44,7 @@ namespace sk {
 template <int NB_, int WN_, int RK_, int DEPTH_, int KMAX_ = 16384, bool TILED_ = false>
 struct TileGemvQ4 {
   typedef SkinnyArgs Args;
+  static constexpr bool LEAN_ENTRY = false;  // see run_persistent
   static constexpr int NB = NB_, WN = WN_, RK = RK_, DEPTH = DEPTH_, KMAX = KMAX_;
   static constexpr int BM = 16, BN = 16 * NB * WN;
   static constexpr int BK = 256;        // K per wave per iteration: two 16-byte loads per lane and block
@@ -288,13 +289,23 @@ struct TileGemvQ4 {
     return tid < WN * 64 && (tid & 3) == 0;
   }
 
-  static __device__ __forceinline__ void store_c(const Args &a, const Acc &acc, int /*pm*/, int pn, char *) {
+  static __device__ __forceinline__ void store_c(const Args &a, const Acc &acc, int /*pm*/, int pn, char *,
+                                                 const void *bias_) {
     int e;
     if (!owns_output(e)) return;
+    const half_t *bias = static_cast<const half_t *>(bias_);
+    if (bias == nullptr) {  // the common case keeps the code it had before the bias existed
 #pragma unroll
-    for (int j = 0; j < NB; ++j) {
-      const int col = pn * BN + e + j * 16;
-      if (col < a.N) a.C[col] = (half_t)acc.y[j];
+      for (int j = 0; j < NB; ++j) {
+        const int col = pn * BN + e + j * 16;
+        if (col < a.N) a.C[col] = (half_t)acc.y[j];
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < NB; ++j) {
+        const int col = pn * BN + e + j * 16;
+        if (col < a.N) a.C[col] = (half_t)(acc.y[j] + (float)bias[col]);
+      }
     }
   }
   static __device__ __forceinline__ void store_partial(const Acc &acc, float *dst) {

@@ -106,6 +106,7 @@ struct TileSkinny {
   static_assert(!TILED_ || Q4_, "tiled weights exist for Q4");
   static_assert(!ZP_ || Q4_, "zero points exist for Q4");
   typedef SkinnyArgs Args;
+  static constexpr bool LEAN_ENTRY = false;  // see run_persistent
   static constexpr int MB = MB_, NB = NB_, WN = WN_, RK = RK_, DEPTH = DEPTH_;
   static constexpr bool Q4 = Q4_;
   static constexpr int BM = 16 * MB, BN = 16 * NB * WN;
@@ -351,7 +352,17 @@ struct TileSkinny {
   }
 
   // acc.c[i][j][r] = C[pm*BM + i*16 + lane%16][pn*BN + (wn*NB + j)*16 + 4*(lane/16) + r]
-  static __device__ __forceinline__ void store_c(const Args &a, const Acc &acc, int pm, int pn, char *) {
+  // (two copies behind one uniform branch: the epilogue without a bias carries none of its code)
+  static __device__ __forceinline__ void store_c(const Args &a, const Acc &acc, int pm, int pn, char *smem,
+                                                 const void *bias) {
+    if (bias == nullptr)
+      store_c_impl<false>(a, acc, pm, pn, smem, nullptr);
+    else
+      store_c_impl<true>(a, acc, pm, pn, smem, static_cast<const half_t *>(bias));
+  }
+  template <bool BIAS>
+  static __device__ __forceinline__ void store_c_impl(const Args &a, const Acc &acc, int pm, int pn, char *,
+                                                      const half_t *bias) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     if (wave >= WN) return;
     const int lr = lane & 15, lg = lane >> 4;
@@ -365,7 +376,11 @@ struct TileSkinny {
         if (row < a.M && col < a.N) {
           half4v h;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) h[e] = (half_t)acc.c[i][j][e];
+          for (int e = 0; e < 4; ++e) {
+            float x = acc.c[i][j][e];
+            if constexpr (BIAS) x += bias_at(bias, col + e, a.N);
+            h[e] = (half_t)x;
+          }
           half_t *dst = a.C + (int64_t)row * a.ldc + col;
           if (vec_ok && col + 4 <= a.N) {
             *reinterpret_cast<half4v *>(dst) = h;

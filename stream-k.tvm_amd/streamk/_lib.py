@@ -34,6 +34,11 @@ class SkPlan(ctypes.Structure):
         return {n: getattr(self, n) for n, _ in self._fields_}
 
 
+class SkEpilogue(ctypes.Structure):
+    """sk_epilogue: optional operands of the *_ex entry points."""
+    _fields_ = [("bias", ctypes.c_void_p), ("reserved", ctypes.c_int64 * 3)]
+
+
 class StreamKError(RuntimeError):
     def __init__(self, status, where):
         self.status = status
@@ -82,6 +87,12 @@ def lib():
     L.sk_q4_quantize_zp_host.restype = ci
     L.sk_q4_quantize_zp.argtypes = [vp, i64, i64, i64, ci, vp, vp, vp, vp]
     L.sk_q4_quantize_zp.restype = ci
+    L.sk_gemm_f16_ex.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, P(SkPlan), vp, sz, vp, P(SkEpilogue)]
+    L.sk_gemm_f16_ex.restype = ci
+    L.sk_gemm_bf16_ex.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, P(SkPlan), vp, sz, vp, P(SkEpilogue)]
+    L.sk_gemm_bf16_ex.restype = ci
+    L.sk_gemm_q4_ex.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, ci, ci, P(SkPlan), vp, sz, vp, P(SkEpilogue)]
+    L.sk_gemm_q4_ex.restype = ci
     L.sk_gemm_f8.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, ctypes.c_float, P(SkPlan), vp, sz, vp]
     L.sk_gemm_f8.restype = ci
     L.sk_gemm_i8.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, P(SkPlan), vp, sz, vp]

@@ -77,14 +77,13 @@ class StreamKLinear(torch.nn.Module):
         M = a.shape[0]
         if M == 0:
             return x.new_zeros(*lead, self.out_features)
+        # the bias is added in the GEMM's epilogue (fp32, before the rounding to fp16)
         if self.weight_format == "float16":
-            c = ops.streamk_fp16(a, self.weight, plan=self.plan_for(M))
+            c = ops.streamk_fp16(a, self.weight, plan=self.plan_for(M), bias=self.bias)
         else:
             # (more rows than one Q4 launch takes: streamk_q4 splits the call itself)
             c = ops.streamk_q4(a, self.qweight, self.scales, plan=self.plan_for(M) if M <= ops.Q4_MAX_M else None,
-                               zero=self.zero, group=self.group, zeros=getattr(self, "zeros", None))
-        if self.bias is not None:
-            c += self.bias
+                               zero=self.zero, group=self.group, zeros=getattr(self, "zeros", None), bias=self.bias)
         return c.view(*lead, self.out_features)
 
     def extra_repr(self):

@@ -631,6 +631,69 @@ def test_int8_tile_kernels(sk, oracle):
     sk.workspace_status()
 
 
+def test_fused_bias_epilogue(sk, oracle):
+    """bias (one value per column, C's type) added in fp32 before the rounding: every kernel family (LDS-tiled
+    with both accumulator layouts and the register-staged variant, NN, bfloat16, small-M, matrix-vector, Q4 in
+    all formats), data-parallel and both fix-ups, ragged N; {-1,0,1} operands with an integer bias must come out
+    exact, which also shows that the bias is added once per tile however many CTAs share it."""
+    import torch
+    rng = np.random.default_rng(91)
+    cases = [  # (M, N, K, layout, config)
+        (200, 1000, 328, "nt", dict(bm=256, bn=256, bk=64, variant=5)), (200, 1000, 328, "nt", dict(bm=128, bn=128, bk=64, variant=2)),
+        (200, 1000, 328, "nt", dict(bm=128, bn=128, bk=64, variant=1)), (200, 1000, 328, "nt", dict(bm=64, bn=64, bk=32, variant=6)),
+        (200, 1000, 328, "nn", dict(bm=128, bn=128, bk=64, variant=5)), (200, 1000, 328, "nn", dict(bm=256, bn=256, bk=64, variant=2)),
+        (40, 1000, 1024, "nt", dict(bm=64, bn=64, bk=128)), (9, 1000, 1024, "nt", dict(bm=16, bn=32, bk=512)),
+        (1, 1000, 1024, "nt", dict(bm=16, bn=16, bk=512, variant=3)), (1, 1000, 1024, "nt", dict(bm=16, bn=64, bk=128, variant=2)),
+    ]
+    for (M, N, K, layout, cfg) in cases:
+        A = rng.integers(-1, 2, (M, K)).astype(np.float16)
+        B = rng.integers(-1, 2, (N, K) if layout == "nt" else (K, N)).astype(np.float16)
+        bias = rng.integers(-300, 300, N).astype(np.float16)
+        want = (A.astype(np.float64) @ (B.T if layout == "nt" else B).astype(np.float64)) + bias.astype(np.float64)
+        Af = (rng.random((M, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+        bf = (rng.random(N, dtype=np.float32) * 20 - 10).astype(np.float16)
+        reff = oracle.matmul_fp32(Af, B, trans_b=layout == "nt") + bf.astype(np.float32)
+        for sch in (dict(schedule="dp"), dict(schedule="basic", fixup="reduce", grid=12), dict(schedule="sk2", fixup="atomic", grid=10)):
+            plan = sk.make_plan(M, N, K, "float16", layout, dict(cfg, **sch))
+            C = sk.streamk_fp16(_t(A), _t(B), layout=layout, plan=plan, bias=_t(bias))
+            assert np.array_equal(C.double().cpu().numpy(), want), (M, N, K, layout, cfg, sch)
+            C = sk.streamk_fp16(_t(Af), _t(B), layout=layout, plan=plan, bias=_t(bf))
+            assert _rel(oracle, C, reff) <= 1e-3, (M, N, K, layout, cfg, sch)
+    # bfloat16: the bias vector is bfloat16 too
+    A, B = torch.randint(-1, 2, (200, 328)).bfloat16(), torch.randint(-1, 2, (1000, 328)).bfloat16()
+    bias = torch.randint(-100, 100, (1000,)).bfloat16()
+    want = A.double() @ B.double().T + bias.double()
+    for cfg in (dict(bm=256, bn=256, bk=64), dict(bm=64, bn=64, bk=32, schedule="basic", fixup="reduce", grid=12)):
+        C = sk.streamk_bf16(A.cuda(), B.cuda(), bias=bias.cuda(), **cfg)
+        assert torch.equal(C.double().cpu(), want), cfg
+    # Q4: general small-M, single row, matrix-vector, tiled and per-group zero points
+    M, N, K = 5, 1000, 1152
+    Wq = rng.integers(0, 256, (N, K // 2), dtype=np.uint8)
+    sc = rng.uniform(0.005, 0.02, (N, K // 128)).astype(np.float16)
+    zp = rng.integers(0, 16, (N, K // 128)).astype(np.float16)
+    bias = (rng.random(N, dtype=np.float32) * 8 - 4).astype(np.float16)
+    for m in (M, 1):
+        A = (rng.random((m, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+        ref = oracle.q4_gemm_ref(A, Wq, sc, 128, 8) + bias.astype(np.float32)
+        refz = oracle.q4_zp_gemm_ref(A, Wq, sc, zp) + bias.astype(np.float32)
+        for sch in (dict(schedule="dp"), dict(schedule="sk2", fixup="reduce", grid=48), dict(schedule="sk2", fixup="atomic", grid=40)):
+            for variant in ((1,) if m > 1 else (1, 2, 3)):
+                C = sk.streamk_q4(_t(A), _t(Wq), _t(sc), bias=_t(bias), variant=variant, **sch)
+                assert _rel(oracle, C, ref) <= 2e-3, (m, variant, sch)
+            C = sk.streamk_q4(_t(A), sk.tile_q4(_t(Wq)), _t(sc), tiled=True, bias=_t(bias), **sch)
+            assert _rel(oracle, C, ref) <= 2e-3, (m, "tiled", sch)
+            C = sk.streamk_q4(_t(A), _t(Wq), _t(sc), zeros=_t(zp), bias=_t(bias), **sch)
+            assert _rel(oracle, C, refz) <= 2e-3, (m, "zp", sch)
+    X, Y = torch.zeros(8, 64, dtype=torch.float16, device="cuda"), torch.zeros(24, 64, dtype=torch.float16, device="cuda")
+    with pytest.raises(ValueError):
+        sk.streamk_fp16(X, Y, bias=torch.zeros(10, dtype=torch.float16, device="cuda"))
+    with pytest.raises(ValueError):
+        sk.streamk_fp16(X, Y, bias=torch.zeros(24, dtype=torch.float32, device="cuda"))
+    with pytest.raises(ValueError):
+        sk.streamk_fp16(X, Y, bias=torch.zeros(24, dtype=torch.float16))
+    sk.workspace_status()
+
+
 def test_cfg5_large_dense(sk, oracle):
     """M = N = K = 8192 and the irregular 3000 x 5120 x 12288, U[-1,1): a random subset of rows is
     checked against an fp64 host product; the Stream-K and data-parallel schedules of the same kernel
