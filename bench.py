@@ -324,6 +324,21 @@ def main():
                 del tiles
             q4.append(row)
         extra["q4_N8192_K8192"] = q4
+
+        # offline side of the Q4 path on the same weight shape: algorithmic bytes over graph-timed launches
+        Wf = (torch.randn(N, K, generator=g) * 0.05).half().cuda()
+        _, _, zp = streamk.quantize_q4(Wf, asymmetric=True)
+        rd, wqb, scb = N * K * 2, N * K // 2, N * (K // 128) * 2
+        tools = {}
+        for name, fn, nbytes in (("quantize_q4", lambda: streamk.quantize_q4(Wf), rd + wqb + scb),
+                                 ("quantize_q4_asymmetric", lambda: streamk.quantize_q4(Wf, asymmetric=True), rd + wqb + 2 * scb),
+                                 ("dequant_q4", lambda: streamk.dequant_q4(Wq, sc), wqb + scb + rd),
+                                 ("dequant_q4_zero_points", lambda: streamk.dequant_q4(Wq, sc, zeros=zp), wqb + 2 * scb + rd),
+                                 ("tile_q4", lambda: streamk.tile_q4(Wq), 2 * wqb)):
+            ms = time_graph(fn, launches=5, replays=5)
+            tools[name] = {"us": round(ms * 1e3, 1), "gbs": round(nbytes / ms / 1e6, 1), "frac_hbm": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
+        extra["q4_tools_N8192_K8192"] = tools
+        del Wf
         extra["q4_note"] = ("34.6 MB of weights stay in the 256 MB Infinity Cache between launches of one weight "
                             "matrix; tuned_weights_from_hbm cycles through 20 copies so that every launch reads HBM")
         streamk.workspace_status()
