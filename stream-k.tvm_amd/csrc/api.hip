@@ -183,6 +183,7 @@ extern "C" int sk_workspace_status(void *ws, void *stream) {
 static int gemm_16bit(int dtype, const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,
                       int64_t lda, int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws,
                       size_t ws_bytes, void *stream, const sk_epilogue *epi = nullptr) {
+  if (epi && (epi->reserved[0] || epi->reserved[1] || epi->reserved[2])) return SK_ERR_CONFIG;
   const half_t *bias = epi ? (const half_t *)epi->bias : nullptr;
   if (reinterpret_cast<uintptr_t>(bias) & 1) return SK_ERR_ALIGN;
   if (!A || !B || !C) return SK_ERR_NULL;
@@ -306,6 +307,7 @@ static int gemm_q4_any(const void *A, const void *Wq, const void *scales, const 
                        int64_t N, int64_t K, int64_t lda, int64_t ldc, int group, int zero, int dtype,
                        const sk_plan *plan, void *ws, size_t ws_bytes, void *stream,
                        const sk_epilogue *epi = nullptr) {
+  if (epi && (epi->reserved[0] || epi->reserved[1] || epi->reserved[2])) return SK_ERR_CONFIG;
   const half_t *bias = epi ? (const half_t *)epi->bias : nullptr;
   if (reinterpret_cast<uintptr_t>(bias) & 1) return SK_ERR_ALIGN;
   if (!A || !Wq || !scales || !C || (dtype == SK_Q4_ZP && !zeros)) return SK_ERR_NULL;
