@@ -184,23 +184,32 @@ def main():
             c = torch.empty(m, N, dtype=torch.float16, device="cuda")
             row = {"M": m}
             cands = {"auto": {}}
+            tiles = {"128": (128, 128), "128x256": (128, 256), "256": (256, 256)}
             if m > 64:
-                cands.update({"sk_128": dict(bm=128, bn=128, bk=64, schedule="sk2", raster=8),
-                              "dp_128": dict(bm=128, bn=128, bk=64, schedule="dp", raster=8),
-                              "sk_256": dict(bm=256, bn=256, bk=64, schedule="sk2", raster=8),
-                              "dp_256": dict(bm=256, bn=256, bk=64, schedule="dp", raster=8)})
+                # per tile shape: the data-parallel-only schedule against the best Stream-K schedule of the same kernel
+                for t, (bm, bn) in tiles.items():
+                    cands["dp_" + t] = dict(bm=bm, bn=bn, bk=64, schedule="dp", raster=8)
+                    for sch in ("sk2", "basic", "splitk"):
+                        cands[f"{sch}_{t}"] = dict(bm=bm, bn=bn, bk=64, schedule=sch, fixup="reduce", raster=8)
             else:
                 cands.update({"dp": dict(schedule="dp"), "sk": dict(schedule="sk2", grid=256)})
             for name, cfg in cands.items():
-                p = streamk.make_plan(m, N, K, "float16", "nt", **cfg)
+                try:
+                    p = streamk.make_plan(m, N, K, "float16", "nt", **cfg)
+                except streamk.StreamKError:
+                    continue  # the fixed split does not divide this shape
                 ms = time_graph(lambda: streamk.streamk_fp16(a, B, out=c, plan=p))
                 row[name] = round(2.0 * m * N * K / ms / 1e9, 1)
-            best = max(v for k, v in row.items() if k != "M")
+            if m > 64:
+                for t in tiles:
+                    sk_best = max((row.pop(f"{sch}_{t}"), sch) for sch in ("sk2", "basic", "splitk") if f"{sch}_{t}" in row)
+                    row["sk_" + t], row["sk_schedule_" + t] = sk_best
+            best = max(v for k, v in row.items() if k != "M" and not isinstance(v, str))
             row["best_tflops"] = best
             row["pct_fp16_peak"] = round(100 * best / PEAK_FP16_TFLOPS, 2)
             row["gbs"] = round(best * 1e3 * (2.0 * (m * K + N * K + m * N)) / (2.0 * m * N * K), 1)
             if m > 64:
-                row["sk_over_dp_same_tile"] = round(max(row["sk_128"] / row["dp_128"], row["sk_256"] / row["dp_256"]), 3)
+                row["sk_over_dp_same_tile"] = round(max(row["sk_" + t] / row["dp_" + t] for t in tiles), 3)
             sweep.append(row)
         extra["sweep_N8192_K8192_tflops"] = sweep
 
