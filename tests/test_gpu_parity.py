@@ -694,6 +694,39 @@ def test_fused_bias_epilogue(sk, oracle):
     sk.workspace_status()
 
 
+def test_one_byte_operands_at_full_size(sk, oracle):
+    """fp8 and int8 at M = N = K = 8192 with the plans the library picks there (tuned cache or heuristic) and with
+    an explicit Stream-K plan: 48 random rows against the host product (int8: equal; fp8: 1e-3), and the exact
+    {-1,0,1} product checked through row and column checksums in int64 for every row and column."""
+    import torch
+    M = N = K = 8192
+    g = torch.Generator(device="cpu").manual_seed(8)
+    rows = np.random.RandomState(8).choice(M, size=48, replace=False)
+    Ai = torch.randint(-1, 2, (M, K), generator=g, dtype=torch.int8)
+    Bi = torch.randint(-1, 2, (N, K), generator=g, dtype=torch.int8)
+    # checksums of the exact product: sum_j C[i][j] = A[i] . (sum_j B[j]),  sum_i C[i][j] = (sum_i A[i]) . B[j]
+    row_sum = (Ai.long() @ Bi.long().sum(0)).numpy()
+    col_sum = (Ai.long().sum(0) @ Bi.long().T).numpy()
+    A8 = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int8)
+    B8 = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int8)
+    ref8 = torch.from_numpy(oracle.i8_gemm_ref(A8.numpy()[rows], B8.numpy()))
+    Af = torch.randn(M, K, generator=g).to(torch.float8_e4m3fn)
+    Bf = torch.randn(N, K, generator=g).to(torch.float8_e4m3fn)
+    reff = oracle.f8_gemm_ref(Af.view(torch.uint8).numpy()[rows], Bf.view(torch.uint8).numpy())
+    dAi, dBi, dA8, dB8, dAf, dBf = (t.cuda() for t in (Ai, Bi, A8, B8, Af, Bf))
+    for cfg in (None, dict(bm=256, bn=256, schedule="sk2", fixup="reduce", grid=200), dict(bm=128, bn=256, schedule="basic", fixup="atomic")):
+        kw = dict(config=cfg) if cfg else {}
+        C = sk.streamk_int8(dA8, dB8, **kw)
+        assert torch.equal(C[torch.from_numpy(rows).cuda()].cpu().long(), ref8), cfg
+        C = sk.streamk_int8(dAi, dBi, **kw)
+        assert np.array_equal(C.sum(1, dtype=torch.int64).cpu().numpy(), row_sum) and np.array_equal(C.sum(0, dtype=torch.int64).cpu().numpy(), col_sum), cfg
+        C = sk.streamk_fp8(dAf, dBf, **kw)
+        assert oracle.max_abs_rel(C[torch.from_numpy(rows).cuda()].float().cpu().numpy(), reff) <= 1e-3, cfg
+        C = sk.streamk_fp8(dAi.to(torch.float16).to(torch.float8_e4m3fn), dBi.to(torch.float16).to(torch.float8_e4m3fn), **kw)
+        assert np.array_equal(C.double().sum(1).cpu().numpy(), row_sum) and np.array_equal(C.double().sum(0).cpu().numpy(), col_sum), cfg
+    sk.workspace_status()
+
+
 def test_cfg5_large_dense(sk, oracle):
     """M = N = K = 8192 and the irregular 3000 x 5120 x 12288, U[-1,1): a random subset of rows is
     checked against an fp64 host product; the Stream-K and data-parallel schedules of the same kernel
