@@ -873,6 +873,38 @@ def test_fp32_reference_shape(sk, oracle):
     sk.workspace_status()
 
 
+def test_linear_layers_replay_in_a_graph(sk):
+    """A decode step as a serving loop would capture it: three StreamKLinear layers (fp16, Q4 with bias, Q4 with
+    per-group zero points and bias) for a batch of 4 rows in one graph, replayed several times with new inputs
+    copied into the static input buffer and eager work in between; every replay must equal the eager result of
+    the same layers on the same input bit for bit (all three use the ordered reduce or no fix-up)."""
+    import torch
+    torch.manual_seed(21)
+    K, H = 1024, 1536
+    l1 = sk.StreamKLinear.from_linear(torch.nn.Linear(K, H, bias=False).cuda().half())
+    l2 = sk.StreamKLinear.from_linear(torch.nn.Linear(H, K, bias=True).cuda().half(), weight_format="q4")
+    l3 = sk.StreamKLinear.from_linear(torch.nn.Linear(K, H, bias=True).cuda().half(), weight_format="q4_zp")
+    x = torch.zeros(4, K, dtype=torch.float16, device="cuda")
+    step = lambda t: l3(l2(l1(t)))
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step(x)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            y = step(x)
+    for replay in range(4):
+        xin = torch.randn(4, K, device="cuda").half()
+        want = step(xin)                       # eager, default stream
+        torch.cuda.synchronize()
+        x.copy_(xin)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, want), replay
+    sk.workspace_status()
+
+
 def test_graph_capture_replays_match_eager(sk, oracle):
     """The launches are capturable (no host synchronisation, no allocation; the workspace is cleared
     by a fill kernel, not by a memset node): a captured sequence reduce fix-up -> atomic fix-up ->
