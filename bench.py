@@ -334,6 +334,20 @@ def main():
             q4.append(row)
         extra["q4_N8192_K8192"] = q4
 
+        # fp16 matrix-vector product at an LLM-sized weight matrix (470 MB: every launch streams it from HBM)
+        nv, kv = 28672, 8192
+        wv = torch.randn(nv, kv, generator=g).half().cuda()
+        av = torch.randn(1, kv, generator=g).half().cuda()
+        cv = torch.empty(1, nv, dtype=torch.float16, device="cuda")
+        pv = streamk.make_plan(1, nv, kv, "float16", "nt")
+        vbytes = 2 * (kv + nv * kv + nv)
+        ms = time_graph(lambda: streamk.streamk_fp16(av, wv, out=cv, plan=pv), launches=5, replays=5)
+        ms_t = time_graph(lambda: torch.matmul(av, wv.T, out=cv), launches=5, replays=5)
+        extra["gemv_f16_M1_N28672_K8192"] = {"kernel": streamk.kernel_name(pv.kernel_id), "bytes": vbytes, "us": round(ms * 1e3, 1),
+                                            "gbs": round(vbytes / ms / 1e6, 1), "frac_hbm": round(vbytes / ms / 1e6 / PEAK_HBM_GBS, 4),
+                                            "torch_matmul_us": round(ms_t * 1e3, 1)}
+        del wv
+
         # offline side of the Q4 path on the same weight shape: algorithmic bytes over graph-timed launches
         Wf = (torch.randn(N, K, generator=g) * 0.05).half().cuda()
         _, _, zp = streamk.quantize_q4(Wf, asymmetric=True)

@@ -228,6 +228,10 @@ def autotune(M, N, K, dtype="float16", layout="nt", *, configs=None, warmup=5, r
             best = (ms, cfg)
     if best is None:
         raise RuntimeError(f"no valid configuration for {M}x{N}x{K} {dtype}/{layout}")
+    # within the noise of the measurement prefer a data-parallel plan: no workspace, no fix-up code in the kernel
+    near = [r for r in results if r[0] <= best[0] * 1.015 and r[1].get("schedule") == "dp"]
+    if near and best[1].get("schedule") != "dp":
+        best = min(near, key=lambda r: r[0])
     if cache:
         c = load_cache(cache_path)
         c[_key(dtype, layout, M, N, K)] = {"config": best[1], "latency_ms": best[0], "ref_latency_ms": ref_ms}
