@@ -179,7 +179,7 @@ def autotune(M, N, K, dtype="float16", layout="nt", *, configs=None, warmup=5, r
         one = torch.ones(1, device=dev)
         try:   # hipBLASLt's fp8 GEMM, where this torch build has it
             ref_ms = _time_ms(lambda: torch._scaled_mm(A8, rotate(Bs).T, scale_a=one, scale_b=one, out_dtype=torch.float16),
-                              warmup, rep, 2.0 * M * N * K < 5e10)
+                              warmup, rep, 2.0 * M * N * K < 5e11)
         except Exception:
             ref_ms = None
     elif dtype == "int8":
@@ -189,7 +189,7 @@ def autotune(M, N, K, dtype="float16", layout="nt", *, configs=None, warmup=5, r
         C = torch.empty(M, N, dtype=torch.int32, device=dev)
         run = lambda p: ops.streamk_int8(Ai, rotate(Bs), out=C, plan=p)  # noqa: E731
         try:   # the vendor's int8 GEMM, where this torch build has it
-            ref_ms = _time_ms(lambda: torch._int_mm(Ai, rotate(Bs).T), warmup, rep, 2.0 * M * N * K < 5e10)
+            ref_ms = _time_ms(lambda: torch._int_mm(Ai, rotate(Bs).T), warmup, rep, 2.0 * M * N * K < 5e11)
         except Exception:
             ref_ms = None
     else:
@@ -197,10 +197,10 @@ def autotune(M, N, K, dtype="float16", layout="nt", *, configs=None, warmup=5, r
         B = (torch.rand(*bshape, generator=g) * 2 - 1).half().to(dev)
         Bs = [B] + [B.clone() for _ in range(copies - 1)]
         run = lambda p: ops.streamk_fp16(A, rotate(Bs), layout=layout, out=C, plan=p)  # noqa: E731
-        small = 2.0 * M * N * K < 5e10
+        small = 2.0 * M * N * K < 5e11
         as_b = (lambda b: b.T) if layout == "nt" else (lambda b: b)
         ref_ms = _time_ms(lambda: torch.matmul(A, as_b(rotate(Bs)), out=C), warmup, rep, small)
-    small = 2.0 * M * N * K < 5e10  # microsecond kernels: time graph-captured batches
+    small = 2.0 * M * N * K < 5e11  # microsecond kernels: time graph-captured batches
     configs = configs if configs is not None else candidate_configs(M, N, K, dtype)
     best, golden, results = None, None, []
     for cfg in configs:
