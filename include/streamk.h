@@ -73,7 +73,8 @@ typedef enum sk_dtype {
   SK_Q4_TILED = 4, /* fp16 A, packed nibbles in 16-row x 64-byte tiles (sk_q4_tile_host / sk_q4_tile) */
   SK_F8E4M3 = 5,   /* A and B one byte per element, OCP e4m3 (bias 7, no infinities, NaN = S.1111.111); C fp16 */
   SK_I8 = 6,       /* A and B int8, C int32 */
-  SK_Q4_ZP = 7     /* as SK_Q4 with one zero point per scale group and row (sk_gemm_q4_zp) */
+  SK_Q4_ZP = 7,    /* as SK_Q4 with one zero point per scale group and row (sk_gemm_q4_zp) */
+  SK_F8E5M2 = 8    /* as SK_F8E4M3 for OCP e5m2 bytes (the upper byte of an fp16: bias 15, infinities and NaNs) */
 } sk_dtype;
 
 /* Tunables; a zero field means "choose for me".  Replaces the module-level constants and
@@ -184,7 +185,8 @@ int sk_gemm_bf16(const void *A, const void *B, void *C, int64_t M, int64_t N, in
                  int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws, size_t ws_bytes, void *stream);
 
 /* fp8 operands: A [M,K] and B [N,K] (NT only) hold OCP e4m3 bytes, C is fp16, accumulation fp32;
- * the plan is made with dtype SK_F8E4M3 (its bk counts fp8 elements).  No counterpart in the
+ * the plan is made with dtype SK_F8E4M3 (its bk counts fp8 elements), or SK_F8E5M2 for OCP e5m2 bytes (the
+ * dtype of the plan tells sk_gemm_f8 which format both operands are in).  No counterpart in the
  * reference's scripts; its Triton comparator takes whatever dtype its inputs have
  * (triton.streamk/first_wave.py:123 picks the accumulator type from them).  Same partitioner,
  * fix-ups and workspace rules as sk_gemm_f16.  K, lda and ldb multiples of 16; A and B 16-byte

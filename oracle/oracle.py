@@ -228,10 +228,18 @@ def f8e4m3_decode(u8):
     return np.where(u8 >> 7 == 1, -mag, mag).astype(np.float32)
 
 
-def f8_gemm_ref(A_u8, B_u8):
-    """float64 host product A [M,K] x B [N,K]^T of e4m3 bytes (each product of two e4m3 values is exact in
-    float32; the sum is taken in float64)."""
-    return f8e4m3_decode(A_u8).astype(np.float64) @ f8e4m3_decode(B_u8).astype(np.float64).T
+def f8e5m2_decode(u8):
+    """Bytes -> float32 values of the OCP format E5M2 (OFP8 rev 1.0, section 5: sign, 5 exponent bits with bias 15,
+    2 mantissa bits, IEEE-style infinities and NaNs): the upper byte of an IEEE binary16 number."""
+    u8 = np.asarray(u8, dtype=np.uint8)
+    return (u8.astype(np.uint16) << 8).view(np.float16).astype(np.float32)
+
+
+def f8_gemm_ref(A_u8, B_u8, fmt="e4m3"):
+    """float64 host product A [M,K] x B [N,K]^T of fp8 bytes, both e4m3 or both e5m2 (each product of two fp8
+    values is exact in float32; the sum is taken in float64)."""
+    dec = f8e4m3_decode if fmt == "e4m3" else f8e5m2_decode
+    return dec(A_u8).astype(np.float64) @ dec(B_u8).astype(np.float64).T
 
 
 def i8_gemm_ref(A_i8, B_i8):

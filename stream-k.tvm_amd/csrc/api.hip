@@ -267,7 +267,8 @@ extern "C" int sk_gemm_f8(const void *A, const void *B, void *C, int64_t M, int6
                           int64_t lda, int64_t ldb, int64_t ldc, float alpha, const sk_plan *plan, void *ws,
                           size_t ws_bytes, void *stream) {
   if (!(alpha == alpha) || alpha - alpha != 0.f) return SK_ERR_CONFIG;  // NaN or infinite
-  return gemm_8bit(SK_F8E4M3, A, B, C, M, N, K, lda, ldb, ldc, alpha, plan, ws, ws_bytes, stream);
+  const int dtype = plan && plan->dtype == SK_F8E5M2 ? SK_F8E5M2 : SK_F8E4M3;  // which format the bytes are in
+  return gemm_8bit(dtype, A, B, C, M, N, K, lda, ldb, ldc, alpha, plan, ws, ws_bytes, stream);
 }
 
 // (C and ldc are int32 here; the kernel casts)

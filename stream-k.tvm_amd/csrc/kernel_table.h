@@ -193,6 +193,13 @@ struct KernelInfo {
   X(72, 128, 256, 2, 4)       \
   X(73, 256, 128, 4, 2)
 
+// the same for OCP e5m2 operands (dtype SK_F8E5M2):  X(id, BM, BN, WM, WN)
+#define SK_TILE_F8E5M2_KERNELS(X) \
+  X(90, 256, 256, 2, 4)           \
+  X(91, 128, 128, 2, 2)           \
+  X(92, 128, 256, 2, 4)           \
+  X(93, 256, 128, 4, 2)
+
 // int8 operands, int32 C, NT layout; bk counts int8 elements (variant 4: 16x16 accumulator blocks):  X(id, BM, BN, WM, WN)
 #define SK_TILE_I8_KERNELS(X) \
   X(80, 256, 256, 2, 4)       \

@@ -31,6 +31,7 @@ static int launch_dma(const GemmArgs &a, const DevPlan &p, const Workspace &ws, 
 #define SK_POLICY_NN16(id, BM, BN, WM, WN) TileF16NTDma<BM, BN, WM, WN, true, 64, true>
 #define SK_POLICY_BF16(id, BM, BN, WM, WN, BK, NN) TileF16NTDma<BM, BN, WM, WN, NN, BK, true, true>
 #define SK_POLICY_F8(id, BM, BN, WM, WN) TileF16NTDma<BM, BN, WM, WN, false, 64, false, false, 1>
+#define SK_POLICY_F8E5M2(id, BM, BN, WM, WN) TileF16NTDma<BM, BN, WM, WN, false, 64, false, false, 2>
 #define SK_POLICY_I8(id, BM, BN, WM, WN) TileF16NTDma<BM, BN, WM, WN, false, 64, true, false, 3>
 
 int tile_kernel_infos(KernelInfo *out, int max) {
@@ -110,6 +111,14 @@ int tile_kernel_infos(KernelInfo *out, int max) {
 #undef X
 #define X(id, BM, BN, WM, WN)                                                                       \
   if (n < max) {                                                                                    \
+    typedef SK_POLICY_F8E5M2(id, BM, BN, WM, WN) P;                                                 \
+    out[n++] = KernelInfo{id, FAMILY_TILE, 8 /* SK_F8E5M2 */, 0, 6, BM, BN, 128, P::NT, P::LDS_TOTAL, P::CTAS_PER_CU, \
+                          P::TILE_ELEMS, 0, 0, 16, "tile_f8e5m2_nt_dma_" #BM "x" #BN "x128"};       \
+  }
+  SK_TILE_F8E5M2_KERNELS(X)
+#undef X
+#define X(id, BM, BN, WM, WN)                                                                       \
+  if (n < max) {                                                                                    \
     typedef SK_POLICY_I8(id, BM, BN, WM, WN) P;                                                     \
     out[n++] = KernelInfo{id, FAMILY_TILE, 6 /* SK_I8 */, 0, 4, BM, BN, 128, P::NT, P::LDS_TOTAL, P::CTAS_PER_CU, \
                           P::TILE_ELEMS, 0, 0, 16, "tile_i8_nt_dma16_" #BM "x" #BN "x128"};         \
@@ -184,6 +193,13 @@ int launch_tile_f16(int id, const GemmArgs &a, const DevPlan &p, const Workspace
     return launch_dma<P>(a, p, ws, s, bias);                                                   \
   }
     SK_TILE_F8_KERNELS(X)
+#undef X
+#define X(id_, BM, BN, WM, WN)                                                           \
+  case id_: {                                                                            \
+    typedef SK_POLICY_F8E5M2(id_, BM, BN, WM, WN) P;                                     \
+    return launch_dma<P>(a, p, ws, s, bias);                                             \
+  }
+    SK_TILE_F8E5M2_KERNELS(X)
 #undef X
 #define X(id_, BM, BN, WM, WN)                                                           \
   case id_: {                                                                            \
@@ -279,6 +295,15 @@ int occupancy_tile(int id) {
     return occ;                                                                                     \
   }
     SK_TILE_F8_KERNELS(X)
+#undef X
+#define X(id_, BM, BN, WM, WN)                                                                      \
+  case id_: {                                                                                       \
+    typedef SK_POLICY_F8E5M2(id_, BM, BN, WM, WN) P;                                                \
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_tile_kernel<P>, P::NT, 0) != hipSuccess) \
+      return -1;                                                                                    \
+    return occ;                                                                                     \
+  }
+    SK_TILE_F8E5M2_KERNELS(X)
 #undef X
 #define X(id_, BM, BN, WM, WN)                                                                      \
   case id_: {                                                                                       \

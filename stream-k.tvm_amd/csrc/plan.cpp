@@ -144,9 +144,9 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
   if (!out) return SK_ERR_NULL;
   if (M <= 0 || N <= 0 || K <= 0 || M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return SK_ERR_SHAPE;
   if (dtype != SK_F16 && dtype != SK_F32 && dtype != SK_Q4 && dtype != SK_BF16 && dtype != SK_Q4_TILED &&
-      dtype != SK_F8E4M3 && dtype != SK_I8 && dtype != SK_Q4_ZP)
+      dtype != SK_F8E4M3 && dtype != SK_I8 && dtype != SK_Q4_ZP && dtype != SK_F8E5M2)
     return SK_ERR_CONFIG;
-  if ((dtype == SK_F8E4M3 || dtype == SK_I8) && layout != SK_LAYOUT_NT) return SK_ERR_CONFIG;
+  if ((dtype == SK_F8E4M3 || dtype == SK_F8E5M2 || dtype == SK_I8) && layout != SK_LAYOUT_NT) return SK_ERR_CONFIG;
   if (layout != SK_LAYOUT_NT && layout != SK_LAYOUT_NN) return SK_ERR_CONFIG;
   if (num_cus <= 0) return SK_ERR_DEVICE;
   const KernelInfo *k = pick_kernel(M, N, K, dtype, layout, cfg, num_cus);

@@ -56,7 +56,7 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
     schedule, grid and fix-up."""
     cus = cus or _plan.num_cus()
     out = []
-    if dtype in ("q4", "q4_zp") or (M <= 64 and dtype not in ("float8_e4m3", "int8")):
+    if dtype in ("q4", "q4_zp") or (M <= 64 and dtype not in ("float8_e4m3", "float8_e5m2", "int8")):
         tiles = _SKINNY_Q4 if dtype in ("q4", "q4_zp") else _SKINNY_F16
         for (bm, bn, bk) in tiles:
             if bm < M and not (bm == 16 and M <= 16):
@@ -84,7 +84,7 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
                 # fixed split-K, the fallback when there are fewer tiles than CUs
                 if -(-M // bm) * -(-N // bn) < cus:
                     out.extend(dict(base, schedule="splitk", fixup=fixup) for fixup in ("reduce", "atomic"))
-    if dtype in ("float8_e4m3", "int8"):
+    if dtype in ("float8_e4m3", "float8_e5m2", "int8"):
         for (bm, bn), raster in itertools.product(((256, 256), (256, 128), (128, 256), (128, 128)), (1, 8)):
             base = dict(bm=bm, bn=bn, raster=raster)
             out.append(dict(base, schedule="dp"))
@@ -154,7 +154,7 @@ def autotune(M, N, K, dtype="float16", layout="nt", *, configs=None, warmup=5, r
     A = (torch.rand(M, K, generator=g) * 2 - 1).half().to(dev)
     C = torch.empty(M, N, dtype=torch.float16, device=dev)
     weights = weights or ("hbm" if M <= 64 else "warm")
-    wbytes = N * K // 2 if dtype in ("q4", "q4_zp") else (N * K if dtype in ("float8_e4m3", "int8") else N * K * 2)
+    wbytes = N * K // 2 if dtype in ("q4", "q4_zp") else (N * K if dtype in ("float8_e4m3", "float8_e5m2", "int8") else N * K * 2)
     copies = 1 if weights == "warm" else max(2, min(rep, -(-(512 << 20) // wbytes)))
     turn = [0]
 
@@ -171,9 +171,10 @@ def autotune(M, N, K, dtype="float16", layout="nt", *, configs=None, warmup=5, r
         else:
             run = lambda p: ops.streamk_q4(A, *rotate(Ws), out=C, plan=p)  # noqa: E731
         ref_ms = None
-    elif dtype == "float8_e4m3":
-        A8 = A.to(torch.float8_e4m3fn)
-        B8 = (torch.rand(N, K, generator=g) * 2 - 1).to(dev).to(torch.float8_e4m3fn)
+    elif dtype in ("float8_e4m3", "float8_e5m2"):
+        f8 = torch.float8_e4m3fn if dtype == "float8_e4m3" else torch.float8_e5m2
+        A8 = A.to(f8)
+        B8 = (torch.rand(N, K, generator=g) * 2 - 1).to(dev).to(f8)
         Bs = [B8] + [B8.clone() for _ in range(copies - 1)]
         run = lambda p: ops.streamk_fp8(A8, rotate(Bs), out=C, plan=p)  # noqa: E731
         one = torch.ones(1, device=dev)

@@ -132,22 +132,32 @@ def streamk_bf16(A, B, *, layout="nt", out=None, plan=None, config=None, bias=No
     return C
 
 
-def streamk_fp8(A, B, *, alpha=1.0, out=None, plan=None, config=None, **kw):
-    """C = alpha * (A @ B.T) for fp8 operands (OCP e4m3: torch.float8_e4m3fn, or the same bytes as
-    uint8), A [M,K], B [N,K]; fp32 accumulation, alpha applied to the fp32 sums, fp16 C.  alpha is
-    the product of the per-tensor scales of a scaled-fp8 caller.  The reference's scripts stop at
-    fp16; this is the same partitioner and fix-ups over the fp8 form of the tile kernel."""
-    f8 = getattr(torch, "float8_e4m3fn", None)
+def streamk_fp8(A, B, *, alpha=1.0, fmt=None, out=None, plan=None, config=None, **kw):
+    """C = alpha * (A @ B.T) for fp8 operands, A [M,K], B [N,K]; fp32 accumulation, alpha applied to the
+    fp32 sums, fp16 C.  Both operands are OCP e4m3 (torch.float8_e4m3fn) or both OCP e5m2
+    (torch.float8_e5m2); raw uint8 bytes are taken as `fmt` ("e4m3" by default, or "e5m2").  alpha is the
+    product of the per-tensor scales of a scaled-fp8 caller.  The reference's scripts stop at fp16; this is
+    the same partitioner and fix-ups over the fp8 form of the tile kernel."""
+    kinds = {getattr(torch, "float8_e4m3fn", None): "e4m3", getattr(torch, "float8_e5m2", None): "e5m2"}
     for t, name in ((A, "A"), (B, "B")):
-        if not isinstance(t, torch.Tensor) or t.dtype not in (torch.uint8, f8):
-            raise TypeError(f"{name} must be a float8_e4m3fn (or uint8) tensor")
+        if not isinstance(t, torch.Tensor) or (t.dtype != torch.uint8 and t.dtype not in kinds):
+            raise TypeError(f"{name} must be a float8_e4m3fn / float8_e5m2 (or uint8) tensor")
         _check_matrix(t, name, t.dtype)
+        if t.dtype != torch.uint8:
+            if fmt not in (None, kinds[t.dtype]):
+                raise TypeError("A and B must be in the same fp8 format")
+            fmt = kinds[t.dtype]
+    fmt = fmt or "e4m3"
+    if fmt not in ("e4m3", "e5m2"):
+        raise ValueError("fmt must be 'e4m3' or 'e5m2'")
     M, K = A.shape
     N, Kb = B.shape
     if K != Kb:
         raise ValueError(f"K mismatch: A is {tuple(A.shape)}, B is {tuple(B.shape)}")
     if plan is None:
-        plan = make_plan(M, N, K, "float8_e4m3", "nt", config, **kw)
+        plan = make_plan(M, N, K, "float8_" + fmt, "nt", config, **kw)
+    elif plan.dtype != (_lib.SK_F8E5M2 if fmt == "e5m2" else _lib.SK_F8E4M3):
+        raise ValueError("the plan was made for the other fp8 format")
     C = out if out is not None else torch.empty((M, N), dtype=torch.float16, device=A.device)
     _check_matrix(C, "out", torch.float16)
     if tuple(C.shape) != (M, N):

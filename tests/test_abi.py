@@ -100,6 +100,9 @@ def test_fp8_plans(sk):
         p = sk.make_plan(M, N, K, "float8_e4m3", "nt", cus=256)
         assert (p.bm, p.bn, p.bk) == (bm, bm, 128) and p.iters_per_tile == K // 128
         assert sk.kernel_name(p.kernel_id) == f"tile_f8e4m3_nt_dma_{bm}x{bm}x128"
+        r = sk.make_plan(M, N, K, "float8_e5m2", "nt", cus=256)
+        assert (r.bm, r.bn, r.bk, r.grid) == (p.bm, p.bn, 128, p.grid)
+        assert sk.kernel_name(r.kernel_id) == f"tile_f8e5m2_nt_dma_{bm}x{bm}x128"
         q = sk.make_plan(M, N, K, "int8", "nt", cus=256)
         assert (q.bm, q.bn, q.bk, q.grid) == (p.bm, p.bn, 128, p.grid)
         assert sk.kernel_name(q.kernel_id) == f"tile_i8_nt_dma16_{bm}x{bm}x128"

@@ -586,6 +586,40 @@ def test_fp8_tile_kernels(sk, oracle):
     sk.workspace_status()
 
 
+def test_fp8_e5m2_tile_kernels(sk, oracle):
+    """The e5m2 instances of the fp8 kernels: same checks as for e4m3 on fewer shapes (the two differ in one
+    immediate operand of the MFMA): host product of the decoded bytes within 1e-3, {-1,0,1} data exact, every
+    finite byte value, mixed formats refused."""
+    import torch
+    torch.manual_seed(13)
+    f8 = torch.float8_e5m2
+    for (M, N, K) in [(200, 136, 336), (520, 264, 1040)]:
+        A, B = torch.randn(M, K).to(f8), torch.randn(N, K).to(f8)
+        Ai, Bi = torch.randint(-1, 2, (M, K)).float().to(f8), torch.randint(-1, 2, (N, K)).float().to(f8)
+        ref = oracle.f8_gemm_ref(A.view(torch.uint8).numpy(), B.view(torch.uint8).numpy(), "e5m2")
+        exact = oracle.f8_gemm_ref(Ai.view(torch.uint8).numpy(), Bi.view(torch.uint8).numpy(), "e5m2")
+        for (bm, bn) in [(256, 256), (128, 128), (128, 256), (256, 128)]:
+            for sch in (dict(schedule="dp"), dict(schedule="basic", fixup="reduce", grid=24), dict(schedule="sk2", fixup="atomic", grid=16)):
+                plan = sk.make_plan(M, N, K, "float8_e5m2", "nt", dict(bm=bm, bn=bn, **sch))
+                assert "e5m2" in sk.kernel_name(plan.kernel_id)
+                C = sk.streamk_fp8(A.cuda(), B.cuda(), plan=plan)
+                assert _rel(oracle, C, ref) <= 1e-3 <= TOL, (M, N, K, bm, bn, sch)
+                Ci = sk.streamk_fp8(Ai.cuda().view(torch.uint8), Bi.cuda().view(torch.uint8), fmt="e5m2", plan=plan)
+                assert np.array_equal(Ci.double().cpu().numpy(), exact), (M, N, K, bm, bn, sch)
+    # every finite byte value against partners 0 and +-2^-14 (57344 * 2^-14 = 3.5)
+    allv = torch.tensor([b for b in range(256) if b & 127 < 0x7C], dtype=torch.uint8)
+    A = torch.stack([allv.repeat(5)[torch.randperm(1240)[:1008]] for _ in range(40)])
+    B = torch.tensor([0x00, 0x04, 0x84], dtype=torch.uint8)[torch.randint(0, 3, (24, 1008))]
+    ref = oracle.f8_gemm_ref(A.numpy(), B.numpy(), "e5m2")
+    assert _rel(oracle, sk.streamk_fp8(A.cuda(), B.cuda(), fmt="e5m2"), ref) <= 1e-3
+    with pytest.raises(TypeError):
+        sk.streamk_fp8(torch.zeros(8, 64, device="cuda").to(f8), torch.zeros(8, 64, device="cuda").to(torch.float8_e4m3fn))
+    with pytest.raises(ValueError):
+        sk.streamk_fp8(torch.zeros(8, 64, device="cuda").to(f8), torch.zeros(8, 64, device="cuda").to(f8),
+                       plan=sk.make_plan(8, 8, 64, "float8_e4m3", "nt"))
+    sk.workspace_status()
+
+
 def test_int8_tile_kernels(sk, oracle):
     """int8 operands, int32 C: integer arithmetic, so every instance, schedule and fix-up (the atomic one
     included) must return the host's exact product, on the full range -128..127, ragged shapes, K tails,

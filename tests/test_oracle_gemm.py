@@ -94,6 +94,24 @@ def test_f8e4m3_decode(oracle):
     assert np.array_equal(oracle.f8_gemm_ref(A, B), [[1 + 2 - 2 + 448 * 2.0 ** -9, 0.0]])
 
 
+def test_f8e5m2_decode(oracle):
+    """e5m2 decoder: known values (1.0 = 0x3C, largest finite 57344 = 0x7B, smallest subnormal 2^-16 = 0x01,
+    smallest normal 2^-14 = 0x04, infinities 0x7C / 0xFC, NaNs above them), a closed form over all finite
+    bytes, and torch's CPU conversion of all 256 bytes."""
+    import torch
+    d = oracle.f8e5m2_decode(np.arange(256, dtype=np.uint8))
+    assert d[0x3C] == 1.0 and d[0x7B] == 57344.0 and d[0x01] == 2.0 ** -16 and d[0x04] == 2.0 ** -14 and d[0xC0] == -2.0
+    assert np.isposinf(d[0x7C]) and np.isneginf(d[0xFC]) and np.isnan(d[0x7D:0x80]).all() and np.isnan(d[0xFD:]).all()
+    for b in range(0x7C):
+        e, m = b >> 2, b & 3
+        assert d[b] == (m * 2.0 ** -16 if e == 0 else (4 + m) * 2.0 ** (e - 17)) and d[b | 0x80] == -d[b]
+    t = torch.arange(256, dtype=torch.uint8).view(torch.float8_e5m2).float().numpy()
+    assert np.array_equal(np.isnan(d), np.isnan(t)) and np.array_equal(d[~np.isnan(d)], t[~np.isnan(t)])
+    A = np.array([[0x3C, 0x40, 0xBC, 0x01]], dtype=np.uint8)   # 1, 2, -1, 2^-16
+    B = np.array([[0x3C, 0x3C, 0x40, 0x7B]], dtype=np.uint8)   # 1, 1, 2, 57344
+    assert np.array_equal(oracle.f8_gemm_ref(A, B, "e5m2"), [[1 + 2 - 2 + 57344 * 2.0 ** -16]])
+
+
 def test_i8_gemm_ref(oracle):
     """The int8 host product: hand-worked values at the ends of the range and agreement with a Python-int loop."""
     A = np.array([[-128, 127, 1, 0], [1, 1, 1, 1]], dtype=np.int8)
