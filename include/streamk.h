@@ -159,11 +159,21 @@ int sk_gemm_f16(const void *A, const void *B, void *C, int64_t M, int64_t N, int
 
 /* Optional epilogue of the *_ex entry points (NULL = none): bias points at N device values of C's type
  * (fp16, or bfloat16 for sk_gemm_bf16_ex) that are added to every row of C in fp32 before the rounding --
- * the bias of a linear layer, which the reference leaves to a separate kernel.  Fix-ups are unaffected
- * (partials stay unbiased; the CTA that stores a tile adds the bias).  reserved must be zero. */
+ * the bias of a linear layer, which the reference leaves to a separate kernel -- or is NULL; activation
+ * (an sk_activation, 0 = none) is applied after the bias, also in fp32 -- the nonlinearity of an MLP's
+ * first projection.  Fix-ups are unaffected (partials stay linear; the CTA that stores a tile applies the
+ * epilogue).  reserved must be zero. */
+typedef enum sk_activation {
+  SK_ACT_NONE = 0,
+  SK_ACT_RELU = 1,      /* max(x, 0) */
+  SK_ACT_GELU_TANH = 2, /* 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))) */
+  SK_ACT_SILU = 3       /* x / (1 + exp(-x)) */
+} sk_activation;
+
 typedef struct sk_epilogue {
   const void *bias;
-  int64_t reserved[3];
+  int64_t activation;
+  int64_t reserved[2];
 } sk_epilogue;
 
 int sk_gemm_f16_ex(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,

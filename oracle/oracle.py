@@ -286,3 +286,21 @@ def q4_zp_gemm_ref(A, Wq, scales, zeros, group=128):
     """fp32 host product of A [M,K] with the dequantised weights [N,K]^T."""
     W = dequant_q4_zp_np(Wq, scales, zeros, group).astype(np.float32)
     return np.asarray(A, dtype=np.float32) @ W.T
+
+
+def activation_ref(x, name):
+    """Epilogue activations in float64 on a numpy array: 'relu' max(x, 0); 'gelu_tanh'
+    0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))) (the tanh form of GELU, Hendrycks & Gimpel 2016, eq. 2);
+    'silu' x / (1 + exp(-x)); None / 'none' the identity.  No counterpart in the reference, whose kernels end
+    at the store of C; pinned in tests/test_oracle_gemm.py against torch's CPU routines and the erf form."""
+    x = np.asarray(x, dtype=np.float64)
+    if name in (None, "none"):
+        return x
+    if name == "relu":
+        return np.maximum(x, 0.0)
+    if name == "gelu_tanh":
+        return 0.5 * x * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (x + 0.044715 * x ** 3)))
+    if name == "silu":
+        with np.errstate(over="ignore"):
+            return x / (1.0 + np.exp(-x))
+    raise ValueError(f"unknown activation {name!r}")

@@ -180,12 +180,24 @@ extern "C" int sk_workspace_status(void *ws, void *stream) {
   return v == 0 ? SK_OK : SK_ERR_TIMEOUT;
 }
 
+// checks an sk_epilogue and packs it into the one word the kernels take (0 = no epilogue)
+static int epilogue_word(const sk_epilogue *epi, const void **word) {
+  *word = nullptr;
+  if (!epi) return SK_OK;
+  if (epi->reserved[0] || epi->reserved[1]) return SK_ERR_CONFIG;
+  if (epi->activation < SK_ACT_NONE || epi->activation > SK_ACT_SILU) return SK_ERR_CONFIG;
+  const uintptr_t b = reinterpret_cast<uintptr_t>(epi->bias);
+  if (b & 1) return SK_ERR_ALIGN;
+  if (b >> EPI_ACT_SHIFT) return SK_ERR_CONFIG;  // not a device address
+  *word = epi_word(epi->bias, (int)epi->activation);
+  return SK_OK;
+}
+
 static int gemm_16bit(int dtype, const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,
                       int64_t lda, int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws,
                       size_t ws_bytes, void *stream, const sk_epilogue *epi = nullptr) {
-  if (epi && (epi->reserved[0] || epi->reserved[1] || epi->reserved[2])) return SK_ERR_CONFIG;
-  const half_t *bias = epi ? (const half_t *)epi->bias : nullptr;
-  if (reinterpret_cast<uintptr_t>(bias) & 1) return SK_ERR_ALIGN;
+  const void *bias = nullptr;  // the kernels' epilogue word: bias pointer and activation code
+  if (int rc = epilogue_word(epi, &bias)) return rc;
   if (!A || !B || !C) return SK_ERR_NULL;
   int rc = check_plan(plan, M, N, K, dtype, plan ? plan->layout : 0);
   if (rc) return rc;
@@ -308,9 +320,8 @@ static int gemm_q4_any(const void *A, const void *Wq, const void *scales, const 
                        int64_t N, int64_t K, int64_t lda, int64_t ldc, int group, int zero, int dtype,
                        const sk_plan *plan, void *ws, size_t ws_bytes, void *stream,
                        const sk_epilogue *epi = nullptr) {
-  if (epi && (epi->reserved[0] || epi->reserved[1] || epi->reserved[2])) return SK_ERR_CONFIG;
-  const half_t *bias = epi ? (const half_t *)epi->bias : nullptr;
-  if (reinterpret_cast<uintptr_t>(bias) & 1) return SK_ERR_ALIGN;
+  const void *bias = nullptr;  // the kernels' epilogue word: bias pointer and activation code
+  if (int rc = epilogue_word(epi, &bias)) return rc;
   if (!A || !Wq || !scales || !C || (dtype == SK_Q4_ZP && !zeros)) return SK_ERR_NULL;
   int rc = check_plan(plan, M, N, K, dtype, SK_LAYOUT_NT);
   if (rc) return rc;

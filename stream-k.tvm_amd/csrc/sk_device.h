@@ -228,6 +228,33 @@ __device__ __forceinline__ int pin_here(int x) {
   return x;
 }
 
+// The epilogue's kernel argument is one 64-bit word: the bias pointer in the low 60 bits (device addresses use 57 at
+// most) and the activation code in the top four.  Zero means "no epilogue", so kernels test one value, and the word
+// costs the kernels that predate the activation no further argument.
+constexpr int EPI_ACT_SHIFT = 60;
+__host__ __device__ __forceinline__ const void *epi_word(const void *bias, int act) {
+  return reinterpret_cast<const void *>(reinterpret_cast<uintptr_t>(bias) | ((uintptr_t)(uint32_t)act << EPI_ACT_SHIFT));
+}
+__device__ __forceinline__ int epi_act(const void *word) {
+  return (int)(reinterpret_cast<uintptr_t>(word) >> EPI_ACT_SHIFT);
+}
+__device__ __forceinline__ const half_t *epi_bias(const void *word) {
+  return reinterpret_cast<const half_t *>(reinterpret_cast<uintptr_t>(word) & (((uintptr_t)1 << EPI_ACT_SHIFT) - 1));
+}
+
+// activation applied in fp32 after the bias, before the rounding to C's type; act is uniform over the grid
+// (codes are sk_activation's: 1 relu, 2 gelu in its tanh form, 3 silu)
+__device__ __forceinline__ float activate(float x, int act) {
+  if (act == 1) return fmaxf(x, 0.f);
+  if (act == 2) {
+    // 0.5 x (1 + tanh(u)) = x / (1 + exp(-2u)),  u = sqrt(2/pi) (x + 0.044715 x^3)
+    const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+    return x / (1.f + __expf(-2.f * u));
+  }
+  if (act == 3) return x / (1.f + __expf(-x));
+  return x;
+}
+
 // optional epilogue operand: a row vector added to every row of C in fp32, before the rounding to C's type
 // (fp16 bits, or bfloat16 bits when BF16).  Returns 0 without a bias or past the last column.
 template <bool BF16 = false>
@@ -244,7 +271,8 @@ __device__ __forceinline__ float bias_at(const half_t *bias, int col, int N) {
 // four consecutive bias values starting at column col (a multiple of 4): one 8-byte load where the row allows it
 template <bool BF16 = false>
 __device__ __forceinline__ floatx4 bias4_at(const half_t *bias, int col, int N) {
-  floatx4 r;
+  floatx4 r = {0.f, 0.f, 0.f, 0.f};
+  if (bias == nullptr) return r;  // an activation without a bias
   if (col + 4 <= N && (reinterpret_cast<uintptr_t>(bias) & 7) == 0) {
     const half4v h = *reinterpret_cast<const half4v *>(bias + col);
 #pragma unroll

@@ -146,11 +146,13 @@ struct TileF16NT {
     if (bias == nullptr)
       store_c_impl<false>(a, acc, pm, pn, smem, nullptr);
     else
-      store_c_impl<true>(a, acc, pm, pn, smem, static_cast<const half_t *>(bias));
+      store_c_impl<true>(a, acc, pm, pn, smem, bias);
   }
   template <bool BIAS>
   static __device__ __forceinline__ void store_c_impl(const Args &a, const Acc &acc, int pm, int pn, char *smem,
-                                                      const half_t *bias) {
+                                                      const void *epi) {
+    const half_t *bias = BIAS ? epi_bias(epi) : nullptr;
+    const int act = BIAS ? epi_act(epi) : 0;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
     half_t *patch = reinterpret_cast<half_t *>(smem) + wave * (WTM * LDC);
@@ -165,7 +167,7 @@ struct TileF16NT {
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             float x = acc.c[i][j][q * 4 + e];
-            if constexpr (BIAS) x += bias_at(bias, bias_col0 + j * 32 + q * 8 + e, a.N);
+            if constexpr (BIAS) x = activate(x + bias_at(bias, bias_col0 + j * 32 + q * 8 + e, a.N), act);
             h[e] = (half_t)x;
           }
           *reinterpret_cast<half4v *>(patch + (i * 32 + (lane & 31)) * LDC + j * 32 + q * 8 +

@@ -621,11 +621,13 @@ struct TileF16NTDma {
     if (bias == nullptr)
       store_c_impl<false>(a, acc, pm, pn, smem, nullptr);
     else
-      store_c_impl<true>(a, acc, pm, pn, smem, static_cast<const half_t *>(bias));
+      store_c_impl<true>(a, acc, pm, pn, smem, bias);
   }
   template <bool BIAS>
   static __device__ __forceinline__ void store_c_impl(const Args &a, const Acc &acc, int pm, int pn, char *,
-                                                      const half_t *bias) {
+                                                      const void *epi) {
+    const half_t *bias = BIAS ? epi_bias(epi) : nullptr;
+    const int act = BIAS ? epi_act(epi) : 0;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
     if constexpr (I8) {
@@ -672,7 +674,7 @@ struct TileF16NTDma {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               float x = acc.v[p * (PATCH_ROWS / 16) + ib][j][e];
-              if constexpr (BIAS) x += bv[e];
+              if constexpr (BIAS) x = activate(x + bv[e], act);
               if constexpr (BF16_) {
                 const __bf16 b = (__bf16)x;
                 h[e] = __builtin_bit_cast(half_t, b);  // the patch only carries 16-bit patterns
@@ -696,7 +698,7 @@ struct TileF16NTDma {
               for (int e = 0; e < 4; ++e) {
                 float x = acc.c[p * BLK + ib][j][q * 4 + e];
                 if constexpr (F8 != 0) x *= a.alpha;  // the product of fp8 operands is scaled before it is rounded to fp16
-                if constexpr (BIAS) x += bv[e];
+                if constexpr (BIAS) x = activate(x + bv[e], act);
                 h[e] = (half_t)x;
               }
               *reinterpret_cast<half4v *>(patch + (ib * 32 + (lane & 31)) * LDC + j * 32 + q * 8 +

@@ -293,18 +293,19 @@ struct TileGemvQ4 {
                                                  const void *bias_) {
     int e;
     if (!owns_output(e)) return;
-    const half_t *bias = static_cast<const half_t *>(bias_);
-    if (bias == nullptr) {  // the common case keeps the code it had before the bias existed
+    if (bias_ == nullptr) {  // the common case keeps the code it had before the epilogue operands existed
 #pragma unroll
       for (int j = 0; j < NB; ++j) {
         const int col = pn * BN + e + j * 16;
         if (col < a.N) a.C[col] = (half_t)acc.y[j];
       }
     } else {
+      const half_t *bias = epi_bias(bias_);
+      const int act = epi_act(bias_);
 #pragma unroll
       for (int j = 0; j < NB; ++j) {
         const int col = pn * BN + e + j * 16;
-        if (col < a.N) a.C[col] = (half_t)(acc.y[j] + (float)bias[col]);
+        if (col < a.N) a.C[col] = (half_t)activate(acc.y[j] + bias_at(bias, col, a.N), act);
       }
     }
   }

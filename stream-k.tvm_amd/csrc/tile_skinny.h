@@ -358,11 +358,13 @@ struct TileSkinny {
     if (bias == nullptr)
       store_c_impl<false>(a, acc, pm, pn, smem, nullptr);
     else
-      store_c_impl<true>(a, acc, pm, pn, smem, static_cast<const half_t *>(bias));
+      store_c_impl<true>(a, acc, pm, pn, smem, bias);
   }
   template <bool BIAS>
   static __device__ __forceinline__ void store_c_impl(const Args &a, const Acc &acc, int pm, int pn, char *,
-                                                      const half_t *bias) {
+                                                      const void *epi) {
+    const half_t *bias = BIAS ? epi_bias(epi) : nullptr;
+    const int act = BIAS ? epi_act(epi) : 0;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     if (wave >= WN) return;
     const int lr = lane & 15, lg = lane >> 4;
@@ -378,7 +380,7 @@ struct TileSkinny {
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             float x = acc.c[i][j][e];
-            if constexpr (BIAS) x += bias_at(bias, col + e, a.N);
+            if constexpr (BIAS) x = activate(x + bias_at(bias, col + e, a.N), act);
             h[e] = (half_t)x;
           }
           half_t *dst = a.C + (int64_t)row * a.ldc + col;

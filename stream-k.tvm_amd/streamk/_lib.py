@@ -34,9 +34,13 @@ class SkPlan(ctypes.Structure):
         return {n: getattr(self, n) for n, _ in self._fields_}
 
 
+# sk_activation
+ACTIVATIONS = {None: 0, "none": 0, "relu": 1, "gelu_tanh": 2, "silu": 3}
+
+
 class SkEpilogue(ctypes.Structure):
     """sk_epilogue: optional operands of the *_ex entry points."""
-    _fields_ = [("bias", ctypes.c_void_p), ("reserved", ctypes.c_int64 * 3)]
+    _fields_ = [("bias", ctypes.c_void_p), ("activation", ctypes.c_int64), ("reserved", ctypes.c_int64 * 2)]
 
 
 class StreamKError(RuntimeError):

@@ -15,8 +15,11 @@ from .plan import make_plan
 
 class StreamKLinear(torch.nn.Module):
     def __init__(self, in_features, out_features, bias=False, *, weight_format="float16", group=128, zero=8,
-                 device=None):
+                 activation=None, device=None):
         super().__init__()
+        if activation not in (None, "relu", "gelu_tanh", "silu"):
+            raise ValueError("activation must be None, 'relu', 'gelu_tanh' or 'silu'")
+        self.activation = activation  # applied in the GEMM's epilogue, after the bias
         if weight_format not in ("float16", "q4", "q4_zp"):
             raise ValueError("weight_format must be 'float16', 'q4' or 'q4_zp' (one zero point per group)")
         if weight_format != "float16" and (group != 128 or in_features % 128):
@@ -37,13 +40,13 @@ class StreamKLinear(torch.nn.Module):
         self._plans = {}
 
     @classmethod
-    def from_linear(cls, linear, *, weight_format="float16", group=128, zero=8):
+    def from_linear(cls, linear, *, weight_format="float16", group=128, zero=8, activation=None):
         """Takes over the weight (and bias) of a torch.nn.Linear; weight_format='q4' / 'q4_zp' quantises
         it with `quantize_q4` (symmetric around `zero` / asymmetric with a zero point per group) on the
         device it lives on."""
         w = linear.weight.detach().to(torch.float16).contiguous()
         m = cls(linear.in_features, linear.out_features, linear.bias is not None, weight_format=weight_format,
-                group=group, zero=zero, device=w.device)
+                group=group, zero=zero, activation=activation, device=w.device)
         if weight_format == "float16":
             m.weight.copy_(w)
         elif weight_format == "q4_zp":
@@ -77,15 +80,16 @@ class StreamKLinear(torch.nn.Module):
         M = a.shape[0]
         if M == 0:
             return x.new_zeros(*lead, self.out_features)
-        # the bias is added in the GEMM's epilogue (fp32, before the rounding to fp16)
+        # bias and activation are applied in the GEMM's epilogue (fp32, before the rounding to fp16)
         if self.weight_format == "float16":
-            c = ops.streamk_fp16(a, self.weight, plan=self.plan_for(M), bias=self.bias)
+            c = ops.streamk_fp16(a, self.weight, plan=self.plan_for(M), bias=self.bias, activation=self.activation)
         else:
             # (more rows than one Q4 launch takes: streamk_q4 splits the call itself)
             c = ops.streamk_q4(a, self.qweight, self.scales, plan=self.plan_for(M) if M <= ops.Q4_MAX_M else None,
-                               zero=self.zero, group=self.group, zeros=getattr(self, "zeros", None), bias=self.bias)
+                               zero=self.zero, group=self.group, zeros=getattr(self, "zeros", None), bias=self.bias,
+                               activation=self.activation)
         return c.view(*lead, self.out_features)
 
     def extra_repr(self):
         return (f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}, "
-                f"weight_format={self.weight_format}")
+                f"weight_format={self.weight_format}, activation={self.activation}")

@@ -58,28 +58,34 @@ def _check_matrix(t, name, dtype):
         raise ValueError(f"{name} must be 2-D with unit stride along its last dimension")
 
 
-def _epilogue(bias, N, dtype, device):
-    """sk_epilogue for a bias vector (N values of C's type on C's device), or None."""
+def _epilogue(bias, N, dtype, device, activation=None):
+    """sk_epilogue for a bias vector (N values of C's type on C's device) and / or an activation
+    ('relu', 'gelu_tanh', 'silu'), or None when there is neither."""
+    if activation not in _lib.ACTIVATIONS:
+        raise ValueError(f"activation must be one of {sorted(k for k in _lib.ACTIVATIONS if k)} or None")
+    act = _lib.ACTIVATIONS[activation]
     if bias is None:
-        return None
+        return _lib.SkEpilogue(bias=None, activation=act) if act else None
     if not isinstance(bias, torch.Tensor) or bias.dtype != dtype or bias.dim() != 1 or bias.shape[0] != N \
             or not bias.is_contiguous() or bias.device != device:
         raise ValueError(f"bias must be a contiguous {dtype} vector of {N} elements on {device}")
-    return _lib.SkEpilogue(bias=bias.data_ptr())
+    return _lib.SkEpilogue(bias=bias.data_ptr(), activation=act)
 
 
 def streamk_fp16(A, B, *, Wq=None, scales=None, layout="nt", out=None, plan=None, config=None,
-                 zero=8, group=128, bias=None, **kw):
+                 zero=8, group=128, bias=None, activation=None, **kw):
     """C = A @ B.T (layout 'nt', B is [N,K]) or A @ B (layout 'nn', B is [K,N]) in fp16 with fp32
     accumulation.
 
     With `Wq` (uint8 [N, K/2], low nibble = even k) and `scales` (fp16 [N, K/group]) the weights
     are dequantised on the fly, w = fp16((q - zero) * scale), and B is ignored (pass None).
     `config`/kwargs: bm, bn, bk, grid, schedule, fixup, raster (see plan.make_config).
-    `bias` (fp16 [N]) is added to every row in fp32 before the rounding to fp16.
+    `bias` (fp16 [N]) is added to every row in fp32 before the rounding to fp16; `activation`
+    ('relu', 'gelu_tanh', 'silu') is applied after it, also in fp32.
     """
     if Wq is not None:
-        return streamk_q4(A, Wq, scales, out=out, plan=plan, config=config, zero=zero, group=group, bias=bias, **kw)
+        return streamk_q4(A, Wq, scales, out=out, plan=plan, config=config, zero=zero, group=group, bias=bias,
+                          activation=activation, **kw)
     _check_matrix(A, "A", torch.float16)
     _check_matrix(B, "B", torch.float16)
     if layout not in ("nt", "nn"):
@@ -95,7 +101,7 @@ def streamk_fp16(A, B, *, Wq=None, scales=None, layout="nt", out=None, plan=None
     if tuple(C.shape) != (M, N):
         raise ValueError("out has the wrong shape")
     ws = _workspace(plan.workspace_bytes, A.device)
-    epi = _epilogue(bias, N, torch.float16, A.device)
+    epi = _epilogue(bias, N, torch.float16, A.device, activation)
     args = (A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, A.stride(0), B.stride(0), C.stride(0),
             ctypes.byref(plan), ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
             _stream_ptr())
@@ -104,7 +110,7 @@ def streamk_fp16(A, B, *, Wq=None, scales=None, layout="nt", out=None, plan=None
     return C
 
 
-def streamk_bf16(A, B, *, layout="nt", out=None, plan=None, config=None, bias=None, **kw):
+def streamk_bf16(A, B, *, layout="nt", out=None, plan=None, config=None, bias=None, activation=None, **kw):
     """streamk_fp16 for bfloat16 operands and output (fp32 accumulation, C rounded to nearest even).
     The reference's scripts are fp16 / fp32 only; this is the bfloat16 instance of the same tile
     kernels."""
@@ -123,7 +129,7 @@ def streamk_bf16(A, B, *, layout="nt", out=None, plan=None, config=None, bias=No
     if tuple(C.shape) != (M, N):
         raise ValueError("out has the wrong shape")
     ws = _workspace(plan.workspace_bytes, A.device)
-    epi = _epilogue(bias, N, torch.bfloat16, A.device)
+    epi = _epilogue(bias, N, torch.bfloat16, A.device, activation)
     args = (A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, A.stride(0), B.stride(0), C.stride(0),
             ctypes.byref(plan), ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
             _stream_ptr())
@@ -240,11 +246,11 @@ def _zero_points(zeros, scales):
 
 
 def streamk_q4(A, Wq, scales, *, out=None, plan=None, config=None, zero=8, group=128, tiled=False, zeros=None,
-               bias=None, **kw):
+               bias=None, activation=None, **kw):
     """C[M,N] fp16 = A[M,K] fp16 @ dequant(Wq)[N,K].T, weights in natural nibble order
     (streamk_fp16_ladder_block_reduce_q4.py:552).  tiled=True: Wq is the output of tile_q4 (N is
     then taken from scales).  zeros: one zero point per scale group and row ([N, K/group], integers
-    0..15) instead of the scalar `zero`."""
+    0..15) instead of the scalar `zero`.  bias / activation: as for streamk_fp16."""
     if zeros is not None:
         if tiled:
             raise ValueError("per-group zero points need the row-major weights")
@@ -273,15 +279,16 @@ def streamk_q4(A, Wq, scales, *, out=None, plan=None, config=None, zero=8, group
         if M <= 4 * Q4_MAX_M:
             for m0 in range(0, M, Q4_MAX_M):
                 streamk_q4(A[m0:m0 + Q4_MAX_M], Wq, scales, out=C[m0:m0 + Q4_MAX_M], config=config, zero=zero,
-                           group=group, tiled=tiled, zeros=zeros, bias=bias, **kw)
+                           group=group, tiled=tiled, zeros=zeros, bias=bias, activation=activation, **kw)
             return C
         if tiled:
             raise ValueError("more than 256 rows of A need the row-major weights (they are dequantised once)")
-        return streamk_fp16(A, dequant_q4(Wq, scales, zero=zero, group=group, zeros=zeros), out=C, bias=bias)
+        return streamk_fp16(A, dequant_q4(Wq, scales, zero=zero, group=group, zeros=zeros), out=C, bias=bias,
+                            activation=activation)
     if plan is None:
         plan = make_plan(M, N, K, "q4_zp" if zeros is not None else ("q4_tiled" if tiled else "q4"), "nt", config, **kw)
     ws = _workspace(plan.workspace_bytes, A.device)
-    epi = _epilogue(bias, N, torch.float16, A.device)
+    epi = _epilogue(bias, N, torch.float16, A.device, activation)
     tail = (ctypes.byref(plan), ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
             _stream_ptr())
     L = _lib.lib()

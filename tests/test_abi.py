@@ -151,7 +151,7 @@ def test_error_codes(sk):
                          None, 0, None) == -3
     assert L.sk_gemm_f16(ctypes.c_void_p(4098), fake, fake, 1024, 1024, 8192, 8192, 8192, 1024,
                          ctypes.byref(plan), None, 0, None) == -3
-    # the extended entry points: reserved fields must be zero, the bias 2-byte aligned; checked before anything runs
+    # the extended entry points: reserved fields must be zero, the bias 2-byte aligned, the activation known; checked before anything runs
     from streamk._lib import SkEpilogue
     epi = SkEpilogue(bias=4096)
     epi.reserved[1] = 7
@@ -159,6 +159,10 @@ def test_error_codes(sk):
                             ctypes.byref(epi)) == -4
     assert L.sk_gemm_f16_ex(fake, fake, fake, 1024, 1024, 8192, 8192, 8192, 1024, ctypes.byref(plan), None, 0, None,
                             ctypes.byref(SkEpilogue(bias=4097))) == -3
+    # activation codes outside sk_activation, and a bias that cannot be a device address
+    for bad in (SkEpilogue(bias=4096, activation=4), SkEpilogue(bias=None, activation=-1), SkEpilogue(bias=1 << 61)):
+        assert L.sk_gemm_f16_ex(fake, fake, fake, 1024, 1024, 8192, 8192, 8192, 1024, ctypes.byref(plan), None, 0, None,
+                                ctypes.byref(bad)) == -4
     assert L.sk_gemm_f16_ex(None, fake, fake, 1024, 1024, 8192, 8192, 8192, 1024, ctypes.byref(plan), None, 0, None,
                             None) == -1
     assert L.sk_dequant_q4(fake, fake, fake, 16, 100, 128, 8, None) == -4

@@ -728,6 +728,86 @@ def test_fused_bias_epilogue(sk, oracle):
     sk.workspace_status()
 
 
+def test_fused_activation_epilogue(sk, oracle):
+    """activation applied after the bias in fp32, before the rounding: relu on {-1,0,1} operands with an integer
+    bias is exact in every kernel family and schedule (and shows that a tile shared by several CTAs is activated
+    once, after its partials are summed); gelu_tanh and silu against the host functions on the fp32 product
+    (1e-3 of the largest value, as for the plain product); with and without a bias; bfloat16; Q4 in all formats;
+    a linear layer with its activation fused."""
+    import torch
+    rng = np.random.default_rng(92)
+    cases = [  # (M, N, K, layout, config)
+        (200, 1000, 328, "nt", dict(bm=256, bn=256, bk=64, variant=5)), (200, 1000, 328, "nt", dict(bm=128, bn=128, bk=64, variant=2)),
+        (200, 1000, 328, "nt", dict(bm=128, bn=128, bk=64, variant=1)), (200, 1000, 328, "nt", dict(bm=64, bn=64, bk=32, variant=6)),
+        (200, 1000, 328, "nn", dict(bm=128, bn=128, bk=64, variant=5)),
+        (40, 1000, 1024, "nt", dict(bm=64, bn=64, bk=128)), (9, 1000, 1024, "nt", dict(bm=16, bn=32, bk=512)),
+        (1, 1000, 1024, "nt", dict(bm=16, bn=16, bk=512, variant=3)), (1, 1000, 1024, "nt", dict(bm=16, bn=64, bk=128, variant=2)),
+    ]
+    for (M, N, K, layout, cfg) in cases:
+        A = rng.integers(-1, 2, (M, K)).astype(np.float16)
+        B = rng.integers(-1, 2, (N, K) if layout == "nt" else (K, N)).astype(np.float16)
+        bias = rng.integers(-20, 20, N).astype(np.float16)
+        prod = A.astype(np.float64) @ (B.T if layout == "nt" else B).astype(np.float64)
+        Af = (rng.random((M, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+        Bf = (B.astype(np.float32) * 0.125).astype(np.float16)  # keeps the product in the curved part of gelu / silu
+        bf = (rng.random(N, dtype=np.float32) * 4 - 2).astype(np.float16)
+        reff = oracle.matmul_fp32(Af, Bf, trans_b=layout == "nt")
+        for sch in (dict(schedule="dp"), dict(schedule="basic", fixup="reduce", grid=12), dict(schedule="sk2", fixup="atomic", grid=10)):
+            plan = sk.make_plan(M, N, K, "float16", layout, dict(cfg, **sch))
+            C = sk.streamk_fp16(_t(A), _t(B), layout=layout, plan=plan, bias=_t(bias), activation="relu")
+            assert np.array_equal(C.double().cpu().numpy(), np.maximum(prod + bias, 0)), (M, N, K, layout, cfg, sch)
+            C = sk.streamk_fp16(_t(A), _t(B), layout=layout, plan=plan, activation="relu")
+            assert np.array_equal(C.double().cpu().numpy(), np.maximum(prod, 0)), (M, N, K, layout, cfg, sch)
+            for act in ("gelu_tanh", "silu"):
+                C = sk.streamk_fp16(_t(Af), _t(Bf), layout=layout, plan=plan, bias=_t(bf), activation=act)
+                assert _rel(oracle, C, oracle.activation_ref(reff + bf.astype(np.float32), act)) <= 1e-3, (M, N, K, layout, cfg, sch, act)
+                C = sk.streamk_fp16(_t(Af), _t(Bf), layout=layout, plan=plan, activation=act)
+                assert _rel(oracle, C, oracle.activation_ref(reff, act)) <= 1e-3, (M, N, K, layout, cfg, sch, act)
+    # bfloat16
+    A, B = torch.randint(-1, 2, (200, 328)).bfloat16(), torch.randint(-1, 2, (1000, 328)).bfloat16()
+    bias = torch.randint(-20, 20, (1000,)).bfloat16()
+    want = torch.relu(A.double() @ B.double().T + bias.double())
+    for cfg in (dict(bm=256, bn=256, bk=64), dict(bm=64, bn=64, bk=32, schedule="basic", fixup="reduce", grid=12)):
+        C = sk.streamk_bf16(A.cuda(), B.cuda(), bias=bias.cuda(), activation="relu", **cfg)
+        assert torch.equal(C.double().cpu(), want), cfg
+        C = sk.streamk_bf16(A.cuda(), (B * 0.125).cuda(), activation="silu", **cfg)
+        ref = oracle.activation_ref((A.double() @ B.double().T * 0.125).numpy(), "silu")
+        assert _rel(oracle, C, ref) <= 6e-3, cfg  # bfloat16 carries 8 bits
+    # Q4: general small-M, single row, matrix-vector, tiled and per-group zero points
+    M, N, K = 5, 1000, 1152
+    Wq = rng.integers(0, 256, (N, K // 2), dtype=np.uint8)
+    sc = rng.uniform(0.005, 0.02, (N, K // 128)).astype(np.float16)
+    zp = rng.integers(0, 16, (N, K // 128)).astype(np.float16)
+    bias = (rng.random(N, dtype=np.float32) * 2 - 1).astype(np.float16)
+    for m in (M, 1):
+        A = (rng.random((m, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+        for act in ("relu", "gelu_tanh", "silu"):
+            ref = oracle.activation_ref(oracle.q4_gemm_ref(A, Wq, sc, 128, 8) + bias.astype(np.float32), act)
+            refz = oracle.activation_ref(oracle.q4_zp_gemm_ref(A, Wq, sc, zp), act)
+            for sch in (dict(schedule="dp"), dict(schedule="sk2", fixup="reduce", grid=48)):
+                for variant in ((1,) if m > 1 else (1, 2, 3)):
+                    C = sk.streamk_q4(_t(A), _t(Wq), _t(sc), bias=_t(bias), activation=act, variant=variant, **sch)
+                    assert _rel(oracle, C, ref) <= 2e-3, (m, variant, sch, act)
+                C = sk.streamk_q4(_t(A), sk.tile_q4(_t(Wq)), _t(sc), tiled=True, bias=_t(bias), activation=act, **sch)
+                assert _rel(oracle, C, ref) <= 2e-3, (m, "tiled", sch, act)
+                C = sk.streamk_q4(_t(A), _t(Wq), _t(sc), zeros=_t(zp), activation=act, **sch)
+                assert _rel(oracle, C, refz) <= 2e-3, (m, "zp", sch, act)
+    # a linear layer with its activation in the epilogue, against torch's own layer + activation
+    lin = torch.nn.Linear(1024, 1000, bias=True).half().cuda()
+    x = torch.randn(3, 7, 1024, dtype=torch.float16, device="cuda") * 0.5
+    for act, fn in (("relu", torch.relu), ("silu", torch.nn.functional.silu),
+                    ("gelu_tanh", lambda v: torch.nn.functional.gelu(v, approximate="tanh"))):
+        m = sk.StreamKLinear.from_linear(lin, activation=act)
+        want = fn(x.float() @ lin.weight.float().T + lin.bias.float())
+        assert _rel(oracle, m(x).reshape(21, 1000), want.detach().reshape(21, 1000).cpu().numpy()) <= 1e-3, act
+    X, Y = torch.zeros(8, 64, dtype=torch.float16, device="cuda"), torch.zeros(24, 64, dtype=torch.float16, device="cuda")
+    with pytest.raises(ValueError):
+        sk.streamk_fp16(X, Y, activation="tanh")
+    with pytest.raises(ValueError):
+        sk.StreamKLinear(64, 24, activation="tanh")
+    sk.workspace_status()
+
+
 def test_one_byte_operands_at_full_size(sk, oracle):
     """fp8 and int8 at M = N = K = 8192 with the plans the library picks there (tuned cache or heuristic) and with
     an explicit Stream-K plan: 48 random rows against the host product (int8: equal; fp8: 1e-3), and the exact

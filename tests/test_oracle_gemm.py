@@ -121,3 +121,24 @@ def test_i8_gemm_ref(oracle):
     A, B = rs.randint(-128, 128, (5, 37)).astype(np.int8), rs.randint(-128, 128, (4, 37)).astype(np.int8)
     want = [[sum(int(a) * int(b) for a, b in zip(ra, rb)) for rb in B] for ra in A]
     assert np.array_equal(oracle.i8_gemm_ref(A, B), want)
+
+
+def test_activation_ref(oracle):
+    """The activations of the fused epilogue against torch's CPU routines (float64), the erf form of GELU (the
+    tanh form stays within 1e-3 of it), and their limits: 0 at 0, the identity far right, 0 far left."""
+    import torch
+    from scipy.special import erf
+    x = np.concatenate([np.linspace(-12, 12, 4801), [0.0, 1e-8, -1e-8, 40.0, -40.0, 700.0, -700.0]])
+    t = torch.from_numpy(x)
+    assert np.array_equal(oracle.activation_ref(x, "relu"), torch.relu(t).numpy())
+    assert np.allclose(oracle.activation_ref(x, "gelu_tanh"), torch.nn.functional.gelu(t, approximate="tanh").numpy(),
+                       rtol=1e-12, atol=1e-14)  # 1 + tanh cancels in the far left tail
+    assert np.allclose(oracle.activation_ref(x, "silu"), torch.nn.functional.silu(t).numpy(), rtol=1e-12,
+                       atol=1e-300)
+    assert np.max(np.abs(oracle.activation_ref(x, "gelu_tanh") - 0.5 * x * (1 + erf(x / np.sqrt(2))))) < 1e-3
+    for name in ("relu", "gelu_tanh", "silu"):
+        y = oracle.activation_ref(np.array([0.0, 40.0, -40.0]), name)
+        assert y[0] == 0 and abs(y[1] - 40.0) < 1e-12 and abs(y[2]) < 1e-12, name
+    assert np.array_equal(oracle.activation_ref(x, None), x)
+    with pytest.raises(ValueError):
+        oracle.activation_ref(x, "tanh")
