@@ -206,6 +206,11 @@ int sk_gemm_bf16(const void *A, const void *B, void *C, int64_t M, int64_t N, in
 int sk_gemm_f8(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
                int64_t ldb, int64_t ldc, float alpha, const sk_plan *plan, void *ws, size_t ws_bytes,
                void *stream);
+/* The same with the epilogue of the *_ex entry points: C = activation(alpha * A B^T + bias), bias in fp16
+ * (C's type). */
+int sk_gemm_f8_ex(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                  int64_t ldb, int64_t ldc, float alpha, const sk_plan *plan, void *ws, size_t ws_bytes,
+                  void *stream, const sk_epilogue *epi);
 
 /* int8 operands: A [M,K] and B [N,K] (NT only) int8, C int32 (ldc in int32 elements), exact int32
  * accumulation (wraps beyond 2^31, i.e. not below K = 133 000); the plan is made with dtype SK_I8.  The

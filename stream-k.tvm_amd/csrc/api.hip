@@ -255,7 +255,9 @@ extern "C" int sk_gemm_bf16(const void *A, const void *B, void *C, int64_t M, in
 // dimensions of A and B are handed to the kernel in 16-bit units
 static int gemm_8bit(int dtype, const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,
                      int64_t lda, int64_t ldb, int64_t ldc, float alpha, const sk_plan *plan, void *ws,
-                     size_t ws_bytes, void *stream) {
+                     size_t ws_bytes, void *stream, const sk_epilogue *epi = nullptr) {
+  const void *bias = nullptr;  // the kernels' epilogue word (fp8 only: the int8 kernels store int32 sums)
+  if (int rc = epilogue_word(epi, &bias)) return rc;
   if (!A || !B || !C) return SK_ERR_NULL;
   int rc = check_plan(plan, M, N, K, dtype, SK_LAYOUT_NT);
   if (rc) return rc;
@@ -272,7 +274,7 @@ static int gemm_8bit(int dtype, const void *A, const void *B, void *C, int64_t M
   rc = make_dev_plan(plan, k, ws, ws_bytes, cached_occupancy(k->id, false), (hipStream_t)stream, &dp, &w);
   if (rc) return rc;
   GemmArgs a{(const half_t *)A, (const half_t *)B, (half_t *)C, (int)M, (int)N, (int)(K / 2), lda / 2, ldb / 2, ldc, alpha};
-  return launch_tile_f16(k->id, a, dp, w, (hipStream_t)stream, nullptr) == 0 ? SK_OK : SK_ERR_LAUNCH;
+  return launch_tile_f16(k->id, a, dp, w, (hipStream_t)stream, bias) == 0 ? SK_OK : SK_ERR_LAUNCH;
 }
 
 extern "C" int sk_gemm_f8(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,
@@ -281,6 +283,14 @@ extern "C" int sk_gemm_f8(const void *A, const void *B, void *C, int64_t M, int6
   if (!(alpha == alpha) || alpha - alpha != 0.f) return SK_ERR_CONFIG;  // NaN or infinite
   const int dtype = plan && plan->dtype == SK_F8E5M2 ? SK_F8E5M2 : SK_F8E4M3;  // which format the bytes are in
   return gemm_8bit(dtype, A, B, C, M, N, K, lda, ldb, ldc, alpha, plan, ws, ws_bytes, stream);
+}
+
+extern "C" int sk_gemm_f8_ex(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,
+                             int64_t lda, int64_t ldb, int64_t ldc, float alpha, const sk_plan *plan, void *ws,
+                             size_t ws_bytes, void *stream, const sk_epilogue *epi) {
+  if (!(alpha == alpha) || alpha - alpha != 0.f) return SK_ERR_CONFIG;
+  const int dtype = plan && plan->dtype == SK_F8E5M2 ? SK_F8E5M2 : SK_F8E4M3;
+  return gemm_8bit(dtype, A, B, C, M, N, K, lda, ldb, ldc, alpha, plan, ws, ws_bytes, stream, epi);
 }
 
 // (C and ldc are int32 here; the kernel casts)

@@ -99,6 +99,8 @@ def lib():
     L.sk_gemm_q4_ex.restype = ci
     L.sk_gemm_f8.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, ctypes.c_float, P(SkPlan), vp, sz, vp]
     L.sk_gemm_f8.restype = ci
+    L.sk_gemm_f8_ex.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, ctypes.c_float, P(SkPlan), vp, sz, vp, P(SkEpilogue)]
+    L.sk_gemm_f8_ex.restype = ci
     L.sk_gemm_i8.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, P(SkPlan), vp, sz, vp]
     L.sk_gemm_i8.restype = ci
     L.sk_gemm_q4.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, ci, ci, P(SkPlan), vp, sz, vp]

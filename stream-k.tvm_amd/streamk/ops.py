@@ -138,11 +138,12 @@ def streamk_bf16(A, B, *, layout="nt", out=None, plan=None, config=None, bias=No
     return C
 
 
-def streamk_fp8(A, B, *, alpha=1.0, fmt=None, out=None, plan=None, config=None, **kw):
-    """C = alpha * (A @ B.T) for fp8 operands, A [M,K], B [N,K]; fp32 accumulation, alpha applied to the
+def streamk_fp8(A, B, *, alpha=1.0, fmt=None, out=None, plan=None, config=None, bias=None, activation=None, **kw):
+    """C = activation(alpha * (A @ B.T) + bias) for fp8 operands, A [M,K], B [N,K]; fp32 accumulation, alpha applied to the
     fp32 sums, fp16 C.  Both operands are OCP e4m3 (torch.float8_e4m3fn) or both OCP e5m2
     (torch.float8_e5m2); raw uint8 bytes are taken as `fmt` ("e4m3" by default, or "e5m2").  alpha is the
-    product of the per-tensor scales of a scaled-fp8 caller.  The reference's scripts stop at fp16; this is
+    product of the per-tensor scales of a scaled-fp8 caller; bias (fp16 [N]) and activation as for
+    streamk_fp16, applied after alpha.  The reference's scripts stop at fp16; this is
     the same partitioner and fix-ups over the fp8 form of the tile kernel."""
     kinds = {getattr(torch, "float8_e4m3fn", None): "e4m3", getattr(torch, "float8_e5m2", None): "e5m2"}
     for t, name in ((A, "A"), (B, "B")):
@@ -169,10 +170,11 @@ def streamk_fp8(A, B, *, alpha=1.0, fmt=None, out=None, plan=None, config=None, 
     if tuple(C.shape) != (M, N):
         raise ValueError("out has the wrong shape")
     ws = _workspace(plan.workspace_bytes, A.device)
-    rc = _lib.lib().sk_gemm_f8(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, A.stride(0),
-                               B.stride(0), C.stride(0), float(alpha), ctypes.byref(plan),
-                               ws.data_ptr() if ws is not None else None,
-                               ws.numel() if ws is not None else 0, _stream_ptr())
+    epi = _epilogue(bias, N, torch.float16, A.device, activation)
+    args = (A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, A.stride(0), B.stride(0), C.stride(0), float(alpha),
+            ctypes.byref(plan), ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
+            _stream_ptr())
+    rc = _lib.lib().sk_gemm_f8(*args) if epi is None else _lib.lib().sk_gemm_f8_ex(*args, ctypes.byref(epi))
     _lib.check(rc, "sk_gemm_f8")
     return C
 

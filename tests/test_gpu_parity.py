@@ -792,6 +792,21 @@ def test_fused_activation_epilogue(sk, oracle):
                 assert _rel(oracle, C, ref) <= 2e-3, (m, "tiled", sch, act)
                 C = sk.streamk_q4(_t(A), _t(Wq), _t(sc), zeros=_t(zp), activation=act, **sch)
                 assert _rel(oracle, C, refz) <= 2e-3, (m, "zp", sch, act)
+    # fp8 (both formats, raw bytes): alpha first, then bias, then the activation; exact with relu on {-1,0,1} data
+    for fmt, dt, ref_fmt in (("e4m3", torch.float8_e4m3fn, "e4m3"), ("e5m2", torch.float8_e5m2, "e5m2")):
+        Ai, Bi = torch.randint(-1, 2, (200, 336)).float().to(dt), torch.randint(-1, 2, (1000, 336)).float().to(dt)
+        bias = torch.randint(-20, 20, (1000,)).half()
+        prod = oracle.f8_gemm_ref(Ai.view(torch.uint8).numpy(), Bi.view(torch.uint8).numpy(), ref_fmt)
+        Af, Bf = torch.randn(200, 336).to(dt), torch.randn(1000, 336).to(dt)
+        reff = oracle.f8_gemm_ref(Af.view(torch.uint8).numpy(), Bf.view(torch.uint8).numpy(), ref_fmt)
+        for cfg in (dict(bm=256, bn=256), dict(bm=128, bn=128, schedule="basic", fixup="reduce", grid=12),
+                    dict(bm=128, bn=256, schedule="sk2", fixup="atomic", grid=10)):
+            C = sk.streamk_fp8(Ai.cuda(), Bi.cuda(), alpha=0.5, bias=bias.cuda(), activation="relu", **cfg)
+            assert np.array_equal(C.double().cpu().numpy(), np.maximum(0.5 * prod + bias.double().numpy(), 0)), (fmt, cfg)
+            C = sk.streamk_fp8(Af.cuda(), Bf.cuda(), alpha=0.0625, bias=bias.cuda(), activation="silu", **cfg)
+            assert _rel(oracle, C, oracle.activation_ref(0.0625 * reff + bias.float().numpy(), "silu")) <= 1e-3, (fmt, cfg)
+            C = sk.streamk_fp8(Af.cuda(), Bf.cuda(), alpha=0.0625, activation="gelu_tanh", **cfg)
+            assert _rel(oracle, C, oracle.activation_ref(0.0625 * reff, "gelu_tanh")) <= 1e-3, (fmt, cfg)
     # a linear layer with its activation in the epilogue, against torch's own layer + activation
     lin = torch.nn.Linear(1024, 1000, bias=True).half().cuda()
     x = torch.randn(3, 7, 1024, dtype=torch.float16, device="cuda") * 0.5
