@@ -119,6 +119,20 @@ struct KernelInfo {
   X(131, 1, 1, 2, 4, 1, 2, 0)    \
   X(132, 1, 1, 4, 2, 1, 2, 0)
 
+// bfloat16 twins of the fp16 small-M kernels above (dtype SK_BF16):  X(id, MB, NB, WN, RK, DEPTH, ROW1)
+#define SK_SKINNY_BF16_KERNELS(X) \
+  X(230, 1, 1, 4, 1, 2, 0)        \
+  X(231, 2, 1, 4, 1, 2, 0)        \
+  X(232, 4, 1, 4, 1, 2, 0)        \
+  X(233, 1, 1, 1, 4, 2, 0)        \
+  X(234, 1, 1, 2, 2, 2, 0)        \
+  X(235, 1, 1, 1, 1, 4, 1)        \
+  X(236, 1, 1, 4, 1, 4, 1)        \
+  X(237, 1, 1, 2, 4, 2, 0)        \
+  X(238, 1, 1, 4, 2, 2, 0)        \
+  X(239, 2, 1, 4, 2, 2, 0)        \
+  X(240, 4, 1, 4, 2, 2, 0)
+
 // M == 1 Q4 matrix-vector kernels (variant 2):  X(id, NB, WN, RK, DEPTH, KMAX)
 // KMAX is the largest K range one segment may span (A is kept in LDS for the whole segment).
 #define SK_GEMV_Q4_KERNELS(X)  \

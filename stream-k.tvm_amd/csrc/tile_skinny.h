@@ -100,9 +100,13 @@ __device__ __forceinline__ void stage_scales(half_t *ldsS, const half_t *scales_
 //
 // ZP_ (Q4 only): one zero point per scale group and row (a.zeros, same shape as the scales) instead of
 // one for the whole matrix; staged in LDS beside the scales.
+//
+// BF16_ (not Q4): operands, bias and C are bfloat16 -- the same 16-bit data movement, the bfloat16 form of the
+// MFMA, C rounded to nearest even.
 template <int MB_, int NB_, int WN_, int RK_, bool Q4_, int DEPTH_, bool ROW1_ = false, bool TILED_ = false,
-          bool ZP_ = false>
+          bool ZP_ = false, bool BF16_ = false>
 struct TileSkinny {
+  static_assert(!BF16_ || !Q4_, "the Q4 decode produces fp16");
   static_assert(!TILED_ || Q4_, "tiled weights exist for Q4");
   static_assert(!ZP_ || Q4_, "zero points exist for Q4");
   typedef SkinnyArgs Args;
@@ -314,7 +318,13 @@ struct TileSkinny {
             }
 #pragma unroll
             for (int i = 0; i < MB; ++i)
-              acc.c[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fw, fa[i], acc.c[i][j], 0, 0, 0);
+              if constexpr (BF16_) {
+                typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+                acc.c[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, fw),
+                                                                      __builtin_bit_cast(bf16x8, fa[i]), acc.c[i][j], 0, 0, 0);
+              } else {
+                acc.c[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fw, fa[i], acc.c[i][j], 0, 0, 0);
+              }
           }
         }
         // A tile of the next iteration into the other LDS buffer, then refill this ring slot
@@ -380,8 +390,13 @@ struct TileSkinny {
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             float x = acc.c[i][j][e];
-            if constexpr (BIAS) x = activate(x + bias_at(bias, col + e, a.N), act);
-            h[e] = (half_t)x;
+            if constexpr (BIAS) x = activate(x + bias_at<BF16_>(bias, col + e, a.N), act);
+            if constexpr (BF16_) {
+              const __bf16 b = (__bf16)x;
+              h[e] = __builtin_bit_cast(half_t, b);  // C carries 16-bit patterns
+            } else {
+              h[e] = (half_t)x;
+            }
           }
           half_t *dst = a.C + (int64_t)row * a.ldc + col;
           if (vec_ok && col + 4 <= a.N) {

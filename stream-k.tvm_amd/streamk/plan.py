@@ -77,6 +77,15 @@ def make_plan(M, N, K, dtype="float16", layout="nt", config=None, cus=None, use_
     kw = {k: v for k, v in kw.items() if v is not None}
     if use_tuned and not config and not kw and cus is None:
         config = tuned_config(M, N, K, dtype, layout)
+        if config is None and dtype == "bfloat16":
+            # the bfloat16 kernels are twins of the fp16 ones (same data movement, same MFMA rate): a shape tuned
+            # for fp16 only takes that entry, where the kernel it names has a twin
+            borrowed = tuned_config(M, N, K, "float16", layout)
+            if borrowed is not None:
+                try:
+                    return make_plan(M, N, K, dtype, layout, borrowed)
+                except _lib.StreamKError:
+                    pass
     cfg = make_config(config, **kw)
     plan = SkPlan()
     rc = _lib.lib().sk_make_plan(M, N, K, _DTYPES[dtype], _LAYOUTS[layout], ctypes.byref(cfg),

@@ -518,6 +518,56 @@ def test_bf16_tile_kernels(sk, oracle):
     sk.workspace_status()
 
 
+def test_bf16_small_m_kernels(sk, oracle):
+    """bfloat16 instances of the weight-streaming small-M kernels (M <= 64): every instance, ragged N, K tails,
+    data-parallel, Stream-K with both fix-ups and fixed split-K; {-1,0,1} operands must come out exact (|sums| <= 256)
+    and random ones within 4e-3 of the fp32 host product (bfloat16 rounds C to 8 bits); the bias and activation
+    epilogue in bfloat16; the plans the library picks by itself for 1..32 rows are these kernels."""
+    import torch
+    torch.manual_seed(17)
+    cfgs = SKINNY_CONFIGS + [dict(bm=16, bn=16, bk=128, variant=2), dict(bm=16, bn=64, bk=128, variant=2)]
+    N, K = 1000, 1032
+    B = (torch.rand(N, K) * 2 - 1).bfloat16()
+    Bi = torch.randint(-1, 2, (N, K)).bfloat16()
+    bias = torch.randint(-20, 20, (N,)).bfloat16()
+    for cfg in cfgs:
+        row1 = cfg.get("variant") == 2
+        for M in ((1,) if row1 else (cfg["bm"], cfg["bm"] - 3, 1)):
+            A = (torch.rand(M, K) * 2 - 1).bfloat16()
+            Ai = torch.randint(-1, 2, (M, K)).bfloat16()
+            Ai[:, 200:] = 0  # keeps the sums within bfloat16's exact integers
+            ref = oracle.matmul_fp32(A.float().numpy(), B.float().numpy(), trans_b=True)
+            exact = (Ai.double() @ Bi.double().T).numpy()
+            assert np.abs(exact).max() <= 256
+            schedules = [dict(schedule="dp"), dict(schedule="sk2", fixup="reduce", grid=24),
+                         dict(schedule="sk2", fixup="atomic", grid=20)]
+            if -(-K // cfg["bk"]) % 3 == 0:  # fixed split-K takes a factor of the K-iteration count
+                schedules.append(dict(schedule="splitk", split=3, fixup="reduce"))
+            for sch in schedules:
+                plan = sk.make_plan(M, N, K, "bfloat16", "nt", dict(cfg, **sch))
+                assert 230 <= plan.kernel_id <= 240, (cfg, plan.kernel_id)
+                C = sk.streamk_bf16(A.cuda(), B.cuda(), plan=plan)
+                assert C.dtype == torch.bfloat16 and _rel(oracle, C, ref) <= 4e-3 <= TOL, (cfg, M, sch)
+                Ci = sk.streamk_bf16(Ai.cuda(), Bi.cuda(), plan=plan)
+                assert np.array_equal(Ci.double().cpu().numpy(), exact), (cfg, M, sch)
+                Cb = sk.streamk_bf16(Ai.cuda(), Bi.cuda(), plan=plan, bias=bias.cuda(), activation="relu")
+                assert np.array_equal(Cb.double().cpu().numpy(), np.maximum(exact + bias.double().numpy(), 0)), (cfg, M, sch)
+                if sch.get("fixup") == "reduce":
+                    assert torch.equal(C, sk.streamk_bf16(A.cuda(), B.cuda(), plan=plan))
+    for M in (1, 2, 16, 32):
+        plan = sk.make_plan(M, 4096, 4096, "bfloat16", "nt")
+        assert 230 <= plan.kernel_id <= 240, (M, plan.kernel_id)
+        A, W = (torch.rand(M, 4096) * 2 - 1).bfloat16(), (torch.rand(4096, 4096) * 2 - 1).bfloat16()
+        ref = oracle.matmul_fp32(A.float().numpy(), W.float().numpy(), trans_b=True)
+        assert _rel(oracle, sk.streamk_bf16(A.cuda(), W.cuda()), ref) <= 4e-3, M
+    # a shape tuned for fp16 only: the bfloat16 plan takes that entry (its kernel has a bfloat16 twin)
+    if sk.tuned_config(16, 8192, 8192, "bfloat16") is None and sk.tuned_config(16, 8192, 8192, "float16"):
+        want = sk.make_plan(16, 8192, 8192, "float16")
+        got = sk.make_plan(16, 8192, 8192, "bfloat16")
+        assert (got.bm, got.bn, got.bk, got.grid, got.schedule) == (want.bm, want.bn, want.bk, want.grid, want.schedule)
+    sk.workspace_status()
+
+
 def test_fp8_tile_kernels(sk, oracle):
     """fp8 (OCP e4m3) operands, fp16 C: every instance, ragged shapes, K tails (K a multiple of 16 but not
     of the 128-value iteration), all schedules and both fix-ups against the float64 host product of the
