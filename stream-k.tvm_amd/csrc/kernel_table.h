@@ -184,6 +184,17 @@ struct KernelInfo {
   X(166, 1, 1, 4, 4, 32768)    \
   X(167, 2, 1, 4, 2, 32768)
 
+// bfloat16 twins of the fp16 matrix-vector kernels (dtype SK_BF16, variant 2)
+#define SK_GEMV_BF16_KERNELS(X) \
+  X(241, 1, 1, 4, 4, 8192)      \
+  X(242, 1, 1, 8, 4, 8192)      \
+  X(243, 2, 1, 4, 2, 8192)      \
+  X(244, 1, 4, 1, 4, 8192)      \
+  X(245, 1, 2, 2, 4, 8192)      \
+  X(246, 1, 1, 2, 4, 8192)      \
+  X(247, 1, 1, 4, 4, 32768)     \
+  X(248, 2, 1, 4, 2, 32768)
+
 // NN layout, 16x16x32 MFMAs (variant 4):  X(id, BM, BN, WM, WN)
 #define SK_TILE_F16_NN_DMA16_KERNELS(X) \
   X(42, 256, 256, 2, 4)                 \

@@ -81,6 +81,15 @@ int skinny_kernel_infos(KernelInfo *out, int max) {
   }
   SK_GEMV_F16_KERNELS(X)
 #undef X
+#define X(id, NB, WN, RK, DEPTH, KMAX)                                                                        \
+  if (n < max) {                                                                                         \
+    typedef TileGemvF16<NB, WN, RK, DEPTH, KMAX, true> P;                                                 \
+    out[n++] = KernelInfo{id, FAMILY_SKINNY, 3, 0, 2, P::BM, P::BN, P::BKC, P::NT, P::LDS_BYTES,         \
+                          P::CTAS_PER_CU, P::TILE_ELEMS, P::MAX_ITERS, P::MAX_M, 8,                      \
+                          "gemv_bf16_nb" #NB "_wn" #WN "_rk" #RK "_k" #KMAX};                                   \
+  }
+  SK_GEMV_BF16_KERNELS(X)
+#undef X
 #define X(id, MB, NB, WN, RK, DEPTH)                                                                     \
   if (n < max) {                                                                                     \
     typedef TileSkinny<MB, NB, WN, RK, true, DEPTH, false, true> P;                                  \
@@ -140,6 +149,13 @@ int launch_skinny(int id, const SkinnyArgs &a, const DevPlan &p, const Workspace
     return launch_policy<P>(a, p, ws, s, bias);                                                         \
   }
     SK_GEMV_F16_KERNELS(X)
+#undef X
+#define X(id_, NB, WN, RK, DEPTH, KMAX)                                                     \
+  case id_: {                                                                              \
+    typedef TileGemvF16<NB, WN, RK, DEPTH, KMAX, true> P;                                   \
+    return launch_policy<P>(a, p, ws, s, bias);                                            \
+  }
+    SK_GEMV_BF16_KERNELS(X)
 #undef X
 #define X(id_, MB, NB, WN, RK, DEPTH)                                                       \
   case id_: {                                                                              \
@@ -204,6 +220,15 @@ int occupancy_skinny(int id) {
     return occ;                                                                                          \
   }
     SK_GEMV_F16_KERNELS(X)
+#undef X
+#define X(id_, NB, WN, RK, DEPTH, KMAX)                                                                      \
+  case id_: {                                                                                            \
+    typedef TileGemvF16<NB, WN, RK, DEPTH, KMAX, true> P;                                                 \
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_skinny_kernel<P>, P::NT, 0) != hipSuccess) \
+      return -1;                                                                                         \
+    return occ;                                                                                          \
+  }
+    SK_GEMV_BF16_KERNELS(X)
 #undef X
 #define X(id_, MB, NB, WN, RK, DEPTH)                                                                     \
   case id_: {                                                                                            \

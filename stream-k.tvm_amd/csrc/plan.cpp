@@ -11,7 +11,7 @@
 
 namespace sk {
 
-static KernelInfo g_table[224];
+static KernelInfo g_table[256];
 static int g_count = -1;
 
 int tile_kernel_infos(KernelInfo *out, int max);
@@ -20,9 +20,9 @@ int f32_kernel_infos(KernelInfo *out, int max);
 
 const KernelInfo *kernel_table(int *count) {
   if (g_count < 0) {
-    int n = tile_kernel_infos(g_table, 224);
-    n += skinny_kernel_infos(g_table + n, 224 - n);
-    n += f32_kernel_infos(g_table + n, 224 - n);
+    int n = tile_kernel_infos(g_table, 256);
+    n += skinny_kernel_infos(g_table + n, 256 - n);
+    n += f32_kernel_infos(g_table + n, 256 - n);
     g_count = n;
   }
   if (count) *count = g_count;
@@ -86,8 +86,8 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
         if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].variant == 0 && t[i].bm == 16 &&
             t[i].bn == 32 && t[i].bk == 1024 && accepts_shape(t[i], M, K))
           return &t[i];
-    // M == 1 with fp16 weights: the same structure, K split over four waves
-    if (dtype == SK_F16 && M == 1 && want_variant < 0)
+    // M == 1 with fp16 / bfloat16 weights: the same structure, K split over four waves
+    if ((dtype == SK_F16 || dtype == SK_BF16) && M == 1 && want_variant < 0)
       for (int i = 0; i < n; ++i)
         if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].layout == layout && t[i].variant == 2 &&
             t[i].bn == 16 && t[i].bk == 512 && accepts_shape(t[i], M, K))

@@ -13,7 +13,8 @@
 
 namespace sk {
 
-template <int NB_, int WN_, int RK_, int DEPTH_, int KMAX_ = 8192>
+// BF16_: the row of A, the weights, the bias and C are bfloat16 (v_mfma_f32_4x4x4_16b_bf16; C rounded to nearest even)
+template <int NB_, int WN_, int RK_, int DEPTH_, int KMAX_ = 8192, bool BF16_ = false>
 struct TileGemvF16 {
   typedef SkinnyArgs Args;
   static constexpr bool LEAN_ENTRY = false;  // see run_persistent
@@ -122,8 +123,16 @@ struct TileGemvF16 {
             const uint4v w = wreg[d][j][c], f = fa[c];
             w0.u[0] = w[0], w0.u[1] = w[1], w1.u[0] = w[2], w1.u[1] = w[3];
             a0.u[0] = f[0], a0.u[1] = f[1], a1.u[0] = f[2], a1.u[1] = f[3];
-            c_acc[j][0] = __builtin_amdgcn_mfma_f32_4x4x4f16(w0.v, a0.v, c_acc[j][0], 0, 0, 0);
-            c_acc[j][1] = __builtin_amdgcn_mfma_f32_4x4x4f16(w1.v, a1.v, c_acc[j][1], 0, 0, 0);
+            if constexpr (BF16_) {
+              typedef short shortx4 __attribute__((ext_vector_type(4)));
+              c_acc[j][0] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(shortx4, w0.v), __builtin_bit_cast(shortx4, a0.v),
+                                                                   c_acc[j][0], 0, 0, 0);
+              c_acc[j][1] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(shortx4, w1.v), __builtin_bit_cast(shortx4, a1.v),
+                                                                   c_acc[j][1], 0, 0, 0);
+            } else {
+              c_acc[j][0] = __builtin_amdgcn_mfma_f32_4x4x4f16(w0.v, a0.v, c_acc[j][0], 0, 0, 0);
+              c_acc[j][1] = __builtin_amdgcn_mfma_f32_4x4x4f16(w1.v, a1.v, c_acc[j][1], 0, 0, 0);
+            }
           }
         issue_loads(d, it + DEPTH);
       }
@@ -165,6 +174,15 @@ struct TileGemvF16 {
     return tid < WN * 64 && (tid & 3) == 0;
   }
 
+  // fp32 -> C's 16-bit pattern
+  static __device__ __forceinline__ half_t to_c(float x) {
+    if constexpr (BF16_) {
+      const __bf16 b = (__bf16)x;
+      return __builtin_bit_cast(half_t, b);
+    } else {
+      return (half_t)x;
+    }
+  }
   static __device__ __forceinline__ void store_c(const Args &a, const Acc &acc, int /*pm*/, int pn, char *,
                                                  const void *bias_) {
     int e;
@@ -173,7 +191,7 @@ struct TileGemvF16 {
 #pragma unroll
       for (int j = 0; j < NB; ++j) {
         const int col = pn * BN + e + j * 16;
-        if (col < a.N) a.C[col] = (half_t)acc.y[j];
+        if (col < a.N) a.C[col] = to_c(acc.y[j]);
       }
     } else {
       const half_t *bias = epi_bias(bias_);
@@ -181,7 +199,7 @@ struct TileGemvF16 {
 #pragma unroll
       for (int j = 0; j < NB; ++j) {
         const int col = pn * BN + e + j * 16;
-        if (col < a.N) a.C[col] = (half_t)activate(acc.y[j] + bias_at(bias, col, a.N), act);
+        if (col < a.N) a.C[col] = to_c(activate(acc.y[j] + bias_at<BF16_>(bias, col, a.N), act));
       }
     }
   }

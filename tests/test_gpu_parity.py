@@ -519,19 +519,22 @@ def test_bf16_tile_kernels(sk, oracle):
 
 
 def test_bf16_small_m_kernels(sk, oracle):
-    """bfloat16 instances of the weight-streaming small-M kernels (M <= 64): every instance, ragged N, K tails,
+    """bfloat16 instances of the weight-streaming small-M kernels (M <= 64) and of the matrix-vector kernels: every instance, ragged N, K tails,
     data-parallel, Stream-K with both fix-ups and fixed split-K; {-1,0,1} operands must come out exact (|sums| <= 256)
     and random ones within 4e-3 of the fp32 host product (bfloat16 rounds C to 8 bits); the bias and activation
     epilogue in bfloat16; the plans the library picks by itself for 1..32 rows are these kernels."""
     import torch
     torch.manual_seed(17)
     cfgs = SKINNY_CONFIGS + [dict(bm=16, bn=16, bk=128, variant=2), dict(bm=16, bn=64, bk=128, variant=2)]
+    # the matrix-vector instances (one row of A, 4x4x4 MFMAs)
+    cfgs += [dict(bm=16, bn=16, bk=512, variant=3), dict(bm=16, bn=16, bk=1024, variant=3), dict(bm=16, bn=32, bk=512, variant=3),
+             dict(bm=16, bn=64, bk=128, variant=3), dict(bm=16, bn=32, bk=256, variant=3), dict(bm=16, bn=16, bk=256, variant=3)]
     N, K = 1000, 1032
     B = (torch.rand(N, K) * 2 - 1).bfloat16()
     Bi = torch.randint(-1, 2, (N, K)).bfloat16()
     bias = torch.randint(-20, 20, (N,)).bfloat16()
     for cfg in cfgs:
-        row1 = cfg.get("variant") == 2
+        row1 = cfg.get("variant") in (2, 3)
         for M in ((1,) if row1 else (cfg["bm"], cfg["bm"] - 3, 1)):
             A = (torch.rand(M, K) * 2 - 1).bfloat16()
             Ai = torch.randint(-1, 2, (M, K)).bfloat16()
@@ -545,7 +548,8 @@ def test_bf16_small_m_kernels(sk, oracle):
                 schedules.append(dict(schedule="splitk", split=3, fixup="reduce"))
             for sch in schedules:
                 plan = sk.make_plan(M, N, K, "bfloat16", "nt", dict(cfg, **sch))
-                assert 230 <= plan.kernel_id <= 240, (cfg, plan.kernel_id)
+                # (without a variant, one row takes the matrix-vector instance of the same tile where there is one)
+                assert (241 if cfg.get("variant") == 3 else 230) <= plan.kernel_id <= (240 if M > 1 else 248), (cfg, plan.kernel_id)
                 C = sk.streamk_bf16(A.cuda(), B.cuda(), plan=plan)
                 assert C.dtype == torch.bfloat16 and _rel(oracle, C, ref) <= 4e-3 <= TOL, (cfg, M, sch)
                 Ci = sk.streamk_bf16(Ai.cuda(), Bi.cuda(), plan=plan)
@@ -556,7 +560,7 @@ def test_bf16_small_m_kernels(sk, oracle):
                     assert torch.equal(C, sk.streamk_bf16(A.cuda(), B.cuda(), plan=plan))
     for M in (1, 2, 16, 32):
         plan = sk.make_plan(M, 4096, 4096, "bfloat16", "nt")
-        assert 230 <= plan.kernel_id <= 240, (M, plan.kernel_id)
+        assert (241 <= plan.kernel_id <= 248) if M == 1 else (230 <= plan.kernel_id <= 240), (M, plan.kernel_id)
         A, W = (torch.rand(M, 4096) * 2 - 1).bfloat16(), (torch.rand(4096, 4096) * 2 - 1).bfloat16()
         ref = oracle.matmul_fp32(A.float().numpy(), W.float().numpy(), trans_b=True)
         assert _rel(oracle, sk.streamk_bf16(A.cuda(), W.cuda()), ref) <= 4e-3, M
