@@ -2,7 +2,7 @@
 
 The reference stops at kernel scripts; wrapping them as an operator of a model is its open item
 ("integrate with BitBLAS", README.md:21).  This module is that wrapper for this library: it owns
-the weight in the layout the kernels read ([N, K] fp16, or packed nibbles + scales), flattens the
+the weight in the layout the kernels read ([N, K] fp16 or bfloat16, or packed nibbles + scales), flattens the
 leading dimensions of the input into M, and keeps one plan per M it has seen (a decode step calls
 with M = batch, a prefill with M = batch * tokens), each taken from the tuned cache when the shape
 is in it.  Inference only: the GEMM is not recorded by autograd.
@@ -20,23 +20,25 @@ class StreamKLinear(torch.nn.Module):
         if activation not in (None, "relu", "gelu_tanh", "silu"):
             raise ValueError("activation must be None, 'relu', 'gelu_tanh' or 'silu'")
         self.activation = activation  # applied in the GEMM's epilogue, after the bias
-        if weight_format not in ("float16", "q4", "q4_zp"):
-            raise ValueError("weight_format must be 'float16', 'q4' or 'q4_zp' (one zero point per group)")
-        if weight_format != "float16" and (group != 128 or in_features % 128):
+        if weight_format not in ("float16", "bfloat16", "q4", "q4_zp"):
+            raise ValueError("weight_format must be 'float16', 'bfloat16', 'q4' or 'q4_zp' (one zero point per group)")
+        if weight_format in ("q4", "q4_zp") and (group != 128 or in_features % 128):
             raise ValueError("Q4 weights need group == 128 and in_features a multiple of 128")
         if in_features % 8:
             raise ValueError("in_features must be a multiple of 8")
         self.in_features, self.out_features = in_features, out_features
         self.weight_format, self.group, self.zero = weight_format, group, zero
         N, K = out_features, in_features
-        if weight_format == "float16":
-            self.register_buffer("weight", torch.zeros(N, K, dtype=torch.float16, device=device))
+        # activations, bias and output are bfloat16 with bfloat16 weights, fp16 otherwise
+        self.dtype = torch.bfloat16 if weight_format == "bfloat16" else torch.float16
+        if weight_format in ("float16", "bfloat16"):
+            self.register_buffer("weight", torch.zeros(N, K, dtype=self.dtype, device=device))
         else:
             self.register_buffer("qweight", torch.zeros(N, K // 2, dtype=torch.uint8, device=device))
             self.register_buffer("scales", torch.zeros(N, K // group, dtype=torch.float16, device=device))
             if weight_format == "q4_zp":
                 self.register_buffer("zeros", torch.zeros(N, K // group, dtype=torch.float16, device=device))
-        self.register_buffer("bias", torch.zeros(N, dtype=torch.float16, device=device) if bias else None)
+        self.register_buffer("bias", torch.zeros(N, dtype=self.dtype, device=device) if bias else None)
         self._plans = {}
 
     @classmethod
@@ -44,10 +46,10 @@ class StreamKLinear(torch.nn.Module):
         """Takes over the weight (and bias) of a torch.nn.Linear; weight_format='q4' / 'q4_zp' quantises
         it with `quantize_q4` (symmetric around `zero` / asymmetric with a zero point per group) on the
         device it lives on."""
-        w = linear.weight.detach().to(torch.float16).contiguous()
+        w = linear.weight.detach().to(torch.bfloat16 if weight_format == "bfloat16" else torch.float16).contiguous()
         m = cls(linear.in_features, linear.out_features, linear.bias is not None, weight_format=weight_format,
                 group=group, zero=zero, activation=activation, device=w.device)
-        if weight_format == "float16":
+        if weight_format in ("float16", "bfloat16"):
             m.weight.copy_(w)
         elif weight_format == "q4_zp":
             q, s, z = ops.quantize_q4(w, group=group, asymmetric=True)
@@ -59,7 +61,7 @@ class StreamKLinear(torch.nn.Module):
             m.qweight.copy_(q)
             m.scales.copy_(s)
         if linear.bias is not None:
-            m.bias.copy_(linear.bias.detach().to(torch.float16))
+            m.bias.copy_(linear.bias.detach().to(m.dtype))
         return m
 
     def plan_for(self, M):
@@ -71,8 +73,8 @@ class StreamKLinear(torch.nn.Module):
 
     @torch.no_grad()
     def forward(self, x):
-        if x.dtype != torch.float16 or x.shape[-1] != self.in_features:
-            raise ValueError(f"input must be fp16 [..., {self.in_features}], got {x.dtype} {tuple(x.shape)}")
+        if x.dtype != self.dtype or x.shape[-1] != self.in_features:
+            raise ValueError(f"input must be {self.dtype} [..., {self.in_features}], got {x.dtype} {tuple(x.shape)}")
         lead = x.shape[:-1]
         a = x.reshape(-1, self.in_features)
         if a.stride(-1) != 1 or (a.shape[0] > 1 and a.stride(0) % 8) or a.data_ptr() % 16:
@@ -80,9 +82,11 @@ class StreamKLinear(torch.nn.Module):
         M = a.shape[0]
         if M == 0:
             return x.new_zeros(*lead, self.out_features)
-        # bias and activation are applied in the GEMM's epilogue (fp32, before the rounding to fp16)
+        # bias and activation are applied in the GEMM's epilogue (fp32, before the rounding to C's type)
         if self.weight_format == "float16":
             c = ops.streamk_fp16(a, self.weight, plan=self.plan_for(M), bias=self.bias, activation=self.activation)
+        elif self.weight_format == "bfloat16":
+            c = ops.streamk_bf16(a, self.weight, plan=self.plan_for(M), bias=self.bias, activation=self.activation)
         else:
             # (more rows than one Q4 launch takes: streamk_q4 splits the call itself)
             c = ops.streamk_q4(a, self.qweight, self.scales, plan=self.plan_for(M) if M <= ops.Q4_MAX_M else None,

@@ -869,6 +869,17 @@ def test_fused_activation_epilogue(sk, oracle):
         m = sk.StreamKLinear.from_linear(lin, activation=act)
         want = fn(x.float() @ lin.weight.float().T + lin.bias.float())
         assert _rel(oracle, m(x).reshape(21, 1000), want.detach().reshape(21, 1000).cpu().numpy()) <= 1e-3, act
+    # the same layer in bfloat16 (weights, activations, bias and output), from one row to a prefill-sized batch
+    linb = torch.nn.Linear(1024, 1000, bias=True).bfloat16().cuda()
+    m = sk.StreamKLinear.from_linear(linb, weight_format="bfloat16", activation="silu")
+    for rows in ((1,), (3, 7), (300,)):
+        xb = (torch.randn(*rows, 1024, device="cuda") * 0.5).bfloat16()
+        want = torch.nn.functional.silu(xb.float() @ linb.weight.float().T + linb.bias.float()).detach()
+        got = m(xb)
+        assert got.dtype == torch.bfloat16 and tuple(got.shape) == rows + (1000,)
+        assert _rel(oracle, got.reshape(-1, 1000), want.reshape(-1, 1000).cpu().numpy()) <= 6e-3, rows
+    with pytest.raises(ValueError):
+        m(x)  # an fp16 input to the bfloat16 layer
     X, Y = torch.zeros(8, 64, dtype=torch.float16, device="cuda"), torch.zeros(24, 64, dtype=torch.float16, device="cuda")
     with pytest.raises(ValueError):
         sk.streamk_fp16(X, Y, activation="tanh")
