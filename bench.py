@@ -351,7 +351,16 @@ def main():
         extra["gemv_f16_M1_N28672_K8192"] = {"kernel": streamk.kernel_name(pv.kernel_id), "bytes": vbytes, "us": round(ms * 1e3, 1),
                                             "gbs": round(vbytes / ms / 1e6, 1), "frac_hbm": round(vbytes / ms / 1e6 / PEAK_HBM_GBS, 4),
                                             "torch_matmul_us": round(ms_t * 1e3, 1)}
-        del wv
+        # the same product in bfloat16 (the twin kernel with the bfloat16 MFMA)
+        wb, ab = wv.bfloat16(), av.bfloat16()
+        cb = torch.empty(1, nv, dtype=torch.bfloat16, device="cuda")
+        pb = streamk.make_plan(1, nv, kv, "bfloat16", "nt")
+        ms = time_graph(lambda: streamk.streamk_bf16(ab, wb, out=cb, plan=pb), launches=5, replays=5)
+        ms_t = time_graph(lambda: torch.matmul(ab, wb.T, out=cb), launches=5, replays=5)
+        extra["gemv_bf16_M1_N28672_K8192"] = {"kernel": streamk.kernel_name(pb.kernel_id), "bytes": vbytes, "us": round(ms * 1e3, 1),
+                                             "gbs": round(vbytes / ms / 1e6, 1), "frac_hbm": round(vbytes / ms / 1e6 / PEAK_HBM_GBS, 4),
+                                             "torch_matmul_us": round(ms_t * 1e3, 1)}
+        del wv, wb
 
         # offline side of the Q4 path on the same weight shape: algorithmic bytes over graph-timed launches
         Wf = (torch.randn(N, K, generator=g) * 0.05).half().cuda()

@@ -18,7 +18,7 @@ sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("shape", help="MxNxK")
-    ap.add_argument("--dtype", default="float16", choices=["float16", "float32", "q4", "float8_e4m3", "int8"])
+    ap.add_argument("--dtype", default="float16", choices=["float16", "bfloat16", "float32", "q4", "float8_e4m3", "int8"])
     ap.add_argument("--layout", default="nt", choices=["nt", "nn"])
     ap.add_argument("--config", default="{}", help="python dict of plan options, e.g. \"dict(bm=256,bn=256,raster=8)\"")
     ap.add_argument("--reps", type=int, default=5)
@@ -58,7 +58,7 @@ def main():
         C = torch.empty(M, N, dtype=torch.float16, device="cuda")
         run = lambda: streamk.streamk_fp8(A, B, out=C, plan=plan)  # noqa: E731
     else:
-        dt = torch.float16 if args.dtype == "float16" else torch.float32
+        dt = {"float16": torch.float16, "bfloat16": torch.bfloat16}.get(args.dtype, torch.float32)
         bshape = (N, K) if args.layout == "nt" else (K, N)
         if args.data == "rand":
             A = (torch.rand(M, K, generator=g) * 2 - 1).to(dt).cuda()
@@ -67,7 +67,7 @@ def main():
             fill = torch.zeros if args.data == "zeros" else torch.ones
             A, B = fill(M, K, dtype=dt, device="cuda"), fill(*bshape, dtype=dt, device="cuda")
         C = torch.empty(M, N, dtype=dt, device="cuda")
-        fn = streamk.streamk_fp16 if args.dtype == "float16" else streamk.streamk_fp32
+        fn = {"float16": streamk.streamk_fp16, "bfloat16": streamk.streamk_bf16}.get(args.dtype, streamk.streamk_fp32)
         run = lambda: fn(A, B, layout=args.layout, out=C, plan=plan)  # noqa: E731
     for _ in range(args.reps):
         run()
