@@ -66,7 +66,7 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
             out.append(dict(bm=bm, bn=bn, bk=bk, schedule="dp"))
             for grid, fixup in itertools.product((cus, 2 * cus, 4 * cus), ("reduce", "atomic")):
                 out.append(dict(bm=bm, bn=bn, bk=bk, schedule="sk2", grid=grid, fixup=fixup))
-    if dtype == "float16" and M > 16:
+    if dtype in ("float16", "bfloat16") and M > 16:
         for (bm, bn, bk) in _TILES_F16:
             # (variant, bk): direct-to-LDS two-stage, register-staged, direct-to-LDS four-stage, 16x16x32 form
             variants = ((2, bk), (1, bk), (4, 32)) if bm * bn > 64 * 128 else ((2, bk), (4, 32))
@@ -195,9 +195,12 @@ def autotune(M, N, K, dtype="float16", layout="nt", *, configs=None, warmup=5, r
             ref_ms = None
     else:
         bshape = (N, K) if layout == "nt" else (K, N)
-        B = (torch.rand(*bshape, generator=g) * 2 - 1).half().to(dev)
+        # (bfloat16: the twins of the fp16 kernels; candidates whose kernel has no twin are skipped below)
+        tdt, gemm = (torch.bfloat16, ops.streamk_bf16) if dtype == "bfloat16" else (torch.float16, ops.streamk_fp16)
+        A, C = A.to(tdt), C.to(tdt)
+        B = (torch.rand(*bshape, generator=g) * 2 - 1).to(tdt).to(dev)
         Bs = [B] + [B.clone() for _ in range(copies - 1)]
-        run = lambda p: ops.streamk_fp16(A, rotate(Bs), layout=layout, out=C, plan=p)  # noqa: E731
+        run = lambda p: gemm(A, rotate(Bs), layout=layout, out=C, plan=p)  # noqa: E731
         small = 2.0 * M * N * K < 5e11
         as_b = (lambda b: b.T) if layout == "nt" else (lambda b: b)
         ref_ms = _time_ms(lambda: torch.matmul(A, as_b(rotate(Bs)), out=C), warmup, rep, small)

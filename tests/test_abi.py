@@ -4,6 +4,7 @@ error codes (no compute entry point is launched here)."""
 import ctypes
 import os
 import re
+import sys
 
 import pytest
 
@@ -177,3 +178,27 @@ def test_product_does_not_touch_the_oracle():
             if f.endswith((".py", ".h", ".hip", ".cpp", "Makefile")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text.lower(), os.path.join(dirpath, f)
+
+
+def test_autotune_candidates_make_plans():
+    """The tuner's search space on the host: for every dtype and a decode-, a batch- and a prefill-sized M the
+    candidates are distinct, and each either makes a plan for the shape or is refused as a configuration (-4) --
+    never another error; at least one per list is valid."""
+    import streamk
+    from streamk._lib import StreamKError
+    at = sys.modules["streamk.autotune"]
+    for dtype in ("float16", "bfloat16", "q4", "q4_zp", "float8_e4m3", "float8_e5m2", "int8"):
+        for M in (1, 16, 64, 512, 4096):
+            if dtype in ("q4", "q4_zp") and M > 64:
+                continue
+            cands = at.candidate_configs(M, 4096, 4096, dtype, cus=256)
+            assert cands and len({tuple(sorted(c.items())) for c in cands}) == len(cands), (dtype, M)
+            valid = 0
+            for c in cands:
+                try:
+                    p = streamk.make_plan(M, 4096, 4096, dtype, "nt", c, cus=256)
+                    assert p.total_tiles > 0 and p.grid > 0
+                    valid += 1
+                except StreamKError as e:
+                    assert e.status == -4, (dtype, M, c, e.status)
+            assert valid > 0, (dtype, M)

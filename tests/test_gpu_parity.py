@@ -565,9 +565,9 @@ def test_bf16_small_m_kernels(sk, oracle):
         ref = oracle.matmul_fp32(A.float().numpy(), W.float().numpy(), trans_b=True)
         assert _rel(oracle, sk.streamk_bf16(A.cuda(), W.cuda()), ref) <= 4e-3, M
     # a shape tuned for fp16 only: the bfloat16 plan takes that entry (its kernel has a bfloat16 twin)
-    if sk.tuned_config(16, 8192, 8192, "bfloat16") is None and sk.tuned_config(16, 8192, 8192, "float16"):
-        want = sk.make_plan(16, 8192, 8192, "float16")
-        got = sk.make_plan(16, 8192, 8192, "bfloat16")
+    if sk.tuned_config(256, 4096, 4096, "bfloat16") is None and sk.tuned_config(256, 4096, 4096, "float16"):
+        want = sk.make_plan(256, 4096, 4096, "float16")
+        got = sk.make_plan(256, 4096, 4096, "bfloat16")
         assert (got.bm, got.bn, got.bk, got.grid, got.schedule) == (want.bm, want.bn, want.bk, want.grid, want.schedule)
     sk.workspace_status()
 
@@ -1212,3 +1212,35 @@ def test_bad_calls_are_refused(sk):
         sk.streamk_fp16(A, torch.zeros(64, 136, dtype=torch.float16, device="cuda"))
     with pytest.raises(sk.StreamKError):
         sk.streamk_fp16(A[:, :100], A[:, :100])  # K = 100 is not a multiple of 8
+
+
+def test_autotune_search_and_cache(sk, oracle, tmp_path):
+    """The per-shape search (autotune/streamk_fp16_autotune.py:376-386 in the reference): every dtype it covers on a
+    small problem with a short candidate list -- the winner is one of the candidates, candidates agree with each
+    other (the tuner checks them), an impossible candidate is skipped, and the result lands in the cache file under
+    the key plans are looked up by."""
+    import json
+    import sys
+    at = sys.modules["streamk.autotune"]
+    cache = str(tmp_path / "tuned.json")
+    cases = [
+        ("float16", 200, 512, 1024, [dict(bm=128, bn=128, bk=64, schedule="dp"), dict(bm=64, bn=64, bk=32, schedule="sk2", fixup="reduce"),
+                                     dict(bm=48, bn=48, bk=64, schedule="dp")]),
+        ("bfloat16", 200, 512, 1024, [dict(bm=128, bn=128, bk=64, schedule="dp"), dict(bm=64, bn=64, bk=32, schedule="basic", fixup="atomic")]),
+        ("bfloat16", 8, 512, 1024, None),
+        ("float16", 1, 512, 1024, None),
+        ("q4", 4, 512, 1024, None),
+        ("float8_e4m3", 200, 512, 1024, [dict(bm=128, bn=128, schedule="dp"), dict(bm=128, bn=128, schedule="sk2", fixup="reduce")]),
+        ("int8", 200, 512, 1024, [dict(bm=128, bn=128, schedule="dp"), dict(bm=256, bn=128, schedule="basic", fixup="atomic")]),
+    ]
+    for dtype, M, N, K, configs in cases:
+        ms, cfg, ref = at.autotune(M, N, K, dtype, "nt", configs=configs, warmup=2, rep=5, cache_path=cache)
+        assert ms > 0 and cfg in (configs if configs is not None else at.candidate_configs(M, N, K, dtype)), (dtype, cfg)
+        assert cfg.get("bm") != 48
+        hit = json.load(open(cache))[f"gfx950/{dtype}/nt/{M}x{N}x{K}"]
+        assert hit["config"] == cfg and hit["latency_ms"] == ms
+        plan = sk.make_plan(M, N, K, dtype, "nt", cfg)   # the recorded configuration makes a plan again
+        assert plan.bm == cfg["bm"] and plan.bn == cfg["bn"]
+    with pytest.raises(RuntimeError):
+        at.autotune(200, 512, 1024, "float16", "nt", configs=[dict(bm=48, bn=48, bk=64)], cache=False)
+    sk.workspace_status()
