@@ -113,9 +113,9 @@ int make_dev_plan(const sk_plan *plan, const KernelInfo *k, void *ws, size_t ws_
 }
 
 int cached_occupancy(int id, bool skinny) {
-  static int cache[256];
-  static bool have[256];
-  int slot = id & 255;
+  static int cache[512];
+  static bool have[512];
+  int slot = id & 511;  // kernel ids stay below 512
   if (!have[slot]) {
     cache[slot] = skinny ? occupancy_skinny(id) : occupancy_tile(id);
     have[slot] = true;
@@ -267,12 +267,18 @@ static int gemm_8bit(int dtype, const void *A, const void *B, void *C, int64_t M
       (reinterpret_cast<uintptr_t>(C) & (dtype == SK_I8 ? 3 : 1)))
     return SK_ERR_ALIGN;
   const KernelInfo *k = kernel_by_id(plan->kernel_id);
-  if (!k || k->dtype != dtype || k->family != FAMILY_TILE) return SK_ERR_CONFIG;
+  if (!k || k->dtype != dtype) return SK_ERR_CONFIG;
   if (lda * k->bm >= (int64_t)1 << 31 || ldb * k->bn >= (int64_t)1 << 31) return SK_ERR_SHAPE;
   DevPlan dp;
   Workspace w;
-  rc = make_dev_plan(plan, k, ws, ws_bytes, cached_occupancy(k->id, false), (hipStream_t)stream, &dp, &w);
+  const bool skinny = k->family == FAMILY_SKINNY;
+  rc = make_dev_plan(plan, k, ws, ws_bytes, cached_occupancy(k->id, skinny), (hipStream_t)stream, &dp, &w);
   if (rc) return rc;
+  if (skinny) {  // small-M fp8 kernels: bytes travel as pairs, alpha in the `zero` field
+    SkinnyArgs a{(const half_t *)A, B, nullptr, (half_t *)C, (int)M, (int)N, (int)(K / 2), lda / 2, ldb / 2, ldc,
+                 __builtin_bit_cast(int, alpha), 0, nullptr};
+    return launch_skinny(k->id, a, dp, w, (hipStream_t)stream, bias) == 0 ? SK_OK : SK_ERR_LAUNCH;
+  }
   GemmArgs a{(const half_t *)A, (const half_t *)B, (half_t *)C, (int)M, (int)N, (int)(K / 2), lda / 2, ldb / 2, ldc, alpha};
   return launch_tile_f16(k->id, a, dp, w, (hipStream_t)stream, bias) == 0 ? SK_OK : SK_ERR_LAUNCH;
 }

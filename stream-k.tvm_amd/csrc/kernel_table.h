@@ -184,6 +184,18 @@ struct KernelInfo {
   X(166, 1, 1, 4, 4, 32768)    \
   X(167, 2, 1, 4, 2, 32768)
 
+// fp8 small-M kernels (dtypes SK_F8E4M3 and SK_F8E5M2, one instance each; the second id is the first + 10);
+// bk counts fp8 elements:  X(id, MB, NB, WN, RK, DEPTH, ROW1)
+#define SK_SKINNY_F8_KERNELS(X) \
+  X(250, 1, 1, 4, 1, 2, 0)      \
+  X(251, 2, 1, 4, 1, 2, 0)      \
+  X(252, 1, 1, 1, 4, 2, 0)      \
+  X(253, 1, 1, 2, 2, 2, 0)      \
+  X(254, 1, 1, 2, 4, 2, 0)      \
+  X(255, 1, 1, 4, 2, 2, 0)      \
+  X(256, 2, 1, 4, 2, 2, 0)      \
+  X(257, 1, 1, 4, 1, 4, 1)
+
 // bfloat16 twins of the fp16 matrix-vector kernels (dtype SK_BF16, variant 2)
 #define SK_GEMV_BF16_KERNELS(X) \
   X(241, 1, 1, 4, 4, 8192)      \

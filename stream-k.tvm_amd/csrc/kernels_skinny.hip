@@ -40,6 +40,8 @@ static int launch_policy(const SkinnyArgs &a, const DevPlan &p, const Workspace 
 #define SK_POLICY(MB, NB, WN, RK, Q4, DEPTH, ROW1) TileSkinny<MB, NB, WN, RK, (Q4) != 0, DEPTH, (ROW1) != 0>
 #define SK_POLICY_BF16(MB, NB, WN, RK, DEPTH, ROW1) \
   TileSkinny<MB, NB, WN, RK, false, DEPTH, (ROW1) != 0, false, false, true>
+#define SK_POLICY_F8(MB, NB, WN, RK, DEPTH, ROW1, FMT) \
+  TileSkinny<MB, NB, WN, RK, false, DEPTH, (ROW1) != 0, false, false, false, FMT>
 
 int skinny_kernel_infos(KernelInfo *out, int max) {
   int n = 0;
@@ -62,6 +64,18 @@ int skinny_kernel_infos(KernelInfo *out, int max) {
                           "skinny_bf16_mb" #MB "_wn" #WN "_rk" #RK "_row1_" #ROW1};                      \
   }
   SK_SKINNY_BF16_KERNELS(X)
+#undef X
+#define X(id, MB, NB, WN, RK, DEPTH, ROW1)                                                                \
+  if (n + 1 < max) {                                                                                  \
+    typedef SK_POLICY_F8(MB, NB, WN, RK, DEPTH, ROW1, 1) P;                                             \
+    out[n++] = KernelInfo{id, FAMILY_SKINNY, 5, 0, (ROW1) ? 1 : 0, P::BM, P::BN, 2 * P::BKC, P::NT,     \
+                          P::LDS_BYTES, P::CTAS_PER_CU, P::TILE_ELEMS, 0, P::MAX_M, 16,               \
+                          "skinny_f8e4m3_mb" #MB "_wn" #WN "_rk" #RK "_row1_" #ROW1};                    \
+    out[n++] = KernelInfo{id + 10, FAMILY_SKINNY, 8, 0, (ROW1) ? 1 : 0, P::BM, P::BN, 2 * P::BKC, P::NT, \
+                          P::LDS_BYTES, P::CTAS_PER_CU, P::TILE_ELEMS, 0, P::MAX_M, 16,               \
+                          "skinny_f8e5m2_mb" #MB "_wn" #WN "_rk" #RK "_row1_" #ROW1};                    \
+  }
+  SK_SKINNY_F8_KERNELS(X)
 #undef X
 #define X(id, NB, WN, RK, DEPTH, KMAX)                                                                        \
   if (n < max) {                                                                                         \
@@ -136,6 +150,17 @@ int launch_skinny(int id, const SkinnyArgs &a, const DevPlan &p, const Workspace
   }
     SK_SKINNY_BF16_KERNELS(X)
 #undef X
+#define X(id_, MB, NB, WN, RK, DEPTH, ROW1)                                                 \
+  case id_: {                                                                              \
+    typedef SK_POLICY_F8(MB, NB, WN, RK, DEPTH, ROW1, 1) P;                                  \
+    return launch_policy<P>(a, p, ws, s, bias);                                            \
+  }                                                                                        \
+  case id_ + 10: {                                                                         \
+    typedef SK_POLICY_F8(MB, NB, WN, RK, DEPTH, ROW1, 2) P;                                  \
+    return launch_policy<P>(a, p, ws, s, bias);                                            \
+  }
+    SK_SKINNY_F8_KERNELS(X)
+#undef X
 #define X(id_, NB, WN, RK, DEPTH, KMAX)                                                        \
   case id_: {                                                                              \
     typedef TileGemvQ4<NB, WN, RK, DEPTH, KMAX> P;                                          \
@@ -202,6 +227,16 @@ int occupancy_skinny(int id) {
     return occ;                                                                                       \
   }
     SK_SKINNY_BF16_KERNELS(X)
+#undef X
+#define X(id_, MB, NB, WN, RK, DEPTH, ROW1)                                                              \
+  case id_:                                                                                           \
+  case id_ + 10: {  /* the two formats differ in one instruction: one occupancy */                    \
+    typedef SK_POLICY_F8(MB, NB, WN, RK, DEPTH, ROW1, 1) P;                                               \
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_skinny_kernel<P>, P::NT, 0) != hipSuccess) \
+      return -1;                                                                                      \
+    return occ;                                                                                       \
+  }
+    SK_SKINNY_F8_KERNELS(X)
 #undef X
 #define X(id_, NB, WN, RK, DEPTH, KMAX)                                                                      \
   case id_: {                                                                                            \

@@ -27,7 +27,7 @@ struct SkinnyArgs {
   half_t *C;
   int M, N, K;
   int64_t lda, ldw, ldc;  // ldw in elements (fp16) or bytes (Q4)
-  int zero;
+  int zero;               // Q4: the scalar zero point; fp8: the bits of the fp32 scalar alpha
   int groups;             // Q4: scales per row
   const half_t *zeros;    // Q4 with per-group zero points: [N, K/group], integer values 0..15 (else unused)
 };
@@ -104,9 +104,16 @@ __device__ __forceinline__ void stage_scales(half_t *ldsS, const half_t *scales_
 // BF16_ (not Q4): operands, bias and C are bfloat16 -- the same 16-bit data movement, the bfloat16 form of the
 // MFMA, C rounded to nearest even.
 template <int MB_, int NB_, int WN_, int RK_, bool Q4_, int DEPTH_, bool ROW1_ = false, bool TILED_ = false,
-          bool ZP_ = false, bool BF16_ = false>
+          bool ZP_ = false, bool BF16_ = false, int F8_ = 0>
 struct TileSkinny {
   static_assert(!BF16_ || !Q4_, "the Q4 decode produces fp16");
+  // F8_ (1: OCP e4m3, 2: OCP e5m2; not Q4, not BF16): A and the weights hold fp8 bytes and travel as pairs -- the
+  // launcher passes K, lda and ldw halved, and all data movement is the 16-bit kernel's.  A lane's 16 bytes are 16
+  // K-values, fed to two v_mfma_f32_16x16x32 fp8 instructions (8 bytes per lane each); A and the weights are cut up
+  // the same way, so which K-values a lane holds does not matter.  C is fp16; a.zero carries the bits of the
+  // scalar that multiplies the fp32 sums before the epilogue.
+  static_assert(F8_ == 0 || (!Q4_ && !BF16_), "fp8 operands exclude the Q4 decode and bfloat16");
+  static constexpr int F8 = F8_;
   static_assert(!TILED_ || Q4_, "tiled weights exist for Q4");
   static_assert(!ZP_ || Q4_, "zero points exist for Q4");
   typedef SkinnyArgs Args;
@@ -318,7 +325,17 @@ struct TileSkinny {
             }
 #pragma unroll
             for (int i = 0; i < MB; ++i)
-              if constexpr (BF16_) {
+              if constexpr (F8 != 0) {
+                typedef long longx2 __attribute__((ext_vector_type(2)));
+                const longx2 w2 = __builtin_bit_cast(longx2, fw), a2 = __builtin_bit_cast(longx2, fa[i]);
+                if constexpr (F8 == 1) {
+                  acc.c[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w2[0], a2[0], acc.c[i][j], 0, 0, 0);
+                  acc.c[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w2[1], a2[1], acc.c[i][j], 0, 0, 0);
+                } else {
+                  acc.c[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf8_bf8(w2[0], a2[0], acc.c[i][j], 0, 0, 0);
+                  acc.c[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf8_bf8(w2[1], a2[1], acc.c[i][j], 0, 0, 0);
+                }
+              } else if constexpr (BF16_) {
                 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
                 acc.c[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, fw),
                                                                       __builtin_bit_cast(bf16x8, fa[i]), acc.c[i][j], 0, 0, 0);
@@ -390,6 +407,7 @@ struct TileSkinny {
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             float x = acc.c[i][j][e];
+            if constexpr (F8 != 0) x *= __builtin_bit_cast(float, a.zero);
             if constexpr (BIAS) x = activate(x + bias_at<BF16_>(bias, col + e, a.N), act);
             if constexpr (BF16_) {
               const __bf16 b = (__bf16)x;

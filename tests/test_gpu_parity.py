@@ -640,6 +640,54 @@ def test_fp8_tile_kernels(sk, oracle):
     sk.workspace_status()
 
 
+def test_fp8_small_m_kernels(sk, oracle):
+    """Weight-streaming fp8 kernels (M <= 32; e4m3 and e5m2): every instance, ragged N, a K tail (K a multiple of 16
+    only), data-parallel and Stream-K with both fix-ups, against the float64 host product of the decoded bytes
+    (1e-3: fp16 rounding of C); {-1,0,1} data must come out exact -- a lane's 16 bytes are split over two MFMAs, so
+    any mispairing of A and weight bytes along K would show; alpha, bias and activation in the epilogue; the plans
+    the library picks for 1..32 rows are these kernels."""
+    import torch
+    torch.manual_seed(23)
+    cfgs = [dict(bm=16, bn=64, bk=256), dict(bm=32, bn=64, bk=256), dict(bm=16, bn=16, bk=1024), dict(bm=16, bn=32, bk=512),
+            dict(bm=16, bn=32, bk=1024), dict(bm=16, bn=64, bk=512), dict(bm=32, bn=64, bk=512), dict(bm=16, bn=64, bk=256, variant=2)]
+    N, K = 1000, 2064
+    bias = torch.randint(-20, 20, (N,)).half()
+    for fmt, dt in (("e4m3", torch.float8_e4m3fn), ("e5m2", torch.float8_e5m2)):
+        first, last = (250, 257) if fmt == "e4m3" else (260, 267)
+        B = torch.randn(N, K).to(dt)
+        Bi = torch.randint(-1, 2, (N, K)).float().to(dt)
+        for cfg in cfgs:
+            for M in ((1,) if cfg.get("variant") == 2 else (cfg["bm"], cfg["bm"] - 3, 1)):
+                A = torch.randn(M, K).to(dt)
+                Ai = torch.randint(-1, 2, (M, K)).float().to(dt)
+                ref = oracle.f8_gemm_ref(A.view(torch.uint8).numpy(), B.view(torch.uint8).numpy(), fmt)
+                exact = oracle.f8_gemm_ref(Ai.view(torch.uint8).numpy(), Bi.view(torch.uint8).numpy(), fmt)
+                assert np.abs(exact).max() <= 2048
+                for sch in (dict(schedule="dp"), dict(schedule="sk2", fixup="reduce", grid=24), dict(schedule="sk2", fixup="atomic", grid=20)):
+                    plan = sk.make_plan(M, N, K, "float8_" + fmt, "nt", dict(cfg, **sch))
+                    assert first <= plan.kernel_id <= last and plan.iters_per_tile == -(-K // cfg["bk"]), (fmt, cfg, plan.kernel_id)
+                    C = sk.streamk_fp8(A.cuda(), B.cuda(), plan=plan)
+                    assert C.dtype == torch.float16 and _rel(oracle, C, ref) <= 1e-3 <= TOL, (fmt, cfg, M, sch)
+                    Ci = sk.streamk_fp8(Ai.cuda(), Bi.cuda(), plan=plan)
+                    assert np.array_equal(Ci.double().cpu().numpy(), exact), (fmt, cfg, M, sch)
+                    Cb = sk.streamk_fp8(Ai.cuda(), Bi.cuda(), plan=plan, alpha=0.5, bias=bias.cuda(), activation="relu")
+                    assert np.array_equal(Cb.double().cpu().numpy(), np.maximum(0.5 * exact + bias.double().numpy(), 0)), (fmt, cfg, M, sch)
+                    if sch.get("fixup") == "reduce":
+                        assert torch.equal(C, sk.streamk_fp8(A.cuda(), B.cuda(), plan=plan))
+        for M in (1, 7, 16, 32):
+            plan = sk.make_plan(M, 4096, 4096, "float8_" + fmt, "nt")
+            assert first <= plan.kernel_id <= last, (fmt, M, plan.kernel_id)
+            A, W = torch.randn(M, 4096).to(dt), torch.randn(4096, 4096).to(dt)
+            ref = oracle.f8_gemm_ref(A.view(torch.uint8).numpy(), W.view(torch.uint8).numpy(), fmt)
+            assert _rel(oracle, sk.streamk_fp8(A.cuda(), W.cuda()), ref) <= 1e-3, (fmt, M)
+    # strided operands (leading dimensions a multiple of 16 bytes)
+    big = torch.randn(300, 4096).to(torch.float8_e4m3fn).cuda()
+    A, W = big[:9, 16:16 + 2048], big[40:, 1024:1024 + 2048]
+    ref = oracle.f8_gemm_ref(A.cpu().view(torch.uint8).numpy(), W.cpu().view(torch.uint8).numpy())
+    assert _rel(oracle, sk.streamk_fp8(A, W), ref) <= 1e-3
+    sk.workspace_status()
+
+
 def test_fp8_e5m2_tile_kernels(sk, oracle):
     """The e5m2 instances of the fp8 kernels: same checks as for e4m3 on fewer shapes (the two differ in one
     immediate operand of the MFMA): host product of the decoded bytes within 1e-3, {-1,0,1} data exact, every
