@@ -274,7 +274,7 @@ static int gemm_8bit(int dtype, const void *A, const void *B, void *C, int64_t M
   const bool skinny = k->family == FAMILY_SKINNY;
   rc = make_dev_plan(plan, k, ws, ws_bytes, cached_occupancy(k->id, skinny), (hipStream_t)stream, &dp, &w);
   if (rc) return rc;
-  if (skinny) {  // small-M fp8 kernels: bytes travel as pairs, alpha in the `zero` field
+  if (skinny) {  // small-M fp8 / int8 kernels: bytes travel as pairs, alpha in the `zero` field (int8: C is int32)
     SkinnyArgs a{(const half_t *)A, B, nullptr, (half_t *)C, (int)M, (int)N, (int)(K / 2), lda / 2, ldb / 2, ldc,
                  __builtin_bit_cast(int, alpha), 0, nullptr};
     return launch_skinny(k->id, a, dp, w, (hipStream_t)stream, bias) == 0 ? SK_OK : SK_ERR_LAUNCH;

@@ -196,6 +196,17 @@ struct KernelInfo {
   X(256, 2, 1, 4, 2, 2, 0)      \
   X(257, 1, 1, 4, 1, 4, 1)
 
+// int8 small-M kernels (dtype SK_I8, int32 C); bk counts int8 elements:  X(id, MB, NB, WN, RK, DEPTH, ROW1)
+#define SK_SKINNY_I8_KERNELS(X) \
+  X(270, 1, 1, 4, 1, 2, 0)      \
+  X(271, 2, 1, 4, 1, 2, 0)      \
+  X(272, 1, 1, 1, 4, 2, 0)      \
+  X(273, 1, 1, 2, 2, 2, 0)      \
+  X(274, 1, 1, 2, 4, 2, 0)      \
+  X(275, 1, 1, 4, 2, 2, 0)      \
+  X(276, 2, 1, 4, 2, 2, 0)      \
+  X(277, 1, 1, 4, 1, 4, 1)
+
 // bfloat16 twins of the fp16 matrix-vector kernels (dtype SK_BF16, variant 2)
 #define SK_GEMV_BF16_KERNELS(X) \
   X(241, 1, 1, 4, 4, 8192)      \

@@ -77,6 +77,15 @@ int skinny_kernel_infos(KernelInfo *out, int max) {
   }
   SK_SKINNY_F8_KERNELS(X)
 #undef X
+#define X(id, MB, NB, WN, RK, DEPTH, ROW1)                                                                \
+  if (n < max) {                                                                                      \
+    typedef SK_POLICY_F8(MB, NB, WN, RK, DEPTH, ROW1, 3) P;                                             \
+    out[n++] = KernelInfo{id, FAMILY_SKINNY, 6, 0, (ROW1) ? 1 : 0, P::BM, P::BN, 2 * P::BKC, P::NT,     \
+                          P::LDS_BYTES, P::CTAS_PER_CU, P::TILE_ELEMS, 0, P::MAX_M, 16,               \
+                          "skinny_i8_mb" #MB "_wn" #WN "_rk" #RK "_row1_" #ROW1};                        \
+  }
+  SK_SKINNY_I8_KERNELS(X)
+#undef X
 #define X(id, NB, WN, RK, DEPTH, KMAX)                                                                        \
   if (n < max) {                                                                                         \
     typedef TileGemvQ4<NB, WN, RK, DEPTH, KMAX> P;                                                        \
@@ -161,6 +170,13 @@ int launch_skinny(int id, const SkinnyArgs &a, const DevPlan &p, const Workspace
   }
     SK_SKINNY_F8_KERNELS(X)
 #undef X
+#define X(id_, MB, NB, WN, RK, DEPTH, ROW1)                                                 \
+  case id_: {                                                                              \
+    typedef SK_POLICY_F8(MB, NB, WN, RK, DEPTH, ROW1, 3) P;                                  \
+    return launch_policy<P>(a, p, ws, s, nullptr);                                         \
+  }
+    SK_SKINNY_I8_KERNELS(X)
+#undef X
 #define X(id_, NB, WN, RK, DEPTH, KMAX)                                                        \
   case id_: {                                                                              \
     typedef TileGemvQ4<NB, WN, RK, DEPTH, KMAX> P;                                          \
@@ -237,6 +253,15 @@ int occupancy_skinny(int id) {
     return occ;                                                                                       \
   }
     SK_SKINNY_F8_KERNELS(X)
+#undef X
+#define X(id_, MB, NB, WN, RK, DEPTH, ROW1)                                                              \
+  case id_: {                                                                                         \
+    typedef SK_POLICY_F8(MB, NB, WN, RK, DEPTH, ROW1, 3) P;                                               \
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_skinny_kernel<P>, P::NT, 0) != hipSuccess) \
+      return -1;                                                                                      \
+    return occ;                                                                                       \
+  }
+    SK_SKINNY_I8_KERNELS(X)
 #undef X
 #define X(id_, NB, WN, RK, DEPTH, KMAX)                                                                      \
   case id_: {                                                                                            \

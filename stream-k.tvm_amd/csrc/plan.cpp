@@ -11,7 +11,7 @@
 
 namespace sk {
 
-static KernelInfo g_table[288];
+static KernelInfo g_table[320];
 static int g_count = -1;
 
 int tile_kernel_infos(KernelInfo *out, int max);
@@ -20,9 +20,9 @@ int f32_kernel_infos(KernelInfo *out, int max);
 
 const KernelInfo *kernel_table(int *count) {
   if (g_count < 0) {
-    int n = tile_kernel_infos(g_table, 288);
-    n += skinny_kernel_infos(g_table + n, 288 - n);
-    n += f32_kernel_infos(g_table + n, 288 - n);
+    int n = tile_kernel_infos(g_table, 320);
+    n += skinny_kernel_infos(g_table + n, 320 - n);
+    n += f32_kernel_infos(g_table + n, 320 - n);
     g_count = n;
   }
   if (count) *count = g_count;

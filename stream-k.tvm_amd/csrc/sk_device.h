@@ -118,6 +118,26 @@ __device__ __forceinline__ floatx4 ld_coherent(const float *p) {
   c.u[1] = __hip_atomic_load(reinterpret_cast<const uint64_t *>(p) + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   return c.f;
 }
+// the same for int32 accumulators (kept in integer registers from the MFMA to memory)
+typedef int intx4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void st_coherent(int *p, intx4_t v) {
+  union { intx4_t i; uint64_t u[2]; } c;
+  c.i = v;
+  __hip_atomic_store(reinterpret_cast<uint64_t *>(p), c.u[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(reinterpret_cast<uint64_t *>(p) + 1, c.u[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ intx4_t ld_coherent(const int *p) {
+  union { intx4_t i; uint64_t u[2]; } c;
+  c.u[0] = __hip_atomic_load(reinterpret_cast<const uint64_t *>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  c.u[1] = __hip_atomic_load(reinterpret_cast<const uint64_t *>(p) + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return c.i;
+}
+__device__ __forceinline__ void st_coherent(int *p, int v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ int ld_coherent_scalar(const int *p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 __device__ __forceinline__ void st_coherent(float *p, float v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }

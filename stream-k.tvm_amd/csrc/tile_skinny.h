@@ -15,6 +15,7 @@
 // K offsets.  For Q4, A is written to LDS in the element order the nibble decode produces
 // (0,4,1,5,2,6,3,7).
 #pragma once
+#include <type_traits>
 #include "q4_dequant.h"
 #include "sk_device.h"
 
@@ -112,8 +113,14 @@ struct TileSkinny {
   // K-values, fed to two v_mfma_f32_16x16x32 fp8 instructions (8 bytes per lane each); A and the weights are cut up
   // the same way, so which K-values a lane holds does not matter.  C is fp16; a.zero carries the bits of the
   // scalar that multiplies the fp32 sums before the epilogue.
-  static_assert(F8_ == 0 || (!Q4_ && !BF16_), "fp8 operands exclude the Q4 decode and bfloat16");
-  static constexpr int F8 = F8_;
+  // F8_ == 3: int8 operands the same way, one v_mfma_i32_16x16x64_i8 per 16 bytes; accumulators, the sums of the
+  // K-splitting waves, partials and C are int32 and stay in integer registers throughout; no epilogue operands.
+  static_assert(F8_ == 0 || (!Q4_ && !BF16_), "one-byte operands exclude the Q4 decode and bfloat16");
+  static constexpr bool I8 = F8_ == 3;
+  static constexpr int F8 = I8 ? 0 : F8_;
+  typedef int intx4 __attribute__((ext_vector_type(4)));
+  typedef typename std::conditional<I8, intx4, floatx4>::type AccV;
+  typedef typename std::conditional<I8, int, float>::type AccT;
   static_assert(!TILED_ || Q4_, "tiled weights exist for Q4");
   static_assert(!ZP_ || Q4_, "zero points exist for Q4");
   typedef SkinnyArgs Args;
@@ -156,7 +163,7 @@ struct TileSkinny {
   static constexpr int WAVES_PER_EU = CTAS_PER_CU * (NT / 64) / 4 > 0 ? CTAS_PER_CU * (NT / 64) / 4 : 1;
 
   struct Acc {
-    floatx4 c[MB][NB];
+    AccV c[MB][NB];
   };
 
   static __device__ __forceinline__ void mac(const Args &a, Acc &acc, int pm, int pn, int k0, int n,
@@ -170,7 +177,7 @@ struct TileSkinny {
 #pragma unroll
     for (int i = 0; i < MB; ++i)
 #pragma unroll
-      for (int j = 0; j < NB; ++j) acc.c[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+      for (int j = 0; j < NB; ++j) acc.c[i][j] = AccV{0, 0, 0, 0};
 
     // ---- weights: one row per lane and block; the buffer descriptor covers the tile's rows, so
     // rows past N read as zero ----
@@ -325,7 +332,10 @@ struct TileSkinny {
             }
 #pragma unroll
             for (int i = 0; i < MB; ++i)
-              if constexpr (F8 != 0) {
+              if constexpr (I8) {
+                acc.c[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(intx4, fw), __builtin_bit_cast(intx4, fa[i]),
+                                                                    acc.c[i][j], 0, 0, 0);
+              } else if constexpr (F8 != 0) {
                 typedef long longx2 __attribute__((ext_vector_type(2)));
                 const longx2 w2 = __builtin_bit_cast(longx2, fw), a2 = __builtin_bit_cast(longx2, fa[i]);
                 if constexpr (F8 == 1) {
@@ -354,13 +364,13 @@ struct TileSkinny {
     SK_TRACE(7);
     // ---- sum the RK partial accumulators into the rk == 0 waves ----
     if (RK > 1) {
-      float *red = reinterpret_cast<float *>(smem + LDS_A + LDS_SC);
+      AccT *red = reinterpret_cast<AccT *>(smem + LDS_A + LDS_SC);
       if (rk > 0) {
 #pragma unroll
         for (int i = 0; i < MB; ++i)
 #pragma unroll
           for (int j = 0; j < NB; ++j)
-            *reinterpret_cast<floatx4 *>(red + ((((rk - 1) * WN + wn) * NV4 + i * NB + j) * 64 + lane) * 4) =
+            *reinterpret_cast<AccV *>(red + ((((rk - 1) * WN + wn) * NV4 + i * NB + j) * 64 + lane) * 4) =
                 acc.c[i][j];
       }
       __syncthreads();
@@ -371,7 +381,7 @@ struct TileSkinny {
           for (int i = 0; i < MB; ++i)
 #pragma unroll
             for (int j = 0; j < NB; ++j)
-              acc.c[i][j] += *reinterpret_cast<const floatx4 *>(
+              acc.c[i][j] += *reinterpret_cast<const AccV *>(
                   red + ((((r - 1) * WN + wn) * NV4 + i * NB + j) * 64 + lane) * 4);
       }
       __syncthreads();
@@ -395,6 +405,27 @@ struct TileSkinny {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     if (wave >= WN) return;
     const int lr = lane & 15, lg = lane >> 4;
+    if constexpr (I8) {  // int32 C straight from the accumulators (ldc counts int32 elements)
+      int *C = reinterpret_cast<int *>(a.C);
+      const bool vec_ok = (a.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(a.C) & 15) == 0);
+#pragma unroll
+      for (int i = 0; i < MB; ++i) {
+        const int row = pm * BM + i * 16 + lr;
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+          const int col = pn * BN + (wave * NB + j) * 16 + lg * 4;
+          if (row < a.M && col < a.N) {
+            int *dst = C + (int64_t)row * a.ldc + col;
+            if (vec_ok && col + 4 <= a.N) {
+              *reinterpret_cast<intx4 *>(dst) = acc.c[i][j];
+            } else {
+              for (int e = 0; e < 4 && col + e < a.N; ++e) dst[e] = acc.c[i][j][e];
+            }
+          }
+        }
+      }
+      return;
+    } else {
     const bool vec_ok = (a.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(a.C) & 7) == 0);
 #pragma unroll
     for (int i = 0; i < MB; ++i) {
@@ -425,41 +456,51 @@ struct TileSkinny {
         }
       }
     }
+    }  // !I8
   }
 
   // Partial tiles are a few KB and there can be thousands of CTAs: every access is a coherent
   // (write-through / L2-bypassing) one, so no CTA ever flushes or invalidates a whole L2.
   static constexpr bool COHERENT_PARTIALS = true;
 
-  static __device__ __forceinline__ void store_partial(const Acc &acc, float *dst) {
+  // (int8: the partial buffer holds int32 sums; the fix-up code addresses it as float, 4 bytes either way)
+  static __device__ __forceinline__ void store_partial(const Acc &acc, float *dst_) {
     if (threadIdx.x >= NTP) return;
+    AccT *dst = reinterpret_cast<AccT *>(dst_);
 #pragma unroll
     for (int v = 0; v < NV4; ++v)
       st_coherent(dst + ((size_t)v * NTP + threadIdx.x) * 4, acc.c[v / NB][v % NB]);
   }
-  static __device__ __forceinline__ void add_partial(Acc &acc, const float *src) {
+  static __device__ __forceinline__ void add_partial(Acc &acc, const float *src_) {
     if (threadIdx.x >= NTP) return;
+    const AccT *src = reinterpret_cast<const AccT *>(src_);
 #pragma unroll
     for (int v = 0; v < NV4; ++v)
       acc.c[v / NB][v % NB] += ld_coherent(src + ((size_t)v * NTP + threadIdx.x) * 4);
   }
-  static __device__ __forceinline__ void atomic_partial(const Acc &acc, float *dst) {
+  static __device__ __forceinline__ void atomic_partial(const Acc &acc, float *dst_) {
     if (threadIdx.x >= NTP) return;
-#pragma unroll
-    for (int v = 0; v < NV4; ++v)
-#pragma unroll
-      for (int e = 0; e < 4; ++e)
-        atomic_add_f32(dst + (size_t)(v * 4 + e) * NTP + threadIdx.x, acc.c[v / NB][v % NB][e]);
-  }
-  static __device__ __forceinline__ void take_partial(Acc &acc, float *src) {
-    if (threadIdx.x >= NTP) return;
+    AccT *dst = reinterpret_cast<AccT *>(dst_);
 #pragma unroll
     for (int v = 0; v < NV4; ++v)
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        float *p = src + (size_t)(v * 4 + e) * NTP + threadIdx.x;
+        if constexpr (I8)
+          atomic_add_i32(dst + (size_t)(v * 4 + e) * NTP + threadIdx.x, acc.c[v / NB][v % NB][e]);
+        else
+          atomic_add_f32(dst + (size_t)(v * 4 + e) * NTP + threadIdx.x, acc.c[v / NB][v % NB][e]);
+      }
+  }
+  static __device__ __forceinline__ void take_partial(Acc &acc, float *src_) {
+    if (threadIdx.x >= NTP) return;
+    AccT *src = reinterpret_cast<AccT *>(src_);
+#pragma unroll
+    for (int v = 0; v < NV4; ++v)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        AccT *p = src + (size_t)(v * 4 + e) * NTP + threadIdx.x;
         acc.c[v / NB][v % NB][e] = ld_coherent_scalar(p);
-        st_coherent(p, 0.f);
+        st_coherent(p, (AccT)0);
       }
   }
 };

@@ -57,8 +57,8 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
     schedule, grid and fix-up."""
     cus = cus or _plan.num_cus()
     out = []
-    f8 = dtype in ("float8_e4m3", "float8_e5m2")
-    if dtype in ("q4", "q4_zp") or (M <= 64 and dtype != "int8" and not (f8 and M > 32)):
+    f8 = dtype in ("float8_e4m3", "float8_e5m2", "int8")  # one-byte operands: small-M kernels up to 32 rows
+    if dtype in ("q4", "q4_zp") or (M <= 64 and not (f8 and M > 32)):
         tiles = _SKINNY_Q4 if dtype in ("q4", "q4_zp") else (_SKINNY_F8 if f8 else _SKINNY_F16)
         for (bm, bn, bk) in tiles:
             if bm < M and not (bm == 16 and M <= 16):

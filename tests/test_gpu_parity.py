@@ -688,6 +688,40 @@ def test_fp8_small_m_kernels(sk, oracle):
     sk.workspace_status()
 
 
+def test_int8_small_m_kernels(sk, oracle):
+    """Weight-streaming int8 kernels (M <= 32, int32 C): every instance, ragged N, a K tail, data-parallel and
+    Stream-K with both fix-ups and the K split over waves -- all must equal the host product in int64 exactly, on
+    the full int8 range (-128 included); strided operands; the plans the library picks for 1..32 rows."""
+    import torch
+    g = torch.Generator().manual_seed(29)
+    cfgs = [dict(bm=16, bn=64, bk=256), dict(bm=32, bn=64, bk=256), dict(bm=16, bn=16, bk=1024), dict(bm=16, bn=32, bk=512),
+            dict(bm=16, bn=32, bk=1024), dict(bm=16, bn=64, bk=512), dict(bm=32, bn=64, bk=512), dict(bm=16, bn=64, bk=256, variant=2)]
+    N, K = 1000, 2064
+    B = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int8)
+    for cfg in cfgs:
+        for M in ((1,) if cfg.get("variant") == 2 else (cfg["bm"], cfg["bm"] - 3, 1)):
+            A = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int8)
+            ref = oracle.i8_gemm_ref(A.numpy(), B.numpy())
+            for sch in (dict(schedule="dp"), dict(schedule="sk2", fixup="reduce", grid=24), dict(schedule="sk2", fixup="atomic", grid=20)):
+                plan = sk.make_plan(M, N, K, "int8", "nt", dict(cfg, **sch))
+                assert 270 <= plan.kernel_id <= 277 and plan.iters_per_tile == -(-K // cfg["bk"]), (cfg, plan.kernel_id)
+                C = sk.streamk_int8(A.cuda(), B.cuda(), plan=plan)
+                assert C.dtype == torch.int32 and np.array_equal(C.cpu().numpy(), ref), (cfg, M, sch)
+    for M in (1, 7, 16, 32):
+        plan = sk.make_plan(M, 4096, 4096, "int8", "nt")
+        assert 270 <= plan.kernel_id <= 277, (M, plan.kernel_id)
+        A = torch.randint(-128, 128, (M, 4096), generator=g, dtype=torch.int8)
+        W = torch.randint(-128, 128, (4096, 4096), generator=g, dtype=torch.int8)
+        assert np.array_equal(sk.streamk_int8(A.cuda(), W.cuda()).cpu().numpy(), oracle.i8_gemm_ref(A.numpy(), W.numpy())), M
+    big = torch.randint(-128, 128, (300, 4096), generator=g, dtype=torch.int8).cuda()
+    A, W = big[:9, 16:16 + 2048], big[40:, 1024:1024 + 2048]
+    out = torch.full((9, 264), 7, dtype=torch.int32, device="cuda")   # a strided C: columns beyond N stay untouched
+    sk.streamk_int8(A, W, out=out[:, :260])
+    assert np.array_equal(out[:, :260].cpu().numpy(), oracle.i8_gemm_ref(A.cpu().numpy(), W.cpu().numpy()))
+    assert bool((out[:, 260:] == 7).all())
+    sk.workspace_status()
+
+
 def test_fp8_e5m2_tile_kernels(sk, oracle):
     """The e5m2 instances of the fp8 kernels: same checks as for e4m3 on fewer shapes (the two differ in one
     immediate operand of the MFMA): host product of the decoded bytes within 1e-3, {-1,0,1} data exact, every
