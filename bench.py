@@ -360,7 +360,22 @@ def main():
         extra["gemv_bf16_M1_N28672_K8192"] = {"kernel": streamk.kernel_name(pb.kernel_id), "bytes": vbytes, "us": round(ms * 1e3, 1),
                                              "gbs": round(vbytes / ms / 1e6, 1), "frac_hbm": round(vbytes / ms / 1e6 / PEAK_HBM_GBS, 4),
                                              "torch_matmul_us": round(ms_t * 1e3, 1)}
-        del wv, wb
+        # and with one-byte weights (fp8 e4m3 -> fp16, int8 -> int32): half the bytes of the same matrix
+        w8 = wv.to(torch.float8_e4m3fn)
+        a8 = av.to(torch.float8_e4m3fn)
+        p8 = streamk.make_plan(1, nv, kv, "float8_e4m3", "nt")
+        bytes8 = kv + nv * kv + 2 * nv
+        ms = time_graph(lambda: streamk.streamk_fp8(a8, w8, out=cv, plan=p8), launches=5, replays=5)
+        extra["gemv_fp8_M1_N28672_K8192"] = {"kernel": streamk.kernel_name(p8.kernel_id), "bytes": bytes8, "us": round(ms * 1e3, 1),
+                                            "gbs": round(bytes8 / ms / 1e6, 1), "frac_hbm": round(bytes8 / ms / 1e6 / PEAK_HBM_GBS, 4)}
+        wi, ai = w8.view(torch.int8), a8.view(torch.int8)
+        ci = torch.empty(1, nv, dtype=torch.int32, device="cuda")
+        pi = streamk.make_plan(1, nv, kv, "int8", "nt")
+        bytesi = kv + nv * kv + 4 * nv
+        ms = time_graph(lambda: streamk.streamk_int8(ai, wi, out=ci, plan=pi), launches=5, replays=5)
+        extra["gemv_int8_M1_N28672_K8192"] = {"kernel": streamk.kernel_name(pi.kernel_id), "bytes": bytesi, "us": round(ms * 1e3, 1),
+                                             "gbs": round(bytesi / ms / 1e6, 1), "frac_hbm": round(bytesi / ms / 1e6 / PEAK_HBM_GBS, 4)}
+        del wv, wb, w8, wi
 
         # offline side of the Q4 path on the same weight shape: algorithmic bytes over graph-timed launches
         Wf = (torch.randn(N, K, generator=g) * 0.05).half().cuda()

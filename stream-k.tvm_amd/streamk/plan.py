@@ -70,6 +70,9 @@ def tuned_config(M, N, K, dtype="float16", layout="nt"):
     return cfg
 
 
+_TWIN_OF = {"bfloat16": "float16", "float8_e5m2": "float8_e4m3"}
+
+
 def make_plan(M, N, K, dtype="float16", layout="nt", config=None, cus=None, use_tuned=True, **kw):
     """Partition an M x N x K GEMM.  `cus` overrides the device's CU count (lets the partitioner
     run without a GPU).  With no configuration given, a tuned one from the autotune cache is used
@@ -77,10 +80,11 @@ def make_plan(M, N, K, dtype="float16", layout="nt", config=None, cus=None, use_
     kw = {k: v for k, v in kw.items() if v is not None}
     if use_tuned and not config and not kw and cus is None:
         config = tuned_config(M, N, K, dtype, layout)
-        if config is None and dtype == "bfloat16":
-            # the bfloat16 kernels are twins of the fp16 ones (same data movement, same MFMA rate): a shape tuned
-            # for fp16 only takes that entry, where the kernel it names has a twin
-            borrowed = tuned_config(M, N, K, "float16", layout)
+        if config is None and dtype in _TWIN_OF:
+            # the bfloat16 kernels are twins of the fp16 ones, the e5m2 kernels of the e4m3 ones (same data
+            # movement, same MFMA rate): a shape tuned for the other type only takes that entry, where the kernel
+            # it names has a twin
+            borrowed = tuned_config(M, N, K, _TWIN_OF[dtype], layout)
             if borrowed is not None:
                 try:
                     return make_plan(M, N, K, dtype, layout, borrowed)

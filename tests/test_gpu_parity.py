@@ -680,6 +680,11 @@ def test_fp8_small_m_kernels(sk, oracle):
             A, W = torch.randn(M, 4096).to(dt), torch.randn(4096, 4096).to(dt)
             ref = oracle.f8_gemm_ref(A.view(torch.uint8).numpy(), W.view(torch.uint8).numpy(), fmt)
             assert _rel(oracle, sk.streamk_fp8(A.cuda(), W.cuda()), ref) <= 1e-3, (fmt, M)
+    # an e5m2 shape without a tuned entry of its own takes the e4m3 entry (twin kernels)
+    if sk.tuned_config(1, 8192, 8192, "float8_e5m2") is None and sk.tuned_config(1, 8192, 8192, "float8_e4m3"):
+        want, got = sk.make_plan(1, 8192, 8192, "float8_e4m3"), sk.make_plan(1, 8192, 8192, "float8_e5m2")
+        assert (got.bm, got.bn, got.bk, got.grid, got.schedule) == (want.bm, want.bn, want.bk, want.grid, want.schedule)
+        assert got.kernel_id == want.kernel_id + 10
     # strided operands (leading dimensions a multiple of 16 bytes)
     big = torch.randn(300, 4096).to(torch.float8_e4m3fn).cuda()
     A, W = big[:9, 16:16 + 2048], big[40:, 1024:1024 + 2048]
