@@ -194,7 +194,9 @@ struct KernelInfo {
   X(254, 1, 1, 2, 4, 2, 0)      \
   X(255, 1, 1, 4, 2, 2, 0)      \
   X(256, 2, 1, 4, 2, 2, 0)      \
-  X(257, 1, 1, 4, 1, 4, 1)
+  X(257, 1, 1, 4, 1, 4, 1)      \
+  X(258, 4, 1, 4, 1, 2, 0)      \
+  X(259, 4, 1, 4, 2, 2, 0)
 
 // int8 small-M kernels (dtype SK_I8, int32 C); bk counts int8 elements:  X(id, MB, NB, WN, RK, DEPTH, ROW1)
 #define SK_SKINNY_I8_KERNELS(X) \
@@ -205,7 +207,9 @@ struct KernelInfo {
   X(274, 1, 1, 2, 4, 2, 0)      \
   X(275, 1, 1, 4, 2, 2, 0)      \
   X(276, 2, 1, 4, 2, 2, 0)      \
-  X(277, 1, 1, 4, 1, 4, 1)
+  X(277, 1, 1, 4, 1, 4, 1)      \
+  X(278, 4, 1, 4, 1, 2, 0)      \
+  X(279, 4, 1, 4, 2, 2, 0)
 
 // bfloat16 twins of the fp16 matrix-vector kernels (dtype SK_BF16, variant 2)
 #define SK_GEMV_BF16_KERNELS(X) \

@@ -70,7 +70,9 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
   const KernelInfo *best = nullptr;
   // (for 32 < M <= 64 the 64x64 LDS tile below is faster than streaming the weights past 64 rows)
   const bool q4 = dtype == SK_Q4 || dtype == SK_Q4_TILED || dtype == SK_Q4_ZP;
-  if ((M <= 32 && layout == SK_LAYOUT_NT) || q4) {
+  // (one-byte operands: up to 64 rows -- their tile kernels start at 128 rows)
+  const bool one_byte = dtype == SK_F8E4M3 || dtype == SK_F8E5M2 || dtype == SK_I8;
+  if ((M <= (one_byte ? 64 : 32) && layout == SK_LAYOUT_NT) || q4) {
     // M == 1 with Q4 weights: the matrix-vector kernel with four waves splitting K (data-parallel
     // over 16-row tiles), the fastest instance at LLM-sized N and K
     if (q4 && M == 1 && want_variant < 0)

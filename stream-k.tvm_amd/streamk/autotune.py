@@ -26,7 +26,8 @@ _TILES_F16 = [(256, 256, 64), (128, 128, 64), (128, 256, 64), (256, 128, 64), (6
               (64, 128, 64)]
 _SKINNY_F16 = [(16, 64, 128), (32, 64, 128), (64, 64, 128), (16, 16, 512), (16, 32, 256), (16, 16, 128),
                (16, 16, 1024), (16, 32, 512), (16, 16, 256), (16, 64, 256), (32, 64, 256), (64, 64, 256)]
-_SKINNY_F8 = [(16, 64, 256), (32, 64, 256), (16, 16, 1024), (16, 32, 512), (16, 32, 1024), (16, 64, 512), (32, 64, 512)]
+_SKINNY_F8 = [(16, 64, 256), (32, 64, 256), (16, 16, 1024), (16, 32, 512), (16, 32, 1024), (16, 64, 512), (32, 64, 512),
+              (64, 64, 256), (64, 64, 512)]
 _SKINNY_Q4 = [(16, 64, 256), (32, 64, 256), (64, 64, 256), (16, 16, 1024), (16, 32, 512), (16, 16, 256),
               (16, 32, 256), (16, 32, 1024), (16, 16, 2048), (16, 64, 512), (16, 16, 512)]
 
@@ -57,8 +58,8 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
     schedule, grid and fix-up."""
     cus = cus or _plan.num_cus()
     out = []
-    f8 = dtype in ("float8_e4m3", "float8_e5m2", "int8")  # one-byte operands: small-M kernels up to 32 rows
-    if dtype in ("q4", "q4_zp") or (M <= 64 and not (f8 and M > 32)):
+    f8 = dtype in ("float8_e4m3", "float8_e5m2", "int8")  # one-byte operands
+    if dtype in ("q4", "q4_zp") or M <= 64:
         tiles = _SKINNY_Q4 if dtype in ("q4", "q4_zp") else (_SKINNY_F8 if f8 else _SKINNY_F16)
         for (bm, bn, bk) in tiles:
             if bm < M and not (bm == 16 and M <= 16):

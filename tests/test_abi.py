@@ -96,16 +96,17 @@ def test_fixed_split_k_schedule(sk):
 
 
 def test_fp8_plans(sk):
-    """fp8 / int8 plans: tile kernels from 33 rows, weight-streaming kernels up to 32 rows; bk counts one-byte
+    """fp8 / int8 plans: tile kernels from 65 rows, weight-streaming kernels up to 64 rows; bk counts one-byte
     elements; NT only."""
-    for (M, bm, name) in [(1, 16, "mb1_wn4_rk1_row1_1"), (16, 16, "mb1_wn4_rk1_row1_0"), (32, 32, "mb2_wn4_rk1_row1_0")]:
+    for (M, bm, name) in [(1, 16, "mb1_wn4_rk1_row1_1"), (16, 16, "mb1_wn4_rk1_row1_0"), (32, 32, "mb2_wn4_rk1_row1_0"),
+                          (64, 64, "mb4_wn4_rk1_row1_0")]:
         for dtype, tag in (("float8_e4m3", "f8e4m3"), ("float8_e5m2", "f8e5m2")):
             p = sk.make_plan(M, 4096, 4096, dtype, "nt", cus=256)
             assert (p.bm, p.bn, p.bk) == (bm, 64, 256) and p.iters_per_tile == 4096 // 256
             assert sk.kernel_name(p.kernel_id) == f"skinny_{tag}_{name}"
         q = sk.make_plan(M, 4096, 4096, "int8", "nt", cus=256)
         assert (q.bm, q.bn, q.bk) == (bm, 64, 256) and sk.kernel_name(q.kernel_id) == f"skinny_i8_{name}"
-    for (M, N, K, bm) in [(8192, 8192, 8192, 256), (512, 512, 4096, 128), (33, 4096, 4096, 128)]:
+    for (M, N, K, bm) in [(8192, 8192, 8192, 256), (512, 512, 4096, 128), (65, 4096, 4096, 128)]:
         p = sk.make_plan(M, N, K, "float8_e4m3", "nt", cus=256)
         assert (p.bm, p.bn, p.bk) == (bm, bm, 128) and p.iters_per_tile == K // 128
         assert sk.kernel_name(p.kernel_id) == f"tile_f8e4m3_nt_dma_{bm}x{bm}x128"

@@ -641,19 +641,20 @@ def test_fp8_tile_kernels(sk, oracle):
 
 
 def test_fp8_small_m_kernels(sk, oracle):
-    """Weight-streaming fp8 kernels (M <= 32; e4m3 and e5m2): every instance, ragged N, a K tail (K a multiple of 16
+    """Weight-streaming fp8 kernels (M <= 64; e4m3 and e5m2): every instance, ragged N, a K tail (K a multiple of 16
     only), data-parallel and Stream-K with both fix-ups, against the float64 host product of the decoded bytes
     (1e-3: fp16 rounding of C); {-1,0,1} data must come out exact -- a lane's 16 bytes are split over two MFMAs, so
     any mispairing of A and weight bytes along K would show; alpha, bias and activation in the epilogue; the plans
-    the library picks for 1..32 rows are these kernels."""
+    the library picks for 1..64 rows are these kernels."""
     import torch
     torch.manual_seed(23)
     cfgs = [dict(bm=16, bn=64, bk=256), dict(bm=32, bn=64, bk=256), dict(bm=16, bn=16, bk=1024), dict(bm=16, bn=32, bk=512),
-            dict(bm=16, bn=32, bk=1024), dict(bm=16, bn=64, bk=512), dict(bm=32, bn=64, bk=512), dict(bm=16, bn=64, bk=256, variant=2)]
+            dict(bm=16, bn=32, bk=1024), dict(bm=16, bn=64, bk=512), dict(bm=32, bn=64, bk=512), dict(bm=16, bn=64, bk=256, variant=2),
+            dict(bm=64, bn=64, bk=256), dict(bm=64, bn=64, bk=512)]
     N, K = 1000, 2064
     bias = torch.randint(-20, 20, (N,)).half()
     for fmt, dt in (("e4m3", torch.float8_e4m3fn), ("e5m2", torch.float8_e5m2)):
-        first, last = (250, 257) if fmt == "e4m3" else (260, 267)
+        first, last = (250, 259) if fmt == "e4m3" else (260, 269)
         B = torch.randn(N, K).to(dt)
         Bi = torch.randint(-1, 2, (N, K)).float().to(dt)
         for cfg in cfgs:
@@ -674,7 +675,7 @@ def test_fp8_small_m_kernels(sk, oracle):
                     assert np.array_equal(Cb.double().cpu().numpy(), np.maximum(0.5 * exact + bias.double().numpy(), 0)), (fmt, cfg, M, sch)
                     if sch.get("fixup") == "reduce":
                         assert torch.equal(C, sk.streamk_fp8(A.cuda(), B.cuda(), plan=plan))
-        for M in (1, 7, 16, 32):
+        for M in (1, 7, 16, 32, 64):
             plan = sk.make_plan(M, 4096, 4096, "float8_" + fmt, "nt")
             assert first <= plan.kernel_id <= last, (fmt, M, plan.kernel_id)
             A, W = torch.randn(M, 4096).to(dt), torch.randn(4096, 4096).to(dt)
@@ -694,13 +695,14 @@ def test_fp8_small_m_kernels(sk, oracle):
 
 
 def test_int8_small_m_kernels(sk, oracle):
-    """Weight-streaming int8 kernels (M <= 32, int32 C): every instance, ragged N, a K tail, data-parallel and
+    """Weight-streaming int8 kernels (M <= 64, int32 C): every instance, ragged N, a K tail, data-parallel and
     Stream-K with both fix-ups and the K split over waves -- all must equal the host product in int64 exactly, on
-    the full int8 range (-128 included); strided operands; the plans the library picks for 1..32 rows."""
+    the full int8 range (-128 included); strided operands; the plans the library picks for 1..64 rows."""
     import torch
     g = torch.Generator().manual_seed(29)
     cfgs = [dict(bm=16, bn=64, bk=256), dict(bm=32, bn=64, bk=256), dict(bm=16, bn=16, bk=1024), dict(bm=16, bn=32, bk=512),
-            dict(bm=16, bn=32, bk=1024), dict(bm=16, bn=64, bk=512), dict(bm=32, bn=64, bk=512), dict(bm=16, bn=64, bk=256, variant=2)]
+            dict(bm=16, bn=32, bk=1024), dict(bm=16, bn=64, bk=512), dict(bm=32, bn=64, bk=512), dict(bm=16, bn=64, bk=256, variant=2),
+            dict(bm=64, bn=64, bk=256), dict(bm=64, bn=64, bk=512)]
     N, K = 1000, 2064
     B = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int8)
     for cfg in cfgs:
@@ -709,12 +711,12 @@ def test_int8_small_m_kernels(sk, oracle):
             ref = oracle.i8_gemm_ref(A.numpy(), B.numpy())
             for sch in (dict(schedule="dp"), dict(schedule="sk2", fixup="reduce", grid=24), dict(schedule="sk2", fixup="atomic", grid=20)):
                 plan = sk.make_plan(M, N, K, "int8", "nt", dict(cfg, **sch))
-                assert 270 <= plan.kernel_id <= 277 and plan.iters_per_tile == -(-K // cfg["bk"]), (cfg, plan.kernel_id)
+                assert 270 <= plan.kernel_id <= 279 and plan.iters_per_tile == -(-K // cfg["bk"]), (cfg, plan.kernel_id)
                 C = sk.streamk_int8(A.cuda(), B.cuda(), plan=plan)
                 assert C.dtype == torch.int32 and np.array_equal(C.cpu().numpy(), ref), (cfg, M, sch)
-    for M in (1, 7, 16, 32):
+    for M in (1, 7, 16, 32, 64):
         plan = sk.make_plan(M, 4096, 4096, "int8", "nt")
-        assert 270 <= plan.kernel_id <= 277, (M, plan.kernel_id)
+        assert 270 <= plan.kernel_id <= 279, (M, plan.kernel_id)
         A = torch.randint(-128, 128, (M, 4096), generator=g, dtype=torch.int8)
         W = torch.randint(-128, 128, (4096, 4096), generator=g, dtype=torch.int8)
         assert np.array_equal(sk.streamk_int8(A.cuda(), W.cuda()).cpu().numpy(), oracle.i8_gemm_ref(A.numpy(), W.numpy())), M
