@@ -141,10 +141,23 @@ int sk_plan_tile_coords(const sk_plan *plan, int tile, int32_t *pid_m, int32_t *
 size_t sk_workspace_bytes(const sk_plan *plan);
 
 /* Must be run once on a freshly allocated workspace (and after an SK_ERR_TIMEOUT); kernels leave
- * the workspace clean for the next launch.  Uses a fill kernel, so it may be graph-captured. */
+ * flags and counters clean for the next launch, and the workspace itself records whether its partial
+ * area holds leftovers (REDUCE launches leave partial tiles behind, ATOMIC launches need zeroed
+ * accumulators: every ATOMIC launch is preceded by a small kernel that zero-fills the area if, and as
+ * far as, it is marked dirty).  That record lives in device memory, so launches replayed from a HIP
+ * graph see what really ran before them: one workspace may serve eager and captured launches of both
+ * fix-ups, as long as they do not overlap in time.  Uses a fill kernel, so it may be graph-captured.
+ * The library remembers which addresses were initialised (launches on any other workspace return
+ * SK_ERR_WORKSPACE); sk_workspace_release forgets one -- call it before freeing the buffer, so that a
+ * later allocation at the same address is not mistaken for it.  No counterpart in the reference, whose
+ * kernels use no workspace (atomicAdd into a pre-zeroed C, streamk_fp16.py:248-255,385). */
 int sk_workspace_init(void *ws, size_t ws_bytes, void *stream);
+int sk_workspace_release(void *ws);
 
-/* Reads the workspace status word (synchronises the stream): SK_OK or SK_ERR_TIMEOUT. */
+/* Reads the workspace status word (synchronises the stream): SK_OK or SK_ERR_TIMEOUT.  A fix-up wait
+ * that timed out stored an incomplete tile to C and may have left flags raised: once this call has
+ * reported it, every launch on the workspace returns SK_ERR_TIMEOUT until sk_workspace_init has run on
+ * it again.  Callers that set a small spin_limit should poll this at their synchronisation points. */
 int sk_workspace_status(void *ws, void *stream);
 
 /*

@@ -1,7 +1,7 @@
 """Per-CTA phase timeline of a small-M kernel, from the tracing build of the library.
 
     make -C stream-k.tvm_amd/csrc trace
-    python3 stream-k.tvm_amd/streamk/phase_trace.py 1x8192x8192 --dtype q4 --config "dict(bm=16,bn=16,bk=1024,schedule='dp')"
+    python3 phase_trace.py 1x8192x8192 --dtype q4 --config "dict(bm=16,bn=16,bk=1024,schedule='dp')"
 
 Thread 0 of every CTA stores the shader cycle counter at fixed points (SK_TRACE in the kernels);
 the counters of different CUs are not synchronised, so every time is relative to the CTA's own
@@ -12,7 +12,7 @@ import ctypes
 import os
 import sys
 
-sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "stream-k.tvm_amd"))
 
 NAMES = {0: "kernel entry", 10: "CTA range known", 11: "tile coordinates known", 1: "segment entered",
          2: "prologue loads issued", 3: "A staged", 4: "scales staged", 5: "barrier passed", 6: "loop entered",

@@ -1,8 +1,8 @@
 """Runs one GEMM case a few times so that a profiler sees nothing else.
 
-    rocprofv3 --kernel-trace --stats -- python3 stream-k.tvm_amd/streamk/profile_case.py 8192x8192x8192
-    python3 stream-k.tvm_amd/streamk/profile_case.py 1x8192x8192 --dtype q4 --config "dict(grid=256)"
-    python3 stream-k.tvm_amd/streamk/profile_case.py 8192x8192x8192 --data zeros --time --vendor
+    rocprofv3 --kernel-trace --stats -- python3 profile_case.py 8192x8192x8192
+    python3 profile_case.py 1x8192x8192 --dtype q4 --config "dict(grid=256)"
+    python3 profile_case.py 8192x8192x8192 --data zeros --time --vendor
 
 --data chooses the operand values (the clock the part sustains depends on how many bits toggle);
 --time prints the average time of --reps launches; --vendor also times torch.matmul (hipBLASLt) on the
@@ -12,7 +12,7 @@ import argparse
 import os
 import sys
 
-sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "stream-k.tvm_amd"))
 
 
 def main():

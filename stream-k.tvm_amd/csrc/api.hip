@@ -15,10 +15,15 @@ namespace {
 struct DeviceInfo {
   int ok = 0, cus = 0, clock_khz = 0, lds = 0;
 };
-DeviceInfo &device_info() {
+// one mutex guards every lazily filled table of this file (device properties, occupancies, the
+// workspace registry): the entry points may be called from several host threads
+std::mutex g_mutex;
+
+DeviceInfo device_info() {
   static DeviceInfo d[16];
   int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) { static DeviceInfo bad; return bad; }
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return DeviceInfo();
+  std::lock_guard<std::mutex> lock(g_mutex);
   if (!d[dev].ok) {
     hipDeviceProp_t p;
     if (hipGetDeviceProperties(&p, dev) == hipSuccess) {
@@ -37,13 +42,40 @@ __global__ void fill_zero_kernel(uint32_t *p, size_t n) {
   for (; i < n; i += stride) p[i] = 0;
 }
 
-// What the library knows about the contents of each workspace it has been handed.  Kernels leave
-// flags and counters at zero.  ATOMIC launches also leave the partial area zeroed (and need it
-// zeroed); REDUCE launches leave partial tiles behind.  An ATOMIC launch on a workspace whose partial
-// area is dirty is therefore preceded by a stream-ordered fill of that area.
-enum WsState { WS_CLEAN = 0, WS_PARTIALS_DIRTY = 1 };
-std::mutex g_ws_mutex;
-std::unordered_map<const void *, int> g_ws_state;
+// Whether the partial area holds leftovers is recorded in the workspace itself, not on the host, so
+// that a launch replayed from a graph sees what actually ran before it.  Kernels leave flags and
+// counters at zero.  ATOMIC launches need the accumulators they add into zeroed and leave them
+// zeroed; REDUCE launches leave partial tiles behind and raise the high-water mark status[WS_DIRTY]
+// (in 256-byte units from the start of the partial area) past every slot they write.  This kernel
+// runs in front of every ATOMIC launch: with the mark at zero it returns at once; otherwise it
+// zero-fills the area up to the mark (as far as the caller's buffer reaches) and the block that
+// finishes last lowers the mark again.
+__global__ void clean_partials_kernel(int *status, uint4v *partials, unsigned capacity_units) {
+  const unsigned mark = (unsigned)__hip_atomic_load(status + WS_DIRTY, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (mark == 0) return;
+  const size_t n16 = (size_t)(mark < capacity_units ? mark : capacity_units) * 16;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) partials[i] = uint4v{0, 0, 0, 0};
+  __syncthreads();  // every thread of the block has read the mark
+  if (threadIdx.x == 0) {
+    const int done = __hip_atomic_fetch_add(status + WS_CLEAN_DONE, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (done == (int)gridDim.x - 1) {
+      __hip_atomic_store(status + WS_CLEAN_DONE, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      // a mark beyond this caller's buffer stays: a later call with the larger buffer cleans the rest
+      if (mark <= capacity_units) __hip_atomic_store(status + WS_DIRTY, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+}
+
+// Workspaces the library has initialised (sk_workspace_init) and not been told to forget
+// (sk_workspace_release).  `poisoned` is set when sk_workspace_status has seen a timed-out fix-up
+// wait: flags of that launch may still be raised, so further launches are refused until the
+// workspace is initialised again.
+struct WsInfo {
+  size_t bytes;
+  bool poisoned;
+};
+std::unordered_map<const void *, WsInfo> g_ws;
 
 int check_plan(const sk_plan *plan, int64_t M, int64_t N, int64_t K, int dtype, int layout) {
   if (!plan) return SK_ERR_NULL;
@@ -57,27 +89,25 @@ int make_dev_plan(const sk_plan *plan, const KernelInfo *k, void *ws, size_t ws_
   if ((size_t)plan->workspace_bytes > ws_bytes) return SK_ERR_WORKSPACE;
   if (plan->workspace_bytes > 0 && !ws) return SK_ERR_WORKSPACE;
   if (plan->workspace_bytes > 0 && (reinterpret_cast<uintptr_t>(ws) & 255)) return SK_ERR_ALIGN;
-  DeviceInfo &d = device_info();
+  const DeviceInfo d = device_info();
   if (!d.ok) return SK_ERR_DEVICE;
   // every CTA of the Stream-K wave may wait on another one: they must all be resident
   if (plan->streamk_tiles > 0 && plan->fixup == SK_FIXUP_REDUCE &&
       (occupancy <= 0 || plan->grid > d.cus * occupancy))
     return SK_ERR_CONFIG;
   if (plan->workspace_bytes > 0) {
-    const size_t part_off = (size_t)WS_PART_OFF;
-    std::lock_guard<std::mutex> lock(g_ws_mutex);
-    auto it = g_ws_state.find(ws);
-    if (it == g_ws_state.end()) return SK_ERR_WORKSPACE;  // sk_workspace_init was never run on it
-    if (plan->fixup == SK_FIXUP_ATOMIC && it->second == WS_PARTIALS_DIRTY) {
-      const size_t n = (ws_bytes - part_off) / 4;
-      int blocks = (int)((n + 255) / 256);
-      if (blocks > 4096) blocks = 4096;
-      hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(256), 0, stream,
-                         reinterpret_cast<uint32_t *>(static_cast<char *>(ws) + part_off), n);
+    {
+      std::lock_guard<std::mutex> lock(g_mutex);
+      auto it = g_ws.find(ws);
+      if (it == g_ws.end() || it->second.bytes < ws_bytes) return SK_ERR_WORKSPACE;  // sk_workspace_init was never run on it
+      if (it->second.poisoned) return SK_ERR_TIMEOUT;
+    }
+    if (plan->fixup == SK_FIXUP_ATOMIC) {
+      char *base = static_cast<char *>(ws);
+      const size_t units = (ws_bytes - (size_t)WS_PART_OFF) / 256;
+      hipLaunchKernelGGL(clean_partials_kernel, dim3(1024), dim3(256), 0, stream, reinterpret_cast<int *>(base),
+                         reinterpret_cast<uint4v *>(base + WS_PART_OFF), (unsigned)(units > 0xffffffffu ? 0xffffffffu : units));
       if (hipGetLastError() != hipSuccess) return SK_ERR_LAUNCH;
-      it->second = WS_CLEAN;
-    } else if (plan->fixup == SK_FIXUP_REDUCE) {
-      it->second = WS_PARTIALS_DIRTY;
     }
   }
   dp->tiles_m = plan->num_block_m;
@@ -112,12 +142,14 @@ int make_dev_plan(const sk_plan *plan, const KernelInfo *k, void *ws, size_t ws_
   return SK_OK;
 }
 
-int cached_occupancy(int id, bool skinny) {
+// family: 0 tile kernels, 1 small-M kernels, 2 fp32 kernels
+int cached_occupancy(int id, int family) {
   static int cache[512];
   static bool have[512];
-  int slot = id & 511;  // kernel ids stay below 512
+  const int slot = id & 511;  // kernel ids stay below 512
+  std::lock_guard<std::mutex> lock(g_mutex);
   if (!have[slot]) {
-    cache[slot] = skinny ? occupancy_skinny(id) : occupancy_tile(id);
+    cache[slot] = family == 1 ? occupancy_skinny(id) : (family == 2 ? occupancy_f32(id) : occupancy_tile(id));
     have[slot] = true;
   }
   return cache[slot];
@@ -148,7 +180,7 @@ extern "C" const char *sk_strerror(int s) {
 }
 
 extern "C" int sk_device_info(int *num_cus, int *clock_khz, int *lds_bytes_per_cu) {
-  DeviceInfo &d = device_info();
+  const DeviceInfo d = device_info();
   if (!d.ok) return SK_ERR_DEVICE;
   if (num_cus) *num_cus = d.cus;
   if (clock_khz) *clock_khz = d.clock_khz;
@@ -166,9 +198,15 @@ extern "C" int sk_workspace_init(void *ws, size_t ws_bytes, void *stream) {
   hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream,
                      static_cast<uint32_t *>(ws), n);
   if (hipGetLastError() != hipSuccess) return SK_ERR_LAUNCH;
-  std::lock_guard<std::mutex> lock(g_ws_mutex);
-  g_ws_state[ws] = WS_CLEAN;
+  std::lock_guard<std::mutex> lock(g_mutex);
+  g_ws[ws] = WsInfo{ws_bytes, false};
   return SK_OK;
+}
+
+extern "C" int sk_workspace_release(void *ws) {
+  if (!ws) return SK_ERR_NULL;
+  std::lock_guard<std::mutex> lock(g_mutex);
+  return g_ws.erase(ws) ? SK_OK : SK_ERR_WORKSPACE;
 }
 
 extern "C" int sk_workspace_status(void *ws, void *stream) {
@@ -177,7 +215,11 @@ extern "C" int sk_workspace_status(void *ws, void *stream) {
   if (hipMemcpyAsync(&v, ws, sizeof(int), hipMemcpyDeviceToHost, (hipStream_t)stream) != hipSuccess)
     return SK_ERR_LAUNCH;
   if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) return SK_ERR_LAUNCH;
-  return v == 0 ? SK_OK : SK_ERR_TIMEOUT;
+  if (v == 0) return SK_OK;
+  std::lock_guard<std::mutex> lock(g_mutex);
+  auto it = g_ws.find(ws);
+  if (it != g_ws.end()) it->second.poisoned = true;
+  return SK_ERR_TIMEOUT;
 }
 
 // checks an sk_epilogue and packs it into the one word the kernels take (0 = no epilogue)
@@ -214,7 +256,7 @@ static int gemm_16bit(int dtype, const void *A, const void *B, void *C, int64_t 
   DevPlan dp;
   Workspace w;
   const bool skinny = k->family == FAMILY_SKINNY;
-  rc = make_dev_plan(plan, k, ws, ws_bytes, cached_occupancy(k->id, skinny), (hipStream_t)stream, &dp, &w);
+  rc = make_dev_plan(plan, k, ws, ws_bytes, cached_occupancy(k->id, skinny ? 1 : 0), (hipStream_t)stream, &dp, &w);
   if (rc) return rc;
   int herr;
   if (skinny) {
@@ -272,7 +314,7 @@ static int gemm_8bit(int dtype, const void *A, const void *B, void *C, int64_t M
   DevPlan dp;
   Workspace w;
   const bool skinny = k->family == FAMILY_SKINNY;
-  rc = make_dev_plan(plan, k, ws, ws_bytes, cached_occupancy(k->id, skinny), (hipStream_t)stream, &dp, &w);
+  rc = make_dev_plan(plan, k, ws, ws_bytes, cached_occupancy(k->id, skinny ? 1 : 0), (hipStream_t)stream, &dp, &w);
   if (rc) return rc;
   if (skinny) {  // small-M fp8 / int8 kernels: bytes travel as pairs, alpha in the `zero` field (int8: C is int32)
     SkinnyArgs a{(const half_t *)A, B, nullptr, (half_t *)C, (int)M, (int)N, (int)(K / 2), lda / 2, ldb / 2, ldc,
@@ -323,10 +365,7 @@ extern "C" int sk_gemm_f32(const void *A, const void *B, void *C, int64_t M, int
   if (lda * 4 * k->bm >= (int64_t)1 << 31 || ldb * 4 * (nn ? K : k->bn) >= (int64_t)1 << 31) return SK_ERR_SHAPE;
   DevPlan dp;
   Workspace w;
-  static int occ[2] = {0, 0};
-  int &o = occ[k->id == 200 ? 0 : 1];
-  if (o == 0) o = occupancy_f32(k->id);
-  rc = make_dev_plan(plan, k, ws, ws_bytes, o, (hipStream_t)stream, &dp, &w);
+  rc = make_dev_plan(plan, k, ws, ws_bytes, cached_occupancy(k->id, 2), (hipStream_t)stream, &dp, &w);
   if (rc) return rc;
   GemmArgsF32 a{(const float *)A, (const float *)B, (float *)C, (int)M, (int)N, (int)K, lda, ldb, ldc};
   return launch_f32(k->id, a, dp, w, (hipStream_t)stream) == 0 ? SK_OK : SK_ERR_LAUNCH;
@@ -353,7 +392,7 @@ static int gemm_q4_any(const void *A, const void *Wq, const void *scales, const 
   if (lda * 2 * k->bm >= (int64_t)1 << 31 || (K / 2) * k->bn >= (int64_t)1 << 31) return SK_ERR_SHAPE;
   DevPlan dp;
   Workspace w;
-  rc = make_dev_plan(plan, k, ws, ws_bytes, cached_occupancy(k->id, true), (hipStream_t)stream, &dp, &w);
+  rc = make_dev_plan(plan, k, ws, ws_bytes, cached_occupancy(k->id, 1), (hipStream_t)stream, &dp, &w);
   if (rc) return rc;
   SkinnyArgs a{(const half_t *)A, Wq, (const half_t *)scales, (half_t *)C, (int)M, (int)N, (int)K,
                lda, K / 2, ldc, zero, (int)(K / group), (const half_t *)zeros};

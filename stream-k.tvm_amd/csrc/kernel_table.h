@@ -6,10 +6,10 @@
 
 namespace sk {
 
-// Workspace layout (bytes): [0,256) status word; [256, 256+WS_FLAG_BYTES) flags (REDUCE: one per
+// Workspace layout (bytes): [0,256) status block; [256, 256+WS_FLAG_BYTES) flags (REDUCE: one per
 // CTA) or arrival counters (ATOMIC: one per Stream-K tile); then the fp32 partial tiles.  The flag
 // area has a fixed size so that partial tiles of one plan never land where another plan keeps
-// its flags.
+// its flags.  The words of the status block are named in sk_device.h (WS_STATUS, ...).
 constexpr int64_t WS_FLAG_BYTES = 262144;
 constexpr int64_t WS_PART_OFF = 256 + WS_FLAG_BYTES;
 constexpr int64_t WS_MAX_FLAGS = WS_FLAG_BYTES / 4;

@@ -6,25 +6,28 @@
 // max(blocking_tiles // total_sm, 1) walks out of range when there are no data-parallel tiles).
 #include <string.h>
 
+#include <mutex>
+
 #include "kernel_table.h"
 #include "streamk.h"
 
 namespace sk {
 
 static KernelInfo g_table[320];
-static int g_count = -1;
+static int g_count = 0;
+static std::once_flag g_table_once;
 
 int tile_kernel_infos(KernelInfo *out, int max);
 int skinny_kernel_infos(KernelInfo *out, int max);
 int f32_kernel_infos(KernelInfo *out, int max);
 
 const KernelInfo *kernel_table(int *count) {
-  if (g_count < 0) {
+  std::call_once(g_table_once, [] {
     int n = tile_kernel_infos(g_table, 320);
     n += skinny_kernel_infos(g_table + n, 320 - n);
     n += f32_kernel_infos(g_table + n, 320 - n);
     g_count = n;
-  }
+  });
   if (count) *count = g_count;
   return g_table;
 }

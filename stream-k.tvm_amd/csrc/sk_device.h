@@ -62,6 +62,11 @@ struct DevPlan {
   FastDiv by_ipt, by_tiles_n, by_width, by_raster, by_tail, by_full1, by_full;
 };
 
+// Words of the workspace's status block: WS_STATUS a timed-out fix-up wait (0 or SK_ERR_TIMEOUT),
+// WS_DIRTY how far the partial area holds leftovers of REDUCE launches (256-byte units from its
+// start), WS_CLEAN_DONE the block counter of the kernel that zero-fills it again.
+enum { WS_STATUS = 0, WS_DIRTY = 1, WS_CLEAN_DONE = 2 };
+
 struct Workspace {
   int *status;
   int *flags;
@@ -144,8 +149,11 @@ __device__ __forceinline__ void st_coherent(float *p, float v) {
 __device__ __forceinline__ float ld_coherent_scalar(const float *p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-// all of this thread's earlier memory operations have been performed (wait counters only)
-__device__ __forceinline__ void wait_own_memory_ops() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup"); }
+// Every vector memory operation this thread has issued -- loads, stores and atomics without return all
+// count on vmcnt on this target -- has been acknowledged by the memory system.  A workgroup-scope
+// fence is not enough: it waits for LDS traffic only, and the barrier that follows adds no wait of
+// its own, so a flag raised after it could overtake the partial it announces.
+__device__ __forceinline__ void wait_own_memory_ops() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // ---- REDUCE fix-up: flags ----
 // Contributor: every thread waits for its own (write-through) partial stores, the barrier
@@ -153,11 +161,14 @@ __device__ __forceinline__ void wait_own_memory_ops() { __builtin_amdgcn_fence(_
 // COHERENT = false: the partial went through the L2 with ordinary stores; thread 0's device-scope
 // release (one L2 write-back for the whole CTA, after the barrier has collected everybody's
 // stores) publishes it together with the flag.
+// dirty_mark / dirty_units: the workspace's record of how far its partial area holds leftovers
+// (256-byte units) is raised past this CTA's slot, for the launch that next needs the area zeroed.
 template <bool COHERENT>
-__device__ __forceinline__ void signal_partial_ready(int *flag) {
+__device__ __forceinline__ void signal_partial_ready(int *flag, int *dirty_mark, int dirty_units) {
   wait_own_memory_ops();
   __syncthreads();
   if (threadIdx.x == 0) {
+    __hip_atomic_fetch_max(dirty_mark, dirty_units, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (COHERENT)
       __hip_atomic_store(flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     else

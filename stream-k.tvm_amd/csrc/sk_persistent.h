@@ -94,13 +94,14 @@ __device__ __forceinline__ void run_persistent(const typename P::Args &a, const 
       } else if (k0 != 0) {
         // not the tile's first CTA: park the partial in this CTA's slot and raise its flag
         P::store_partial(acc, ws.partials + (size_t)pid * P::TILE_ELEMS);
-        signal_partial_ready<P::COHERENT_PARTIALS>(&ws.flags[pid]);
+        signal_partial_ready<P::COHERENT_PARTIALS>(
+            &ws.flags[pid], ws.status + WS_DIRTY, (int)(((size_t)(pid + 1) * P::TILE_ELEMS * 4 + 255) >> 8));
       } else {
         // tile's first CTA: wait for all followers at once, then add their partials in ascending
         // CTA order and store
         const int npeers = sk_pid_of_iter(plan, (tile + 1) * ipt - 1) - pid;
         if (!wait_partials_ready<P::COHERENT_PARTIALS>(&ws.flags[pid + 1], npeers, plan.spin_limit)) {
-          if (threadIdx.x == 0) *ws.status = -8;  // SK_ERR_TIMEOUT
+          if (threadIdx.x == 0) ws.status[WS_STATUS] = -8;  // SK_ERR_TIMEOUT
         } else {
           for (int p = 1; p <= npeers; ++p) P::add_partial(acc, ws.partials + (size_t)(pid + p) * P::TILE_ELEMS);
           clear_flags_after_use(&ws.flags[pid + 1], npeers);

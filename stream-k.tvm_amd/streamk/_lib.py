@@ -79,6 +79,8 @@ def lib():
     L.sk_workspace_bytes.restype = sz
     L.sk_workspace_init.argtypes = [vp, sz, vp]
     L.sk_workspace_status.argtypes = [vp, vp]
+    L.sk_workspace_release.argtypes = [vp]
+    L.sk_workspace_release.restype = ci
     L.sk_gemm_f16.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, P(SkPlan), vp, sz, vp]
     L.sk_gemm_f32.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, P(SkPlan), vp, sz, vp]
     L.sk_gemm_bf16.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, P(SkPlan), vp, sz, vp]

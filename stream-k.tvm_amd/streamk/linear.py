@@ -65,6 +65,7 @@ class StreamKLinear(torch.nn.Module):
         return m
 
     def plan_for(self, M):
+        """The plan a call with M rows runs (what forward's operator call resolves to)."""
         p = self._plans.get(M)
         if p is None:
             dtype = self.weight_format
@@ -73,25 +74,25 @@ class StreamKLinear(torch.nn.Module):
 
     @torch.no_grad()
     def forward(self, x):
+        """Calls the registered operators (torch.ops.streamk.gemm_*) with tensors and plain values only, so the
+        module traces under torch.compile without a graph break; the operator keeps one plan per M it has seen
+        (from the tuned cache where the shape is in it)."""
         if x.dtype != self.dtype or x.shape[-1] != self.in_features:
             raise ValueError(f"input must be {self.dtype} [..., {self.in_features}], got {x.dtype} {tuple(x.shape)}")
         lead = x.shape[:-1]
         a = x.reshape(-1, self.in_features)
-        if a.stride(-1) != 1 or (a.shape[0] > 1 and a.stride(0) % 8) or a.data_ptr() % 16:
-            a = a.contiguous()
-        M = a.shape[0]
-        if M == 0:
+        if a.shape[0] == 0:
             return x.new_zeros(*lead, self.out_features)
         # bias and activation are applied in the GEMM's epilogue (fp32, before the rounding to C's type)
+        act = self.activation or "none"
         if self.weight_format == "float16":
-            c = ops.streamk_fp16(a, self.weight, plan=self.plan_for(M), bias=self.bias, activation=self.activation)
+            c = torch.ops.streamk.gemm_f16(a, self.weight, "nt", "", self.bias, act)
         elif self.weight_format == "bfloat16":
-            c = ops.streamk_bf16(a, self.weight, plan=self.plan_for(M), bias=self.bias, activation=self.activation)
+            c = torch.ops.streamk.gemm_bf16(a, self.weight, "nt", "", self.bias, act)
         else:
-            # (more rows than one Q4 launch takes: streamk_q4 splits the call itself)
-            c = ops.streamk_q4(a, self.qweight, self.scales, plan=self.plan_for(M) if M <= ops.Q4_MAX_M else None,
-                               zero=self.zero, group=self.group, zeros=getattr(self, "zeros", None), bias=self.bias,
-                               activation=self.activation)
+            zeros = self.zeros if self.weight_format == "q4_zp" else None
+            c = torch.ops.streamk.gemm_q4(a, self.qweight, self.scales, zeros, self.zero, self.group, False, "",
+                                          self.bias, act)
         return c.view(*lead, self.out_features)
 
     def extra_repr(self):

@@ -6,7 +6,16 @@ Mirrors the reference's operator surface:
   * `tl_matmul_streamk(M, N, K, ...)` returns a callable `kernel(A, B, C)` that writes C in place,
     the shape of the reference's `tl_mod = TL.Profiler(...)`; `tl_mod(A, B, b_c)`
     (streamk_fp16.py:382-387), including `do_bench`.
-torch is used for device memory and streams only.
+
+Every GEMM is registered with the PyTorch dispatcher as a custom operator of the `streamk` namespace
+(`torch.ops.streamk.gemm_f16`, `gemm_bf16`, `gemm_f32`, `gemm_q4`, `gemm_f8`, `gemm_i8`, each with an
+`_out` twin that writes a caller's C, plus `dequant_q4`): a HIP implementation that hands data
+pointers and the current stream to the C ABI, and a fake (meta) implementation that gives shape and
+dtype of the result, so that `torch.compile`, FakeTensor tracing and graph capture see an ordinary
+operator.  This is the role of the reference's `@jit(out_idx=[2])` wrapper, which turns the kernel
+into `f(A, B) -> C` (autotune/streamk_fp16_autotune.py:93-94).  The functions below are thin argument
+adapters over those operators.  torch is used for device memory, streams and the dispatcher only;
+all arithmetic happens in libstreamk.so.
 """
 import ctypes
 
@@ -30,6 +39,8 @@ def _workspace(nbytes, device):
            torch.cuda.current_stream().cuda_stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
+        if ws is not None:  # the library must not take a later allocation at this address for this workspace
+            _lib.lib().sk_workspace_release(ws.data_ptr())
         ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
         _lib.check(_lib.lib().sk_workspace_init(ws.data_ptr(), ws.numel(), _stream_ptr()),
                    "sk_workspace_init")
@@ -37,13 +48,26 @@ def _workspace(nbytes, device):
     return ws
 
 
+def _ws_args(plan, device):
+    ws = _workspace(plan.workspace_bytes, device)
+    return (ctypes.byref(plan), ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
+            _stream_ptr())
+
+
 def reset_workspaces():
-    """Drops cached workspaces (needed after a StreamKError with status SK_ERR_TIMEOUT)."""
+    """Drops cached workspaces.  Needed after workspace_status() (or a launch) has raised StreamKError
+    with status SK_ERR_TIMEOUT: the library refuses a workspace on which a fix-up wait gave up until it
+    has been initialised again, which the next call on a fresh workspace does."""
+    for ws in _workspaces.values():
+        _lib.lib().sk_workspace_release(ws.data_ptr())
     _workspaces.clear()
 
 
 def workspace_status():
-    """SK_OK / raises if any fix-up wait on the current stream's workspace timed out."""
+    """Synchronises the current stream and raises StreamKError(SK_ERR_TIMEOUT) if a fix-up wait on its
+    workspace gave up (the tile it was waiting for is then incomplete in C).  The launches themselves
+    only enqueue work, so this is where a timeout surfaces: call it wherever the caller synchronises
+    anyway (bench_ms, StreamKKernel.do_bench and the autotuner do)."""
     for (dev, stream), ws in _workspaces.items():
         if stream == torch.cuda.current_stream().cuda_stream:
             _lib.check(_lib.lib().sk_workspace_status(ws.data_ptr(), _stream_ptr()), "sk_workspace_status")
@@ -72,6 +96,324 @@ def _epilogue(bias, N, dtype, device, activation=None):
     return _lib.SkEpilogue(bias=bias.data_ptr(), activation=act)
 
 
+# ---------------------------------------------------------------------------------------------
+# Plans behind the operators.  An operator's schema carries tensors, numbers and strings only, so a
+# configuration travels as a string: "" (tuned cache, else the library's heuristic), "k=v;k=v" for
+# make_config keys, or "#n" for a plan object the caller made itself (kept in a registry here).
+# ---------------------------------------------------------------------------------------------
+_plan_registry = {}
+_plan_cache = {}
+
+
+def _plan_handle(plan):
+    h = getattr(plan, "_sk_handle", None)
+    if h is None:
+        h = plan._sk_handle = f"#{len(_plan_registry) + 1}"
+        _plan_registry[h] = plan
+    return h
+
+
+def _config_string(plan, config, kw):
+    if plan is not None:
+        return _plan_handle(plan)
+    d = dict(config or {})
+    d.update({k: v for k, v in kw.items() if v is not None})
+    return ";".join(f"{k}={d[k]}" for k in sorted(d))
+
+
+def _parse_config(text):
+    out = {}
+    for item in text.split(";"):
+        k, v = item.split("=", 1)
+        out[k] = int(v) if v.lstrip("-").isdigit() else v
+    return out
+
+
+def _plan_for(config, M, N, K, dtype, layout):
+    """The plan an operator call runs: the registered plan object, or one made from the configuration
+    string for this shape (made once per (shape, type, layout, configuration))."""
+    if config.startswith("#"):
+        plan = _plan_registry.get(config)
+        if plan is None:
+            raise ValueError(f"unknown plan handle {config!r}")
+        return plan
+    key = (M, N, K, dtype, layout, config)
+    plan = _plan_cache.get(key)
+    if plan is None:
+        plan = make_plan(M, N, K, dtype, layout, _parse_config(config) if config else None)
+        if len(_plan_cache) < 4096:
+            _plan_cache[key] = plan
+    return plan
+
+
+def _nk_of(B, layout):
+    if layout not in ("nt", "nn"):
+        raise ValueError("layout must be 'nt' (B is [N,K]) or 'nn' (B is [K,N])")
+    return tuple(B.shape) if layout == "nt" else (B.shape[1], B.shape[0])
+
+
+def _check_out(C, M, N, dtype):
+    _check_matrix(C, "out", dtype)
+    if tuple(C.shape) != (M, N):
+        raise ValueError("out has the wrong shape")
+
+
+def _act(activation):
+    return None if activation in (None, "none", "") else activation
+
+
+def _aligned_rows(A):
+    """A as the kernels can read it: unit stride along K, rows 16 bytes apart or more in multiples of 16, first
+    element 16-byte aligned.  Views that are not (a column slice, an odd storage offset) are copied."""
+    if isinstance(A, torch.Tensor) and A.dim() == 2 and A.is_cuda and A.shape[0] > 0 and (
+            A.stride(1) != 1 or (A.shape[0] > 1 and A.stride(0) * A.element_size() % 16) or A.data_ptr() % 16):
+        return A.clone(memory_format=torch.contiguous_format)
+    return A
+
+
+# ---- HIP implementations (write `C`) ----
+def _run_16bit(A, B, C, layout, config, bias, activation, tdtype, name):
+    A = _aligned_rows(A)
+    _check_matrix(A, "A", tdtype)
+    _check_matrix(B, "B", tdtype)
+    M, K = A.shape
+    N, Kb = _nk_of(B, layout)
+    if K != Kb:
+        raise ValueError(f"K mismatch: A is {tuple(A.shape)}, B is {tuple(B.shape)}")
+    _check_out(C, M, N, tdtype)
+    plan = _plan_for(config, M, N, K, name, layout)
+    epi = _epilogue(bias, N, tdtype, A.device, _act(activation))
+    args = (A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, A.stride(0), B.stride(0), C.stride(0),
+            *_ws_args(plan, A.device))
+    L = _lib.lib()
+    plain, ex = (L.sk_gemm_f16, L.sk_gemm_f16_ex) if tdtype == torch.float16 else (L.sk_gemm_bf16, L.sk_gemm_bf16_ex)
+    rc = plain(*args) if epi is None else ex(*args, ctypes.byref(epi))
+    _lib.check(rc, "sk_gemm_f16" if tdtype == torch.float16 else "sk_gemm_bf16")
+
+
+def _run_f32(A, B, C, layout, config):
+    _check_matrix(A, "A", torch.float32)
+    _check_matrix(B, "B", torch.float32)
+    M, K = A.shape
+    N, Kb = _nk_of(B, layout)
+    if K != Kb:
+        raise ValueError(f"K mismatch: A is {tuple(A.shape)}, B is {tuple(B.shape)}")
+    _check_out(C, M, N, torch.float32)
+    plan = _plan_for(config, M, N, K, "float32", layout)
+    rc = _lib.lib().sk_gemm_f32(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, A.stride(0), B.stride(0),
+                                C.stride(0), *_ws_args(plan, A.device))
+    _lib.check(rc, "sk_gemm_f32")
+
+
+_F8_KINDS = {getattr(torch, "float8_e4m3fn", None): "e4m3", getattr(torch, "float8_e5m2", None): "e5m2"}
+
+
+def _f8_format(A, B, fmt):
+    fmt = fmt or None
+    for t, name in ((A, "A"), (B, "B")):
+        if not isinstance(t, torch.Tensor) or (t.dtype != torch.uint8 and t.dtype not in _F8_KINDS):
+            raise TypeError(f"{name} must be a float8_e4m3fn / float8_e5m2 (or uint8) tensor")
+        if t.dtype != torch.uint8:
+            if fmt not in (None, _F8_KINDS[t.dtype]):
+                raise TypeError("A and B must be in the same fp8 format")
+            fmt = _F8_KINDS[t.dtype]
+    fmt = fmt or "e4m3"
+    if fmt not in ("e4m3", "e5m2"):
+        raise ValueError("fmt must be 'e4m3' or 'e5m2'")
+    return fmt
+
+
+def _run_f8(A, B, C, alpha, fmt, config, bias, activation):
+    fmt = _f8_format(A, B, fmt)
+    _check_matrix(A, "A", A.dtype)
+    _check_matrix(B, "B", B.dtype)
+    M, K = A.shape
+    N, Kb = B.shape
+    if K != Kb:
+        raise ValueError(f"K mismatch: A is {tuple(A.shape)}, B is {tuple(B.shape)}")
+    _check_out(C, M, N, torch.float16)
+    plan = _plan_for(config, M, N, K, "float8_" + fmt, "nt")
+    if plan.dtype != (_lib.SK_F8E5M2 if fmt == "e5m2" else _lib.SK_F8E4M3):
+        raise ValueError("the plan was made for the other fp8 format")
+    epi = _epilogue(bias, N, torch.float16, A.device, _act(activation))
+    args = (A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, A.stride(0), B.stride(0), C.stride(0), float(alpha),
+            *_ws_args(plan, A.device))
+    rc = _lib.lib().sk_gemm_f8(*args) if epi is None else _lib.lib().sk_gemm_f8_ex(*args, ctypes.byref(epi))
+    _lib.check(rc, "sk_gemm_f8")
+
+
+def _run_i8(A, B, C, config):
+    _check_matrix(A, "A", torch.int8)
+    _check_matrix(B, "B", torch.int8)
+    M, K = A.shape
+    N, Kb = B.shape
+    if K != Kb:
+        raise ValueError(f"K mismatch: A is {tuple(A.shape)}, B is {tuple(B.shape)}")
+    _check_out(C, M, N, torch.int32)
+    plan = _plan_for(config, M, N, K, "int8", "nt")
+    rc = _lib.lib().sk_gemm_i8(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, A.stride(0), B.stride(0),
+                               C.stride(0), *_ws_args(plan, A.device))
+    _lib.check(rc, "sk_gemm_i8")
+
+
+Q4_MAX_M = 64  # rows of A the Q4 kernels take in one launch
+
+
+def _zero_points(zeros, scales):
+    """Per-group zero points as the library takes them: fp16 [N, K/group] holding integers 0..15.  Integer
+    tensors are converted (an allocation per call: keep them as fp16 to avoid it)."""
+    if zeros.dtype != torch.float16:
+        zeros = zeros.to(torch.float16)
+    _check_matrix(zeros, "zeros", torch.float16)
+    if tuple(zeros.shape) != tuple(scales.shape) or not zeros.is_contiguous():
+        raise ValueError(f"zeros must be contiguous and shaped like scales; got {tuple(zeros.shape)}")
+    return zeros
+
+
+def _run_q4(A, Wq, scales, zeros, C, zero, group, tiled, config, bias, activation):
+    if zeros is not None:
+        if tiled:
+            raise ValueError("per-group zero points need the row-major weights")
+        zeros = _zero_points(zeros, scales)
+    A = _aligned_rows(A)
+    _check_matrix(A, "A", torch.float16)
+    _check_matrix(Wq, "Wq", torch.uint8)
+    _check_matrix(scales, "scales", torch.float16)
+    M, K = A.shape
+    N = scales.shape[0] if tiled else Wq.shape[0]
+    if Wq.shape[1] * 2 != K or not Wq.is_contiguous() or (tiled and Wq.shape[0] != (N + 15) // 16 * 16):
+        raise ValueError(f"Wq must be contiguous [N, K/2] (tiled: ceil(N/16)*16 rows); got {tuple(Wq.shape)} for K={K}")
+    if tuple(scales.shape) != (N, K // group) or not scales.is_contiguous():
+        raise ValueError(f"scales must be contiguous [N, K/group]; got {tuple(scales.shape)}")
+    _check_out(C, M, N, torch.float16)
+    if M > Q4_MAX_M and not config.startswith("#"):
+        # the Q4 kernels stream the weights past at most 64 rows of A.  Up to 256 rows: one launch
+        # per block of 64 rows.  Beyond: dequantise once (bit-exact device function) and run the
+        # fp16 tile kernels, whose time then dwarfs the extra pass over the weights.
+        if M <= 4 * Q4_MAX_M:
+            for m0 in range(0, M, Q4_MAX_M):
+                _run_q4(A[m0:m0 + Q4_MAX_M], Wq, scales, zeros, C[m0:m0 + Q4_MAX_M], zero, group, tiled, config,
+                        bias, activation)
+            return
+        if tiled:
+            raise ValueError("more than 256 rows of A need the row-major weights (they are dequantised once)")
+        W = torch.empty((N, K), dtype=torch.float16, device=Wq.device)
+        _run_dequant_q4(Wq, scales, zeros, W, zero, group)
+        _run_16bit(A, W, C, "nt", "", bias, activation, torch.float16, "float16")
+        return
+    name = "q4_zp" if zeros is not None else ("q4_tiled" if tiled else "q4")
+    plan = _plan_for(config, M, N, K, name, "nt")
+    if (plan.dtype == _lib.SK_Q4_TILED) != bool(tiled):
+        raise ValueError("the plan was made for the other weight layout")
+    if (plan.dtype == _lib.SK_Q4_ZP) != (zeros is not None):
+        raise ValueError("the plan was made with / without per-group zero points")
+    epi = _epilogue(bias, N, torch.float16, A.device, _act(activation))
+    tail = _ws_args(plan, A.device)
+    L = _lib.lib()
+    if epi is not None:
+        rc = L.sk_gemm_q4_ex(A.data_ptr(), Wq.data_ptr(), scales.data_ptr(), zeros.data_ptr() if zeros is not None else None,
+                             C.data_ptr(), M, N, K, A.stride(0), C.stride(0), group, zero, *tail, ctypes.byref(epi))
+    elif zeros is not None:
+        rc = L.sk_gemm_q4_zp(A.data_ptr(), Wq.data_ptr(), scales.data_ptr(), zeros.data_ptr(), C.data_ptr(), M, N, K,
+                             A.stride(0), C.stride(0), group, *tail)
+    else:
+        rc = L.sk_gemm_q4(A.data_ptr(), Wq.data_ptr(), scales.data_ptr(), C.data_ptr(), M, N, K, A.stride(0),
+                          C.stride(0), group, zero, *tail)
+    _lib.check(rc, "sk_gemm_q4")
+
+
+def _run_dequant_q4(Wq, scales, zeros, W, zero, group):
+    _check_matrix(Wq, "Wq", torch.uint8)
+    _check_matrix(scales, "scales", torch.float16)
+    N, K = Wq.shape[0], Wq.shape[1] * 2
+    if not Wq.is_contiguous() or not scales.is_contiguous():
+        raise ValueError("Wq and scales must be contiguous")
+    _check_out(W, N, K, torch.float16)
+    if not W.is_contiguous():
+        raise ValueError("the dequantised matrix must be contiguous")
+    if zeros is not None:
+        zeros = _zero_points(zeros, scales)
+        rc = _lib.lib().sk_dequant_q4_zp(Wq.data_ptr(), scales.data_ptr(), zeros.data_ptr(), W.data_ptr(), N, K,
+                                         group, _stream_ptr())
+        _lib.check(rc, "sk_dequant_q4_zp")
+        return
+    rc = _lib.lib().sk_dequant_q4(Wq.data_ptr(), scales.data_ptr(), W.data_ptr(), N, K, group, zero, _stream_ptr())
+    _lib.check(rc, "sk_dequant_q4")
+
+
+# ---------------------------------------------------------------------------------------------
+# Registration with the dispatcher: `torch.ops.streamk.<name>` (functional, allocates C) and
+# `<name>_out` (writes the caller's C).  The functional form's fake implementation is what FakeTensor
+# tracing and torch.compile use in place of the kernel.
+# ---------------------------------------------------------------------------------------------
+_LIBRARY = torch.library.Library("streamk", "DEF")
+_EPI = "Tensor? bias=None, str activation=\"none\""
+
+
+def _register(name, before_out, after_out, run, out_meta):
+    """Defines streamk::<name>(before_out, after_out) -> Tensor and streamk::<name>_out(before_out, out,
+    after_out) -> ().  run(*args) with C at position len(before_out arguments) performs the launch;
+    out_meta(*functional args) -> (shape, dtype) of C."""
+    out_pos = before_out.count("Tensor")
+    _LIBRARY.define(f"{name}({before_out}, {after_out}) -> Tensor")
+    _LIBRARY.define(f"{name}_out({before_out}, Tensor(a!) out, {after_out}) -> ()")
+
+    def functional(*args):
+        shape, dtype = out_meta(*args)
+        C = torch.empty(shape, dtype=dtype, device=args[0].device)
+        run(*args[:out_pos], C, *args[out_pos:])
+        return C
+
+    def functional_fake(*args):
+        shape, dtype = out_meta(*args)
+        return args[0].new_empty(shape, dtype=dtype)
+
+    def out_variant(*args):
+        run(*args)
+
+    _LIBRARY.impl(name, functional, "CUDA")
+    _LIBRARY.impl(f"{name}_out", out_variant, "CUDA")
+    torch.library.register_fake(f"streamk::{name}", functional_fake, lib=_LIBRARY)
+    torch.library.register_fake(f"streamk::{name}_out", lambda *args: None, lib=_LIBRARY)
+
+
+def _mn(A, B, layout):
+    return (A.shape[0], _nk_of(B, layout)[0])
+
+
+_register("gemm_f16", "Tensor A, Tensor B", f"str layout=\"nt\", str config=\"\", {_EPI}",
+          lambda A, B, C, layout="nt", config="", bias=None, activation="none":
+          _run_16bit(A, B, C, layout, config, bias, activation, torch.float16, "float16"),
+          lambda A, B, layout="nt", *rest: (_mn(A, B, layout), torch.float16))
+_register("gemm_bf16", "Tensor A, Tensor B", f"str layout=\"nt\", str config=\"\", {_EPI}",
+          lambda A, B, C, layout="nt", config="", bias=None, activation="none":
+          _run_16bit(A, B, C, layout, config, bias, activation, torch.bfloat16, "bfloat16"),
+          lambda A, B, layout="nt", *rest: (_mn(A, B, layout), torch.bfloat16))
+_register("gemm_f32", "Tensor A, Tensor B", "str layout=\"nn\", str config=\"\"",
+          lambda A, B, C, layout="nn", config="": _run_f32(A, B, C, layout, config),
+          lambda A, B, layout="nn", *rest: (_mn(A, B, layout), torch.float32))
+_register("gemm_f8", "Tensor A, Tensor B", f"float alpha=1.0, str fmt=\"\", str config=\"\", {_EPI}",
+          lambda A, B, C, alpha=1.0, fmt="", config="", bias=None, activation="none":
+          _run_f8(A, B, C, alpha, fmt, config, bias, activation),
+          lambda A, B, *rest: ((A.shape[0], B.shape[0]), torch.float16))
+_register("gemm_i8", "Tensor A, Tensor B", "str config=\"\"",
+          lambda A, B, C, config="": _run_i8(A, B, C, config),
+          lambda A, B, *rest: ((A.shape[0], B.shape[0]), torch.int32))
+_register("gemm_q4", "Tensor A, Tensor Wq, Tensor scales, Tensor? zeros",
+          f"int zero=8, int group=128, bool tiled=False, str config=\"\", {_EPI}",
+          lambda A, Wq, scales, zeros, C, zero=8, group=128, tiled=False, config="", bias=None, activation="none":
+          _run_q4(A, Wq, scales, zeros, C, zero, group, tiled, config, bias, activation),
+          lambda A, Wq, scales, *rest: ((A.shape[0], scales.shape[0]), torch.float16))
+_register("dequant_q4", "Tensor Wq, Tensor scales, Tensor? zeros", "int zero=8, int group=128",
+          lambda Wq, scales, zeros, W, zero=8, group=128: _run_dequant_q4(Wq, scales, zeros, W, zero, group),
+          lambda Wq, scales, *rest: ((Wq.shape[0], Wq.shape[1] * 2), torch.float16))
+
+_ops = torch.ops.streamk
+
+
+# ---------------------------------------------------------------------------------------------
+# The reference-shaped entry points
+# ---------------------------------------------------------------------------------------------
 def streamk_fp16(A, B, *, Wq=None, scales=None, layout="nt", out=None, plan=None, config=None,
                  zero=8, group=128, bias=None, activation=None, **kw):
     """C = A @ B.T (layout 'nt', B is [N,K]) or A @ B (layout 'nn', B is [K,N]) in fp16 with fp32
@@ -86,56 +428,22 @@ def streamk_fp16(A, B, *, Wq=None, scales=None, layout="nt", out=None, plan=None
     if Wq is not None:
         return streamk_q4(A, Wq, scales, out=out, plan=plan, config=config, zero=zero, group=group, bias=bias,
                           activation=activation, **kw)
-    _check_matrix(A, "A", torch.float16)
-    _check_matrix(B, "B", torch.float16)
-    if layout not in ("nt", "nn"):
-        raise ValueError("layout must be 'nt' (B is [N,K]) or 'nn' (B is [K,N])")
-    M, K = A.shape
-    N, Kb = B.shape if layout == "nt" else (B.shape[1], B.shape[0])
-    if K != Kb:
-        raise ValueError(f"K mismatch: A is {tuple(A.shape)}, B is {tuple(B.shape)}")
-    if plan is None:
-        plan = make_plan(M, N, K, "float16", layout, config, **kw)
-    C = out if out is not None else torch.empty((M, N), dtype=torch.float16, device=A.device)
-    _check_matrix(C, "out", torch.float16)
-    if tuple(C.shape) != (M, N):
-        raise ValueError("out has the wrong shape")
-    ws = _workspace(plan.workspace_bytes, A.device)
-    epi = _epilogue(bias, N, torch.float16, A.device, activation)
-    args = (A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, A.stride(0), B.stride(0), C.stride(0),
-            ctypes.byref(plan), ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
-            _stream_ptr())
-    rc = _lib.lib().sk_gemm_f16(*args) if epi is None else _lib.lib().sk_gemm_f16_ex(*args, ctypes.byref(epi))
-    _lib.check(rc, "sk_gemm_f16")
-    return C
+    cfg = _config_string(plan, config, kw)
+    if out is None:
+        return _ops.gemm_f16(A, B, layout, cfg, bias, activation or "none")
+    _ops.gemm_f16_out(A, B, out, layout, cfg, bias, activation or "none")
+    return out
 
 
 def streamk_bf16(A, B, *, layout="nt", out=None, plan=None, config=None, bias=None, activation=None, **kw):
     """streamk_fp16 for bfloat16 operands and output (fp32 accumulation, C rounded to nearest even).
     The reference's scripts are fp16 / fp32 only; this is the bfloat16 instance of the same tile
     kernels."""
-    _check_matrix(A, "A", torch.bfloat16)
-    _check_matrix(B, "B", torch.bfloat16)
-    if layout not in ("nt", "nn"):
-        raise ValueError("layout must be 'nt' (B is [N,K]) or 'nn' (B is [K,N])")
-    M, K = A.shape
-    N, Kb = B.shape if layout == "nt" else (B.shape[1], B.shape[0])
-    if K != Kb:
-        raise ValueError(f"K mismatch: A is {tuple(A.shape)}, B is {tuple(B.shape)}")
-    if plan is None:
-        plan = make_plan(M, N, K, "bfloat16", layout, config, **kw)
-    C = out if out is not None else torch.empty((M, N), dtype=torch.bfloat16, device=A.device)
-    _check_matrix(C, "out", torch.bfloat16)
-    if tuple(C.shape) != (M, N):
-        raise ValueError("out has the wrong shape")
-    ws = _workspace(plan.workspace_bytes, A.device)
-    epi = _epilogue(bias, N, torch.bfloat16, A.device, activation)
-    args = (A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, A.stride(0), B.stride(0), C.stride(0),
-            ctypes.byref(plan), ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
-            _stream_ptr())
-    rc = _lib.lib().sk_gemm_bf16(*args) if epi is None else _lib.lib().sk_gemm_bf16_ex(*args, ctypes.byref(epi))
-    _lib.check(rc, "sk_gemm_bf16")
-    return C
+    cfg = _config_string(plan, config, kw)
+    if out is None:
+        return _ops.gemm_bf16(A, B, layout, cfg, bias, activation or "none")
+    _ops.gemm_bf16_out(A, B, out, layout, cfg, bias, activation or "none")
+    return out
 
 
 def streamk_fp8(A, B, *, alpha=1.0, fmt=None, out=None, plan=None, config=None, bias=None, activation=None, **kw):
@@ -145,66 +453,22 @@ def streamk_fp8(A, B, *, alpha=1.0, fmt=None, out=None, plan=None, config=None, 
     product of the per-tensor scales of a scaled-fp8 caller; bias (fp16 [N]) and activation as for
     streamk_fp16, applied after alpha.  The reference's scripts stop at fp16; this is
     the same partitioner and fix-ups over the fp8 form of the tile kernel."""
-    kinds = {getattr(torch, "float8_e4m3fn", None): "e4m3", getattr(torch, "float8_e5m2", None): "e5m2"}
-    for t, name in ((A, "A"), (B, "B")):
-        if not isinstance(t, torch.Tensor) or (t.dtype != torch.uint8 and t.dtype not in kinds):
-            raise TypeError(f"{name} must be a float8_e4m3fn / float8_e5m2 (or uint8) tensor")
-        _check_matrix(t, name, t.dtype)
-        if t.dtype != torch.uint8:
-            if fmt not in (None, kinds[t.dtype]):
-                raise TypeError("A and B must be in the same fp8 format")
-            fmt = kinds[t.dtype]
-    fmt = fmt or "e4m3"
-    if fmt not in ("e4m3", "e5m2"):
-        raise ValueError("fmt must be 'e4m3' or 'e5m2'")
-    M, K = A.shape
-    N, Kb = B.shape
-    if K != Kb:
-        raise ValueError(f"K mismatch: A is {tuple(A.shape)}, B is {tuple(B.shape)}")
-    if plan is None:
-        plan = make_plan(M, N, K, "float8_" + fmt, "nt", config, **kw)
-    elif plan.dtype != (_lib.SK_F8E5M2 if fmt == "e5m2" else _lib.SK_F8E4M3):
-        raise ValueError("the plan was made for the other fp8 format")
-    C = out if out is not None else torch.empty((M, N), dtype=torch.float16, device=A.device)
-    _check_matrix(C, "out", torch.float16)
-    if tuple(C.shape) != (M, N):
-        raise ValueError("out has the wrong shape")
-    ws = _workspace(plan.workspace_bytes, A.device)
-    epi = _epilogue(bias, N, torch.float16, A.device, activation)
-    args = (A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, A.stride(0), B.stride(0), C.stride(0), float(alpha),
-            ctypes.byref(plan), ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
-            _stream_ptr())
-    rc = _lib.lib().sk_gemm_f8(*args) if epi is None else _lib.lib().sk_gemm_f8_ex(*args, ctypes.byref(epi))
-    _lib.check(rc, "sk_gemm_f8")
-    return C
+    cfg = _config_string(plan, config, kw)
+    if out is None:
+        return _ops.gemm_f8(A, B, float(alpha), fmt or "", cfg, bias, activation or "none")
+    _ops.gemm_f8_out(A, B, out, float(alpha), fmt or "", cfg, bias, activation or "none")
+    return out
 
 
 def streamk_int8(A, B, *, out=None, plan=None, config=None, **kw):
     """C = A @ B.T for int8 operands, A [M,K], B [N,K]; exact int32 accumulation, int32 C (the accumulator
     type the reference's Triton comparator picks for integer inputs, triton.streamk/first_wave.py:123).
     Every schedule and fix-up returns the same bits."""
-    _check_matrix(A, "A", torch.int8)
-    _check_matrix(B, "B", torch.int8)
-    M, K = A.shape
-    N, Kb = B.shape
-    if K != Kb:
-        raise ValueError(f"K mismatch: A is {tuple(A.shape)}, B is {tuple(B.shape)}")
-    if plan is None:
-        plan = make_plan(M, N, K, "int8", "nt", config, **kw)
-    C = out if out is not None else torch.empty((M, N), dtype=torch.int32, device=A.device)
-    _check_matrix(C, "out", torch.int32)
-    if tuple(C.shape) != (M, N):
-        raise ValueError("out has the wrong shape")
-    ws = _workspace(plan.workspace_bytes, A.device)
-    rc = _lib.lib().sk_gemm_i8(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, A.stride(0),
-                               B.stride(0), C.stride(0), ctypes.byref(plan),
-                               ws.data_ptr() if ws is not None else None,
-                               ws.numel() if ws is not None else 0, _stream_ptr())
-    _lib.check(rc, "sk_gemm_i8")
-    return C
-
-
-Q4_MAX_M = 64  # rows of A the Q4 kernels take in one launch
+    cfg = _config_string(plan, config, kw)
+    if out is None:
+        return _ops.gemm_i8(A, B, cfg)
+    _ops.gemm_i8_out(A, B, out, cfg)
+    return out
 
 
 def tile_q4(Wq):
@@ -236,95 +500,22 @@ def untile_q4(tiled, N):
     return Wq
 
 
-def _zero_points(zeros, scales):
-    """Per-group zero points as the library takes them: fp16 [N, K/group] holding integers 0..15.  Integer
-    tensors are converted (an allocation per call: keep them as fp16 to avoid it)."""
-    if zeros.dtype != torch.float16:
-        zeros = zeros.to(torch.float16)
-    _check_matrix(zeros, "zeros", torch.float16)
-    if tuple(zeros.shape) != tuple(scales.shape) or not zeros.is_contiguous():
-        raise ValueError(f"zeros must be contiguous and shaped like scales; got {tuple(zeros.shape)}")
-    return zeros
-
-
 def streamk_q4(A, Wq, scales, *, out=None, plan=None, config=None, zero=8, group=128, tiled=False, zeros=None,
                bias=None, activation=None, **kw):
     """C[M,N] fp16 = A[M,K] fp16 @ dequant(Wq)[N,K].T, weights in natural nibble order
     (streamk_fp16_ladder_block_reduce_q4.py:552).  tiled=True: Wq is the output of tile_q4 (N is
     then taken from scales).  zeros: one zero point per scale group and row ([N, K/group], integers
     0..15) instead of the scalar `zero`.  bias / activation: as for streamk_fp16."""
-    if zeros is not None:
-        if tiled:
-            raise ValueError("per-group zero points need the row-major weights")
-        zeros = _zero_points(zeros, scales)
-    _check_matrix(A, "A", torch.float16)
-    _check_matrix(Wq, "Wq", torch.uint8)
-    _check_matrix(scales, "scales", torch.float16)
-    M, K = A.shape
-    N = scales.shape[0] if tiled else Wq.shape[0]
-    if Wq.shape[1] * 2 != K or not Wq.is_contiguous() or (tiled and Wq.shape[0] != (N + 15) // 16 * 16):
-        raise ValueError(f"Wq must be contiguous [N, K/2] (tiled: ceil(N/16)*16 rows); got {tuple(Wq.shape)} for K={K}")
-    if tuple(scales.shape) != (N, K // group) or not scales.is_contiguous():
-        raise ValueError(f"scales must be contiguous [N, K/group]; got {tuple(scales.shape)}")
-    if plan is not None and (plan.dtype == _lib.SK_Q4_TILED) != bool(tiled):
-        raise ValueError("the plan was made for the other weight layout")
-    if plan is not None and (plan.dtype == _lib.SK_Q4_ZP) != (zeros is not None):
-        raise ValueError("the plan was made with / without per-group zero points")
-    C = out if out is not None else torch.empty((M, N), dtype=torch.float16, device=A.device)
-    _check_matrix(C, "out", torch.float16)
-    if tuple(C.shape) != (M, N):
-        raise ValueError("out has the wrong shape")
-    if plan is None and M > Q4_MAX_M:
-        # the Q4 kernels stream the weights past at most 64 rows of A.  Up to 256 rows: one launch
-        # per block of 64 rows.  Beyond: dequantise once (bit-exact device function) and run the
-        # fp16 tile kernels, whose time then dwarfs the extra pass over the weights.
-        if M <= 4 * Q4_MAX_M:
-            for m0 in range(0, M, Q4_MAX_M):
-                streamk_q4(A[m0:m0 + Q4_MAX_M], Wq, scales, out=C[m0:m0 + Q4_MAX_M], config=config, zero=zero,
-                           group=group, tiled=tiled, zeros=zeros, bias=bias, activation=activation, **kw)
-            return C
-        if tiled:
-            raise ValueError("more than 256 rows of A need the row-major weights (they are dequantised once)")
-        return streamk_fp16(A, dequant_q4(Wq, scales, zero=zero, group=group, zeros=zeros), out=C, bias=bias,
-                            activation=activation)
-    if plan is None:
-        plan = make_plan(M, N, K, "q4_zp" if zeros is not None else ("q4_tiled" if tiled else "q4"), "nt", config, **kw)
-    ws = _workspace(plan.workspace_bytes, A.device)
-    epi = _epilogue(bias, N, torch.float16, A.device, activation)
-    tail = (ctypes.byref(plan), ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
-            _stream_ptr())
-    L = _lib.lib()
-    if epi is not None:
-        rc = L.sk_gemm_q4_ex(A.data_ptr(), Wq.data_ptr(), scales.data_ptr(), zeros.data_ptr() if zeros is not None else None,
-                             C.data_ptr(), M, N, K, A.stride(0), C.stride(0), group, zero, *tail, ctypes.byref(epi))
-    elif zeros is not None:
-        rc = L.sk_gemm_q4_zp(A.data_ptr(), Wq.data_ptr(), scales.data_ptr(), zeros.data_ptr(), C.data_ptr(), M, N, K,
-                             A.stride(0), C.stride(0), group, *tail)
-    else:
-        rc = L.sk_gemm_q4(A.data_ptr(), Wq.data_ptr(), scales.data_ptr(), C.data_ptr(), M, N, K, A.stride(0),
-                          C.stride(0), group, zero, *tail)
-    _lib.check(rc, "sk_gemm_q4")
-    return C
+    cfg = _config_string(plan, config, kw)
+    if out is None:
+        return _ops.gemm_q4(A, Wq, scales, zeros, zero, group, bool(tiled), cfg, bias, activation or "none")
+    _ops.gemm_q4_out(A, Wq, scales, zeros, out, zero, group, bool(tiled), cfg, bias, activation or "none")
+    return out
 
 
 def dequant_q4(Wq, scales, *, zero=8, group=128, zeros=None):
     """fp16 W[N,K] from packed nibbles, by the same device function the Q4 GEMM uses."""
-    _check_matrix(Wq, "Wq", torch.uint8)
-    _check_matrix(scales, "scales", torch.float16)
-    N, K = Wq.shape[0], Wq.shape[1] * 2
-    if not Wq.is_contiguous() or not scales.is_contiguous():
-        raise ValueError("Wq and scales must be contiguous")
-    W = torch.empty((N, K), dtype=torch.float16, device=Wq.device)
-    if zeros is not None:
-        zeros = _zero_points(zeros, scales)
-        rc = _lib.lib().sk_dequant_q4_zp(Wq.data_ptr(), scales.data_ptr(), zeros.data_ptr(), W.data_ptr(), N, K,
-                                         group, _stream_ptr())
-        _lib.check(rc, "sk_dequant_q4_zp")
-        return W
-    rc = _lib.lib().sk_dequant_q4(Wq.data_ptr(), scales.data_ptr(), W.data_ptr(), N, K, group, zero,
-                                  _stream_ptr())
-    _lib.check(rc, "sk_dequant_q4")
-    return W
+    return _ops.dequant_q4(Wq, scales, zeros, zero, group)
 
 
 def pack_q4(q):
@@ -383,25 +574,11 @@ def quantize_q4(W, *, group=128, zero=8, asymmetric=False):
 
 def streamk_fp32(A, B, *, layout="nn", out=None, plan=None, config=None, **kw):
     """C = A @ B in fp32 (layout 'nn', B is [K,N]: streamk_fp32.py:65-76)."""
-    _check_matrix(A, "A", torch.float32)
-    _check_matrix(B, "B", torch.float32)
-    if layout not in ("nt", "nn"):
-        raise ValueError("layout must be 'nn' (B is [K,N]) or 'nt' (B is [N,K])")
-    M, K = A.shape
-    N, Kb = (B.shape[1], B.shape[0]) if layout == "nn" else B.shape
-    if K != Kb:
-        raise ValueError(f"K mismatch: A is {tuple(A.shape)}, B is {tuple(B.shape)}")
-    if plan is None:
-        plan = make_plan(M, N, K, "float32", layout, config, **kw)
-    C = out if out is not None else torch.empty((M, N), dtype=torch.float32, device=A.device)
-    _check_matrix(C, "out", torch.float32)
-    ws = _workspace(plan.workspace_bytes, A.device)
-    rc = _lib.lib().sk_gemm_f32(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, A.stride(0),
-                                B.stride(0), C.stride(0), ctypes.byref(plan),
-                                ws.data_ptr() if ws is not None else None,
-                                ws.numel() if ws is not None else 0, _stream_ptr())
-    _lib.check(rc, "sk_gemm_f32")
-    return C
+    cfg = _config_string(plan, config, kw)
+    if out is None:
+        return _ops.gemm_f32(A, B, layout, cfg)
+    _ops.gemm_f32_out(A, B, out, layout, cfg)
+    return out
 
 
 class StreamKKernel:
@@ -439,6 +616,7 @@ def bench_ms(fn, warmup=25, rep=100):
         fn()
     end.record()
     torch.cuda.synchronize()
+    workspace_status()
     return start.elapsed_time(end) / rep
 
 

@@ -469,7 +469,12 @@ def test_linear_module_matches_functional_linear(sk, oracle):
             assert y.shape == x.shape[:-1] + (1536,) and y.dtype == torch.float16
             ref = xf @ W.T + b
             assert oracle.max_abs_rel(y.float().cpu().numpy().reshape(-1, 1536), ref) <= 2e-3 <= TOL
-    assert set(fp._plans) == {1, 16, 150, 40, 600} and set(q4._plans) == {1, 16, 40} and set(q4.state_dict()) == {"qweight", "scales", "bias"}
+    # the operators keep one plan per (M, N, K, type, layout) they have been called with
+    import sys
+    cache = sys.modules["streamk.ops"]._plan_cache
+    assert {k[0] for k in cache if k[1:5] == (1536, 1024, "float16", "nt")} >= {1, 16, 150, 40, 600}
+    assert {k[0] for k in cache if k[1:5] == (1536, 1024, "q4", "nt")} >= {1, 16, 40}
+    assert set(q4.state_dict()) == {"qweight", "scales", "bias"}
     # state round trip into a freshly constructed module
     fresh = sk.StreamKLinear(1024, 1536, bias=True, weight_format="q4", device="cuda")
     fresh.load_state_dict(q4.state_dict())
@@ -1010,21 +1015,25 @@ def test_one_byte_operands_at_full_size(sk, oracle):
     sk.workspace_status()
 
 
-def test_cfg5_large_dense(sk, oracle):
-    """M = N = K = 8192 and the irregular 3000 x 5120 x 12288, U[-1,1): a random subset of rows is
-    checked against an fp64 host product; the Stream-K and data-parallel schedules of the same kernel
-    must agree within tolerance, and the GEMM must be linear in A."""
+@pytest.mark.parametrize("layout", ["nn", "nt"])
+def test_cfg5_large_dense(sk, oracle, layout):
+    """M = N = K = 8192 and the irregular 3000 x 5120 x 12288, U[-1,1), in the NN layout the large dense
+    configuration names (B is [K,N], streamk.fp16.breakdown/streamk_fp16_nn.py) and in NT: a random subset
+    of rows is checked against an fp64 host product; the Stream-K and data-parallel schedules of the same
+    kernel must agree within tolerance."""
     import torch
     for (M, N, K) in [(8192, 8192, 8192), (3000, 5120, 12288)]:
         A, B = _uniform16((M, K), 5), _uniform16((N, K), 6)
-        dA, dB = _t(A), _t(B)
         rows = np.sort(np.random.default_rng(7).choice(M, 96, replace=False))
         ref = A[rows].astype(np.float64) @ B.astype(np.float64).T
+        if layout == "nn":
+            B = np.ascontiguousarray(B.T)
+        dA, dB = _t(A), _t(B)
         outs = {}
         for name, cfg in [("auto", dict()), ("sk128", dict(bm=128, bn=128, bk=64, schedule="sk2")),
                           ("dp128", dict(bm=128, bn=128, bk=64, schedule="dp")),
                           ("sk256", dict(bm=256, bn=256, bk=64, schedule="sk2", raster=8))]:
-            C = sk.streamk_fp16(dA, dB, **cfg)
+            C = sk.streamk_fp16(dA, dB, layout=layout, **cfg)
             outs[name] = C
             got = C[torch.from_numpy(rows).cuda()].float().cpu().numpy()
             assert oracle.max_abs_rel(got, ref) <= 1e-3 <= TOL, (M, name)
@@ -1033,7 +1042,7 @@ def test_cfg5_large_dense(sk, oracle):
     sk.workspace_status()
 
 
-@pytest.mark.parametrize("shape", [(8192, 8192, 8192), (3000, 5120, 12288), (1024, 1024, 8192),
+@pytest.mark.parametrize("shape", [(8192, 8192, 8192), (8192, 8192, 8192, "nn"), (3000, 5120, 12288), (1024, 1024, 8192),
                                    (16, 8192, 8192)], ids=lambda s: "x".join(map(str, s)))
 def test_full_size_exact_integer_checksums(sk, shape):
     """With entries in {-1, 0, 1} every product and partial sum is an integer far below 2^24 and the
@@ -1042,7 +1051,8 @@ def test_full_size_exact_integer_checksums(sk, shape):
     full benchmark sizes through row and column checksums (C 1 = A (B^T 1), 1^T C = (1^T A) B^T) in
     int64 on the host, plus a block of rows against the full integer product."""
     import torch
-    M, N, K = shape
+    M, N, K = shape[:3]
+    layout = shape[3] if len(shape) > 3 else "nt"   # "nn": B handed over as [K,N] (the large dense configuration)
     rng = np.random.default_rng(11)
     A = rng.integers(-1, 2, (M, K)).astype(np.int8)
     B = rng.integers(-1, 2, (N, K)).astype(np.int8)
@@ -1051,11 +1061,12 @@ def test_full_size_exact_integer_checksums(sk, shape):
     rows = slice(0, min(M, 64))
     block = A[rows].astype(np.int32) @ B.astype(np.int32).T
     assert np.abs(block).max() < 2048
-    dA, dB = _t(A.astype(np.float16)), _t(B.astype(np.float16))
+    dA, dB = _t(A.astype(np.float16)), _t(np.ascontiguousarray(B.T if layout == "nn" else B).astype(np.float16))
     cfgs = [dict(), dict(fixup="atomic"), dict(schedule="basic")]
     if M > 64:
         cfgs += [dict(bm=128, bn=128, bk=64, schedule="sk2", fixup="atomic"),
                  dict(bm=256, bn=256, bk=64, schedule="sk2", raster=8), dict(bm=128, bn=256, bk=64)]
+    cfgs = [dict(c, layout=layout) for c in cfgs]
     for cfg in cfgs:
         C = sk.streamk_fp16(dA, dB, **cfg)
         Cd = C.double()
@@ -1237,6 +1248,51 @@ def test_graph_capture_replays_match_eager(sk, oracle):
     sk.workspace_status()
 
 
+def test_one_workspace_serves_graph_and_eager_launches_of_both_fixups(sk, oracle):
+    """Whether the partial area needs zeroing before an atomic launch is recorded in the workspace, not
+    on the host: an atomic launch captured while the workspace was clean must still be right when an
+    eager reduce launch on the SAME stream and workspace has left partial tiles behind before the
+    replay (and the other way round).  Integer data: the result is exact whatever the order."""
+    import torch
+    rng = np.random.default_rng(78)
+    M, N, K = 512, 1024, 2048
+    A = rng.integers(-1, 2, (M, K)).astype(np.float16)
+    B = rng.integers(-1, 2, (N, K)).astype(np.float16)
+    want = torch.from_numpy((A.astype(np.int32) @ B.astype(np.int32).T).astype(np.float16)).cuda()
+    dA, dB = _t(A), _t(B)
+    red = dict(bm=128, bn=128, bk=64, schedule="basic", fixup="reduce", grid=40)
+    atm = dict(bm=128, bn=128, bk=64, schedule="basic", fixup="atomic", grid=40)
+    c_atm = torch.empty(M, N, dtype=torch.float16, device="cuda")
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        p_red = sk.make_plan(M, N, K, "float16", "nt", red)
+        p_atm = sk.make_plan(M, N, K, "float16", "nt", atm)
+        sk.streamk_fp16(dA, dB, out=c_atm, plan=p_atm)   # creates this stream's workspace; leaves it clean
+        torch.cuda.synchronize()
+        assert torch.equal(c_atm, want)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            sk.streamk_fp16(dA, dB, out=c_atm, plan=p_atm)
+        for replay in range(3):
+            c_atm.zero_()
+            got = sk.streamk_fp16(dA, dB, plan=p_red)    # eager, same stream, same workspace: dirties the partials
+            torch.cuda.synchronize()
+            assert torch.equal(got, want), replay
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(c_atm, want), replay
+            graph.replay()                               # and twice in a row
+            torch.cuda.synchronize()
+            assert torch.equal(c_atm, want), replay
+        # eager atomic after eager reduce, larger tiles than before (other slot sizes)
+        for cfg in (dict(bm=256, bn=256, bk=64, schedule="basic", fixup="reduce", grid=16),
+                    dict(bm=256, bn=256, bk=64, schedule="basic", fixup="atomic", grid=16),
+                    dict(bm=128, bn=128, bk=64, schedule="basic", fixup="atomic", grid=24)):
+            assert torch.equal(sk.streamk_fp16(dA, dB, **cfg), want), cfg
+    torch.cuda.synchronize()
+    sk.workspace_status()
+
+
 def test_strided_operands_and_out(sk, oracle):
     """Leading dimensions larger than the rows, and writing into a caller-provided C."""
     import torch
@@ -1258,6 +1314,10 @@ def test_wait_gives_up_instead_of_hanging(sk):
     sk.streamk_fp16(A, B, bm=128, bn=128, bk=64, schedule="basic", fixup="reduce", grid=256, spin_limit=1)
     with pytest.raises(sk.StreamKError) as e:
         sk.workspace_status()
+    assert e.value.status == -8
+    # flags of the abandoned wait may still be raised: the workspace is refused until it is initialised again
+    with pytest.raises(sk.StreamKError) as e:
+        sk.streamk_fp16(A, B, bm=128, bn=128, bk=64, schedule="basic", fixup="reduce", grid=256)
     assert e.value.status == -8
     sk.reset_workspaces()
     # and the library is usable again afterwards
@@ -1301,6 +1361,12 @@ def test_bad_calls_are_refused(sk):
         sk.streamk_fp16(A, torch.zeros(64, 136, dtype=torch.float16, device="cuda"))
     with pytest.raises(sk.StreamKError):
         sk.streamk_fp16(A[:, :100], A[:, :100])  # K = 100 is not a multiple of 8
+    # an `out` of the wrong shape is refused on the host by every wrapper (the kernel would write past it)
+    A32 = torch.zeros(64, 128, dtype=torch.float32, device="cuda")
+    with pytest.raises(ValueError):
+        sk.streamk_fp32(A32, A32, layout="nt", out=torch.zeros(32, 64, dtype=torch.float32, device="cuda"))
+    with pytest.raises(ValueError):
+        sk.streamk_fp16(A, A, out=torch.zeros(32, 64, dtype=torch.float16, device="cuda"))
 
 
 def test_autotune_search_and_cache(sk, oracle, tmp_path):
