@@ -170,6 +170,24 @@ int sk_gemm_f16(const void *A, const void *B, void *C, int64_t M, int64_t N, int
                 int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws, size_t ws_bytes,
                 void *stream);
 
+/*
+ * sk_gemm_f16 without a workspace argument, for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+ * The partial tiles and flags of the fix-up live in an array that is part of the library's code object: one
+ * copy of SK_STATIC_WORKSPACE_BYTES per GPU, held until the process ends.  The call allocates and frees
+ * nothing; every call is preceded by a small kernel that clears the flags the plan uses (and, for the ATOMIC
+ * fix-up, zero-fills the accumulators if an earlier call left partial tiles there).  A plan whose
+ * sk_workspace_bytes() exceeds SK_STATIC_WORKSPACE_BYTES is refused with SK_ERR_WORKSPACE (the limit covers
+ * every fp16 plan up to 256 partial tiles of 256 x 256, e.g. M = N = K = 8192 with the two-tile Stream-K
+ * schedule on 256 CUs).  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU
+ * (two streams, two threads) race; serialise them.  There is no status word to poll: a fix-up wait that gives
+ * up (spin_limit) leaves its tile incomplete as with sk_gemm_f16, but unreported -- callers that lower
+ * spin_limit should use sk_gemm_f16 with their own workspace.
+ */
+#define SK_STATIC_WORKSPACE_BYTES (64u * 1024u * 1024u + 262144u + 256u)
+int sk_gemm_f16_static(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                       int64_t ldb, int64_t ldc, const sk_plan *plan, void *stream);
+
 /* Optional epilogue of the *_ex entry points (NULL = none): bias points at N device values of C's type
  * (fp16, or bfloat16 for sk_gemm_bf16_ex) that are added to every row of C in fp32 before the rounding --
  * the bias of a linear layer, which the reference leaves to a separate kernel -- or is NULL; activation

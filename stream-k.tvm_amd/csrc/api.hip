@@ -77,6 +77,50 @@ struct WsInfo {
 };
 std::unordered_map<const void *, WsInfo> g_ws;
 
+// Workspace of sk_gemm_f16_static, for callers that must not allocate: one array per device, part of
+// the code object (zero-filled when the module is loaded), laid out like a caller's workspace.  In host
+// code its name is only a handle: the address kernels are given comes from hipGetSymbolAddress, once
+// per device, and is kept in g_scratch_ptr.
+static __device__ __align__(256) unsigned char scratch[SK_STATIC_WORKSPACE_BYTES];
+void *g_scratch_ptr[16];
+
+int static_scratch(void **ptr) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return SK_ERR_DEVICE;
+  std::lock_guard<std::mutex> lock(g_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void *p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return SK_ERR_DEVICE;
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return SK_OK;
+}
+
+// Runs in front of every launch on the static workspace, whose contents are whatever the previous call
+// left: clears the status word and the flags / counters the plan uses (an abandoned wait of an earlier
+// call may have left some raised) and, for an ATOMIC plan, zero-fills the partial area as far as it is
+// marked dirty (see clean_partials_kernel).
+__global__ void prepare_static_kernel(int *status, int *flags, int nflags, uint4v *partials, unsigned capacity_units,
+                                      int atomic) {
+  const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x, stride = (size_t)gridDim.x * blockDim.x;
+  if (tid == 0) status[WS_STATUS] = 0;
+  for (size_t i = tid; i < (size_t)nflags; i += stride) flags[i] = 0;
+  if (!atomic) return;
+  const unsigned mark = (unsigned)__hip_atomic_load(status + WS_DIRTY, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (mark == 0) return;
+  const size_t n16 = (size_t)(mark < capacity_units ? mark : capacity_units) * 16;
+  for (size_t i = tid; i < n16; i += stride) partials[i] = uint4v{0, 0, 0, 0};
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const int done = __hip_atomic_fetch_add(status + WS_CLEAN_DONE, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (done == (int)gridDim.x - 1) {
+      __hip_atomic_store(status + WS_CLEAN_DONE, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (mark <= capacity_units) __hip_atomic_store(status + WS_DIRTY, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+}
+
 int check_plan(const sk_plan *plan, int64_t M, int64_t N, int64_t K, int dtype, int layout) {
   if (!plan) return SK_ERR_NULL;
   if (plan->M != M || plan->N != N || plan->K != K || plan->dtype != dtype || plan->layout != layout)
@@ -84,8 +128,9 @@ int check_plan(const sk_plan *plan, int64_t M, int64_t N, int64_t K, int dtype, 
   return SK_OK;
 }
 
+// is_static: ws is the library's own static workspace (no registry entry; prepared by its own kernel)
 int make_dev_plan(const sk_plan *plan, const KernelInfo *k, void *ws, size_t ws_bytes, int occupancy,
-                  hipStream_t stream, DevPlan *dp, Workspace *w) {
+                  hipStream_t stream, DevPlan *dp, Workspace *w, bool is_static = false) {
   if ((size_t)plan->workspace_bytes > ws_bytes) return SK_ERR_WORKSPACE;
   if (plan->workspace_bytes > 0 && !ws) return SK_ERR_WORKSPACE;
   if (plan->workspace_bytes > 0 && (reinterpret_cast<uintptr_t>(ws) & 255)) return SK_ERR_ALIGN;
@@ -95,7 +140,15 @@ int make_dev_plan(const sk_plan *plan, const KernelInfo *k, void *ws, size_t ws_
   if (plan->streamk_tiles > 0 && plan->fixup == SK_FIXUP_REDUCE &&
       (occupancy <= 0 || plan->grid > d.cus * occupancy))
     return SK_ERR_CONFIG;
-  if (plan->workspace_bytes > 0) {
+  if (plan->workspace_bytes > 0 && is_static) {
+    char *base = static_cast<char *>(ws);
+    const int nflags = plan->fixup == SK_FIXUP_REDUCE ? plan->grid : plan->streamk_tiles;
+    const size_t units = (ws_bytes - (size_t)WS_PART_OFF) / 256;
+    hipLaunchKernelGGL(prepare_static_kernel, dim3(1024), dim3(256), 0, stream, reinterpret_cast<int *>(base),
+                       reinterpret_cast<int *>(base + 256), nflags, reinterpret_cast<uint4v *>(base + WS_PART_OFF),
+                       (unsigned)units, plan->fixup == SK_FIXUP_ATOMIC ? 1 : 0);
+    if (hipGetLastError() != hipSuccess) return SK_ERR_LAUNCH;
+  } else if (plan->workspace_bytes > 0) {
     {
       std::lock_guard<std::mutex> lock(g_mutex);
       auto it = g_ws.find(ws);
@@ -237,7 +290,7 @@ static int epilogue_word(const sk_epilogue *epi, const void **word) {
 
 static int gemm_16bit(int dtype, const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,
                       int64_t lda, int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws,
-                      size_t ws_bytes, void *stream, const sk_epilogue *epi = nullptr) {
+                      size_t ws_bytes, void *stream, const sk_epilogue *epi = nullptr, bool is_static = false) {
   const void *bias = nullptr;  // the kernels' epilogue word: bias pointer and activation code
   if (int rc = epilogue_word(epi, &bias)) return rc;
   if (!A || !B || !C) return SK_ERR_NULL;
@@ -256,7 +309,8 @@ static int gemm_16bit(int dtype, const void *A, const void *B, void *C, int64_t 
   DevPlan dp;
   Workspace w;
   const bool skinny = k->family == FAMILY_SKINNY;
-  rc = make_dev_plan(plan, k, ws, ws_bytes, cached_occupancy(k->id, skinny ? 1 : 0), (hipStream_t)stream, &dp, &w);
+  rc = make_dev_plan(plan, k, ws, ws_bytes, cached_occupancy(k->id, skinny ? 1 : 0), (hipStream_t)stream, &dp, &w,
+                     is_static);
   if (rc) return rc;
   int herr;
   if (skinny) {
@@ -273,6 +327,17 @@ extern "C" int sk_gemm_f16(const void *A, const void *B, void *C, int64_t M, int
                            int64_t lda, int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws,
                            size_t ws_bytes, void *stream) {
   return gemm_16bit(SK_F16, A, B, C, M, N, K, lda, ldb, ldc, plan, ws, ws_bytes, stream);
+}
+
+extern "C" int sk_gemm_f16_static(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,
+                                  int64_t lda, int64_t ldb, int64_t ldc, const sk_plan *plan, void *stream) {
+  if (!plan) return SK_ERR_NULL;
+  if ((uint64_t)plan->workspace_bytes > (uint64_t)SK_STATIC_WORKSPACE_BYTES) return SK_ERR_WORKSPACE;
+  void *ws = nullptr;
+  if (plan->workspace_bytes > 0)
+    if (int rc = static_scratch(&ws)) return rc;
+  return gemm_16bit(SK_F16, A, B, C, M, N, K, lda, ldb, ldc, plan, ws, ws ? (size_t)SK_STATIC_WORKSPACE_BYTES : 0, stream,
+                    nullptr, true);
 }
 
 extern "C" int sk_gemm_f16_ex(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,
