@@ -170,8 +170,27 @@ def main():
             for _ in range(reps):
                 oracle.matmul_fp32(Ah, Bn, trans_b=True)
             dt = (time.perf_counter() - t0) / reps
+        # what the product actually ran on: the BLAS numpy is linked against reports its own thread count; the
+        # process may be confined to fewer logical CPUs than the box has
+        affinity = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else os.cpu_count()
+        blas_threads, blas_name = None, None
+        try:
+            from threadpoolctl import threadpool_info
+            for pool in threadpool_info():
+                if pool.get("user_api") == "blas":
+                    blas_threads, blas_name = pool.get("num_threads"), pool.get("internal_api")
+        except Exception:
+            pass
+        cpu_model = None
+        try:
+            with open("/proc/cpuinfo") as f:
+                cpu_model = next((ln.split(":", 1)[1].strip() for ln in f if ln.startswith("model name")), None)
+        except OSError:
+            pass
         out["cpu_baseline"] = {"value": round(2.0 * rows * N * K / dt / 1e12, 4), "unit": "TFLOP/s",
-                               "cores": os.cpu_count(), "kind": "port",
+                               "cores": blas_threads or affinity, "kind": "port",
+                               "blas": blas_name, "blas_threads": blas_threads, "cpus_in_affinity_mask": affinity,
+                               "logical_cpus": os.cpu_count(), "cpu_model": cpu_model,
                                "sample": f"oracle fp32 host matmul (numpy) of the first {rows} rows of the "
                                          f"same A against all of B ({rows}x{N}x{K}), {reps} x {dt:.2f} s"}
 
@@ -212,7 +231,28 @@ def main():
             best = max(v for k, v in row.items() if k != "M" and not isinstance(v, str))
             row["best_tflops"] = best
             row["pct_fp16_peak"] = round(100 * best / PEAK_FP16_TFLOPS, 2)
-            row["gbs"] = round(best * 1e3 * (2.0 * (m * K + N * K + m * N)) / (2.0 * m * N * K), 1)
+            nbytes = 2.0 * (m * K + N * K + m * N)
+            if m <= 64:
+                # one 134 MB B launched repeatedly is served by the 256 MB Infinity Cache: that rate is not an HBM
+                # rate.  The HBM figure rotates the launches of a batch over copies of B totalling > 512 MB.
+                row["gbs_weights_in_infinity_cache"] = round(best * 1e3 * nbytes / (2.0 * m * N * K), 1)
+                copies = [B] + [B.clone() for _ in range(4)]
+                turn = [0]
+                p = streamk.make_plan(m, N, K, "float16", "nt")
+
+                def rotating():
+                    w = copies[turn[0] % len(copies)]
+                    turn[0] += 1
+                    streamk.streamk_fp16(a, w, out=c, plan=p)
+                ms = time_graph(rotating)
+                del copies
+                row["auto_weights_from_hbm_us"] = round(ms * 1e3, 2)
+                row["gbs"] = round(nbytes / ms / 1e6, 1)
+                row["gbs_is"] = "weights from HBM (launches rotate over 5 copies of B, 671 MB)"
+                row["frac_hbm"] = round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)
+            else:
+                row["gbs"] = round(best * 1e3 * nbytes / (2.0 * m * N * K), 1)
+                row["gbs_is"] = "algorithmic bytes over time; compute-bound row, operands stay in the Infinity Cache"
             if m > 64:
                 row["sk_over_dp_same_tile"] = round(max(row["sk_" + t] / row["dp_" + t] for t in tiles), 3)
             sweep.append(row)
@@ -304,7 +344,13 @@ def main():
             for name, cfg in {"tuned": dict(),
                               "streamk_reduce": dict(schedule="sk2", fixup="reduce", grid=256),
                               "streamk_atomic": dict(schedule="sk2", fixup="atomic", grid=256),
-                              "dp": dict(schedule="dp")}.items():
+                              "dp": dict(schedule="dp"),
+                              # M = 1: `tuned` is a matrix-vector kernel, which multiplies the unrounded
+                              # (q - zero) * scale; this is the fastest instance that forms the fp16-rounded
+                              # weights of the dequantisation contract bit for bit (all kernels do for M > 1)
+                              "rounded_weights": dict(variant=2, schedule="dp")}.items():
+                if name == "rounded_weights" and m != 1:
+                    continue
                 p = streamk.make_plan(m, N, K, "q4", "nt", **cfg)
                 ms = time_graph(lambda: streamk.streamk_q4(a, Wq, sc, out=c, plan=p))
                 row[name] = {"us": round(ms * 1e3, 2), "gbs": round(nbytes / ms / 1e6, 1),
@@ -323,6 +369,10 @@ def main():
                 ms = time_graph(cold)
                 row["tuned_weights_from_hbm"] = {"us": round(ms * 1e3, 2), "gbs": round(nbytes / ms / 1e6, 1),
                                                  "frac_hbm": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
+                p_cold = streamk.make_plan(m, N, K, "q4", "nt", variant=2, schedule="dp")
+                ms = time_graph(cold)
+                row["rounded_weights_from_hbm"] = {"us": round(ms * 1e3, 2), "gbs": round(nbytes / ms / 1e6, 1),
+                                                   "frac_hbm": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
                 # the same with the weights in the tiled layout (one contiguous KB per load instruction)
                 tiles = [(streamk.tile_q4(w), s_) for (w, s_) in copies]
                 del copies

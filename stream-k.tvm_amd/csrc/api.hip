@@ -177,6 +177,9 @@ int make_dev_plan(const sk_plan *plan, const KernelInfo *k, void *ws, size_t ws_
   dp->xcd_remap = (plan->grid % 8 == 0) ? 1 : 0;
   const int raster = plan->raster > 0 ? plan->raster : 1;
   dp->raster_tail = plan->num_block_m % raster ? plan->num_block_m % raster : raster;
+  // every Stream-K tile cut into exactly two equal CTA segments: both CTAs of a pair finish half a tile
+  dp->halves = (plan->fixup == SK_FIXUP_REDUCE && plan->streamk_tiles > 0 && plan->streamk_partial_tiles == 0 &&
+                2 * plan->streamk_full_tiles == plan->iters_per_tile) ? 1 : 0;
   dp->by_ipt = FastDiv::make(plan->iters_per_tile);
   dp->by_tiles_n = FastDiv::make(plan->num_block_n);
   dp->by_width = FastDiv::make((uint32_t)raster * plan->num_block_n);

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace sk {
 
 typedef _Float16 half_t;
@@ -49,6 +51,17 @@ struct FastDiv {
   }
 };
 
+// A loop over [I0, I1) whose counter is a compile-time constant inside the body (f receives
+// std::integral_constant<int, I>).  For loops that index the accumulator arrays and are too large for
+// the unroller's size limit: a dynamic index would keep the accumulators in scratch memory.
+template <int I0, int I1, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+  if constexpr (I0 < I1) {
+    f(std::integral_constant<int, I0>{});
+    static_for<I0 + 1, I1>(f);
+  }
+}
+
 struct DevPlan {
   int tiles_m, tiles_n, ipt;  // tile grid, K-iterations per tile
   int total_tiles, sk_tiles;  // Stream-K tiles are ids [0, sk_tiles)
@@ -59,6 +72,7 @@ struct DevPlan {
   int spin_limit;             // polls before a waiting owner gives up
   int xcd_remap;              // 1: spread logical CTA ids so each XCD owns a contiguous range
   int raster_tail;            // tile rows in the last raster group (tiles_m % raster, or raster)
+  int halves;                 // 1: REDUCE plan whose every Stream-K tile is cut into two equal CTA segments
   FastDiv by_ipt, by_tiles_n, by_width, by_raster, by_tail, by_full1, by_full;
 };
 
@@ -223,6 +237,17 @@ __device__ __forceinline__ uint4v buffer_load_16(BufferRsrc r, uint32_t lane_off
   return __builtin_bit_cast(uint4v, __builtin_amdgcn_raw_buffer_load_b128(r, lane_off, uniform_off, 0));
 }
 constexpr uint32_t OOB_OFFSET = 0x80000000u;
+
+// 16-byte accesses of device scope (the sc1 bit: stores write through to memory, loads never return
+// a line another XCD's L2 has since overwritten) -- the full-width form of st_coherent / ld_coherent
+// for partial tiles of hundreds of KB.  off = per-lane byte offset, uoff = wave-uniform byte offset.
+constexpr int CACHE_POLICY_SC1 = 16;
+__device__ __forceinline__ void st_coherent16(BufferRsrc r, uint32_t off, uint32_t uoff, uint4v v) {
+  __builtin_amdgcn_raw_buffer_store_b128(v, r, off, uoff, CACHE_POLICY_SC1);
+}
+__device__ __forceinline__ uint4v ld_coherent16(BufferRsrc r, uint32_t off, uint32_t uoff) {
+  return __builtin_bit_cast(uint4v, __builtin_amdgcn_raw_buffer_load_b128(r, off, uoff, CACHE_POLICY_SC1));
+}
 
 // Direct global -> LDS load, 16 bytes per lane: lane l's data lands at lds_base + 16*l.  Issued as
 // inline assembly on purpose: the compiler's wait-count insertion cannot tell which LDS stage an

@@ -9,9 +9,23 @@
 // Control flow follows the reference's persistent kernel: every CTA first walks its share of the
 // Stream-K iteration space (streamk_fp32.py:93-136), then its data-parallel tiles (:149-158).
 #pragma once
+#include <type_traits>
+
 #include "sk_device.h"
 
 namespace sk {
+
+// optional members of a policy: COHERENT_REDUCE (partials of the REDUCE fix-up travel with device-scope
+// accesses; default: as COHERENT_PARTIALS says) and HALVES (the policy has store_partial_half /
+// add_partial_half / store_c_half, see below)
+template <class P, class = void>
+struct reduce_is_coherent { static constexpr bool value = P::COHERENT_PARTIALS; };
+template <class P>
+struct reduce_is_coherent<P, std::void_t<decltype(P::COHERENT_REDUCE)>> { static constexpr bool value = P::COHERENT_REDUCE; };
+template <class P, class = void>
+struct has_halves { static constexpr bool value = false; };
+template <class P>
+struct has_halves<P, std::void_t<decltype(P::HALVES)>> { static constexpr bool value = P::HALVES; };
 
 // FIXUP = false: an instance for launches without Stream-K tiles.  Every segment is a whole tile
 // and the fix-up code is not compiled in -- its hundreds of partial-tile addresses otherwise
@@ -91,16 +105,36 @@ __device__ __forceinline__ void run_persistent(const typename P::Args &a, const 
           if (threadIdx.x == 0)
             __hip_atomic_store(&ws.flags[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
+      } else if (has_halves<P>::value && plan.halves) {
+        // Every Stream-K tile of this plan is shared by exactly two CTAs, each with this one segment.
+        // Instead of one of them finishing the whole tile while the other idles, each finishes half of
+        // it: it parks the other half of its accumulators in its slot, raises its flag, waits for the
+        // peer's, adds the peer's contribution to the half it kept and stores that half of C.  The
+        // exchange moves the same bytes as the owner scheme, but over twice as many CTAs at once, and
+        // the sum of two terms does not depend on their order.
+        if constexpr (has_halves<P>::value) {
+          const int half = k0 != 0 ? 1 : 0, peer = k0 != 0 ? pid - 1 : pid + 1;
+          P::store_partial_half(acc, ws.partials + (size_t)pid * P::TILE_ELEMS, 1 - half);
+          signal_partial_ready<true>(&ws.flags[pid], ws.status + WS_DIRTY,
+                                     (int)(((size_t)(pid + 1) * P::TILE_ELEMS * 4 + 255) >> 8));
+          if (!wait_partials_ready<true>(&ws.flags[peer], 1, plan.spin_limit)) {
+            if (threadIdx.x == 0) ws.status[WS_STATUS] = -8;  // SK_ERR_TIMEOUT
+          } else {
+            P::add_partial_half(acc, ws.partials + (size_t)peer * P::TILE_ELEMS, half);
+            clear_flags_after_use(&ws.flags[peer], 1);
+          }
+          P::store_c_half(a, acc, pm, pn, smem, bias, half);
+        }
       } else if (k0 != 0) {
         // not the tile's first CTA: park the partial in this CTA's slot and raise its flag
         P::store_partial(acc, ws.partials + (size_t)pid * P::TILE_ELEMS);
-        signal_partial_ready<P::COHERENT_PARTIALS>(
+        signal_partial_ready<reduce_is_coherent<P>::value>(
             &ws.flags[pid], ws.status + WS_DIRTY, (int)(((size_t)(pid + 1) * P::TILE_ELEMS * 4 + 255) >> 8));
       } else {
         // tile's first CTA: wait for all followers at once, then add their partials in ascending
         // CTA order and store
         const int npeers = sk_pid_of_iter(plan, (tile + 1) * ipt - 1) - pid;
-        if (!wait_partials_ready<P::COHERENT_PARTIALS>(&ws.flags[pid + 1], npeers, plan.spin_limit)) {
+        if (!wait_partials_ready<reduce_is_coherent<P>::value>(&ws.flags[pid + 1], npeers, plan.spin_limit)) {
           if (threadIdx.x == 0) ws.status[WS_STATUS] = -8;  // SK_ERR_TIMEOUT
         } else {
           for (int p = 1; p <= npeers; ++p) P::add_partial(acc, ws.partials + (size_t)(pid + p) * P::TILE_ELEMS);

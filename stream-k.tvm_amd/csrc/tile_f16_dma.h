@@ -619,13 +619,31 @@ struct TileF16NTDma {
   static __device__ __forceinline__ void store_c(const Args &a, const Acc &acc, int pm, int pn, char *smem,
                                                  const void *bias) {
     if (bias == nullptr)
-      store_c_impl<false>(a, acc, pm, pn, smem, nullptr);
+      store_c_impl<false, -1>(a, acc, pm, pn, smem, nullptr);
     else
-      store_c_impl<true>(a, acc, pm, pn, smem, bias);
+      store_c_impl<true, -1>(a, acc, pm, pn, smem, bias);
   }
-  template <bool BIAS>
+  // Half h of the tile, in the sense of the halves fix-up: the rows of every wave's block that live in the
+  // first (h = 0) or second (h = 1) half of that wave's accumulators.
+  static __device__ __forceinline__ void store_c_half(const Args &a, const Acc &acc, int pm, int pn, char *smem,
+                                                      const void *bias, int h) {
+    if constexpr (HALVES) {
+      if (bias == nullptr) {
+        if (h == 0) store_c_impl<false, 0>(a, acc, pm, pn, smem, nullptr);
+        else store_c_impl<false, 1>(a, acc, pm, pn, smem, nullptr);
+      } else {
+        if (h == 0) store_c_impl<true, 0>(a, acc, pm, pn, smem, bias);
+        else store_c_impl<true, 1>(a, acc, pm, pn, smem, bias);
+      }
+    }
+  }
+  // HALF < 0: the whole tile; 0 / 1: rows [HALF * WTM / 2, (HALF + 1) * WTM / 2) of every wave's block
+  template <bool BIAS, int HALF>
   static __device__ __forceinline__ void store_c_impl(const Args &a, const Acc &acc, int pm, int pn, char *,
                                                       const void *epi) {
+    constexpr int ROW_BEGIN = HALF < 0 ? 0 : HALF * (WTM / 2), NROWS = HALF < 0 ? WTM : WTM / 2;
+    constexpr int PR = PATCH_ROWS < NROWS ? PATCH_ROWS : NROWS;  // rows of the wave's block per pass
+    constexpr int NPASS = NROWS / PR;
     const half_t *bias = BIAS ? epi_bias(epi) : nullptr;
     const int act = BIAS ? epi_act(epi) : 0;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -637,7 +655,7 @@ struct TileF16NTDma {
       const bool vec_ok = (a.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(a.C) & 15) == 0);
       const int row0 = pm * BM + wm * WTM + (lane & 15), col0 = pn * BN + wn * WTN + 4 * (lane >> 4);
 #pragma unroll
-      for (int ii = 0; ii < FM; ++ii)
+      for (int ii = ROW_BEGIN / 16; ii < (ROW_BEGIN + NROWS) / 16; ++ii)
 #pragma unroll
         for (int jj = 0; jj < FN; ++jj) {
           const int grow = row0 + 16 * ii, gcol = col0 + 16 * jj;
@@ -659,13 +677,14 @@ struct TileF16NTDma {
                     (wave % WAVES_PER_STAGE) * (PATCH_ROWS * LDC);
     const bool vec_ok = (a.ldc % 8 == 0) && ((reinterpret_cast<uintptr_t>(a.C) & 15) == 0);
     constexpr int CPRC = WTN / 8;
-    constexpr int BLK = PATCH_ROWS / 32;  // 32-row blocks per pass
-#pragma unroll
-    for (int p = 0; p < PASSES; ++p) {
+    constexpr int BLK = PR / 32;  // 32-row blocks per pass
+    static_assert(MFMA16 ? PR % 16 == 0 : PR % 32 == 0, "an epilogue pass holds whole accumulator blocks");
+    static_for<0, NPASS>([&](auto pass) {
+      constexpr int p = decltype(pass)::value;
       if constexpr (I8) {
       } else if constexpr (MFMA16) {
 #pragma unroll
-        for (int ib = 0; ib < PATCH_ROWS / 16; ++ib)
+        for (int ib = 0; ib < PR / 16; ++ib)
 #pragma unroll
           for (int j = 0; j < FN; ++j) {
             half4v h;
@@ -673,7 +692,7 @@ struct TileF16NTDma {
             if constexpr (BIAS) bv = bias4_at<BF16_>(bias, bias_col0 + j * 16, a.N);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-              float x = acc.v[p * (PATCH_ROWS / 16) + ib][j][e];
+              float x = acc.v[ROW_BEGIN / 16 + p * (PR / 16) + ib][j][e];
               if constexpr (BIAS) x = activate(x + bv[e], act);
               if constexpr (BF16_) {
                 const __bf16 b = (__bf16)x;
@@ -696,7 +715,7 @@ struct TileF16NTDma {
               if constexpr (BIAS) bv = bias4_at(bias, bias_col0 + j * 32 + q * 8, a.N);
 #pragma unroll
               for (int e = 0; e < 4; ++e) {
-                float x = acc.c[p * BLK + ib][j][q * 4 + e];
+                float x = acc.c[ROW_BEGIN / 32 + p * BLK + ib][j][q * 4 + e];
                 if constexpr (F8 != 0) x *= a.alpha;  // the product of fp8 operands is scaled before it is rounded to fp16
                 if constexpr (BIAS) x = activate(x + bv[e], act);
                 h[e] = (half_t)x;
@@ -708,9 +727,9 @@ struct TileF16NTDma {
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      const int row0 = pm * BM + wm * WTM + p * PATCH_ROWS, col0 = pn * BN + wn * WTN;
+      const int row0 = pm * BM + wm * WTM + ROW_BEGIN + p * PR, col0 = pn * BN + wn * WTN;
 #pragma unroll
-      for (int s = 0; s < PATCH_ROWS * CPRC / 64; ++s) {
+      for (int s = 0; s < PR * CPRC / 64; ++s) {
         const int idx = s * 64 + lane;
         const int r = idx / CPRC, cc = idx % CPRC;
         const int grow = row0 + r, gcol = col0 + cc * 8;
@@ -727,34 +746,64 @@ struct TileF16NTDma {
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    }
+    });
     __syncthreads();  // patches overlap the stages of the next tile
   }
 
   static constexpr bool COHERENT_PARTIALS = false;
+  // The 16x16x32 forms exchange the partial tiles of the REDUCE fix-up with 16-byte device-scope accesses:
+  // stores write through, loads bypass stale lines, and no CTA pays a write-back or invalidate of its XCD's
+  // whole L2 (which, with 16 CTAs per XCD finishing at the same moment, cost more than the exchange itself).
+  static constexpr bool COHERENT_REDUCE = MFMA16_;
+  // both CTAs of a tile cut in two finish half of it each (see run_persistent); needs accumulator blocks of
+  // 16 rows and at least two of them per wave
+  static constexpr bool HALVES = MFMA16_ && FM % 2 == 0;
   // partials in the workspace: float4 group v of thread t at (v * NT + t) * 4 (ordered reduce),
   // element s of thread t at s * NT + t (atomic accumulation buffer); see tile_f16.h
+  template <int V0, int V1>
+  static __device__ __forceinline__ void store_groups(const Acc &acc, float *dst) {
+    if constexpr (MFMA16) {
+      const BufferRsrc r = make_rsrc(dst, TILE_ELEMS * 4);
+      const uint32_t off = (uint32_t)pin_here((int)threadIdx.x) * 16;
+#pragma unroll
+      for (int v = V0; v < V1; ++v)
+        st_coherent16(r, off, (uint32_t)v * NT * 16, __builtin_bit_cast(uint4v, acc.v[v / FN][v % FN]));
+    }
+  }
+  template <int V0, int V1>
+  static __device__ __forceinline__ void add_groups(Acc &acc, const float *src) {
+    if constexpr (MFMA16) {
+      const BufferRsrc r = make_rsrc(src, TILE_ELEMS * 4);
+      const uint32_t off = (uint32_t)pin_here((int)threadIdx.x) * 16;
+#pragma unroll
+      for (int v = V0; v < V1; ++v) {
+        acc.v[v / FN][v % FN] += __builtin_bit_cast(AccV, ld_coherent16(r, off, (uint32_t)v * NT * 16));
+        if (v % 8 == 7) asm volatile("" ::: "memory");  // at most 8 loads in flight
+      }
+    }
+  }
   static __device__ __forceinline__ void store_partial(const Acc &acc, float *dst) {
     if constexpr (MFMA16) {
-      dst = pin_here(dst);
-#pragma unroll
-      for (int v = 0; v < NV4; ++v)
-        *reinterpret_cast<AccV *>(dst + ((size_t)v * NT + threadIdx.x) * 4) = acc.v[v / FN][v % FN];
+      store_groups<0, NV4>(acc, dst);
     } else {
       Base::store_partial(acc, dst);
     }
   }
   static __device__ __forceinline__ void add_partial(Acc &acc, const float *src) {
     if constexpr (MFMA16) {
-      src = pin_here(src);
-#pragma unroll
-      for (int v = 0; v < NV4; ++v) {
-        acc.v[v / FN][v % FN] += *reinterpret_cast<const AccV *>(src + ((size_t)v * NT + threadIdx.x) * 4);
-        if (v % 8 == 7) asm volatile("" ::: "memory");  // at most 8 loads in flight
-      }
+      add_groups<0, NV4>(acc, src);
     } else {
       Base::add_partial(acc, src);
     }
+  }
+  // half h of the accumulators: blocks [h * FM / 2, (h + 1) * FM / 2), i.e. groups [h * NV4 / 2, (h + 1) * NV4 / 2)
+  static __device__ __forceinline__ void store_partial_half(const Acc &acc, float *dst, int h) {
+    if (h == 0) store_groups<0, NV4 / 2>(acc, dst);
+    else store_groups<NV4 / 2, NV4>(acc, dst);
+  }
+  static __device__ __forceinline__ void add_partial_half(Acc &acc, const float *src, int h) {
+    if (h == 0) add_groups<0, NV4 / 2>(acc, src);
+    else add_groups<NV4 / 2, NV4>(acc, src);
   }
   static __device__ __forceinline__ void atomic_partial(const Acc &acc, float *dst) {
     if constexpr (MFMA16) {

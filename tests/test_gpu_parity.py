@@ -376,6 +376,42 @@ def test_q4_matrix_vector_exact_on_integer_data(sk):
     sk.workspace_status()
 
 
+def test_q4_matrix_vector_deviation_from_rounded_weights_is_bounded(sk, oracle):
+    """The M = 1 matrix-vector kernels multiply the unrounded (q - zero) * scale instead of the fp16-rounded
+    weights the other kernels (and sk_dequant_q4) form.  Per output that moves the result by at most
+    sum_k |a_k| |w_exact - w_rounded| <= 2^-11 sum_k |a_k w_k|, plus the rounding of C to fp16 (2^-11 |c|) and fp32
+    accumulation noise; and the result is the fp16 rounding of the exact (unrounded-weight) product up to that
+    noise.  Checked at N = K = 8192 on the benchmark's data for every matrix-vector instance, beside the
+    instances that form the rounded weights bit for bit (which meet the rounded-weight product itself)."""
+    N = K = 8192
+    rng = np.random.default_rng(41)
+    A = rng.standard_normal((1, K), dtype=np.float32).astype(np.float16)
+    Wq = rng.integers(0, 256, (N, K // 2), dtype=np.uint8)
+    sc = rng.uniform(0.005, 0.02, (N, K // 128)).astype(np.float16)
+    a64 = A[0].astype(np.float64)
+    w_rounded = oracle.dequant_q4(Wq, sc, 128, 8).astype(np.float64)
+    w_exact = (oracle.unpack_q4_np(Wq).astype(np.float64) - 8.0) * np.repeat(sc.astype(np.float64), 128, axis=1)
+    assert np.abs(w_exact - w_rounded).max() <= 2.0 ** -11 * np.abs(w_exact).max()   # per-weight premise
+    y_rounded, y_exact = w_rounded @ a64, w_exact @ a64
+    mass = np.abs(w_exact) @ np.abs(a64)          # sum_k |a_k w_k| per output
+    noise = 2e-5 * mass                           # fp32 accumulation over 8192 terms (25 times below the 2^-11 term)
+    dA, dW, dS = _t(A), _t(Wq), _t(sc)
+    ran = 0
+    for (bm, bn, bk) in Q4_TILES[:8]:
+        for variant, rounded in ((3, False), (2, True), (1, True)):
+            try:
+                plan = sk.make_plan(1, N, K, "q4", "nt", dict(bm=bm, bn=bn, bk=bk, variant=variant, schedule="dp"))
+            except sk.StreamKError:
+                continue
+            y = sk.streamk_q4(dA, dW, dS, plan=plan).double().cpu().numpy()[0]
+            assert np.all(np.abs(y - y_rounded) <= 2.0 ** -11 * mass + 2.0 ** -11 * np.abs(y_rounded) + noise), (bm, bn, bk, variant)
+            target = y_rounded if rounded else y_exact
+            assert np.all(np.abs(y - target) <= 2.0 ** -11 * np.abs(target) + 2.0 ** -24 + noise), (bm, bn, bk, variant)
+            ran += 1
+    assert ran >= 12
+    sk.workspace_status()
+
+
 F16_GEMV_TILES = [(16, 16, 512), (16, 16, 1024), (16, 32, 512), (16, 64, 128), (16, 32, 256), (16, 16, 256)]
 
 
