@@ -1,0 +1,182 @@
+#!/usr/bin/env python3
+"""Writes tile_f16_asm_gen.h: the K loop of the four-wave 256 x 256 x 64 tile kernel as one block of gfx950
+assembly (used by tile_f16_asm.h inside an `asm volatile` statement).
+
+    python3 gen_tile_asm.py > tile_f16_asm_gen.h        (the Makefile does this when the script changes)
+
+Why assembly: each of the four waves owns a 128 x 128 block of C, 256 fp32 accumulators per lane, which must
+live in the accumulation registers a[0:255] for the whole loop while the 256 architectural registers hold
+operand fragments.  The compiler will not keep that assignment (it moves accumulators between the two files
+inside the loop), so the loop is written out with fixed registers:
+
+  a[(8 i + j) 4 .. +3]   16 x 16 block (i, j) of the wave's 128 x 128 result (i: rows of A, j: rows of B)
+  v[128:159] v[160:191]  A / B fragments of K-step 0 (eight 16-row blocks each, four registers per block)
+  v[192:223] v[224:255]  A / B fragments of K-step 1
+  v[120:121]             per-lane byte offsets of the A / B loads of this iteration
+  s[80:87]               loop state (see the text)
+
+One iteration (stage `cur` of the two 64 KB LDS stages holds its tiles, `nxt` the next iteration's):
+  block 0   64 MFMAs on the K-step-0 fragments; the 16 fragment reads of K-step 1 (from cur) ride along
+  sync      wait for them, wait for this wave's direct-to-LDS loads into nxt, barrier
+  block 1   64 MFMAs on the K-step-1 fragments; along ride the 16 loads of iteration it + 2 into cur (which
+            every wave has finished reading) and the 16 fragment reads of K-step 0 of nxt
+The loads of iterations past the segment get an out-of-range offset (they fetch nothing and zero a stage
+nobody reads), so the loop has no branch but its own back edge.
+"""
+
+A0, B0, A1, B1 = 128, 160, 192, 224     # first registers of the fragment buffers
+VOA, VOB = 120, 121                     # v120 / v121: load offsets of this iteration
+S_IT, S_KA, S_KB, S_T, S_OOB, S_M0, S_LDS, S_T2 = 80, 81, 82, 83, 84, 85, 86, 87
+
+
+def emit(lines, text):
+    lines.append(text)
+
+
+def mfma(lines, i, j, a_base, b_base):
+    c = (8 * i + j) * 4
+    emit(lines, f'MF " a[{c}:{c + 3}], v[{b_base + 4 * j}:{b_base + 4 * j + 3}], v[{a_base + 4 * i}:{a_base + 4 * i + 3}], a[{c}:{c + 3}]')
+
+
+def frag_read(lines, f, a_base, b_base, addr_a, addr_b):
+    """fragment f: 0..7 blocks of A, 8..15 blocks of B; 16 rows of 128 bytes per block"""
+    if f < 8:
+        emit(lines, f'"ds_read_b128 v[{a_base + 4 * f}:{a_base + 4 * f + 3}], {addr_a} offset:{f * 2048}')
+    else:
+        g = f - 8
+        emit(lines, f'"ds_read_b128 v[{b_base + 4 * g}:{b_base + 4 * g + 3}], {addr_b} offset:{g * 2048}')
+
+
+def dma(lines, x, first):
+    """load x of a stage: 0..7 row groups of A, 8..15 of B (a wave's groups are 4 KB apart in LDS);
+    s[S_T] walks the global offsets of the groups, s[S_LDS] is the stage's LDS address for this wave"""
+    if x == 0:
+        emit(lines, f'"s_mov_b32 s{S_T}, s{S_KA}')
+    if x == 8:
+        emit(lines, f'"s_mov_b32 s{S_T}, s{S_KB}')
+    lds_off = (x * 4096) if x < 8 else (32768 + (x - 8) * 4096)
+    emit(lines, f'"s_add_u32 m0, s{S_LDS}, {lds_off}')
+    emit(lines, '"s_nop 0')
+    if x < 8:
+        emit(lines, f'"buffer_load_dwordx4 v{VOA}, %[rsa], s{S_T} offen lds')
+        emit(lines, f'"s_add_u32 s{S_T}, s{S_T}, %[gas]')
+    else:
+        emit(lines, f'"buffer_load_dwordx4 v{VOB}, %[rsb], s{S_T} offen lds')
+        emit(lines, f'"s_add_u32 s{S_T}, s{S_T}, %[gbs]')
+
+
+def offsets_for(lines, ahead):
+    """v120 / v121 = the lane offsets, pushed out of range if iteration it + ahead is past the segment"""
+    emit(lines, f'"s_add_u32 s{S_T2}, s{S_IT}, {ahead}')
+    emit(lines, f'"s_cmp_lt_u32 s{S_T2}, %[n]')
+    emit(lines, f'"s_cselect_b32 s{S_OOB}, 0, 0x80000000')
+    emit(lines, f'"v_or_b32 v{VOA}, s{S_OOB}, %[voa]')
+    emit(lines, f'"v_or_b32 v{VOB}, s{S_OOB}, %[vob]')
+
+
+def mfma_order():
+    # walk the 8 x 8 blocks so that consecutive instructions share one operand
+    order = []
+    for i in range(8):
+        js = range(8) if i % 2 == 0 else range(7, -1, -1)
+        order += [(i, j) for j in js]
+    return order
+
+
+def slots(count, total, first, every):
+    """MFMA indices after which `count` riders are issued: every `every`-th instruction from `first` on"""
+    out = [first + k * every for k in range(count)]
+    assert out[-1] < total, (count, total, first, every)
+    return out
+
+
+def main():
+    import os
+    # where the fragment reads and the loads ride along the 64 MFMAs of a block (tunables of the schedule)
+    rd0 = slots(16, 64, int(os.environ.get("SK_ASM_RD0_FIRST", 1)), int(os.environ.get("SK_ASM_RD0_EVERY", 3)))
+    rd1 = slots(16, 64, int(os.environ.get("SK_ASM_RD1_FIRST", 2)), int(os.environ.get("SK_ASM_RD1_EVERY", 3)))
+    ld1 = slots(16, 64, int(os.environ.get("SK_ASM_LD1_FIRST", 0)), int(os.environ.get("SK_ASM_LD1_EVERY", 3)))
+    L = []
+    # ---- accumulators start at zero
+    for r in range(256):
+        emit(L, f'"v_accvgpr_write_b32 a{r}, 0')
+    # ---- prologue: both stages requested, wait for the first
+    emit(L, f'"s_mov_b32 s{S_IT}, 0')
+    emit(L, f'"s_mov_b32 s{S_LDS}, %[lds]')
+    emit(L, f'"s_mov_b32 s{S_KA}, %[ga0]')
+    emit(L, f'"s_mov_b32 s{S_KB}, %[gb0]')
+    offsets_for(L, 0)
+    for x in range(16):
+        dma(L, x, True)
+    emit(L, f'"s_add_u32 s{S_KA}, s{S_KA}, 128')
+    emit(L, f'"s_add_u32 s{S_KB}, s{S_KB}, 128')
+    emit(L, f'"s_xor_b32 s{S_LDS}, s{S_LDS}, 0x10000')
+    offsets_for(L, 1)
+    for x in range(16):
+        dma(L, x, False)
+    emit(L, f'"s_add_u32 s{S_KA}, s{S_KA}, 128')
+    emit(L, f'"s_add_u32 s{S_KB}, s{S_KB}, 128')
+    emit(L, f'"s_xor_b32 s{S_LDS}, s{S_LDS}, 0x10000')
+    emit(L, '"s_waitcnt vmcnt(16)')
+    emit(L, '"s_barrier')
+    for f in range(16):
+        frag_read(L, f, A0, B0, "%[ra0]", "%[rb0]")
+    emit(L, '"s_nop 7')   # accumulator writes above are long done; cheap insurance before the first MFMA
+    # ---- the loop
+    emit(L, '"L_sk_loop%=:')
+    # the K-step-0 fragments were requested in the order A0..A7, B0..B7: the first MFMAs need A0 and the first
+    # B blocks only, the youngest reads (the last B blocks) get until MFMA `late_at` to arrive
+    late = int(os.environ.get("SK_ASM_TOP_LATE", 0))
+    late_at = int(os.environ.get("SK_ASM_TOP_LATE_AT", 4))
+    emit(L, f'"s_waitcnt lgkmcnt({late})')
+    order = mfma_order()
+    for m, (i, j) in enumerate(order):
+        if late and m == late_at:
+            emit(L, '"s_waitcnt lgkmcnt(0)')
+        mfma(L, i, j, A0, B0)
+        if m in rd0:
+            frag_read(L, rd0.index(m), A1, B1, "%[ra1]", "%[rb1]")
+    emit(L, '"s_waitcnt lgkmcnt(0)')
+    emit(L, '"s_waitcnt vmcnt(0)')
+    emit(L, '"s_barrier')
+    offsets_for(L, 2)
+    # from here on the fragment addresses point at the other stage
+    for reg in ("%[ra0]", "%[ra1]", "%[rb0]", "%[rb1]"):
+        emit(L, f'"v_xor_b32 {reg}, 0x10000, {reg}')
+    for m, (i, j) in enumerate(order):
+        mfma(L, i, j, A1, B1)
+        if m in ld1:
+            dma(L, ld1.index(m), False)
+        if m in rd1:
+            frag_read(L, rd1.index(m), A0, B0, "%[ra0]", "%[rb0]")
+    emit(L, f'"s_add_u32 s{S_KA}, s{S_KA}, 128')
+    emit(L, f'"s_add_u32 s{S_KB}, s{S_KB}, 128')
+    emit(L, f'"s_xor_b32 s{S_LDS}, s{S_LDS}, 0x10000')
+    emit(L, f'"s_add_u32 s{S_IT}, s{S_IT}, 1')
+    emit(L, f'"s_cmp_lt_u32 s{S_IT}, %[n]')
+    emit(L, '"s_cbranch_scc1 L_sk_loop%=')
+    # ---- drain: the empty loads of the last two iterations still write LDS; the accumulators must have left
+    # the matrix pipe before ordinary instructions read them
+    emit(L, '"s_waitcnt vmcnt(0) lgkmcnt(0)')
+    for _ in range(3):
+        emit(L, '"s_nop 7')
+
+    print("// Generated by gen_tile_asm.py -- do not edit; see that file for the register plan and the schedule.")
+    print("// SK_TILE_ASM_LOOP(MF): the loop text, MF = the MFMA mnemonic as a string literal.")
+    print("#pragma once")
+    print("#define SK_TILE_ASM_LOOP(MF) \\")
+    for text in L:
+        if text.startswith("MF "):
+            print(f"  {text}\\n\\t\" \\")
+        else:
+            print(f"  {text}\\n\\t\" \\")
+    print("  \"\"")
+    clob = [f'"a{r}"' for r in range(256)] + [f'"v{r}"' for r in range(120, 256)] + [f'"s{r}"' for r in range(80, 88)]
+    print("#define SK_TILE_ASM_CLOBBERS \\")
+    for k in range(0, len(clob), 16):
+        tail = ", \\" if k + 16 < len(clob) else ""
+        print("  " + ", ".join(clob[k:k + 16]) + tail)
+
+
+if __name__ == "__main__":
+    main()

@@ -24,7 +24,8 @@ struct KernelInfo {
   int variant;  // tile kernels -- 0: registers -> padded LDS rows; 1: direct global -> LDS loads,
                 // swizzled rows; 2: as 1 with four waves per CTA (one per SIMD, accumulators in AGPRs);
                 // 3: as 1 with BK = 32 and four LDS stages (loads three iterations ahead);
-                // 4: as 1 with 16x16x32 MFMAs; 5: as 3 with 16x16x32 MFMAs; 6: as 1 for fp8 operands (32x32x64 MFMAs)
+                // 4: as 1 with 16x16x32 MFMAs; 5: as 3 with 16x16x32 MFMAs; 6: as 1 for fp8 operands (32x32x64 MFMAs);
+                // 7: as 4 with four waves per CTA, the K loop in assembly and the accumulators in a[0:255]
                 // small-M kernels -- 0: up to 16*MB rows of A; 1: M == 1; 2: M == 1, matrix-vector on 4x4x4 MFMA
   int bm, bn, bk;  // CTA tile; bk is the K extent of one CTA iteration
   int threads;
@@ -258,6 +259,11 @@ struct KernelInfo {
   X(81, 128, 128, 2, 2)       \
   X(82, 128, 256, 2, 4)       \
   X(83, 256, 128, 4, 2)
+
+// 256 x 256 x 64 on four waves, K loop in assembly (variant 7), NT layout, K a multiple of 64:  X(id, BF16)
+#define SK_TILE_ASM_KERNELS(X) \
+  X(34, false)                 \
+  X(66, true)
 
 const KernelInfo *kernel_table(int *count);
 const KernelInfo *kernel_by_id(int id);

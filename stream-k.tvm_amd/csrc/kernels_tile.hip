@@ -209,7 +209,7 @@ int launch_tile_f16(int id, const GemmArgs &a, const DevPlan &p, const Workspace
     SK_TILE_I8_KERNELS(X)
 #undef X
   }
-  return (int)hipErrorInvalidValue;
+  return launch_tile_asm(id, a, p, ws, s, bias);
 }
 
 int occupancy_tile(int id) {
@@ -315,7 +315,7 @@ int occupancy_tile(int id) {
     SK_TILE_I8_KERNELS(X)
 #undef X
   }
-  return -1;
+  return occupancy_tile_asm(id);
 }
 
 }  // namespace sk

@@ -1,0 +1,62 @@
+// Four-wave 256 x 256 x 64 Stream-K tile kernels whose K loop is hand-scheduled assembly (tile_f16_asm.h).
+#include "launch.h"
+#include "sk_persistent.h"
+#include "tile_f16_asm.h"
+
+namespace sk {
+
+template <class P, bool FIXUP>
+__global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_tile_asm_kernel(typename P::Args a, DevPlan plan, Workspace ws,
+                                                                            const void *bias) {
+  __shared__ __attribute__((aligned(16))) char smem[P::LDS_BYTES];
+  run_persistent<P, FIXUP, true>(a, plan, ws, smem, bias);
+}
+
+int tile_asm_kernel_infos(KernelInfo *out, int max) {
+  int n = 0;
+#define X(id, BF16)                                                                                              \
+  if (n < max) {                                                                                                 \
+    typedef TileF16Asm<BF16> P;                                                                                  \
+    out[n++] = KernelInfo{id, FAMILY_TILE, (BF16) ? 3 /* SK_BF16 */ : 0, 0, 7, P::BM, P::BN, P::BK, P::NT, P::LDS_TOTAL, \
+                          P::CTAS_PER_CU, P::TILE_ELEMS, 0, 0, 64,                                               \
+                          (BF16) ? "tile_bf16_nt_asm_256x256x64" : "tile_f16_nt_asm_256x256x64"};                \
+  }
+  SK_TILE_ASM_KERNELS(X)
+#undef X
+  return n;
+}
+
+// data-parallel launches use the instance without fix-up code
+int launch_tile_asm(int id, const GemmArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s, const void *bias) {
+  switch (id) {
+#define X(id_, BF16)                                                                                              \
+  case id_: {                                                                                                     \
+    typedef TileF16Asm<BF16> P;                                                                                   \
+    if (p.sk_tiles == 0)                                                                                          \
+      hipLaunchKernelGGL((sk_tile_asm_kernel<P, false>), dim3(p.grid), dim3(P::NT), 0, s, a, p, ws, bias);        \
+    else                                                                                                          \
+      hipLaunchKernelGGL((sk_tile_asm_kernel<P, true>), dim3(p.grid), dim3(P::NT), 0, s, a, p, ws, bias);         \
+    return (int)hipGetLastError();                                                                                \
+  }
+    SK_TILE_ASM_KERNELS(X)
+#undef X
+  }
+  return (int)hipErrorInvalidValue;
+}
+
+int occupancy_tile_asm(int id) {
+  int occ = 0;
+  switch (id) {
+#define X(id_, BF16)                                                                                                    \
+  case id_: {                                                                                                           \
+    typedef TileF16Asm<BF16> P;                                                                                         \
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_tile_asm_kernel<P, true>, P::NT, 0) != hipSuccess) return -1; \
+    return occ;                                                                                                         \
+  }
+    SK_TILE_ASM_KERNELS(X)
+#undef X
+  }
+  return -1;
+}
+
+}  // namespace sk

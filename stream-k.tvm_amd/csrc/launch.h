@@ -20,6 +20,10 @@ int skinny_kernel_infos(KernelInfo *out, int max);
 // bias: optional row of N values of C's type added in the epilogue (null: none)
 int launch_tile_f16(int id, const GemmArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s, const void *bias);
 int launch_skinny(int id, const SkinnyArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s, const void *bias);
+// the four-wave kernels whose K loop is assembly live in a translation unit of their own
+int tile_asm_kernel_infos(KernelInfo *out, int max);
+int launch_tile_asm(int id, const GemmArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s, const void *bias);
+int occupancy_tile_asm(int id);
 int f32_kernel_infos(KernelInfo *out, int max);
 int launch_f32(int id, const GemmArgsF32 &a, const DevPlan &p, const Workspace &ws, hipStream_t s);
 int occupancy_f32(int id);

@@ -18,12 +18,14 @@ static int g_count = 0;
 static std::once_flag g_table_once;
 
 int tile_kernel_infos(KernelInfo *out, int max);
+int tile_asm_kernel_infos(KernelInfo *out, int max);
 int skinny_kernel_infos(KernelInfo *out, int max);
 int f32_kernel_infos(KernelInfo *out, int max);
 
 const KernelInfo *kernel_table(int *count) {
   std::call_once(g_table_once, [] {
     int n = tile_kernel_infos(g_table, 320);
+    n += tile_asm_kernel_infos(g_table + n, 320 - n);
     n += skinny_kernel_infos(g_table + n, 320 - n);
     n += f32_kernel_infos(g_table + n, 320 - n);
     g_count = n;

@@ -1,0 +1,246 @@
+// fp16 / bfloat16 NT tile arithmetic, 256 x 256 x 64 CTA tile on FOUR waves (2 x 2), each owning a 128 x 128
+// block of C: 256 fp32 accumulators per lane, kept in the accumulation registers a[0:255] from the first MFMA
+// of a segment to the store of C.  A wave tile of 128 x 128 reads a third fewer LDS bytes per FLOP than the
+// 128 x 64 blocks of the eight-wave kernel (tile_f16_dma.h), and on a part whose matrix clock is set by the
+// power drawn, bytes moved are clock.
+//
+// The data movement is that of tile_f16_dma.h (direct global -> LDS loads of 16 bytes per lane, LDS rows of 128
+// bytes with chunk c of row r at position c ^ ((r >> 1) & 7), two stages of 64 KB, fragments for
+// v_mfma_f32_16x16x32_f16 read with ds_read_b128; replaces the reference's inner MAC, streamk_fp16.py:196-240).
+// The K loop itself is one block of assembly with fixed registers (gen_tile_asm.py writes it, with the register
+// plan and the schedule): the compiler does not keep 256 accumulators in one register file while it schedules
+// the loop around them.  Everything else -- addressing, fix-up, epilogue -- is ordinary code that reaches the
+// accumulators four at a time through v_accvgpr_read_b32 / v_accvgpr_write_b32.  The compiler itself must not
+// touch the accumulation registers between those statements: the kernels of this policy contain no other MFMA
+// and stay far below 256 architectural registers, so it has no reason to (the build checks the generated
+// assembly for accumulation-register instructions outside the hand-written blocks).
+//
+// Restrictions: NT layout, K a multiple of 64.
+#pragma once
+#include "sk_device.h"
+#include "tile_f16.h"
+#include "tile_f16_asm_gen.h"
+
+namespace sk {
+
+// accumulators a[R .. R+3] <-> four floats
+template <int R>
+__device__ __forceinline__ floatx4 agpr_read4() {
+  float x0, x1, x2, x3;
+  asm volatile(
+      "v_accvgpr_read_b32 %0, a[%4]\n\tv_accvgpr_read_b32 %1, a[%5]\n\t"
+      "v_accvgpr_read_b32 %2, a[%6]\n\tv_accvgpr_read_b32 %3, a[%7]"
+      : "=v"(x0), "=v"(x1), "=v"(x2), "=v"(x3)
+      : "n"(R), "n"(R + 1), "n"(R + 2), "n"(R + 3));
+  return floatx4{x0, x1, x2, x3};
+}
+template <int R>
+__device__ __forceinline__ void agpr_write4(floatx4 x) {
+  asm volatile(
+      "v_accvgpr_write_b32 a[%4], %0\n\tv_accvgpr_write_b32 a[%5], %1\n\t"
+      "v_accvgpr_write_b32 a[%6], %2\n\tv_accvgpr_write_b32 a[%7], %3"
+      :
+      : "v"(x[0]), "v"(x[1]), "v"(x[2]), "v"(x[3]), "n"(R), "n"(R + 1), "n"(R + 2), "n"(R + 3));
+}
+
+template <bool BF16_ = false>
+struct TileF16Asm {
+  typedef GemmArgs Args;
+  static constexpr bool LEAN_ENTRY = true;  // see run_persistent
+  static constexpr int BM = 256, BN = 256, BK = 64, WM = 2, WN = 2, NW = 4, NT = 256;
+  static constexpr int WTM = 128, WTN = 128, FM = 8, FN = 8;  // wave tile; 16 x 16 accumulator blocks per wave
+  static constexpr int ROW_BYTES = 128, A_BYTES = BM * ROW_BYTES, STAGE_BYTES = 2 * A_BYTES;
+  static constexpr int LDS_TOTAL = 2 * STAGE_BYTES, LDS_BYTES = 16;
+  static constexpr int TILE_ELEMS = BM * BN, NV4 = FM * FN;
+  static constexpr int CTAS_PER_CU = 1, WAVES_PER_EU = 1;
+  static constexpr int LDC = WTN + 8, PATCH_ROWS = 64;  // epilogue patch: 64 rows x 136 halfs per wave and pass
+  static_assert(PATCH_ROWS * LDC * 2 <= LDS_TOTAL / NW, "epilogue patches must fit the stages");
+
+  struct Acc {};  // the accumulators live in a[0:255]: block (i, j) in a[(8 i + j) 4 .. + 3]
+
+  static __device__ __forceinline__ char *lds() {
+    __shared__ __attribute__((aligned(1024))) char buf[LDS_TOTAL];
+    return buf;
+  }
+
+  static __device__ __forceinline__ void mac(const Args &a, Acc &, int pm, int pn, int k0, int n, char *) {
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int rows_a = min(BM, a.M - pm * BM), rows_b = min(BN, a.N - pn * BN);
+    // rows past the matrix edge lie beyond the descriptors' ranges and read as zero
+    const uint4v rsrc_a = make_rsrc_words(a.A + (int64_t)pm * BM * a.lda, (uint32_t)(rows_a * a.lda * 2));
+    const uint4v rsrc_b = make_rsrc_words(a.B + (int64_t)pn * BN * a.ldb, (uint32_t)(rows_b * a.ldb * 2));
+    // a wave-wide load fills 8 LDS rows; lane l writes (row l / 8, position l % 8) and therefore fetches
+    // chunk (l % 8) ^ swizzle(row); a wave only loads row groups of its own parity (see tile_f16_dma.h)
+    const int my_chunk = (lane & 7) ^ (((wave & 1) << 2) | (lane >> 4)), my_row = lane >> 3;
+    const uint32_t voff_a = (uint32_t)(my_row * a.lda + my_chunk * 8) * 2;
+    const uint32_t voff_b = (uint32_t)(my_row * a.ldb + my_chunk * 8) * 2;
+    // row group g = wave + 4 x of a stage: rows 8 g .. 8 g + 7, at wave-uniform byte offset 16 g ld
+    const uint32_t goff_a = (uint32_t)k0 * (BK * 2) + (uint32_t)(wave * 16 * a.lda), gstep_a = (uint32_t)(64 * a.lda);
+    const uint32_t goff_b = (uint32_t)k0 * (BK * 2) + (uint32_t)(wave * 16 * a.ldb), gstep_b = (uint32_t)(64 * a.ldb);
+    const uint32_t base = lds_address(lds());
+    const uint32_t lds_wave = base + wave * 1024;
+    // fragments: lane (r = l % 16, g = l / 16) reads row r of a 16-row block, chunk 4 kk + g at position
+    // (4 kk + g) ^ ((r >> 1) & 7); K-step 1 is K-step 0 with address bit 6 flipped
+    const uint32_t pos0 = (uint32_t)((lane >> 4) ^ ((lane >> 1) & 7)) * 16;
+    uint32_t ra0 = base + (uint32_t)(wm * WTM + (lane & 15)) * ROW_BYTES + pos0, ra1 = ra0 ^ 64;
+    uint32_t rb0 = base + A_BYTES + (uint32_t)(wn * WTN + (lane & 15)) * ROW_BYTES + pos0, rb1 = rb0 ^ 64;
+    const uint32_t iters = (uint32_t)n;
+    if constexpr (BF16_) {
+      asm volatile(SK_TILE_ASM_LOOP("v_mfma_f32_16x16x32_bf16")
+                   : [ra0] "+v"(ra0), [ra1] "+v"(ra1), [rb0] "+v"(rb0), [rb1] "+v"(rb1)
+                   : [rsa] "s"(rsrc_a), [rsb] "s"(rsrc_b), [voa] "v"(voff_a), [vob] "v"(voff_b), [ga0] "s"(goff_a),
+                     [gb0] "s"(goff_b), [gas] "s"(gstep_a), [gbs] "s"(gstep_b), [n] "s"(iters), [lds] "s"(lds_wave)
+                   : "memory", "m0", "scc", SK_TILE_ASM_CLOBBERS);
+    } else {
+      asm volatile(SK_TILE_ASM_LOOP("v_mfma_f32_16x16x32_f16")
+                   : [ra0] "+v"(ra0), [ra1] "+v"(ra1), [rb0] "+v"(rb0), [rb1] "+v"(rb1)
+                   : [rsa] "s"(rsrc_a), [rsb] "s"(rsrc_b), [voa] "v"(voff_a), [vob] "v"(voff_b), [ga0] "s"(goff_a),
+                     [gb0] "s"(goff_b), [gas] "s"(gstep_a), [gbs] "s"(gstep_b), [n] "s"(iters), [lds] "s"(lds_wave)
+                   : "memory", "m0", "scc", SK_TILE_ASM_CLOBBERS);
+    }
+    __syncthreads();  // both stages are free for the epilogue / the next segment
+  }
+
+  // ---- epilogue: fp32 -> C's type through a per-wave LDS patch, 16-byte stores of whole rows ----
+  static __device__ __forceinline__ void store_c(const Args &a, const Acc &, int pm, int pn, char *, const void *bias) {
+    if (bias == nullptr)
+      store_c_impl<false, -1>(a, pm, pn, nullptr);
+    else
+      store_c_impl<true, -1>(a, pm, pn, bias);
+  }
+  static __device__ __forceinline__ void store_c_half(const Args &a, const Acc &, int pm, int pn, char *,
+                                                      const void *bias, int h) {
+    if (bias == nullptr) {
+      if (h == 0) store_c_impl<false, 0>(a, pm, pn, nullptr);
+      else store_c_impl<false, 1>(a, pm, pn, nullptr);
+    } else {
+      if (h == 0) store_c_impl<true, 0>(a, pm, pn, bias);
+      else store_c_impl<true, 1>(a, pm, pn, bias);
+    }
+  }
+  // HALF < 0: the whole tile; 0 / 1: rows [HALF * 64, HALF * 64 + 64) of every wave's block
+  template <bool BIAS, int HALF>
+  static __device__ __forceinline__ void store_c_impl(const Args &a, int pm, int pn, const void *epi) {
+    constexpr int ROW_BEGIN = HALF < 0 ? 0 : HALF * (WTM / 2), NPASS = HALF < 0 ? 2 : 1;
+    const half_t *bias = BIAS ? epi_bias(epi) : nullptr;
+    const int act = BIAS ? epi_act(epi) : 0;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int bias_col0 = BIAS ? pn * BN + wn * WTN + pin_here(lane >> 4) * 4 : 0;
+    half_t *patch = reinterpret_cast<half_t *>(lds() + wave * (LDS_TOTAL / NW));
+    const bool vec_ok = (a.ldc % 8 == 0) && ((reinterpret_cast<uintptr_t>(a.C) & 15) == 0);
+    constexpr int CPRC = WTN / 8;
+    static_for<0, NPASS>([&](auto pass) {
+      constexpr int p = decltype(pass)::value;
+      static_for<0, PATCH_ROWS / 16>([&](auto blk) {
+        constexpr int ib = decltype(blk)::value;
+        constexpr int ii = ROW_BEGIN / 16 + p * (PATCH_ROWS / 16) + ib;
+        static_for<0, FN>([&](auto col) {
+          constexpr int j = decltype(col)::value;
+          const floatx4 x = agpr_read4<(ii * FN + j) * 4>();
+          floatx4 bv = {0.f, 0.f, 0.f, 0.f};
+          if constexpr (BIAS) bv = bias4_at<BF16_>(bias, bias_col0 + j * 16, a.N);
+          half4v h;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            float y = x[e];
+            if constexpr (BIAS) y = activate(y + bv[e], act);
+            if constexpr (BF16_) {
+              const __bf16 b = (__bf16)y;
+              h[e] = __builtin_bit_cast(half_t, b);  // the patch only carries 16-bit patterns
+            } else {
+              h[e] = (half_t)y;
+            }
+          }
+          *reinterpret_cast<half4v *>(patch + (ib * 16 + (lane & 15)) * LDC + j * 16 + (lane >> 4) * 4) = h;
+        });
+      });
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      const int row0 = pm * BM + wm * WTM + ROW_BEGIN + p * PATCH_ROWS, col0 = pn * BN + wn * WTN;
+#pragma unroll
+      for (int s = 0; s < PATCH_ROWS * CPRC / 64; ++s) {
+        const int idx = s * 64 + lane;
+        const int r = idx / CPRC, cc = idx % CPRC;
+        const int grow = row0 + r, gcol = col0 + cc * 8;
+        if (grow < a.M && gcol < a.N) {
+          const half_t *src = patch + r * LDC + cc * 8;
+          half_t *dst = a.C + (int64_t)grow * a.ldc + gcol;
+          if (vec_ok && gcol + 8 <= a.N) {
+            *reinterpret_cast<uint4v *>(dst) = *reinterpret_cast<const uint4v *>(src);
+          } else {
+            for (int e = 0; e < 8 && gcol + e < a.N; ++e) dst[e] = src[e];
+          }
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    });
+    __syncthreads();  // patches overlap the stages of the next tile
+  }
+
+  // ---- partial tiles (same workspace layouts as tile_f16_dma.h: float4 group v of thread t at
+  // (v * NT + t) * 4 for the ordered reduce, element s of thread t at s * NT + t for the atomic buffer) ----
+  static constexpr bool COHERENT_PARTIALS = false;
+  static constexpr bool COHERENT_REDUCE = true;
+  static constexpr bool HALVES = true;
+  template <int V0, int V1>
+  static __device__ __forceinline__ void store_groups(float *dst) {
+    const BufferRsrc r = make_rsrc(dst, TILE_ELEMS * 4);
+    const uint32_t off = (uint32_t)pin_here((int)threadIdx.x) * 16;
+    static_for<V0, V1>([&](auto g) {
+      constexpr int v = decltype(g)::value;
+      st_coherent16(r, off, (uint32_t)v * NT * 16, __builtin_bit_cast(uint4v, agpr_read4<v * 4>()));
+    });
+  }
+  template <int V0, int V1>
+  static __device__ __forceinline__ void add_groups(const float *src) {
+    const BufferRsrc r = make_rsrc(src, TILE_ELEMS * 4);
+    const uint32_t off = (uint32_t)pin_here((int)threadIdx.x) * 16;
+    static_for<V0, V1>([&](auto g) {
+      constexpr int v = decltype(g)::value;
+      const floatx4 x = __builtin_bit_cast(floatx4, ld_coherent16(r, off, (uint32_t)v * NT * 16));
+      agpr_write4<v * 4>(agpr_read4<v * 4>() + x);
+    });
+  }
+  static __device__ __forceinline__ void store_partial(const Acc &, float *dst) { store_groups<0, NV4>(dst); }
+  static __device__ __forceinline__ void add_partial(Acc &, const float *src) { add_groups<0, NV4>(src); }
+  static __device__ __forceinline__ void store_partial_half(const Acc &, float *dst, int h) {
+    if (h == 0) store_groups<0, NV4 / 2>(dst);
+    else store_groups<NV4 / 2, NV4>(dst);
+  }
+  static __device__ __forceinline__ void add_partial_half(Acc &, const float *src, int h) {
+    if (h == 0) add_groups<0, NV4 / 2>(src);
+    else add_groups<NV4 / 2, NV4>(src);
+  }
+  static __device__ __forceinline__ void atomic_partial(const Acc &, float *dst) {
+    dst = pin_here(dst) + threadIdx.x;
+    static_for<0, NV4>([&](auto g) {
+      constexpr int v = decltype(g)::value;
+      const floatx4 x = agpr_read4<v * 4>();
+#pragma unroll
+      for (int e = 0; e < 4; ++e) atomic_add_f32(dst + (size_t)(v * 4 + e) * NT, x[e]);
+    });
+  }
+  // reads the completed sum and leaves zeros behind
+  static __device__ __forceinline__ void take_partial(Acc &, float *src) {
+    src = pin_here(src) + threadIdx.x;
+    static_for<0, NV4>([&](auto g) {
+      constexpr int v = decltype(g)::value;
+      floatx4 x;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float *p = src + (size_t)(v * 4 + e) * NT;
+        x[e] = *p;
+        *p = 0.f;
+      }
+      agpr_write4<v * 4>(x);
+    });
+  }
+};
+
+}  // namespace sk
