@@ -93,9 +93,14 @@ def slots(count, total, first, every):
 def main():
     import os
     # where the fragment reads and the loads ride along the 64 MFMAs of a block (tunables of the schedule)
-    rd0 = slots(16, 64, int(os.environ.get("SK_ASM_RD0_FIRST", 1)), int(os.environ.get("SK_ASM_RD0_EVERY", 3)))
-    rd1 = slots(16, 64, int(os.environ.get("SK_ASM_RD1_FIRST", 2)), int(os.environ.get("SK_ASM_RD1_EVERY", 3)))
-    ld1 = slots(16, 64, int(os.environ.get("SK_ASM_LD1_FIRST", 0)), int(os.environ.get("SK_ASM_LD1_EVERY", 3)))
+    # (measured at 8192^3 on random operands, each against the eight-wave kernel in the same run: the defaults
+    # 1.07-1.08 x; all 16 loads in the first 16 or 32 MFMA slots behind the barrier 0.98 x -- the wave then stalls
+    # at the texture addresser, and with one wave per SIMD that is a stalled matrix pipe; loads every third slot
+    # 1.05 x; later or denser fragment reads, a partial wait at the loop top, MFMAs issued ahead of the barrier:
+    # within 1 % of the defaults.  The same loop on four 32 KB buffers with a barrier per K-step of 32: 1.00 x.)
+    rd0 = slots(16, 64, int(os.environ.get("SK_ASM_RD0_FIRST", 0)), int(os.environ.get("SK_ASM_RD0_EVERY", 3)))
+    rd1 = slots(16, 64, int(os.environ.get("SK_ASM_RD1_FIRST", 1)), int(os.environ.get("SK_ASM_RD1_EVERY", 4)))
+    ld1 = slots(16, 64, int(os.environ.get("SK_ASM_LD1_FIRST", 3)), int(os.environ.get("SK_ASM_LD1_EVERY", 4)))
     L = []
     # ---- accumulators start at zero
     for r in range(256):
@@ -137,6 +142,11 @@ def main():
         if m in rd0:
             frag_read(L, rd0.index(m), A1, B1, "%[ra1]", "%[rb1]")
     emit(L, '"s_waitcnt lgkmcnt(0)')
+    # the first MFMAs of block 1 need the K-step-1 fragments only: issued ahead of the barrier they keep the
+    # matrix pipe busy while the wave waits there
+    early = int(os.environ.get("SK_ASM_EARLY", 0))
+    for m in range(early):
+        mfma(L, *order[m], A1, B1)
     emit(L, '"s_waitcnt vmcnt(0)')
     emit(L, '"s_barrier')
     offsets_for(L, 2)
@@ -144,7 +154,8 @@ def main():
     for reg in ("%[ra0]", "%[ra1]", "%[rb0]", "%[rb1]"):
         emit(L, f'"v_xor_b32 {reg}, 0x10000, {reg}')
     for m, (i, j) in enumerate(order):
-        mfma(L, i, j, A1, B1)
+        if m >= early:
+            mfma(L, i, j, A1, B1)
         if m in ld1:
             dma(L, ld1.index(m), False)
         if m in rd1:

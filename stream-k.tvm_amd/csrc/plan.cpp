@@ -48,10 +48,12 @@ static int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // eight-wave direct-to-LDS tile kernels; the most specialised small-M kernel that accepts the shape
 static int variant_rank(const KernelInfo &k) {
   if (k.family == FAMILY_SKINNY) return k.variant;
-  return k.variant == 4 ? 3 : (k.variant == 1 ? 2 : (k.variant == 2 ? 1 : 0));
+  return k.variant == 7 ? 4 : (k.variant == 4 ? 3 : (k.variant == 1 ? 2 : (k.variant == 2 ? 1 : 0)));
 }
 static bool accepts_shape(const KernelInfo &k, int64_t M, int64_t K) {
-  return (k.max_m == 0 || M <= k.max_m) && (k.max_ipt == 0 || (K + k.bk - 1) / k.bk <= k.max_ipt);
+  // (the assembly-loop tile kernels have no K tail: other K go to the next-best variant of the tile)
+  return (k.max_m == 0 || M <= k.max_m) && (k.max_ipt == 0 || (K + k.bk - 1) / k.bk <= k.max_ipt) &&
+         (k.family != FAMILY_TILE || k.variant != 7 || K % k.k_align == 0);
 }
 
 static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype, int layout,
@@ -123,8 +125,10 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
   // or two waves per SIMD, where the four-stage (BK = 32) pipeline hides the load latency better;
   // it exists for the NT layout only.
   const int64_t tiles256 = cdiv(M, 256) * cdiv(N, 256), tiles128 = cdiv(M, 128) * cdiv(N, 128);
-  // (256x256: the 16x16x32-MFMA form)
+  // (256x256: the four-wave kernel with the K loop in assembly where it applies -- NT, K a multiple of 64 --
+  // else the eight-wave 16x16x32-MFMA form)
   int pref[3][4] = {{256, 256, 64, 4}, {128, 128, 32, 3}, {64, 64, 32, 3}};  // bm, bn, bk, variant
+  if (layout == SK_LAYOUT_NT && K % 64 == 0 && (dtype == SK_F16 || dtype == SK_BF16)) pref[0][3] = 7;
   const int first = tiles256 * 4 >= (int64_t)num_cus * 3 ? 0 : (tiles128 * 2 >= num_cus ? 1 : 2);
   const int order[3][3] = {{0, 1, 2}, {1, 2, 0}, {2, 1, 0}};  // smaller tiles first, then larger ones
   for (int oi = 0; oi < 3 && !best; ++oi) {
@@ -135,6 +139,7 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
         if (t[i].bm != pref[pi][0] || t[i].bn != pref[pi][1]) continue;
         if (want_variant >= 0 && t[i].variant != want_variant) continue;
         if (pass == 0 && want_variant < 0 && (t[i].bk != pref[pi][2] || t[i].variant != pref[pi][3])) continue;
+        if (!accepts_shape(t[i], M, K)) continue;
         if (best == nullptr || variant_rank(t[i]) > variant_rank(*best)) best = &t[i];
       }
     }

@@ -100,6 +100,66 @@ def test_cfg2_streamk_both_fixups(sk, oracle, cfg, fixup):
     assert _rel(oracle, C, ref) <= 1e-3 <= TOL
 
 
+def test_assembly_loop_tile_kernels(sk, oracle, golden_dir):
+    """The four-wave 256 x 256 x 64 kernels whose K loop is hand-scheduled assembly (accumulators in the
+    accumulation registers): fp16 and bfloat16, ragged M and N, K any multiple of 64 (odd and even iteration
+    counts, a single iteration), every schedule and both fix-ups including the halves exchange -- exact on
+    integer data, bit-identical to the eight-wave 16x16x32 kernel on random data (same instruction, same order
+    of the K-steps), within tolerance of the oracle; a K that is no multiple of 64 falls back to the eight-wave
+    kernel; bias and activation epilogue."""
+    import torch
+    rng = np.random.default_rng(91)
+    assert sk.kernel_name(sk.make_plan(8192, 8192, 8192, "float16", "nt", use_tuned=False).kernel_id) == "tile_f16_nt_asm_256x256x64"
+    assert sk.kernel_name(sk.make_plan(2048, 2048, 2048, "bfloat16", "nt", dict(bm=256, bn=256)).kernel_id) == "tile_bf16_nt_asm_256x256x64"
+    assert "asm" not in sk.kernel_name(sk.make_plan(2048, 2048, 2056, "float16", "nt", dict(bm=256, bn=256)).kernel_id)
+    assert "asm" not in sk.kernel_name(sk.make_plan(2048, 2048, 2048, "float16", "nn", dict(bm=256, bn=256)).kernel_id)
+    with pytest.raises(sk.StreamKError):
+        sk.make_plan(2048, 2048, 2056, "float16", "nt", dict(bm=256, bn=256, variant=8))
+    ran = 0
+    for (M, N, K) in [(256, 256, 64), (256, 256, 192), (200, 136, 320), (1000, 1096, 4096), (520, 264, 448), (512, 1024, 2048)]:
+        Ai = rng.integers(-2, 3, (M, K)).astype(np.float16)
+        Bi = rng.integers(-2, 3, (N, K)).astype(np.float16)
+        exact = torch.from_numpy((Ai.astype(np.int32) @ Bi.astype(np.int32).T).astype(np.float32)).cuda()
+        Ar = (rng.random((M, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+        Br = (rng.random((N, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+        ref = oracle.matmul_fp32(Ar, Br, trans_b=True)
+        dAi, dBi, dAr, dBr = _t(Ai), _t(Bi), _t(Ar), _t(Br)
+        for sch in (dict(schedule="dp"), dict(schedule="basic", fixup="reduce", grid=7), dict(schedule="basic", fixup="atomic", grid=5),
+                    dict(schedule="sk2", fixup="reduce", grid=3), dict(schedule="splitk", split=2, fixup="reduce"),
+                    dict(schedule="splitk", split=2, fixup="atomic"), dict(schedule="sk1", fixup="reduce", grid=2, raster=2)):
+            try:
+                plan = sk.make_plan(M, N, K, "float16", "nt", dict(bm=256, bn=256, bk=64, variant=8, **sch))
+            except sk.StreamKError:
+                assert sch["schedule"] == "splitk"      # the split does not divide this K
+                continue
+            assert sk.kernel_name(plan.kernel_id) == "tile_f16_nt_asm_256x256x64"
+            assert torch.equal(sk.streamk_fp16(dAi, dBi, plan=plan).float(), exact), (M, N, K, sch)
+            C = sk.streamk_fp16(dAr, dBr, plan=plan)
+            assert _rel(oracle, C, ref) <= 2e-3 <= TOL, (M, N, K, sch)
+            if sch["schedule"] == "dp" or sch.get("fixup") == "reduce":
+                twin = sk.streamk_fp16(dAr, dBr, **dict(sch, bm=256, bn=256, bk=64, variant=5))
+                assert torch.equal(C, twin), (M, N, K, sch)
+            # bfloat16 twin of the loop
+            pb = sk.make_plan(M, N, K, "bfloat16", "nt", dict(bm=256, bn=256, bk=64, variant=8, **sch))
+            # (the exact integer sums, rounded once to bfloat16's eight bits)
+            assert torch.equal(sk.streamk_bf16(dAi.bfloat16(), dBi.bfloat16(), plan=pb), exact.bfloat16()), (M, N, K, sch)
+            ran += 1
+    assert ran >= 30
+    # epilogue: integer bias + relu exact; silu within tolerance
+    M, N, K = 520, 264, 448
+    Ai = rng.integers(-1, 2, (M, K)).astype(np.float16)
+    Bi = rng.integers(-1, 2, (N, K)).astype(np.float16)
+    bias = rng.integers(-3, 4, N).astype(np.float16)
+    want = np.maximum(Ai.astype(np.int32) @ Bi.astype(np.int32).T + bias.astype(np.int32), 0)
+    for sch in (dict(schedule="dp"), dict(schedule="basic", fixup="reduce", grid=7), dict(schedule="splitk", split=1)):
+        C = sk.streamk_fp16(_t(Ai), _t(Bi), bm=256, bn=256, bk=64, variant=8, bias=_t(bias), activation="relu", **sch)
+        assert np.array_equal(C.cpu().numpy().astype(np.int32), want), sch
+    x = Ai.astype(np.float64) @ Bi.astype(np.float64).T * 0.125 + bias.astype(np.float64)
+    C = sk.streamk_fp16(_t((Ai * np.float16(0.125)).astype(np.float16)), _t(Bi), bm=256, bn=256, bk=64, variant=8, bias=_t(bias), activation="silu")
+    assert oracle.max_abs_rel(C.float().cpu().numpy(), oracle.activation_ref(x, "silu")) <= 2e-3
+    sk.workspace_status()
+
+
 def test_fixed_split_k(sk, oracle):
     """Fixed split-K (the reference's data-parallel comparator with splitk_factor,
     thread_level_gemm_with_macro_ladder_atomic_reduce.py:129-199) on tile and small-M kernels, both
