@@ -76,6 +76,8 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
             variants += ((6, 32),)  # four-stage with 16x16x32 MFMAs
             if bm >= 128 and bn >= 128:
                 variants += ((5, bk),)  # two-stage with 16x16x32 MFMAs
+            if (bm, bn) == (256, 256) and K % 64 == 0:
+                variants += ((8, bk),)  # four waves, the K loop in assembly
             if (bm, bn) == (64, 64):
                 variants += ((1, bk),)
             for (variant, vbk), raster in itertools.product(variants, (1, 8)):
@@ -99,6 +101,23 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
 
 
 _MIN_TIMED_MS = 8.0  # a candidate is timed over at least this much GPU time
+
+_box_reference = None
+
+
+def box_reference_tflops():
+    """What this box sustains on one fixed launch (fp16 4096^3 NT, the eight-wave 256 x 256 data-parallel kernel,
+    U[-1,1) operands), measured once per process.  Boxes of one pool differ by more than 10 % on compute-bound
+    shapes; stored beside every cache entry, the figure shows on which kind of box the entry's latency was taken."""
+    global _box_reference
+    if _box_reference is None:
+        g = torch.Generator(device="cpu").manual_seed(1)
+        A = (torch.rand(4096, 4096, generator=g) * 2 - 1).half().cuda()
+        C = torch.empty(4096, 4096, dtype=torch.float16, device="cuda")
+        p = _plan.make_plan(4096, 4096, 4096, "float16", "nt", dict(bm=256, bn=256, bk=64, variant=5, schedule="dp", raster=8))
+        ms = _time_ms(lambda: ops.streamk_fp16(A, A, out=C, plan=p), 5, 10, True, min_ms=40.0)
+        _box_reference = round(2.0 * 4096 ** 3 / ms / 1e9, 1)
+    return _box_reference
 
 
 def _time_ms(fn, warmup, rep, graph, min_ms=None):
@@ -241,7 +260,8 @@ def autotune(M, N, K, dtype="float16", layout="nt", *, configs=None, warmup=5, r
         best = min(near, key=lambda r: r[0])
     if cache:
         c = load_cache(cache_path)
-        c[_key(dtype, layout, M, N, K)] = {"config": best[1], "latency_ms": best[0], "ref_latency_ms": ref_ms}
+        c[_key(dtype, layout, M, N, K)] = {"config": best[1], "latency_ms": best[0], "ref_latency_ms": ref_ms,
+                                           "box_reference_tflops": box_reference_tflops()}
         save_cache(c, cache_path)
         _plan.invalidate_tuned_cache()
     return best[0], best[1], ref_ms
