@@ -456,10 +456,21 @@ static int gemm_q4_any(const void *A, const void *Wq, const void *scales, const 
       (reinterpret_cast<uintptr_t>(C) & 1))
     return SK_ERR_ALIGN;
   const KernelInfo *k = kernel_by_id(plan->kernel_id);
-  if (!k || k->dtype != dtype || k->family != FAMILY_SKINNY) return SK_ERR_CONFIG;
+  if (!k || k->dtype != dtype) return SK_ERR_CONFIG;
   if (lda * 2 * k->bm >= (int64_t)1 << 31 || (K / 2) * k->bn >= (int64_t)1 << 31) return SK_ERR_SHAPE;
   DevPlan dp;
   Workspace w;
+  if (k->family == FAMILY_TILE) {
+    // more than 64 rows of A: the tile kernels that dequantise B on its way into LDS (scalar zero point,
+    // row-major nibbles)
+    if (dtype != SK_Q4) return SK_ERR_CONFIG;
+    rc = make_dev_plan(plan, k, ws, ws_bytes, cached_occupancy(k->id, 0), (hipStream_t)stream, &dp, &w);
+    if (rc) return rc;
+    GemmArgs g{(const half_t *)A, (const half_t *)Wq, (half_t *)C, (int)M, (int)N, (int)K, lda, K / 2, ldc, 1.f,
+               (const half_t *)scales, zero, (int)(K / group)};
+    return launch_tile_f16(k->id, g, dp, w, (hipStream_t)stream, bias) == 0 ? SK_OK : SK_ERR_LAUNCH;
+  }
+  if (k->family != FAMILY_SKINNY) return SK_ERR_CONFIG;
   rc = make_dev_plan(plan, k, ws, ws_bytes, cached_occupancy(k->id, 1), (hipStream_t)stream, &dp, &w);
   if (rc) return rc;
   SkinnyArgs a{(const half_t *)A, Wq, (const half_t *)scales, (half_t *)C, (int)M, (int)N, (int)K,

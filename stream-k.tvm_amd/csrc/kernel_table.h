@@ -265,6 +265,13 @@ struct KernelInfo {
   X(34, false)                 \
   X(66, true)
 
+// Q4 weights (dtype SK_Q4) for more rows of A than the weight-streaming kernels take: the two-stage 16x16x32 tile
+// kernel with B dequantised into its LDS stage (variant 4):  X(id, BM, BN, WM, WN)
+#define SK_TILE_Q4_KERNELS(X) \
+  X(46, 128, 128, 2, 2)       \
+  X(47, 256, 128, 4, 2)       \
+  X(48, 256, 256, 2, 4)
+
 const KernelInfo *kernel_table(int *count);
 const KernelInfo *kernel_by_id(int id);
 

@@ -19,6 +19,7 @@ static std::once_flag g_table_once;
 
 int tile_kernel_infos(KernelInfo *out, int max);
 int tile_asm_kernel_infos(KernelInfo *out, int max);
+int tile_q4_kernel_infos(KernelInfo *out, int max);
 int skinny_kernel_infos(KernelInfo *out, int max);
 int f32_kernel_infos(KernelInfo *out, int max);
 
@@ -26,6 +27,7 @@ const KernelInfo *kernel_table(int *count) {
   std::call_once(g_table_once, [] {
     int n = tile_kernel_infos(g_table, 320);
     n += tile_asm_kernel_infos(g_table + n, 320 - n);
+    n += tile_q4_kernel_infos(g_table + n, 320 - n);
     n += skinny_kernel_infos(g_table + n, 320 - n);
     n += f32_kernel_infos(g_table + n, 320 - n);
     g_count = n;
@@ -79,6 +81,16 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
   const bool q4 = dtype == SK_Q4 || dtype == SK_Q4_TILED || dtype == SK_Q4_ZP;
   // (one-byte operands: up to 64 rows -- their tile kernels start at 128 rows)
   const bool one_byte = dtype == SK_F8E4M3 || dtype == SK_F8E5M2 || dtype == SK_I8;
+  if (dtype == SK_Q4 && M > 64 && want_variant < 0) {
+    // more rows than the weight-streaming kernels take: the tile kernels that dequantise B on its way into LDS;
+    // the largest tile that still gives most CUs one
+    const int64_t t256 = cdiv(M, 256) * cdiv(N, 256), t256x128 = cdiv(M, 256) * cdiv(N, 128);
+    const int want_bm = t256x128 * 4 >= (int64_t)num_cus * 3 ? 256 : 128;
+    const int want_bn = (want_bm == 256 && t256 * 4 >= (int64_t)num_cus * 3) ? 256 : 128;
+    for (int i = 0; i < n; ++i)
+      if (t[i].family == FAMILY_TILE && t[i].dtype == SK_Q4 && t[i].bm == want_bm && t[i].bn == want_bn) return &t[i];
+    return nullptr;
+  }
   if ((M <= (one_byte ? 64 : 32) && layout == SK_LAYOUT_NT) || q4) {
     // M == 1 with Q4 weights: the matrix-vector kernel with four waves splitting K (data-parallel
     // over 16-row tiles), the fastest instance at LLM-sized N and K

@@ -17,6 +17,10 @@ struct GemmArgs {
   int M, N, K;
   int64_t lda, ldb, ldc;
   float alpha;  // fp8 kernels: C = fp16(alpha * A B^T); unused elsewhere
+  // Q4 tile kernels: B points at the packed nibbles [N, K/2] (ldb = K/2 bytes per row); scales [N, groups] fp16,
+  // one per 128 K-values; the scalar zero point
+  const half_t *scales;
+  int zero, groups;
 };
 
 template <int BM_, int BN_, int BK_, int WM_, int WN_>

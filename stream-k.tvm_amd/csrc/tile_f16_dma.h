@@ -21,6 +21,7 @@
 #pragma once
 #include <type_traits>
 
+#include "q4_dequant.h"
 #include "sk_device.h"
 #include "tile_f16.h"
 
@@ -70,9 +71,20 @@ struct LdsArray {
 // form); partial tiles travel through the workspace as int32 in the fp32 slots, so both fix-ups are
 // exact and independent of the order of the additions.  C is stored from registers (a lane holds four
 // consecutive int32 of a row).
+//
+// Q4_: B is not fp16 but packed nibbles with one fp16 scale per 128 K-values (the weight-only format of
+// q4_dequant.h), for calls with more rows of A than the weight-streaming kernels take.  A travels as before.  B's
+// nibbles of iteration it + 3 are loaded straight into one of two small LDS buffers (32 bytes per weight row);
+// behind the barrier of iteration it, where the fp16 kernel requests B of iteration it + 2, every thread instead
+// reads its share of the nibbles of iteration it + 2, dequantises them in registers with dequant_word_q4 -- the
+// bit-exact decode (the reference dequantises in registers right before the MMA,
+// streamk_fp16_ladder_block_reduce_q4.py:283-294) -- puts the eight weights of a word back into K order and stores
+// them where the direct load would have put them.  The fragment reads and the MFMAs do not know the difference.
 template <int BM_, int BN_, int WM_, int WN_, bool B_KN_ = false, int BK_ = 64, bool MFMA16_ = false, bool BF16_ = false,
-          int F8_ = 0>
+          int F8_ = 0, bool Q4_ = false>
 struct TileF16NTDma {
+  static constexpr bool Q4 = Q4_;
+  static_assert(!Q4_ || (MFMA16_ && !B_KN_ && BK_ == 64 && !BF16_ && F8_ == 0), "Q4: the two-stage 16x16x32 fp16 form");
   static constexpr bool B_KN = B_KN_, MFMA16 = MFMA16_;
   static constexpr bool I8 = F8_ == 3;
   static constexpr int F8 = I8 ? 0 : F8_;
@@ -97,7 +109,11 @@ struct TileF16NTDma {
   static constexpr int FROWS = MFMA16_ ? 16 : 32;              // rows of one operand fragment
   static constexpr int FM = WTM / FROWS, FN = WTN / FROWS;     // fragments per K-step
   static constexpr int A_BYTES = BM * ROW_BYTES, B_BYTES = BN * ROW_BYTES, STAGE_BYTES = A_BYTES + B_BYTES;
-  static constexpr int A_DMA = A_BYTES / 1024 / NW, B_DMA = B_BYTES / 1024 / NW, DMA_PER_WAVE = A_DMA + B_DMA;
+  static constexpr int A_DMA = A_BYTES / 1024 / NW, B_DMA = Q4_ ? 0 : B_BYTES / 1024 / NW, DMA_PER_WAVE = A_DMA + B_DMA;
+  // Q4: raw nibbles of one iteration: BN rows x 32 bytes; a wave-wide load covers 32 rows; a thread converts
+  // Q4_WORDS 32-bit words (eight weights each)
+  static constexpr int RAW_BYTES = BN * 32, RAW_DMA = RAW_BYTES / 1024, Q4_WORDS = BN * 8 / NT;
+  static_assert(!Q4_ || (RAW_DMA <= NW && Q4_WORDS >= 1 && Q4_WORDS <= A_DMA && 8 % Q4_WORDS == 0), "Q4 tile shape");
   static constexpr int LDC = WTN + 8;
   // epilogue patches: the waves share out the stages evenly; split the wave tile's rows into
   // passes until the patches fit
@@ -110,7 +126,7 @@ struct TileF16NTDma {
   static constexpr int PASSES = patch_passes();
   static constexpr int PATCH_ROWS = WTM / PASSES;
   static constexpr int LDS_BYTES = 16;  // the kernel's generic buffer is unused
-  static constexpr int LDS_TOTAL = NSTAGE * STAGE_BYTES;
+  static constexpr int LDS_TOTAL = NSTAGE * STAGE_BYTES + (Q4_ ? 2 * RAW_BYTES : 0);
   static constexpr int TILE_ELEMS = BM * BN;
   static constexpr int NV4 = TM * TN * 4;
   static constexpr int CTAS_PER_CU_REGS = (NT >= 512 || TM * TN > 4) ? 1 : (TM * TN <= 2 ? 4 : 2);
@@ -118,7 +134,7 @@ struct TileF16NTDma {
   static constexpr int CTAS_PER_CU = CTAS_PER_CU_REGS < CTAS_PER_CU_LDS ? CTAS_PER_CU_REGS : CTAS_PER_CU_LDS;
   static constexpr int WAVES_PER_EU = CTAS_PER_CU * (NT / 64) / 4 > 0 ? CTAS_PER_CU * (NT / 64) / 4 : 1;
   static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "tile shape");
-  static_assert((A_BYTES / 1024) % NW == 0 && (B_BYTES / 1024) % NW == 0, "DMA groups must divide over the waves");
+  static_assert((A_BYTES / 1024) % NW == 0 && (Q4_ || (B_BYTES / 1024) % NW == 0), "DMA groups must divide over the waves");
   static_assert(NW % NSTAGE == 0, "a wave must keep to row groups of one parity; patches per stage");
   static_assert(PATCH_ROWS % 32 == 0, "epilogue pass must hold whole 32-row blocks");
   static_assert(F8 == 0 || TM % 2 == 0, "fp8: the wave tile's rows are processed in two halves");
@@ -204,7 +220,14 @@ struct TileF16NTDma {
     // matrix read as zero; columns past N are masked per lane (N % 8 == 0).
     uint4v rsrc_b;
     uint32_t voff_b, grp_b, kstep_b;
-    if (!B_KN) {
+    if constexpr (Q4_) {
+      // packed nibbles: ldb is the row pitch in bytes; a wave-wide load covers 32 rows x 32 bytes, lane l the
+      // 16-byte half l % 2 of row l / 2
+      rsrc_b = make_rsrc_words(reinterpret_cast<const char *>(a.B) + (int64_t)pn * BN * a.ldb, (uint32_t)(rows_b * a.ldb));
+      voff_b = (uint32_t)((32 * wave + (lane >> 1)) * a.ldb + (lane & 1) * 16);
+      grp_b = 0;
+      kstep_b = 32;
+    } else if (!B_KN) {
       rsrc_b = make_rsrc_words(a.B + (int64_t)pn * BN * a.ldb, (uint32_t)(rows_b * a.ldb * 2));
       voff_b = (uint32_t)(my_row * a.ldb + my_chunk * 8) * 2;
       grp_b = (uint32_t)(ROWS_PER_DMA * a.ldb * 2);
@@ -538,6 +561,122 @@ struct TileF16NTDma {
       if (it + 2 < n) iteration4(s2, s3, it + 2);
       // the (empty) loads of the iterations past the segment still write LDS: drain them before
       // the stages are handed to the epilogue / the next tile
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    } else if constexpr (Q4_) {
+      // ---- Q4 weights: the pipeline of the 16x16x32 fp16 kernel, B produced by a conversion step ----
+      char *s0 = stage(0), *s1 = stage(1);
+      char *raw0 = LdsArray<RAW_BYTES, 4>::get(), *raw1 = LdsArray<RAW_BYTES, 5>::get();
+      const Q4Consts qc = q4_consts(a.zero);
+      // this thread converts words [tid * Q4_WORDS, +Q4_WORDS) of the tile's BN x 8 words: one row's
+      const int cv_row = (tid * Q4_WORDS) >> 3, cv_c0 = (tid * Q4_WORDS) & 7;
+      const BufferRsrc rsrc_s = make_rsrc(a.scales + (int64_t)pn * BN * a.groups, (uint32_t)(rows_b * a.groups * 2));
+      const uint32_t voff_s = (uint32_t)(cv_row * a.groups * 2);
+      auto load_scale = [&](int kt) {  // the scale of this thread's row for K-iteration kt (zero past K or N)
+        return __builtin_bit_cast(half_t, (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(
+                                              rsrc_s, (kt * BK < a.K) ? voff_s : OOB_OFFSET, (uint32_t)(kt >> 1) * 2, 0));
+      };
+      auto raw_dma = [&](char *raw, int kt, bool dead) {
+        if (wave < RAW_DMA)
+          dma_load_16(rsrc_b, lds_address(raw) + wave * 1024, dead ? OOB_OFFSET : voff_b, (uint32_t)kt * kstep_b);
+      };
+      auto a_dma = [&](char *st, int kt, bool dead, int x) {
+        const int g = wave + x * NW;
+        dma_load_16(rsrc_a, lds_address(st) + g * 1024, dead ? OOB_OFFSET : voff_a, (uint32_t)kt * (BK * 2) + g * grp_a);
+      };
+      // word w of this thread: eight weights -> their 16-byte chunk of the B stage, in K order
+      auto convert_word = [&](char *st, uint32_t word, int w, half_t scale) {
+        union { half8v v; uint32_t u[4]; } d;
+        d.v = dequant_word_q4(word, qc, half2v{scale, scale});
+        uint4v o;  // (e0,e4)(e1,e5)(e2,e6)(e3,e7) -> (e0,e1)(e2,e3)(e4,e5)(e6,e7)
+        o[0] = __builtin_amdgcn_perm(d.u[1], d.u[0], 0x05040100u);
+        o[1] = __builtin_amdgcn_perm(d.u[3], d.u[2], 0x05040100u);
+        o[2] = __builtin_amdgcn_perm(d.u[1], d.u[0], 0x07060302u);
+        o[3] = __builtin_amdgcn_perm(d.u[3], d.u[2], 0x07060302u);
+        *reinterpret_cast<uint4v *>(st + A_BYTES + cv_row * ROW_BYTES + (((cv_c0 + w) ^ ((cv_row >> 1) & 7)) * 16)) = o;
+      };
+      typedef uint32_t rawv __attribute__((ext_vector_type(Q4_WORDS)));
+      auto read_raw = [&](const char *raw) {
+        rawv r;
+        if constexpr (Q4_WORDS == 1) r = rawv(*reinterpret_cast<const uint32_t *>(raw + tid * 4));
+        else r = *reinterpret_cast<const rawv *>(raw + tid * (Q4_WORDS * 4));
+        return r;
+      };
+      auto word_of = [&](const rawv &r, int w) {
+        if constexpr (Q4_WORDS == 1) return (uint32_t)r;
+        else return (uint32_t)r[w];
+      };
+      // the half-step behind the barrier: A loads of iteration kt_next into `cur`, nibble loads of iteration
+      // kt_next + 1, conversion of iteration kt_next (raw_cv -> cur's B rows), first fragments of `nxt`, MFMAs
+      auto tail_q4 = [&](char *cur, const char *nxt, const char *raw_cv, char *raw_ld, int kt_next, bool dead, bool dead1,
+                         half_t scale) {
+        constexpr int CH = A_DMA, NRD = FA + FN, NMF = FA * FN;
+        const rawv words = read_raw(raw_cv);
+#pragma unroll
+        for (int x = 0; x < CH; ++x) {
+#pragma unroll
+          for (int r = 0; r < NRD; ++r)
+            if (r * CH / NRD == x) {
+              if (r < FA)
+                fa[0][r] = *reinterpret_cast<const half8v *>(nxt + rd_a[0] + r * FROWS * ROW_BYTES);
+              else
+                read_b16_one(nxt, 0, 0, r - FA);
+            }
+          a_dma(cur, kt_next, dead, x);
+          if (x == 0) raw_dma(raw_ld, kt_next + 1, dead1);
+          if (x < Q4_WORDS) convert_word(cur, word_of(words, x), x, scale);
+#pragma unroll
+          for (int m = 0; m < NMF; ++m)
+            if (m * CH / NMF == x) mfma_one16(1, 1, 1, m);
+        }
+      };
+      half_t sc_next;  // scale for the conversion the next tail performs
+      auto iteration_q4 = [&](char *cur, char *nxt, char *raw_cv, char *raw_ld, int it) {
+        read_a16(cur, 1, 0, 1);
+        read_b16(cur, 1, 1);
+        mfma_half16(0, 0, 0);
+        interleave16<FA + FN, FA * FN / (FA + FN)>();
+        read_a16(cur, 0, 1, 0);
+        mfma_half16(1, 0, 1);
+        interleave16<FA, FN>();
+        read_a16(cur, 1, 1, 1);
+        mfma_half16(0, 1, 0);
+        interleave16<FA, FN>();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        wait_dma_then_barrier<0>();
+        const half_t sc = sc_next;
+        sc_next = load_scale(k0 + it + 3);
+        tail_q4(cur, nxt, raw_cv, raw_ld, k0 + it + 2, it + 2 >= n, it + 3 >= n, sc);
+      };
+      // prologue: nibbles of the first two iterations and A of the first; convert both; then the loads that a
+      // tail would have issued
+      raw_dma(raw0, k0, false);
+      raw_dma(raw1, k0 + 1, n < 2);
+#pragma unroll
+      for (int x = 0; x < A_DMA; ++x) a_dma(s0, k0, false, x);
+      {
+        const half_t sc0 = load_scale(k0), sc1 = load_scale(k0 + 1);
+        sc_next = load_scale(k0 + 2);
+        wait_dma_then_barrier<0>();
+        const rawv w0 = read_raw(raw0), w1 = read_raw(raw1);
+#pragma unroll
+        for (int w = 0; w < Q4_WORDS; ++w) {
+          convert_word(s0, word_of(w0, w), w, sc0);
+          convert_word(s1, word_of(w1, w), w, sc1);
+        }
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      wait_dma_then_barrier<0>();
+#pragma unroll
+      for (int x = 0; x < A_DMA; ++x) a_dma(s1, k0 + 1, n < 2, x);
+      raw_dma(raw0, k0 + 2, n < 3);
+      read_a16(s0, 0, 0, 0);
+      read_b16(s0, 0, 0);
+      int it = 0;
+      for (; it + 1 < n; it += 2) {
+        iteration_q4(s0, s1, raw0, raw1, it);
+        iteration_q4(s1, s0, raw1, raw0, it + 1);
+      }
+      if (it < n) iteration_q4(s0, s1, raw0, raw1, it);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     } else if constexpr (MFMA16) {
       // one K-iteration on stage `cur`: two K-steps of 32, each in two halves of the wave tile's

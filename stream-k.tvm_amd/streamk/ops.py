@@ -256,7 +256,19 @@ def _run_i8(A, B, C, config):
     _lib.check(rc, "sk_gemm_i8")
 
 
-Q4_MAX_M = 64  # rows of A the Q4 kernels take in one launch
+Q4_MAX_M = 64  # rows of A the weight-streaming Q4 kernels take in one launch
+Q4_FUSED_MAX_M = 1024  # up to here the Q4 tile kernels (dequantisation inside the GEMM) beat dequantise-then-GEMM
+_stagings = {}
+
+
+def _staging(nbytes, device):
+    """Scratch for dequantised weights: one buffer per (device, stream), grown on demand, never freed."""
+    key = (device.index if device.index is not None else torch.cuda.current_device(),
+           torch.cuda.current_stream().cuda_stream)
+    buf = _stagings.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = _stagings[key] = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    return buf
 
 
 def _zero_points(zeros, scales):
@@ -286,10 +298,11 @@ def _run_q4(A, Wq, scales, zeros, C, zero, group, tiled, config, bias, activatio
     if tuple(scales.shape) != (N, K // group) or not scales.is_contiguous():
         raise ValueError(f"scales must be contiguous [N, K/group]; got {tuple(scales.shape)}")
     _check_out(C, M, N, torch.float16)
-    if M > Q4_MAX_M and not config.startswith("#"):
-        # the Q4 kernels stream the weights past at most 64 rows of A.  Up to 256 rows: one launch
-        # per block of 64 rows.  Beyond: dequantise once (bit-exact device function) and run the
-        # fp16 tile kernels, whose time then dwarfs the extra pass over the weights.
+    if M > Q4_MAX_M and (zeros is not None or tiled) and not config.startswith("#"):
+        # The weight-streaming kernels take at most 64 rows of A; beyond that row-major weights with a scalar zero
+        # point go to the Q4 tile kernels (below, like any other plan).  Per-group zero points and the tiled
+        # layout have no tile kernel: up to 256 rows one launch per block of 64 rows, beyond that the weights are
+        # dequantised once (bit-exact device function) for the fp16 tile kernels.
         if M <= 4 * Q4_MAX_M:
             for m0 in range(0, M, Q4_MAX_M):
                 _run_q4(A[m0:m0 + Q4_MAX_M], Wq, scales, zeros, C[m0:m0 + Q4_MAX_M], zero, group, tiled, config,
@@ -299,6 +312,16 @@ def _run_q4(A, Wq, scales, zeros, C, zero, group, tiled, config, bias, activatio
             raise ValueError("more than 256 rows of A need the row-major weights (they are dequantised once)")
         W = torch.empty((N, K), dtype=torch.float16, device=Wq.device)
         _run_dequant_q4(Wq, scales, zeros, W, zero, group)
+        _run_16bit(A, W, C, "nt", "", bias, activation, torch.float16, "float16")
+        return
+    if M > Q4_FUSED_MAX_M and config == "":
+        # Prefill-sized calls: one pass that dequantises the weights (bit-exact device function) into a staging
+        # buffer kept per stream, then the fp16 tile kernels on it.  The pass costs 26 us for 8192 x 8192 weights,
+        # under 7 % of the product from 4096 rows on, where the fused Q4 tile kernels (the register-limited
+        # eight-wave form) are 20-25 % behind the four-wave fp16 kernel.  The buffer is allocated on first use and
+        # kept: no allocation per call.
+        W = _staging(N * K * 2, A.device).view(torch.float16)[:N * K].view(N, K)
+        _run_dequant_q4(Wq, scales, None, W, zero, group)
         _run_16bit(A, W, C, "nt", "", bias, activation, torch.float16, "float16")
         return
     name = "q4_zp" if zeros is not None else ("q4_tiled" if tiled else "q4")

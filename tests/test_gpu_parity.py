@@ -302,6 +302,86 @@ def test_q4_ragged_shapes_every_kernel(sk, oracle, variant):
     sk.workspace_status()
 
 
+def test_q4_tile_kernels_more_than_64_rows(sk, oracle):
+    """Q4 weights with more rows of A than the weight-streaming kernels take: the tile kernels that dequantise B
+    in registers on its way into the LDS stage (the reference dequantises right before the MMA,
+    streamk_fp16_ladder_block_reduce_q4.py:283-294).  Every tile shape, schedule and fix-up on ragged shapes and
+    zero points 0 / 5 / 8 / 15: exact on integer data with unit scales (any wrong nibble, K order or scale row
+    shows), within 2e-3 of the oracle on random data; the weights the kernel multiplies are the bit-exact ones
+    (it must equal the fp16 kernel of the same tile on sk_dequant_q4's output bit for bit)."""
+    import torch
+    rng = np.random.default_rng(53)
+    ran = 0
+    for (M, N, K, zero) in [(128, 128, 128, 8), (200, 136, 384, 5), (300, 520, 1152, 0), (1000, 1096, 4096, 8), (65, 72, 128, 15)]:
+        Ai = rng.integers(-1, 2, (M, K)).astype(np.float16)
+        Wq = rng.integers(0, 256, (N, K // 2), dtype=np.uint8)
+        exact = Ai.astype(np.int64) @ (oracle.unpack_q4_np(Wq).astype(np.int64) - zero).T
+        ones = torch.ones(N, K // 128, dtype=torch.float16, device="cuda")
+        sc = rng.uniform(0.005, 0.02, (N, K // 128)).astype(np.float16)
+        Ar = (rng.random((M, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+        ref = oracle.q4_gemm_ref(Ar, Wq, sc, 128, zero)
+        dAi, dAr, dW, dS = _t(Ai), _t(Ar), _t(Wq), _t(sc)
+        W16 = sk.dequant_q4(dW, dS, zero=zero)
+        for (bm, bn) in ((128, 128), (256, 128), (256, 256)):
+            for sch in (dict(schedule="dp"), dict(schedule="basic", fixup="reduce", grid=7),
+                        dict(schedule="basic", fixup="atomic", grid=5), dict(schedule="sk2", fixup="reduce", grid=3)):
+                plan = sk.make_plan(M, N, K, "q4", "nt", dict(bm=bm, bn=bn, **sch))
+                assert sk.kernel_name(plan.kernel_id) == f"tile_q4_nt_dma16_{bm}x{bn}x64"
+                C = sk.streamk_q4(dAi, dW, ones, zero=zero, plan=plan)
+                assert np.array_equal(C.cpu().numpy().astype(np.int64), exact), (M, N, K, zero, bm, bn, sch)
+                C = sk.streamk_q4(dAr, dW, dS, zero=zero, plan=plan)
+                assert _rel(oracle, C, ref) <= 2e-3 <= TOL, (M, N, K, zero, bm, bn, sch)
+                if sch.get("fixup") != "atomic":
+                    twin = sk.streamk_fp16(dAr, W16, **dict(sch, bm=bm, bn=bn, bk=64, variant=5))
+                    assert torch.equal(C, twin), (M, N, K, zero, bm, bn, sch)
+                ran += 1
+    assert ran == 60
+    # the planner's own choice, bias and activation in the epilogue
+    M, N, K = 300, 520, 1152
+    A = rng.integers(-1, 2, (M, K)).astype(np.float16)
+    Wq = rng.integers(0, 256, (N, K // 2), dtype=np.uint8)
+    bias = rng.integers(-3, 4, N).astype(np.float16)
+    want = np.maximum(A.astype(np.int64) @ (oracle.unpack_q4_np(Wq).astype(np.int64) - 8).T + bias.astype(np.int64), 0)
+    C = sk.streamk_q4(_t(A), _t(Wq), torch.ones(N, K // 128, dtype=torch.float16, device="cuda"), bias=_t(bias), activation="relu")
+    assert np.array_equal(C.cpu().numpy().astype(np.int64), want)
+    sk.workspace_status()
+
+
+def test_q4_prefill_sizes_at_full_width(sk, oracle):
+    """N = K = 8192, M = 128 / 512 / 4096 (the fused tile kernels up to 1024 rows, beyond that one dequantisation
+    pass into a per-stream staging buffer and the fp16 tile kernels): a sample of rows within 2e-3 of the oracle,
+    exact integer checksums, and no allocation once the first call of a size has run."""
+    import torch
+    N = K = 8192
+    rng = np.random.default_rng(54)
+    Wq = rng.integers(0, 256, (N, K // 2), dtype=np.uint8)
+    sc = rng.uniform(0.005, 0.02, (N, K // 128)).astype(np.float16)
+    W = oracle.dequant_q4(Wq, sc, 128, 8).astype(np.float32)
+    q8 = oracle.unpack_q4_np(Wq).astype(np.int64) - 8
+    dW, dS = _t(Wq), _t(sc)
+    ones = torch.ones(N, K // 128, dtype=torch.float16, device="cuda")
+    for M in (128, 512, 4096):
+        A = rng.standard_normal((M, K), dtype=np.float32).astype(np.float16)
+        dA = _t(A)
+        C = sk.streamk_q4(dA, dW, dS)
+        rows = np.sort(rng.choice(M, 48, replace=False))
+        ref = A[rows].astype(np.float32) @ W.T
+        assert oracle.max_abs_rel(C[torch.from_numpy(rows).cuda()].float().cpu().numpy(), ref) <= 2e-3 <= TOL, M
+        torch.cuda.synchronize()
+        before = torch.cuda.memory_allocated()
+        out = torch.empty_like(C)
+        after_out = torch.cuda.memory_allocated()
+        sk.streamk_q4(dA, dW, dS, out=out)
+        torch.cuda.synchronize()
+        assert torch.cuda.memory_allocated() == after_out and torch.equal(out, C), M   # nothing allocated inside the call
+        del out
+        Ai = rng.integers(-1, 2, (M, K)).astype(np.int8)
+        Ci = sk.streamk_q4(_t(Ai.astype(np.float16)), dW, ones).double()
+        assert np.array_equal(Ci.sum(dim=1).cpu().numpy().astype(np.int64), Ai.astype(np.int64) @ q8.sum(axis=0)), M
+        assert np.array_equal(Ci.sum(dim=0).cpu().numpy().astype(np.int64), Ai.astype(np.int64).sum(axis=0) @ q8.T), M
+    sk.workspace_status()
+
+
 def test_q4_per_group_zero_points(sk, oracle):
     """Q4 with one zero point per scale group and row: device dequantisation bit for bit against the
     oracle; the GEMM on every kernel instance, ragged shapes, all schedules, within 2e-3 of the fp32 host
@@ -665,11 +745,16 @@ def test_bf16_small_m_kernels(sk, oracle):
         A, W = (torch.rand(M, 4096) * 2 - 1).bfloat16(), (torch.rand(4096, 4096) * 2 - 1).bfloat16()
         ref = oracle.matmul_fp32(A.float().numpy(), W.float().numpy(), trans_b=True)
         assert _rel(oracle, sk.streamk_bf16(A.cuda(), W.cuda()), ref) <= 4e-3, M
-    # a shape tuned for fp16 only: the bfloat16 plan takes that entry (its kernel has a bfloat16 twin)
-    if sk.tuned_config(256, 4096, 4096, "bfloat16") is None and sk.tuned_config(256, 4096, 4096, "float16"):
-        want = sk.make_plan(256, 4096, 4096, "float16")
-        got = sk.make_plan(256, 4096, 4096, "bfloat16")
-        assert (got.bm, got.bn, got.bk, got.grid, got.schedule) == (want.bm, want.bn, want.bk, want.grid, want.schedule)
+    # a shape tuned for fp16 only: the bfloat16 plan takes that entry where its kernel has a bfloat16 twin
+    for shape in ((256, 4096, 4096), (16, 4096, 4096), (2048, 8192, 8192)):
+        cfg = sk.tuned_config(*shape, "float16")
+        if sk.tuned_config(*shape, "bfloat16") is None and cfg:
+            try:
+                want = sk.make_plan(*shape, "bfloat16", "nt", cfg)
+            except sk.StreamKError:
+                continue  # no bfloat16 instance of that kernel: the heuristic plans the shape
+            got = sk.make_plan(*shape, "bfloat16")
+            assert (got.kernel_id, got.grid, got.schedule) == (want.kernel_id, want.grid, want.schedule), shape
     sk.workspace_status()
 
 
