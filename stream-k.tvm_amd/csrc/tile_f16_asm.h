@@ -15,7 +15,7 @@
 // and stay far below 256 architectural registers, so it has no reason to (the build checks the generated
 // assembly for accumulation-register instructions outside the hand-written blocks).
 //
-// Restrictions: NT layout, K a multiple of 64.
+// Restrictions: NT layout, K a multiple of 64 (int8: of 128 bytes).
 #pragma once
 #include "sk_device.h"
 #include "tile_f16.h"
@@ -43,9 +43,13 @@ __device__ __forceinline__ void agpr_write4(floatx4 x) {
       : "v"(x[0]), "v"(x[1]), "v"(x[2]), "v"(x[3]), "n"(R), "n"(R + 1), "n"(R + 2), "n"(R + 3));
 }
 
-template <bool BF16_ = false>
+// MODE_: 0 fp16, 1 bfloat16, 2 int8 (int32 C; the bytes travel as pairs, so K and the leading dimensions of A
+// and B arrive in 16-bit units and the loop is the fp16 one with v_mfma_i32_16x16x64_i8 on the same fragments)
+template <int MODE_ = 0>
 struct TileF16Asm {
   typedef GemmArgs Args;
+  static constexpr bool BF16_ = MODE_ == 1, I8 = MODE_ == 2;
+  typedef int intx4 __attribute__((ext_vector_type(4)));
   static constexpr bool LEAN_ENTRY = true;  // see run_persistent
   static constexpr int BM = 256, BN = 256, BK = 64, WM = 2, WN = 2, NW = 4, NT = 256;
   static constexpr int WTM = 128, WTN = 128, FM = 8, FN = 8;  // wave tile; 16 x 16 accumulator blocks per wave
@@ -87,7 +91,13 @@ struct TileF16Asm {
     uint32_t ra0 = base + (uint32_t)(wm * WTM + (lane & 15)) * ROW_BYTES + pos0, ra1 = ra0 ^ 64;
     uint32_t rb0 = base + A_BYTES + (uint32_t)(wn * WTN + (lane & 15)) * ROW_BYTES + pos0, rb1 = rb0 ^ 64;
     const uint32_t iters = (uint32_t)n;
-    if constexpr (BF16_) {
+    if constexpr (I8) {
+      asm volatile(SK_TILE_ASM_LOOP("v_mfma_i32_16x16x64_i8")
+                   : [ra0] "+v"(ra0), [ra1] "+v"(ra1), [rb0] "+v"(rb0), [rb1] "+v"(rb1)
+                   : [rsa] "s"(rsrc_a), [rsb] "s"(rsrc_b), [voa] "v"(voff_a), [vob] "v"(voff_b), [ga0] "s"(goff_a),
+                     [gb0] "s"(goff_b), [gas] "s"(gstep_a), [gbs] "s"(gstep_b), [n] "s"(iters), [lds] "s"(lds_wave)
+                   : "memory", "m0", "scc", SK_TILE_ASM_CLOBBERS);
+    } else if constexpr (BF16_) {
       asm volatile(SK_TILE_ASM_LOOP("v_mfma_f32_16x16x32_bf16")
                    : [ra0] "+v"(ra0), [ra1] "+v"(ra1), [rb0] "+v"(rb0), [rb1] "+v"(rb1)
                    : [rsa] "s"(rsrc_a), [rsb] "s"(rsrc_b), [voa] "v"(voff_a), [vob] "v"(voff_b), [ga0] "s"(goff_a),
@@ -128,6 +138,30 @@ struct TileF16Asm {
     const int act = BIAS ? epi_act(epi) : 0;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
+    if constexpr (I8) {
+      // int32 C straight from the accumulators: lane l of block (ii, j) holds row 16 ii + l % 16, columns
+      // 16 j + 4 (l / 16) .. + 3
+      int *C = reinterpret_cast<int *>(a.C);
+      const bool vec_ok = (a.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(a.C) & 15) == 0);
+      const int row0 = pm * BM + wm * WTM + (lane & 15), col0 = pn * BN + wn * WTN + 4 * (lane >> 4);
+      static_for<ROW_BEGIN / 16, ROW_BEGIN / 16 + NPASS * (PATCH_ROWS / 16)>([&](auto blk) {
+        constexpr int ii = decltype(blk)::value;
+        static_for<0, FN>([&](auto col) {
+          constexpr int j = decltype(col)::value;
+          const intx4 x = __builtin_bit_cast(intx4, agpr_read4<(ii * FN + j) * 4>());
+          const int grow = row0 + 16 * ii, gcol = col0 + 16 * j;
+          if (grow < a.M && gcol < a.N) {
+            int *dst = C + (int64_t)grow * a.ldc + gcol;
+            if (vec_ok && gcol + 4 <= a.N) {
+              *reinterpret_cast<intx4 *>(dst) = x;
+            } else {
+              for (int e = 0; e < 4 && gcol + e < a.N; ++e) dst[e] = x[e];
+            }
+          }
+        });
+      });
+      return;
+    }
     const int bias_col0 = BIAS ? pn * BN + wn * WTN + pin_here(lane >> 4) * 4 : 0;
     half_t *patch = reinterpret_cast<half_t *>(lds() + wave * (LDS_TOTAL / NW));
     const bool vec_ok = (a.ldc % 8 == 0) && ((reinterpret_cast<uintptr_t>(a.C) & 15) == 0);
@@ -203,8 +237,13 @@ struct TileF16Asm {
     const uint32_t off = (uint32_t)pin_here((int)threadIdx.x) * 16;
     static_for<V0, V1>([&](auto g) {
       constexpr int v = decltype(g)::value;
-      const floatx4 x = __builtin_bit_cast(floatx4, ld_coherent16(r, off, (uint32_t)v * NT * 16));
-      agpr_write4<v * 4>(agpr_read4<v * 4>() + x);
+      const uint4v raw = ld_coherent16(r, off, (uint32_t)v * NT * 16);
+      if constexpr (I8) {
+        const intx4 sum = __builtin_bit_cast(intx4, agpr_read4<v * 4>()) + __builtin_bit_cast(intx4, raw);
+        agpr_write4<v * 4>(__builtin_bit_cast(floatx4, sum));
+      } else {
+        agpr_write4<v * 4>(agpr_read4<v * 4>() + __builtin_bit_cast(floatx4, raw));
+      }
     });
   }
   static __device__ __forceinline__ void store_partial(const Acc &, float *dst) { store_groups<0, NV4>(dst); }
@@ -222,8 +261,14 @@ struct TileF16Asm {
     static_for<0, NV4>([&](auto g) {
       constexpr int v = decltype(g)::value;
       const floatx4 x = agpr_read4<v * 4>();
+      const intx4 xi = __builtin_bit_cast(intx4, x);  // (the whole vector: a bit cast of one element reads element 0)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) atomic_add_f32(dst + (size_t)(v * 4 + e) * NT, x[e]);
+      for (int e = 0; e < 4; ++e) {
+        if constexpr (I8)
+          atomic_add_i32(reinterpret_cast<int *>(dst) + (size_t)(v * 4 + e) * NT, xi[e]);
+        else
+          atomic_add_f32(dst + (size_t)(v * 4 + e) * NT, x[e]);
+      }
     });
   }
   // reads the completed sum and leaves zeros behind

@@ -969,6 +969,26 @@ def test_int8_tile_kernels(sk, oracle):
                 assert plan.bk == 128 and plan.iters_per_tile == -(-K // 128)
                 C = sk.streamk_int8(dA, dB, plan=plan)
                 assert C.dtype == torch.int32 and torch.equal(C.cpu().long(), ref), (M, N, K, bm, bn, sch)
+    # the four-wave kernel with the K loop in assembly (K a multiple of 128): every schedule, both fix-ups, the
+    # halves exchange of a tile split in two
+    assert sk.kernel_name(sk.make_plan(4096, 4096, 4096, "int8", "nt", use_tuned=False).kernel_id) == "tile_i8_nt_asm_256x256x128"
+    assert "asm" not in sk.kernel_name(sk.make_plan(4096, 4096, 4112, "int8", "nt", use_tuned=False).kernel_id)
+    for (M, N, K) in [(256, 256, 128), (200, 136, 384), (1000, 1096, 2048), (520, 264, 896)]:
+        A = torch.randint(-128, 128, (M, K), dtype=torch.int8)
+        B = torch.randint(-128, 128, (N, K), dtype=torch.int8)
+        ref = torch.from_numpy(oracle.i8_gemm_ref(A.numpy(), B.numpy()))
+        dA, dB = A.cuda(), B.cuda()
+        for sch in (dict(schedule="dp"), dict(schedule="basic", fixup="reduce", grid=7), dict(schedule="basic", fixup="atomic", grid=5),
+                    dict(schedule="sk2", fixup="reduce", grid=3), dict(schedule="splitk", split=2, fixup="reduce"),
+                    dict(schedule="splitk", split=2, fixup="atomic"), dict(schedule="sk1", fixup="reduce", grid=2, raster=2)):
+            try:
+                plan = sk.make_plan(M, N, K, "int8", "nt", dict(bm=256, bn=256, variant=8, **sch))
+            except sk.StreamKError:
+                assert sch["schedule"] == "splitk"
+                continue
+            assert sk.kernel_name(plan.kernel_id) == "tile_i8_nt_asm_256x256x128"
+            C = sk.streamk_int8(dA, dB, plan=plan)
+            assert torch.equal(C.cpu().long(), ref), (M, N, K, sch)
     # heuristic plans; extreme values (K * 128 * 128 stays below 2^31)
     for (M, N, K) in [(1, 512, 1024), (16, 4096, 4096), (2048, 2048, 2048), (1024, 8192, 8192)]:
         A = torch.randint(-128, 128, (M, K), dtype=torch.int8)
