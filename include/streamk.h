@@ -269,8 +269,11 @@ int sk_gemm_f32(const void *A, const void *B, void *C, int64_t M, int64_t N, int
  * scale to fp32 group sums, i.e. they use the unrounded (q - zero) * scale: at least as close to
  * the exact product as the rounded-weight form (within 2^-11 relative per weight of it).
  * sk_dequant_q4 and the M > 1 kernels produce the rounded weights bit for bit.
+ * Up to 64 rows of A the plan is a weight-streaming kernel; for more rows (plan dtype SK_Q4) it is a tile kernel
+ * that moves the nibbles through LDS and dequantises them, bit for bit as above, on their way into the fp16
+ * stage of the 16x16x32 MFMA loop (256x256, 256x128 or 128x128 tiles; every schedule and fix-up).
  * A plan made with dtype SK_Q4_TILED takes Wq in the tiled layout instead (see sk_q4_tile_host): same
- * results bit for bit, the weights stream faster.
+ * results bit for bit, the weights stream faster; at most 64 rows of A per call.
  */
 int sk_gemm_q4(const void *A, const void *Wq, const void *scales, void *C, int64_t M, int64_t N,
                int64_t K, int64_t lda, int64_t ldc, int group, int zero, const sk_plan *plan,
