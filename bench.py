@@ -126,6 +126,37 @@ def main():
     err = oracle.max_abs_rel(C[:64].float().cpu().numpy(), ref)
     assert err <= 1e-2, err
 
+    # What the matrix pipes alone sustain on this box, in this process, right after the timed steps (the device
+    # is at its sustained clock): a loop of nothing but 16x16x32 fp16 MFMAs on U[-1,1) register operands, ~40 ms
+    # untimed, then ~40 ms timed.  The published peak assumes the maximum clock; this is the part's own ceiling.
+    def mfma_only(shape):
+        import ctypes
+        L = streamk.lib()
+        scratch = torch.empty(cus * 256, dtype=torch.float32, device="cuda")
+        flop = ctypes.c_double(0.0)
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        iters = 4000  # ~2.5 ms per launch
+        def launch():
+            rc = L.sk_diag_mfma_only(shape, iters, 0, scratch.data_ptr(), scratch.numel() * 4, stream, ctypes.byref(flop))
+            assert rc == 0, rc
+        for _ in range(16):
+            launch()
+        st, en = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        st.record()
+        for _ in range(16):
+            launch()
+        en.record()
+        torch.cuda.synchronize()
+        return flop.value / (st.elapsed_time(en) / 16 * 1e-3) / 1e12
+    mfma_only_tflops = mfma_only(1)
+    # ... and the vendor's kernel for the same product, same operands, same moment (hipBLASLt through torch.matmul)
+    vendor = lambda: torch.matmul(A, B.t(), out=C)  # noqa: E731
+    for _ in range(10):
+        vendor()
+    torch.cuda.synchronize()
+    vendor_ms, _ = time_eager(vendor, 5, max(10, args.steps // 2))
+    step()  # C holds this library's result again
+
     # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/)
     traffic = None
     tpath = os.path.join(ROOT, "profiles", f"traffic_{streamk.kernel_name(plan.kernel_id)}_8192.json")
@@ -145,7 +176,10 @@ def main():
         "roofline": {"bound": "mfma", "achieved": round(kernel_tflops, 2), "peak": PEAK_FP16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(kernel_tflops / PEAK_FP16_TFLOPS, 4),
                      "traffic": traffic, "kernel": streamk.kernel_name(plan.kernel_id),
-                     "avg_launch_ms": round(ev_ms, 5)},
+                     "avg_launch_ms": round(ev_ms, 5),
+                     "mfma_only_tflops": round(mfma_only_tflops, 1),
+                     "frac_of_mfma_only": round(kernel_tflops / mfma_only_tflops, 4),
+                     "vendor_matmul_tflops": round(flops / (vendor_ms * 1e-3) / 1e12, 1)},
     }
 
     # ---------------------------------------------------------------- CPU baseline (oracle, bounded)
@@ -388,6 +422,24 @@ def main():
                 del tiles
             q4.append(row)
         extra["q4_N8192_K8192"] = q4
+        # more rows of A than the weight-streaming kernels take: the Q4 tile kernels (nibbles dequantised on their
+        # way into the LDS stage), the staged path (dequantise once, fp16 tile kernels) and the fp16 product alone
+        pre = []
+        Wd = streamk.dequant_q4(Wq, sc)
+        for m in (128, 512, 1024, 4096):
+            a = torch.randn(m, K, generator=g).half().cuda()
+            c = torch.empty(m, N, dtype=torch.float16, device="cuda")
+            p = streamk.make_plan(m, N, K, "q4", "nt")
+            fl = 2.0 * m * N * K
+            t_tile = time_graph(lambda: streamk.streamk_q4(a, Wq, sc, out=c, plan=p), launches=10, replays=5)
+            t_auto = time_graph(lambda: streamk.streamk_q4(a, Wq, sc, out=c), launches=10, replays=5)
+            t_f16 = time_graph(lambda: streamk.streamk_fp16(a, Wd, out=c), launches=10, replays=5)
+            pre.append({"M": m, "kernel": streamk.kernel_name(p.kernel_id),
+                        "q4_tile_kernel": {"us": round(t_tile * 1e3, 1), "tflops": round(fl / t_tile / 1e9, 1)},
+                        "streamk_q4_default": {"us": round(t_auto * 1e3, 1), "tflops": round(fl / t_auto / 1e9, 1)},
+                        "fp16_product_alone": {"us": round(t_f16 * 1e3, 1), "tflops": round(fl / t_f16 / 1e9, 1)}})
+        del Wd
+        extra["q4_prefill_N8192_K8192"] = pre
 
         # fp16 matrix-vector product at an LLM-sized weight matrix (470 MB: every launch streams it from HBM)
         nv, kv = 28672, 8192

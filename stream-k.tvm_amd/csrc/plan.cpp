@@ -82,10 +82,13 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
   // (one-byte operands: up to 64 rows -- their tile kernels start at 128 rows)
   const bool one_byte = dtype == SK_F8E4M3 || dtype == SK_F8E5M2 || dtype == SK_I8;
   if (dtype == SK_Q4 && M > 64 && want_variant < 0) {
-    // more rows than the weight-streaming kernels take: the tile kernels that dequantise B on its way into LDS;
-    // the largest tile that still gives most CUs one
-    const int64_t t256 = cdiv(M, 256) * cdiv(N, 256), t256x128 = cdiv(M, 256) * cdiv(N, 128);
-    const int want_bm = t256x128 * 4 >= (int64_t)num_cus * 3 ? 256 : 128;
+    // more rows than the weight-streaming kernels take: the tile kernels that dequantise B on its way into LDS.
+    // 256 rows of A per tile as soon as M has them: a CTA decodes its BN weight rows whatever BM is, and the
+    // four-wave 128 x 128 kernel waits for its loads (one wave per SIMD, a short iteration), so a 256 x 128 tile
+    // takes no longer than a 128 x 128 one; where that leaves CUs without a tile the Stream-K schedule splits K
+    // (N = K = 8192, M = 512: 73 us against 109 us on 128 x 128 tiles).  256 x 256 when those fill the device.
+    const int64_t t256 = cdiv(M, 256) * cdiv(N, 256);
+    const int want_bm = M > 128 ? 256 : 128;
     const int want_bn = (want_bm == 256 && t256 * 4 >= (int64_t)num_cus * 3) ? 256 : 128;
     for (int i = 0; i < n; ++i)
       if (t[i].family == FAMILY_TILE && t[i].dtype == SK_Q4 && t[i].bm == want_bm && t[i].bn == want_bn) return &t[i];
