@@ -22,10 +22,18 @@ One iteration (stage `cur` of the two 64 KB LDS stages holds its tiles, `nxt` th
             every wave has finished reading) and the 16 fragment reads of K-step 0 of nxt
 The loads of iterations past the segment get an out-of-range offset (they fetch nothing and zero a stage
 nobody reads), so the loop has no branch but its own back edge.
+
+NN layout (B is [K, N] row-major; SK_TILE_ASM_LOOP_NN): the B half of a stage is 64 K-rows of 512 bytes, a
+wave-wide load fills two of them (row group g = wave + 4 x: K-rows 2 g, 2 g + 1), 16-byte chunk c of K-row k sits
+at position c ^ (4 (k & 3)) ^ (2 ((k >> 3) & 1)).  Bit 3 of a lane's K-row is the parity of x, so the lane fetches
+one of two global chunks: v121 for even x, v122 for odd x.  A 16-column block of B is read with two transposing
+8-byte reads per K-step (K-rows 8 g' .. + 3 and + 4 .. + 7 for lane group g'), from one address register per block
+(%[rbt0] .. %[rbt7]; the swizzle makes the blocks' addresses differ by an XOR, not a sum): K-step 1 is 32 rows =
+16384 bytes further.  Per iteration the global offset of B advances by %[kbs] = 64 rows.
 """
 
 A0, B0, A1, B1 = 128, 160, 192, 224     # first registers of the fragment buffers
-VOA, VOB = 120, 121                     # v120 / v121: load offsets of this iteration
+VOA, VOB, VOB1 = 120, 121, 122          # v120 / v121 (/ v122, NN: odd row groups of B): load offsets of this iteration
 S_IT, S_KA, S_KB, S_T, S_OOB, S_M0, S_LDS, S_T2 = 80, 81, 82, 83, 84, 85, 86, 87
 
 
@@ -38,13 +46,25 @@ def mfma(lines, i, j, a_base, b_base):
     emit(lines, f'MF " a[{c}:{c + 3}], v[{b_base + 4 * j}:{b_base + 4 * j + 3}], v[{a_base + 4 * i}:{a_base + 4 * i + 3}], a[{c}:{c + 3}]')
 
 
-def frag_read(lines, f, a_base, b_base, addr_a, addr_b):
-    """fragment f: 0..7 blocks of A, 8..15 blocks of B; 16 rows of 128 bytes per block"""
+NN = False   # set by main() while it writes the NN form of the loop
+
+
+def frag_read(lines, f, a_base, b_base, addr_a, addr_b, kk=0):
+    """fragment f: 0..7 blocks of A, 8.. blocks of B; 16 rows of 128 bytes per block.  NN: f = 8 + 2 g + h is
+    half h of block g of B, four K-rows of K-step kk"""
     if f < 8:
         emit(lines, f'"ds_read_b128 v[{a_base + 4 * f}:{a_base + 4 * f + 3}], {addr_a} offset:{f * 2048}')
-    else:
+    elif not NN:
         g = f - 8
         emit(lines, f'"ds_read_b128 v[{b_base + 4 * g}:{b_base + 4 * g + 3}], {addr_b} offset:{g * 2048}')
+    else:
+        g, h = (f - 8) // 2, (f - 8) % 2
+        r = b_base + 4 * g + 2 * h
+        emit(lines, f'"ds_read_b64_tr_b16 v[{r}:{r + 1}], %[rbt{g}] offset:{kk * 16384 + h * 2048}')
+
+
+def n_frags():
+    return 24 if NN else 16
 
 
 def dma(lines, x, first):
@@ -61,7 +81,8 @@ def dma(lines, x, first):
         emit(lines, f'"buffer_load_dwordx4 v{VOA}, %[rsa], s{S_T} offen lds')
         emit(lines, f'"s_add_u32 s{S_T}, s{S_T}, %[gas]')
     else:
-        emit(lines, f'"buffer_load_dwordx4 v{VOB}, %[rsb], s{S_T} offen lds')
+        vob = VOB1 if (NN and x % 2 == 1) else VOB
+        emit(lines, f'"buffer_load_dwordx4 v{vob}, %[rsb], s{S_T} offen lds')
         emit(lines, f'"s_add_u32 s{S_T}, s{S_T}, %[gbs]')
 
 
@@ -72,6 +93,8 @@ def offsets_for(lines, ahead):
     emit(lines, f'"s_cselect_b32 s{S_OOB}, 0, 0x80000000')
     emit(lines, f'"v_or_b32 v{VOA}, s{S_OOB}, %[voa]')
     emit(lines, f'"v_or_b32 v{VOB}, s{S_OOB}, %[vob]')
+    if NN:
+        emit(lines, f'"v_or_b32 v{VOB1}, s{S_OOB}, %[vob1]')
 
 
 def mfma_order():
@@ -90,7 +113,10 @@ def slots(count, total, first, every):
     return out
 
 
-def main():
+def loop_text(nn):
+    """the lines of the loop for the NT (nn = False) or the NN layout"""
+    global NN
+    NN = nn
     import os
     # where the fragment reads and the loads ride along the 64 MFMAs of a block (tunables of the schedule)
     # (measured at 8192^3 on random operands, each against the eight-wave kernel in the same run: the defaults
@@ -98,9 +124,17 @@ def main():
     # at the texture addresser, and with one wave per SIMD that is a stalled matrix pipe; loads every third slot
     # 1.05 x; later or denser fragment reads, a partial wait at the loop top, MFMAs issued ahead of the barrier:
     # within 1 % of the defaults.  The same loop on four 32 KB buffers with a barrier per K-step of 32: 1.00 x.)
-    rd0 = slots(16, 64, int(os.environ.get("SK_ASM_RD0_FIRST", 0)), int(os.environ.get("SK_ASM_RD0_EVERY", 3)))
-    rd1 = slots(16, 64, int(os.environ.get("SK_ASM_RD1_FIRST", 1)), int(os.environ.get("SK_ASM_RD1_EVERY", 4)))
+    # NN: 8 + 16 reads per K-step, on the even slots; the loads keep the odd slots 3, 7, ...
+    nf = n_frags()
+    if nn:
+        rd0 = slots(nf, 64, 0, 2)
+        rd1 = slots(nf, 64, 0, 2)
+    else:
+        rd0 = slots(nf, 64, int(os.environ.get("SK_ASM_RD0_FIRST", 0)), int(os.environ.get("SK_ASM_RD0_EVERY", 3)))
+        rd1 = slots(nf, 64, int(os.environ.get("SK_ASM_RD1_FIRST", 1)), int(os.environ.get("SK_ASM_RD1_EVERY", 4)))
     ld1 = slots(16, 64, int(os.environ.get("SK_ASM_LD1_FIRST", 3)), int(os.environ.get("SK_ASM_LD1_EVERY", 4)))
+    kb_step = "%[kbs]" if nn else "128"
+    frag_addrs = ["%[ra0]", "%[ra1]"] + ([f"%[rbt{g}]" for g in range(8)] if nn else ["%[rb0]", "%[rb1]"])
     L = []
     # ---- accumulators start at zero
     for r in range(256):
@@ -114,18 +148,18 @@ def main():
     for x in range(16):
         dma(L, x, True)
     emit(L, f'"s_add_u32 s{S_KA}, s{S_KA}, 128')
-    emit(L, f'"s_add_u32 s{S_KB}, s{S_KB}, 128')
+    emit(L, f'"s_add_u32 s{S_KB}, s{S_KB}, {kb_step}')
     emit(L, f'"s_xor_b32 s{S_LDS}, s{S_LDS}, 0x10000')
     offsets_for(L, 1)
     for x in range(16):
         dma(L, x, False)
     emit(L, f'"s_add_u32 s{S_KA}, s{S_KA}, 128')
-    emit(L, f'"s_add_u32 s{S_KB}, s{S_KB}, 128')
+    emit(L, f'"s_add_u32 s{S_KB}, s{S_KB}, {kb_step}')
     emit(L, f'"s_xor_b32 s{S_LDS}, s{S_LDS}, 0x10000')
     emit(L, '"s_waitcnt vmcnt(16)')
     emit(L, '"s_barrier')
-    for f in range(16):
-        frag_read(L, f, A0, B0, "%[ra0]", "%[rb0]")
+    for f in range(nf):
+        frag_read(L, f, A0, B0, "%[ra0]", "%[rb0]", 0)
     emit(L, '"s_nop 7')   # accumulator writes above are long done; cheap insurance before the first MFMA
     # ---- the loop
     emit(L, '"L_sk_loop%=:')
@@ -140,7 +174,7 @@ def main():
             emit(L, '"s_waitcnt lgkmcnt(0)')
         mfma(L, i, j, A0, B0)
         if m in rd0:
-            frag_read(L, rd0.index(m), A1, B1, "%[ra1]", "%[rb1]")
+            frag_read(L, rd0.index(m), A1, B1, "%[ra1]", "%[rb1]", 1)
     emit(L, '"s_waitcnt lgkmcnt(0)')
     # the first MFMAs of block 1 need the K-step-1 fragments only: issued ahead of the barrier they keep the
     # matrix pipe busy while the wave waits there
@@ -151,7 +185,7 @@ def main():
     emit(L, '"s_barrier')
     offsets_for(L, 2)
     # from here on the fragment addresses point at the other stage
-    for reg in ("%[ra0]", "%[ra1]", "%[rb0]", "%[rb1]"):
+    for reg in frag_addrs:
         emit(L, f'"v_xor_b32 {reg}, 0x10000, {reg}')
     for m, (i, j) in enumerate(order):
         if m >= early:
@@ -159,9 +193,9 @@ def main():
         if m in ld1:
             dma(L, ld1.index(m), False)
         if m in rd1:
-            frag_read(L, rd1.index(m), A0, B0, "%[ra0]", "%[rb0]")
+            frag_read(L, rd1.index(m), A0, B0, "%[ra0]", "%[rb0]", 0)
     emit(L, f'"s_add_u32 s{S_KA}, s{S_KA}, 128')
-    emit(L, f'"s_add_u32 s{S_KB}, s{S_KB}, 128')
+    emit(L, f'"s_add_u32 s{S_KB}, s{S_KB}, {kb_step}')
     emit(L, f'"s_xor_b32 s{S_LDS}, s{S_LDS}, 0x10000')
     emit(L, f'"s_add_u32 s{S_IT}, s{S_IT}, 1')
     emit(L, f'"s_cmp_lt_u32 s{S_IT}, %[n]')
@@ -171,17 +205,19 @@ def main():
     emit(L, '"s_waitcnt vmcnt(0) lgkmcnt(0)')
     for _ in range(3):
         emit(L, '"s_nop 7')
+    return L
 
+
+def main():
     print("// Generated by gen_tile_asm.py -- do not edit; see that file for the register plan and the schedule.")
-    print("// SK_TILE_ASM_LOOP(MF): the loop text, MF = the MFMA mnemonic as a string literal.")
+    print("// SK_TILE_ASM_LOOP(MF) / SK_TILE_ASM_LOOP_NN(MF): the loop text for the NT / NN layout, MF = the MFMA")
+    print("// mnemonic as a string literal.")
     print("#pragma once")
-    print("#define SK_TILE_ASM_LOOP(MF) \\")
-    for text in L:
-        if text.startswith("MF "):
+    for name, nn in (("SK_TILE_ASM_LOOP", False), ("SK_TILE_ASM_LOOP_NN", True)):
+        print(f"#define {name}(MF) \\")
+        for text in loop_text(nn):
             print(f"  {text}\\n\\t\" \\")
-        else:
-            print(f"  {text}\\n\\t\" \\")
-    print("  \"\"")
+        print("  \"\"")
     clob = [f'"a{r}"' for r in range(256)] + [f'"v{r}"' for r in range(120, 256)] + [f'"s{r}"' for r in range(80, 88)]
     print("#define SK_TILE_ASM_CLOBBERS \\")
     for k in range(0, len(clob), 16):

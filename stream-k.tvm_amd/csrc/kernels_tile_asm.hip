@@ -16,14 +16,15 @@ int tile_asm_kernel_infos(KernelInfo *out, int max) {
   int n = 0;
   // (the int8 instance counts bk and K in int8 elements: 128 per iteration)
   static const int dtypes[3] = {0 /* SK_F16 */, 3 /* SK_BF16 */, 6 /* SK_I8 */};
-  static const char *const names[3] = {"tile_f16_nt_asm_256x256x64", "tile_bf16_nt_asm_256x256x64",
-                                       "tile_i8_nt_asm_256x256x128"};
-#define X(id, MODE)                                                                                              \
+  static const char *const names[2][3] = {
+      {"tile_f16_nt_asm_256x256x64", "tile_bf16_nt_asm_256x256x64", "tile_i8_nt_asm_256x256x128"},
+      {"tile_f16_nn_asm_256x256x64", "tile_bf16_nn_asm_256x256x64", ""}};
+#define X(id, MODE, NN)                                                                                          \
   if (n < max) {                                                                                                 \
-    typedef TileF16Asm<MODE> P;                                                                                  \
+    typedef TileF16Asm<MODE, NN> P;                                                                              \
     const int kb = (MODE) == 2 ? 2 : 1;                                                                          \
-    out[n++] = KernelInfo{id, FAMILY_TILE, dtypes[MODE], 0, 7, P::BM, P::BN, P::BK * kb, P::NT, P::LDS_TOTAL,    \
-                          P::CTAS_PER_CU, P::TILE_ELEMS, 0, 0, 64 * kb, names[MODE]};                            \
+    out[n++] = KernelInfo{id, FAMILY_TILE, dtypes[MODE], (NN) ? 1 : 0, 7, P::BM, P::BN, P::BK * kb, P::NT,       \
+                          P::LDS_TOTAL, P::CTAS_PER_CU, P::TILE_ELEMS, 0, 0, 64 * kb, names[(NN) ? 1 : 0][MODE]}; \
   }
   SK_TILE_ASM_KERNELS(X)
 #undef X
@@ -33,9 +34,9 @@ int tile_asm_kernel_infos(KernelInfo *out, int max) {
 // data-parallel launches use the instance without fix-up code
 int launch_tile_asm(int id, const GemmArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s, const void *bias) {
   switch (id) {
-#define X(id_, MODE)                                                                                              \
+#define X(id_, MODE, NN)                                                                                              \
   case id_: {                                                                                                     \
-    typedef TileF16Asm<MODE> P;                                                                                   \
+    typedef TileF16Asm<MODE, NN> P;                                                                                   \
     if (p.sk_tiles == 0)                                                                                          \
       hipLaunchKernelGGL((sk_tile_asm_kernel<P, false>), dim3(p.grid), dim3(P::NT), 0, s, a, p, ws, bias);        \
     else                                                                                                          \
@@ -51,9 +52,9 @@ int launch_tile_asm(int id, const GemmArgs &a, const DevPlan &p, const Workspace
 int occupancy_tile_asm(int id) {
   int occ = 0;
   switch (id) {
-#define X(id_, MODE)                                                                                                    \
+#define X(id_, MODE, NN)                                                                                                    \
   case id_: {                                                                                                           \
-    typedef TileF16Asm<MODE> P;                                                                                         \
+    typedef TileF16Asm<MODE, NN> P;                                                                                         \
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_tile_asm_kernel<P, true>, P::NT, 0) != hipSuccess) return -1; \
     return occ;                                                                                                         \
   }

@@ -140,10 +140,10 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
   // or two waves per SIMD, where the four-stage (BK = 32) pipeline hides the load latency better;
   // it exists for the NT layout only.
   const int64_t tiles256 = cdiv(M, 256) * cdiv(N, 256), tiles128 = cdiv(M, 128) * cdiv(N, 128);
-  // (256x256: the four-wave kernel with the K loop in assembly where it applies -- NT, K a multiple of 64 --
+  // (256x256: the four-wave kernel with the K loop in assembly where it applies -- K a multiple of 64 --
   // else the eight-wave 16x16x32-MFMA form)
   int pref[3][4] = {{256, 256, 64, 4}, {128, 128, 32, 3}, {64, 64, 32, 3}};  // bm, bn, bk, variant
-  if (layout == SK_LAYOUT_NT && K % 64 == 0 && (dtype == SK_F16 || dtype == SK_BF16)) pref[0][3] = 7;
+  if (K % 64 == 0 && (dtype == SK_F16 || dtype == SK_BF16)) pref[0][3] = 7;
   const int first = tiles256 * 4 >= (int64_t)num_cus * 3 ? 0 : (tiles128 * 2 >= num_cus ? 1 : 2);
   const int order[3][3] = {{0, 1, 2}, {1, 2, 0}, {2, 1, 0}};  // smaller tiles first, then larger ones
   for (int oi = 0; oi < 3 && !best; ++oi) {

@@ -15,7 +15,10 @@
 // and stay far below 256 architectural registers, so it has no reason to (the build checks the generated
 // assembly for accumulation-register instructions outside the hand-written blocks).
 //
-// Restrictions: NT layout, K a multiple of 64 (int8: of 128 bytes).
+// NN_ (B is [K, N] row-major): the B half of a stage holds 64 K-rows of 512 bytes, swizzled and read with
+// transposing 8-byte LDS reads as in the NN form of tile_f16_dma.h; see gen_tile_asm.py for the loop's side.
+//
+// Restrictions: K a multiple of 64 (int8: NT only, K a multiple of 128 bytes).
 #pragma once
 #include "sk_device.h"
 #include "tile_f16.h"
@@ -45,8 +48,9 @@ __device__ __forceinline__ void agpr_write4(floatx4 x) {
 
 // MODE_: 0 fp16, 1 bfloat16, 2 int8 (int32 C; the bytes travel as pairs, so K and the leading dimensions of A
 // and B arrive in 16-bit units and the loop is the fp16 one with v_mfma_i32_16x16x64_i8 on the same fragments)
-template <int MODE_ = 0>
+template <int MODE_ = 0, bool NN_ = false>
 struct TileF16Asm {
+  static_assert(!(NN_ && MODE_ == 2), "int8: NT layout only");
   typedef GemmArgs Args;
   static constexpr bool BF16_ = MODE_ == 1, I8 = MODE_ == 2;
   typedef int intx4 __attribute__((ext_vector_type(4)));
@@ -91,7 +95,41 @@ struct TileF16Asm {
     uint32_t ra0 = base + (uint32_t)(wm * WTM + (lane & 15)) * ROW_BYTES + pos0, ra1 = ra0 ^ 64;
     uint32_t rb0 = base + A_BYTES + (uint32_t)(wn * WTN + (lane & 15)) * ROW_BYTES + pos0, rb1 = rb0 ^ 64;
     const uint32_t iters = (uint32_t)n;
-    if constexpr (I8) {
+    if constexpr (NN_) {
+      // B: the descriptor starts at the tile's first column and ends with the last valid element of row K - 1;
+      // columns past N are masked per lane (N is a multiple of 8).  A wave-wide load fills K-rows 2 g, 2 g + 1 of
+      // the stage (g = wave + 4 x): lane l writes position l % 32 of row 2 g + l / 32 and therefore fetches chunk
+      // (l % 32) ^ swizzle(row); bit 3 of the row is the parity of x, hence two offsets.
+      const uint4v rsrc_bn = make_rsrc_words(a.B + (int64_t)pn * BN, (uint32_t)(((int64_t)(a.K - 1) * a.ldb + rows_b) * 2));
+      const int row_in = lane >> 5, k_bits = 2 * wave + row_in;
+      const int chunk0 = (lane & 31) ^ (4 * (k_bits & 3)), chunk1 = chunk0 ^ 2;
+      const uint32_t vob0 = chunk0 * 8 < rows_b ? (uint32_t)(row_in * a.ldb + chunk0 * 8) * 2 : OOB_OFFSET;
+      const uint32_t vob1 = chunk1 * 8 < rows_b ? (uint32_t)(row_in * a.ldb + chunk1 * 8) * 2 : OOB_OFFSET;
+      const uint32_t kstep_bn = (uint32_t)(128 * a.ldb);  // 64 K-rows
+      const uint32_t goff_bn = (uint32_t)k0 * kstep_bn + (uint32_t)(wave * 4 * a.ldb), gstep_bn = (uint32_t)(16 * a.ldb);
+      // fragments of B: lane group g' = l / 16 reads K-rows 8 g' .. 8 g' + 7 of a 16-column block, four rows per
+      // transposing read; block j's address differs from block 0's by an XOR (the swizzle), so each has its own
+      const int k_lane = 8 * (lane >> 4) + ((lane & 15) >> 2);
+      const int swz = (4 * (k_lane & 3)) ^ (2 * ((k_lane >> 3) & 1));
+      uint32_t rbt[FN];
+#pragma unroll
+      for (int j = 0; j < FN; ++j) {
+        const int col = wn * WTN + j * 16 + 4 * (lane & 3);
+        rbt[j] = base + A_BYTES + (uint32_t)(k_lane * 512 + (((col >> 3) ^ swz) * 16) + (col & 7) * 2);
+      }
+#define SK_ASM_NN_OPERANDS                                                                                            \
+  : [ra0] "+v"(ra0), [ra1] "+v"(ra1), [rbt0] "+v"(rbt[0]), [rbt1] "+v"(rbt[1]), [rbt2] "+v"(rbt[2]),                    \
+    [rbt3] "+v"(rbt[3]), [rbt4] "+v"(rbt[4]), [rbt5] "+v"(rbt[5]), [rbt6] "+v"(rbt[6]), [rbt7] "+v"(rbt[7])            \
+  : [rsa] "s"(rsrc_a), [rsb] "s"(rsrc_bn), [voa] "v"(voff_a), [vob] "v"(vob0), [vob1] "v"(vob1), [ga0] "s"(goff_a),     \
+    [gb0] "s"(goff_bn), [gas] "s"(gstep_a), [gbs] "s"(gstep_bn), [kbs] "s"(kstep_bn), [n] "s"(iters), [lds] "s"(lds_wave) \
+  : "memory", "m0", "scc", SK_TILE_ASM_CLOBBERS
+      if constexpr (BF16_) {
+        asm volatile(SK_TILE_ASM_LOOP_NN("v_mfma_f32_16x16x32_bf16") SK_ASM_NN_OPERANDS);
+      } else {
+        asm volatile(SK_TILE_ASM_LOOP_NN("v_mfma_f32_16x16x32_f16") SK_ASM_NN_OPERANDS);
+      }
+#undef SK_ASM_NN_OPERANDS
+    } else if constexpr (I8) {
       asm volatile(SK_TILE_ASM_LOOP("v_mfma_i32_16x16x64_i8")
                    : [ra0] "+v"(ra0), [ra1] "+v"(ra1), [rb0] "+v"(rb0), [rb1] "+v"(rb1)
                    : [rsa] "s"(rsrc_a), [rsb] "s"(rsrc_b), [voa] "v"(voff_a), [vob] "v"(voff_b), [ga0] "s"(goff_a),

@@ -102,7 +102,7 @@ def test_cfg2_streamk_both_fixups(sk, oracle, cfg, fixup):
 
 def test_assembly_loop_tile_kernels(sk, oracle, golden_dir):
     """The four-wave 256 x 256 x 64 kernels whose K loop is hand-scheduled assembly (accumulators in the
-    accumulation registers): fp16 and bfloat16, ragged M and N, K any multiple of 64 (odd and even iteration
+    accumulation registers): fp16 and bfloat16, NT and NN, ragged M and N, K any multiple of 64 (odd and even iteration
     counts, a single iteration), every schedule and both fix-ups including the halves exchange -- exact on
     integer data, bit-identical to the eight-wave 16x16x32 kernel on random data (same instruction, same order
     of the K-steps), within tolerance of the oracle; a K that is no multiple of 64 falls back to the eight-wave
@@ -112,7 +112,8 @@ def test_assembly_loop_tile_kernels(sk, oracle, golden_dir):
     assert sk.kernel_name(sk.make_plan(8192, 8192, 8192, "float16", "nt", use_tuned=False).kernel_id) == "tile_f16_nt_asm_256x256x64"
     assert sk.kernel_name(sk.make_plan(2048, 2048, 2048, "bfloat16", "nt", dict(bm=256, bn=256)).kernel_id) == "tile_bf16_nt_asm_256x256x64"
     assert "asm" not in sk.kernel_name(sk.make_plan(2048, 2048, 2056, "float16", "nt", dict(bm=256, bn=256)).kernel_id)
-    assert "asm" not in sk.kernel_name(sk.make_plan(2048, 2048, 2048, "float16", "nn", dict(bm=256, bn=256)).kernel_id)
+    assert sk.kernel_name(sk.make_plan(2048, 2048, 2048, "float16", "nn", dict(bm=256, bn=256)).kernel_id) == "tile_f16_nn_asm_256x256x64"
+    assert "asm" not in sk.kernel_name(sk.make_plan(2048, 2048, 2056, "float16", "nn", dict(bm=256, bn=256)).kernel_id)
     with pytest.raises(sk.StreamKError):
         sk.make_plan(2048, 2048, 2056, "float16", "nt", dict(bm=256, bn=256, variant=8))
     ran = 0
@@ -145,6 +146,36 @@ def test_assembly_loop_tile_kernels(sk, oracle, golden_dir):
             assert torch.equal(sk.streamk_bf16(dAi.bfloat16(), dBi.bfloat16(), plan=pb), exact.bfloat16()), (M, N, K, sch)
             ran += 1
     assert ran >= 30
+    # the NN form of the loop (B is [K, N]: 512-byte K-rows in LDS, transposing fragment reads): the same checks
+    # against the eight-wave NN kernel; N ragged in multiples of 8
+    ran = 0
+    for (M, N, K) in [(256, 256, 64), (256, 256, 192), (200, 136, 320), (1000, 1096, 1024), (520, 264, 448)]:
+        Ai = rng.integers(-2, 3, (M, K)).astype(np.float16)
+        Bi = rng.integers(-2, 3, (K, N)).astype(np.float16)
+        exact = torch.from_numpy((Ai.astype(np.int32) @ Bi.astype(np.int32)).astype(np.float32)).cuda()
+        Ar = (rng.random((M, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+        Br = (rng.random((K, N), dtype=np.float32) * 2 - 1).astype(np.float16)
+        ref = oracle.matmul_fp32(Ar, Br, trans_b=False)
+        dAi, dBi, dAr, dBr = _t(Ai), _t(Bi), _t(Ar), _t(Br)
+        for sch in (dict(schedule="dp"), dict(schedule="basic", fixup="reduce", grid=7), dict(schedule="basic", fixup="atomic", grid=5),
+                    dict(schedule="splitk", split=2, fixup="reduce"), dict(schedule="sk1", fixup="reduce", grid=2, raster=2)):
+            try:
+                plan = sk.make_plan(M, N, K, "float16", "nn", dict(bm=256, bn=256, bk=64, variant=8, **sch))
+            except sk.StreamKError:
+                assert sch["schedule"] == "splitk"
+                continue
+            assert sk.kernel_name(plan.kernel_id) == "tile_f16_nn_asm_256x256x64"
+            assert torch.equal(sk.streamk_fp16(dAi, dBi, plan=plan, layout="nn").float(), exact), (M, N, K, sch)
+            C = sk.streamk_fp16(dAr, dBr, plan=plan, layout="nn")
+            assert _rel(oracle, C, ref) <= 2e-3 <= TOL, (M, N, K, sch)
+            if sch["schedule"] == "dp" or sch.get("fixup") == "reduce":
+                twin = sk.streamk_fp16(dAr, dBr, layout="nn", **dict(sch, bm=256, bn=256, bk=64, variant=5))
+                assert torch.equal(C, twin), (M, N, K, sch)
+            pb = sk.make_plan(M, N, K, "bfloat16", "nn", dict(bm=256, bn=256, bk=64, variant=8, **sch))
+            assert sk.kernel_name(pb.kernel_id) == "tile_bf16_nn_asm_256x256x64"
+            assert torch.equal(sk.streamk_bf16(dAi.bfloat16(), dBi.bfloat16(), plan=pb, layout="nn"), exact.bfloat16()), (M, N, K, sch)
+            ran += 1
+    assert ran >= 20
     # epilogue: integer bias + relu exact; silu within tolerance
     M, N, K = 520, 264, 448
     Ai = rng.integers(-1, 2, (M, K)).astype(np.float16)
