@@ -282,8 +282,10 @@ int sk_gemm_q4(const void *A, const void *Wq, const void *scales, void *C, int64
 /* The same with one zero point per scale group and row: zeros [N, K/group] fp16 holding integers 0..15,
  * w = fp16_rn((fp16(q) - zeros[n][k/group]) * scales[n][k/group]) -- the asymmetric formats of weight-only
  * quantisers (min/max per group), which the reference's unsigned nibbles with one implied zero point do
- * not cover.  The plan is made with dtype SK_Q4_ZP; every M goes through the general small-M kernels
- * (bit-exact rounded weights; there is no matrix-vector specialisation), at most 64 rows per call. */
+ * not cover.  The plan is made with dtype SK_Q4_ZP; at most 64 rows per call.  M == 1 takes matrix-vector kernels
+ * that, like sk_gemm_q4's, multiply the nibbles undecoded and apply zero point and scale to fp32 group sums (the
+ * unrounded (q - zero) * scale); 2 <= M <= 64, and M == 1 with an explicit variant-0 plan, the general small-M
+ * kernels, which form the rounded weights bit for bit. */
 int sk_gemm_q4_zp(const void *A, const void *Wq, const void *scales, const void *zeros, void *C, int64_t M,
                   int64_t N, int64_t K, int64_t lda, int64_t ldc, int group, const sk_plan *plan, void *ws,
                   size_t ws_bytes, void *stream);

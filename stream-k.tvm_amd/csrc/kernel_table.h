@@ -150,6 +150,14 @@ struct KernelInfo {
   X(150, 1, 1, 4, 4, 32768)    \
   X(151, 1, 2, 4, 4, 32768)
 
+// M == 1 with per-group zero points (dtype SK_Q4_ZP): the matrix-vector kernels with the zero points staged beside
+// the scales:  X(id, NB, WN, RK, DEPTH, KMAX)
+#define SK_GEMV_Q4ZP_KERNELS(X) \
+  X(152, 1, 1, 4, 4, 16384)     \
+  X(153, 1, 2, 2, 4, 16384)     \
+  X(154, 1, 4, 1, 4, 16384)     \
+  X(155, 1, 1, 4, 4, 32768)
+
 // Q4 kernels reading tiled weights (dtype SK_Q4_TILED), same variants as their row-major twins.
 // general small-M:  X(id, MB, NB, WN, RK, DEPTH);  matrix-vector:  X(id, NB, WN, RK, DEPTH, KMAX)
 #define SK_SKINNY_Q4T_KERNELS(X) \

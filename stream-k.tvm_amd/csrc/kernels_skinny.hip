@@ -127,6 +127,15 @@ int skinny_kernel_infos(KernelInfo *out, int max) {
 #undef X
 #define X(id, NB, WN, RK, DEPTH, KMAX)                                                                        \
   if (n < max) {                                                                                         \
+    typedef TileGemvQ4<NB, WN, RK, DEPTH, KMAX, false, true> P;                                           \
+    out[n++] = KernelInfo{id, FAMILY_SKINNY, 7 /* SK_Q4_ZP */, 0, 2, P::BM, P::BN, P::BKC, P::NT, P::LDS_BYTES, \
+                          P::CTAS_PER_CU, P::TILE_ELEMS, P::MAX_ITERS, P::MAX_M, 128,                    \
+                          "gemv_q4zp_nb" #NB "_wn" #WN "_rk" #RK "_k" #KMAX};                                   \
+  }
+  SK_GEMV_Q4ZP_KERNELS(X)
+#undef X
+#define X(id, NB, WN, RK, DEPTH, KMAX)                                                                        \
+  if (n < max) {                                                                                         \
     typedef TileGemvF16<NB, WN, RK, DEPTH, KMAX> P;                                                       \
     out[n++] = KernelInfo{id, FAMILY_SKINNY, 0, 0, 2, P::BM, P::BN, P::BKC, P::NT, P::LDS_BYTES,         \
                           P::CTAS_PER_CU, P::TILE_ELEMS, P::MAX_ITERS, P::MAX_M, 8,                      \
@@ -216,6 +225,13 @@ int launch_skinny(int id, const SkinnyArgs &a, const DevPlan &p, const Workspace
 #undef X
 #define X(id_, NB, WN, RK, DEPTH, KMAX)                                                        \
   case id_: {                                                                              \
+    typedef TileGemvQ4<NB, WN, RK, DEPTH, KMAX, false, true> P;                             \
+    return launch_policy<P>(a, p, ws, s, bias);                                                         \
+  }
+    SK_GEMV_Q4ZP_KERNELS(X)
+#undef X
+#define X(id_, NB, WN, RK, DEPTH, KMAX)                                                        \
+  case id_: {                                                                              \
     typedef TileGemvF16<NB, WN, RK, DEPTH, KMAX> P;                                         \
     return launch_policy<P>(a, p, ws, s, bias);                                                         \
   }
@@ -301,6 +317,15 @@ int occupancy_skinny(int id) {
     return occ;                                                                                          \
   }
     SK_GEMV_Q4_KERNELS(X)
+#undef X
+#define X(id_, NB, WN, RK, DEPTH, KMAX)                                                                      \
+  case id_: {                                                                                            \
+    typedef TileGemvQ4<NB, WN, RK, DEPTH, KMAX, false, true> P;                                           \
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_skinny_kernel<P>, P::NT, 0) != hipSuccess) \
+      return -1;                                                                                         \
+    return occ;                                                                                          \
+  }
+    SK_GEMV_Q4ZP_KERNELS(X)
 #undef X
 #define X(id_, NB, WN, RK, DEPTH, KMAX)                                                                      \
   case id_: {                                                                                            \

@@ -104,7 +104,6 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
           return &t[i];
     // 2 <= M <= 16 with Q4 weights: eight waves per CTA (two per SIMD cover each other's waits),
     // 32 weight rows, K split over four waves
-    // (per-group zero points: also for M == 1, which has no matrix-vector kernel of its own)
     if (((dtype == SK_Q4 && M > 1) || dtype == SK_Q4_ZP) && M <= 16 && want_variant < 0)
       for (int i = 0; i < n; ++i)
         if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].variant == 0 && t[i].bm == 16 &&

@@ -41,8 +41,14 @@ namespace sk {
 //
 // TILED_: the weights come in 16-row x 64-byte tiles (see tile_skinny.h); the lane order of the
 // loads, row = lane/4, piece = lane%4, is then the byte order of a tile: one contiguous KB per load.
-template <int NB_, int WN_, int RK_, int DEPTH_, int KMAX_ = 16384, bool TILED_ = false>
+//
+// ZP_: one zero point per scale group and row (a.zeros, the shape of the scales; a.zero is ignored).  The
+// bracket above splits into a part that depends on A only and one that is linear in the zero point:
+//     sum a_k (q_k - z) = c_lo + c_hi / 16 - [1024 sum_even a_k + 64 sum_odd a_k] - z [sum_even a_k + sum_odd a_k]
+// Both sums of A are kept per 32 K-values; the zero points are staged in LDS beside the scales.
+template <int NB_, int WN_, int RK_, int DEPTH_, int KMAX_ = 16384, bool TILED_ = false, bool ZP_ = false>
 struct TileGemvQ4 {
+  static_assert(!(TILED_ && ZP_), "zero points come with row-major weights");
   typedef SkinnyArgs Args;
   static constexpr bool LEAN_ENTRY = false;  // see run_persistent
   static constexpr int NB = NB_, WN = WN_, RK = RK_, DEPTH = DEPTH_, KMAX = KMAX_;
@@ -56,8 +62,10 @@ struct TileGemvQ4 {
   static constexpr int MAX_ITERS = KMAX / BKC;              // iterations one segment may span
   static constexpr int SC_ROW = KMAX / QGROUP + 8;          // halfs per LDS scale row
   static constexpr int LDS_A = KMAX * 2;
-  static constexpr int LDS_CORR = KMAX / 32 * 4;            // one correction per 32 K-values
-  static constexpr int LDS_SC = BN * SC_ROW * 2;
+  static constexpr int LDS_CORR1 = KMAX / 32 * 4;           // one correction per 32 K-values
+  static constexpr int LDS_CORR = ZP_ ? 2 * LDS_CORR1 : LDS_CORR1;  // ZP_: then the plain sums of A
+  static constexpr int LDS_SC1 = BN * SC_ROW * 2;
+  static constexpr int LDS_SC = ZP_ ? 2 * LDS_SC1 : LDS_SC1;        // scales, then zero points
   static constexpr int LDS_RED = RK > 1 ? (RK - 1) * WN * NB * 64 * 4 : 0;
   static constexpr int LDS_BYTES = LDS_A + LDS_CORR + LDS_SC + LDS_RED;
   static constexpr int TILE_ELEMS = BN;
@@ -144,13 +152,18 @@ struct TileGemvQ4 {
     ScaleStager<BN, SC_ROW, NT> scales;
     scales.begin(ldsS, a.scales + (int64_t)pn * BN * a.groups, rows_w, a.groups, g0,
                  (sc_shift + n * SC_PER_ITER + 7) >> 3);
+    ScaleStager<BN, SC_ROW, NT> zero_points;
+    if constexpr (ZP_)
+      zero_points.begin(ldsS + BN * SC_ROW, a.zeros + (int64_t)pn * BN * a.groups, rows_w, a.groups, g0,
+                        (sc_shift + n * SC_PER_ITER + 7) >> 3);
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) issue_loads(d, d);
     // nothing of what follows is to be scheduled ahead of these loads
     __builtin_amdgcn_sched_barrier(0);
     SK_TRACE(2);
 
-    const float w_even = (float)(1024 + a.zero), w_odd = (float)(64 + a.zero);
+    const float w_even = (float)(1024 + (ZP_ ? 0 : a.zero)), w_odd = (float)(64 + (ZP_ ? 0 : a.zero));
+    float *ldsSumA = ldsCorr + KMAX / 32;  // ZP_: sum of the 32 K-values of A, beside their correction
     auto stage_a_block = [&](int b, uint4v v0, uint4v v1) {
       uint4v u0, u1;  // [even | odd] of K-values 0..7 and 8..15 of the block
       u0[0] = __builtin_amdgcn_perm(v0[2], v0[0], 0x05040100u);
@@ -173,10 +186,15 @@ struct TileGemvQ4 {
       }
       float corr = w_even * se + w_odd * so;
       corr += __shfl_xor(corr, 1);
+      float sum_a = se + so;
+      if constexpr (ZP_) sum_a += __shfl_xor(sum_a, 1);
       if (b < nblk) {
         *reinterpret_cast<uint4v *>(ldsA + b * 32) = u0;
         *reinterpret_cast<uint4v *>(ldsA + b * 32 + 16) = u1;
-        if ((tid & 1) == 0) ldsCorr[b >> 1] = corr;
+        if ((tid & 1) == 0) {
+          ldsCorr[b >> 1] = corr;
+          if constexpr (ZP_) ldsSumA[b >> 1] = sum_a;
+        }
       }
     };
 #pragma unroll
@@ -188,6 +206,7 @@ struct TileGemvQ4 {
     }
     SK_TRACE(3);
     scales.finish();
+    if constexpr (ZP_) zero_points.finish();
     SK_TRACE(4);
     __syncthreads();
     SK_TRACE(5);
@@ -213,6 +232,11 @@ struct TileGemvQ4 {
         const int its = min(it, n - 1);
         const float live = it < n ? 1.f : 0.f;
         const float corr0 = c_rd[its * (BKC / 32)], corr1 = c_rd[its * (BKC / 32) + 4];
+        float suma0 = 0.f, suma1 = 0.f;
+        if constexpr (ZP_) {
+          suma0 = c_rd[KMAX / 32 + its * (BKC / 32)];
+          suma1 = c_rd[KMAX / 32 + its * (BKC / 32) + 4];
+        }
         uint4v fa[2][4];  // [load c][word]: {even half, odd half} of the word's eight K-values of A
 #pragma unroll
         for (int c = 0; c < 2; ++c)
@@ -222,6 +246,8 @@ struct TileGemvQ4 {
 #pragma unroll
         for (int j = 0; j < NB; ++j) {
           const half2v s2 = *reinterpret_cast<const half2v *>(s_rd[j] + its * SC_PER_ITER);
+          half2v z2 = {(half_t)0.f, (half_t)0.f};
+          if constexpr (ZP_) z2 = *reinterpret_cast<const half2v *>(s_rd[j] + BN * SC_ROW + its * SC_PER_ITER);
 #pragma unroll
           for (int c = 0; c < 2; ++c) {
             const uint4v w = wreg[d][j][c];
@@ -248,7 +274,8 @@ struct TileGemvQ4 {
             // register `piece` of each result is this lane's term
             const float se = p2 ? (p1 ? ce[3] : ce[2]) : (p1 ? ce[1] : ce[0]);
             const float so = p2 ? (p1 ? co[3] : co[2]) : (p1 ? co[1] : co[0]);
-            const float sum32 = __builtin_fmaf(so, 0.0625f, se) - (c == 0 ? corr0 : corr1);
+            float sum32 = __builtin_fmaf(so, 0.0625f, se) - (c == 0 ? corr0 : corr1);
+            if constexpr (ZP_) sum32 = __builtin_fmaf(-(float)z2[c], c == 0 ? suma0 : suma1, sum32);
             acc.y[j] = __builtin_fmaf(sum32, (float)s2[c] * live, acc.y[j]);
           }
         }

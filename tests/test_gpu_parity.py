@@ -421,7 +421,7 @@ def test_q4_per_group_zero_points(sk, oracle):
     the host one."""
     import torch
     rng = np.random.default_rng(77)
-    tiles = [(16, 64, 256), (32, 64, 256), (64, 64, 256), (16, 32, 1024), (16, 64, 512), (16, 16, 1024)]
+    tiles = [(16, 64, 256), (32, 64, 256), (64, 64, 256), (16, 32, 1024), (16, 64, 512), (16, 16, 1024), (16, 32, 512)]
     ran = 0
     for (M, N, K) in [(1, 1000, 1152), (5, 520, 384), (16, 264, 4096), (33, 200, 640), (64, 136, 2048), (1, 72, 16384)]:
         A = (rng.random((M, K), dtype=np.float32) * 2 - 1).astype(np.float16)
@@ -442,9 +442,15 @@ def test_q4_per_group_zero_points(sk, oracle):
                     continue  # the instance does not take this M / K
                 C = sk.streamk_q4(dA, dW, dS, zeros=dZ, plan=plan)
                 assert _rel(oracle, C, ref) <= 2e-3 <= TOL, (M, N, K, bm, bn, bk, sch, plan.kernel_id)
-                if sch.get("fixup") != "atomic":
+                gemv = sk.kernel_name(plan.kernel_id).startswith("gemv_q4zp")
+                assert gemv == (M == 1 and (bm, bn, bk) in ((16, 32, 512), (16, 64, 256), (16, 16, 1024))), (M, bm, bn, bk)
+                if sch.get("fixup") != "atomic" and not gemv:
                     same = sk.make_plan(M, N, K, "q4", "nt", dict(bm=bm, bn=bn, bk=bk, variant=1, **sch))
                     assert torch.equal(sk.streamk_q4(dA, dW, dS, zeros=z7, plan=plan), sk.streamk_q4(dA, dW, dS, zero=7, plan=same))
+                if gemv and (bm, bn, bk) != (16, 32, 512):   # the general kernel of the tile (bit-exact rounded weights) stays selectable
+                    general = sk.make_plan(M, N, K, "q4_zp", "nt", dict(bm=bm, bn=bn, bk=bk, variant=1, **sch))
+                    assert sk.kernel_name(general.kernel_id).startswith("skinny_q4zp")
+                    assert _rel(oracle, sk.streamk_q4(dA, dW, dS, zeros=dZ, plan=general), ref) <= 2e-3
                 ran += 1
         C = sk.streamk_q4(dA, dW, dS, zeros=_t(zp.astype(np.uint8)))      # heuristic plan; integer zero points are converted
         assert _rel(oracle, C, ref) <= 2e-3
@@ -580,6 +586,30 @@ def test_q4_matrix_vector_deviation_from_rounded_weights_is_bounded(sk, oracle):
             assert np.all(np.abs(y - target) <= 2.0 ** -11 * np.abs(target) + 2.0 ** -24 + noise), (bm, bn, bk, variant)
             ran += 1
     assert ran >= 12
+    # the same bound for the matrix-vector kernels with one zero point per group and row
+    zp = rng.integers(0, 16, (N, K // 128)).astype(np.float16)
+    w_rounded = oracle.dequant_q4_zp_np(Wq, sc, zp).astype(np.float64)
+    w_exact = (oracle.unpack_q4_np(Wq).astype(np.float64) - np.repeat(zp.astype(np.float64), 128, axis=1)) * \
+        np.repeat(sc.astype(np.float64), 128, axis=1)
+    assert np.abs(w_exact - w_rounded).max() <= 2.0 ** -11 * np.abs(w_exact).max()
+    y_rounded, y_exact = w_rounded @ a64, w_exact @ a64
+    mass = np.abs(w_exact) @ np.abs(a64)
+    noise = 2e-5 * mass
+    dZ = _t(zp)
+    ran = 0
+    for (bm, bn, bk) in ((16, 16, 1024), (16, 32, 512), (16, 64, 256)):
+        for variant, rounded in ((3, False), (1, True)):
+            if rounded and (bm, bn, bk) == (16, 32, 512):
+                continue   # this tile exists as a matrix-vector kernel only
+            plan = sk.make_plan(1, N, K, "q4_zp", "nt", dict(bm=bm, bn=bn, bk=bk, variant=variant, schedule="dp"))
+            assert sk.kernel_name(plan.kernel_id).startswith("skinny_q4zp" if rounded else "gemv_q4zp")
+            y = sk.streamk_q4(dA, dW, dS, zeros=dZ, plan=plan).double().cpu().numpy()[0]
+            assert np.all(np.abs(y - y_rounded) <= 2.0 ** -11 * mass + 2.0 ** -11 * np.abs(y_rounded) + noise), (bm, bn, bk, variant)
+            target = y_rounded if rounded else y_exact
+            assert np.all(np.abs(y - target) <= 2.0 ** -11 * np.abs(target) + 2.0 ** -24 + noise), (bm, bn, bk, variant)
+            ran += 1
+    assert ran == 5
+    assert sk.kernel_name(sk.make_plan(1, N, K, "q4_zp", "nt", use_tuned=False).kernel_id) == "gemv_q4zp_nb1_wn1_rk4_k16384"
     sk.workspace_status()
 
 
