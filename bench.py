@@ -251,41 +251,46 @@ def main():
             p = streamk.make_plan(m, N, K, "float16", "nt")
             for _ in range(min(2000, max(PREWARM, int(0.05 / (2.0 * m * N * K / 1e15))))):  # about 50 ms of load
                 streamk.streamk_fp16(a, B, out=c, plan=p)
+            # M <= 64: one 134 MB B launched repeatedly is served by the 256 MB Infinity Cache, which is not an HBM
+            # rate; these rows are timed with the launches of a batch rotating over copies of B totalling > 512 MB
+            # (the figures with one B are kept beside them as `weights_in_infinity_cache`)
+            copies = [B] + [B.clone() for _ in range(4)] if m <= 64 else None
+            warm = {}
             for name, cfg in cands.items():
                 try:
                     p = streamk.make_plan(m, N, K, "float16", "nt", **cfg)
                 except streamk.StreamKError:
                     continue  # the fixed split does not divide this shape
                 ms = time_graph(lambda: streamk.streamk_fp16(a, B, out=c, plan=p))
-                row[name] = round(2.0 * m * N * K / ms / 1e9, 1)
-            if m > 64:
-                for t in tiles:
-                    sk_best = max((row.pop(f"{sch}_{t}"), sch) for sch in ("sk2", "basic", "splitk") if f"{sch}_{t}" in row)
-                    row["sk_" + t], row["sk_schedule_" + t] = sk_best
-            best = max(v for k, v in row.items() if k != "M" and not isinstance(v, str))
-            row["best_tflops"] = best
-            row["pct_fp16_peak"] = round(100 * best / PEAK_FP16_TFLOPS, 2)
-            nbytes = 2.0 * (m * K + N * K + m * N)
-            if m <= 64:
-                # one 134 MB B launched repeatedly is served by the 256 MB Infinity Cache: that rate is not an HBM
-                # rate.  The HBM figure rotates the launches of a batch over copies of B totalling > 512 MB.
-                row["gbs_weights_in_infinity_cache"] = round(best * 1e3 * nbytes / (2.0 * m * N * K), 1)
-                copies = [B] + [B.clone() for _ in range(4)]
+                if m > 64:
+                    row[name] = round(2.0 * m * N * K / ms / 1e9, 1)
+                    continue
+                warm[name] = round(2.0 * m * N * K / ms / 1e9, 1)
                 turn = [0]
-                p = streamk.make_plan(m, N, K, "float16", "nt")
 
                 def rotating():
                     w = copies[turn[0] % len(copies)]
                     turn[0] += 1
                     streamk.streamk_fp16(a, w, out=c, plan=p)
                 ms = time_graph(rotating)
-                del copies
-                row["auto_weights_from_hbm_us"] = round(ms * 1e3, 2)
-                row["gbs"] = round(nbytes / ms / 1e6, 1)
+                row[name] = round(2.0 * m * N * K / ms / 1e9, 1)
+                if name == "auto":
+                    row["auto_weights_from_hbm_us"] = round(ms * 1e3, 2)
+            copies = None
+            if m > 64:
+                for t in tiles:
+                    sk_best = max((row.pop(f"{sch}_{t}"), sch) for sch in ("sk2", "basic", "splitk") if f"{sch}_{t}" in row)
+                    row["sk_" + t], row["sk_schedule_" + t] = sk_best
+            best = max(v for k, v in row.items() if k not in ("M", "auto_weights_from_hbm_us") and not isinstance(v, str))
+            row["best_tflops"] = best
+            row["pct_fp16_peak"] = round(100 * best / PEAK_FP16_TFLOPS, 2)
+            nbytes = 2.0 * (m * K + N * K + m * N)
+            row["gbs"] = round(best * 1e3 * nbytes / (2.0 * m * N * K), 1)
+            if m <= 64:
+                row["weights_in_infinity_cache"] = warm
                 row["gbs_is"] = "weights from HBM (launches rotate over 5 copies of B, 671 MB)"
-                row["frac_hbm"] = round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)
+                row["frac_hbm"] = round(row["gbs"] / PEAK_HBM_GBS, 4)
             else:
-                row["gbs"] = round(best * 1e3 * nbytes / (2.0 * m * N * K), 1)
                 row["gbs_is"] = "algorithmic bytes over time; compute-bound row, operands stay in the Infinity Cache"
             if m > 64:
                 row["sk_over_dp_same_tile"] = round(max(row["sk_" + t] / row["dp_" + t] for t in tiles), 3)
@@ -391,7 +396,7 @@ def main():
                              "frac_hbm": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
             # the same launch with the weights coming from HBM: the 20 launches of a batch read 20
             # different copies (692 MB, against 256 MB of Infinity Cache)
-            if m == 1:
+            if True:
                 copies = [(Wq.clone(), sc.clone()) for _ in range(20)]
                 turn = [0]
 
@@ -403,10 +408,21 @@ def main():
                 ms = time_graph(cold)
                 row["tuned_weights_from_hbm"] = {"us": round(ms * 1e3, 2), "gbs": round(nbytes / ms / 1e6, 1),
                                                  "frac_hbm": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
+            if m == 1:
                 p_cold = streamk.make_plan(m, N, K, "q4", "nt", variant=2, schedule="dp")
                 ms = time_graph(cold)
                 row["rounded_weights_from_hbm"] = {"us": round(ms * 1e3, 2), "gbs": round(nbytes / ms / 1e6, 1),
                                                    "frac_hbm": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
+                # one zero point per scale group and row (asymmetric quantisers) instead of the scalar 8
+                zp = torch.randint(0, 16, (N, K // 128), generator=g).half().cuda()
+                p_zp = streamk.make_plan(m, N, K, "q4_zp", "nt")
+
+                def cold_zp():
+                    w, s_ = copies[turn[0] % len(copies)]
+                    turn[0] += 1
+                    streamk.streamk_q4(a, w, s_, zeros=zp, out=c, plan=p_zp)
+                ms = time_graph(cold_zp)
+                row["per_group_zero_points_from_hbm"] = {"us": round(ms * 1e3, 2), "kernel": streamk.kernel_name(p_zp.kernel_id)}
                 # the same with the weights in the tiled layout (one contiguous KB per load instruction)
                 tiles = [(streamk.tile_q4(w), s_) for (w, s_) in copies]
                 del copies
@@ -420,6 +436,7 @@ def main():
                 row["tiled_weights_from_hbm"] = {"us": round(ms * 1e3, 2), "gbs": round(nbytes / ms / 1e6, 1),
                                                  "frac_hbm": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
                 del tiles
+            copies = None
             q4.append(row)
         extra["q4_N8192_K8192"] = q4
         # more rows of A than the weight-streaming kernels take: the Q4 tile kernels (nibbles dequantised on their
