@@ -220,6 +220,18 @@ struct KernelInfo {
   X(278, 4, 1, 4, 1, 2, 0)      \
   X(279, 4, 1, 4, 2, 2, 0)
 
+// 2 <= M <= 4, fp16 / bfloat16 weights (NT): the matrix-vector kernels' quad-coalesced weight stream against up to
+// MR rows of A (variant 3):  X(id, MR, WN, RK, DEPTH).  (Instances with MR = 8 and 16 were measured and are not
+// kept: every row of A costs a 16-byte LDS read per weight load and lane, and from 8 rows on that traffic, not
+// the weight stream, sets the time -- 43 and 57 us at 8192 x 8192 against 33 us for the general kernel.)
+#define SK_GEMV_ROWS_F16_KERNELS(X) \
+  X(168, 4, 1, 4, 4)                \
+  X(169, 4, 2, 4, 2)                \
+  X(170, 4, 4, 2, 2)
+#define SK_GEMV_ROWS_BF16_KERNELS(X) \
+  X(200, 4, 1, 4, 4)                 \
+  X(201, 4, 2, 4, 2)
+
 // bfloat16 twins of the fp16 matrix-vector kernels (dtype SK_BF16, variant 2)
 #define SK_GEMV_BF16_KERNELS(X) \
   X(241, 1, 1, 4, 4, 8192)      \

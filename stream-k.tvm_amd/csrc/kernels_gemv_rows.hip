@@ -1,0 +1,72 @@
+// Small-M kernels in the matrix-vector kernels' form (tile_gemv_rows.h): 2 <= M <= 16, fp16 / bfloat16, NT.
+#include "skinny_launch.h"
+
+namespace sk {
+
+int gemv_rows_kernel_infos(KernelInfo *out, int max) {
+  int n = 0;
+#define X(id, MR, WN, RK, DEPTH)                                                                               \
+  if (n < max) {                                                                                               \
+    typedef TileGemvRows<MR, WN, RK, DEPTH, false> P;                                                          \
+    out[n++] = KernelInfo{id, FAMILY_SKINNY, 0, 0, 3, P::BM, P::BN, P::BKC, P::NT, P::LDS_BYTES, P::CTAS_PER_CU, \
+                          P::TILE_ELEMS, 0, P::MAX_M, 8, "gemv_rows_f16_m" #MR "_wn" #WN "_rk" #RK};            \
+  }
+  SK_GEMV_ROWS_F16_KERNELS(X)
+#undef X
+#define X(id, MR, WN, RK, DEPTH)                                                                               \
+  if (n < max) {                                                                                               \
+    typedef TileGemvRows<MR, WN, RK, DEPTH, true> P;                                                           \
+    out[n++] = KernelInfo{id, FAMILY_SKINNY, 3, 0, 3, P::BM, P::BN, P::BKC, P::NT, P::LDS_BYTES, P::CTAS_PER_CU, \
+                          P::TILE_ELEMS, 0, P::MAX_M, 8, "gemv_rows_bf16_m" #MR "_wn" #WN "_rk" #RK};           \
+  }
+  SK_GEMV_ROWS_BF16_KERNELS(X)
+#undef X
+  return n;
+}
+
+int launch_gemv_rows(int id, const SkinnyArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s, const void *bias) {
+  switch (id) {
+#define X(id_, MR, WN, RK, DEPTH)                        \
+  case id_: {                                            \
+    typedef TileGemvRows<MR, WN, RK, DEPTH, false> P;    \
+    return launch_policy<P>(a, p, ws, s, bias);          \
+  }
+    SK_GEMV_ROWS_F16_KERNELS(X)
+#undef X
+#define X(id_, MR, WN, RK, DEPTH)                        \
+  case id_: {                                            \
+    typedef TileGemvRows<MR, WN, RK, DEPTH, true> P;     \
+    return launch_policy<P>(a, p, ws, s, bias);          \
+  }
+    SK_GEMV_ROWS_BF16_KERNELS(X)
+#undef X
+  }
+  return (int)hipErrorInvalidValue;
+}
+
+int occupancy_gemv_rows(int id) {
+  int occ = 0;
+  switch (id) {
+#define X(id_, MR, WN, RK, DEPTH)                                                                        \
+  case id_: {                                                                                            \
+    typedef TileGemvRows<MR, WN, RK, DEPTH, false> P;                                                    \
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_skinny_kernel<P>, P::NT, 0) != hipSuccess) \
+      return -1;                                                                                         \
+    return occ;                                                                                          \
+  }
+    SK_GEMV_ROWS_F16_KERNELS(X)
+#undef X
+#define X(id_, MR, WN, RK, DEPTH)                                                                        \
+  case id_: {                                                                                            \
+    typedef TileGemvRows<MR, WN, RK, DEPTH, true> P;                                                     \
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_skinny_kernel<P>, P::NT, 0) != hipSuccess) \
+      return -1;                                                                                         \
+    return occ;                                                                                          \
+  }
+    SK_GEMV_ROWS_BF16_KERNELS(X)
+#undef X
+  }
+  return -1;
+}
+
+}  // namespace sk

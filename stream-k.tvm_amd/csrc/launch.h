@@ -9,6 +9,7 @@
 #include "tile_f32.h"
 #include "tile_gemv_f16.h"
 #include "tile_gemv_q4.h"
+#include "tile_gemv_rows.h"
 #include "tile_skinny.h"
 
 namespace sk {
@@ -28,6 +29,10 @@ int occupancy_tile_asm(int id);
 int tile_q4_kernel_infos(KernelInfo *out, int max);
 int launch_tile_q4(int id, const GemmArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s, const void *bias);
 int occupancy_tile_q4(int id);
+// 2 <= M <= 16 kernels in the matrix-vector kernels' form (translation unit kernels_gemv_rows.hip)
+int gemv_rows_kernel_infos(KernelInfo *out, int max);
+int launch_gemv_rows(int id, const SkinnyArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s, const void *bias);
+int occupancy_gemv_rows(int id);
 int f32_kernel_infos(KernelInfo *out, int max);
 int launch_f32(int id, const GemmArgsF32 &a, const DevPlan &p, const Workspace &ws, hipStream_t s);
 int occupancy_f32(int id);

@@ -13,7 +13,7 @@
 
 namespace sk {
 
-static KernelInfo g_table[320];
+static KernelInfo g_table[400];
 static int g_count = 0;
 static std::once_flag g_table_once;
 
@@ -25,11 +25,11 @@ int f32_kernel_infos(KernelInfo *out, int max);
 
 const KernelInfo *kernel_table(int *count) {
   std::call_once(g_table_once, [] {
-    int n = tile_kernel_infos(g_table, 320);
-    n += tile_asm_kernel_infos(g_table + n, 320 - n);
-    n += tile_q4_kernel_infos(g_table + n, 320 - n);
-    n += skinny_kernel_infos(g_table + n, 320 - n);
-    n += f32_kernel_infos(g_table + n, 320 - n);
+    int n = tile_kernel_infos(g_table, 400);
+    n += tile_asm_kernel_infos(g_table + n, 400 - n);
+    n += tile_q4_kernel_infos(g_table + n, 400 - n);
+    n += skinny_kernel_infos(g_table + n, 400 - n);
+    n += f32_kernel_infos(g_table + n, 400 - n);
     g_count = n;
   });
   if (count) *count = g_count;
@@ -49,7 +49,8 @@ static int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // preference among kernel variants of one tile shape when the caller does not ask for one: the
 // eight-wave direct-to-LDS tile kernels; the most specialised small-M kernel that accepts the shape
 static int variant_rank(const KernelInfo &k) {
-  if (k.family == FAMILY_SKINNY) return k.variant;
+  // (small-M: general 0 < rows-of-A matrix-vector form 3 < single-row 1 < matrix-vector 2)
+  if (k.family == FAMILY_SKINNY) return k.variant == 3 ? 1 : (k.variant == 0 ? 0 : k.variant + 1);
   return k.variant == 7 ? 4 : (k.variant == 4 ? 3 : (k.variant == 1 ? 2 : (k.variant == 2 ? 1 : 0)));
 }
 static bool accepts_shape(const KernelInfo &k, int64_t M, int64_t K) {
@@ -108,6 +109,12 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
       for (int i = 0; i < n; ++i)
         if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].variant == 0 && t[i].bm == 16 &&
             t[i].bn == 32 && t[i].bk == 1024 && accepts_shape(t[i], M, K))
+          return &t[i];
+    // 2 <= M <= 4 with fp16 / bfloat16 weights: the matrix-vector form with four rows of A
+    if ((dtype == SK_F16 || dtype == SK_BF16) && M >= 2 && M <= 4 && want_variant < 0)
+      for (int i = 0; i < n; ++i)
+        if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].layout == layout && t[i].variant == 3 &&
+            t[i].bn == 16 && t[i].bk == 512 && accepts_shape(t[i], M, K))
           return &t[i];
     // M == 1 with fp16 / bfloat16 weights: the same structure, K split over four waves
     if ((dtype == SK_F16 || dtype == SK_BF16) && M == 1 && want_variant < 0)

@@ -1,0 +1,68 @@
+// Kernel entry points and the launcher shared by the small-M translation units.
+#pragma once
+#include "launch.h"
+#include "sk_persistent.h"
+
+namespace sk {
+
+template <class P, bool FIXUP = true>
+__global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_skinny_kernel(typename P::Args a, DevPlan plan, Workspace ws) {
+  __shared__ __attribute__((aligned(16))) char smem[P::LDS_BYTES];
+  run_persistent<P, FIXUP>(a, plan, ws, smem);
+}
+// the same with a bias row added in the epilogue (a second instance: see run_persistent)
+template <class P, bool FIXUP = true>
+__global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_skinny_kernel_bias(typename P::Args a, DevPlan plan, Workspace ws,
+                                                                               const void *bias) {
+  __shared__ __attribute__((aligned(16))) char smem[P::LDS_BYTES];
+  run_persistent<P, FIXUP, true>(a, plan, ws, smem, bias);
+}
+
+// Launches without Stream-K tiles: every CTA owns whole tiles (tile = block index, then strides of the grid;
+// one row of tiles, since these kernels take all of A's rows in one tile), so the kernel needs neither the plan
+// nor the workspace.  These kernels run for a few microseconds, most of which is set-up executed from a cold
+// instruction cache: without the plan's argument loads, the range and tile-coordinate arithmetic and the fix-up
+// code the first loads go out earlier.
+template <class P>
+__global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_skinny_dp_kernel(typename P::Args a, int total_tiles, int ipt) {
+  __shared__ __attribute__((aligned(16))) char smem[P::LDS_BYTES];
+  typename P::Acc acc;
+  SK_TRACE(0);
+  for (int tile = blockIdx.x; tile < total_tiles; tile += gridDim.x) {
+    SK_TRACE(11);
+    P::mac(a, acc, 0, tile, 0, ipt, smem);
+    SK_TRACE(8);
+    P::store_c(a, acc, 0, tile, smem, nullptr);
+    SK_TRACE(9);
+  }
+}
+template <class P>
+__global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_skinny_dp_kernel_bias(typename P::Args a, int total_tiles, int ipt,
+                                                                                  const void *bias_arg) {
+  __shared__ __attribute__((aligned(16))) char smem[P::LDS_BYTES];
+  const void *bias = bias_arg;
+  asm volatile("" ::"s"(bias));  // fetched with the other arguments, not before the first store
+  typename P::Acc acc;
+  for (int tile = blockIdx.x; tile < total_tiles; tile += gridDim.x) {
+    P::mac(a, acc, 0, tile, 0, ipt, smem);
+    P::store_c(a, acc, 0, tile, smem, bias);
+  }
+}
+
+template <class P>
+static inline int launch_policy(const SkinnyArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s, const void *bias) {
+  if (p.sk_tiles == 0 && p.tiles_m != 1) return (int)hipErrorInvalidValue;  // (no plan of these kernels has two tile rows)
+  if (bias != nullptr) {
+    if (p.sk_tiles == 0)
+      hipLaunchKernelGGL((sk_skinny_dp_kernel_bias<P>), dim3(p.grid), dim3(P::NT), 0, s, a, p.total_tiles, p.ipt, bias);
+    else
+      hipLaunchKernelGGL((sk_skinny_kernel_bias<P, true>), dim3(p.grid), dim3(P::NT), 0, s, a, p, ws, bias);
+  } else if (p.sk_tiles == 0) {
+    hipLaunchKernelGGL((sk_skinny_dp_kernel<P>), dim3(p.grid), dim3(P::NT), 0, s, a, p.total_tiles, p.ipt);
+  } else {
+    hipLaunchKernelGGL((sk_skinny_kernel<P, true>), dim3(p.grid), dim3(P::NT), 0, s, a, p, ws);
+  }
+  return (int)hipGetLastError();
+}
+
+}  // namespace sk

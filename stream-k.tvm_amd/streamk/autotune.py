@@ -69,6 +69,12 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
             out.append(dict(bm=bm, bn=bn, bk=bk, schedule="dp"))
             for grid, fixup in itertools.product((cus, 2 * cus, 4 * cus), ("reduce", "atomic")):
                 out.append(dict(bm=bm, bn=bn, bk=bk, schedule="sk2", grid=grid, fixup=fixup))
+            # 2 <= M <= 4: these tiles resolve to the matrix-vector form with four rows of A; the general kernel
+            # of the same tile stays in the search as variant 1
+            if 2 <= M <= 4 and dtype in ("float16", "bfloat16") and (bm, bn, bk) in ((16, 16, 512), (16, 32, 512), (16, 64, 256)):
+                out.append(dict(bm=bm, bn=bn, bk=bk, variant=1, schedule="dp"))
+                for grid in (cus, 2 * cus):
+                    out.append(dict(bm=bm, bn=bn, bk=bk, variant=1, schedule="sk2", grid=grid, fixup="reduce"))
     if dtype in ("float16", "bfloat16") and M > 16:
         for (bm, bn, bk) in _TILES_F16:
             # (variant, bk): direct-to-LDS two-stage, register-staged, direct-to-LDS four-stage, 16x16x32 form

@@ -649,7 +649,58 @@ def test_f16_matrix_vector_every_kernel(sk, oracle):
     assert ran >= 100
     # the heuristic plan for M = 1 is one of these kernels
     plan = sk.make_plan(1, 4096, 4096, "float16", "nt", {})
-    assert (plan.bm, plan.bn, plan.bk) == (16, 16, 512) and 160 <= plan.kernel_id < 170
+    assert (plan.bm, plan.bn, plan.bk) == (16, 16, 512) and 160 <= plan.kernel_id < 168
+    sk.workspace_status()
+
+
+def test_f16_few_rows_in_the_matrix_vector_form(sk, oracle):
+    """2 <= M <= 4 on the kernels that stream the weights as the matrix-vector kernels do and multiply them with
+    four rows of A: ragged N, K a multiple of 8 only, strided A and W, K beyond the 8192 values of A that stay in
+    LDS at a time (several windows), all schedules and both fix-ups, fp16 and bfloat16, bias and activation;
+    exact on integer data, within 2e-3 of the fp32 host product otherwise; 5 rows fall to the general kernel."""
+    import torch
+    rng = np.random.default_rng(73)
+    ran = 0
+    for (M, N, K, pad) in [(2, 1000, 1160, 0), (3, 520, 392, 8), (4, 72, 4096, 0), (4, 2048, 8192, 64), (3, 264, 28672, 0), (2, 4099, 11008, 0)]:
+        A = (rng.random((M, K + pad), dtype=np.float32) * 2 - 1).astype(np.float16)
+        W = (rng.random((N, K + pad), dtype=np.float32) * 2 - 1).astype(np.float16)
+        Ai = rng.integers(-1, 2, (M, K + pad)).astype(np.float16)
+        Wi = rng.integers(-2, 3, (N, K + pad)).astype(np.float16)
+        ref = oracle.matmul_fp32(A[:, :K], W[:, :K], trans_b=True)
+        exact = Ai[:, :K].astype(np.int64) @ Wi[:, :K].astype(np.int64).T
+        assert np.abs(exact).max() < 2048
+        dA, dW, dAi, dWi = _t(A)[:, :K], _t(W)[:, :K], _t(Ai)[:, :K], _t(Wi)[:, :K]
+        for (bn, bk) in ((16, 512), (32, 512), (64, 256)):
+            for sch in (dict(schedule="dp"), dict(schedule="sk2", fixup="reduce", grid=48),
+                        dict(schedule="sk2", fixup="atomic", grid=40), dict(schedule="basic", fixup="reduce", grid=56)):
+                plan = sk.make_plan(M, N, K, "float16", "nt", dict(bm=16, bn=bn, bk=bk, variant=4, **sch))
+                assert sk.kernel_name(plan.kernel_id).startswith("gemv_rows_f16_m4")
+                C = sk.streamk_fp16(dA, dW, plan=plan)
+                assert _rel(oracle, C, ref) <= 2e-3 <= TOL, (M, N, K, bn, bk, sch)
+                C = sk.streamk_fp16(dAi, dWi, plan=plan)
+                assert np.array_equal(C.cpu().numpy().astype(np.int64), exact), (M, N, K, bn, bk, sch)
+                if bn != 64:   # bfloat16 twins of the first two
+                    pb = sk.make_plan(M, N, K, "bfloat16", "nt", dict(bm=16, bn=bn, bk=bk, variant=4, **sch))
+                    assert sk.kernel_name(pb.kernel_id).startswith("gemv_rows_bf16_m4")
+                    C = sk.streamk_bf16(dAi.bfloat16(), dWi.bfloat16(), plan=pb)
+                    # (the exact sums, rounded once to bfloat16's eight bits)
+                    assert torch.equal(C.cpu(), torch.from_numpy(exact).float().bfloat16()), (M, N, K, bn, bk, sch)
+                ran += 1
+    assert ran >= 70
+    # heuristic plans, bias and activation, an output with a row stride
+    M, N, K = 3, 1000, 2048
+    Ai = rng.integers(-1, 2, (M, K)).astype(np.float16)
+    Wi = rng.integers(-1, 2, (N, K)).astype(np.float16)
+    bias = rng.integers(-3, 4, N).astype(np.float16)
+    want = np.maximum(Ai.astype(np.int64) @ Wi.astype(np.int64).T + bias.astype(np.int64), 0)
+    assert sk.kernel_name(sk.make_plan(M, N, K, "float16", "nt", use_tuned=False).kernel_id) == "gemv_rows_f16_m4_wn1_rk4"
+    for sch in (dict(), dict(schedule="sk2", fixup="reduce", grid=64), dict(schedule="sk2", fixup="atomic", grid=64)):
+        out = torch.zeros(M, N + 24, dtype=torch.float16, device="cuda")[:, 8:8 + N]
+        C = sk.streamk_fp16(_t(Ai), _t(Wi), out=out, bias=_t(bias), activation="relu", **sch)
+        assert np.array_equal(C.cpu().numpy().astype(np.int64), want), sch
+    assert not sk.kernel_name(sk.make_plan(5, N, K, "float16", "nt", use_tuned=False).kernel_id).startswith("gemv_rows")
+    with pytest.raises(sk.StreamKError):
+        sk.make_plan(5, N, K, "float16", "nt", dict(bm=16, bn=16, bk=512, variant=4))
     sk.workspace_status()
 
 
