@@ -208,6 +208,137 @@ def loop_text(nn):
     return L
 
 
+class LdsTracker:
+    """issue order of the fragment reads and the s_waitcnt lgkmcnt(n) a consumer needs (reads return in order)"""
+
+    def __init__(self, outstanding):
+        self.q = list(outstanding)      # tags still possibly in flight, oldest first
+
+    def issue(self, tag):
+        self.q.append(tag)
+
+    def need(self, lines, tags):
+        last = max((k for k, t in enumerate(self.q) if t in tags), default=-1)
+        if last < 0:
+            return
+        allowed = len(self.q) - 1 - last
+        emit(lines, f'"s_waitcnt lgkmcnt({min(allowed, 15)})')
+        self.q = self.q[last + 1:] if allowed <= 15 else self.q[len(self.q) - 15:]
+
+    def drain(self, lines):
+        emit(lines, '"s_waitcnt lgkmcnt(0)')
+        self.q = []
+
+
+def loop_text_f8():
+    """fp8 operands (SK_TILE_ASM_LOOP_F8): one v_mfma_f32_16x16x128_f8f6f4 per accumulator block and iteration, on
+    32-byte fragments made of the two 16-byte fragments of the 16-bit loop (which K-values a lane's bytes stand for
+    does not matter as long as A and B agree).  Block i of A lives in v[128 + 8 i .. + 7], block j of B in
+    v[192 + 8 j .. + 7]: all 128 fragment registers hold one iteration, so there is no second set to read ahead
+    into.  Instead an iteration runs in two phases of 32 MFMAs (32 cycles each):
+      phase 1   blocks i = 0..3 of A against j = 7..0; the fragments of i = 4..7 (same stage) ride along
+      sync      wait for them and for this wave's loads into the other stage, barrier
+      phase 2   blocks i = 4..7 against j = 7..0; along ride the 16 loads of iteration it + 2 into the stage just
+                read, the next iteration's fragments of i = 0..3, and its fragment of B block j once the four
+                MFMAs that use the old one have been issued and a further one behind them
+    The waits before the MFMAs are computed from the order in which the reads were issued."""
+    global NN
+    NN = False
+    A8 = lambda i: 128 + 8 * i
+    B8 = lambda j: 192 + 8 * j
+    L = []
+
+    def read_half(tr, which, blk, h, stage_next):
+        base = (A8 if which == "A" else B8)(blk) + 4 * h
+        addr = ("%[ra1]" if h else "%[ra0]") if which == "A" else ("%[rb1]" if h else "%[rb0]")
+        emit(L, f'"ds_read_b128 v[{base}:{base + 3}], {addr} offset:{blk * 2048}')
+        tr.issue((which, blk))
+
+    def mf(i, j):
+        c = (8 * i + j) * 4
+        emit(L, f'MF " a[{c}:{c + 3}], v[{B8(j)}:{B8(j) + 7}], v[{A8(i)}:{A8(i) + 7}], a[{c}:{c + 3}] " MOD "')
+
+    for r in range(256):
+        emit(L, f'"v_accvgpr_write_b32 a{r}, 0')
+    emit(L, f'"s_mov_b32 s{S_IT}, 0')
+    emit(L, f'"s_mov_b32 s{S_LDS}, %[lds]')
+    emit(L, f'"s_mov_b32 s{S_KA}, %[ga0]')
+    emit(L, f'"s_mov_b32 s{S_KB}, %[gb0]')
+    for ahead in (0, 1):
+        offsets_for(L, ahead)
+        for x in range(16):
+            dma(L, x, ahead == 0)
+        emit(L, f'"s_add_u32 s{S_KA}, s{S_KA}, 128')
+        emit(L, f'"s_add_u32 s{S_KB}, s{S_KB}, 128')
+        emit(L, f'"s_xor_b32 s{S_LDS}, s{S_LDS}, 0x10000')
+    emit(L, '"s_waitcnt vmcnt(16)')
+    emit(L, '"s_barrier')
+    tr = LdsTracker([])
+    for i in range(4):
+        for h in range(2):
+            read_half(tr, "A", i, h, False)
+    for j in range(7, -1, -1):
+        for h in range(2):
+            read_half(tr, "B", j, h, False)
+    emit(L, '"s_nop 7')
+    emit(L, '"L_sk_loop%=:')
+    # both ways into the loop end with the four reads of B blocks 1 and 0
+    emit(L, '"s_waitcnt lgkmcnt(4)')
+    tr = LdsTracker([("B", 1), ("B", 1), ("B", 0), ("B", 0)])
+    # ---- phase 1
+    pending = [("A", i, h) for i in range(4, 8) for h in range(2)]
+    m = 0
+    for j in range(7, -1, -1):
+        for i in range(4):
+            tr.need(L, {("A", i), ("B", j)})
+            mf(i, j)
+            if m % 2 == 0 and pending:
+                w, blk, h = pending.pop(0)
+                read_half(tr, w, blk, h, False)
+            m += 1
+    assert not pending
+    tr.drain(L)
+    emit(L, '"s_waitcnt vmcnt(0)')
+    emit(L, '"s_barrier')
+    offsets_for(L, 2)
+    for reg in ("%[ra0]", "%[ra1]", "%[rb0]", "%[rb1]"):
+        emit(L, f'"v_xor_b32 {reg}, 0x10000, {reg}')
+    # ---- phase 2
+    a_next = [("A", i, h) for i in range(4) for h in range(2)]
+    b_next = {}      # slot -> reads of the next iteration's B fragments
+    for j in range(7, -1, -1):
+        s0 = 4 * (7 - j) + 5
+        b_next.setdefault(s0, []).append(("B", j, 0))
+        b_next.setdefault(s0 + 1, []).append(("B", j, 1))
+    m = 0
+    for j in range(7, -1, -1):
+        for i in range(4, 8):
+            tr.need(L, {("A", i), ("B", j)})
+            mf(i, j)
+            if m % 2 == 1:
+                dma(L, m // 2, False)
+            if m % 2 == 0 and a_next:
+                w, blk, h = a_next.pop(0)
+                read_half(tr, w, blk, h, True)
+            for (w, blk, h) in b_next.pop(m, []):
+                read_half(tr, w, blk, h, True)
+            m += 1
+    for slot in sorted(b_next):
+        for (w, blk, h) in b_next[slot]:
+            read_half(tr, w, blk, h, True)
+    assert not a_next and tr.q[-4:] == [("B", 1), ("B", 1), ("B", 0), ("B", 0)]
+    emit(L, f'"s_add_u32 s{S_KA}, s{S_KA}, 128')
+    emit(L, f'"s_add_u32 s{S_KB}, s{S_KB}, 128')
+    emit(L, f'"s_xor_b32 s{S_LDS}, s{S_LDS}, 0x10000')
+    emit(L, f'"s_add_u32 s{S_IT}, s{S_IT}, 1')
+    emit(L, f'"s_cmp_lt_u32 s{S_IT}, %[n]')
+    emit(L, '"s_cbranch_scc1 L_sk_loop%=')
+    emit(L, '"s_waitcnt vmcnt(0) lgkmcnt(0)')
+    for _ in range(3):
+        emit(L, '"s_nop 7')
+    return L
+
+
 def main():
     print("// Generated by gen_tile_asm.py -- do not edit; see that file for the register plan and the schedule.")
     print("// SK_TILE_ASM_LOOP(MF) / SK_TILE_ASM_LOOP_NN(MF): the loop text for the NT / NN layout, MF = the MFMA")
@@ -218,6 +349,11 @@ def main():
         for text in loop_text(nn):
             print(f"  {text}\\n\\t\" \\")
         print("  \"\"")
+    print("// SK_TILE_ASM_LOOP_F8(MF, MOD): fp8 operands; MOD = the format modifiers of the MFMA (\"\" for e4m3)")
+    print("#define SK_TILE_ASM_LOOP_F8(MF, MOD) \\")
+    for text in loop_text_f8():
+        print(f"  {text}\\n\\t\" \\")
+    print("  \"\"")
     clob = [f'"a{r}"' for r in range(256)] + [f'"v{r}"' for r in range(120, 256)] + [f'"s{r}"' for r in range(80, 88)]
     print("#define SK_TILE_ASM_CLOBBERS \\")
     for k in range(0, len(clob), 16):

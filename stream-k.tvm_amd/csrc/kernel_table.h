@@ -281,13 +281,15 @@ struct KernelInfo {
   X(83, 256, 128, 4, 2)
 
 // 256 x 256 x 64 on four waves, K loop in assembly (variant 7), K a multiple of 64 (int8: 128 bytes per
-// iteration):  X(id, MODE, NN)  with MODE 0 fp16, 1 bfloat16, 2 int8; NN: B is [K,N]
+// iteration):  X(id, MODE, NN)  with MODE 0 fp16, 1 bfloat16, 2 int8, 3 fp8 e4m3, 4 fp8 e5m2; NN: B is [K,N]
 #define SK_TILE_ASM_KERNELS(X) \
   X(34, 0, false)              \
   X(66, 1, false)              \
   X(84, 2, false)              \
   X(49, 0, true)               \
-  X(67, 1, true)
+  X(67, 1, true)               \
+  X(74, 3, false)              \
+  X(94, 4, false)
 
 // Q4 weights (dtype SK_Q4) for more rows of A than the weight-streaming kernels take: the two-stage 16x16x32 tile
 // kernel with B dequantised into its LDS stage (variant 4):  X(id, BM, BN, WM, WN)

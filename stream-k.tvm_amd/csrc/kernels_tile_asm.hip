@@ -14,15 +14,16 @@ __global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_tile_asm_kernel(typ
 
 int tile_asm_kernel_infos(KernelInfo *out, int max) {
   int n = 0;
-  // (the int8 instance counts bk and K in int8 elements: 128 per iteration)
-  static const int dtypes[3] = {0 /* SK_F16 */, 3 /* SK_BF16 */, 6 /* SK_I8 */};
-  static const char *const names[2][3] = {
-      {"tile_f16_nt_asm_256x256x64", "tile_bf16_nt_asm_256x256x64", "tile_i8_nt_asm_256x256x128"},
-      {"tile_f16_nn_asm_256x256x64", "tile_bf16_nn_asm_256x256x64", ""}};
+  // (the one-byte instances count bk and K in elements: 128 per iteration)
+  static const int dtypes[5] = {0 /* SK_F16 */, 3 /* SK_BF16 */, 6 /* SK_I8 */, 5 /* SK_F8E4M3 */, 8 /* SK_F8E5M2 */};
+  static const char *const names[2][5] = {
+      {"tile_f16_nt_asm_256x256x64", "tile_bf16_nt_asm_256x256x64", "tile_i8_nt_asm_256x256x128",
+       "tile_f8e4m3_nt_asm_256x256x128", "tile_f8e5m2_nt_asm_256x256x128"},
+      {"tile_f16_nn_asm_256x256x64", "tile_bf16_nn_asm_256x256x64", "", "", ""}};
 #define X(id, MODE, NN)                                                                                          \
   if (n < max) {                                                                                                 \
     typedef TileF16Asm<MODE, NN> P;                                                                              \
-    const int kb = (MODE) == 2 ? 2 : 1;                                                                          \
+    const int kb = (MODE) >= 2 ? 2 : 1;                                                                          \
     out[n++] = KernelInfo{id, FAMILY_TILE, dtypes[MODE], (NN) ? 1 : 0, 7, P::BM, P::BN, P::BK * kb, P::NT,       \
                           P::LDS_TOTAL, P::CTAS_PER_CU, P::TILE_ELEMS, 0, 0, 64 * kb, names[(NN) ? 1 : 0][MODE]}; \
   }

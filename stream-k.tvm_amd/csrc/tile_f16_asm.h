@@ -47,12 +47,15 @@ __device__ __forceinline__ void agpr_write4(floatx4 x) {
 }
 
 // MODE_: 0 fp16, 1 bfloat16, 2 int8 (int32 C; the bytes travel as pairs, so K and the leading dimensions of A
-// and B arrive in 16-bit units and the loop is the fp16 one with v_mfma_i32_16x16x64_i8 on the same fragments)
+// and B arrive in 16-bit units and the loop is the fp16 one with v_mfma_i32_16x16x64_i8 on the same fragments),
+// 3 / 4 fp8 e4m3 / e5m2 (fp16 C scaled by alpha; bytes as pairs again, one v_mfma_f32_16x16x128_f8f6f4 per block
+// and iteration in a two-phase loop of its own, see gen_tile_asm.py)
 template <int MODE_ = 0, bool NN_ = false>
 struct TileF16Asm {
-  static_assert(!(NN_ && MODE_ == 2), "int8: NT layout only");
+  static_assert(!(NN_ && MODE_ >= 2), "one-byte operands: NT layout only");
   typedef GemmArgs Args;
   static constexpr bool BF16_ = MODE_ == 1, I8 = MODE_ == 2;
+  static constexpr int F8 = MODE_ >= 3 ? MODE_ - 2 : 0;  // 1: e4m3, 2: e5m2
   typedef int intx4 __attribute__((ext_vector_type(4)));
   static constexpr bool LEAN_ENTRY = true;  // see run_persistent
   static constexpr int BM = 256, BN = 256, BK = 64, WM = 2, WN = 2, NW = 4, NT = 256;
@@ -129,6 +132,18 @@ struct TileF16Asm {
         asm volatile(SK_TILE_ASM_LOOP_NN("v_mfma_f32_16x16x32_f16") SK_ASM_NN_OPERANDS);
       }
 #undef SK_ASM_NN_OPERANDS
+    } else if constexpr (F8 != 0) {
+#define SK_ASM_NT_OPERANDS                                                                                         \
+  : [ra0] "+v"(ra0), [ra1] "+v"(ra1), [rb0] "+v"(rb0), [rb1] "+v"(rb1)                                             \
+  : [rsa] "s"(rsrc_a), [rsb] "s"(rsrc_b), [voa] "v"(voff_a), [vob] "v"(voff_b), [ga0] "s"(goff_a), [gb0] "s"(goff_b), \
+    [gas] "s"(gstep_a), [gbs] "s"(gstep_b), [n] "s"(iters), [lds] "s"(lds_wave)                                    \
+  : "memory", "m0", "scc", SK_TILE_ASM_CLOBBERS
+      if constexpr (F8 == 1) {
+        asm volatile(SK_TILE_ASM_LOOP_F8("v_mfma_f32_16x16x128_f8f6f4", "") SK_ASM_NT_OPERANDS);
+      } else {
+        asm volatile(SK_TILE_ASM_LOOP_F8("v_mfma_f32_16x16x128_f8f6f4", "cbsz:1 blgp:1") SK_ASM_NT_OPERANDS);
+      }
+#undef SK_ASM_NT_OPERANDS
     } else if constexpr (I8) {
       asm volatile(SK_TILE_ASM_LOOP("v_mfma_i32_16x16x64_i8")
                    : [ra0] "+v"(ra0), [ra1] "+v"(ra1), [rb0] "+v"(rb0), [rb1] "+v"(rb1)
@@ -218,6 +233,7 @@ struct TileF16Asm {
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             float y = x[e];
+            if constexpr (F8 != 0) y *= a.alpha;  // the product of fp8 operands is scaled before bias and rounding
             if constexpr (BIAS) y = activate(y + bv[e], act);
             if constexpr (BF16_) {
               const __bf16 b = (__bf16)y;

@@ -109,13 +109,13 @@ def test_fp8_plans(sk):
     for (M, N, K, bm) in [(8192, 8192, 8192, 256), (512, 512, 4096, 128), (65, 4096, 4096, 128)]:
         p = sk.make_plan(M, N, K, "float8_e4m3", "nt", cus=256)
         assert (p.bm, p.bn, p.bk) == (bm, bm, 128) and p.iters_per_tile == K // 128
-        assert sk.kernel_name(p.kernel_id) == f"tile_f8e4m3_nt_dma_{bm}x{bm}x128"
+        # (256 x 256 with K a multiple of 128: the four-wave kernels whose K loop is assembly)
+        assert sk.kernel_name(p.kernel_id) == ("tile_f8e4m3_nt_asm_256x256x128" if bm == 256 else f"tile_f8e4m3_nt_dma_{bm}x{bm}x128")
         r = sk.make_plan(M, N, K, "float8_e5m2", "nt", cus=256)
         assert (r.bm, r.bn, r.bk, r.grid) == (p.bm, p.bn, 128, p.grid)
-        assert sk.kernel_name(r.kernel_id) == f"tile_f8e5m2_nt_dma_{bm}x{bm}x128"
+        assert sk.kernel_name(r.kernel_id) == ("tile_f8e5m2_nt_asm_256x256x128" if bm == 256 else f"tile_f8e5m2_nt_dma_{bm}x{bm}x128")
         q = sk.make_plan(M, N, K, "int8", "nt", cus=256)
         assert (q.bm, q.bn, q.bk, q.grid) == (p.bm, p.bn, 128, p.grid)
-        # (256 x 256 with K a multiple of 128: the four-wave kernel whose K loop is assembly)
         assert sk.kernel_name(q.kernel_id) == ("tile_i8_nt_asm_256x256x128" if bm == 256 else f"tile_i8_nt_dma16_{bm}x{bm}x128")
     with pytest.raises(sk.StreamKError):
         sk.make_plan(256, 256, 256, "int8", "nn", cus=256)

@@ -898,6 +898,44 @@ def test_fp8_tile_kernels(sk, oracle):
                 assert np.array_equal(Ci.double().cpu().numpy(), exact), (M, N, K, bm, bn, sch)
                 if sch.get("fixup") == "reduce":
                     assert torch.equal(C, sk.streamk_fp8(dA, dB, plan=plan))
+    # the four-wave kernels whose K loop is assembly (K a multiple of 128; one 16x16x128 MFMA per accumulator block
+    # and iteration): both formats, every schedule and fix-up incl. the halves exchange, alpha, bias and activation;
+    # same bits as the eight-wave 32x32x64 kernel (the K-values are summed in the same groups of 128)
+    assert sk.kernel_name(sk.make_plan(4096, 4096, 4096, "float8_e4m3", "nt", use_tuned=False).kernel_id) == "tile_f8e4m3_nt_asm_256x256x128"
+    assert "asm" not in sk.kernel_name(sk.make_plan(4096, 4096, 4112, "float8_e4m3", "nt", use_tuned=False).kernel_id)
+    ran = 0
+    for (M, N, K) in [(256, 256, 128), (200, 136, 384), (1000, 1096, 2048), (520, 264, 896)]:
+        for fmt, name, dec in ((f8, "float8_e4m3", oracle.f8_gemm_ref), (torch.float8_e5m2, "float8_e5m2", None)):
+            A, B = torch.randn(M, K).to(fmt), torch.randn(N, K).to(fmt)
+            Ai, Bi = torch.randint(-1, 2, (M, K)).float().to(fmt), torch.randint(-1, 2, (N, K)).float().to(fmt)
+            ref = (A.double() @ B.double().T).numpy() * 0.25
+            exact = (Ai.double() @ Bi.double().T).numpy()
+            if dec is not None:
+                assert np.array_equal(dec(Ai.view(torch.uint8).numpy(), Bi.view(torch.uint8).numpy()), exact)
+            dA, dB, dAi, dBi = A.cuda(), B.cuda(), Ai.cuda(), Bi.cuda()
+            for sch in (dict(schedule="dp"), dict(schedule="basic", fixup="reduce", grid=7), dict(schedule="basic", fixup="atomic", grid=5),
+                        dict(schedule="splitk", split=2, fixup="reduce"), dict(schedule="sk1", fixup="reduce", grid=2, raster=2)):
+                try:
+                    plan = sk.make_plan(M, N, K, name, "nt", dict(bm=256, bn=256, variant=8, **sch))
+                except sk.StreamKError:
+                    assert sch["schedule"] == "splitk"
+                    continue
+                assert sk.kernel_name(plan.kernel_id) == f"tile_f8{'e4m3' if fmt is f8 else 'e5m2'}_nt_asm_256x256x128"
+                assert np.array_equal(sk.streamk_fp8(dAi, dBi, plan=plan).double().cpu().numpy(), exact), (M, N, K, name, sch)
+                C = sk.streamk_fp8(dA, dB, alpha=0.25, plan=plan)
+                assert _rel(oracle, C, ref) <= 1e-3 <= TOL, (M, N, K, name, sch)
+                if sch["schedule"] == "dp" or sch.get("fixup") == "reduce":
+                    twin = sk.streamk_fp8(dA, dB, alpha=0.25, **dict(sch, bm=256, bn=256, variant=7))
+                    assert torch.equal(C, twin), (M, N, K, name, sch)
+                ran += 1
+    assert ran >= 30
+    M, N, K = 520, 264, 896
+    Ai, Bi = torch.randint(-1, 2, (M, K)).float().to(f8).cuda(), torch.randint(-1, 2, (N, K)).float().to(f8).cuda()
+    bias = torch.randint(-3, 4, (N,)).half().cuda()
+    want = torch.relu((Ai.float() @ Bi.float().T) * 2.0 + bias.float())
+    for sch in (dict(schedule="dp"), dict(schedule="basic", fixup="reduce", grid=7)):
+        C = sk.streamk_fp8(Ai, Bi, alpha=2.0, bias=bias, activation="relu", bm=256, bn=256, variant=8, **sch)
+        assert torch.equal(C.float(), want), sch
     # heuristic plans from one row to many tiles; strided operands (leading dimension a multiple of 16)
     for (M, N, K) in [(1, 512, 1024), (16, 4096, 4096), (2048, 2048, 2048), (1024, 8192, 8192)]:
         A, B = torch.randn(M, K).to(f8), torch.randn(N, K).to(f8)
