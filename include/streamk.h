@@ -118,6 +118,9 @@ const char *sk_strerror(int status);
 /* Name of the compiled kernel instance a plan runs (sk_plan.kernel_id), e.g. for reading profiler
  * output; NULL for an unknown id.  The reference names its generated kernel after the script. */
 const char *sk_kernel_name(int kernel_id);
+/* Consistency of the compiled-in kernel table (every instance has a name and an id of its own, below 512):
+ * SK_OK, or SK_ERR_CONFIG for a library that was built wrong.  Needs no GPU. */
+int sk_selfcheck(void);
 
 /* Number of compute units and max co-resident CTAs per CU are read from the current HIP device.
  * Replaces `total_sm = 108` (streamk_fp32.py:17). */

@@ -229,8 +229,8 @@ struct KernelInfo {
   X(169, 4, 2, 4, 2)                \
   X(170, 4, 4, 2, 2)
 #define SK_GEMV_ROWS_BF16_KERNELS(X) \
-  X(200, 4, 1, 4, 4)                 \
-  X(201, 4, 2, 4, 2)
+  X(210, 4, 1, 4, 4)                 \
+  X(211, 4, 2, 4, 2)
 
 // bfloat16 twins of the fp16 matrix-vector kernels (dtype SK_BF16, variant 2)
 #define SK_GEMV_BF16_KERNELS(X) \

@@ -172,6 +172,18 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
 
 using namespace sk;
 
+extern "C" int sk_selfcheck(void) {
+  int n;
+  const KernelInfo *t = kernel_table(&n);
+  if (n <= 0 || n >= 400) return SK_ERR_CONFIG;  // (400: the table's capacity)
+  for (int i = 0; i < n; ++i) {
+    if (t[i].id < 0 || t[i].id >= 512 || !t[i].name || !t[i].name[0]) return SK_ERR_CONFIG;
+    for (int j = 0; j < i; ++j)
+      if (t[j].id == t[i].id) return SK_ERR_CONFIG;
+  }
+  return SK_OK;
+}
+
 extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layout, const sk_config *cfg,
                             int num_cus, sk_plan *out) {
   if (!out) return SK_ERR_NULL;

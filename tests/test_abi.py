@@ -28,6 +28,7 @@ def test_exports_every_declared_symbol(sk):
     for n in sorted(names):
         assert hasattr(L, n), f"{n} is declared in streamk.h but not exported"
     assert L.sk_version() == 100
+    assert L.sk_selfcheck() == 0        # kernel ids are unique, every instance is named
     assert sk.strerror(0) == "ok" and "workspace" in sk.strerror(-5)
 
 

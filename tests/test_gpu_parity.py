@@ -853,7 +853,8 @@ def test_bf16_small_m_kernels(sk, oracle):
                     assert torch.equal(C, sk.streamk_bf16(A.cuda(), B.cuda(), plan=plan))
     for M in (1, 2, 16, 32):
         plan = sk.make_plan(M, 4096, 4096, "bfloat16", "nt")
-        assert (241 <= plan.kernel_id <= 248) if M == 1 else (230 <= plan.kernel_id <= 240), (M, plan.kernel_id)
+        # (one row: matrix-vector kernels; two to four rows: their form with four rows of A; else the general kernels)
+        assert (241 <= plan.kernel_id <= 248) if M == 1 else ((210 <= plan.kernel_id <= 211) if M <= 4 else (230 <= plan.kernel_id <= 240)), (M, plan.kernel_id)
         A, W = (torch.rand(M, 4096) * 2 - 1).bfloat16(), (torch.rand(4096, 4096) * 2 - 1).bfloat16()
         ref = oracle.matmul_fp32(A.float().numpy(), W.float().numpy(), trans_b=True)
         assert _rel(oracle, sk.streamk_bf16(A.cuda(), W.cuda()), ref) <= 4e-3, M
