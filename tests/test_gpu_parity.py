@@ -1430,6 +1430,44 @@ def test_full_size_exact_integer_checksums(sk, shape):
     sk.workspace_status()
 
 
+def test_full_size_one_byte_operands_exact_checksums(sk):
+    """The one-byte kernels at M = N = K = 8192 (the assembly-loop instances by default): int8 over its full
+    range against int64 row and column checksums and a block of rows (sums stay below 2^31); fp8 on {-1, 0, 1}
+    (sums stay below 2048, exact in fp16), both formats; data-parallel and a Stream-K schedule with either fix-up."""
+    import torch
+    M = N = K = 8192
+    rng = np.random.default_rng(13)
+    A = rng.integers(-128, 128, (M, K)).astype(np.int8)
+    B = rng.integers(-128, 128, (N, K)).astype(np.int8)
+    row_sum = A.astype(np.int64) @ B.astype(np.int64).sum(axis=0)
+    col_sum = A.astype(np.int64).sum(axis=0) @ B.astype(np.int64).T
+    block = A[:32].astype(np.int64) @ B.astype(np.int64).T
+    dA, dB = _t(A), _t(B)
+    assert sk.kernel_name(sk.make_plan(M, N, K, "int8", "nt").kernel_id) == "tile_i8_nt_asm_256x256x128"
+    for cfg in (dict(), dict(bm=256, bn=256, schedule="sk2", fixup="reduce", grid=250), dict(bm=256, bn=256, schedule="sk2", fixup="atomic", grid=250)):
+        C = sk.streamk_int8(dA, dB, **cfg)
+        assert np.array_equal(C.sum(dim=1, dtype=torch.int64).cpu().numpy(), row_sum), cfg
+        assert np.array_equal(C.sum(dim=0, dtype=torch.int64).cpu().numpy(), col_sum), cfg
+        assert np.array_equal(C[:32].cpu().numpy().astype(np.int64), block), cfg
+    del dA, dB
+    A = rng.integers(-1, 2, (M, K)).astype(np.int8)
+    B = rng.integers(-1, 2, (N, K)).astype(np.int8)
+    row_sum = A.astype(np.int64) @ B.astype(np.int64).sum(axis=0)
+    col_sum = A.astype(np.int64).sum(axis=0) @ B.astype(np.int64).T
+    block = A[:32].astype(np.int32) @ B.astype(np.int32).T
+    assert np.abs(block).max() < 2048
+    for fmt, name in ((torch.float8_e4m3fn, "float8_e4m3"), (torch.float8_e5m2, "float8_e5m2")):
+        dA, dB = _t(A.astype(np.float32)).to(fmt), _t(B.astype(np.float32)).to(fmt)
+        assert "asm" in sk.kernel_name(sk.make_plan(M, N, K, name, "nt").kernel_id)
+        for cfg in (dict(), dict(bm=256, bn=256, schedule="sk2", fixup="reduce", grid=250)):
+            C = sk.streamk_fp8(dA, dB, **cfg)
+            Cd = C.double()
+            assert np.array_equal(Cd.sum(dim=1).cpu().numpy().astype(np.int64), row_sum), (name, cfg)
+            assert np.array_equal(Cd.sum(dim=0).cpu().numpy().astype(np.int64), col_sum), (name, cfg)
+            assert np.array_equal(C[:32].cpu().numpy().astype(np.int32), block), (name, cfg)
+    sk.workspace_status()
+
+
 @pytest.mark.parametrize("variant", [2, 5], ids=["mfma32", "mfma16"])
 @pytest.mark.parametrize("cfg", [dict(bm=256, bn=256), dict(bm=128, bn=128), dict(bm=128, bn=256), dict(bm=256, bn=128)],
                          ids=lambda c: f"{c['bm']}x{c['bn']}")
