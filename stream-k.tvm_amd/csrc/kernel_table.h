@@ -285,10 +285,12 @@ struct KernelInfo {
 #define SK_TILE_ASM_KERNELS(X) \
   X(34, 0, false)              \
   X(66, 1, false)              \
-  X(84, 2, false)              \
   X(49, 0, true)               \
-  X(67, 1, true)               \
-  X(74, 3, false)              \
+  X(67, 1, true)
+// (the one-byte instances, translation unit kernels_tile_asm8.hip)
+#define SK_TILE_ASM8_KERNELS(X) \
+  X(84, 2, false)               \
+  X(74, 3, false)               \
   X(94, 4, false)
 
 // Q4 weights (dtype SK_Q4) for more rows of A than the weight-streaming kernels take: the two-stage 16x16x32 tile

@@ -47,7 +47,7 @@ int launch_tile_asm(int id, const GemmArgs &a, const DevPlan &p, const Workspace
     SK_TILE_ASM_KERNELS(X)
 #undef X
   }
-  return launch_tile_q4(id, a, p, ws, s, bias);
+  return launch_tile_asm8(id, a, p, ws, s, bias);
 }
 
 int occupancy_tile_asm(int id) {
@@ -62,7 +62,7 @@ int occupancy_tile_asm(int id) {
     SK_TILE_ASM_KERNELS(X)
 #undef X
   }
-  return occupancy_tile_q4(id);
+  return occupancy_tile_asm8(id);
 }
 
 }  // namespace sk

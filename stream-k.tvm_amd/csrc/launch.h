@@ -25,6 +25,9 @@ int launch_skinny(int id, const SkinnyArgs &a, const DevPlan &p, const Workspace
 int tile_asm_kernel_infos(KernelInfo *out, int max);
 int launch_tile_asm(int id, const GemmArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s, const void *bias);
 int occupancy_tile_asm(int id);
+int tile_asm8_kernel_infos(KernelInfo *out, int max);
+int launch_tile_asm8(int id, const GemmArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s, const void *bias);
+int occupancy_tile_asm8(int id);
 // tile kernels for Q4 weights (translation unit kernels_tile_q4.hip)
 int tile_q4_kernel_infos(KernelInfo *out, int max);
 int launch_tile_q4(int id, const GemmArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s, const void *bias);
