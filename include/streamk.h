@@ -61,8 +61,15 @@ typedef enum sk_fixup {
   SK_FIXUP_AUTO = 0,
   SK_FIXUP_ATOMIC = 1,     /* fp32 atomicAdd of partial accumulators (streamk_fp32.py:127-134);
                               summation order varies run to run */
-  SK_FIXUP_REDUCE = 2      /* per-CTA fp32 partial + flag; the tile's first CTA adds the others in
+  SK_FIXUP_REDUCE = 2,     /* per-CTA fp32 partial + flag; the tile's first CTA adds the others in
                               ascending CTA order: bitwise reproducible */
+  SK_FIXUP_ATOMIC_C = 3    /* the reference's own fix-up (streamk_fp16.py:248-255, atomic_addx2 on half2): every
+                              segment of a split tile rounds its partial sums to C's 16-bit type and adds them
+                              into C with packed 16-bit atomic adds; no workspace.  The library zero-fills C
+                              first (the reference leaves that to its caller).  Every partial is rounded, so it
+                              is less accurate than the other two, and like ATOMIC not reproducible.  fp16 and
+                              bfloat16 tile kernels with 16x16 accumulator blocks only (256x256, 128x128,
+                              128x256, 256x128); N and ldc even, C 4-byte aligned; no bias / activation */
 } sk_fixup;
 
 typedef enum sk_dtype {

@@ -121,6 +121,16 @@ __global__ void prepare_static_kernel(int *status, int *flags, int nflags, uint4
   }
 }
 
+// zero-fill of a 16-bit C, two elements per store (rows of `pairs` pairs, `ld` pairs apart), for the fix-up that adds
+// its partial tiles into C
+__global__ void zero_pairs_kernel(uint32_t *C, int M, int pairs, int64_t ld) {
+  const int64_t total = (int64_t)M * pairs;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = i / pairs;
+    C[r * ld + (i - r * pairs)] = 0u;
+  }
+}
+
 int check_plan(const sk_plan *plan, int64_t M, int64_t N, int64_t K, int dtype, int layout) {
   if (!plan) return SK_ERR_NULL;
   if (plan->M != M || plan->N != N || plan->K != K || plan->dtype != dtype || plan->layout != layout)
@@ -171,7 +181,7 @@ int make_dev_plan(const sk_plan *plan, const KernelInfo *k, void *ws, size_t ws_
   dp->sk_full = plan->streamk_full_tiles;
   dp->sk_extra = plan->streamk_partial_tiles;
   dp->grid = plan->grid;
-  dp->fixup = plan->fixup == SK_FIXUP_ATOMIC ? FIXUP_ATOMIC : FIXUP_REDUCE;
+  dp->fixup = plan->fixup == SK_FIXUP_ATOMIC ? FIXUP_ATOMIC : (plan->fixup == SK_FIXUP_ATOMIC_C ? FIXUP_ATOMIC_C : FIXUP_REDUCE);
   dp->raster = plan->raster;
   dp->spin_limit = plan->spin_limit > 0 ? plan->spin_limit : (1 << 22);
   dp->xcd_remap = (plan->grid % 8 == 0) ? 1 : 0;
@@ -312,6 +322,15 @@ static int gemm_16bit(int dtype, const void *A, const void *B, void *C, int64_t 
   DevPlan dp;
   Workspace w;
   const bool skinny = k->family == FAMILY_SKINNY;
+  if (plan->fixup == SK_FIXUP_ATOMIC_C && plan->streamk_tiles > 0) {
+    // partial tiles are added into C itself, two elements per atomic: C starts at zero, pairs must be aligned,
+    // and there is no CTA that would apply a bias once
+    if (bias != nullptr || skinny) return SK_ERR_CONFIG;
+    if ((N % 2) || (ldc % 2) || (reinterpret_cast<uintptr_t>(C) & 3)) return SK_ERR_ALIGN;
+    hipLaunchKernelGGL(zero_pairs_kernel, dim3(1024), dim3(256), 0, (hipStream_t)stream, reinterpret_cast<uint32_t *>(C),
+                       (int)M, (int)(N / 2), (int64_t)(ldc / 2));
+    if (hipGetLastError() != hipSuccess) return SK_ERR_LAUNCH;
+  }
   rc = make_dev_plan(plan, k, ws, ws_bytes, cached_occupancy(k->id, skinny ? 1 : 0), (hipStream_t)stream, &dp, &w,
                      is_static);
   if (rc) return rc;

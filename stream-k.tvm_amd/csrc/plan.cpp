@@ -280,7 +280,12 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
   out->dp_waves = (int32_t)cdiv(out->blocking_tiles, grid);
   int fixup = cfg ? cfg->fixup : SK_FIXUP_AUTO;
   if (fixup == SK_FIXUP_AUTO) fixup = SK_FIXUP_REDUCE;
-  if (fixup != SK_FIXUP_ATOMIC && fixup != SK_FIXUP_REDUCE) return SK_ERR_CONFIG;
+  if (fixup != SK_FIXUP_ATOMIC && fixup != SK_FIXUP_REDUCE && fixup != SK_FIXUP_ATOMIC_C) return SK_ERR_CONFIG;
+  // packed 16-bit atomics into C: the 16-bit tile kernels with 16x16 accumulator blocks
+  if (fixup == SK_FIXUP_ATOMIC_C &&
+      !(k->family == FAMILY_TILE && (k->variant == 4 || k->variant == 5 || k->variant == 7) &&
+        (dtype == SK_F16 || dtype == SK_BF16) && N % 2 == 0))
+    return SK_ERR_CONFIG;
   out->fixup = fixup;
   out->spin_limit = cfg && cfg->spin_limit > 0 ? cfg->spin_limit : (1 << 22);
   out->raster = cfg ? cfg->raster : 0;
@@ -292,7 +297,7 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
 
   // workspace: status block, fixed-size flag area, fp32 partial tiles
   int64_t ws = 0;
-  if (sk_tiles > 0) {
+  if (sk_tiles > 0 && fixup != SK_FIXUP_ATOMIC_C) {
     const int64_t nflags = fixup == SK_FIXUP_REDUCE ? grid : sk_tiles;
     if (nflags > WS_MAX_FLAGS) return SK_ERR_CONFIG;
     ws = WS_PART_OFF + nflags * (int64_t)k->partial_elems * 4;

@@ -16,7 +16,7 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 
-enum { FIXUP_ATOMIC = 1, FIXUP_REDUCE = 2 };
+enum { FIXUP_ATOMIC = 1, FIXUP_REDUCE = 2, FIXUP_ATOMIC_C = 3 };
 
 // Phase tracing (off unless the small-M translation unit is built with -DSK_PHASE_TRACE): thread 0
 // of every CTA stores the shader clock counter into slot `slot` of its row of g_trace_buf; the host
@@ -67,7 +67,7 @@ struct DevPlan {
   int total_tiles, sk_tiles;  // Stream-K tiles are ids [0, sk_tiles)
   int sk_full, sk_extra;      // iterations per CTA / CTAs that get one more
   int grid;                   // persistent CTAs
-  int fixup;                  // FIXUP_ATOMIC or FIXUP_REDUCE
+  int fixup;                  // FIXUP_ATOMIC, FIXUP_REDUCE or FIXUP_ATOMIC_C
   int raster;                 // 0 row-major, g > 0 grouped by g tile rows
   int spin_limit;             // polls before a waiting owner gives up
   int xcd_remap;              // 1: spread logical CTA ids so each XCD owns a contiguous range
@@ -348,6 +348,20 @@ __device__ __forceinline__ floatx4 bias4_at(const half_t *bias, int col, int N) 
 __device__ __forceinline__ void atomic_add_f32(float *p, float v) {
   // hardware global_atomic_add_f32, no return value, device scope
   __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Two fp32 values, rounded to C's 16-bit type, added to two adjacent elements of C with one packed atomic
+// (global_atomic_pk_add_f16 / _bf16; p 4-byte aligned): the reference's atomic_addx2, streamk_fp16.py:248-255
+template <bool BF16>
+__device__ __forceinline__ void atomic_add_pair16(half_t *p, float x0, float x1) {
+  if constexpr (BF16) {
+    typedef short short2v __attribute__((ext_vector_type(2)));
+    const __bf16 b0 = (__bf16)x0, b1 = (__bf16)x1;
+    const short2v v = {__builtin_bit_cast(short, b0), __builtin_bit_cast(short, b1)};
+    __builtin_amdgcn_global_atomic_fadd_v2bf16((__attribute__((address_space(1))) short2v *)p, v);
+  } else {
+    const half2v v = {(half_t)x0, (half_t)x1};
+    __builtin_amdgcn_global_atomic_fadd_v2f16((__attribute__((address_space(1))) half2v *)p, v);
+  }
 }
 __device__ __forceinline__ void atomic_add_i32(int *p, int v) {
   __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -16,12 +16,17 @@
 namespace sk {
 
 // optional members of a policy: COHERENT_REDUCE (partials of the REDUCE fix-up travel with device-scope
-// accesses; default: as COHERENT_PARTIALS says) and HALVES (the policy has store_partial_half /
-// add_partial_half / store_c_half, see below)
+// accesses; default: as COHERENT_PARTIALS says), HALVES (the policy has store_partial_half /
+// add_partial_half / store_c_half, see below) and ATOMIC_C (the policy has atomic_c: its accumulators added to C
+// with packed 16-bit atomics)
 template <class P, class = void>
 struct reduce_is_coherent { static constexpr bool value = P::COHERENT_PARTIALS; };
 template <class P>
 struct reduce_is_coherent<P, std::void_t<decltype(P::COHERENT_REDUCE)>> { static constexpr bool value = P::COHERENT_REDUCE; };
+template <class P, class = void>
+struct has_atomic_c { static constexpr bool value = false; };
+template <class P>
+struct has_atomic_c<P, std::void_t<decltype(P::ATOMIC_C)>> { static constexpr bool value = P::ATOMIC_C; };
 template <class P, class = void>
 struct has_halves { static constexpr bool value = false; };
 template <class P>
@@ -84,7 +89,11 @@ __device__ __forceinline__ void run_persistent(const typename P::Args &a, const 
     // a segment that is the whole tile is simply stored (streamk_fp32.py:128-129)
     bool store = (n == ipt) || !FIXUP;
     if (FIXUP && !store) {
-      if (plan.fixup == FIXUP_ATOMIC) {
+      if (plan.fixup == FIXUP_ATOMIC_C) {
+        // the reference's fix-up (streamk_fp16.py:248-255): every partial goes straight into C, which the
+        // launcher has zero-filled; nobody finishes the tile
+        if constexpr (has_atomic_c<P>::value) P::atomic_c(a, acc, pm, pn);
+      } else if (plan.fixup == FIXUP_ATOMIC) {
         // fp32 atomicAdd into the tile's accumulation buffer; whoever completes the K range
         // converts and stores, then leaves buffer and counter zeroed for the next launch.
         float *part = ws.partials + (size_t)tile * P::TILE_ELEMS;

@@ -276,6 +276,28 @@ struct TileF16Asm {
   static constexpr bool COHERENT_PARTIALS = false;
   static constexpr bool COHERENT_REDUCE = true;
   static constexpr bool HALVES = true;
+  // the reference's fix-up: partial sums rounded to C's type and added into C (fp16 / bfloat16 only)
+  static constexpr bool ATOMIC_C = MODE_ <= 1;
+  static __device__ __forceinline__ void atomic_c(const Args &a, const Acc &, int pm, int pn) {
+    if constexpr (ATOMIC_C) {
+      const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+      const int wm = wave >> 1, wn = wave & 1;
+      const int row0 = pm * BM + wm * WTM + (lane & 15), col0 = pn * BN + wn * WTN + 4 * (lane >> 4);
+      static_for<0, FM>([&](auto bi) {
+        constexpr int ii = decltype(bi)::value;
+        static_for<0, FN>([&](auto bj) {
+          constexpr int j = decltype(bj)::value;
+          const floatx4 x = agpr_read4<(ii * FN + j) * 4>();
+          const int grow = row0 + 16 * ii, gcol = col0 + 16 * j;
+          if (grow < a.M && gcol < a.N) {  // (N is even: a pair never straddles the edge)
+            half_t *p = a.C + (int64_t)grow * a.ldc + gcol;
+            atomic_add_pair16<BF16_>(p, x[0], x[1]);
+            if (gcol + 2 < a.N) atomic_add_pair16<BF16_>(p + 2, x[2], x[3]);
+          }
+        });
+      });
+    }
+  }
   template <int V0, int V1>
   static __device__ __forceinline__ void store_groups(float *dst) {
     const BufferRsrc r = make_rsrc(dst, TILE_ELEMS * 4);

@@ -897,6 +897,27 @@ struct TileF16NTDma {
   // both CTAs of a tile cut in two finish half of it each (see run_persistent); needs accumulator blocks of
   // 16 rows and at least two of them per wave
   static constexpr bool HALVES = MFMA16_ && FM % 2 == 0;
+  // the reference's fix-up: partial sums rounded to C's type and added into C (fp16 / bfloat16, 16x16 blocks)
+  static constexpr bool ATOMIC_C = MFMA16_ && F8_ == 0 && !Q4_;
+  static __device__ __forceinline__ void atomic_c(const Args &a, const Acc &acc, int pm, int pn) {
+    if constexpr (ATOMIC_C) {
+      // lane l of block (ii, jj) holds row 16 ii + l % 16, columns 16 jj + 4 (l / 16) .. + 3 of the wave tile
+      const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+      const int wm = wave / WN, wn = wave % WN;
+      const int row0 = pm * BM + wm * WTM + (lane & 15), col0 = pn * BN + wn * WTN + 4 * (lane >> 4);
+#pragma unroll
+      for (int ii = 0; ii < FM; ++ii)
+#pragma unroll
+        for (int jj = 0; jj < FN; ++jj) {
+          const int grow = row0 + 16 * ii, gcol = col0 + 16 * jj;
+          if (grow < a.M && gcol < a.N) {  // (N is even: a pair never straddles the edge)
+            half_t *p = a.C + (int64_t)grow * a.ldc + gcol;
+            atomic_add_pair16<BF16_>(p, acc.v[ii][jj][0], acc.v[ii][jj][1]);
+            if (gcol + 2 < a.N) atomic_add_pair16<BF16_>(p + 2, acc.v[ii][jj][2], acc.v[ii][jj][3]);
+          }
+        }
+    }
+  }
   // partials in the workspace: float4 group v of thread t at (v * NT + t) * 4 (ordered reduce),
   // element s of thread t at s * NT + t (atomic accumulation buffer); see tile_f16.h
   template <int V0, int V1>

@@ -24,7 +24,7 @@ def num_cus():
 
 def make_config(config=None, **kw):
     """dict / kwargs -> SkConfig.  Keys: bm, bn, bk, grid, schedule ('auto'|'dp'|'sk2'|'sk1'|
-    'basic'|'splitk'), split, fixup ('auto'|'atomic'|'reduce'), raster, spin_limit, variant."""
+    'basic'|'splitk'), split, fixup ('auto'|'atomic'|'reduce'|'atomic_c'), raster, spin_limit, variant."""
     d = dict(config or {})
     d.update(kw)
     c = SkConfig()

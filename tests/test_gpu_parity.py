@@ -100,6 +100,67 @@ def test_cfg2_streamk_both_fixups(sk, oracle, cfg, fixup):
     assert _rel(oracle, C, ref) <= 1e-3 <= TOL
 
 
+def test_reference_fixup_packed_atomics_into_c(sk, oracle):
+    """The reference's own fix-up (streamk_fp16.py:248-255): every segment of a split tile rounds its partial to
+    C's type and adds it into C with packed 16-bit atomics, no workspace, C zero-filled by the library (handed
+    over full of garbage here).  Exact on integer data (every partial and every sum is an integer below 2048);
+    within 1e-2 of the fp32 host product on U[-1,1) data (each of the few partials is rounded once); fp16 and
+    bfloat16, NT and NN, the eight-wave 16x16x32 kernels and the assembly-loop kernel, ragged M and N (N even);
+    refused for other kernels, an odd N, a bias."""
+    import torch
+    rng = np.random.default_rng(29)
+    ran = 0
+    for (M, N, K) in [(1024, 1024, 8192), (200, 136, 320), (1000, 1096, 2048), (520, 266, 448)]:
+        Ai = rng.integers(-1, 2, (M, K)).astype(np.float16)
+        Bi = rng.integers(-1, 2, (N, K)).astype(np.float16)
+        Ai[:, 1500:] = 0
+        exact = Ai.astype(np.int32) @ Bi.astype(np.int32).T
+        assert np.abs(exact).max() < 2048
+        Ar = (rng.random((M, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+        Br = (rng.random((N, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+        ref = oracle.matmul_fp32(Ar, Br, trans_b=True)
+        for layout in ("nt", "nn"):
+            if layout == "nn" and N % 8:
+                continue
+            dAi, dAr = _t(Ai), _t(Ar)
+            dBi = _t(np.ascontiguousarray(Bi.T) if layout == "nn" else Bi)
+            dBr = _t(np.ascontiguousarray(Br.T) if layout == "nn" else Br)
+            for tile in (dict(bm=128, bn=128, bk=64, variant=5), dict(bm=256, bn=256, bk=64, variant=5), dict(bm=256, bn=256, bk=64, variant=8),
+                         dict(bm=128, bn=256, bk=64, variant=5)):
+                if layout == "nn" and tile["bm"] != tile["bn"]:
+                    continue
+                for sch in (dict(schedule="sk2"), dict(schedule="basic", grid=24), dict(schedule="splitk", split=2)):
+                    try:
+                        plan = sk.make_plan(M, N, K, "float16", layout, dict(tile, fixup="atomic_c", **sch))
+                    except sk.StreamKError:
+                        assert tile.get("variant") == 8 and K % 64 or sch["schedule"] == "splitk"
+                        continue
+                    assert plan.workspace_bytes == 0
+                    out = torch.full((M, N), 777.0, dtype=torch.float16, device="cuda")
+                    C = sk.streamk_fp16(dAi, dBi, plan=plan, layout=layout, out=out)
+                    assert np.array_equal(C.cpu().numpy().astype(np.int32), exact), (M, N, K, layout, tile, sch)
+                    C = sk.streamk_fp16(dAr, dBr, plan=plan, layout=layout, out=out)
+                    assert _rel(oracle, C, ref) <= 4e-3 <= TOL, (M, N, K, layout, tile, sch)
+                    if tile == dict(bm=256, bn=256, bk=64, variant=8) and layout == "nt":
+                        pb = sk.make_plan(M, N, K, "bfloat16", layout, dict(tile, fixup="atomic_c", **sch))
+                        Cb = sk.streamk_bf16(dAi.bfloat16(), dBi.bfloat16(), plan=pb, out=torch.full((M, N), -3.0, dtype=torch.bfloat16, device="cuda"))
+                        # (partials and sums are rounded to bfloat16's eight bits: integers are exact only below 256)
+                        assert _rel(oracle, Cb, exact.astype(np.float32)) <= 2e-2, (M, N, K, tile, sch)
+                    ran += 1
+    assert ran >= 40
+    # not for the 32x32 accumulator kernels, the small-M kernels, an odd N or a bias
+    with pytest.raises(sk.StreamKError):
+        sk.make_plan(1024, 1024, 8192, "float16", "nt", dict(bm=128, bn=128, bk=64, variant=2, schedule="sk2", fixup="atomic_c"))
+    with pytest.raises(sk.StreamKError):
+        sk.make_plan(16, 1024, 8192, "float16", "nt", dict(schedule="sk2", fixup="atomic_c"))
+    with pytest.raises(sk.StreamKError):
+        sk.make_plan(1024, 1023, 8192, "float16", "nt", dict(bm=128, bn=128, bk=64, variant=5, schedule="sk2", fixup="atomic_c"))
+    A, B = _t(_uniform16((512, 1024), 3)), _t(_uniform16((512, 1024), 4))
+    with pytest.raises(sk.StreamKError):
+        sk.streamk_fp16(A, B, bm=128, bn=128, bk=64, variant=5, schedule="sk2", fixup="atomic_c", bias=torch.zeros(512, dtype=torch.float16, device="cuda"))
+    sk.workspace_status()
+
+
 def test_assembly_loop_tile_kernels(sk, oracle, golden_dir):
     """The four-wave 256 x 256 x 64 kernels whose K loop is hand-scheduled assembly (accumulators in the
     accumulation registers): fp16 and bfloat16, NT and NN, ragged M and N, K any multiple of 64 (odd and even iteration
