@@ -384,7 +384,8 @@ def _register(name, before_out, after_out, run, out_meta):
     def functional(*args):
         shape, dtype = out_meta(*args)
         C = torch.empty(shape, dtype=dtype, device=args[0].device)
-        run(*args[:out_pos], C, *args[out_pos:])
+        if C.numel() > 0:   # an empty batch (no rows of A) has nothing to launch
+            run(*args[:out_pos], C, *args[out_pos:])
         return C
 
     def functional_fake(*args):
@@ -392,7 +393,8 @@ def _register(name, before_out, after_out, run, out_meta):
         return args[0].new_empty(shape, dtype=dtype)
 
     def out_variant(*args):
-        run(*args)
+        if args[out_pos].numel() > 0 or args[0].shape[0] > 0:
+            run(*args)
 
     _LIBRARY.impl(name, functional, "CUDA")
     _LIBRARY.impl(f"{name}_out", out_variant, "CUDA")

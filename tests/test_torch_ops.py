@@ -86,6 +86,24 @@ def test_operator_equals_direct_c_abi_call(sk):
 
 
 @pytest.mark.gpu
+def test_empty_batch_returns_an_empty_result(sk):
+    """No rows of A: the operators return an empty C without a launch (torch.nn.Linear does the same); a wrong
+    `out` is still refused."""
+    import torch
+    A = torch.empty(0, 256, dtype=torch.float16, device="cuda")
+    B = torch.randn(72, 256, device="cuda").half()
+    C = torch.ops.streamk.gemm_f16(A, B)
+    assert C.shape == (0, 72) and C.dtype == torch.float16
+    assert sk.streamk_fp16(A, B).shape == (0, 72)
+    lin = sk.StreamKLinear.from_linear(torch.nn.Linear(256, 72).cuda().half())
+    assert lin(A).shape == (0, 72) and lin(A.reshape(0, 3, 256)).shape == (0, 3, 72)
+    out = torch.empty(0, 72, dtype=torch.float16, device="cuda")
+    assert torch.ops.streamk.gemm_f16_out(A, B, out) is None
+    with pytest.raises(ValueError):
+        torch.ops.streamk.gemm_f16_out(A, B, torch.empty(1, 72, dtype=torch.float16, device="cuda"))
+
+
+@pytest.mark.gpu
 def test_linear_module_compiles_without_a_graph_break(sk):
     import torch
     import torch._dynamo
