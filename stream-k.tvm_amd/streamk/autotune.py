@@ -238,6 +238,8 @@ def autotune(M, N, K, dtype="float16", layout="nt", *, configs=None, warmup=5, r
     for cfg in configs:
         try:
             p = _plan.make_plan(M, N, K, dtype, layout, cfg)
+            if cfg.get("schedule", "dp") != "dp" and p.streamk_tiles == 0:
+                continue  # the grid leaves no tile to split: this candidate is the data-parallel one under another name
             run(p)
             torch.cuda.synchronize()
             ops.workspace_status()
@@ -260,8 +262,24 @@ def autotune(M, N, K, dtype="float16", layout="nt", *, configs=None, warmup=5, r
             best = (ms, cfg)
     if best is None:
         raise RuntimeError(f"no valid configuration for {M}x{N}x{K} {dtype}/{layout}")
+    # Microsecond kernels: one timing of a candidate is good to a few percent, which is also what separates the
+    # leaders.  The five best (and the best data-parallel one) are timed again, twice, in alternation; a candidate's
+    # figure is the smaller of the two.
+    if small and len(results) > 1:
+        results.sort(key=lambda r: r[0])
+        finalists = results[:5] + [r for r in results[5:] if r[1].get("schedule") == "dp"][:1]
+        again = {id(r): [] for r in finalists}
+        for _ in range(2):
+            for r in finalists:
+                p = _plan.make_plan(M, N, K, dtype, layout, r[1])
+                again[id(r)].append(_time_ms(lambda: run(p), warmup, 2 * rep, small))
+        results = [(min(again[id(r)]), r[1]) for r in finalists]
+        best = min(results, key=lambda r: r[0])
+        if verbose:
+            for ms, cfg in sorted(results, key=lambda r: r[0]):
+                print(f"  again {ms * 1e3:9.2f} us  {cfg}")
     # within the noise of the measurement prefer a data-parallel plan: no workspace, no fix-up code in the kernel
-    near = [r for r in results if r[0] <= best[0] * 1.015 and r[1].get("schedule") == "dp"]
+    near = [r for r in results if r[0] <= best[0] * (1.03 if small else 1.015) and r[1].get("schedule") == "dp"]
     if near and best[1].get("schedule") != "dp":
         best = min(near, key=lambda r: r[0])
     if cache:
