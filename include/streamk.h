@@ -81,7 +81,8 @@ typedef enum sk_dtype {
   SK_F8E4M3 = 5,   /* A and B one byte per element, OCP e4m3 (bias 7, no infinities, NaN = S.1111.111); C fp16 */
   SK_I8 = 6,       /* A and B int8, C int32 */
   SK_Q4_ZP = 7,    /* as SK_Q4 with one zero point per scale group and row (sk_gemm_q4_zp) */
-  SK_F8E5M2 = 8    /* as SK_F8E4M3 for OCP e5m2 bytes (the upper byte of an fp16: bias 15, infinities and NaNs) */
+  SK_F8E5M2 = 8,   /* as SK_F8E4M3 for OCP e5m2 bytes (the upper byte of an fp16: bias 15, infinities and NaNs) */
+  SK_Q4_ZP_TILED = 9 /* as SK_Q4_ZP with the nibbles in the tiled layout of SK_Q4_TILED (scales and zero points row-major) */
 } sk_dtype;
 
 /* Tunables; a zero field means "choose for me".  Replaces the module-level constants and
@@ -224,7 +225,7 @@ int sk_gemm_bf16_ex(const void *A, const void *B, void *C, int64_t M, int64_t N,
                     int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws, size_t ws_bytes, void *stream,
                     const sk_epilogue *epi);
 /* Q4 with the epilogue: zeros == NULL is sk_gemm_q4 (plan dtype SK_Q4 or SK_Q4_TILED, scalar `zero`),
- * otherwise sk_gemm_q4_zp (plan dtype SK_Q4_ZP, `zero` ignored). */
+ * otherwise sk_gemm_q4_zp (plan dtype SK_Q4_ZP or SK_Q4_ZP_TILED, `zero` ignored). */
 int sk_gemm_q4_ex(const void *A, const void *Wq, const void *scales, const void *zeros, void *C, int64_t M,
                   int64_t N, int64_t K, int64_t lda, int64_t ldc, int group, int zero, const sk_plan *plan,
                   void *ws, size_t ws_bytes, void *stream, const sk_epilogue *epi);
@@ -295,7 +296,9 @@ int sk_gemm_q4(const void *A, const void *Wq, const void *scales, void *C, int64
  * not cover.  The plan is made with dtype SK_Q4_ZP; at most 64 rows per call.  M == 1 takes matrix-vector kernels
  * that, like sk_gemm_q4's, multiply the nibbles undecoded and apply zero point and scale to fp32 group sums (the
  * unrounded (q - zero) * scale); 2 <= M <= 64, and M == 1 with an explicit variant-0 plan, the general small-M
- * kernels, which form the rounded weights bit for bit. */
+ * kernels, which form the rounded weights bit for bit.
+ * A plan made with dtype SK_Q4_ZP_TILED takes Wq in the tiled layout (sk_q4_tile_host / sk_q4_tile; scales and
+ * zeros stay row-major): the same kernels with the tiled loads, results bit for bit those of SK_Q4_ZP. */
 int sk_gemm_q4_zp(const void *A, const void *Wq, const void *scales, const void *zeros, void *C, int64_t M,
                   int64_t N, int64_t K, int64_t lda, int64_t ldc, int group, const sk_plan *plan, void *ws,
                   size_t ws_bytes, void *stream);

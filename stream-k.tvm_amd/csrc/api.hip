@@ -464,7 +464,7 @@ static int gemm_q4_any(const void *A, const void *Wq, const void *scales, const 
                        const sk_epilogue *epi = nullptr) {
   const void *bias = nullptr;  // the kernels' epilogue word: bias pointer and activation code
   if (int rc = epilogue_word(epi, &bias)) return rc;
-  if (!A || !Wq || !scales || !C || (dtype == SK_Q4_ZP && !zeros)) return SK_ERR_NULL;
+  if (!A || !Wq || !scales || !C || ((dtype == SK_Q4_ZP || dtype == SK_Q4_ZP_TILED) && !zeros)) return SK_ERR_NULL;
   int rc = check_plan(plan, M, N, K, dtype, SK_LAYOUT_NT);
   if (rc) return rc;
   if (group != 128 || zero < 0 || zero > 15) return SK_ERR_CONFIG;
@@ -508,7 +508,8 @@ extern "C" int sk_gemm_q4(const void *A, const void *Wq, const void *scales, voi
 extern "C" int sk_gemm_q4_ex(const void *A, const void *Wq, const void *scales, const void *zeros, void *C,
                              int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc, int group, int zero,
                              const sk_plan *plan, void *ws, size_t ws_bytes, void *stream, const sk_epilogue *epi) {
-  const int dtype = zeros ? SK_Q4_ZP : (plan && plan->dtype == SK_Q4_TILED ? SK_Q4_TILED : SK_Q4);
+  const int dtype = zeros ? (plan && plan->dtype == SK_Q4_ZP_TILED ? SK_Q4_ZP_TILED : SK_Q4_ZP)
+                          : (plan && plan->dtype == SK_Q4_TILED ? SK_Q4_TILED : SK_Q4);
   return gemm_q4_any(A, Wq, scales, zeros, C, M, N, K, lda, ldc, group, zeros ? 0 : zero, dtype, plan, ws, ws_bytes,
                      stream, epi);
 }
@@ -516,7 +517,8 @@ extern "C" int sk_gemm_q4_ex(const void *A, const void *Wq, const void *scales, 
 extern "C" int sk_gemm_q4_zp(const void *A, const void *Wq, const void *scales, const void *zeros, void *C,
                              int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc, int group,
                              const sk_plan *plan, void *ws, size_t ws_bytes, void *stream) {
-  return gemm_q4_any(A, Wq, scales, zeros, C, M, N, K, lda, ldc, group, 0, SK_Q4_ZP, plan, ws, ws_bytes, stream);
+  const int dtype = plan && plan->dtype == SK_Q4_ZP_TILED ? SK_Q4_ZP_TILED : SK_Q4_ZP;  // which layout Wq is in
+  return gemm_q4_any(A, Wq, scales, zeros, C, M, N, K, lda, ldc, group, 0, dtype, plan, ws, ws_bytes, stream);
 }
 
 namespace {

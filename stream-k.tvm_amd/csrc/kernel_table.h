@@ -182,6 +182,21 @@ struct KernelInfo {
   X(224, 1, 1, 4, 2, 2)           \
   X(225, 1, 1, 1, 4, 4)
 
+// Per-group zero points with tiled weights (dtype SK_Q4_ZP_TILED): twins of SK_GEMV_Q4ZP_KERNELS and
+// SK_SKINNY_Q4ZP_KERNELS (translation unit kernels_gemv_rows.hip)
+#define SK_GEMV_Q4ZPT_KERNELS(X) \
+  X(156, 1, 1, 4, 4, 16384)      \
+  X(157, 1, 2, 2, 4, 16384)      \
+  X(158, 1, 1, 4, 4, 32768)      \
+  X(159, 1, 4, 1, 4, 16384)
+#define SK_SKINNY_Q4ZPT_KERNELS(X) \
+  X(300, 1, 1, 4, 1, 4)            \
+  X(301, 2, 1, 4, 1, 2)            \
+  X(302, 4, 1, 4, 1, 2)            \
+  X(303, 1, 1, 2, 4, 2)            \
+  X(304, 1, 1, 4, 2, 2)            \
+  X(305, 1, 1, 1, 4, 4)
+
 // M == 1 fp16 (NT) matrix-vector kernels (variant 2):  X(id, NB, WN, RK, DEPTH, KMAX)
 #define SK_GEMV_F16_KERNELS(X) \
   X(160, 1, 1, 4, 4, 8192)     \

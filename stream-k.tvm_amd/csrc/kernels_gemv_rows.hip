@@ -1,4 +1,5 @@
-// Small-M kernels in the matrix-vector kernels' form (tile_gemv_rows.h): 2 <= M <= 16, fp16 / bfloat16, NT.
+// Small-M kernels in the matrix-vector kernels' form (tile_gemv_rows.h): 2 <= M <= 16, fp16 / bfloat16, NT;
+// and the Q4 kernels for per-group zero points with tiled weights (dtype 9, SK_Q4_ZP_TILED).
 #include "skinny_launch.h"
 
 namespace sk {
@@ -21,6 +22,23 @@ int gemv_rows_kernel_infos(KernelInfo *out, int max) {
   }
   SK_GEMV_ROWS_BF16_KERNELS(X)
 #undef X
+#define X(id, NB, WN, RK, DEPTH, KMAX)                                                                         \
+  if (n < max) {                                                                                               \
+    typedef TileGemvQ4<NB, WN, RK, DEPTH, KMAX, true, true> P;                                                 \
+    out[n++] = KernelInfo{id, FAMILY_SKINNY, 9, 0, 2, P::BM, P::BN, P::BKC, P::NT, P::LDS_BYTES, P::CTAS_PER_CU, \
+                          P::TILE_ELEMS, P::MAX_ITERS, P::MAX_M, 128,                                          \
+                          "gemv_q4zpt_nb" #NB "_wn" #WN "_rk" #RK "_k" #KMAX};                                  \
+  }
+  SK_GEMV_Q4ZPT_KERNELS(X)
+#undef X
+#define X(id, MB, NB, WN, RK, DEPTH)                                                                           \
+  if (n < max) {                                                                                               \
+    typedef TileSkinny<MB, NB, WN, RK, true, DEPTH, false, true, true> P;                                      \
+    out[n++] = KernelInfo{id, FAMILY_SKINNY, 9, 0, 0, P::BM, P::BN, P::BKC, P::NT, P::LDS_BYTES, P::CTAS_PER_CU, \
+                          P::TILE_ELEMS, P::SC_MAX_ITERS, P::MAX_M, 128, "skinny_q4zpt_mb" #MB "_wn" #WN "_rk" #RK}; \
+  }
+  SK_SKINNY_Q4ZPT_KERNELS(X)
+#undef X
   return n;
 }
 
@@ -39,6 +57,20 @@ int launch_gemv_rows(int id, const SkinnyArgs &a, const DevPlan &p, const Worksp
     return launch_policy<P>(a, p, ws, s, bias);          \
   }
     SK_GEMV_ROWS_BF16_KERNELS(X)
+#undef X
+#define X(id_, NB, WN, RK, DEPTH, KMAX)                        \
+  case id_: {                                                  \
+    typedef TileGemvQ4<NB, WN, RK, DEPTH, KMAX, true, true> P; \
+    return launch_policy<P>(a, p, ws, s, bias);                \
+  }
+    SK_GEMV_Q4ZPT_KERNELS(X)
+#undef X
+#define X(id_, MB, NB, WN, RK, DEPTH)                                      \
+  case id_: {                                                              \
+    typedef TileSkinny<MB, NB, WN, RK, true, DEPTH, false, true, true> P;  \
+    return launch_policy<P>(a, p, ws, s, bias);                            \
+  }
+    SK_SKINNY_Q4ZPT_KERNELS(X)
 #undef X
   }
   return (int)hipErrorInvalidValue;
@@ -64,6 +96,24 @@ int occupancy_gemv_rows(int id) {
     return occ;                                                                                          \
   }
     SK_GEMV_ROWS_BF16_KERNELS(X)
+#undef X
+#define X(id_, NB, WN, RK, DEPTH, KMAX)                                                                  \
+  case id_: {                                                                                            \
+    typedef TileGemvQ4<NB, WN, RK, DEPTH, KMAX, true, true> P;                                           \
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_skinny_kernel<P>, P::NT, 0) != hipSuccess) \
+      return -1;                                                                                         \
+    return occ;                                                                                          \
+  }
+    SK_GEMV_Q4ZPT_KERNELS(X)
+#undef X
+#define X(id_, MB, NB, WN, RK, DEPTH)                                                                    \
+  case id_: {                                                                                            \
+    typedef TileSkinny<MB, NB, WN, RK, true, DEPTH, false, true, true> P;                                \
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_skinny_kernel<P>, P::NT, 0) != hipSuccess) \
+      return -1;                                                                                         \
+    return occ;                                                                                          \
+  }
+    SK_SKINNY_Q4ZPT_KERNELS(X)
 #undef X
   }
   return -1;

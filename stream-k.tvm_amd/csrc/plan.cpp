@@ -81,7 +81,7 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
   // every CU something to do
   const KernelInfo *best = nullptr;
   // (for 32 < M <= 64 the 64x64 LDS tile below is faster than streaming the weights past 64 rows)
-  const bool q4 = dtype == SK_Q4 || dtype == SK_Q4_TILED || dtype == SK_Q4_ZP;
+  const bool q4 = dtype == SK_Q4 || dtype == SK_Q4_TILED || dtype == SK_Q4_ZP || dtype == SK_Q4_ZP_TILED;
   // (one-byte operands: up to 64 rows -- their tile kernels start at 128 rows)
   const bool one_byte = dtype == SK_F8E4M3 || dtype == SK_F8E5M2 || dtype == SK_I8;
   if (dtype == SK_Q4 && M > 64 && want_variant < 0) {
@@ -107,7 +107,7 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
           return &t[i];
     // 2 <= M <= 16 with Q4 weights: eight waves per CTA (two per SIMD cover each other's waits),
     // 32 weight rows, K split over four waves
-    if (((dtype == SK_Q4 && M > 1) || dtype == SK_Q4_ZP) && M <= 16 && want_variant < 0)
+    if (((dtype == SK_Q4 && M > 1) || dtype == SK_Q4_ZP || dtype == SK_Q4_ZP_TILED) && M <= 16 && want_variant < 0)
       for (int i = 0; i < n; ++i)
         if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].variant == 0 && t[i].bm == 16 &&
             t[i].bn == 32 && t[i].bk == 1024 && accepts_shape(t[i], M, K))
@@ -191,7 +191,7 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
   if (!out) return SK_ERR_NULL;
   if (M <= 0 || N <= 0 || K <= 0 || M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return SK_ERR_SHAPE;
   if (dtype != SK_F16 && dtype != SK_F32 && dtype != SK_Q4 && dtype != SK_BF16 && dtype != SK_Q4_TILED &&
-      dtype != SK_F8E4M3 && dtype != SK_I8 && dtype != SK_Q4_ZP && dtype != SK_F8E5M2)
+      dtype != SK_F8E4M3 && dtype != SK_I8 && dtype != SK_Q4_ZP && dtype != SK_F8E5M2 && dtype != SK_Q4_ZP_TILED)
     return SK_ERR_CONFIG;
   if ((dtype == SK_F8E4M3 || dtype == SK_F8E5M2 || dtype == SK_I8) && layout != SK_LAYOUT_NT) return SK_ERR_CONFIG;
   if (layout != SK_LAYOUT_NT && layout != SK_LAYOUT_NN) return SK_ERR_CONFIG;

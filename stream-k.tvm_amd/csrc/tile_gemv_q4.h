@@ -45,10 +45,10 @@ namespace sk {
 // ZP_: one zero point per scale group and row (a.zeros, the shape of the scales; a.zero is ignored).  The
 // bracket above splits into a part that depends on A only and one that is linear in the zero point:
 //     sum a_k (q_k - z) = c_lo + c_hi / 16 - [1024 sum_even a_k + 64 sum_odd a_k] - z [sum_even a_k + sum_odd a_k]
-// Both sums of A are kept per 32 K-values; the zero points are staged in LDS beside the scales.
+// Both sums of A are kept per 32 K-values; the zero points are staged in LDS beside the scales.  (Scales and
+// zero points are row-major [N, groups] also where the weights are tiled.)
 template <int NB_, int WN_, int RK_, int DEPTH_, int KMAX_ = 16384, bool TILED_ = false, bool ZP_ = false>
 struct TileGemvQ4 {
-  static_assert(!(TILED_ && ZP_), "zero points come with row-major weights");
   typedef SkinnyArgs Args;
   static constexpr bool LEAN_ENTRY = false;  // see run_persistent
   static constexpr int NB = NB_, WN = WN_, RK = RK_, DEPTH = DEPTH_, KMAX = KMAX_;

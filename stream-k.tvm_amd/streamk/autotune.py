@@ -129,7 +129,8 @@ def box_reference_tflops():
 def _time_ms(fn, warmup, rep, graph, min_ms=None):
     """Per-launch time in ms.  The part sets its clock by the power drawn over the last milliseconds, so a burst
     of 20 launches of a compute-bound kernel runs up to 20 % faster than the same kernel sustained; a measurement
-    therefore runs for at least `min_ms` (default _MIN_TIMED_MS), the first half untimed."""
+    therefore runs for at least `min_ms` (default _MIN_TIMED_MS), the first half untimed.  With `graph` (microsecond
+    kernels) the launches are captured and the median of seven groups over a longer window is taken (ops.graph_ms)."""
     min_ms = _MIN_TIMED_MS if min_ms is None else min_ms
     if not graph:
         ms = ops.bench_ms(fn, warmup, rep)
@@ -137,31 +138,7 @@ def _time_ms(fn, warmup, rep, graph, min_ms=None):
         if more > 2 * rep:
             ms = ops.bench_ms(fn, more // 2, more // 2)
         return ms
-    s = torch.cuda.Stream()
-    with torch.cuda.stream(s):
-        for _ in range(max(1, warmup)):
-            fn()
-        torch.cuda.synchronize()
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g, stream=s):
-            for _ in range(rep):
-                fn()
-        g.replay()
-        torch.cuda.synchronize()
-        st, en = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        replays, ms = 3, None
-        for _ in range(2):
-            st.record()
-            for _ in range(replays):
-                g.replay()
-            en.record()
-            torch.cuda.synchronize()
-            ms = st.elapsed_time(en) / (replays * rep)
-            more = int(min_ms / 2 / max(ms * rep, 1e-4)) + 1
-            if more <= replays:
-                break
-            replays = more  # (the pass just timed serves as the untimed half)
-    return ms
+    return ops.graph_ms(fn, launches=rep, warmup=warmup, window_ms=max(3.0 * min_ms, 24.0), groups=7)
 
 
 def autotune(M, N, K, dtype="float16", layout="nt", *, configs=None, warmup=5, rep=20, check=True,

@@ -6,7 +6,7 @@ from ._lib import SkConfig, SkPlan
 
 _DTYPES = {"float16": _lib.SK_F16, "float32": _lib.SK_F32, "q4": _lib.SK_Q4, "bfloat16": _lib.SK_BF16,
            "q4_tiled": _lib.SK_Q4_TILED, "float8_e4m3": _lib.SK_F8E4M3, "float8_e5m2": _lib.SK_F8E5M2,
-           "int8": _lib.SK_I8, "q4_zp": _lib.SK_Q4_ZP}
+           "int8": _lib.SK_I8, "q4_zp": _lib.SK_Q4_ZP, "q4_zp_tiled": _lib.SK_Q4_ZP_TILED}
 _LAYOUTS = {"nt": _lib.LAYOUT_NT, "nn": _lib.LAYOUT_NN}
 _num_cus = None
 

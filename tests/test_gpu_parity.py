@@ -584,6 +584,57 @@ def test_q4_tiled_weights_give_identical_results(sk, oracle):
     sk.workspace_status()
 
 
+def test_q4_tiled_weights_with_per_group_zero_points(sk, oracle):
+    """Per-group zero points with the weights in the tiled layout (scales and zero points stay row-major): every
+    kernel instance reproduces its row-major twin bit for bit (data-parallel and ordered-reduce schedules) and
+    stays within 2e-3 of the fp32 host product of the dequantised weights; ragged N, M from 1 to 64, more than 64
+    rows through the blocks of 64."""
+    import torch
+    rng = np.random.default_rng(93)
+    tiles = [(16, 64, 256), (32, 64, 256), (64, 64, 256), (16, 32, 1024), (16, 64, 512), (16, 16, 1024), (16, 32, 512)]
+    ran, gemv_ran = 0, 0
+    for (M, N, K) in [(1, 1000, 1152), (1, 2048, 4096), (1, 72, 28672), (5, 520, 384), (16, 264, 4096), (33, 200, 640),
+                      (64, 136, 2048)]:
+        A = (rng.random((M, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+        Wq = rng.integers(0, 256, (N, K // 2), dtype=np.uint8)
+        sc = rng.uniform(0.005, 0.02, (N, K // 128)).astype(np.float16)
+        zp = rng.integers(0, 16, (N, K // 128)).astype(np.float16)
+        dA, dW, dS, dZ = _t(A), _t(Wq), _t(sc), _t(zp)
+        dT = sk.tile_q4(dW)
+        ref = oracle.q4_zp_gemm_ref(A, Wq, sc, zp)
+        C = sk.streamk_q4(dA, dT, dS, zeros=dZ, tiled=True)            # heuristic plan
+        assert _rel(oracle, C, ref) <= 2e-3 <= TOL, (M, N, K)
+        assert torch.equal(C, sk.streamk_q4(dA, dW, dS, zeros=dZ)), (M, N, K)
+        for (bm, bn, bk) in tiles:
+            for variant in (0, 1):
+                for sch in (dict(schedule="dp"), dict(schedule="sk2", fixup="reduce", grid=48)):
+                    cfg = dict(bm=bm, bn=bn, bk=bk, **sch)
+                    if variant:
+                        cfg["variant"] = variant
+                    try:
+                        pt = sk.make_plan(M, N, K, "q4_zp_tiled", "nt", cfg)
+                        pr = sk.make_plan(M, N, K, "q4_zp", "nt", cfg)
+                    except sk.StreamKError:
+                        continue
+                    name_t, name_r = sk.kernel_name(pt.kernel_id), sk.kernel_name(pr.kernel_id)
+                    assert name_t.replace("q4zpt", "q4zp") == name_r, (name_t, name_r)
+                    Ct = sk.streamk_q4(dA, dT, dS, zeros=dZ, plan=pt, tiled=True)
+                    assert torch.equal(Ct, sk.streamk_q4(dA, dW, dS, zeros=dZ, plan=pr)), (M, N, K, cfg, name_t)
+                    assert _rel(oracle, Ct, ref) <= 2e-3, (M, N, K, cfg, name_t)
+                    ran += 1
+                    gemv_ran += name_t.startswith("gemv_q4zpt")
+    assert ran >= 60 and gemv_ran >= 8, (ran, gemv_ran)
+    with pytest.raises(ValueError):
+        sk.streamk_q4(dA, dW, dS, zeros=dZ, plan=pt)   # a tiled plan with row-major weights
+    with pytest.raises(ValueError):
+        sk.streamk_q4(dA, dT, dS, plan=pt, tiled=True)  # a zero-point plan without zero points
+    # more rows than one launch takes: blocks of 64 rows
+    A = (rng.random((150, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+    C = sk.streamk_q4(_t(A), dT, dS, zeros=dZ, tiled=True)
+    assert _rel(oracle, C, oracle.q4_zp_gemm_ref(A, Wq, sc, zp)) <= 2e-3
+    sk.workspace_status()
+
+
 def test_q4_matrix_vector_exact_on_integer_data(sk):
     """M = 1, N = K = 8192, A in {-1, 0, 1}, scales 1 (and 0.5): every group sum is an integer
     below 2^24, so the fp32 arithmetic of the matrix-vector kernels is exact and C must equal the
