@@ -99,7 +99,8 @@ typedef struct sk_config {
   int32_t spin_limit;     /* REDUCE fix-up: polls of a peer flag before giving up; 0 = default */
   int32_t reserved[4];    /* reserved[0]: 0 = preferred kernel variant of the tile, v > 0 = variant v - 1
                              (implementation alternatives of one tile shape, for the autotuner);
-                             reserved[1]: split factor of SK_SCHED_SPLIT_K, 0 = choose */
+                             reserved[1]: split factor of SK_SCHED_SPLIT_K, 0 = choose;
+                             reserved[2]: 1 = interleaved order of the Stream-K tiles (see sk_plan.interleave) */
 } sk_config;
 
 /* Result of the host partitioner: the integers of streamk_fp32.py:30-54 for the chosen tile/grid. */
@@ -117,6 +118,14 @@ typedef struct sk_plan {
   int32_t threads;               /* workgroup size of that kernel */
   int32_t lds_bytes;             /* static LDS of that kernel */
   int32_t spin_limit;            /* REDUCE fix-up: polls of a peer's flag before giving up */
+  int32_t interleave;            /* 0 or 1: Stream-K tile ids are positions in the tile order; S > 1: tile id v stands
+                                    at position (v % S) * (streamk_tiles / S) + v / S of it.  With g =
+                                    gcd(streamk_tiles, grid) and S = streamk_tiles / g, the CTAs pid, pid + grid/g,
+                                    pid + 2 grid/g, ... are at the same K offset of their tiles at the same time
+                                    (their ranges start S tiles apart); the interleaved order puts the g tiles they
+                                    work on next to each other in the tile order, so that with a grouped raster they
+                                    share rows of A and columns of B while those are in the L2, as the tiles of a
+                                    data-parallel wave do.  Those CTAs sit on one XCD when grid/g is a multiple of 8. */
   int64_t workspace_bytes;       /* what sk_gemm_* needs for this plan */
   int64_t M, N, K;
 } sk_plan;

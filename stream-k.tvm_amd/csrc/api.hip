@@ -184,7 +184,12 @@ int make_dev_plan(const sk_plan *plan, const KernelInfo *k, void *ws, size_t ws_
   dp->fixup = plan->fixup == SK_FIXUP_ATOMIC ? FIXUP_ATOMIC : (plan->fixup == SK_FIXUP_ATOMIC_C ? FIXUP_ATOMIC_C : FIXUP_REDUCE);
   dp->raster = plan->raster;
   dp->spin_limit = plan->spin_limit > 0 ? plan->spin_limit : (1 << 22);
-  dp->xcd_remap = (plan->grid % 8 == 0) ? 1 : 0;
+  // (the interleaved Stream-K order relies on the hardware's round-robin placement: CTAs a multiple of 8 apart
+  // share an XCD)
+  dp->xcd_remap = (plan->grid % 8 == 0 && plan->interleave <= 1) ? 1 : 0;
+  dp->perm_s = plan->interleave > 1 ? plan->interleave : 1;
+  dp->perm_g = plan->interleave > 1 ? plan->streamk_tiles / plan->interleave : 1;
+  dp->by_perm = FastDiv::make(dp->perm_s);
   const int raster = plan->raster > 0 ? plan->raster : 1;
   dp->raster_tail = plan->num_block_m % raster ? plan->num_block_m % raster : raster;
   // every Stream-K tile cut into exactly two equal CTA segments: both CTAs of a pair finish half a tile

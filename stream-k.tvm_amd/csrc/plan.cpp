@@ -288,6 +288,13 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
     return SK_ERR_CONFIG;
   out->fixup = fixup;
   out->spin_limit = cfg && cfg->spin_limit > 0 ? cfg->spin_limit : (1 << 22);
+  out->interleave = 0;
+  if (cfg && cfg->reserved[2] != 0) {
+    if (cfg->reserved[2] != 1) return SK_ERR_CONFIG;
+    int g = sk_tiles, b = grid;  // gcd
+    while (b) { const int t = g % b; g = b; b = t; }
+    if (sk_tiles > 0 && g > 1 && sk_tiles / g > 1) out->interleave = sk_tiles / g;
+  }
   out->raster = cfg ? cfg->raster : 0;
   if (out->raster < 0) return SK_ERR_CONFIG;
   // default tile order of the LDS-tiled 16-bit and fp8 kernels: groups of 8 tile rows.  Concurrent CTAs
@@ -318,6 +325,8 @@ extern "C" int sk_plan_cta_range(const sk_plan *p, int pid, int32_t *start, int3
 extern "C" int sk_plan_tile_coords(const sk_plan *p, int tile, int32_t *pid_m, int32_t *pid_n) {
   if (!p || !pid_m || !pid_n) return SK_ERR_NULL;
   if (tile < 0 || tile >= p->total_tiles) return SK_ERR_CONFIG;
+  if (p->interleave > 1 && tile < p->streamk_tiles)
+    tile = (tile % p->interleave) * (p->streamk_tiles / p->interleave) + tile / p->interleave;
   if (p->raster <= 0) {  // streamk_fp32.py:106-107
     *pid_m = tile / p->num_block_n;
     *pid_n = tile % p->num_block_n;

@@ -73,7 +73,8 @@ struct DevPlan {
   int xcd_remap;              // 1: spread logical CTA ids so each XCD owns a contiguous range
   int raster_tail;            // tile rows in the last raster group (tiles_m % raster, or raster)
   int halves;                 // 1: REDUCE plan whose every Stream-K tile is cut into two equal CTA segments
-  FastDiv by_ipt, by_tiles_n, by_width, by_raster, by_tail, by_full1, by_full;
+  int perm_s, perm_g;         // perm_s > 1: Stream-K tile v stands at position (v % perm_s) * perm_g + v / perm_s
+  FastDiv by_ipt, by_tiles_n, by_width, by_raster, by_tail, by_full1, by_full, by_perm;
 };
 
 // Words of the workspace's status block: WS_STATUS a timed-out fix-up wait (0 or SK_ERR_TIMEOUT),
@@ -101,6 +102,10 @@ __device__ __forceinline__ void sk_range(const DevPlan &p, int pid, int &start, 
 }
 
 __device__ __forceinline__ void tile_coords(const DevPlan &p, int tile, int &pm, int &pn) {
+  if (p.perm_s > 1 && tile < p.sk_tiles) {  // interleaved order of the Stream-K tiles (sk_plan.interleave)
+    const int q = p.by_perm.div(tile);
+    tile = (tile - q * p.perm_s) * p.perm_g + q;
+  }
   if (p.tiles_m == 1) {
     pm = 0;
     pn = tile;

@@ -26,7 +26,7 @@ class SkPlan(ctypes.Structure):
         "bm", "bn", "bk", "grid", "schedule", "fixup", "raster", "dtype", "layout",
         "num_block_m", "num_block_n", "iters_per_tile", "total_tiles", "streamk_tiles",
         "blocking_tiles", "streamk_iters", "streamk_full_tiles", "streamk_partial_tiles",
-        "dp_waves", "kernel_id", "threads", "lds_bytes", "spin_limit")] + [
+        "dp_waves", "kernel_id", "threads", "lds_bytes", "spin_limit", "interleave")] + [
         ("workspace_bytes", ctypes.c_int64), ("M", ctypes.c_int64), ("N", ctypes.c_int64),
         ("K", ctypes.c_int64)]
 

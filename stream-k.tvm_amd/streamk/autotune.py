@@ -92,6 +92,9 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
                 grids = (None,) if bm * bn >= 256 * 256 else (None, cus)
                 for sched, fixup, grid in itertools.product(("sk2", "sk1", "basic"), ("reduce", "atomic"), grids):
                     out.append(dict(base, schedule=sched, fixup=fixup, **({"grid": grid} if grid else {})))
+                # the interleaved order of the Stream-K tiles (CTAs at the same K offset on neighbouring tiles)
+                if raster == 8 and bm * bn >= 128 * 128:
+                    out.extend(dict(base, schedule=sched, fixup="reduce", interleave=1) for sched in ("sk2", "basic"))
                 # fixed split-K, the fallback when there are fewer tiles than CUs
                 if -(-M // bm) * -(-N // bn) < cus:
                     out.extend(dict(base, schedule="splitk", fixup=fixup) for fixup in ("reduce", "atomic"))
@@ -101,6 +104,8 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
             out.append(dict(base, schedule="dp"))
             for sched, fixup in itertools.product(("sk2", "sk1", "basic"), ("reduce", "atomic")):
                 out.append(dict(base, schedule=sched, fixup=fixup))
+            if raster == 8:
+                out.extend(dict(base, schedule=sched, fixup="reduce", interleave=1) for sched in ("sk2", "basic"))
             if -(-M // bm) * -(-N // bn) < cus:
                 out.extend(dict(base, schedule="splitk", fixup=fixup) for fixup in ("reduce", "atomic"))
     return out
@@ -217,6 +222,8 @@ def autotune(M, N, K, dtype="float16", layout="nt", *, configs=None, warmup=5, r
             p = _plan.make_plan(M, N, K, dtype, layout, cfg)
             if cfg.get("schedule", "dp") != "dp" and p.streamk_tiles == 0:
                 continue  # the grid leaves no tile to split: this candidate is the data-parallel one under another name
+            if cfg.get("interleave") and p.interleave <= 1:
+                continue  # every CTA is at its own K offset, or all at the same one: the order changes nothing
             run(p)
             torch.cuda.synchronize()
             ops.workspace_status()

@@ -24,7 +24,7 @@ def num_cus():
 
 def make_config(config=None, **kw):
     """dict / kwargs -> SkConfig.  Keys: bm, bn, bk, grid, schedule ('auto'|'dp'|'sk2'|'sk1'|
-    'basic'|'splitk'), split, fixup ('auto'|'atomic'|'reduce'|'atomic_c'), raster, spin_limit, variant."""
+    'basic'|'splitk'), split, fixup ('auto'|'atomic'|'reduce'|'atomic_c'), raster, spin_limit, variant, interleave."""
     d = dict(config or {})
     d.update(kw)
     c = SkConfig()
@@ -40,6 +40,9 @@ def make_config(config=None, **kw):
             continue
         if k == "split":  # factor of schedule 'splitk'; 0 = choose
             c.reserved[1] = int(v)
+            continue
+        if k == "interleave":  # 1: interleaved order of the Stream-K tiles (sk_plan.interleave)
+            c.reserved[2] = int(v)
             continue
         if k not in ("bm", "bn", "bk", "grid", "schedule", "fixup", "raster", "spin_limit"):
             raise KeyError(f"unknown Stream-K config key {k!r}")

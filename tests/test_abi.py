@@ -135,6 +135,39 @@ def test_raster_is_a_permutation(sk):
     assert sk.tile_coords(plan, 8) == (0, 1)
 
 
+def test_interleaved_streamk_tile_order(sk):
+    """interleave=1: with g = gcd(streamk_tiles, grid) and S = streamk_tiles / g, the CTAs pid, pid + grid/g, ...
+    start S tiles apart at the same K offset; the interleaved order puts the tiles they work on next to each other.
+    It permutes the Stream-K tiles among themselves and leaves the data-parallel ones alone."""
+    base = dict(bm=256, bn=256, bk=64, raster=4, schedule="basic", fixup="reduce")
+    plain = sk.make_plan(3000, 5120, 12288, "float16", "nt", cus=256, **base)
+    plan = sk.make_plan(3000, 5120, 12288, "float16", "nt", cus=256, interleave=1, **base)
+    assert (plan.grid, plan.streamk_tiles, plan.streamk_full_tiles, plan.streamk_partial_tiles) == (256, 240, 180, 0)
+    assert plain.interleave == 0 and plan.interleave == 15        # g = gcd(240, 256) = 16, S = 15
+    for v in range(plan.streamk_tiles):
+        assert sk.tile_coords(plan, v) == sk.tile_coords(plain, (v % 15) * 16 + v // 15)
+    assert len({sk.tile_coords(plan, v) for v in range(plan.total_tiles)}) == plan.total_tiles
+    # the CTAs 16 apart are at the same offset of their tiles, and their tiles form one 4 x 4 block of the tile grid
+    for pid in range(16):
+        starts = [sk.cta_range(plan, pid + 16 * j)[0] for j in range(16)]
+        assert len({s % plan.iters_per_tile for s in starts}) == 1
+        tiles = [sk.tile_coords(plan, s // plan.iters_per_tile) for s in starts]
+        assert max(m for m, _ in tiles) - min(m for m, _ in tiles) == 3 and max(n for _, n in tiles) - min(n for _, n in tiles) == 3
+    # a hybrid schedule: only the Stream-K tiles move
+    hy = sk.make_plan(8192, 8192 + 1280, 4096, "float16", "nt", cus=256, bm=256, bn=256, bk=64, raster=8, schedule="sk1",
+                      fixup="reduce", interleave=1)
+    hy0 = sk.make_plan(8192, 8192 + 1280, 4096, "float16", "nt", cus=256, bm=256, bn=256, bk=64, raster=8, schedule="sk1",
+                       fixup="reduce")
+    assert 0 < hy.streamk_tiles < hy.total_tiles and hy.interleave > 1
+    assert {sk.tile_coords(hy, v) for v in range(hy.streamk_tiles)} == {sk.tile_coords(hy0, v) for v in range(hy.streamk_tiles)}
+    assert all(sk.tile_coords(hy, v) == sk.tile_coords(hy0, v) for v in range(hy.streamk_tiles, hy.total_tiles))
+    # nothing to interleave: every tile cut in two equal halves (all CTAs at offset 0 or ipt/2), data-parallel plans
+    assert sk.make_plan(1024, 8192, 8192, "float16", "nt", cus=256, interleave=1, **base).interleave == 0
+    assert sk.make_plan(8192, 8192, 8192, "float16", "nt", cus=256, bm=256, bn=256, schedule="dp", interleave=1).interleave == 0
+    with pytest.raises(sk.StreamKError):
+        sk.make_plan(3000, 5120, 12288, "float16", "nt", cus=256, interleave=2, **base)
+
+
 def test_error_codes(sk):
     L = sk.lib()
     with pytest.raises(sk.StreamKError) as e:

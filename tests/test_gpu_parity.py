@@ -100,6 +100,55 @@ def test_cfg2_streamk_both_fixups(sk, oracle, cfg, fixup):
     assert _rel(oracle, C, ref) <= 1e-3 <= TOL
 
 
+def test_interleaved_streamk_tile_order(sk, oracle):
+    """The interleaved order of the Stream-K tiles only changes which tile of C a tile id stands for: every
+    kernel family and fix-up gives the product within the usual bound on ragged shapes; with exact (integer) data the
+    result equals that of the plain order bit for bit."""
+    import torch
+    rng = np.random.default_rng(31)
+    ran = 0
+    for (M, N, K, grid) in [(1100, 1400, 1024, 40), (3000, 1300, 512, 56), (640, 2000, 2048, 48)]:
+        A = (rng.random((M, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+        B = (rng.random((N, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+        Ai, Bi = rng.integers(-1, 2, (M, K)).astype(np.float16), rng.integers(-1, 2, (N, K)).astype(np.float16)
+        ref = oracle.matmul_fp32(A, B, trans_b=True)
+        dA, dB, dAi, dBi = _t(A), _t(B), _t(Ai), _t(Bi)
+        for tile in (dict(bm=256, bn=256, bk=64, variant=8), dict(bm=256, bn=256, bk=64, variant=5), dict(bm=128, bn=128, bk=64, variant=5),
+                     dict(bm=128, bn=256, bk=32, variant=6), dict(bm=128, bn=128, bk=64, variant=2)):
+            for sch in (dict(schedule="basic", fixup="reduce"), dict(schedule="basic", fixup="atomic"),
+                        dict(schedule="sk2", fixup="reduce"), dict(schedule="basic", fixup="atomic_c")):
+                for raster in (1, 4):
+                    cfg = dict(tile, grid=grid, raster=raster, **sch)
+                    try:
+                        plan = sk.make_plan(M, N, K, "float16", "nt", dict(cfg, interleave=1))
+                        plain = sk.make_plan(M, N, K, "float16", "nt", cfg)
+                    except sk.StreamKError:
+                        continue
+                    if plan.interleave <= 1:
+                        continue
+                    assert plan.streamk_tiles % plan.interleave == 0
+                    C = sk.streamk_fp16(dA, dB, plan=plan)
+                    assert _rel(oracle, C, ref) <= (1e-2 if sch["fixup"] == "atomic_c" else 1e-3) <= TOL, (M, N, K, cfg)
+                    assert torch.equal(sk.streamk_fp16(dAi, dBi, plan=plan), sk.streamk_fp16(dAi, dBi, plan=plain)), (M, N, K, cfg)
+                    ran += 1
+    assert ran >= 40, ran
+    # one-byte operands (assembly-loop and eight-wave kernels) and the small-M kernels share the tile mapping
+    M, N, K = 1100, 1400, 1024
+    Ai8, Bi8 = rng.integers(-8, 9, (M, K)).astype(np.int8), rng.integers(-8, 9, (N, K)).astype(np.int8)
+    exact = Ai8.astype(np.int32) @ Bi8.astype(np.int32).T
+    for bm, grid in ((256, 40), (128, 44)):   # 30 and 99 tiles
+        plan = sk.make_plan(M, N, K, "int8", "nt", dict(bm=bm, bn=bm, grid=grid, schedule="basic", fixup="reduce", raster=4, interleave=1))
+        assert plan.interleave > 1
+        assert np.array_equal(sk.streamk_int8(_t(Ai8), _t(Bi8), plan=plan).cpu().numpy(), exact)
+    M, N, K = 16, 2000, 4096
+    A = (rng.random((M, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+    B = (rng.random((N, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+    plan = sk.make_plan(M, N, K, "float16", "nt", dict(bm=16, bn=64, bk=256, grid=24, schedule="basic", fixup="reduce", interleave=1))
+    assert plan.interleave > 1
+    assert _rel(oracle, sk.streamk_fp16(_t(A), _t(B), plan=plan), oracle.matmul_fp32(A, B, trans_b=True)) <= 1e-3
+    sk.workspace_status()
+
+
 def test_reference_fixup_packed_atomics_into_c(sk, oracle):
     """The reference's own fix-up (streamk_fp16.py:248-255): every segment of a split tile rounds its partial to
     C's type and adds it into C with packed 16-bit atomics, no workspace, C zero-filled by the library (handed
