@@ -170,6 +170,132 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
   return best;
 }
 
+// ---- which tile kernel and which split of K, when the caller leaves both open (M > 64) ----
+// A cost model with four constants per kernel family, fitted to 80 shapes x 5 families x splits 1, 2, 4 timed on
+// an MI355X (mean |log error| 5-10 %):
+//     time = rounds * (n * tau * clock + o) + phi * (split - 1)
+//   n       K-iterations per CTA (iterations per tile / split)
+//   clock   1 + 0.4 * (busy CUs / CUs)^2: the part is power-limited, busy CUs slow each other down
+//   rounds  CTAs the busiest CU runs one after another; a family whose CTAs share a CU (occ > 1) is charged
+//           1 + (rounds - 1) * gamma for them
+//   o       prologue and epilogue of a CTA, phi the fix-up of a split tile (256 x 256: only the split in two
+//           halves, which both CTAs finish in parallel; four ways the owner adds three 256 KB partials alone)
+// Choosing by it is within 5 % of the fastest of the candidates on average (worst case 23 %) on those shapes, where
+// the earlier rule (largest tile that fills the device, Stream-K for what is left) was 49 % behind on average.
+static int gcd_int(int a, int b) {
+  while (b) {
+    const int r = a % b;
+    a = b;
+    b = r;
+  }
+  return a;
+}
+
+// The automatic schedule of a tile kernel with more tiles than CTAs.  Returns the schedule and, in *sk_tiles, how
+// many tiles it splits.  Data-parallel when the last wave of tiles is at least 90 % full; else Stream-K over the
+// remainder tiles (with two or more full waves beside them) or over the remainder plus one wave
+// (streamk_fp32.py:37-43) -- but only where every CTA range starts at the beginning or in the middle of a tile
+// (grid / gcd(Stream-K tiles, grid) <= 2).  The tile kernels live on the L2 reuse of CTAs that walk K in lock-step
+// and their partial tiles are large: such a schedule gains 3-14 % over data-parallel where it applies; with 4 or 8
+// distinct offsets it measured between 8 % faster and 40 % slower, with ranges that start anywhere, or a handful
+// of remainder tiles cut into dozens of partials that one CTA adds up, 1.2x to 8x slower.
+static int auto_tile_schedule(int64_t total, int grid, int *sk_tiles) {
+  *sk_tiles = 0;
+  const int64_t waves = (total + grid - 1) / grid;
+  if (total * 10 >= waves * grid * 9) return SK_SCHED_DP;
+  const int sched = total >= 2 * (int64_t)grid ? SK_SCHED_SK_ONE_TILE : SK_SCHED_SK_TWO_TILE;
+  int skt = (int)(total % grid);
+  if (sched == SK_SCHED_SK_TWO_TILE && total - skt > grid) skt += grid;
+  if (skt == 0 || grid / gcd_int(skt, grid) > 2) return SK_SCHED_DP;
+  *sk_tiles = skt;
+  return sched;
+}
+
+struct TileFamily {
+  int bm, bn, bk, variant, occ, max_split;  // variant -1: the preferred variant of the tile
+  float tau, gamma, o, phi;
+};
+static const TileFamily kFamilies16[] = {
+    {256, 256, 64, 7, 1, 2, 0.999f, 0.20f, 4.5f, 20.0f},  // four waves, K loop in assembly (K % 64 == 0)
+    {256, 256, 64, 4, 1, 2, 1.080f, 0.20f, 4.5f, 20.0f},  // eight waves, for the other K
+    {128, 128, 64, 4, 2, 4, 0.497f, 0.47f, 4.9f, 5.1f},
+    {64, 128, 32, 5, 3, 4, 0.154f, 0.89f, 3.5f, 3.2f},
+    {128, 256, 64, 4, 1, 4, 0.689f, 1.00f, 6.0f, 5.9f},
+    {256, 128, 64, 4, 1, 4, 0.685f, 0.20f, 5.3f, 5.8f},
+};
+// one-byte operands (BK = 128), fitted the same way to 36 shapes each
+static const TileFamily kFamiliesF8[] = {
+    {256, 256, 128, -1, 1, 2, 1.007f, 1.00f, 3.5f, 19.9f},
+    {128, 128, 128, -1, 2, 2, 0.435f, 0.52f, 6.3f, 6.6f},
+    {128, 256, 128, -1, 1, 2, 0.580f, 0.20f, 9.3f, 6.7f},
+    {256, 128, 128, -1, 1, 2, 0.608f, 1.00f, 7.2f, 7.8f},
+};
+static const TileFamily kFamiliesI8[] = {
+    {256, 256, 128, -1, 1, 2, 1.121f, 0.20f, 2.8f, 20.2f},
+    {128, 128, 128, -1, 2, 2, 0.531f, 0.52f, 2.3f, 6.4f},
+    {128, 256, 128, -1, 1, 2, 0.674f, 0.20f, 6.5f, 6.5f},
+    {256, 128, 128, -1, 1, 2, 0.700f, 1.00f, 4.9f, 6.5f},
+};
+
+static const KernelInfo *model_pick(int64_t M, int64_t N, int64_t K, int dtype, int layout, int num_cus, int *split,
+                                    int *sched) {
+  const TileFamily *fams = kFamilies16;
+  int nfams = (int)(sizeof(kFamilies16) / sizeof(kFamilies16[0]));
+  if (dtype == SK_F8E4M3 || dtype == SK_F8E5M2) {
+    fams = kFamiliesF8;
+    nfams = (int)(sizeof(kFamiliesF8) / sizeof(kFamiliesF8[0]));
+  } else if (dtype == SK_I8) {
+    fams = kFamiliesI8;
+    nfams = (int)(sizeof(kFamiliesI8) / sizeof(kFamiliesI8[0]));
+  }
+  const KernelInfo *best = nullptr;
+  double best_time = 0;
+  bool have_asm = false;
+  for (int fi = 0; fi < nfams; ++fi) {
+    const TileFamily &f = fams[fi];
+    sk_config want;
+    memset(&want, 0, sizeof(want));
+    want.bm = f.bm; want.bn = f.bn; want.bk = f.bk;
+    want.reserved[0] = f.variant + 1;
+    const KernelInfo *k = pick_kernel(M, N, K, dtype, layout, &want, num_cus);
+    if (!k || k->family != FAMILY_TILE || K % k->k_align != 0) continue;
+    if (f.variant == 7) have_asm = true;
+    if (f.variant == 4 && f.bm == 256 && f.bn == 256 && have_asm) continue;  // the assembly kernel applies
+    const int64_t tiles = cdiv(M, f.bm) * cdiv(N, f.bn);
+    const int64_t ipt = cdiv(K, f.bk);
+    for (int s = 1; s <= f.max_split; s *= 2) {
+      if (ipt % s != 0 || (s > 1 && ipt / s < 8)) continue;
+      const int64_t ctas = tiles * s;
+      if (s > 1 && ctas > (int64_t)num_cus * k->ctas_per_cu) continue;  // the CTAs of a split tile wait for each other
+      const double busy = ctas < num_cus ? (double)ctas / num_cus : 1.0;
+      const double clock = 1.0 + 0.4 * busy * busy;
+      const int64_t rounds = ctas > num_cus ? cdiv(ctas, num_cus) : 1;
+      const double eff = f.occ == 1 ? (double)rounds : 1.0 + (rounds - 1) * f.gamma;
+      const double time = eff * ((double)(ipt / s) * f.tau * clock + f.o) + (s > 1 ? f.phi * (s - 1) : 0.0);
+      if (!best || time < best_time) {
+        best = k;
+        best_time = time;
+        *split = s;
+        *sched = s > 1 ? SK_SCHED_SPLIT_K : SK_SCHED_DP;
+      }
+    }
+    // more tiles than CUs on a one-CTA-per-CU kernel, and a Stream-K schedule that the automatic rule admits: the
+    // iterations spread evenly over the CUs, plus one exchange of partial tiles (the rule is applied again below,
+    // to the same effect, when the plan is made)
+    int skt = 0;
+    if (f.occ == 1 && tiles > num_cus && auto_tile_schedule(tiles, num_cus, &skt) != SK_SCHED_DP) {
+      const double time = (double)tiles * ipt / num_cus * f.tau * 1.4 + f.o * (double)cdiv(tiles, num_cus) + 0.5 * f.phi;
+      if (!best || time < best_time) {
+        best = k;
+        best_time = time;
+        *split = 1;
+        *sched = SK_SCHED_AUTO;
+      }
+    }
+  }
+  return best;
+}
+
 }  // namespace sk
 
 using namespace sk;
@@ -196,6 +322,22 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
   if ((dtype == SK_F8E4M3 || dtype == SK_F8E5M2 || dtype == SK_I8) && layout != SK_LAYOUT_NT) return SK_ERR_CONFIG;
   if (layout != SK_LAYOUT_NT && layout != SK_LAYOUT_NN) return SK_ERR_CONFIG;
   if (num_cus <= 0) return SK_ERR_DEVICE;
+  // tile, variant, schedule and grid all left open for a 16-bit or one-byte problem with more rows than the
+  // weight-streaming kernels take: the cost model chooses kernel and split
+  sk_config modelled;
+  if ((dtype == SK_F16 || dtype == SK_BF16 || dtype == SK_F8E4M3 || dtype == SK_F8E5M2 || dtype == SK_I8) && M > 64 &&
+      (!cfg || (cfg->bm == 0 && cfg->bn == 0 && cfg->bk == 0 && cfg->reserved[0] == 0 &&
+                cfg->schedule == SK_SCHED_AUTO && cfg->grid == 0))) {
+    int split = 1, model_sched = SK_SCHED_AUTO;
+    if (const KernelInfo *mk = model_pick(M, N, K, dtype, layout, num_cus, &split, &model_sched)) {
+      if (cfg) modelled = *cfg; else memset(&modelled, 0, sizeof(modelled));
+      modelled.bm = mk->bm; modelled.bn = mk->bn; modelled.bk = mk->bk;
+      modelled.reserved[0] = mk->variant + 1;
+      modelled.schedule = model_sched;
+      if (split > 1) modelled.reserved[1] = split;
+      cfg = &modelled;
+    }
+  }
   const KernelInfo *k = pick_kernel(M, N, K, dtype, layout, cfg, num_cus);
   if (!k) return SK_ERR_CONFIG;
   if (K % k->k_align != 0) return SK_ERR_ALIGN;
@@ -254,6 +396,22 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
     const int64_t waves = (total64 + grid - 1) / grid;
     if (total64 * 10 >= waves * grid * 9) sched = SK_SCHED_DP;
     else sched = total64 >= 2 * (int64_t)grid ? SK_SCHED_SK_ONE_TILE : SK_SCHED_SK_TWO_TILE;
+    if (k->family == FAMILY_TILE && sched != SK_SCHED_DP) {
+      // Fewer tiles than CUs: the idle CUs are put to work by an aligned split (two halves of a 256 x 256 tile, up
+      // to four parts of a smaller one), never by CTA ranges that start anywhere.  More tiles than CTAs: see
+      // auto_tile_schedule.
+      if (total64 < num_cus && !(cfg && cfg->grid > 0)) {
+        const int ipt = out->iters_per_tile, max_split = (int64_t)k->bm * k->bn >= 256 * 256 ? 2 : 4;
+        int split = 1;
+        for (int s = 2; s <= max_split && total64 * s <= max_grid; s *= 2)
+          if (ipt % s == 0 && ipt / s >= 8) split = s;
+        sched = split > 1 ? SK_SCHED_SPLIT_K : SK_SCHED_DP;
+        grid = split > 1 ? (int)(total64 * split) : grid;
+      } else {
+        int skt;
+        sched = auto_tile_schedule(total64, grid, &skt);
+      }
+    }
   }
   // a data-parallel-only launch never has more CTAs than tiles (idle CTAs would also skew the
   // CTA -> XCD mapping: the low logical ids sit on the first XCDs)

@@ -135,6 +135,45 @@ def test_raster_is_a_permutation(sk):
     assert sk.tile_coords(plan, 8) == (0, 1)
 
 
+def test_untuned_plans_keep_cta_ranges_aligned(sk):
+    """With tile, schedule and grid left to the planner, a tile kernel never gets CTA ranges that start anywhere in
+    their tiles: the plan is data-parallel, a fixed split of K in two or four, or a Stream-K schedule whose ranges
+    start at the beginning or in the middle of a tile; and a Stream-K tile never has more than four contributors."""
+    import math
+    SPLITK, DP = sk._lib.SCHEDULES["splitk"], sk._lib.SCHEDULES["dp"]
+    seen = set()
+    for dtype, layout in (("float16", "nt"), ("float16", "nn"), ("bfloat16", "nt"), ("float8_e4m3", "nt"), ("int8", "nt"), ("q4", "nt")):
+        for (N, K) in ((4096, 4096), (8192, 8192), (11008, 4096), (4096, 11008 if dtype != "q4" else 11008 + 128 - 11008 % 128), (5120, 5120), (6144, 4096)):
+            for M in (65, 128, 200, 384, 768, 1000, 1536, 2048, 2560, 3000, 3584, 4096, 8192):
+                if dtype in ("float8_e4m3", "int8") and K % 16:
+                    continue
+                plan = sk.make_plan(M, N, K, dtype, layout, cus=256, use_tuned=False)
+                name = sk.kernel_name(plan.kernel_id)
+                if not name.startswith("tile_"):
+                    continue
+                seen.add(plan.schedule)
+                if plan.streamk_tiles == 0:
+                    continue
+                per_cta = plan.streamk_iters / plan.grid
+                assert plan.streamk_partial_tiles == 0, (dtype, M, N, K, name, plan.as_dict())
+                if plan.schedule == SPLITK:
+                    assert plan.iters_per_tile / per_cta in (2, 4), (dtype, M, N, K, name)
+                else:
+                    assert plan.grid // math.gcd(plan.streamk_tiles, plan.grid) <= 2, (dtype, M, N, K, name)
+                    assert 2 * per_cta % plan.iters_per_tile == 0, (dtype, M, N, K, name)
+    assert SPLITK in seen and DP in seen and len(seen) >= 3   # some shape takes a Stream-K schedule too
+    # the assembly-loop kernel where it applies and the device is filled; a split in two halves below that
+    p = sk.make_plan(8192, 8192, 8192, "float16", "nt", cus=256, use_tuned=False)
+    assert (sk.kernel_name(p.kernel_id), p.schedule, p.grid) == ("tile_f16_nt_asm_256x256x64", DP, 256)
+    p = sk.make_plan(1024, 8192, 8192, "float16", "nt", cus=256, use_tuned=False)
+    assert (sk.kernel_name(p.kernel_id), p.schedule, p.grid) == ("tile_f16_nt_asm_256x256x64", SPLITK, 256)
+    # a caller's tile or schedule is not overridden
+    p = sk.make_plan(1024, 8192, 8192, "float16", "nt", cus=256, use_tuned=False, bm=128, bn=128)
+    assert (p.bm, p.bn) == (128, 128)
+    p = sk.make_plan(3000, 5120, 12288, "float16", "nt", cus=256, use_tuned=False, schedule="basic")
+    assert p.schedule == sk._lib.SCHEDULES["basic"] and p.streamk_tiles == p.total_tiles
+
+
 def test_interleaved_streamk_tile_order(sk):
     """interleave=1: with g = gcd(streamk_tiles, grid) and S = streamk_tiles / g, the CTAs pid, pid + grid/g, ...
     start S tiles apart at the same K offset; the interleaved order puts the tiles they work on next to each other.
