@@ -191,22 +191,29 @@ static int gcd_int(int a, int b) {
   return a;
 }
 
-// The automatic schedule of a tile kernel with more tiles than CTAs.  Returns the schedule and, in *sk_tiles, how
-// many tiles it splits.  Data-parallel when the last wave of tiles is at least 90 % full; else Stream-K over the
-// remainder tiles (with two or more full waves beside them) or over the remainder plus one wave
-// (streamk_fp32.py:37-43) -- but only where every CTA range starts at the beginning or in the middle of a tile
-// (grid / gcd(Stream-K tiles, grid) <= 2).  The tile kernels live on the L2 reuse of CTAs that walk K in lock-step
-// and their partial tiles are large: such a schedule gains 3-14 % over data-parallel where it applies; with 4 or 8
-// distinct offsets it measured between 8 % faster and 40 % slower, with ranges that start anywhere, or a handful
-// of remainder tiles cut into dozens of partials that one CTA adds up, 1.2x to 8x slower.
-static int auto_tile_schedule(int64_t total, int grid, int *sk_tiles) {
+// The automatic schedule of a tile kernel with more tiles than CTAs; *sk_tiles: how many tiles it splits.
+// Data-parallel when the last wave of tiles is at least 90 % full.  Else Stream-K over the remainder plus one
+// wave of tiles (`sk2`, streamk_fp32.py:37-43; with fewer than two waves that is every tile, `basic` -- the
+// reference's formula would split the remainder alone there, 2 tiles over 256 CTAs for 258 tiles, and the ordered
+// fix-up has one CTA add up 63 partial tiles per tile: 1243 us against 130 us) -- but only where the CTAs of an
+// XCD stay close to lock-step on K, which the L2 reuse of the tile kernels depends on: either every CTA range
+// starts at the beginning or in the middle of a tile (grid / gcd(Stream-K tiles, grid) <= 2), or consecutive
+// ranges start within ipt / 2 iterations of each other across the grid / 8 CTAs of an XCD.  Measured against
+// data-parallel: 3-22 % faster where admitted; 4 or 8 distinct offsets between 8 % faster and 40 % slower;
+// ranges that start anywhere up to 1.5x slower.
+static int auto_tile_schedule(int64_t total, int grid, int ipt, int *sk_tiles) {
   *sk_tiles = 0;
   const int64_t waves = (total + grid - 1) / grid;
-  if (total * 10 >= waves * grid * 9) return SK_SCHED_DP;
-  const int sched = total >= 2 * (int64_t)grid ? SK_SCHED_SK_ONE_TILE : SK_SCHED_SK_TWO_TILE;
-  int skt = (int)(total % grid);
-  if (sched == SK_SCHED_SK_TWO_TILE && total - skt > grid) skt += grid;
-  if (skt == 0 || grid / gcd_int(skt, grid) > 2) return SK_SCHED_DP;
+  if (total < grid || total * 10 >= waves * grid * 9 || ipt < 64) return SK_SCHED_DP;  // (short K: the fix-up outweighs the tail)
+  const int sched = total >= 2 * (int64_t)grid ? SK_SCHED_SK_TWO_TILE : SK_SCHED_SK_BASIC;
+  const int skt = (int)(total % grid) + grid;
+  const int64_t iters = (int64_t)skt * ipt;          // spread over `grid` CTAs
+  const double per_cta = (double)iters / grid;       // in [ipt, 2 ipt)
+  const double r = per_cta - ipt;                    // how far consecutive ranges drift apart, in iterations
+  const double d = r < ipt - r ? r : ipt - r;
+  const bool aligned = grid / gcd_int(skt, grid) <= 2;
+  const bool close = d * (grid / 8 > 0 ? grid / 8 : 1) <= ipt / 2.0;
+  if (!aligned && !close) return SK_SCHED_DP;
   *sk_tiles = skt;
   return sched;
 }
@@ -283,7 +290,7 @@ static const KernelInfo *model_pick(int64_t M, int64_t N, int64_t K, int dtype, 
     // iterations spread evenly over the CUs, plus one exchange of partial tiles (the rule is applied again below,
     // to the same effect, when the plan is made)
     int skt = 0;
-    if (f.occ == 1 && tiles > num_cus && auto_tile_schedule(tiles, num_cus, &skt) != SK_SCHED_DP) {
+    if (f.occ == 1 && tiles > num_cus && auto_tile_schedule(tiles, num_cus, (int)ipt, &skt) != SK_SCHED_DP) {
       const double time = (double)tiles * ipt / num_cus * f.tau * 1.4 + f.o * (double)cdiv(tiles, num_cus) + 0.5 * f.phi;
       if (!best || time < best_time) {
         best = k;
@@ -409,7 +416,7 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
         grid = split > 1 ? (int)(total64 * split) : grid;
       } else {
         int skt;
-        sched = auto_tile_schedule(total64, grid, &skt);
+        sched = auto_tile_schedule(total64, grid, out->iters_per_tile, &skt);
       }
     }
   }

@@ -141,7 +141,7 @@ def test_untuned_plans_keep_cta_ranges_aligned(sk):
     start at the beginning or in the middle of a tile; and a Stream-K tile never has more than four contributors."""
     import math
     SPLITK, DP = sk._lib.SCHEDULES["splitk"], sk._lib.SCHEDULES["dp"]
-    seen = set()
+    seen, streamk_seen = set(), set()
     for dtype, layout in (("float16", "nt"), ("float16", "nn"), ("bfloat16", "nt"), ("float8_e4m3", "nt"), ("int8", "nt"), ("q4", "nt")):
         for (N, K) in ((4096, 4096), (8192, 8192), (11008, 4096), (4096, 11008 if dtype != "q4" else 11008 + 128 - 11008 % 128), (5120, 5120), (6144, 4096)):
             for M in (65, 128, 200, 384, 768, 1000, 1536, 2048, 2560, 3000, 3584, 4096, 8192):
@@ -154,14 +154,22 @@ def test_untuned_plans_keep_cta_ranges_aligned(sk):
                 seen.add(plan.schedule)
                 if plan.streamk_tiles == 0:
                     continue
-                per_cta = plan.streamk_iters / plan.grid
-                assert plan.streamk_partial_tiles == 0, (dtype, M, N, K, name, plan.as_dict())
+                per_cta, ipt = plan.streamk_iters / plan.grid, plan.iters_per_tile
                 if plan.schedule == SPLITK:
-                    assert plan.iters_per_tile / per_cta in (2, 4), (dtype, M, N, K, name)
+                    assert ipt / per_cta in (2, 4) and plan.streamk_partial_tiles == 0, (dtype, M, N, K, name)
                 else:
-                    assert plan.grid // math.gcd(plan.streamk_tiles, plan.grid) <= 2, (dtype, M, N, K, name)
-                    assert 2 * per_cta % plan.iters_per_tile == 0, (dtype, M, N, K, name)
-    assert SPLITK in seen and DP in seen and len(seen) >= 3   # some shape takes a Stream-K schedule too
+                    # at least a tile's worth of iterations per CTA (a tile has at most three contributors), and
+                    # either ranges that start at the beginning or in the middle of a tile, or consecutive ranges
+                    # that stay within half a tile of each other across the CTAs of an XCD
+                    assert ipt <= per_cta < 2 * ipt, (dtype, M, N, K, name)
+                    drift = min(per_cta - ipt, 2 * ipt - per_cta)
+                    aligned = plan.grid // math.gcd(plan.streamk_tiles, plan.grid) <= 2
+                    assert aligned or drift * (plan.grid // 8) <= ipt / 2, (dtype, M, N, K, name, plan.as_dict())
+                    streamk_seen.add(aligned)
+    assert SPLITK in seen and DP in seen and streamk_seen == {True, False}   # both kinds of Stream-K plan occur
+    # 258 tiles on 256 CUs: every tile is split (64.5 iterations per CTA), not the two remainder tiles alone
+    p = sk.make_plan(1536, 11008, 4096, "float16", "nt", cus=256, use_tuned=False)
+    assert (p.bm, p.bn, p.schedule, p.streamk_tiles, p.grid) == (256, 256, sk._lib.SCHEDULES["basic"], 258, 256)
     # the assembly-loop kernel where it applies and the device is filled; a split in two halves below that
     p = sk.make_plan(8192, 8192, 8192, "float16", "nt", cus=256, use_tuned=False)
     assert (sk.kernel_name(p.kernel_id), p.schedule, p.grid) == ("tile_f16_nt_asm_256x256x64", DP, 256)
