@@ -272,7 +272,12 @@ struct KernelInfo {
   X(62, 128, 128, 2, 2, 32, false) \
   X(63, 64, 64, 2, 2, 32, false)   \
   X(64, 256, 256, 2, 4, 64, true)  \
-  X(65, 128, 128, 2, 2, 64, true)
+  X(65, 128, 128, 2, 2, 64, true)  \
+  X(50, 128, 256, 2, 4, 64, false) \
+  X(51, 256, 128, 4, 2, 64, false) \
+  X(52, 64, 128, 2, 2, 32, false)  \
+  X(53, 128, 256, 2, 4, 64, true)  \
+  X(54, 256, 128, 4, 2, 64, true)
 
 // fp8 (OCP e4m3) operands, fp16 C, NT layout; bk counts fp8 elements (variant 6):  X(id, BM, BN, WM, WN)
 #define SK_TILE_F8_KERNELS(X) \

@@ -941,7 +941,8 @@ def test_bf16_tile_kernels(sk, oracle):
     result must be exact, and the ordered reduce bitwise repeatable."""
     import torch
     torch.manual_seed(7)
-    tiles = {"nt": [(256, 256, 64), (128, 128, 64), (128, 128, 32), (64, 64, 32)], "nn": [(256, 256, 64), (128, 128, 64)]}
+    tiles = {"nt": [(256, 256, 64), (128, 128, 64), (128, 128, 32), (64, 64, 32), (128, 256, 64), (256, 128, 64), (64, 128, 32)],
+             "nn": [(256, 256, 64), (128, 128, 64), (128, 256, 64), (256, 128, 64)]}
     for (M, N, K) in [(200, 136, 328), (1000, 1096, 1032), (520, 264, 64), (64, 512, 2048)]:
         A = (torch.rand(M, K) * 2 - 1).bfloat16()
         Ai = torch.randint(-1, 2, (M, K)).bfloat16()
