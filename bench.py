@@ -28,6 +28,57 @@ PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E, published
 
 
+def planner_sweep(torch, streamk, time_graph):
+    """Untuned plans (sk_make_plan with no configuration and no tuned-cache lookup) against the vendor GEMM that
+    torch calls, M from 128 to 4096 over six (N, K) pairs, per operand type and layout.  Prints one JSON line:
+    per type the mean and the worst ratio time / vendor time (below 1: faster than the vendor) and the rows."""
+    schedules = {v: k for k, v in streamk._lib.SCHEDULES.items()}
+    out = {}
+    for dt, lay in (("float16", "nt"), ("float16", "nn"), ("bfloat16", "nt"), ("bfloat16", "nn"), ("float8_e4m3", "nt"),
+                    ("int8", "nt")):
+        rows = []
+        for (N, K) in ((4096, 4096), (8192, 8192), (4096, 11008), (11008, 4096), (5120, 5120), (6144, 4096)):
+            for M in (128, 256, 512, 768, 1024, 1536, 2048, 3000, 4096):
+                g = torch.Generator().manual_seed(0)
+                if dt == "int8":
+                    A = torch.randint(-8, 9, (M, K), generator=g, dtype=torch.int8).cuda()
+                    B = torch.randint(-8, 9, (N, K), generator=g, dtype=torch.int8).cuda()
+                    C = torch.empty(M, N, dtype=torch.int32, device="cuda")
+                    run = lambda p: streamk.streamk_int8(A, B, out=C, plan=p)  # noqa: E731
+                    ref = lambda: torch._int_mm(A, B.T, out=C)  # noqa: E731
+                elif dt == "float8_e4m3":
+                    if K % 16:
+                        continue
+                    A = (torch.rand(M, K, generator=g) * 2 - 1).cuda().to(torch.float8_e4m3fn)
+                    B = (torch.rand(N, K, generator=g) * 2 - 1).cuda().to(torch.float8_e4m3fn)
+                    C = torch.empty(M, N, dtype=torch.float16, device="cuda")
+                    one = torch.ones((), device="cuda")
+                    run = lambda p: streamk.streamk_fp8(A, B, out=C, plan=p)  # noqa: E731
+                    ref = lambda: torch._scaled_mm(A, B.T, one, one, out_dtype=torch.float16, out=C)  # noqa: E731
+                else:
+                    tdt = torch.float16 if dt == "float16" else torch.bfloat16
+                    A = (torch.rand(M, K, generator=g) * 2 - 1).to(tdt).cuda()
+                    B = (torch.rand(*((N, K) if lay == "nt" else (K, N)), generator=g) * 2 - 1).to(tdt).cuda()
+                    C = torch.empty(M, N, dtype=tdt, device="cuda")
+                    gemm = streamk.streamk_fp16 if dt == "float16" else streamk.streamk_bf16
+                    run = lambda p: gemm(A, B, layout=lay, out=C, plan=p)  # noqa: E731
+                    ref = lambda: torch.matmul(A, B.T if lay == "nt" else B, out=C)  # noqa: E731
+                p = streamk.make_plan(M, N, K, dt, lay, use_tuned=False)
+                try:
+                    t_ref = time_graph(ref, launches=10)
+                except Exception:   # no such GEMM in this torch build
+                    continue
+                t_sk = time_graph(lambda: run(p), launches=10)
+                rows.append({"M": M, "N": N, "K": K, "us": round(t_sk * 1e3, 1), "vendor_us": round(t_ref * 1e3, 1),
+                             "ratio": round(t_sk / t_ref, 3), "kernel": streamk.kernel_name(p.kernel_id),
+                             "schedule": schedules.get(p.schedule, p.schedule), "grid": p.grid})
+        if rows:
+            out[f"{dt}_{lay}"] = {"shapes": len(rows), "mean_ratio": round(sum(r["ratio"] for r in rows) / len(rows), 3),
+                                  "worst": sorted(rows, key=lambda r: -r["ratio"])[:3], "rows": rows}
+    streamk.workspace_status()
+    print(json.dumps({"planner_sweep": out}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -35,6 +86,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-extra", action="store_true", help="skip the sweep / Q4 section")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--planner-sweep", action="store_true",
+                    help="instead of the benchmark: time the planner's own choice (no tuned cache) against the vendor "
+                         "GEMM on a grid of shapes, per operand type and layout; one JSON line")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a 1 GiB device-to-device copy (reference point for rocprofv3 byte counters)")
     args = ap.parse_args()
@@ -79,6 +133,10 @@ def main():
         of seven timed groups of replays over 40 ms, on the side stream whose launches are quickest (see
         streamk.timing_stream: streams differ by 1.6 us per HBM-streaming launch on this part)"""
         return streamk.graph_ms(fn, launches=launches, **kw)
+
+    if args.planner_sweep:
+        planner_sweep(torch, streamk, time_graph)
+        return
 
     if args.copy_calibration:
         src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").fill_(1)
