@@ -100,6 +100,42 @@ def test_cfg2_streamk_both_fixups(sk, oracle, cfg, fixup):
     assert _rel(oracle, C, ref) <= 1e-3 <= TOL
 
 
+def test_untuned_plans_on_ragged_shapes(sk, oracle):
+    """The planner's own choice (no configuration, no tuned cache: cost model, aligned split, admitted Stream-K)
+    on shapes that exercise each of its branches, ragged edges included: fp16 NT / NN and bfloat16 against the
+    fp32 host product (1e-3 / 4e-3), int8 exactly."""
+    import torch
+    rng = np.random.default_rng(47)
+    kinds = set()
+    for (M, N, K) in [(65, 136, 328), (200, 1000, 1032), (384, 4096, 1024), (520, 2048, 4096), (768, 4096, 2048), (1000, 1096, 8192),
+                      (1536, 11008, 1024), (2100, 4000, 512), (3000, 5120, 1024), (3000, 8192, 4096), (4096, 4096, 64), (1536, 11008, 4096),
+                      (1024, 8192, 512), (512, 8192, 1024)]:
+        A = (rng.random((M, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+        B = (rng.random((N, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+        ref = oracle.matmul_fp32(A, B, trans_b=True)
+        for layout in ("nt", "nn"):
+            dB = _t(np.ascontiguousarray(B.T) if layout == "nn" else B)
+            plan = sk.make_plan(M, N, K, "float16", layout, use_tuned=False)
+            kinds.add((plan.schedule, plan.streamk_tiles > 0))
+            C = sk.streamk_fp16(_t(A), dB, layout=layout, plan=plan)
+            assert _rel(oracle, C, ref) <= 1e-3 <= TOL, (M, N, K, layout, sk.kernel_name(plan.kernel_id), plan.as_dict())
+            if M * N * K > 5e9:   # (the host reference of the large shapes is computed once, for fp16)
+                continue
+            pb = sk.make_plan(M, N, K, "bfloat16", layout, use_tuned=False)
+            Ab, Bb = torch.from_numpy(A).bfloat16(), torch.from_numpy(np.ascontiguousarray(B.T) if layout == "nn" else B).bfloat16()
+            refb = oracle.matmul_fp32(Ab.float().numpy(), Bb.float().numpy(), trans_b=layout == "nt")
+            Cb = sk.streamk_bf16(Ab.cuda(), Bb.cuda(), layout=layout, plan=pb)
+            assert _rel(oracle, Cb, refb) <= 4e-3 <= TOL, (M, N, K, layout, sk.kernel_name(pb.kernel_id))
+        if K % 16 == 0 and M * N * K <= 5e9:
+            Ai, Bi = rng.integers(-8, 9, (M, K)).astype(np.int8), rng.integers(-8, 9, (N, K)).astype(np.int8)
+            pi = sk.make_plan(M, N, K, "int8", "nt", use_tuned=False)
+            kinds.add((pi.schedule, pi.streamk_tiles > 0))
+            assert np.array_equal(sk.streamk_int8(_t(Ai), _t(Bi), plan=pi).cpu().numpy(), Ai.astype(np.int32) @ Bi.astype(np.int32).T), (M, N, K)
+    S = sk._lib.SCHEDULES
+    assert (S["dp"], False) in kinds and (S["splitk"], True) in kinds and ((S["basic"], True) in kinds or (S["sk2"], True) in kinds), kinds
+    sk.workspace_status()
+
+
 def test_interleaved_streamk_tile_order(sk, oracle):
     """The interleaved order of the Stream-K tiles only changes which tile of C a tile id stands for: every
     kernel family and fix-up gives the product within the usual bound on ragged shapes; with exact (integer) data the
