@@ -178,8 +178,8 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
 //   clock   1 + 0.4 * (busy CUs / CUs)^2: the part is power-limited, busy CUs slow each other down
 //   rounds  CTAs the busiest CU runs one after another; a family whose CTAs share a CU (occ > 1) is charged
 //           1 + (rounds - 1) * gamma for them
-//   o       prologue and epilogue of a CTA, phi the fix-up of a split tile (256 x 256: only the split in two
-//           halves, which both CTAs finish in parallel; four ways the owner adds three 256 KB partials alone)
+//   o       prologue and epilogue of a CTA, phi the fix-up per extra contributor of a split tile (two halves of a
+//           256 x 256 tile are finished by both CTAs in parallel: 5 us; four ways the owner adds three partials)
 // Choosing by it is within 5 % of the fastest of the candidates on average (worst case 23 %) on those shapes, where
 // the earlier rule (largest tile that fills the device, Stream-K for what is left) was 49 % behind on average.
 static int gcd_int(int a, int b) {
@@ -223,8 +223,8 @@ struct TileFamily {
   float tau, gamma, o, phi;
 };
 static const TileFamily kFamilies16[] = {
-    {256, 256, 64, 7, 1, 2, 0.999f, 0.20f, 4.5f, 20.0f},  // four waves, K loop in assembly (K % 64 == 0)
-    {256, 256, 64, 4, 1, 2, 1.080f, 0.20f, 4.5f, 20.0f},  // eight waves, for the other K
+    {256, 256, 64, 7, 1, 4, 0.987f, 0.20f, 9.3f, 5.2f},   // four waves, K loop in assembly (K % 64 == 0)
+    {256, 256, 64, 4, 1, 2, 1.080f, 0.20f, 9.3f, 10.0f},  // eight waves, for the other K
     {128, 128, 64, 4, 2, 4, 0.497f, 0.47f, 4.9f, 5.1f},
     {64, 128, 32, 5, 3, 4, 0.154f, 0.89f, 3.5f, 3.2f},
     {128, 256, 64, 4, 1, 4, 0.689f, 1.00f, 6.0f, 5.9f},
@@ -232,13 +232,13 @@ static const TileFamily kFamilies16[] = {
 };
 // one-byte operands (BK = 128), fitted the same way to 36 shapes each
 static const TileFamily kFamiliesF8[] = {
-    {256, 256, 128, -1, 1, 2, 1.007f, 1.00f, 3.5f, 19.9f},
+    {256, 256, 128, -1, 1, 4, 0.916f, 1.00f, 9.7f, 5.6f},
     {128, 128, 128, -1, 2, 2, 0.435f, 0.52f, 6.3f, 6.6f},
     {128, 256, 128, -1, 1, 2, 0.580f, 0.20f, 9.3f, 6.7f},
     {256, 128, 128, -1, 1, 2, 0.608f, 1.00f, 7.2f, 7.8f},
 };
 static const TileFamily kFamiliesI8[] = {
-    {256, 256, 128, -1, 1, 2, 1.121f, 0.20f, 2.8f, 20.2f},
+    {256, 256, 128, -1, 1, 4, 0.948f, 0.20f, 13.6f, 4.0f},
     {128, 128, 128, -1, 2, 2, 0.531f, 0.52f, 2.3f, 6.4f},
     {128, 256, 128, -1, 1, 2, 0.674f, 0.20f, 6.5f, 6.5f},
     {256, 128, 128, -1, 1, 2, 0.700f, 1.00f, 4.9f, 6.5f},
@@ -291,7 +291,7 @@ static const KernelInfo *model_pick(int64_t M, int64_t N, int64_t K, int dtype, 
     // to the same effect, when the plan is made)
     int skt = 0;
     if (f.occ == 1 && tiles > num_cus && auto_tile_schedule(tiles, num_cus, (int)ipt, &skt) != SK_SCHED_DP) {
-      const double time = (double)tiles * ipt / num_cus * f.tau * 1.4 + f.o * (double)cdiv(tiles, num_cus) + 0.5 * f.phi;
+      const double time = (double)tiles * ipt / num_cus * f.tau * 1.4 + f.o * (double)cdiv(tiles, num_cus) + 2.0 * f.phi;
       if (!best || time < best_time) {
         best = k;
         best_time = time;
@@ -404,11 +404,11 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
     if (total64 * 10 >= waves * grid * 9) sched = SK_SCHED_DP;
     else sched = total64 >= 2 * (int64_t)grid ? SK_SCHED_SK_ONE_TILE : SK_SCHED_SK_TWO_TILE;
     if (k->family == FAMILY_TILE && sched != SK_SCHED_DP) {
-      // Fewer tiles than CUs: the idle CUs are put to work by an aligned split (two halves of a 256 x 256 tile, up
-      // to four parts of a smaller one), never by CTA ranges that start anywhere.  More tiles than CTAs: see
+      // Fewer tiles than CUs: the idle CUs are put to work by an aligned split in two or four, never by CTA ranges
+      // that start anywhere.  More tiles than CTAs: see
       // auto_tile_schedule.
       if (total64 < num_cus && !(cfg && cfg->grid > 0)) {
-        const int ipt = out->iters_per_tile, max_split = (int64_t)k->bm * k->bn >= 256 * 256 ? 2 : 4;
+        const int ipt = out->iters_per_tile, max_split = 4;
         int split = 1;
         for (int s = 2; s <= max_split && total64 * s <= max_grid; s *= 2)
           if (ipt % s == 0 && ipt / s >= 8) split = s;

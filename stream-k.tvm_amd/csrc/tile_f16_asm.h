@@ -311,15 +311,27 @@ struct TileF16Asm {
   static __device__ __forceinline__ void add_groups(const float *src) {
     const BufferRsrc r = make_rsrc(src, TILE_ELEMS * 4);
     const uint32_t off = (uint32_t)pin_here((int)threadIdx.x) * 16;
-    static_for<V0, V1>([&](auto g) {
-      constexpr int v = decltype(g)::value;
-      const uint4v raw = ld_coherent16(r, off, (uint32_t)v * NT * 16);
-      if constexpr (I8) {
-        const intx4 sum = __builtin_bit_cast(intx4, agpr_read4<v * 4>()) + __builtin_bit_cast(intx4, raw);
-        agpr_write4<v * 4>(__builtin_bit_cast(floatx4, sum));
-      } else {
-        agpr_write4<v * 4>(agpr_read4<v * 4>() + __builtin_bit_cast(floatx4, raw));
-      }
+    // sixteen loads in flight per lane, then the sixteen sums: the accumulator moves are assembly statements, which
+    // the compiler keeps in order, so a loop of load-then-add leaves one load in flight and the exchange of a
+    // 256 KB partial tile waits out 64 memory round trips
+    constexpr int BATCH = 16;
+    static_assert((V1 - V0) % BATCH == 0, "whole batches");
+    static_for<0, (V1 - V0) / BATCH>([&](auto b) {
+      constexpr int base = V0 + decltype(b)::value * BATCH;
+      uint4v raw[BATCH];
+      static_for<0, BATCH>([&](auto i) {
+        constexpr int v = base + decltype(i)::value;
+        raw[decltype(i)::value] = ld_coherent16(r, off, (uint32_t)v * NT * 16);
+      });
+      static_for<0, BATCH>([&](auto i) {
+        constexpr int v = base + decltype(i)::value;
+        if constexpr (I8) {
+          const intx4 sum = __builtin_bit_cast(intx4, agpr_read4<v * 4>()) + __builtin_bit_cast(intx4, raw[decltype(i)::value]);
+          agpr_write4<v * 4>(__builtin_bit_cast(floatx4, sum));
+        } else {
+          agpr_write4<v * 4>(agpr_read4<v * 4>() + __builtin_bit_cast(floatx4, raw[decltype(i)::value]));
+        }
+      });
     });
   }
   static __device__ __forceinline__ void store_partial(const Acc &, float *dst) { store_groups<0, NV4>(dst); }
@@ -350,16 +362,20 @@ struct TileF16Asm {
   // reads the completed sum and leaves zeros behind
   static __device__ __forceinline__ void take_partial(Acc &, float *src) {
     src = pin_here(src) + threadIdx.x;
-    static_for<0, NV4>([&](auto g) {
-      constexpr int v = decltype(g)::value;
-      floatx4 x;
+    constexpr int BATCH = 8;  // (loads in flight per lane: see add_groups)
+    static_for<0, NV4 / BATCH>([&](auto b) {
+      constexpr int base = decltype(b)::value * BATCH;
+      floatx4 x[BATCH];
+      static_for<0, BATCH>([&](auto i) {
+        constexpr int v = base + decltype(i)::value;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        float *p = src + (size_t)(v * 4 + e) * NT;
-        x[e] = *p;
-        *p = 0.f;
-      }
-      agpr_write4<v * 4>(x);
+        for (int e = 0; e < 4; ++e) {
+          float *p = src + (size_t)(v * 4 + e) * NT;
+          x[decltype(i)::value][e] = *p;
+          *p = 0.f;
+        }
+      });
+      static_for<0, BATCH>([&](auto i) { agpr_write4<(base + decltype(i)::value) * 4>(x[decltype(i)::value]); });
     });
   }
 };
