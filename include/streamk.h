@@ -126,7 +126,7 @@ typedef struct sk_plan {
                                     work on next to each other in the tile order, so that with a grouped raster they
                                     share rows of A and columns of B while those are in the L2, as the tiles of a
                                     data-parallel wave do.  Those CTAs sit on one XCD when grid/g is a multiple of 8. */
-  int64_t workspace_bytes;       /* what sk_gemm_* needs for this plan */
+  int64_t workspace_bytes;       /* what sk_gemm_* needs for this plan (0: data-parallel, ATOMIC_C, or CTA ranges that are whole tiles) */
   int64_t M, N, K;
 } sk_plan;
 

@@ -469,7 +469,10 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
 
   // workspace: status block, fixed-size flag area, fp32 partial tiles
   int64_t ws = 0;
-  if (sk_tiles > 0 && fixup != SK_FIXUP_ATOMIC_C) {
+  // (CTA ranges that are whole tiles -- e.g. `basic` on a tile count that is a multiple of the grid, which only
+  // changes which tiles a CTA takes -- never reach the fix-up: no workspace)
+  const bool whole_tiles = out->streamk_partial_tiles == 0 && out->streamk_full_tiles % out->iters_per_tile == 0;
+  if (sk_tiles > 0 && fixup != SK_FIXUP_ATOMIC_C && !whole_tiles) {
     const int64_t nflags = fixup == SK_FIXUP_REDUCE ? grid : sk_tiles;
     if (nflags > WS_MAX_FLAGS) return SK_ERR_CONFIG;
     ws = WS_PART_OFF + nflags * (int64_t)k->partial_elems * 4;

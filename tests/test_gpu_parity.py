@@ -100,6 +100,31 @@ def test_cfg2_streamk_both_fixups(sk, oracle, cfg, fixup):
     assert _rel(oracle, C, ref) <= 1e-3 <= TOL
 
 
+def test_whole_tile_ranges_need_no_workspace(sk, oracle):
+    """A Stream-K schedule whose CTA ranges are whole tiles (`basic` on a tile count that is a multiple of the grid)
+    only changes which tiles a CTA takes: the plan asks for no workspace and the result equals the data-parallel
+    one bit for bit."""
+    import torch
+    rng = np.random.default_rng(53)
+    M, N, K = 2048, 1024, 512
+    A = (rng.random((M, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+    B = (rng.random((N, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+    for tile in (dict(bm=256, bn=256, bk=64, variant=8), dict(bm=128, bn=128, bk=64, variant=5)):
+        tiles = (M // tile["bm"]) * (N // tile["bn"])
+        for fixup in ("reduce", "atomic"):
+            plan = sk.make_plan(M, N, K, "float16", "nt", dict(tile, schedule="basic", fixup=fixup, grid=tiles // 4, raster=1))
+            assert plan.streamk_tiles == tiles and plan.workspace_bytes == 0
+            dp = sk.make_plan(M, N, K, "float16", "nt", dict(tile, schedule="dp"))
+            C = sk.streamk_fp16(_t(A), _t(B), plan=plan)
+            assert torch.equal(C, sk.streamk_fp16(_t(A), _t(B), plan=dp))
+            assert _rel(oracle, C, oracle.matmul_fp32(A, B, trans_b=True)) <= 1e-3
+    Ai, Bi = rng.integers(-8, 9, (M, K)).astype(np.int8), rng.integers(-8, 9, (N, K)).astype(np.int8)
+    plan = sk.make_plan(M, N, K, "int8", "nt", dict(bm=256, bn=256, schedule="basic", fixup="reduce", grid=8))
+    assert plan.workspace_bytes == 0
+    assert np.array_equal(sk.streamk_int8(_t(Ai), _t(Bi), plan=plan).cpu().numpy(), Ai.astype(np.int32) @ Bi.astype(np.int32).T)
+    sk.workspace_status()
+
+
 def test_untuned_plans_on_ragged_shapes(sk, oracle):
     """The planner's own choice (no configuration, no tuned cache: cost model, aligned split, admitted Stream-K)
     on shapes that exercise each of its branches, ragged edges included: fp16 NT / NN and bfloat16 against the
