@@ -64,7 +64,7 @@ def test_static_workspace_entry_point_matches_sk_gemm_f16():
     torch.cuda.synchronize()
     assert torch.equal(C, streamk.streamk_fp16(A, A, bm=128, bn=128, bk=64, schedule="dp"))
     # a plan that needs more than the static array holds is refused
-    big = streamk.make_plan(8192, 8192, 8192, "float16", "nt", dict(bm=256, bn=256, bk=64, schedule="basic", fixup="atomic"))
+    big = streamk.make_plan(8192, 8192, 8192, "float16", "nt", dict(bm=256, bn=256, bk=64, schedule="basic", fixup="atomic", grid=255))
     assert big.workspace_bytes > 64 * 1024 * 1024 + 262144 + 256
     assert L.sk_gemm_f16_static(A.data_ptr(), A.data_ptr(), C.data_ptr(), 8192, 8192, 8192, 8192, 8192, 8192,
                                 ctypes.byref(big), stream) == -5
