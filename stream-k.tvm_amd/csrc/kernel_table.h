@@ -284,21 +284,24 @@ struct KernelInfo {
   X(70, 256, 256, 2, 4)       \
   X(71, 128, 128, 2, 2)       \
   X(72, 128, 256, 2, 4)       \
-  X(73, 256, 128, 4, 2)
+  X(73, 256, 128, 4, 2)       \
+  X(75, 64, 128, 1, 4)
 
 // the same for OCP e5m2 operands (dtype SK_F8E5M2):  X(id, BM, BN, WM, WN)
 #define SK_TILE_F8E5M2_KERNELS(X) \
   X(90, 256, 256, 2, 4)           \
   X(91, 128, 128, 2, 2)           \
   X(92, 128, 256, 2, 4)           \
-  X(93, 256, 128, 4, 2)
+  X(93, 256, 128, 4, 2)           \
+  X(95, 64, 128, 1, 4)
 
 // int8 operands, int32 C, NT layout; bk counts int8 elements (variant 4: 16x16 accumulator blocks):  X(id, BM, BN, WM, WN)
 #define SK_TILE_I8_KERNELS(X) \
   X(80, 256, 256, 2, 4)       \
   X(81, 128, 128, 2, 2)       \
   X(82, 128, 256, 2, 4)       \
-  X(83, 256, 128, 4, 2)
+  X(83, 256, 128, 4, 2)       \
+  X(85, 64, 128, 2, 2)
 
 // 256 x 256 x 64 on four waves, K loop in assembly (variant 7), K a multiple of 64 (int8: 128 bytes per
 // iteration):  X(id, MODE, NN)  with MODE 0 fp16, 1 bfloat16, 2 int8, 3 fp8 e4m3, 4 fp8 e5m2; NN: B is [K,N]

@@ -230,18 +230,20 @@ static const TileFamily kFamilies16[] = {
     {128, 256, 64, 4, 1, 4, 0.689f, 1.00f, 6.0f, 5.9f},
     {256, 128, 64, 4, 1, 4, 0.685f, 0.20f, 5.3f, 5.8f},
 };
-// one-byte operands (BK = 128), fitted the same way to 36 shapes each
+// one-byte operands (BK = 128), fitted the same way to 36 shapes each (64 x 128: to 42 shapes with M <= 1024)
 static const TileFamily kFamiliesF8[] = {
     {256, 256, 128, -1, 1, 4, 0.916f, 1.00f, 9.7f, 5.6f},
     {128, 128, 128, -1, 2, 2, 0.435f, 0.52f, 6.3f, 6.6f},
     {128, 256, 128, -1, 1, 2, 0.580f, 0.20f, 9.3f, 6.7f},
     {256, 128, 128, -1, 1, 2, 0.608f, 1.00f, 7.2f, 7.8f},
+    {64, 128, 128, -1, 2, 2, 0.335f, 0.46f, 4.3f, 6.5f},
 };
 static const TileFamily kFamiliesI8[] = {
     {256, 256, 128, -1, 1, 4, 0.948f, 0.20f, 13.6f, 4.0f},
     {128, 128, 128, -1, 2, 2, 0.531f, 0.52f, 2.3f, 6.4f},
     {128, 256, 128, -1, 1, 2, 0.674f, 0.20f, 6.5f, 6.5f},
     {256, 128, 128, -1, 1, 2, 0.700f, 1.00f, 4.9f, 6.5f},
+    {64, 128, 128, -1, 2, 2, 0.392f, 0.39f, 3.3f, 4.0f},
 };
 
 static const KernelInfo *model_pick(int64_t M, int64_t N, int64_t K, int dtype, int layout, int num_cus, int *split,

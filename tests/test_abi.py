@@ -107,17 +107,21 @@ def test_fp8_plans(sk):
             assert sk.kernel_name(p.kernel_id) == f"skinny_{tag}_{name}"
         q = sk.make_plan(M, 4096, 4096, "int8", "nt", cus=256)
         assert (q.bm, q.bn, q.bk) == (bm, 64, 256) and sk.kernel_name(q.kernel_id) == f"skinny_i8_{name}"
-    for (M, N, K, bm) in [(8192, 8192, 8192, 256), (512, 512, 4096, 128), (65, 4096, 4096, 128)]:
-        p = sk.make_plan(M, N, K, "float8_e4m3", "nt", cus=256)
-        assert (p.bm, p.bn, p.bk) == (bm, bm, 128) and p.iters_per_tile == K // 128
+    for (M, N, K, bm, bn) in [(8192, 8192, 8192, 256, 256), (512, 512, 4096, 128, 128), (65, 4096, 4096, 64, 128), (300, 4096, 4096, 128, 256)]:
+        p = sk.make_plan(M, N, K, "float8_e4m3", "nt", cus=256, bm=bm, bn=bn)
+        assert (p.bm, p.bn, p.bk) == (bm, bn, 128) and p.iters_per_tile == K // 128
         # (256 x 256 with K a multiple of 128: the four-wave kernels whose K loop is assembly)
-        assert sk.kernel_name(p.kernel_id) == ("tile_f8e4m3_nt_asm_256x256x128" if bm == 256 else f"tile_f8e4m3_nt_dma_{bm}x{bm}x128")
-        r = sk.make_plan(M, N, K, "float8_e5m2", "nt", cus=256)
+        assert sk.kernel_name(p.kernel_id) == ("tile_f8e4m3_nt_asm_256x256x128" if bm == 256 else f"tile_f8e4m3_nt_dma_{bm}x{bn}x128")
+        r = sk.make_plan(M, N, K, "float8_e5m2", "nt", cus=256, bm=bm, bn=bn)
         assert (r.bm, r.bn, r.bk, r.grid) == (p.bm, p.bn, 128, p.grid)
-        assert sk.kernel_name(r.kernel_id) == ("tile_f8e5m2_nt_asm_256x256x128" if bm == 256 else f"tile_f8e5m2_nt_dma_{bm}x{bm}x128")
-        q = sk.make_plan(M, N, K, "int8", "nt", cus=256)
-        assert (q.bm, q.bn, q.bk, q.grid) == (p.bm, p.bn, 128, p.grid)
-        assert sk.kernel_name(q.kernel_id) == ("tile_i8_nt_asm_256x256x128" if bm == 256 else f"tile_i8_nt_dma16_{bm}x{bm}x128")
+        assert sk.kernel_name(r.kernel_id) == ("tile_f8e5m2_nt_asm_256x256x128" if bm == 256 else f"tile_f8e5m2_nt_dma_{bm}x{bn}x128")
+        q = sk.make_plan(M, N, K, "int8", "nt", cus=256, bm=bm, bn=bn)
+        assert (q.bm, q.bn, q.bk) == (p.bm, p.bn, 128)
+        assert sk.kernel_name(q.kernel_id) == ("tile_i8_nt_asm_256x256x128" if bm == 256 else f"tile_i8_nt_dma16_{bm}x{bn}x128")
+    # the planner's own choice: the assembly-loop kernel where 256 x 256 tiles fill the device, 64 x 128 tiles for few rows
+    for dtype, tag in (("float8_e4m3", "f8e4m3_nt_dma"), ("float8_e5m2", "f8e5m2_nt_dma"), ("int8", "i8_nt_dma16")):
+        assert sk.kernel_name(sk.make_plan(8192, 8192, 8192, dtype, "nt", cus=256, use_tuned=False).kernel_id).endswith("_nt_asm_256x256x128")
+        assert sk.kernel_name(sk.make_plan(65, 4096, 4096, dtype, "nt", cus=256, use_tuned=False).kernel_id) == f"tile_{tag}_64x128x128"
     with pytest.raises(sk.StreamKError):
         sk.make_plan(256, 256, 256, "int8", "nn", cus=256)
     with pytest.raises(sk.StreamKError):

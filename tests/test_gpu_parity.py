@@ -1103,7 +1103,7 @@ def test_fp8_tile_kernels(sk, oracle):
     import torch
     torch.manual_seed(11)
     f8 = torch.float8_e4m3fn
-    tiles = [(256, 256), (128, 128), (128, 256), (256, 128)]
+    tiles = [(256, 256), (128, 128), (128, 256), (256, 128), (64, 128)]
     for (M, N, K) in [(200, 136, 336), (1000, 1096, 1040), (520, 264, 128), (64, 512, 2048), (300, 300, 16)]:
         A, B = torch.randn(M, K).to(f8), torch.randn(N, K).to(f8)
         Ai, Bi = torch.randint(-1, 2, (M, K)).float().to(f8), torch.randint(-1, 2, (N, K)).float().to(f8)
@@ -1301,7 +1301,7 @@ def test_fp8_e5m2_tile_kernels(sk, oracle):
         Ai, Bi = torch.randint(-1, 2, (M, K)).float().to(f8), torch.randint(-1, 2, (N, K)).float().to(f8)
         ref = oracle.f8_gemm_ref(A.view(torch.uint8).numpy(), B.view(torch.uint8).numpy(), "e5m2")
         exact = oracle.f8_gemm_ref(Ai.view(torch.uint8).numpy(), Bi.view(torch.uint8).numpy(), "e5m2")
-        for (bm, bn) in [(256, 256), (128, 128), (128, 256), (256, 128)]:
+        for (bm, bn) in [(256, 256), (128, 128), (128, 256), (256, 128), (64, 128)]:
             for sch in (dict(schedule="dp"), dict(schedule="basic", fixup="reduce", grid=24), dict(schedule="sk2", fixup="atomic", grid=16)):
                 plan = sk.make_plan(M, N, K, "float8_e5m2", "nt", dict(bm=bm, bn=bn, **sch))
                 assert "e5m2" in sk.kernel_name(plan.kernel_id)
@@ -1329,7 +1329,7 @@ def test_int8_tile_kernels(sk, oracle):
     strided operands and an output whose rows are not 16-byte aligned."""
     import torch
     torch.manual_seed(12)
-    tiles = [(256, 256), (128, 128), (128, 256), (256, 128)]
+    tiles = [(256, 256), (128, 128), (128, 256), (256, 128), (64, 128)]
     for (M, N, K) in [(200, 136, 336), (1000, 1096, 1040), (520, 264, 128), (64, 512, 2048), (300, 300, 16)]:
         A = torch.randint(-128, 128, (M, K), dtype=torch.int8)
         B = torch.randint(-128, 128, (N, K), dtype=torch.int8)
