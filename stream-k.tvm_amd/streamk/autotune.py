@@ -98,8 +98,9 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
                 # fixed split-K, the fallback when there are fewer tiles than CUs
                 if -(-M // bm) * -(-N // bn) < cus:
                     out.extend(dict(base, schedule="splitk", fixup=fixup) for fixup in ("reduce", "atomic"))
+                    out.append(dict(base, schedule="splitk", split=2, fixup="reduce"))
     if dtype in ("float8_e4m3", "float8_e5m2", "int8"):
-        for (bm, bn), raster in itertools.product(((256, 256), (256, 128), (128, 256), (128, 128)), (1, 8)):
+        for (bm, bn), raster in itertools.product(((256, 256), (256, 128), (128, 256), (128, 128), (64, 128)), (1, 8)):
             base = dict(bm=bm, bn=bn, raster=raster)
             out.append(dict(base, schedule="dp"))
             for sched, fixup in itertools.product(("sk2", "sk1", "basic"), ("reduce", "atomic")):
@@ -108,6 +109,7 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
                 out.extend(dict(base, schedule=sched, fixup="reduce", interleave=1) for sched in ("sk2", "basic"))
             if -(-M // bm) * -(-N // bn) < cus:
                 out.extend(dict(base, schedule="splitk", fixup=fixup) for fixup in ("reduce", "atomic"))
+                out.append(dict(base, schedule="splitk", split=2, fixup="reduce"))
     return out
 
 
