@@ -58,11 +58,14 @@ typedef enum sk_schedule {
 
 /* How partial tiles of the Stream-K wave are combined. */
 typedef enum sk_fixup {
-  SK_FIXUP_AUTO = 0,
+  SK_FIXUP_AUTO = 0,       /* SK_FIXUP_REDUCE */
   SK_FIXUP_ATOMIC = 1,     /* fp32 atomicAdd of partial accumulators (streamk_fp32.py:127-134);
                               summation order varies run to run */
   SK_FIXUP_REDUCE = 2,     /* per-CTA fp32 partial + flag; the tile's first CTA adds the others in
-                              ascending CTA order: bitwise reproducible */
+                              ascending CTA order: bitwise reproducible.  One CTA adds a tile's partials one after
+                              the other, so a schedule that cuts a few tiles into dozens of segments (an explicit
+                              sk1 / sk2 over a handful of remainder tiles) is better served by SK_FIXUP_ATOMIC;
+                              the planner's own schedules keep to at most four contributors per tile */
   SK_FIXUP_ATOMIC_C = 3    /* the reference's own fix-up (streamk_fp16.py:248-255, atomic_addx2 on half2): every
                               segment of a split tile rounds its partial sums to C's 16-bit type and adds them
                               into C with packed 16-bit atomic adds; no workspace.  The library zero-fills C
