@@ -65,7 +65,8 @@ typedef enum sk_fixup {
                               ascending CTA order: bitwise reproducible.  One CTA adds a tile's partials one after
                               the other, so a schedule that cuts a few tiles into dozens of segments (an explicit
                               sk1 / sk2 over a handful of remainder tiles) is better served by SK_FIXUP_ATOMIC;
-                              the planner's own schedules keep to at most four contributors per tile */
+                              the planner's own schedules for the tile kernels keep to at most four contributors per
+                              tile (the small-M kernels' partials are a few KB) */
   SK_FIXUP_ATOMIC_C = 3    /* the reference's own fix-up (streamk_fp16.py:248-255, atomic_addx2 on half2): every
                               segment of a split tile rounds its partial sums to C's 16-bit type and adds them
                               into C with packed 16-bit atomic adds; no workspace.  The library zero-fills C
