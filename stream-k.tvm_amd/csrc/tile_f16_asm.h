@@ -249,18 +249,34 @@ struct TileF16Asm {
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
       const int row0 = pm * BM + wm * WTM + ROW_BEGIN + p * PATCH_ROWS, col0 = pn * BN + wn * WTN;
+      constexpr int NCH = PATCH_ROWS * CPRC / 64;  // 16-byte pieces per lane and pass
+      // eight LDS reads go out before the first of their stores: inside the edge tests each read would wait out
+      // its own LDS round trip
+      constexpr int BATCH = 8;
+      static_assert(NCH % BATCH == 0, "whole batches");
 #pragma unroll
-      for (int s = 0; s < PATCH_ROWS * CPRC / 64; ++s) {
-        const int idx = s * 64 + lane;
-        const int r = idx / CPRC, cc = idx % CPRC;
-        const int grow = row0 + r, gcol = col0 + cc * 8;
-        if (grow < a.M && gcol < a.N) {
-          const half_t *src = patch + r * LDC + cc * 8;
-          half_t *dst = a.C + (int64_t)grow * a.ldc + gcol;
-          if (vec_ok && gcol + 8 <= a.N) {
-            *reinterpret_cast<uint4v *>(dst) = *reinterpret_cast<const uint4v *>(src);
-          } else {
-            for (int e = 0; e < 8 && gcol + e < a.N; ++e) dst[e] = src[e];
+      for (int s0 = 0; s0 < NCH; s0 += BATCH) {
+        uint4v v[BATCH];
+#pragma unroll
+        for (int s = 0; s < BATCH; ++s) {
+          const int idx = (s0 + s) * 64 + lane;
+          v[s] = *reinterpret_cast<const uint4v *>(patch + (idx / CPRC) * LDC + (idx % CPRC) * 8);
+        }
+#pragma unroll
+        for (int s = 0; s < BATCH; ++s) {
+          const int idx = (s0 + s) * 64 + lane;
+          const int grow = row0 + idx / CPRC, gcol = col0 + (idx % CPRC) * 8;
+          if (grow < a.M && gcol < a.N) {
+            half_t *dst = a.C + (int64_t)grow * a.ldc + gcol;
+            if (vec_ok && gcol + 8 <= a.N) {
+              *reinterpret_cast<uint4v *>(dst) = v[s];
+            } else {
+              union { uint4v q; half_t h[8]; } u;
+              u.q = v[s];
+#pragma unroll
+              for (int e = 0; e < 8; ++e)
+                if (gcol + e < a.N) dst[e] = u.h[e];
+            }
           }
         }
       }
