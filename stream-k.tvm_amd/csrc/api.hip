@@ -152,7 +152,8 @@ int make_dev_plan(const sk_plan *plan, const KernelInfo *k, void *ws, size_t ws_
     return SK_ERR_CONFIG;
   if (plan->workspace_bytes > 0 && is_static) {
     char *base = static_cast<char *>(ws);
-    const int nflags = plan->fixup == SK_FIXUP_REDUCE ? plan->grid : plan->streamk_tiles;
+    // (REDUCE: one flag per CTA, and a second one for the two-round exchange of tiles cut into four)
+    const int nflags = plan->fixup == SK_FIXUP_REDUCE ? 2 * plan->grid : plan->streamk_tiles;
     const size_t units = (ws_bytes - (size_t)WS_PART_OFF) / 256;
     hipLaunchKernelGGL(prepare_static_kernel, dim3(1024), dim3(256), 0, stream, reinterpret_cast<int *>(base),
                        reinterpret_cast<int *>(base + 256), nflags, reinterpret_cast<uint4v *>(base + WS_PART_OFF),
@@ -193,8 +194,12 @@ int make_dev_plan(const sk_plan *plan, const KernelInfo *k, void *ws, size_t ws_
   const int raster = plan->raster > 0 ? plan->raster : 1;
   dp->raster_tail = plan->num_block_m % raster ? plan->num_block_m % raster : raster;
   // every Stream-K tile cut into exactly two equal CTA segments: both CTAs of a pair finish half a tile
-  dp->halves = (plan->fixup == SK_FIXUP_REDUCE && plan->streamk_tiles > 0 && plan->streamk_partial_tiles == 0 &&
-                2 * plan->streamk_full_tiles == plan->iters_per_tile) ? 1 : 0;
+  dp->halves = 0;
+  if (plan->fixup == SK_FIXUP_REDUCE && plan->streamk_tiles > 0 && plan->streamk_partial_tiles == 0) {
+    if (2 * plan->streamk_full_tiles == plan->iters_per_tile) dp->halves = 1;
+    // four equal segments: two rounds of the same exchange (the second round's flags follow the first `grid` ones)
+    if (4 * plan->streamk_full_tiles == plan->iters_per_tile && 2 * (int64_t)plan->grid <= WS_MAX_FLAGS) dp->halves = 2;
+  }
   dp->by_ipt = FastDiv::make(plan->iters_per_tile);
   dp->by_tiles_n = FastDiv::make(plan->num_block_n);
   dp->by_width = FastDiv::make((uint32_t)raster * plan->num_block_n);

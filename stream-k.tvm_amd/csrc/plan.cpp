@@ -173,13 +173,13 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
 // ---- which tile kernel and which split of K, when the caller leaves both open (M > 64) ----
 // A cost model with four constants per kernel family, fitted to 80 shapes x 5 families x splits 1, 2, 4 timed on
 // an MI355X (mean |log error| 5-10 %):
-//     time = rounds * (n * tau * clock + o) + phi * (split - 1)
+//     time = rounds * (n * tau * clock + o) + phi * log2(split)
 //   n       K-iterations per CTA (iterations per tile / split)
 //   clock   1 + 0.4 * (busy CUs / CUs)^2: the part is power-limited, busy CUs slow each other down
 //   rounds  CTAs the busiest CU runs one after another; a family whose CTAs share a CU (occ > 1) is charged
 //           1 + (rounds - 1) * gamma for them
-//   o       prologue and epilogue of a CTA, phi the fix-up per extra contributor of a split tile (two halves of a
-//           256 x 256 tile are finished by both CTAs in parallel: 5 us; four ways the owner adds three partials)
+//   o       prologue and epilogue of a CTA, phi one exchange of half tiles between the CTAs of a split tile (a
+//           tile cut in two takes one, a tile cut in four two in a row: see run_persistent)
 // Choosing by it is within 5 % of the fastest of the candidates on average (worst case 23 %) on those shapes, where
 // the earlier rule (largest tile that fills the device, Stream-K for what is left) was 49 % behind on average.
 static int gcd_int(int a, int b) {
@@ -223,7 +223,7 @@ struct TileFamily {
   float tau, gamma, o, phi;
 };
 static const TileFamily kFamilies16[] = {
-    {256, 256, 64, 7, 1, 4, 0.987f, 0.20f, 9.3f, 5.2f},   // four waves, K loop in assembly (K % 64 == 0)
+    {256, 256, 64, 7, 1, 4, 0.999f, 0.20f, 8.4f, 6.0f},   // four waves, K loop in assembly (K % 64 == 0)
     {256, 256, 64, 4, 1, 2, 1.080f, 0.20f, 9.3f, 10.0f},  // eight waves, for the other K
     {128, 128, 64, 4, 2, 4, 0.497f, 0.47f, 4.9f, 5.1f},
     {64, 128, 32, 5, 3, 4, 0.154f, 0.89f, 3.5f, 3.2f},
@@ -232,14 +232,14 @@ static const TileFamily kFamilies16[] = {
 };
 // one-byte operands (BK = 128), fitted the same way to 36 shapes each (64 x 128: to 42 shapes with M <= 1024)
 static const TileFamily kFamiliesF8[] = {
-    {256, 256, 128, -1, 1, 4, 0.916f, 1.00f, 9.7f, 5.6f},
+    {256, 256, 128, -1, 1, 4, 0.934f, 1.00f, 8.8f, 6.1f},
     {128, 128, 128, -1, 2, 2, 0.435f, 0.52f, 6.3f, 6.6f},
     {128, 256, 128, -1, 1, 2, 0.580f, 0.20f, 9.3f, 6.7f},
     {256, 128, 128, -1, 1, 2, 0.608f, 1.00f, 7.2f, 7.8f},
     {64, 128, 128, -1, 2, 2, 0.335f, 0.46f, 4.3f, 6.5f},
 };
 static const TileFamily kFamiliesI8[] = {
-    {256, 256, 128, -1, 1, 4, 0.948f, 0.20f, 13.6f, 4.0f},
+    {256, 256, 128, -1, 1, 4, 0.962f, 0.20f, 13.3f, 4.2f},
     {128, 128, 128, -1, 2, 2, 0.531f, 0.52f, 2.3f, 6.4f},
     {128, 256, 128, -1, 1, 2, 0.674f, 0.20f, 6.5f, 6.5f},
     {256, 128, 128, -1, 1, 2, 0.700f, 1.00f, 4.9f, 6.5f},
@@ -280,7 +280,7 @@ static const KernelInfo *model_pick(int64_t M, int64_t N, int64_t K, int dtype, 
       const double clock = 1.0 + 0.4 * busy * busy;
       const int64_t rounds = ctas > num_cus ? cdiv(ctas, num_cus) : 1;
       const double eff = f.occ == 1 ? (double)rounds : 1.0 + (rounds - 1) * f.gamma;
-      const double time = eff * ((double)(ipt / s) * f.tau * clock + f.o) + (s > 1 ? f.phi * (s - 1) : 0.0);
+      const double time = eff * ((double)(ipt / s) * f.tau * clock + f.o) + (s == 1 ? 0.0 : (s == 2 ? f.phi : 2.0 * f.phi));
       if (!best || time < best_time) {
         best = k;
         best_time = time;

@@ -72,7 +72,7 @@ struct DevPlan {
   int spin_limit;             // polls before a waiting owner gives up
   int xcd_remap;              // 1: spread logical CTA ids so each XCD owns a contiguous range
   int raster_tail;            // tile rows in the last raster group (tiles_m % raster, or raster)
-  int halves;                 // 1: REDUCE plan whose every Stream-K tile is cut into two equal CTA segments
+  int halves;                 // REDUCE plan whose every Stream-K tile is cut into two (1) or four (2) equal CTA segments
   int perm_s, perm_g;         // perm_s > 1: Stream-K tile v stands at position (v % perm_s) * perm_g + v / perm_s
   FastDiv by_ipt, by_tiles_n, by_width, by_raster, by_tail, by_full1, by_full, by_perm;
 };

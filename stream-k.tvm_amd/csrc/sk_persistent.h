@@ -122,6 +122,41 @@ __device__ __forceinline__ void run_persistent(const typename P::Args &a, const 
         // exchange moves the same bytes as the owner scheme, but over twice as many CTAs at once, and
         // the sum of two terms does not depend on their order.
         if constexpr (has_halves<P>::value) {
+          if (plan.halves == 2) {
+            // Four equal segments per tile, CTAs base .. base + 3.  Round 1: the pairs (0, 1) and (2, 3) exchange
+            // halves as above; CTAs 0 and 2 then hold the pair's sum of half 0, CTAs 1 and 3 that of half 1.
+            // Round 2: CTA 2 hands its half to CTA 0 and CTA 3 its half to CTA 1 (parked in the other half of
+            // their slots, which nobody reads in round 1; flags of their own, grid entries further on), and CTAs 0
+            // and 1 finish half of C each.  Every flag has one reader, who clears it; the order of the sums is
+            // fixed.  Two half-tile exchanges in a row instead of one CTA adding three partial tiles.
+            const int q = plan.by_full.div(k0), base = pid - q;
+            const int half = q & 1, peer1 = base + (q ^ 1);
+            const int units = (int)(((size_t)(pid + 1) * P::TILE_ELEMS * 4 + 255) >> 8);
+            bool ok = true;
+            P::store_partial_half(acc, ws.partials + (size_t)pid * P::TILE_ELEMS, 1 - half);
+            signal_partial_ready<true>(&ws.flags[pid], ws.status + WS_DIRTY, units);
+            if (wait_partials_ready<true>(&ws.flags[peer1], 1, plan.spin_limit)) {
+              P::add_partial_half(acc, ws.partials + (size_t)peer1 * P::TILE_ELEMS, half);
+              clear_flags_after_use(&ws.flags[peer1], 1);
+            } else {
+              ok = false;
+            }
+            if (q >= 2) {
+              P::store_partial_half(acc, ws.partials + (size_t)pid * P::TILE_ELEMS, half);
+              signal_partial_ready<true>(&ws.flags[plan.grid + pid], ws.status + WS_DIRTY, units);
+            } else {
+              const int peer2 = pid + 2;
+              if (wait_partials_ready<true>(&ws.flags[plan.grid + peer2], 1, plan.spin_limit)) {
+                P::add_partial_half(acc, ws.partials + (size_t)peer2 * P::TILE_ELEMS, half);
+                clear_flags_after_use(&ws.flags[plan.grid + peer2], 1);
+              } else {
+                ok = false;
+              }
+              P::store_c_half(a, acc, pm, pn, smem, bias, half);
+            }
+            if (!ok && threadIdx.x == 0) ws.status[WS_STATUS] = -8;  // SK_ERR_TIMEOUT
+            continue;
+          }
           const int half = k0 != 0 ? 1 : 0, peer = k0 != 0 ? pid - 1 : pid + 1;
           P::store_partial_half(acc, ws.partials + (size_t)pid * P::TILE_ELEMS, 1 - half);
           signal_partial_ready<true>(&ws.flags[pid], ws.status + WS_DIRTY,

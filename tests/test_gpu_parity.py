@@ -100,6 +100,77 @@ def test_cfg2_streamk_both_fixups(sk, oracle, cfg, fixup):
     assert _rel(oracle, C, ref) <= 1e-3 <= TOL
 
 
+def test_four_equal_segments_two_round_exchange(sk, oracle):
+    """Every Stream-K tile cut into four equal segments (fixed split 4, or `basic` on four CTAs per tile) with the
+    ordered fix-up: the four CTAs exchange halves in two rounds and two of them finish half of C each.  Against the
+    fp32 host product, exact on integer data, bitwise repeatable, equal between `splitk` and `basic` on the same grid,
+    with ragged edges, a bias, data-parallel tiles beside the split ones, fp16 / bfloat16 / int8 / fp8, and after an
+    ATOMIC launch on the same workspace."""
+    import torch
+    rng = np.random.default_rng(59)
+    ran = 0
+    for (M, N, K) in [(512, 512, 1024), (300, 700, 2048), (1000, 264, 512)]:
+        A = (rng.random((M, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+        B = (rng.random((N, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+        Ai, Bi = rng.integers(-1, 2, (M, K)).astype(np.float16), rng.integers(-1, 2, (N, K)).astype(np.float16)
+        bias = (rng.random(N, dtype=np.float32) - 0.5).astype(np.float16)
+        ref = oracle.matmul_fp32(A, B, trans_b=True)
+        exact = Ai.astype(np.int32) @ Bi.astype(np.int32).T
+        for layout in ("nt", "nn"):
+            if layout == "nn" and N % 8:
+                continue
+            dB = _t(np.ascontiguousarray(B.T) if layout == "nn" else B)
+            dBi = _t(np.ascontiguousarray(Bi.T) if layout == "nn" else Bi)
+            for tile in (dict(bm=256, bn=256, bk=64, variant=8), dict(bm=256, bn=256, bk=64, variant=5), dict(bm=128, bn=128, bk=64, variant=5),
+                         dict(bm=128, bn=256, bk=64, variant=5)):
+                try:
+                    plan = sk.make_plan(M, N, K, "float16", layout, dict(tile, schedule="splitk", split=4, fixup="reduce"))
+                except sk.StreamKError:
+                    continue
+                assert plan.streamk_tiles == plan.total_tiles and 4 * plan.streamk_full_tiles == plan.iters_per_tile
+                C = sk.streamk_fp16(_t(A), dB, layout=layout, plan=plan)
+                assert _rel(oracle, C, ref) <= 1e-3 <= TOL, (M, N, K, layout, tile)
+                assert torch.equal(C, sk.streamk_fp16(_t(A), dB, layout=layout, plan=plan))
+                basic = sk.make_plan(M, N, K, "float16", layout, dict(tile, schedule="basic", grid=plan.grid, fixup="reduce"))
+                assert torch.equal(C, sk.streamk_fp16(_t(A), dB, layout=layout, plan=basic))
+                assert np.array_equal(sk.streamk_fp16(_t(Ai), dBi, layout=layout, plan=plan).cpu().numpy().astype(np.int32), exact)
+                # an ATOMIC launch in between leaves the workspace fit for the next ordered launch
+                atomic = sk.make_plan(M, N, K, "float16", layout, dict(tile, schedule="splitk", split=4, fixup="atomic"))
+                assert _rel(oracle, sk.streamk_fp16(_t(A), dB, layout=layout, plan=atomic), ref) <= 1e-3
+                assert torch.equal(C, sk.streamk_fp16(_t(A), dB, layout=layout, plan=plan))
+                if layout == "nt":
+                    Cb = sk.streamk_fp16(_t(A), dB, plan=plan, bias=_t(bias))
+                    assert _rel(oracle, Cb, ref + bias.astype(np.float32)[None, :]) <= 1e-3
+                ran += 1
+    assert ran >= 14, ran
+    # split tiles beside data-parallel ones: sk2 on a grid that gives every split tile four CTAs
+    M, N, K = 1280, 1024, 2048   # 5 x 4 = 20 tiles of 256 x 256; grid 16: 4 Stream-K tiles over 16 CTAs, 16 data-parallel
+    A = (rng.random((M, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+    B = (rng.random((N, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+    plan = sk.make_plan(M, N, K, "float16", "nt", dict(bm=256, bn=256, bk=64, variant=8, schedule="sk1", grid=16, fixup="reduce"))
+    assert plan.streamk_tiles == 4 and plan.blocking_tiles == 16 and 4 * plan.streamk_full_tiles == plan.iters_per_tile
+    C = sk.streamk_fp16(_t(A), _t(B), plan=plan)
+    assert _rel(oracle, C, oracle.matmul_fp32(A, B, trans_b=True)) <= 1e-3
+    assert torch.equal(C, sk.streamk_fp16(_t(A), _t(B), plan=plan))
+    # one-byte operands and bfloat16
+    M, N, K = 512, 512, 2048
+    Ai8, Bi8 = rng.integers(-128, 128, (M, K)).astype(np.int8), rng.integers(-128, 128, (N, K)).astype(np.int8)
+    for bm in (256, 128):
+        p8 = sk.make_plan(M, N, K, "int8", "nt", dict(bm=bm, bn=bm, schedule="splitk", split=4, fixup="reduce"))
+        assert np.array_equal(sk.streamk_int8(_t(Ai8), _t(Bi8), plan=p8).cpu().numpy(), Ai8.astype(np.int32) @ Bi8.astype(np.int32).T)
+    f8 = torch.float8_e4m3fn
+    Af, Bf = torch.randn(M, K).to(f8), torch.randn(N, K).to(f8)
+    pf = sk.make_plan(M, N, K, "float8_e4m3", "nt", dict(bm=256, bn=256, schedule="splitk", split=4, fixup="reduce"))
+    Cf = sk.streamk_fp8(Af.cuda(), Bf.cuda(), plan=pf)
+    assert _rel(oracle, Cf, oracle.f8_gemm_ref(Af.view(torch.uint8).numpy(), Bf.view(torch.uint8).numpy())) <= 2e-3
+    assert torch.equal(Cf, sk.streamk_fp8(Af.cuda(), Bf.cuda(), plan=pf))
+    Ab, Bb = torch.randn(M, K).bfloat16(), torch.randn(N, K).bfloat16()
+    pb = sk.make_plan(M, N, K, "bfloat16", "nt", dict(bm=256, bn=256, bk=64, variant=8, schedule="splitk", split=4, fixup="reduce"))
+    Cb = sk.streamk_bf16(Ab.cuda(), Bb.cuda(), plan=pb)
+    assert _rel(oracle, Cb, oracle.matmul_fp32(Ab.float().numpy(), Bb.float().numpy(), trans_b=True)) <= 4e-3
+    sk.workspace_status()
+
+
 def test_whole_tile_ranges_need_no_workspace(sk, oracle):
     """A Stream-K schedule whose CTA ranges are whole tiles (`basic` on a tile count that is a multiple of the grid)
     only changes which tiles a CTA takes: the plan asks for no workspace and the result equals the data-parallel
