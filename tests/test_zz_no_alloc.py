@@ -55,6 +55,9 @@ def test_static_workspace_entry_point_matches_sk_gemm_f16():
     both(520, 264, 1032, dict(red, grid=24), integer=True)
     # the large tile of the headline kernel
     both(1024, 1024, 2048, dict(bm=256, bn=256, bk=64, schedule="basic", fixup="reduce", grid=48), integer=False)
+    # tiles cut into four equal segments: the two-round exchange and its second set of flags
+    both(512, 512, 1024, dict(bm=128, bn=128, bk=64, schedule="splitk", split=4, fixup="reduce"), integer=False)
+    both(512, 512, 1024, dict(bm=256, bn=256, bk=64, schedule="splitk", split=4, fixup="reduce"), integer=True)
     # a plan without Stream-K tiles needs no workspace at all
     plan = streamk.make_plan(512, 512, 512, "float16", "nt", dict(bm=128, bn=128, bk=64, schedule="dp"))
     A = torch.randn(512, 512, device="cuda").half()
