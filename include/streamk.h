@@ -104,7 +104,9 @@ typedef struct sk_config {
   int32_t reserved[4];    /* reserved[0]: 0 = preferred kernel variant of the tile, v > 0 = variant v - 1
                              (implementation alternatives of one tile shape, for the autotuner);
                              reserved[1]: split factor of SK_SCHED_SPLIT_K, 0 = choose;
-                             reserved[2]: 1 = interleaved order of the Stream-K tiles (see sk_plan.interleave) */
+                             reserved[2]: 1 = interleaved order of the Stream-K tiles (see sk_plan.interleave); with 0 the
+                             automatic schedule still chooses it for 256 x 256 tiles whose CTA ranges would start
+                             anywhere in their tiles */
 } sk_config;
 
 /* Result of the host partitioner: the integers of streamk_fp32.py:30-54 for the chosen tile/grid. */

@@ -200,9 +200,14 @@ static int gcd_int(int a, int b) {
 // starts at the beginning or in the middle of a tile (grid / gcd(Stream-K tiles, grid) <= 2), or consecutive
 // ranges start within ipt / 2 iterations of each other across the grid / 8 CTAs of an XCD.  Measured against
 // data-parallel: 3-22 % faster where admitted; 4 or 8 distinct offsets between 8 % faster and 40 % slower;
-// ranges that start anywhere up to 1.5x slower.
-static int auto_tile_schedule(int64_t total, int grid, int ipt, int *sk_tiles) {
+// ranges that start anywhere up to 1.5x slower.  `interleave` (may be null: not offered) opens a third way for a
+// one-CTA-per-CU kernel: with g = gcd(Stream-K tiles, grid) >= 8 the interleaved tile order puts the g CTAs that
+// start at the same offset side by side on one XCD, which restores their lock-step (fp16 256 x 256 tiles, every
+// tile split: 4096 x 5120 x 5120 172 us against 203 us in raster order, 3000 x 6144 x 4096 132 against 172,
+// 2048 x 11008 x 4096 171 against 172; the best data-parallel plan of any tile: 215 / 160 / 178 us).
+static int auto_tile_schedule(int64_t total, int grid, int ipt, int *sk_tiles, int *interleave = nullptr) {
   *sk_tiles = 0;
+  if (interleave) *interleave = 0;
   const int64_t waves = (total + grid - 1) / grid;
   if (total < grid || total * 10 >= waves * grid * 9 || ipt < 64) return SK_SCHED_DP;  // (short K: the fix-up outweighs the tail)
   const int sched = total >= 2 * (int64_t)grid ? SK_SCHED_SK_TWO_TILE : SK_SCHED_SK_BASIC;
@@ -213,7 +218,11 @@ static int auto_tile_schedule(int64_t total, int grid, int ipt, int *sk_tiles) {
   const double d = r < ipt - r ? r : ipt - r;
   const bool aligned = grid / gcd_int(skt, grid) <= 2;
   const bool close = d * (grid / 8 > 0 ? grid / 8 : 1) <= ipt / 2.0;
-  if (!aligned && !close) return SK_SCHED_DP;
+  if (!aligned && !close) {
+    const int g = gcd_int(skt, grid);
+    if (!interleave || g < 8 || skt / g < 2) return SK_SCHED_DP;
+    *interleave = 1;
+  }
   *sk_tiles = skt;
   return sched;
 }
@@ -292,7 +301,9 @@ static const KernelInfo *model_pick(int64_t M, int64_t N, int64_t K, int dtype, 
     // iterations spread evenly over the CUs, plus one exchange of partial tiles (the rule is applied again below,
     // to the same effect, when the plan is made)
     int skt = 0;
-    if (f.occ == 1 && tiles > num_cus && auto_tile_schedule(tiles, num_cus, (int)ipt, &skt) != SK_SCHED_DP) {
+    int ilv = 0;
+    int *offer = f.bm == 256 && f.bn == 256 ? &ilv : nullptr;  // (the interleaved order: measured on these tiles)
+    if (f.occ == 1 && tiles > num_cus && auto_tile_schedule(tiles, num_cus, (int)ipt, &skt, offer) != SK_SCHED_DP) {
       const double time = (double)tiles * ipt / num_cus * f.tau * 1.4 + f.o * (double)cdiv(tiles, num_cus) + 2.0 * f.phi;
       if (!best || time < best_time) {
         best = k;
@@ -398,6 +409,7 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
     if (ipt % split != 0 || total64 * split > max_grid) return SK_ERR_CONFIG;
     grid = (int)(total64 * split);
   }
+  int auto_interleave = 0;  // the automatic schedule asks for the interleaved order of its Stream-K tiles
   if (sched == SK_SCHED_AUTO) {
     // data-parallel when the last wave of tiles is (nearly) full: Stream-K's fix-up and the L2
     // reuse it gives up cost more than a tail of under 10 %.  Otherwise Stream-K, splitting only
@@ -418,7 +430,7 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
         grid = split > 1 ? (int)(total64 * split) : grid;
       } else {
         int skt;
-        sched = auto_tile_schedule(total64, grid, out->iters_per_tile, &skt);
+        sched = auto_tile_schedule(total64, grid, out->iters_per_tile, &skt, occ == 1 && k->bm == 256 && k->bn == 256 ? &auto_interleave : nullptr);  // (measured on these)
       }
     }
   }
@@ -456,8 +468,8 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
   out->fixup = fixup;
   out->spin_limit = cfg && cfg->spin_limit > 0 ? cfg->spin_limit : (1 << 22);
   out->interleave = 0;
-  if (cfg && cfg->reserved[2] != 0) {
-    if (cfg->reserved[2] != 1) return SK_ERR_CONFIG;
+  if (cfg && cfg->reserved[2] != 0 && cfg->reserved[2] != 1) return SK_ERR_CONFIG;
+  if ((cfg && cfg->reserved[2] == 1) || auto_interleave) {
     int g = sk_tiles, b = grid;  // gcd
     while (b) { const int t = g % b; g = b; b = t; }
     if (sk_tiles > 0 && g > 1 && sk_tiles / g > 1) out->interleave = sk_tiles / g;

@@ -141,8 +141,10 @@ def test_raster_is_a_permutation(sk):
 
 def test_untuned_plans_keep_cta_ranges_aligned(sk):
     """With tile, schedule and grid left to the planner, a tile kernel never gets CTA ranges that start anywhere in
-    their tiles: the plan is data-parallel, a fixed split of K in two or four, or a Stream-K schedule whose ranges
-    start at the beginning or in the middle of a tile; and a Stream-K tile never has more than four contributors."""
+    their tiles and in raster order: the plan is data-parallel, a fixed split of K in two or four, a Stream-K
+    schedule whose ranges start at the beginning or in the middle of a tile or close to each other, or (one CTA per
+    CU only) a Stream-K schedule in the interleaved tile order with at least eight CTAs at every offset; and a
+    Stream-K tile never has more than four contributors."""
     import math
     SPLITK, DP = sk._lib.SCHEDULES["splitk"], sk._lib.SCHEDULES["dp"]
     seen, streamk_seen = set(), set()
@@ -167,13 +169,22 @@ def test_untuned_plans_keep_cta_ranges_aligned(sk):
                     # that stay within half a tile of each other across the CTAs of an XCD
                     assert ipt <= per_cta < 2 * ipt, (dtype, M, N, K, name)
                     drift = min(per_cta - ipt, 2 * ipt - per_cta)
-                    aligned = plan.grid // math.gcd(plan.streamk_tiles, plan.grid) <= 2
+                    g = math.gcd(plan.streamk_tiles, plan.grid)
+                    aligned = plan.grid // g <= 2
+                    if plan.interleave > 1:
+                        assert not aligned and g >= 8 and plan.interleave == plan.streamk_tiles // g, (dtype, M, N, K)
+                        assert plan.grid == 256 and "256x256" in name, (dtype, M, N, K, name)
+                        streamk_seen.add("interleaved")
+                        continue
                     assert aligned or drift * (plan.grid // 8) <= ipt / 2, (dtype, M, N, K, name, plan.as_dict())
                     streamk_seen.add(aligned)
-    assert SPLITK in seen and DP in seen and streamk_seen == {True, False}   # both kinds of Stream-K plan occur
+    assert SPLITK in seen and DP in seen and streamk_seen == {True, False, "interleaved"}   # every kind occurs
     # 258 tiles on 256 CUs: every tile is split (64.5 iterations per CTA), not the two remainder tiles alone
     p = sk.make_plan(1536, 11008, 4096, "float16", "nt", cus=256, use_tuned=False)
     assert (p.bm, p.bn, p.schedule, p.streamk_tiles, p.grid) == (256, 256, sk._lib.SCHEDULES["basic"], 258, 256)
+    # 320 tiles of 80 iterations: 100 per CTA, five distinct offsets, 64 CTAs at each: the interleaved order
+    p = sk.make_plan(4096, 5120, 5120, "float16", "nt", cus=256, use_tuned=False)
+    assert (p.bm, p.bn, p.schedule, p.streamk_tiles, p.grid, p.interleave) == (256, 256, sk._lib.SCHEDULES["basic"], 320, 256, 5)
     # the assembly-loop kernel where it applies and the device is filled; a split in two halves below that
     p = sk.make_plan(8192, 8192, 8192, "float16", "nt", cus=256, use_tuned=False)
     assert (sk.kernel_name(p.kernel_id), p.schedule, p.grid) == ("tile_f16_nt_asm_256x256x64", DP, 256)

@@ -197,15 +197,15 @@ def test_whole_tile_ranges_need_no_workspace(sk, oracle):
 
 
 def test_untuned_plans_on_ragged_shapes(sk, oracle):
-    """The planner's own choice (no configuration, no tuned cache: cost model, aligned split, admitted Stream-K)
-    on shapes that exercise each of its branches, ragged edges included: fp16 NT / NN and bfloat16 against the
+    """The planner's own choice (no configuration, no tuned cache: cost model, aligned split, admitted Stream-K in
+    raster and in interleaved tile order) on shapes that exercise each of its branches, ragged edges included: fp16 NT / NN and bfloat16 against the
     fp32 host product (1e-3 / 4e-3), int8 exactly."""
     import torch
     rng = np.random.default_rng(47)
-    kinds = set()
+    kinds, interleaved = set(), 0
     for (M, N, K) in [(65, 136, 328), (200, 1000, 1032), (384, 4096, 1024), (520, 2048, 4096), (768, 4096, 2048), (1000, 1096, 8192),
                       (1536, 11008, 1024), (2100, 4000, 512), (3000, 5120, 1024), (3000, 8192, 4096), (4096, 4096, 64), (1536, 11008, 4096),
-                      (1024, 8192, 512), (512, 8192, 1024)]:
+                      (1024, 8192, 512), (512, 8192, 1024), (2990, 6104, 4096)]:
         A = (rng.random((M, K), dtype=np.float32) * 2 - 1).astype(np.float16)
         B = (rng.random((N, K), dtype=np.float32) * 2 - 1).astype(np.float16)
         ref = oracle.matmul_fp32(A, B, trans_b=True)
@@ -213,6 +213,7 @@ def test_untuned_plans_on_ragged_shapes(sk, oracle):
             dB = _t(np.ascontiguousarray(B.T) if layout == "nn" else B)
             plan = sk.make_plan(M, N, K, "float16", layout, use_tuned=False)
             kinds.add((plan.schedule, plan.streamk_tiles > 0))
+            interleaved += plan.interleave > 1
             C = sk.streamk_fp16(_t(A), dB, layout=layout, plan=plan)
             assert _rel(oracle, C, ref) <= 1e-3 <= TOL, (M, N, K, layout, sk.kernel_name(plan.kernel_id), plan.as_dict())
             if M * N * K > 5e9:   # (the host reference of the large shapes is computed once, for fp16)
@@ -229,6 +230,7 @@ def test_untuned_plans_on_ragged_shapes(sk, oracle):
             assert np.array_equal(sk.streamk_int8(_t(Ai), _t(Bi), plan=pi).cpu().numpy(), Ai.astype(np.int32) @ Bi.astype(np.int32).T), (M, N, K)
     S = sk._lib.SCHEDULES
     assert (S["dp"], False) in kinds and (S["splitk"], True) in kinds and ((S["basic"], True) in kinds or (S["sk2"], True) in kinds), kinds
+    assert interleaved >= 2   # 288 tiles of 64 iterations on 256 CUs: nine offsets, 32 CTAs at each (both layouts)
     sk.workspace_status()
 
 
