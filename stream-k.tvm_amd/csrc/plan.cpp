@@ -235,6 +235,7 @@ static const TileFamily kFamilies16[] = {
     {256, 256, 64, 7, 1, 4, 0.999f, 0.20f, 8.4f, 6.0f},   // four waves, K loop in assembly (K % 64 == 0)
     {256, 256, 64, 4, 1, 2, 1.080f, 0.20f, 9.3f, 10.0f},  // eight waves, for the other K
     {128, 128, 64, 4, 2, 4, 0.497f, 0.47f, 4.9f, 5.1f},
+    {128, 128, 32, 5, 2, 4, 0.218f, 0.89f, 3.8f, 4.5f},   // four stages of 32 (NT only)
     {64, 128, 32, 5, 3, 4, 0.154f, 0.89f, 3.5f, 3.2f},
     {128, 256, 64, 4, 1, 4, 0.689f, 1.00f, 6.0f, 5.9f},
     {256, 128, 64, 4, 1, 4, 0.685f, 0.20f, 5.3f, 5.8f},
