@@ -303,6 +303,11 @@ struct KernelInfo {
   X(83, 256, 128, 4, 2)       \
   X(85, 64, 128, 2, 2)
 
+// the same in four stages of 64 int8 per row (variant 5), for short rows of CTAs:  X(id, BM, BN, WM, WN)
+#define SK_TILE_I8_BK64_KERNELS(X) \
+  X(86, 128, 128, 2, 2)            \
+  X(87, 64, 128, 2, 2)
+
 // 256 x 256 x 64 on four waves, K loop in assembly (variant 7), K a multiple of 64 (int8: 128 bytes per
 // iteration):  X(id, MODE, NN)  with MODE 0 fp16, 1 bfloat16, 2 int8, 3 fp8 e4m3, 4 fp8 e5m2; NN: B is [K,N]
 #define SK_TILE_ASM_KERNELS(X) \

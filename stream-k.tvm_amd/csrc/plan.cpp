@@ -254,6 +254,8 @@ static const TileFamily kFamiliesI8[] = {
     {128, 256, 128, -1, 1, 2, 0.674f, 0.20f, 6.5f, 6.5f},
     {256, 128, 128, -1, 1, 2, 0.700f, 1.00f, 4.9f, 6.5f},
     {64, 128, 128, -1, 2, 2, 0.392f, 0.39f, 3.3f, 4.0f},
+    {128, 128, 64, 5, 2, 4, 0.222f, 0.77f, 4.7f, 3.9f},   // four stages of 64 (fitted to 48 shapes with M <= 1024)
+    {64, 128, 64, 5, 3, 4, 0.143f, 0.88f, 4.0f, 4.1f},
 };
 
 static const KernelInfo *model_pick(int64_t M, int64_t N, int64_t K, int dtype, int layout, int num_cus, int *split,

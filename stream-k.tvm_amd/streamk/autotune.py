@@ -100,8 +100,11 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
                     out.extend(dict(base, schedule="splitk", fixup=fixup) for fixup in ("reduce", "atomic"))
                     out.append(dict(base, schedule="splitk", split=2, fixup="reduce"))
     if dtype in ("float8_e4m3", "float8_e5m2", "int8"):
-        for (bm, bn), raster in itertools.product(((256, 256), (256, 128), (128, 256), (128, 128), (64, 128)), (1, 8)):
-            base = dict(bm=bm, bn=bn, raster=raster)
+        tiles = [(256, 256, 0), (256, 128, 0), (128, 256, 0), (128, 128, 0), (64, 128, 0)]
+        if dtype == "int8":  # four stages of 64 K-values
+            tiles += [(128, 128, 64), (64, 128, 64)]
+        for (bm, bn, bk), raster in itertools.product(tiles, (1, 8)):
+            base = dict(bm=bm, bn=bn, raster=raster, **({"bk": bk} if bk else {}))
             out.append(dict(base, schedule="dp"))
             for sched, fixup in itertools.product(("sk2", "sk1", "basic"), ("reduce", "atomic")):
                 out.append(dict(base, schedule=sched, fixup=fixup))

@@ -1402,20 +1402,22 @@ def test_int8_tile_kernels(sk, oracle):
     strided operands and an output whose rows are not 16-byte aligned."""
     import torch
     torch.manual_seed(12)
-    tiles = [(256, 256), (128, 128), (128, 256), (256, 128), (64, 128)]
+    # (bm, bn, bk): two stages of 128 K-values (the default of a tile shape), four stages of 64
+    tiles = [(256, 256, 128), (128, 128, 128), (128, 256, 128), (256, 128, 128), (64, 128, 128), (128, 128, 64), (64, 128, 64)]
     for (M, N, K) in [(200, 136, 336), (1000, 1096, 1040), (520, 264, 128), (64, 512, 2048), (300, 300, 16)]:
         A = torch.randint(-128, 128, (M, K), dtype=torch.int8)
         B = torch.randint(-128, 128, (N, K), dtype=torch.int8)
         ref = torch.from_numpy(oracle.i8_gemm_ref(A.numpy(), B.numpy()))
         dA, dB = A.cuda(), B.cuda()
-        for (bm, bn) in tiles:
+        for (bm, bn, bk) in tiles:
             for sch in (dict(schedule="dp"), dict(schedule="basic", fixup="reduce", grid=24),
                         dict(schedule="sk2", fixup="atomic", grid=16), dict(schedule="sk1", fixup="reduce", grid=7),
                         dict(schedule="basic", fixup="atomic", grid=40, raster=1)):
-                plan = sk.make_plan(M, N, K, "int8", "nt", dict(bm=bm, bn=bn, **sch))
-                assert plan.bk == 128 and plan.iters_per_tile == -(-K // 128)
+                plan = sk.make_plan(M, N, K, "int8", "nt", dict(bm=bm, bn=bn, **(dict(bk=64) if bk == 64 else {}), **sch))
+                assert plan.bk == bk and plan.iters_per_tile == -(-K // bk)
+                assert sk.kernel_name(plan.kernel_id).endswith(f"_{bm}x{bn}x{bk}")
                 C = sk.streamk_int8(dA, dB, plan=plan)
-                assert C.dtype == torch.int32 and torch.equal(C.cpu().long(), ref), (M, N, K, bm, bn, sch)
+                assert C.dtype == torch.int32 and torch.equal(C.cpu().long(), ref), (M, N, K, bm, bn, bk, sch)
     # the four-wave kernel with the K loop in assembly (K a multiple of 128): every schedule, both fix-ups, the
     # halves exchange of a tile split in two
     assert sk.kernel_name(sk.make_plan(4096, 4096, 4096, "int8", "nt", use_tuned=False).kernel_id) == "tile_i8_nt_asm_256x256x128"
