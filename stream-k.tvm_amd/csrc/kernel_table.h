@@ -308,6 +308,14 @@ struct KernelInfo {
   X(86, 128, 128, 2, 2)            \
   X(87, 64, 128, 2, 2)
 
+// fp8 in four stages of 64 K-values (variant 5; e5m2: ids + 20):  X(id, BM, BN, WM, WN)
+#define SK_TILE_F8_BK64_KERNELS(X) \
+  X(76, 128, 128, 2, 2)            \
+  X(77, 64, 128, 1, 4)
+#define SK_TILE_F8E5M2_BK64_KERNELS(X) \
+  X(96, 128, 128, 2, 2)                \
+  X(97, 64, 128, 1, 4)
+
 // 256 x 256 x 64 on four waves, K loop in assembly (variant 7), K a multiple of 64 (int8: 128 bytes per
 // iteration):  X(id, MODE, NN)  with MODE 0 fp16, 1 bfloat16, 2 int8, 3 fp8 e4m3, 4 fp8 e5m2; NN: B is [K,N]
 #define SK_TILE_ASM_KERNELS(X) \

@@ -247,6 +247,8 @@ static const TileFamily kFamiliesF8[] = {
     {128, 256, 128, -1, 1, 2, 0.580f, 0.20f, 9.3f, 6.7f},
     {256, 128, 128, -1, 1, 2, 0.608f, 1.00f, 7.2f, 7.8f},
     {64, 128, 128, -1, 2, 2, 0.335f, 0.46f, 4.3f, 6.5f},
+    {128, 128, 64, 5, 2, 4, 0.218f, 0.88f, 2.3f, 11.0f},  // four stages of 64 (fitted to 48 shapes with M <= 1024)
+    {64, 128, 64, 5, 3, 4, 0.135f, 1.00f, 2.9f, 8.6f},
 };
 static const TileFamily kFamiliesI8[] = {
     {256, 256, 128, -1, 1, 4, 0.962f, 0.20f, 13.3f, 4.2f},

@@ -64,7 +64,8 @@ struct LdsArray {
 // operand) into the 32x32 accumulator blocks of the fp16 kernel.  Lane (r = l%32, g = l/32) hands
 // the instruction, for K-step s of 64 bytes, chunks 4s + g and 4s + 2 + g of row r as its 32-byte
 // operand.  Which K-values a lane's bytes stand for does not matter as long as A and B agree: the
-// instruction pairs byte b of lane group g of one operand with the same byte of the other.
+// instruction pairs byte b of lane group g of one operand with the same byte of the other.  With BK_ = 32
+// an LDS row is 64 bytes, one K-step, and the loop is the four-stage one of the 16x16x32 form.
 //
 // F8_ = 3: int8 operands, int32 accumulators and C.  The 16x16x32 pipeline as it is, with
 // v_mfma_i32_16x16x64_i8 on the same 16-byte fragments (64 K-values per K-step, same cycles as the fp16
@@ -88,7 +89,7 @@ struct TileF16NTDma {
   static constexpr bool B_KN = B_KN_, MFMA16 = MFMA16_;
   static constexpr bool I8 = F8_ == 3;
   static constexpr int F8 = I8 ? 0 : F8_;
-  static_assert(F8 == 0 || (!MFMA16_ && !B_KN_ && BK_ == 64 && !BF16_), "fp8: NT layout, two stages");
+  static_assert(F8 == 0 || (!MFMA16_ && !B_KN_ && !BF16_), "fp8: NT layout (two stages of 128 K-values or four of 64)");
   static_assert(!I8 || (MFMA16_ && !B_KN_ && !BF16_), "int8: NT layout, 16x16 accumulator blocks");
   // BF16_: operands and C are bfloat16 (same 16-bit data movement; v_mfma_f32_16x16x32_bf16; C rounded to
   // nearest even with v_cvt_pk_bf16_f32)
@@ -436,7 +437,7 @@ struct TileF16NTDma {
     // the half-step behind the barrier, sliced like tail16: loads of K-iteration kt_next into `cur`,
     // the first fragments of `nxt` (A into fa8[0], B into fb8[0]) and the MFMAs of (K-step 1, second
     // half of the rows)
-    auto tail8 = [&](char *cur, const char *nxt, int kt_next, bool dead) {
+    auto tail8 = [&](char *cur, const char *nxt, int kt_next, bool dead, int bcur = 1, int bnext = 0) {
       const bool oob = dead || (kt_next == tail_kt && kt_next * BK + my_chunk * 8 >= a.K);
       const uint32_t va = oob ? OOB_OFFSET : voff_a, vb = oob ? OOB_OFFSET : voff_b;
       constexpr int CH = DMA_PER_WAVE, NRD = FA8 + TN, NMF = FA8 * TN;
@@ -448,7 +449,7 @@ struct TileF16NTDma {
             if (r < FA8)
               read_a8_one(nxt, 0, 0, 0, r);
             else
-              read_b8_one(nxt, 0, 0, r - FA8);
+              read_b8_one(nxt, bnext, 0, r - FA8);
           }
         if (x < A_DMA) {
           const int g = wave + x * NW;
@@ -459,10 +460,41 @@ struct TileF16NTDma {
         }
 #pragma unroll
         for (int m = 0; m < NMF; ++m)
-          if (m * CH / NMF == x) mfma_one8(1, 1, 1, m);
+          if (m * CH / NMF == x) mfma_one8(1, bcur, 1, m);
       }
     };
-    if constexpr (F8 != 0) {
+    if constexpr (F8 != 0 && NSTAGE == 4) {
+      // BK = 32 (64 K-values) is one K-step: two half-steps per iteration, the four-stage schedule of the
+      // 16x16x32 form below.  Entering, fa8[0] holds the first half of the A rows and fb8[par] the B
+      // fragments of stage `cur` (par = iteration parity).
+      auto iteration4 = [&](char *cur, char *nxt, int it, int par) {
+        read_a8(cur, 1, 0, 1);
+        mfma_half8(0, par, 0);
+        interleave8<FA8 * TN, 2 * FA8>();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        wait_dma_then_barrier<2 * DMA_PER_WAVE>();
+        tail8(cur, nxt, k0 + it + 4, it + 4 >= n, par, par ^ 1);
+      };
+      char *s0 = stage(0), *s1 = stage(1), *s2 = stage(2), *s3 = stage(3);
+      issue_dma(s0, k0);
+      issue_dma(s1, k0 + 1);
+      issue_dma(s2, k0 + 2);
+      wait_dma_then_barrier<2 * DMA_PER_WAVE>();
+      issue_dma(s3, k0 + 3);
+      read_a8(s0, 0, 0, 0);
+      read_b8(s0, 0, 0);
+      int it = 0;
+      for (; it + 3 < n; it += 4) {
+        iteration4(s0, s1, it, 0);
+        iteration4(s1, s2, it + 1, 1);
+        iteration4(s2, s3, it + 2, 0);
+        iteration4(s3, s0, it + 3, 1);
+      }
+      if (it < n) iteration4(s0, s1, it, 0);
+      if (it + 1 < n) iteration4(s1, s2, it + 1, 1);
+      if (it + 2 < n) iteration4(s2, s3, it + 2, 0);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    } else if constexpr (F8 != 0) {
       // one K-iteration (128 K-values) on stage `cur`: two K-steps of 64, each in two halves of the
       // wave tile's rows.  Entering, fa8[0] / fb8[0] hold the fragments of (K-step 0, first half).
       auto iteration8 = [&](char *cur, char *nxt, int it) {

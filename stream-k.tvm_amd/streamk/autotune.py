@@ -100,9 +100,8 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
                     out.extend(dict(base, schedule="splitk", fixup=fixup) for fixup in ("reduce", "atomic"))
                     out.append(dict(base, schedule="splitk", split=2, fixup="reduce"))
     if dtype in ("float8_e4m3", "float8_e5m2", "int8"):
-        tiles = [(256, 256, 0), (256, 128, 0), (128, 256, 0), (128, 128, 0), (64, 128, 0)]
-        if dtype == "int8":  # four stages of 64 K-values
-            tiles += [(128, 128, 64), (64, 128, 64)]
+        # (bk 0: the tile's default, two stages of 128 K-values; 64: four stages of 64)
+        tiles = [(256, 256, 0), (256, 128, 0), (128, 256, 0), (128, 128, 0), (64, 128, 0), (128, 128, 64), (64, 128, 64)]
         for (bm, bn, bk), raster in itertools.product(tiles, (1, 8)):
             base = dict(bm=bm, bn=bn, raster=raster, **({"bk": bk} if bk else {}))
             out.append(dict(base, schedule="dp"))

@@ -119,8 +119,8 @@ def test_fp8_plans(sk):
         assert (q.bm, q.bn, q.bk) == (p.bm, p.bn, 128)
         assert sk.kernel_name(q.kernel_id) == ("tile_i8_nt_asm_256x256x128" if bm == 256 else f"tile_i8_nt_dma16_{bm}x{bn}x128")
     # the planner's own choice: the assembly-loop kernel where 256 x 256 tiles fill the device, 64 x 128 tiles for few
-    # rows (int8: the four-stage kernel, 64 K-values per stage)
-    for dtype, tag in (("float8_e4m3", "f8e4m3_nt_dma_64x128x128"), ("float8_e5m2", "f8e5m2_nt_dma_64x128x128"), ("int8", "i8_nt_dma16_64x128x64")):
+    # rows (the four-stage kernels, 64 K-values per stage)
+    for dtype, tag in (("float8_e4m3", "f8e4m3_nt_dma_64x128x64"), ("float8_e5m2", "f8e5m2_nt_dma_64x128x64"), ("int8", "i8_nt_dma16_64x128x64")):
         assert sk.kernel_name(sk.make_plan(8192, 8192, 8192, dtype, "nt", cus=256, use_tuned=False).kernel_id).endswith("_nt_asm_256x256x128")
         assert sk.kernel_name(sk.make_plan(65, 4096, 4096, dtype, "nt", cus=256, use_tuned=False).kernel_id) == f"tile_{tag}"
     with pytest.raises(sk.StreamKError):

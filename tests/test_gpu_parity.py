@@ -1176,7 +1176,8 @@ def test_fp8_tile_kernels(sk, oracle):
     import torch
     torch.manual_seed(11)
     f8 = torch.float8_e4m3fn
-    tiles = [(256, 256), (128, 128), (128, 256), (256, 128), (64, 128)]
+    # (bm, bn, bk): two stages of 128 K-values (the default of a tile shape), four stages of 64
+    tiles = [(256, 256, 128), (128, 128, 128), (128, 256, 128), (256, 128, 128), (64, 128, 128), (128, 128, 64), (64, 128, 64)]
     for (M, N, K) in [(200, 136, 336), (1000, 1096, 1040), (520, 264, 128), (64, 512, 2048), (300, 300, 16)]:
         A, B = torch.randn(M, K).to(f8), torch.randn(N, K).to(f8)
         Ai, Bi = torch.randint(-1, 2, (M, K)).float().to(f8), torch.randint(-1, 2, (N, K)).float().to(f8)
@@ -1184,17 +1185,23 @@ def test_fp8_tile_kernels(sk, oracle):
         exact = oracle.f8_gemm_ref(Ai.view(torch.uint8).numpy(), Bi.view(torch.uint8).numpy())
         assert np.abs(exact).max() <= 2048
         dA, dB, dAi, dBi = A.cuda(), B.cuda(), Ai.cuda(), Bi.cuda()
-        for (bm, bn) in tiles:
+        for (bm, bn, bk) in tiles:
             for sch in (dict(schedule="dp"), dict(schedule="basic", fixup="reduce", grid=24),
                         dict(schedule="sk2", fixup="atomic", grid=16), dict(schedule="sk1", fixup="reduce", grid=7)):
-                plan = sk.make_plan(M, N, K, "float8_e4m3", "nt", dict(bm=bm, bn=bn, **sch))
-                assert plan.bk == 128 and plan.iters_per_tile == -(-K // 128)
+                plan = sk.make_plan(M, N, K, "float8_e4m3", "nt", dict(bm=bm, bn=bn, **(dict(bk=64) if bk == 64 else {}), **sch))
+                assert plan.bk == bk and plan.iters_per_tile == -(-K // bk)
+                assert sk.kernel_name(plan.kernel_id) == (f"tile_f8e4m3_nt_dma_{bm}x{bn}x{bk}" if (bm, bn) != (256, 256) or K % 128 else "tile_f8e4m3_nt_asm_256x256x128")
                 C = sk.streamk_fp8(dA, dB, plan=plan)
-                assert C.dtype == torch.float16 and _rel(oracle, C, ref) <= 1e-3 <= TOL, (M, N, K, bm, bn, sch)
+                assert C.dtype == torch.float16 and _rel(oracle, C, ref) <= 1e-3 <= TOL, (M, N, K, bm, bn, bk, sch)
                 Ci = sk.streamk_fp8(dAi.view(torch.uint8), dBi.view(torch.uint8), plan=plan)   # raw bytes are accepted too
-                assert np.array_equal(Ci.double().cpu().numpy(), exact), (M, N, K, bm, bn, sch)
+                assert np.array_equal(Ci.double().cpu().numpy(), exact), (M, N, K, bm, bn, bk, sch)
                 if sch.get("fixup") == "reduce":
                     assert torch.equal(C, sk.streamk_fp8(dA, dB, plan=plan))
+                if bk == 64:   # the e5m2 twin of the four-stage kernels, on exact data
+                    p5 = sk.make_plan(M, N, K, "float8_e5m2", "nt", dict(bm=bm, bn=bn, bk=64, **sch))
+                    assert sk.kernel_name(p5.kernel_id) == f"tile_f8e5m2_nt_dma_{bm}x{bn}x64"
+                    C5 = sk.streamk_fp8(Ai.to(torch.float8_e5m2).cuda(), Bi.to(torch.float8_e5m2).cuda(), plan=p5)
+                    assert np.array_equal(C5.double().cpu().numpy(), exact), (M, N, K, bm, bn, sch)
     # the four-wave kernels whose K loop is assembly (K a multiple of 128; one 16x16x128 MFMA per accumulator block
     # and iteration): both formats, every schedule and fix-up incl. the halves exchange, alpha, bias and activation;
     # same bits as the eight-wave 32x32x64 kernel (the K-values are summed in the same groups of 128)
