@@ -415,6 +415,40 @@ def main():
                 del a8, b8, c
             extra[key] = rows8
 
+        # few rows of one-byte operands: the 64 x 128 tile kernel in two stages of 128 K-values against the same tile
+        # in four stages of 64 (three loads in flight per CTA instead of one), the planner's own choice and the vendor
+        # GEMM; graph-timed (these launches take 10-30 us)
+        few = []
+        for dt in ("float8_e4m3", "int8"):
+            for (m, n, k) in ((128, 11008, 4096), (256, 5120, 5120)):
+                g8 = torch.Generator(device="cpu").manual_seed(8)
+                if dt == "int8":
+                    a8 = torch.randint(-8, 9, (m, k), generator=g8, dtype=torch.int8).cuda()
+                    b8 = torch.randint(-8, 9, (n, k), generator=g8, dtype=torch.int8).cuda()
+                    c = torch.empty(m, n, dtype=torch.int32, device="cuda")
+                    ours, vendor = streamk.streamk_int8, (lambda: torch._int_mm(a8, b8.T, out=c))
+                else:
+                    a8 = (torch.rand(m, k, generator=g8) * 2 - 1).cuda().to(torch.float8_e4m3fn)
+                    b8 = (torch.rand(n, k, generator=g8) * 2 - 1).cuda().to(torch.float8_e4m3fn)
+                    c = torch.empty(m, n, dtype=torch.float16, device="cuda")
+                    one = torch.ones((), device="cuda")
+                    ours = streamk.streamk_fp8
+                    vendor = lambda: torch._scaled_mm(a8, b8.T, one, one, out_dtype=torch.float16, out=c)  # noqa: E731
+                pa = streamk.make_plan(m, n, k, dt, "nt", use_tuned=False)
+                p2 = streamk.make_plan(m, n, k, dt, "nt", dict(bm=64, bn=128, bk=128, schedule="dp"))
+                p4 = streamk.make_plan(m, n, k, dt, "nt", dict(bm=64, bn=128, bk=64, schedule="dp"))
+                row = {"dtype": dt, "shape": [m, n, k], "planner_kernel": streamk.kernel_name(pa.kernel_id), "planner_grid": pa.grid,
+                       "planner_us": round(time_graph(lambda: ours(a8, b8, out=c, plan=pa), launches=10) * 1e3, 1),
+                       "two_stage_64x128x128_us": round(time_graph(lambda: ours(a8, b8, out=c, plan=p2), launches=10) * 1e3, 1),
+                       "four_stage_64x128x64_us": round(time_graph(lambda: ours(a8, b8, out=c, plan=p4), launches=10) * 1e3, 1)}
+                try:
+                    row["vendor_us"] = round(time_graph(vendor, launches=10) * 1e3, 1)
+                except Exception:   # no such GEMM in this torch build
+                    row["vendor_us"] = None
+                few.append(row)
+                del a8, b8, c
+        extra["one_byte_few_rows"] = few
+
         q4 = []
         g = torch.Generator(device="cpu").manual_seed(4)
         Wq = torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8).cuda()
