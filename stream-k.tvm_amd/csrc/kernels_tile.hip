@@ -30,12 +30,6 @@ static int launch_dma(const GemmArgs &a, const DevPlan &p, const Workspace &ws, 
 #define SK_POLICY_DMA32_16(id, BM, BN, WM, WN) TileF16NTDma<BM, BN, WM, WN, false, 32, true>
 #define SK_POLICY_NN16(id, BM, BN, WM, WN) TileF16NTDma<BM, BN, WM, WN, true, 64, true>
 #define SK_POLICY_BF16(id, BM, BN, WM, WN, BK, NN) TileF16NTDma<BM, BN, WM, WN, NN, BK, true, true>
-#define SK_POLICY_F8(id, BM, BN, WM, WN) TileF16NTDma<BM, BN, WM, WN, false, 64, false, false, 1>
-#define SK_POLICY_F8E5M2(id, BM, BN, WM, WN) TileF16NTDma<BM, BN, WM, WN, false, 64, false, false, 2>
-#define SK_POLICY_I8(id, BM, BN, WM, WN) TileF16NTDma<BM, BN, WM, WN, false, 64, true, false, 3>
-#define SK_POLICY_I8_BK64(id, BM, BN, WM, WN) TileF16NTDma<BM, BN, WM, WN, false, 32, true, false, 3>
-#define SK_POLICY_F8_BK64(id, BM, BN, WM, WN) TileF16NTDma<BM, BN, WM, WN, false, 32, false, false, 1>
-#define SK_POLICY_F8E5M2_BK64(id, BM, BN, WM, WN) TileF16NTDma<BM, BN, WM, WN, false, 32, false, false, 2>
 
 int tile_kernel_infos(KernelInfo *out, int max) {
   int n = 0;
@@ -104,54 +98,6 @@ int tile_kernel_infos(KernelInfo *out, int max) {
   }
   SK_TILE_BF16_KERNELS(X)
 #undef X
-#define X(id, BM, BN, WM, WN)                                                                       \
-  if (n < max) {                                                                                    \
-    typedef SK_POLICY_F8(id, BM, BN, WM, WN) P;                                                     \
-    out[n++] = KernelInfo{id, FAMILY_TILE, 5 /* SK_F8E4M3 */, 0, 6, BM, BN, 128, P::NT, P::LDS_TOTAL, P::CTAS_PER_CU, \
-                          P::TILE_ELEMS, 0, 0, 16, "tile_f8e4m3_nt_dma_" #BM "x" #BN "x128"};       \
-  }
-  SK_TILE_F8_KERNELS(X)
-#undef X
-#define X(id, BM, BN, WM, WN)                                                                       \
-  if (n < max) {                                                                                    \
-    typedef SK_POLICY_F8E5M2(id, BM, BN, WM, WN) P;                                                 \
-    out[n++] = KernelInfo{id, FAMILY_TILE, 8 /* SK_F8E5M2 */, 0, 6, BM, BN, 128, P::NT, P::LDS_TOTAL, P::CTAS_PER_CU, \
-                          P::TILE_ELEMS, 0, 0, 16, "tile_f8e5m2_nt_dma_" #BM "x" #BN "x128"};       \
-  }
-  SK_TILE_F8E5M2_KERNELS(X)
-#undef X
-#define X(id, BM, BN, WM, WN)                                                                       \
-  if (n < max) {                                                                                    \
-    typedef SK_POLICY_I8(id, BM, BN, WM, WN) P;                                                     \
-    out[n++] = KernelInfo{id, FAMILY_TILE, 6 /* SK_I8 */, 0, 4, BM, BN, 128, P::NT, P::LDS_TOTAL, P::CTAS_PER_CU, \
-                          P::TILE_ELEMS, 0, 0, 16, "tile_i8_nt_dma16_" #BM "x" #BN "x128"};         \
-  }
-  SK_TILE_I8_KERNELS(X)
-#undef X
-#define X(id, BM, BN, WM, WN)                                                                       \
-  if (n < max) {                                                                                    \
-    typedef SK_POLICY_I8_BK64(id, BM, BN, WM, WN) P;                                                \
-    out[n++] = KernelInfo{id, FAMILY_TILE, 6 /* SK_I8 */, 0, 5, BM, BN, 64, P::NT, P::LDS_TOTAL, P::CTAS_PER_CU, \
-                          P::TILE_ELEMS, 0, 0, 16, "tile_i8_nt_dma16_" #BM "x" #BN "x64"};          \
-  }
-  SK_TILE_I8_BK64_KERNELS(X)
-#undef X
-#define X(id, BM, BN, WM, WN)                                                                       \
-  if (n < max) {                                                                                    \
-    typedef SK_POLICY_F8_BK64(id, BM, BN, WM, WN) P;                                                \
-    out[n++] = KernelInfo{id, FAMILY_TILE, 5 /* SK_F8E4M3 */, 0, 5, BM, BN, 64, P::NT, P::LDS_TOTAL, P::CTAS_PER_CU, \
-                          P::TILE_ELEMS, 0, 0, 16, "tile_f8e4m3_nt_dma_" #BM "x" #BN "x64"};        \
-  }
-  SK_TILE_F8_BK64_KERNELS(X)
-#undef X
-#define X(id, BM, BN, WM, WN)                                                                       \
-  if (n < max) {                                                                                    \
-    typedef SK_POLICY_F8E5M2_BK64(id, BM, BN, WM, WN) P;                                            \
-    out[n++] = KernelInfo{id, FAMILY_TILE, 8 /* SK_F8E5M2 */, 0, 5, BM, BN, 64, P::NT, P::LDS_TOTAL, P::CTAS_PER_CU, \
-                          P::TILE_ELEMS, 0, 0, 16, "tile_f8e5m2_nt_dma_" #BM "x" #BN "x64"};        \
-  }
-  SK_TILE_F8E5M2_BK64_KERNELS(X)
-#undef X
   return n;
 }
 
@@ -213,48 +159,6 @@ int launch_tile_f16(int id, const GemmArgs &a, const DevPlan &p, const Workspace
     return launch_dma<P>(a, p, ws, s, bias);                                                       \
   }
     SK_TILE_BF16_KERNELS(X)
-#undef X
-#define X(id_, BM, BN, WM, WN)                                                           \
-  case id_: {                                                                            \
-    typedef SK_POLICY_F8(id_, BM, BN, WM, WN) P;                                         \
-    return launch_dma<P>(a, p, ws, s, bias);                                                   \
-  }
-    SK_TILE_F8_KERNELS(X)
-#undef X
-#define X(id_, BM, BN, WM, WN)                                                           \
-  case id_: {                                                                            \
-    typedef SK_POLICY_F8E5M2(id_, BM, BN, WM, WN) P;                                     \
-    return launch_dma<P>(a, p, ws, s, bias);                                             \
-  }
-    SK_TILE_F8E5M2_KERNELS(X)
-#undef X
-#define X(id_, BM, BN, WM, WN)                                                           \
-  case id_: {                                                                            \
-    typedef SK_POLICY_I8(id_, BM, BN, WM, WN) P;                                         \
-    return launch_dma<P>(a, p, ws, s, bias);                                                   \
-  }
-    SK_TILE_I8_KERNELS(X)
-#undef X
-#define X(id_, BM, BN, WM, WN)                                                           \
-  case id_: {                                                                            \
-    typedef SK_POLICY_I8_BK64(id_, BM, BN, WM, WN) P;                                    \
-    return launch_dma<P>(a, p, ws, s, bias);                                             \
-  }
-    SK_TILE_I8_BK64_KERNELS(X)
-#undef X
-#define X(id_, BM, BN, WM, WN)                                                           \
-  case id_: {                                                                            \
-    typedef SK_POLICY_F8_BK64(id_, BM, BN, WM, WN) P;                                    \
-    return launch_dma<P>(a, p, ws, s, bias);                                             \
-  }
-    SK_TILE_F8_BK64_KERNELS(X)
-#undef X
-#define X(id_, BM, BN, WM, WN)                                                           \
-  case id_: {                                                                            \
-    typedef SK_POLICY_F8E5M2_BK64(id_, BM, BN, WM, WN) P;                                \
-    return launch_dma<P>(a, p, ws, s, bias);                                             \
-  }
-    SK_TILE_F8E5M2_BK64_KERNELS(X)
 #undef X
   }
   return launch_tile_asm(id, a, p, ws, s, bias);
@@ -334,60 +238,6 @@ int occupancy_tile(int id) {
     return occ;                                                                                     \
   }
     SK_TILE_BF16_KERNELS(X)
-#undef X
-#define X(id_, BM, BN, WM, WN)                                                                      \
-  case id_: {                                                                                       \
-    typedef SK_POLICY_F8(id_, BM, BN, WM, WN) P;                                                    \
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_tile_kernel<P>, P::NT, 0) != hipSuccess) \
-      return -1;                                                                                    \
-    return occ;                                                                                     \
-  }
-    SK_TILE_F8_KERNELS(X)
-#undef X
-#define X(id_, BM, BN, WM, WN)                                                                      \
-  case id_: {                                                                                       \
-    typedef SK_POLICY_F8E5M2(id_, BM, BN, WM, WN) P;                                                \
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_tile_kernel<P>, P::NT, 0) != hipSuccess) \
-      return -1;                                                                                    \
-    return occ;                                                                                     \
-  }
-    SK_TILE_F8E5M2_KERNELS(X)
-#undef X
-#define X(id_, BM, BN, WM, WN)                                                                      \
-  case id_: {                                                                                       \
-    typedef SK_POLICY_I8(id_, BM, BN, WM, WN) P;                                                    \
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_tile_kernel<P>, P::NT, 0) != hipSuccess) \
-      return -1;                                                                                    \
-    return occ;                                                                                     \
-  }
-    SK_TILE_I8_KERNELS(X)
-#undef X
-#define X(id_, BM, BN, WM, WN)                                                                      \
-  case id_: {                                                                                       \
-    typedef SK_POLICY_I8_BK64(id_, BM, BN, WM, WN) P;                                               \
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_tile_kernel<P>, P::NT, 0) != hipSuccess) \
-      return -1;                                                                                    \
-    return occ;                                                                                     \
-  }
-    SK_TILE_I8_BK64_KERNELS(X)
-#undef X
-#define X(id_, BM, BN, WM, WN)                                                                      \
-  case id_: {                                                                                       \
-    typedef SK_POLICY_F8_BK64(id_, BM, BN, WM, WN) P;                                               \
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_tile_kernel<P>, P::NT, 0) != hipSuccess) \
-      return -1;                                                                                    \
-    return occ;                                                                                     \
-  }
-    SK_TILE_F8_BK64_KERNELS(X)
-#undef X
-#define X(id_, BM, BN, WM, WN)                                                                      \
-  case id_: {                                                                                       \
-    typedef SK_POLICY_F8E5M2_BK64(id_, BM, BN, WM, WN) P;                                           \
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_tile_kernel<P>, P::NT, 0) != hipSuccess) \
-      return -1;                                                                                    \
-    return occ;                                                                                     \
-  }
-    SK_TILE_F8E5M2_BK64_KERNELS(X)
 #undef X
   }
   return occupancy_tile_asm(id);

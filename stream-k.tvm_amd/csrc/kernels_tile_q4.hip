@@ -41,7 +41,7 @@ int launch_tile_q4(int id, const GemmArgs &a, const DevPlan &p, const Workspace 
     SK_TILE_Q4_KERNELS(X)
 #undef X
   }
-  return (int)hipErrorInvalidValue;
+  return launch_tile_8bit(id, a, p, ws, s, bias);
 }
 
 int occupancy_tile_q4(int id) {
@@ -56,7 +56,7 @@ int occupancy_tile_q4(int id) {
     SK_TILE_Q4_KERNELS(X)
 #undef X
   }
-  return -1;
+  return occupancy_tile_8bit(id);
 }
 
 }  // namespace sk

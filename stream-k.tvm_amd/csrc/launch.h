@@ -32,6 +32,10 @@ int occupancy_tile_asm8(int id);
 int tile_q4_kernel_infos(KernelInfo *out, int max);
 int launch_tile_q4(int id, const GemmArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s, const void *bias);
 int occupancy_tile_q4(int id);
+// tile kernels for one-byte operands (translation unit kernels_tile_8bit.hip)
+int tile_8bit_kernel_infos(KernelInfo *out, int max);
+int launch_tile_8bit(int id, const GemmArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s, const void *bias);
+int occupancy_tile_8bit(int id);
 // 2 <= M <= 16 kernels in the matrix-vector kernels' form, and the Q4 kernels for tiled weights with per-group zero
 // points (translation unit kernels_gemv_rows.hip)
 int gemv_rows_kernel_infos(KernelInfo *out, int max);

@@ -21,12 +21,14 @@ int tile_kernel_infos(KernelInfo *out, int max);
 int tile_asm_kernel_infos(KernelInfo *out, int max);
 int tile_asm8_kernel_infos(KernelInfo *out, int max);
 int tile_q4_kernel_infos(KernelInfo *out, int max);
+int tile_8bit_kernel_infos(KernelInfo *out, int max);
 int skinny_kernel_infos(KernelInfo *out, int max);
 int f32_kernel_infos(KernelInfo *out, int max);
 
 const KernelInfo *kernel_table(int *count) {
   std::call_once(g_table_once, [] {
     int n = tile_kernel_infos(g_table, 400);
+    n += tile_8bit_kernel_infos(g_table + n, 400 - n);
     n += tile_asm_kernel_infos(g_table + n, 400 - n);
     n += tile_asm8_kernel_infos(g_table + n, 400 - n);
     n += tile_q4_kernel_infos(g_table + n, 400 - n);
