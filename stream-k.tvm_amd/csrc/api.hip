@@ -187,7 +187,7 @@ int make_dev_plan(const sk_plan *plan, const KernelInfo *k, void *ws, size_t ws_
   dp->spin_limit = plan->spin_limit > 0 ? plan->spin_limit : (1 << 22);
   // (the interleaved Stream-K order relies on the hardware's round-robin placement: CTAs a multiple of 8 apart
   // share an XCD)
-  dp->xcd_remap = (plan->grid % 8 == 0 && plan->interleave <= 1) ? 1 : 0;
+  dp->xcd_remap = plan->interleave <= 1 ? 1 : 0;
   dp->perm_s = plan->interleave > 1 ? plan->interleave : 1;
   dp->perm_g = plan->interleave > 1 ? plan->streamk_tiles / plan->interleave : 1;
   dp->by_perm = FastDiv::make(dp->perm_s);

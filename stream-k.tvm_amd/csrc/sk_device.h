@@ -88,11 +88,15 @@ struct Workspace {
   float *partials;
 };
 
-// Workgroups are dealt round-robin to the 8 XCDs (each with its own L2).  Giving XCD x the logical
-// ids [x*grid/8, (x+1)*grid/8) makes neighbouring tiles share an L2.
+// Workgroups are dealt round-robin to the 8 XCDs (each with its own L2).  Giving XCD x a contiguous range of
+// logical ids makes neighbouring tiles share an L2: XCD x runs the grid/8 workgroups b = x, x + 8, ... (one more
+// on the first grid % 8 XCDs), and they get the ids from x * (grid / 8) + min(x, grid % 8) on.
 __device__ __forceinline__ int logical_pid(const DevPlan &p) {
-  int b = blockIdx.x;
-  if (p.xcd_remap) return (b & 7) * (p.grid >> 3) + (b >> 3);
+  const int b = blockIdx.x;
+  if (p.xcd_remap) {
+    const int x = b & 7;
+    return x * (p.grid >> 3) + min(x, p.grid & 7) + (b >> 3);
+  }
   return b;
 }
 
