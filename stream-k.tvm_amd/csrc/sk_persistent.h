@@ -27,6 +27,12 @@ template <class P, class = void>
 struct has_atomic_c { static constexpr bool value = false; };
 template <class P>
 struct has_atomic_c<P, std::void_t<decltype(P::ATOMIC_C)>> { static constexpr bool value = P::ATOMIC_C; };
+// CROSS_TILE_PREFETCH: the policy has prefetch_first_stage / epilogue_lds_free and mac takes a last argument that says
+// the first stage of the segment has already been requested (see the loop below)
+template <class P, class = void>
+struct has_prefetch { static constexpr bool value = false; };
+template <class P>
+struct has_prefetch<P, std::void_t<decltype(P::CROSS_TILE_PREFETCH)>> { static constexpr bool value = P::CROSS_TILE_PREFETCH; };
 template <class P, class = void>
 struct has_halves { static constexpr bool value = false; };
 template <class P>
@@ -66,6 +72,11 @@ __device__ __forceinline__ void run_persistent(const typename P::Args &a, const 
   // One loop body serves both phases so that the MAC loop and the epilogue exist once in the
   // kernel: first the CTA's Stream-K segments, then its data-parallel tiles
   // (tile = streamk_tiles + pid + wave * grid, streamk_fp32.py:149-158).
+  // Policies with CROSS_TILE_PREFETCH: once every wave has left the MAC loop the LDS stages are free, and where the
+  // epilogue of this tile will not use them (stores straight from registers) the loads of the next segment's first
+  // stage go out before the fix-up and the epilogue instead of after them: a tile costs the 256 x 256 kernels about
+  // 13 000 cycles outside its loop, most of them the epilogue and the first loads' trip to memory, one after the other.
+  bool first_stage_requested = false;
   for (;;) {
     int tile, k0, n;
     if (start < last) {
@@ -84,7 +95,27 @@ __device__ __forceinline__ void run_persistent(const typename P::Args &a, const 
     int pm, pn;
     tile_coords(plan, tile, pm, pn);
     SK_TRACE(11);
-    P::mac(a, acc, pm, pn, k0, n, smem);
+    if constexpr (has_prefetch<P>::value) {
+      P::mac(a, acc, pm, pn, k0, n, smem, first_stage_requested);
+      first_stage_requested = false;
+      // the segment after this one (start and dp_tile already point behind the current one)
+      int next_tile = -1, next_k0 = 0, next_n = ipt;
+      if (start < last) {
+        next_tile = plan.by_ipt.div(start);
+        next_k0 = start - next_tile * ipt;
+        next_n = min(ipt - next_k0, last - start);
+      } else if (dp_tile < plan.total_tiles) {
+        next_tile = dp_tile;
+      }
+      if (next_tile >= 0 && P::epilogue_lds_free(a, pn, bias)) {
+        int npm, npn;
+        tile_coords(plan, next_tile, npm, npn);
+        P::prefetch_first_stage(a, npm, npn, next_k0, next_n);
+        first_stage_requested = true;
+      }
+    } else {
+      P::mac(a, acc, pm, pn, k0, n, smem);
+    }
 
     // a segment that is the whole tile is simply stored (streamk_fp32.py:128-129)
     bool store = (n == ipt) || !FIXUP;

@@ -61,11 +61,13 @@ struct TileF16Asm {
   static constexpr int BM = 256, BN = 256, BK = 64, WM = 2, WN = 2, NW = 4, NT = 256;
   static constexpr int WTM = 128, WTN = 128, FM = 8, FN = 8;  // wave tile; 16 x 16 accumulator blocks per wave
   static constexpr int ROW_BYTES = 128, A_BYTES = BM * ROW_BYTES, STAGE_BYTES = 2 * A_BYTES;
-  static constexpr int LDS_TOTAL = 2 * STAGE_BYTES, LDS_BYTES = 16;
+  // behind the two stages: one patch of 16 rows x 272 bytes per wave for the epilogue that leaves the stages alone
+  static constexpr int PATCH_STRIDE = 272, FAST_PATCH_BYTES = 16 * PATCH_STRIDE;
+  static constexpr int LDS_TOTAL = 2 * STAGE_BYTES + NW * FAST_PATCH_BYTES, LDS_BYTES = 16;
   static constexpr int TILE_ELEMS = BM * BN, NV4 = FM * FN;
   static constexpr int CTAS_PER_CU = 1, WAVES_PER_EU = 1;
   static constexpr int LDC = WTN + 8, PATCH_ROWS = 64;  // epilogue patch: 64 rows x 136 halfs per wave and pass
-  static_assert(PATCH_ROWS * LDC * 2 <= LDS_TOTAL / NW, "epilogue patches must fit the stages");
+  static_assert(PATCH_ROWS * LDC * 2 <= 2 * STAGE_BYTES / NW, "epilogue patches must fit the stages");
 
   struct Acc {};  // the accumulators live in a[0:255]: block (i, j) in a[(8 i + j) 4 .. + 3]
 
@@ -74,57 +76,116 @@ struct TileF16Asm {
     return buf;
   }
 
-  static __device__ __forceinline__ void mac(const Args &a, Acc &, int pm, int pn, int k0, int n, char *) {
+  // Everything the loads and the loop of one segment need: descriptors, lane offsets, wave-uniform global offsets
+  // (iteration k0 of tile (pm, pn)), LDS addresses.
+  struct Ctx {
+    uint4v rsrc_a, rsrc_b;
+    uint32_t voff_a, voff_b, voff_b1;  // voff_b1: NN only (odd row groups of B)
+    uint32_t goff_a, goff_b, gstep_a, gstep_b, kstep_b;  // kstep_b: bytes B advances per iteration
+    uint32_t lds_wave;
+    uint32_t ra0, ra1, rb0, rb1, rbt[8];  // fragment addresses (rbt: NN)
+  };
+  static __device__ __forceinline__ Ctx make_ctx(const Args &a, int pm, int pn, int k0) {
+    Ctx c;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
     const int rows_a = min(BM, a.M - pm * BM), rows_b = min(BN, a.N - pn * BN);
     // rows past the matrix edge lie beyond the descriptors' ranges and read as zero
-    const uint4v rsrc_a = make_rsrc_words(a.A + (int64_t)pm * BM * a.lda, (uint32_t)(rows_a * a.lda * 2));
-    const uint4v rsrc_b = make_rsrc_words(a.B + (int64_t)pn * BN * a.ldb, (uint32_t)(rows_b * a.ldb * 2));
+    c.rsrc_a = make_rsrc_words(a.A + (int64_t)pm * BM * a.lda, (uint32_t)(rows_a * a.lda * 2));
     // a wave-wide load fills 8 LDS rows; lane l writes (row l / 8, position l % 8) and therefore fetches
     // chunk (l % 8) ^ swizzle(row); a wave only loads row groups of its own parity (see tile_f16_dma.h)
     const int my_chunk = (lane & 7) ^ (((wave & 1) << 2) | (lane >> 4)), my_row = lane >> 3;
-    const uint32_t voff_a = (uint32_t)(my_row * a.lda + my_chunk * 8) * 2;
-    const uint32_t voff_b = (uint32_t)(my_row * a.ldb + my_chunk * 8) * 2;
+    c.voff_a = (uint32_t)(my_row * a.lda + my_chunk * 8) * 2;
     // row group g = wave + 4 x of a stage: rows 8 g .. 8 g + 7, at wave-uniform byte offset 16 g ld
-    const uint32_t goff_a = (uint32_t)k0 * (BK * 2) + (uint32_t)(wave * 16 * a.lda), gstep_a = (uint32_t)(64 * a.lda);
-    const uint32_t goff_b = (uint32_t)k0 * (BK * 2) + (uint32_t)(wave * 16 * a.ldb), gstep_b = (uint32_t)(64 * a.ldb);
+    c.goff_a = (uint32_t)k0 * (BK * 2) + (uint32_t)(wave * 16 * a.lda);
+    c.gstep_a = (uint32_t)(64 * a.lda);
     const uint32_t base = lds_address(lds());
-    const uint32_t lds_wave = base + wave * 1024;
+    c.lds_wave = base + wave * 1024;
     // fragments: lane (r = l % 16, g = l / 16) reads row r of a 16-row block, chunk 4 kk + g at position
     // (4 kk + g) ^ ((r >> 1) & 7); K-step 1 is K-step 0 with address bit 6 flipped
     const uint32_t pos0 = (uint32_t)((lane >> 4) ^ ((lane >> 1) & 7)) * 16;
-    uint32_t ra0 = base + (uint32_t)(wm * WTM + (lane & 15)) * ROW_BYTES + pos0, ra1 = ra0 ^ 64;
-    uint32_t rb0 = base + A_BYTES + (uint32_t)(wn * WTN + (lane & 15)) * ROW_BYTES + pos0, rb1 = rb0 ^ 64;
-    const uint32_t iters = (uint32_t)n;
+    c.ra0 = base + (uint32_t)(wm * WTM + (lane & 15)) * ROW_BYTES + pos0;
+    c.ra1 = c.ra0 ^ 64;
     if constexpr (NN_) {
       // B: the descriptor starts at the tile's first column and ends with the last valid element of row K - 1;
       // columns past N are masked per lane (N is a multiple of 8).  A wave-wide load fills K-rows 2 g, 2 g + 1 of
       // the stage (g = wave + 4 x): lane l writes position l % 32 of row 2 g + l / 32 and therefore fetches chunk
       // (l % 32) ^ swizzle(row); bit 3 of the row is the parity of x, hence two offsets.
-      const uint4v rsrc_bn = make_rsrc_words(a.B + (int64_t)pn * BN, (uint32_t)(((int64_t)(a.K - 1) * a.ldb + rows_b) * 2));
+      c.rsrc_b = make_rsrc_words(a.B + (int64_t)pn * BN, (uint32_t)(((int64_t)(a.K - 1) * a.ldb + rows_b) * 2));
       const int row_in = lane >> 5, k_bits = 2 * wave + row_in;
       const int chunk0 = (lane & 31) ^ (4 * (k_bits & 3)), chunk1 = chunk0 ^ 2;
-      const uint32_t vob0 = chunk0 * 8 < rows_b ? (uint32_t)(row_in * a.ldb + chunk0 * 8) * 2 : OOB_OFFSET;
-      const uint32_t vob1 = chunk1 * 8 < rows_b ? (uint32_t)(row_in * a.ldb + chunk1 * 8) * 2 : OOB_OFFSET;
-      const uint32_t kstep_bn = (uint32_t)(128 * a.ldb);  // 64 K-rows
-      const uint32_t goff_bn = (uint32_t)k0 * kstep_bn + (uint32_t)(wave * 4 * a.ldb), gstep_bn = (uint32_t)(16 * a.ldb);
+      c.voff_b = chunk0 * 8 < rows_b ? (uint32_t)(row_in * a.ldb + chunk0 * 8) * 2 : OOB_OFFSET;
+      c.voff_b1 = chunk1 * 8 < rows_b ? (uint32_t)(row_in * a.ldb + chunk1 * 8) * 2 : OOB_OFFSET;
+      c.kstep_b = (uint32_t)(128 * a.ldb);  // 64 K-rows
+      c.goff_b = (uint32_t)k0 * c.kstep_b + (uint32_t)(wave * 4 * a.ldb);
+      c.gstep_b = (uint32_t)(16 * a.ldb);
       // fragments of B: lane group g' = l / 16 reads K-rows 8 g' .. 8 g' + 7 of a 16-column block, four rows per
       // transposing read; block j's address differs from block 0's by an XOR (the swizzle), so each has its own
       const int k_lane = 8 * (lane >> 4) + ((lane & 15) >> 2);
       const int swz = (4 * (k_lane & 3)) ^ (2 * ((k_lane >> 3) & 1));
-      uint32_t rbt[FN];
 #pragma unroll
       for (int j = 0; j < FN; ++j) {
         const int col = wn * WTN + j * 16 + 4 * (lane & 3);
-        rbt[j] = base + A_BYTES + (uint32_t)(k_lane * 512 + (((col >> 3) ^ swz) * 16) + (col & 7) * 2);
+        c.rbt[j] = base + A_BYTES + (uint32_t)(k_lane * 512 + (((col >> 3) ^ swz) * 16) + (col & 7) * 2);
       }
+      c.rb0 = c.rb1 = 0;
+    } else {
+      c.rsrc_b = make_rsrc_words(a.B + (int64_t)pn * BN * a.ldb, (uint32_t)(rows_b * a.ldb * 2));
+      c.voff_b = (uint32_t)(my_row * a.ldb + my_chunk * 8) * 2;
+      c.voff_b1 = 0;
+      c.kstep_b = 128;
+      c.goff_b = (uint32_t)k0 * (BK * 2) + (uint32_t)(wave * 16 * a.ldb);
+      c.gstep_b = (uint32_t)(64 * a.ldb);
+      c.rb0 = base + A_BYTES + (uint32_t)(wn * WTN + (lane & 15)) * ROW_BYTES + pos0;
+      c.rb1 = c.rb0 ^ 64;
+    }
+    return c;
+  }
+
+  // the 16 loads of stage `stage` (iteration k0 + stage of the segment; nothing is fetched if the segment is shorter)
+  static __device__ __forceinline__ void stage_loads(const Ctx &c, int stage, int n) {
+    const uint32_t oob = stage < n ? 0u : OOB_OFFSET;
+    const uint32_t voa = c.voff_a | oob, vob = c.voff_b | oob, vob1 = c.voff_b1 | oob;
+    const uint32_t ga = c.goff_a + (uint32_t)stage * 128, gb = c.goff_b + (uint32_t)stage * c.kstep_b;
+    const uint32_t lds_stage = c.lds_wave + (uint32_t)stage * STAGE_BYTES;
+    if constexpr (NN_) {
+      asm volatile(SK_TILE_ASM_LOADS_NN
+                   :
+                   : [rsa] "s"(c.rsrc_a), [rsb] "s"(c.rsrc_b), [voa] "v"(voa), [vob] "v"(vob), [vob1] "v"(vob1), [ga] "s"(ga),
+                     [gb] "s"(gb), [gas] "s"(c.gstep_a), [gbs] "s"(c.gstep_b), [lds] "s"(lds_stage)
+                   : "memory", "m0", "scc", "s83");
+    } else {
+      asm volatile(SK_TILE_ASM_LOADS
+                   :
+                   : [rsa] "s"(c.rsrc_a), [rsb] "s"(c.rsrc_b), [voa] "v"(voa), [vob] "v"(vob), [ga] "s"(ga), [gb] "s"(gb),
+                     [gas] "s"(c.gstep_a), [gbs] "s"(c.gstep_b), [lds] "s"(lds_stage)
+                   : "memory", "m0", "scc", "s83");
+    }
+  }
+
+  // Cross-segment prefetch (see run_persistent): the first stage of the NEXT segment is requested as soon as every
+  // wave has left the loop of the current one, ahead of an epilogue that does not use LDS, and mac() is then told
+  // that the stage is on its way.
+  static constexpr bool CROSS_TILE_PREFETCH = true;
+  static __device__ __forceinline__ void prefetch_first_stage(const Args &a, int pm, int pn, int k0, int n) {
+    const Ctx c = make_ctx(a, pm, pn, k0);
+    stage_loads(c, 0, n);
+  }
+
+  static __device__ __forceinline__ void mac(const Args &a, Acc &, int pm, int pn, int k0, int n, char *,
+                                             bool first_stage_requested = false) {
+    Ctx c = make_ctx(a, pm, pn, k0);
+    if (!first_stage_requested) stage_loads(c, 0, n);
+    stage_loads(c, 1, n);  // (directly ahead of the loop, whose first wait counts on these being the 16 youngest operations)
+    const uint32_t iters = (uint32_t)n;
+    if constexpr (NN_) {
 #define SK_ASM_NN_OPERANDS                                                                                            \
-  : [ra0] "+v"(ra0), [ra1] "+v"(ra1), [rbt0] "+v"(rbt[0]), [rbt1] "+v"(rbt[1]), [rbt2] "+v"(rbt[2]),                    \
-    [rbt3] "+v"(rbt[3]), [rbt4] "+v"(rbt[4]), [rbt5] "+v"(rbt[5]), [rbt6] "+v"(rbt[6]), [rbt7] "+v"(rbt[7])            \
-  : [rsa] "s"(rsrc_a), [rsb] "s"(rsrc_bn), [voa] "v"(voff_a), [vob] "v"(vob0), [vob1] "v"(vob1), [ga0] "s"(goff_a),     \
-    [gb0] "s"(goff_bn), [gas] "s"(gstep_a), [gbs] "s"(gstep_bn), [kbs] "s"(kstep_bn), [n] "s"(iters), [lds] "s"(lds_wave) \
+  : [ra0] "+v"(c.ra0), [ra1] "+v"(c.ra1), [rbt0] "+v"(c.rbt[0]), [rbt1] "+v"(c.rbt[1]), [rbt2] "+v"(c.rbt[2]),          \
+    [rbt3] "+v"(c.rbt[3]), [rbt4] "+v"(c.rbt[4]), [rbt5] "+v"(c.rbt[5]), [rbt6] "+v"(c.rbt[6]), [rbt7] "+v"(c.rbt[7])  \
+  : [rsa] "s"(c.rsrc_a), [rsb] "s"(c.rsrc_b), [voa] "v"(c.voff_a), [vob] "v"(c.voff_b), [vob1] "v"(c.voff_b1),          \
+    [ga0] "s"(c.goff_a), [gb0] "s"(c.goff_b), [gas] "s"(c.gstep_a), [gbs] "s"(c.gstep_b), [kbs] "s"(c.kstep_b),         \
+    [n] "s"(iters), [lds] "s"(c.lds_wave)                                                                             \
   : "memory", "m0", "scc", SK_TILE_ASM_CLOBBERS
       if constexpr (BF16_) {
         asm volatile(SK_TILE_ASM_LOOP_NN("v_mfma_f32_16x16x32_bf16") SK_ASM_NN_OPERANDS);
@@ -132,50 +193,95 @@ struct TileF16Asm {
         asm volatile(SK_TILE_ASM_LOOP_NN("v_mfma_f32_16x16x32_f16") SK_ASM_NN_OPERANDS);
       }
 #undef SK_ASM_NN_OPERANDS
-    } else if constexpr (F8 != 0) {
-#define SK_ASM_NT_OPERANDS                                                                                         \
-  : [ra0] "+v"(ra0), [ra1] "+v"(ra1), [rb0] "+v"(rb0), [rb1] "+v"(rb1)                                             \
-  : [rsa] "s"(rsrc_a), [rsb] "s"(rsrc_b), [voa] "v"(voff_a), [vob] "v"(voff_b), [ga0] "s"(goff_a), [gb0] "s"(goff_b), \
-    [gas] "s"(gstep_a), [gbs] "s"(gstep_b), [n] "s"(iters), [lds] "s"(lds_wave)                                    \
+    } else {
+#define SK_ASM_NT_OPERANDS                                                                                          \
+  : [ra0] "+v"(c.ra0), [ra1] "+v"(c.ra1), [rb0] "+v"(c.rb0), [rb1] "+v"(c.rb1)                                      \
+  : [rsa] "s"(c.rsrc_a), [rsb] "s"(c.rsrc_b), [voa] "v"(c.voff_a), [vob] "v"(c.voff_b), [ga0] "s"(c.goff_a),          \
+    [gb0] "s"(c.goff_b), [gas] "s"(c.gstep_a), [gbs] "s"(c.gstep_b), [n] "s"(iters), [lds] "s"(c.lds_wave)            \
   : "memory", "m0", "scc", SK_TILE_ASM_CLOBBERS
       if constexpr (F8 == 1) {
         asm volatile(SK_TILE_ASM_LOOP_F8("v_mfma_f32_16x16x128_f8f6f4", "") SK_ASM_NT_OPERANDS);
-      } else {
+      } else if constexpr (F8 == 2) {
         asm volatile(SK_TILE_ASM_LOOP_F8("v_mfma_f32_16x16x128_f8f6f4", "cbsz:1 blgp:1") SK_ASM_NT_OPERANDS);
+      } else if constexpr (I8) {
+        asm volatile(SK_TILE_ASM_LOOP("v_mfma_i32_16x16x64_i8") SK_ASM_NT_OPERANDS);
+      } else if constexpr (BF16_) {
+        asm volatile(SK_TILE_ASM_LOOP("v_mfma_f32_16x16x32_bf16") SK_ASM_NT_OPERANDS);
+      } else {
+        asm volatile(SK_TILE_ASM_LOOP("v_mfma_f32_16x16x32_f16") SK_ASM_NT_OPERANDS);
       }
 #undef SK_ASM_NT_OPERANDS
-    } else if constexpr (I8) {
-      asm volatile(SK_TILE_ASM_LOOP("v_mfma_i32_16x16x64_i8")
-                   : [ra0] "+v"(ra0), [ra1] "+v"(ra1), [rb0] "+v"(rb0), [rb1] "+v"(rb1)
-                   : [rsa] "s"(rsrc_a), [rsb] "s"(rsrc_b), [voa] "v"(voff_a), [vob] "v"(voff_b), [ga0] "s"(goff_a),
-                     [gb0] "s"(goff_b), [gas] "s"(gstep_a), [gbs] "s"(gstep_b), [n] "s"(iters), [lds] "s"(lds_wave)
-                   : "memory", "m0", "scc", SK_TILE_ASM_CLOBBERS);
-    } else if constexpr (BF16_) {
-      asm volatile(SK_TILE_ASM_LOOP("v_mfma_f32_16x16x32_bf16")
-                   : [ra0] "+v"(ra0), [ra1] "+v"(ra1), [rb0] "+v"(rb0), [rb1] "+v"(rb1)
-                   : [rsa] "s"(rsrc_a), [rsb] "s"(rsrc_b), [voa] "v"(voff_a), [vob] "v"(voff_b), [ga0] "s"(goff_a),
-                     [gb0] "s"(goff_b), [gas] "s"(gstep_a), [gbs] "s"(gstep_b), [n] "s"(iters), [lds] "s"(lds_wave)
-                   : "memory", "m0", "scc", SK_TILE_ASM_CLOBBERS);
-    } else {
-      asm volatile(SK_TILE_ASM_LOOP("v_mfma_f32_16x16x32_f16")
-                   : [ra0] "+v"(ra0), [ra1] "+v"(ra1), [rb0] "+v"(rb0), [rb1] "+v"(rb1)
-                   : [rsa] "s"(rsrc_a), [rsb] "s"(rsrc_b), [voa] "v"(voff_a), [vob] "v"(voff_b), [ga0] "s"(goff_a),
-                     [gb0] "s"(goff_b), [gas] "s"(gstep_a), [gbs] "s"(gstep_b), [n] "s"(iters), [lds] "s"(lds_wave)
-                   : "memory", "m0", "scc", SK_TILE_ASM_CLOBBERS);
     }
-    __syncthreads();  // both stages are free for the epilogue / the next segment
+    // every wave has left the loop and its own loads have landed: both stages are free (for the epilogue's patches,
+    // for the loads of the next segment)
+    __syncthreads();
+  }
+
+  // ---- epilogue that leaves the stages alone (patches of their own behind them; gen_tile_asm.py: store_text) ----
+  // Possible where the tile's 256 columns are inside the matrix and rows of C are 16-byte aligned; rows past M are
+  // dropped by the descriptor's range.  The bias / activation epilogue and tiles on the right edge take the path below.
+  static __device__ __forceinline__ bool direct_store_ok(const Args &a, int pn, const void *bias) {
+    if constexpr (I8) return false;  // (its own register epilogue, below)
+    return bias == nullptr && (pn + 1) * BN <= a.N && (a.ldc & 7) == 0 && (reinterpret_cast<uintptr_t>(a.C) & 15) == 0;
+  }
+  // true if the epilogue of this tile will not touch the stages (the int32 epilogue uses no LDS at all)
+  static __device__ __forceinline__ bool epilogue_lds_free(const Args &a, int pn, const void *bias) {
+    return I8 || direct_store_ok(a, pn, bias);
+  }
+  template <int HALF>
+  static __device__ __forceinline__ void store_c_direct(const Args &a, int pm, int pn) {
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int row0 = pm * BM + wm * WTM, col0 = pn * BN + wn * WTN;
+    const int rows = max(0, min(WTM, a.M - row0));
+    const uint32_t bytes = rows > 0 ? (uint32_t)(((int64_t)(rows - 1) * a.ldc + WTN) * 2) : 0u;
+    const uint4v words = make_rsrc_words(a.C + (int64_t)row0 * a.ldc + col0, bytes);
+    // (the descriptor depends on the wave: make the compiler keep it in scalar registers)
+    const uint4v rsrc_c = {(uint32_t)__builtin_amdgcn_readfirstlane((int)words[0]), (uint32_t)__builtin_amdgcn_readfirstlane((int)words[1]),
+                           (uint32_t)__builtin_amdgcn_readfirstlane((int)words[2]), words[3]};
+    const uint32_t patch = lds_address(lds()) + 2 * STAGE_BYTES + (uint32_t)wave * FAST_PATCH_BYTES;
+    const uint32_t wr = patch + (uint32_t)((lane & 15) * PATCH_STRIDE + (lane >> 4) * 8);
+    const uint32_t rd = patch + (uint32_t)((lane >> 4) * PATCH_STRIDE + (lane & 15) * 16);
+    const uint32_t voff = (uint32_t)((lane >> 4) * a.ldc + (lane & 15) * 8) * 2;
+    const uint32_t rowstep = (uint32_t)(16 * a.ldc * 2), q1 = (uint32_t)(4 * a.ldc * 2);
+#define SK_ASM_STORE_OPERANDS                                                                                        \
+  : : [rsc] "s"(rsrc_c), [voff] "v"(voff), [wr] "v"(wr), [rd] "v"(rd), [rowstep] "s"(rowstep), [q1] "s"(q1),         \
+      [alpha] "s"(a.alpha) : "memory", "scc", SK_TILE_ASM_CLOBBERS
+#define SK_ASM_STORE(WHICH)                                                                            \
+  if constexpr (F8 != 0) {                                                                             \
+    asm volatile(SK_TILE_ASM_STORE_##WHICH##_SCALED("v_cvt_pk_f16_f32") SK_ASM_STORE_OPERANDS);        \
+  } else if constexpr (BF16_) {                                                                        \
+    asm volatile(SK_TILE_ASM_STORE_##WHICH("v_cvt_pk_bf16_f32") SK_ASM_STORE_OPERANDS);                \
+  } else {                                                                                             \
+    asm volatile(SK_TILE_ASM_STORE_##WHICH("v_cvt_pk_f16_f32") SK_ASM_STORE_OPERANDS);                 \
+  }
+    if constexpr (HALF < 0) {
+      SK_ASM_STORE(ALL)
+    } else if constexpr (HALF == 0) {
+      SK_ASM_STORE(HALF0)
+    } else {
+      SK_ASM_STORE(HALF1)
+    }
+#undef SK_ASM_STORE
+#undef SK_ASM_STORE_OPERANDS
   }
 
   // ---- epilogue: fp32 -> C's type through a per-wave LDS patch, 16-byte stores of whole rows ----
   static __device__ __forceinline__ void store_c(const Args &a, const Acc &, int pm, int pn, char *, const void *bias) {
-    if (bias == nullptr)
+    if (direct_store_ok(a, pn, bias))
+      store_c_direct<-1>(a, pm, pn);
+    else if (bias == nullptr)
       store_c_impl<false, -1>(a, pm, pn, nullptr);
     else
       store_c_impl<true, -1>(a, pm, pn, bias);
   }
   static __device__ __forceinline__ void store_c_half(const Args &a, const Acc &, int pm, int pn, char *,
                                                       const void *bias, int h) {
-    if (bias == nullptr) {
+    if (direct_store_ok(a, pn, bias)) {
+      if (h == 0) store_c_direct<0>(a, pm, pn);
+      else store_c_direct<1>(a, pm, pn);
+    } else if (bias == nullptr) {
       if (h == 0) store_c_impl<false, 0>(a, pm, pn, nullptr);
       else store_c_impl<false, 1>(a, pm, pn, nullptr);
     } else {
@@ -216,7 +322,7 @@ struct TileF16Asm {
       return;
     }
     const int bias_col0 = BIAS ? pn * BN + wn * WTN + pin_here(lane >> 4) * 4 : 0;
-    half_t *patch = reinterpret_cast<half_t *>(lds() + wave * (LDS_TOTAL / NW));
+    half_t *patch = reinterpret_cast<half_t *>(lds() + wave * (2 * STAGE_BYTES / NW));
     const bool vec_ok = (a.ldc % 8 == 0) && ((reinterpret_cast<uintptr_t>(a.C) & 15) == 0);
     constexpr int CPRC = WTN / 8;
     static_for<0, NPASS>([&](auto pass) {
