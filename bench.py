@@ -1,6 +1,8 @@
 """Benchmark of the Stream-K GEMM hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extra] [--no-cpu]
+    python bench.py --case MxNxK [--dtype D] [--layout nt|nn] [--config "dict(...)"] [--data rand|zeros|ones]
+                    [--reps R] [--time] [--vendor]       one GEMM case on its own, for a profiler
 
 One "step" is one fp16 GEMM call through the C ABI on inputs already resident in HBM.  The headline
 workload is M = N = K = 8192 (NT layout, U[-1,1) from seed 0), the compute-bound end of the
@@ -8,9 +10,12 @@ metric's sweep; `value` is whole-job TFLOP/s over exactly `steps` timed calls.  
 carries
   roofline      the dominant kernel's achieved rate from HIP events on the launch stream,
   cpu_baseline  the oracle's fp32 host matmul timed on this box's cores on a bounded sample,
-  extra         the rest of the metric: M sweep at N = K = 8192 (Stream-K vs data-parallel-only
-                schedule of the same kernel), 1024x1024x8192 with both fix-ups, Q4 GEMM GB/s at
-                M = 1 / 16 (kernels this short are timed as graph-captured batches).
+  config.metric_parts   the other two parts of the metric in short: Stream-K against the data-parallel schedule at
+                M = 256 / 512 / 1024 (same tile, and the best data-parallel tile), Q4 GEMM at M = 1 / 16 as a
+                fraction of HBM peak with the weights in the Infinity Cache and from HBM,
+  extra         the measurements behind them and the rest: M sweep at N = K = 8192, 1024x1024x8192 with all
+                fix-ups, the large dense shapes in both layouts and types, the reference's own run shapes
+                (kernels this short are timed as graph-captured batches).
 The oracle is used here as the timed CPU baseline and as a result check only.
 """
 import argparse
@@ -79,6 +84,72 @@ def planner_sweep(torch, streamk, time_graph):
     print(json.dumps({"planner_sweep": out}))
 
 
+def run_case(args):
+    """One GEMM case a few times, so that a profiler sees nothing else (--case).  --data chooses the operand values
+    (the clock the part sustains depends on how many bits toggle); --time prints the average time of --reps launches;
+    --vendor also times the vendor GEMM torch calls (hipBLASLt) on the same operands."""
+    import torch
+    import streamk
+    M, N, K = (int(x) for x in args.case.split("x"))
+    cfg = eval(args.config, {"dict": dict})  # noqa: S307 (developer option)
+    g = torch.Generator(device="cpu").manual_seed(0)
+    plan = streamk.make_plan(M, N, K, args.dtype, args.layout, cfg)
+    vendor = None
+    if args.dtype == "q4":
+        A = torch.randn(M, K, generator=g).half().cuda()
+        Wq = torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8).cuda()
+        sc = (torch.rand(N, K // 128, generator=g) * 0.015 + 0.005).half().cuda()
+        run = lambda: streamk.streamk_q4(A, Wq, sc, plan=plan)  # noqa: E731
+    elif args.dtype == "int8":
+        if args.data == "rand":
+            A = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int8).cuda()
+            B = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int8).cuda()
+        else:
+            fill = torch.zeros if args.data == "zeros" else torch.ones
+            A, B = fill(M, K, dtype=torch.int8, device="cuda"), fill(N, K, dtype=torch.int8, device="cuda")
+        C = torch.empty(M, N, dtype=torch.int32, device="cuda")
+        run = lambda: streamk.streamk_int8(A, B, out=C, plan=plan)  # noqa: E731
+        vendor = ("torch._int_mm", lambda: torch._int_mm(A, B.T))
+    elif args.dtype == "float8_e4m3":
+        f8 = torch.float8_e4m3fn
+        if args.data == "rand":
+            A = (torch.rand(M, K, generator=g) * 2 - 1).cuda().to(f8)
+            B = (torch.rand(N, K, generator=g) * 2 - 1).cuda().to(f8)
+        else:
+            fill = torch.zeros if args.data == "zeros" else torch.ones
+            A, B = fill(M, K, device="cuda").to(f8), fill(N, K, device="cuda").to(f8)
+        C = torch.empty(M, N, dtype=torch.float16, device="cuda")
+        one = torch.ones(1, device="cuda")
+        run = lambda: streamk.streamk_fp8(A, B, out=C, plan=plan)  # noqa: E731
+        vendor = ("torch._scaled_mm", lambda: torch._scaled_mm(A, B.T, scale_a=one, scale_b=one, out_dtype=torch.float16))
+    else:
+        dt = {"float16": torch.float16, "bfloat16": torch.bfloat16}.get(args.dtype, torch.float32)
+        bshape = (N, K) if args.layout == "nt" else (K, N)
+        if args.data == "rand":
+            A = (torch.rand(M, K, generator=g) * 2 - 1).to(dt).cuda()
+            B = (torch.rand(*bshape, generator=g) * 2 - 1).to(dt).cuda()
+        else:
+            fill = torch.zeros if args.data == "zeros" else torch.ones
+            A, B = fill(M, K, dtype=dt, device="cuda"), fill(*bshape, dtype=dt, device="cuda")
+        C = torch.empty(M, N, dtype=dt, device="cuda")
+        fn = {"float16": streamk.streamk_fp16, "bfloat16": streamk.streamk_bf16}.get(args.dtype, streamk.streamk_fp32)
+        run = lambda: fn(A, B, layout=args.layout, out=C, plan=plan)  # noqa: E731
+        Bt = B.T if args.layout == "nt" else B
+        vendor = ("torch.matmul", lambda: torch.matmul(A, Bt, out=C))
+    for _ in range(args.reps):
+        run()
+    torch.cuda.synchronize()
+    streamk.workspace_status()
+    if args.time:
+        ms = streamk.bench_ms(run, 3, args.reps)
+        print(f"{args.data}: {ms * 1e3:.2f} us, {2.0 * M * N * K / ms / 1e9:.0f} TFLOP/s")
+    if args.vendor and vendor is not None:
+        ms = streamk.bench_ms(vendor[1], 3, args.reps)
+        print(f"{args.data}: {vendor[0]} {ms * 1e3:.2f} us, {2.0 * M * N * K / ms / 1e9:.0f} TFLOP/s")
+    print(f"ran {args.reps} x {args.dtype} {args.layout} {M}x{N}x{K} kernel {streamk.kernel_name(plan.kernel_id)} grid {plan.grid} "
+          f"streamk_tiles {plan.streamk_tiles}")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -89,6 +160,14 @@ def main():
     ap.add_argument("--planner-sweep", action="store_true",
                     help="instead of the benchmark: time the planner's own choice (no tuned cache) against the vendor "
                          "GEMM on a grid of shapes, per operand type and layout; one JSON line")
+    ap.add_argument("--case", default=None, metavar="MxNxK", help="instead of the benchmark: run this one GEMM --reps times")
+    ap.add_argument("--dtype", default="float16", choices=["float16", "bfloat16", "float32", "q4", "float8_e4m3", "int8"])
+    ap.add_argument("--layout", default="nt", choices=["nt", "nn"])
+    ap.add_argument("--config", default="{}", help="--case: python dict of plan options, e.g. \"dict(bm=256,bn=256,raster=8)\"")
+    ap.add_argument("--reps", type=int, default=5)
+    ap.add_argument("--data", default="rand", choices=["rand", "zeros", "ones"])
+    ap.add_argument("--time", action="store_true", help="--case: print the average time of the launches")
+    ap.add_argument("--vendor", action="store_true", help="--case: also run (and with --time, time) the vendor GEMM")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a 1 GiB device-to-device copy (reference point for rocprofv3 byte counters)")
     args = ap.parse_args()
@@ -137,6 +216,9 @@ def main():
     if args.planner_sweep:
         planner_sweep(torch, streamk, time_graph)
         return
+    if args.case:
+        run_case(args)
+        return
 
     if args.copy_calibration:
         src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").fill_(1)
@@ -174,13 +256,16 @@ def main():
     # untimed, then ~40 ms timed.  The published peak assumes the maximum clock; this is the part's own ceiling.
     def mfma_only(shape):
         import ctypes
-        L = streamk.lib()
+        # (bench.py's own helper, built beside the library by the same Makefile; not part of the product's C ABI)
+        L = ctypes.CDLL(os.path.join(os.path.dirname(streamk._lib.LIB_PATH), "libstreamk_bench.so"))
+        L.skb_mfma_only.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p,
+                                    ctypes.POINTER(ctypes.c_double)]
         scratch = torch.empty(cus * 256, dtype=torch.float32, device="cuda")
         flop = ctypes.c_double(0.0)
         stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
         iters = 4000  # ~2.5 ms per launch
         def launch():
-            rc = L.sk_diag_mfma_only(shape, iters, 0, scratch.data_ptr(), scratch.numel() * 4, stream, ctypes.byref(flop))
+            rc = L.skb_mfma_only(shape, iters, 0, scratch.data_ptr(), scratch.numel() * 4, stream, ctypes.byref(flop))
             assert rc == 0, rc
         for _ in range(16):
             launch()
@@ -208,7 +293,7 @@ def main():
             traffic = json.load(f).get("hbm_bytes_per_launch")
 
     out = {
-        "metric": "fp16 Stream-K GEMM TFLOP/s (M=N=K=8192; sweep and Q4 GB/s in extra)",
+        "metric": "fp16 Stream-K GEMM TFLOP/s (M=N=K=8192; Stream-K / data-parallel ratios and Q4 GB/s in config.metric_parts, sweep in extra)",
         "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(wall_ms, 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f16 (fp32 accumulate)", "data": "synthetic",
@@ -319,12 +404,35 @@ def main():
                 row[name] = round(2.0 * m * N * K / ms / 1e9, 1)
                 if name == "auto":
                     row["auto_weights_from_hbm_us"] = round(ms * 1e3, 2)
+            if m <= 64:
+                # the vendor GEMM on the same rotation of weights
+                def rotating_vendor():
+                    w = copies[turn[0] % len(copies)]
+                    turn[0] += 1
+                    torch.matmul(a, w.T, out=c)
+                turn = [0]
+                row["torch_matmul_weights_from_hbm_us"] = round(time_graph(rotating_vendor) * 1e3, 2)
             copies = None
             if m > 64:
                 for t in tiles:
                     sk_best = max((row.pop(f"{sch}_{t}"), sch) for sch in ("sk2", "basic", "splitk") if f"{sch}_{t}" in row)
                     row["sk_" + t], row["sk_schedule_" + t] = sk_best
-            best = max(v for k, v in row.items() if k not in ("M", "auto_weights_from_hbm_us") and not isinstance(v, str))
+                # the plan the library makes by itself: its tile, and the data-parallel-only schedule of that tile
+                pa = streamk.make_plan(m, N, K, "float16", "nt")
+                key = {(bm, bn): t for t, (bm, bn) in tiles.items()}.get((pa.bm, pa.bn))
+                row["auto_tile"], row["auto_kernel"] = [pa.bm, pa.bn, pa.bk], streamk.kernel_name(pa.kernel_id)
+                row["auto_streamk_tiles"], row["auto_grid"] = pa.streamk_tiles, pa.grid
+                if key is None:
+                    pd = streamk.make_plan(m, N, K, "float16", "nt", bm=pa.bm, bn=pa.bn, bk=pa.bk, schedule="dp", raster=8)
+                    ms = time_graph(lambda: streamk.streamk_fp16(a, B, out=c, plan=pd))
+                    key = f"{pa.bm}x{pa.bn}"
+                    row["dp_" + key] = round(2.0 * m * N * K / ms / 1e9, 1)
+                best_dp = max(v for k, v in row.items() if k.startswith("dp_"))
+                # Stream-K against data-parallel on the tile the library chose, and the library's plan against the best
+                # data-parallel plan of any tile measured
+                row["sk_over_dp_same_tile"] = round(max(row["auto"], row.get("sk_" + key, 0.0)) / row["dp_" + key], 3)
+                row["auto_over_best_dp"] = round(row["auto"] / best_dp, 3)
+            best = max(v for k, v in row.items() if isinstance(v, float) and (k == "auto" or k.startswith(("dp", "sk"))) and not k.endswith("_us") and "over" not in k)
             row["best_tflops"] = best
             row["pct_fp16_peak"] = round(100 * best / PEAK_FP16_TFLOPS, 2)
             nbytes = 2.0 * (m * K + N * K + m * N)
@@ -335,8 +443,6 @@ def main():
                 row["frac_hbm"] = round(row["gbs"] / PEAK_HBM_GBS, 4)
             else:
                 row["gbs_is"] = "algorithmic bytes over time; compute-bound row, operands stay in the Infinity Cache"
-            if m > 64:
-                row["sk_over_dp_same_tile"] = round(max(row["sk_" + t] / row["dp_" + t] for t in tiles), 3)
             sweep.append(row)
         extra["sweep_N8192_K8192_tflops"] = sweep
 
@@ -601,9 +707,85 @@ def main():
             tools[name] = {"us": round(ms * 1e3, 1), "gbs": round(nbytes / ms / 1e6, 1), "frac_hbm": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
         extra["q4_tools_N8192_K8192"] = tools
         del Wf
+        # the reference's own run shapes: fp16 NT 16 x 16384 x 8192 (streamk_fp16.py:61) and Q4 16 x 16384 x 16384
+        # (streamk.fp16.breakdown/streamk_fp16_ladder_block_reduce_q4.py:73 and the autotune scripts), weights from HBM
+        # (the launches of a batch rotate over copies); beside them the vendor GEMM on fp16 weights
+        ref_rows = []
+        m, n, k = 16, 16384, 8192
+        a16 = (torch.rand(m, k, generator=g) * 2 - 1).half().cuda()
+        ws16 = [(torch.rand(n, k, generator=g) * 2 - 1).half().cuda() for _ in range(3)]
+        c16 = torch.empty(m, n, dtype=torch.float16, device="cuda")
+        p16 = streamk.make_plan(m, n, k, "float16", "nt")
+        turn = [0]
+
+        def ref_fp16():
+            turn[0] += 1
+            streamk.streamk_fp16(a16, ws16[turn[0] % 3], out=c16, plan=p16)
+
+        def ref_fp16_vendor():
+            turn[0] += 1
+            torch.matmul(a16, ws16[turn[0] % 3].T, out=c16)
+        nbytes = 2 * (m * k + n * k + m * n)
+        ms, ms_t = time_graph(ref_fp16, launches=6), time_graph(ref_fp16_vendor, launches=6)
+        ref_rows.append({"shape": [m, n, k], "dtype": "float16 NT", "kernel": streamk.kernel_name(p16.kernel_id), "us": round(ms * 1e3, 1),
+                         "gbs": round(nbytes / ms / 1e6, 1), "frac_hbm": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4),
+                         "torch_matmul_us": round(ms_t * 1e3, 1)})
+        del ws16
+        m, n, k = 16, 16384, 16384
+        aq = torch.randn(m, k, generator=g).half().cuda()
+        wqs = [(torch.randint(0, 256, (n, k // 2), generator=g, dtype=torch.uint8).cuda(),
+                (torch.rand(n, k // 128, generator=g) * 0.015 + 0.005).half().cuda()) for _ in range(4)]
+        cq = torch.empty(m, n, dtype=torch.float16, device="cuda")
+        pq = streamk.make_plan(m, n, k, "q4", "nt")
+
+        def ref_q4():
+            turn[0] += 1
+            w, s_ = wqs[turn[0] % 4]
+            streamk.streamk_q4(aq, w, s_, out=cq, plan=pq)
+        nbytes = 2 * m * k + n * k // 2 + 2 * n * (k // 128) + 2 * m * n
+        ms = time_graph(ref_q4, launches=8)
+        wd = streamk.dequant_q4(*wqs[0])   # 537 MB of fp16 weights: more than the Infinity Cache holds
+        ms_t = time_graph(lambda: torch.matmul(aq, wd.T, out=cq), launches=4)
+        ref_rows.append({"shape": [m, n, k], "dtype": "q4 (group 128, zero 8)", "kernel": streamk.kernel_name(pq.kernel_id),
+                         "us": round(ms * 1e3, 1), "gbs": round(nbytes / ms / 1e6, 1),
+                         "frac_hbm": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4),
+                         "torch_matmul_on_fp16_weights_us": round(ms_t * 1e3, 1)})
+        del wqs, wd
+        extra["reference_run_shapes"] = ref_rows
+
+        # bfloat16 at the headline shape, both layouts, against the vendor GEMM in interleaved rounds
+        bf = []
+        ab, bb = A.bfloat16(), B.bfloat16()
+        bbt = bb.T.contiguous()
+        cb = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+        for layout, bmat in (("nt", bb), ("nn", bbt)):
+            pb16 = streamk.make_plan(M, N, K, "bfloat16", layout)
+            fns = {"tuned": lambda: streamk.streamk_bf16(ab, bmat, layout=layout, out=cb, plan=pb16),
+                   "torch_matmul": lambda: torch.matmul(ab, bmat.T if layout == "nt" else bmat, out=cb)}
+            best = {}
+            for _ in range(3):
+                for name, fn in fns.items():
+                    best[name] = min(best.get(name, 1e9), time_eager(fn, 3, 10)[0])
+            bf.append({"shape": [M, N, K], "layout": layout, "kernel": streamk.kernel_name(pb16.kernel_id),
+                       **{name: {"us": round(ms * 1e3, 1), "tflops": round(flops / ms / 1e9, 1)} for name, ms in best.items()}})
+        del ab, bb, bbt, cb
+        extra["bf16_dense"] = bf
+
         extra["q4_note"] = ("34.6 MB of weights stay in the 256 MB Infinity Cache between launches of one weight "
                             "matrix; tuned_weights_from_hbm cycles through 20 copies so that every launch reads HBM")
         streamk.workspace_status()
+        # the metric's other two parts in short, where the record of a run keeps them
+        parts = {"streamk_vs_data_parallel_N8192_K8192": {}, "q4_gemm_N8192_K8192": {}}
+        for row in sweep:
+            if row["M"] in (256, 512, 1024):
+                parts["streamk_vs_data_parallel_N8192_K8192"][f"M{row['M']}"] = {
+                    "auto_tflops": row["auto"], "auto_tile": row["auto_tile"], "sk_over_dp_same_tile": row["sk_over_dp_same_tile"],
+                    "auto_over_best_dp": row["auto_over_best_dp"]}
+        for row in q4:
+            parts["q4_gemm_N8192_K8192"][f"M{row['M']}"] = {
+                "us_weights_in_infinity_cache": row["tuned"]["us"], "frac_hbm_weights_in_infinity_cache": row["tuned"]["frac_hbm"],
+                "us_weights_from_hbm": row["tuned_weights_from_hbm"]["us"], "frac_hbm_weights_from_hbm": row["tuned_weights_from_hbm"]["frac_hbm"]}
+        out["config"]["metric_parts"] = parts
         out["extra"] = extra
 
     print(json.dumps(out))

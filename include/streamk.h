@@ -364,15 +364,6 @@ int sk_q4_quantize_host(const uint16_t *W, int64_t N, int64_t K, int64_t ldw, in
 int sk_q4_quantize(const void *W, int64_t N, int64_t K, int64_t ldw, int group, int zero, void *Wq,
                    void *scales, void *stream);
 
-/* Measurement aid with no counterpart in the reference: launches, on one workgroup of four waves per CU, a loop
- * of `iters` x 2^20 FLOP per wave of nothing but fp16 MFMAs (shape 0: v_mfma_f32_32x32x16_f16, 1:
- * v_mfma_f32_16x16x32_f16; issued in the order of a 256 x 256 tile kernel's accumulator blocks) on U[-1,1)
- * operands held in registers (zeros != 0: all-zero operands), and stores the
- * launch's FLOP count in *flop.  Timed by the caller, it gives the rate the matrix pipes of this box sustain under
- * its power limit, which is what a GEMM's fraction of the published peak should be read against.  scratch: device
- * memory of at least 1 KiB per CU (results the compiler must not drop). */
-int sk_diag_mfma_only(int shape, int iters, int zeros, void *scratch, size_t scratch_bytes, void *stream, double *flop);
-
 #ifdef __cplusplus
 }
 #endif

@@ -1,10 +1,10 @@
-// Measurement aid: what the matrix pipes of this part sustain with nothing else in flight.
+// Measurement aid for bench.py (built into libstreamk_bench.so, not part of the library or its C ABI): what the
+// matrix pipes of this part sustain with nothing else in flight.
 // The published fp16 peak assumes the maximum clock; under its power limit the part clocks down as soon as the
 // operands are not zero, by an amount that differs from box to box.  A benchmark that prices a GEMM against the
 // peak can run this loop in the same process to say how much of the gap no GEMM kernel can close.
 #include <hip/hip_runtime.h>
 
-#include "../../include/streamk.h"
 
 namespace sk {
 
@@ -76,18 +76,18 @@ __global__ __launch_bounds__(256) void mfma_only_kernel(float *out, int iters, i
 
 }  // namespace sk
 
-extern "C" int sk_diag_mfma_only(int shape, int iters, int zeros, void *scratch, size_t scratch_bytes, void *stream,
+extern "C" int skb_mfma_only(int shape, int iters, int zeros, void *scratch, size_t scratch_bytes, void *stream,
                                  double *flop) {
   int dev = 0, cus = 0;
   if (hipGetDevice(&dev) != hipSuccess ||
       hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
-    return SK_ERR_LAUNCH;
-  if (!scratch || iters <= 0 || (shape != 0 && shape != 1)) return SK_ERR_CONFIG;
-  if (scratch_bytes < (size_t)cus * 256 * sizeof(float)) return SK_ERR_WORKSPACE;
+    return -1;
+  if (!scratch || iters <= 0 || (shape != 0 && shape != 1)) return -2;
+  if (scratch_bytes < (size_t)cus * 256 * sizeof(float)) return -3;
   if (shape == 0)
     hipLaunchKernelGGL(sk::mfma_only_kernel<true>, dim3(cus), dim3(256), 0, (hipStream_t)stream, (float *)scratch, iters, zeros);
   else
     hipLaunchKernelGGL(sk::mfma_only_kernel<false>, dim3(cus), dim3(256), 0, (hipStream_t)stream, (float *)scratch, iters, zeros);
   if (flop) *flop = (double)cus * 4.0 * (double)iters * 1048576.0;  // 32 x 32x32x16 = 64 x 16x16x32 = 2^20 FLOP per wave and iteration
-  return hipGetLastError() == hipSuccess ? SK_OK : SK_ERR_LAUNCH;
+  return hipGetLastError() == hipSuccess ? 0 : -1;
 }

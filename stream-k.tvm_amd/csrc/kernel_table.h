@@ -40,28 +40,23 @@ struct KernelInfo {
 
 // fp16 LDS-tiled kernels, NT layout:  X(id, BM, BN, BK, WM, WN)
 #define SK_TILE_F16_NT_KERNELS(X) \
-  X(0, 256, 256, 64, 2, 4)        \
   X(1, 128, 128, 64, 2, 2)        \
   X(2, 128, 256, 64, 2, 4)        \
   X(3, 256, 128, 64, 4, 2)        \
   X(4, 64, 64, 64, 2, 2)          \
-  X(5, 256, 256, 32, 2, 4)        \
   X(6, 128, 128, 32, 2, 2)
 
 // fp16 LDS-tiled kernels with direct-to-LDS loads (BK = 64), NT layout:  X(id, BM, BN, WM, WN)
 #define SK_TILE_F16_NT_DMA_KERNELS(X) \
-  X(10, 256, 256, 2, 4)               \
   X(11, 128, 128, 2, 2)               \
   X(12, 128, 256, 2, 4)               \
   X(13, 256, 128, 4, 2)               \
-  X(14, 256, 256, 2, 2)               \
   X(24, 64, 64, 2, 2)                 \
   X(25, 128, 64, 2, 2)                \
   X(26, 64, 128, 2, 2)
 
 // direct-to-LDS loads, BK = 32, four stages (variant 3), NT layout:  X(id, BM, BN, WM, WN)
 #define SK_TILE_F16_NT_DMA32_KERNELS(X) \
-  X(15, 256, 256, 2, 4)                 \
   X(16, 128, 128, 2, 2)                 \
   X(17, 128, 256, 2, 4)                 \
   X(18, 256, 128, 4, 2)                 \
@@ -78,7 +73,6 @@ struct KernelInfo {
 
 // BK = 32, four stages, 16x16x32 MFMAs (variant 5), NT layout:  X(id, BM, BN, WM, WN)
 #define SK_TILE_F16_NT_DMA32_16_KERNELS(X) \
-  X(35, 256, 256, 2, 4)                    \
   X(36, 128, 128, 2, 2)                    \
   X(37, 128, 256, 2, 4)                    \
   X(38, 256, 128, 4, 2)                    \
@@ -88,7 +82,6 @@ struct KernelInfo {
 
 // the same for the NN layout (B is [K,N]), fragments through transposing LDS reads:  X(id, BM, BN, WM, WN)
 #define SK_TILE_F16_NN_DMA_KERNELS(X) \
-  X(20, 256, 256, 2, 4)               \
   X(21, 128, 128, 2, 2)               \
   X(22, 128, 256, 2, 4)               \
   X(23, 256, 128, 4, 2)
@@ -333,8 +326,7 @@ struct KernelInfo {
 // kernel with B dequantised into its LDS stage (variant 4):  X(id, BM, BN, WM, WN)
 #define SK_TILE_Q4_KERNELS(X) \
   X(46, 128, 128, 2, 2)       \
-  X(47, 256, 128, 4, 2)       \
-  X(48, 256, 256, 2, 4)
+  X(47, 256, 128, 4, 2)
 
 const KernelInfo *kernel_table(int *count);
 const KernelInfo *kernel_by_id(int id);

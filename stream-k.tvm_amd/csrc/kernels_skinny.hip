@@ -2,10 +2,6 @@
 #include "skinny_launch.h"
 
 namespace sk {
-#ifdef SK_PHASE_TRACE
-__device__ long long g_trace_buf[2048 * 16];
-#endif
-
 #define SK_POLICY(MB, NB, WN, RK, Q4, DEPTH, ROW1) TileSkinny<MB, NB, WN, RK, (Q4) != 0, DEPTH, (ROW1) != 0>
 #define SK_POLICY_BF16(MB, NB, WN, RK, DEPTH, ROW1) \
   TileSkinny<MB, NB, WN, RK, false, DEPTH, (ROW1) != 0, false, false, true>
@@ -317,9 +313,3 @@ int occupancy_skinny(int id) {
 }
 
 }  // namespace sk
-
-#ifdef SK_PHASE_TRACE
-extern "C" int sk_debug_trace_read(long long *out) {
-  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(sk::g_trace_buf), sizeof(long long) * 2048 * 16);
-}
-#endif

@@ -91,10 +91,11 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
     // 256 rows of A per tile as soon as M has them: a CTA decodes its BN weight rows whatever BM is, and the
     // four-wave 128 x 128 kernel waits for its loads (one wave per SIMD, a short iteration), so a 256 x 128 tile
     // takes no longer than a 128 x 128 one; where that leaves CUs without a tile the Stream-K schedule splits K
-    // (N = K = 8192, M = 512: 73 us against 109 us on 128 x 128 tiles).  256 x 256 when those fill the device.
-    const int64_t t256 = cdiv(M, 256) * cdiv(N, 256);
+    // (N = K = 8192, M = 512: 73 us against 109 us on 128 x 128 tiles).  There is no 256 x 256 instance: eight waves
+    // that decode and hold 128 x 64 accumulators each do not fit the register file (it spilled); large M is better
+    // served by dequantising once and running the fp16 kernels, which is what streamk_q4 does from 1024 rows on.
     const int want_bm = M > 128 ? 256 : 128;
-    const int want_bn = (want_bm == 256 && t256 * 4 >= (int64_t)num_cus * 3) ? 256 : 128;
+    const int want_bn = 128;
     for (int i = 0; i < n; ++i)
       if (t[i].family == FAMILY_TILE && t[i].dtype == SK_Q4 && t[i].bm == want_bm && t[i].bn == want_bn) return &t[i];
     return nullptr;

@@ -18,21 +18,6 @@ typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 
 enum { FIXUP_ATOMIC = 1, FIXUP_REDUCE = 2, FIXUP_ATOMIC_C = 3 };
 
-// Phase tracing (off unless the small-M translation unit is built with -DSK_PHASE_TRACE): thread 0
-// of every CTA stores the shader clock counter into slot `slot` of its row of g_trace_buf; the host
-// reads the table back with sk_debug_trace_read.  Slots: 0 kernel entry, 1-7 inside the
-// matrix-vector kernel's segment (loads issued, A staged, scales staged, barrier, loop start,
-// loop end), 8/9 before/after the store of C, 10/11 after the CTA's range / tile coordinates.
-#ifdef SK_PHASE_TRACE
-extern __device__ long long g_trace_buf[2048 * 16];
-#define SK_TRACE(slot)                                                              \
-  do {                                                                              \
-    if (threadIdx.x == 0) g_trace_buf[blockIdx.x * 16 + (slot)] = (long long)__builtin_readcyclecounter();  \
-  } while (0)
-#else
-#define SK_TRACE(slot)
-#endif
-
 // Division of a non-negative 32-bit integer by a divisor known on the host: the host stores
 // mul = floor(2^32 (2^shift - d) / d) + 1 with shift = ceil(log2 d), and
 // n / d == (umulhi(n, mul) + n) >> shift for every 0 <= n < 2^31.  The kernels divide wave-uniform

@@ -55,7 +55,6 @@ __device__ __forceinline__ void run_persistent(const typename P::Args &a, const 
     bias = bias_arg;
     asm volatile("" ::"s"(bias));
   }
-  SK_TRACE(0);
   const int pid = logical_pid(plan);
   const int ipt = plan.ipt;
   typename P::Acc acc;
@@ -66,7 +65,6 @@ __device__ __forceinline__ void run_persistent(const typename P::Args &a, const 
   // keep it.
   int start = 0, last = 0;
   if constexpr (FIXUP || !P::LEAN_ENTRY) sk_range(plan, pid, start, last);
-  SK_TRACE(10);
   int dp_tile = (FIXUP || !P::LEAN_ENTRY) ? plan.sk_tiles + pid : pid;
 
   // One loop body serves both phases so that the MAC loop and the epilogue exist once in the
@@ -94,7 +92,6 @@ __device__ __forceinline__ void run_persistent(const typename P::Args &a, const 
     }
     int pm, pn;
     tile_coords(plan, tile, pm, pn);
-    SK_TRACE(11);
     if constexpr (has_prefetch<P>::value) {
       P::mac(a, acc, pm, pn, k0, n, smem, first_stage_requested);
       first_stage_requested = false;
@@ -218,9 +215,7 @@ __device__ __forceinline__ void run_persistent(const typename P::Args &a, const 
         store = true;
       }
     }
-    SK_TRACE(8);
     if (store) P::store_c(a, acc, pm, pn, smem, bias);
-    SK_TRACE(9);
   }
 }
 

@@ -27,13 +27,9 @@ template <class P>
 __global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_skinny_dp_kernel(typename P::Args a, int total_tiles, int ipt) {
   __shared__ __attribute__((aligned(16))) char smem[P::LDS_BYTES];
   typename P::Acc acc;
-  SK_TRACE(0);
   for (int tile = blockIdx.x; tile < total_tiles; tile += gridDim.x) {
-    SK_TRACE(11);
     P::mac(a, acc, 0, tile, 0, ipt, smem);
-    SK_TRACE(8);
     P::store_c(a, acc, 0, tile, smem, nullptr);
-    SK_TRACE(9);
   }
 }
 template <class P>

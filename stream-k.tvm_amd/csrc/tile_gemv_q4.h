@@ -125,7 +125,6 @@ struct TileGemvQ4 {
                      : buffer_load_16(rsrc_w, klane + c * 128 < klimit ? voff_w[j] : OOB_OFFSET,
                                       (uint32_t)(kbase / 2) + c * 64);
     };
-    SK_TRACE(1);
 
     // ---- all global loads of the prologue go out back to back, in the order they are consumed:
     // A (first two rounds of the CTA), the first round of scale pieces, then DEPTH iterations of
@@ -160,7 +159,6 @@ struct TileGemvQ4 {
     for (int d = 0; d < DEPTH; ++d) issue_loads(d, d);
     // nothing of what follows is to be scheduled ahead of these loads
     __builtin_amdgcn_sched_barrier(0);
-    SK_TRACE(2);
 
     const float w_even = (float)(1024 + (ZP_ ? 0 : a.zero)), w_odd = (float)(64 + (ZP_ ? 0 : a.zero));
     float *ldsSumA = ldsCorr + KMAX / 32;  // ZP_: sum of the 32 K-values of A, beside their correction
@@ -204,12 +202,9 @@ struct TileGemvQ4 {
       const uint32_t off = (uint32_t)(k0 * BKC + (b0 + tid) * 16) * 2;
       stage_a_block(b0 + tid, buffer_load_16(rsrc_a, off, 0), buffer_load_16(rsrc_a, off, 16));
     }
-    SK_TRACE(3);
     scales.finish();
     if constexpr (ZP_) zero_points.finish();
-    SK_TRACE(4);
     __syncthreads();
-    SK_TRACE(5);
 
     Q4Consts qc;
     q4_pin_patterns(qc);
@@ -222,7 +217,6 @@ struct TileGemvQ4 {
     const bool p1 = piece & 1, p2 = piece & 2;
 
     // ---- main loop: rounds of DEPTH iterations without an exit inside a round ----
-    SK_TRACE(6);
     for (int it0 = 0; it0 < n; it0 += DEPTH) {
 #pragma unroll
       for (int d = 0; d < DEPTH; ++d) {
@@ -283,7 +277,6 @@ struct TileGemvQ4 {
       }
     }
 
-    SK_TRACE(7);
     // ---- add up the four pieces of each row (the lanes of a quad), then the RK partial results
     // into the rk == 0 waves.  Either way the segment ends with a barrier: the next segment's
     // prologue overwrites the LDS without waiting. ----

@@ -261,10 +261,8 @@ struct TileSkinny {
     const Q4Consts qc = q4_consts(a.zero);
 
     // ---- prologue: DEPTH iterations of loads in flight ----
-    SK_TRACE(1);
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) issue_loads(d, d);
-    SK_TRACE(2);
 
     // ---- Q4: stage the scales of this segment, 16 bytes at a time.  Row r of the tile needs
     // groups [k0*SC_PER_ITER, (k0+n)*SC_PER_ITER); the copy starts at the 8-aligned group below
@@ -278,11 +276,8 @@ struct TileSkinny {
       if (ZP_)
         stage_scales<BN, SC_ROW, NT>(ldsS + BN * SC_ROW, a.zeros + (int64_t)pn * BN * a.groups, rows_w, a.groups, g0, chunks);
     }
-    SK_TRACE(4);
     stage_a(0, 0);
-    SK_TRACE(3);
     __syncthreads();
-    SK_TRACE(6);
 
     // ---- main loop: rounds of DEPTH iterations, no exit inside a round.  Iterations past the
     // segment multiply zeros (their loads were pushed out of range), so n need not be a multiple
@@ -361,7 +356,6 @@ struct TileSkinny {
       }
     }
 
-    SK_TRACE(7);
     // ---- sum the RK partial accumulators into the rk == 0 waves ----
     if (RK > 1) {
       AccT *red = reinterpret_cast<AccT *>(smem + LDS_A + LDS_SC);

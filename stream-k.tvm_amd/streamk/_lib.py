@@ -116,8 +116,6 @@ def lib():
     L.sk_q4_tile_host.argtypes = [vp, i64, i64, vp]
     L.sk_q4_untile_host.argtypes = [vp, i64, i64, vp]
     L.sk_q4_tile.argtypes = [vp, i64, i64, vp, vp]
-    L.sk_diag_mfma_only.argtypes = [ci, ci, ci, vp, sz, vp, P(ctypes.c_double)]
-    L.sk_diag_mfma_only.restype = ci
     for f in ("sk_q4_pack_host", "sk_q4_unpack_host", "sk_q4_quantize_host", "sk_q4_quantize", "sk_q4_tile_host",
               "sk_q4_untile_host", "sk_q4_tile"):
         getattr(L, f).restype = ci

@@ -82,8 +82,9 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
             variants += ((6, 32),)  # four-stage with 16x16x32 MFMAs
             if bm >= 128 and bn >= 128:
                 variants += ((5, bk),)  # two-stage with 16x16x32 MFMAs
-            if (bm, bn) == (256, 256) and K % 64 == 0:
-                variants += ((8, bk),)  # four waves, the K loop in assembly
+            if (bm, bn) == (256, 256):
+                # 256 x 256 tiles: four waves with the K loop in assembly, or the eight-wave 16x16x32 kernel for other K
+                variants = ((5, bk),) + (((8, bk),) if K % 64 == 0 else ())
             if (bm, bn) == (64, 64):
                 variants += ((1, bk),)
             for (variant, vbk), raster in itertools.product(variants, (1, 8)):
