@@ -45,6 +45,33 @@ __global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_skinny_dp_kernel_bi
   }
 }
 
+// The same with the operands as 14 scalar kernel arguments instead of the argument structure, for the common call
+// (rows of A and C packed, no per-group zero points, no bias).  Scalar arguments can be preloaded into scalar
+// registers by the command processor before the first wave starts (this translation unit is compiled with a
+// kernel-argument preload count; a structure passed by value cannot be), which takes the ~1 us "wait for the kernel
+// arguments" off the front of launches that run for 6 to 40 us.  One tile per CTA; the iterations per tile follow from
+// K.  (Where the firmware does not preload, the kernel starts at its ordinary entry, which loads the arguments.)
+template <class P>
+__global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_skinny_flat_kernel(const half_t *A, const void *W, const half_t *scales,
+                                                                              half_t *C, int M, int N, int K, int ldw, int zero,
+                                                                              int groups) {
+  __shared__ __attribute__((aligned(16))) char smem[P::LDS_BYTES];
+  SkinnyArgs a;
+  a.A = A; a.W = W; a.scales = scales; a.C = C;
+  a.M = M; a.N = N; a.K = K;
+  a.lda = K; a.ldw = ldw; a.ldc = N;
+  a.zero = zero; a.groups = groups; a.zeros = nullptr;
+  typename P::Acc acc;
+  P::mac(a, acc, 0, blockIdx.x, 0, (K + P::BKC - 1) / P::BKC, smem);
+  P::store_c(a, acc, 0, blockIdx.x, smem, nullptr);
+}
+
+// NO_FLAT_ARGS: policies whose scalar-argument instance the compiler does not fit into the register budget
+template <class P, class = void>
+struct no_flat_args { static constexpr bool value = false; };
+template <class P>
+struct no_flat_args<P, std::void_t<decltype(P::NO_FLAT_ARGS)>> { static constexpr bool value = P::NO_FLAT_ARGS; };
+
 template <class P>
 static inline int launch_policy(const SkinnyArgs &a, const DevPlan &p, const Workspace &ws, hipStream_t s, const void *bias) {
   if (p.sk_tiles == 0 && p.tiles_m != 1) return (int)hipErrorInvalidValue;  // (no plan of these kernels has two tile rows)
@@ -54,6 +81,14 @@ static inline int launch_policy(const SkinnyArgs &a, const DevPlan &p, const Wor
     else
       hipLaunchKernelGGL((sk_skinny_kernel_bias<P, true>), dim3(p.grid), dim3(P::NT), 0, s, a, p, ws, bias);
   } else if (p.sk_tiles == 0) {
+    if constexpr (!no_flat_args<P>::value) {
+      if (p.grid == p.total_tiles && p.ipt == (a.K + P::BKC - 1) / P::BKC && a.zeros == nullptr && a.lda == a.K && a.ldc == a.N &&
+          a.ldw <= 0x7fffffff) {
+        hipLaunchKernelGGL((sk_skinny_flat_kernel<P>), dim3(p.grid), dim3(P::NT), 0, s, a.A, a.W, a.scales, a.C, a.M, a.N, a.K,
+                           (int)a.ldw, a.zero, a.groups);
+        return (int)hipGetLastError();
+      }
+    }
     hipLaunchKernelGGL((sk_skinny_dp_kernel<P>), dim3(p.grid), dim3(P::NT), 0, s, a, p.total_tiles, p.ipt);
   } else {
     hipLaunchKernelGGL((sk_skinny_kernel<P, true>), dim3(p.grid), dim3(P::NT), 0, s, a, p, ws);

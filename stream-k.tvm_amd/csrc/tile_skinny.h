@@ -127,6 +127,8 @@ struct TileSkinny {
   static constexpr bool LEAN_ENTRY = false;  // see run_persistent
   static constexpr int MB = MB_, NB = NB_, WN = WN_, RK = RK_, DEPTH = DEPTH_;
   static constexpr bool Q4 = Q4_;
+  // the Q4 instances of one row block per wave without K split: their scalar-argument form spills (skinny_launch.h)
+  static constexpr bool NO_FLAT_ARGS = Q4_ && NB_ == 1 && WN_ == 4 && RK_ == 1 && !ROW1_;
   static constexpr int BM = 16 * MB, BN = 16 * NB * WN;
   static constexpr int BK = Q4 ? 256 : 128;  // K per wave per iteration
   static constexpr int BKC = BK * RK;        // K per CTA iteration
