@@ -209,8 +209,15 @@ int sk_gemm_f16(const void *A, const void *B, void *C, int64_t M, int64_t N, int
  * (two streams, two threads) race; serialise them.  There is no status word to poll: a fix-up wait that gives
  * up (spin_limit) leaves its tile incomplete as with sk_gemm_f16, but unreported -- callers that lower
  * spin_limit should use sk_gemm_f16 with their own workspace.
+ *
+ * sk_static_init() looks up the array's address on the current device (one symbol query per device and
+ * process; later calls return at once).  sk_gemm_f16_static does the same on its first call on a device, so
+ * the call is optional -- except for callers that record sk_gemm_f16_static into a HIP graph: they call
+ * sk_static_init() on that device before the capture begins, so that the capture holds kernel launches only.
+ * No counterpart in the reference.
  */
 #define SK_STATIC_WORKSPACE_BYTES (64u * 1024u * 1024u + 262144u + 256u)
+int sk_static_init(void);
 int sk_gemm_f16_static(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
                        int64_t ldb, int64_t ldc, const sk_plan *plan, void *stream);
 

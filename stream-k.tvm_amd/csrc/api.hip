@@ -74,6 +74,9 @@ __global__ void clean_partials_kernel(int *status, uint4v *partials, unsigned ca
 struct WsInfo {
   size_t bytes;
   bool poisoned;
+  // host-side hint: a launch enqueued through this library may have left partial tiles in the workspace (the
+  // authoritative record is the dirty mark in the workspace itself; a stale hint only costs time)
+  bool maybe_dirty;
 };
 std::unordered_map<const void *, WsInfo> g_ws;
 
@@ -160,16 +163,30 @@ int make_dev_plan(const sk_plan *plan, const KernelInfo *k, void *ws, size_t ws_
                        (unsigned)units, plan->fixup == SK_FIXUP_ATOMIC ? 1 : 0);
     if (hipGetLastError() != hipSuccess) return SK_ERR_LAUNCH;
   } else if (plan->workspace_bytes > 0) {
+    bool wide_clean = false;
+    size_t registered_bytes = ws_bytes;
     {
       std::lock_guard<std::mutex> lock(g_mutex);
       auto it = g_ws.find(ws);
       if (it == g_ws.end() || it->second.bytes < ws_bytes) return SK_ERR_WORKSPACE;  // sk_workspace_init was never run on it
       if (it->second.poisoned) return SK_ERR_TIMEOUT;
+      registered_bytes = it->second.bytes;
+      if (plan->fixup == SK_FIXUP_ATOMIC) {
+        wide_clean = it->second.maybe_dirty;
+        it->second.maybe_dirty = false;
+      } else if (plan->fixup == SK_FIXUP_REDUCE && plan->streamk_tiles > 0) {
+        it->second.maybe_dirty = true;
+      }
     }
     if (plan->fixup == SK_FIXUP_ATOMIC) {
+      // The cleaner reads the mark the workspace carries and returns at once when it is zero.  Where this library has
+      // not enqueued anything that could have raised it, one small block does that; it still cleans correctly (only
+      // slowly) if a captured REDUCE launch replayed in between proves the hint wrong.
+      // (the capacity is that of the workspace as it was initialised, not of this call's share of it: the mark can
+      // then never lie beyond what the cleaner may touch, and a cleaned workspace always reads as clean)
       char *base = static_cast<char *>(ws);
-      const size_t units = (ws_bytes - (size_t)WS_PART_OFF) / 256;
-      hipLaunchKernelGGL(clean_partials_kernel, dim3(1024), dim3(256), 0, stream, reinterpret_cast<int *>(base),
+      const size_t units = (registered_bytes - (size_t)WS_PART_OFF) / 256;
+      hipLaunchKernelGGL(clean_partials_kernel, dim3(wide_clean ? 1024 : 1), dim3(256), 0, stream, reinterpret_cast<int *>(base),
                          reinterpret_cast<uint4v *>(base + WS_PART_OFF), (unsigned)(units > 0xffffffffu ? 0xffffffffu : units));
       if (hipGetLastError() != hipSuccess) return SK_ERR_LAUNCH;
     }
@@ -337,13 +354,16 @@ static int gemm_16bit(int dtype, const void *A, const void *B, void *C, int64_t 
     // and there is no CTA that would apply a bias once
     if (bias != nullptr || skinny) return SK_ERR_CONFIG;
     if ((N % 2) || (ldc % 2) || (reinterpret_cast<uintptr_t>(C) & 3)) return SK_ERR_ALIGN;
-    hipLaunchKernelGGL(zero_pairs_kernel, dim3(1024), dim3(256), 0, (hipStream_t)stream, reinterpret_cast<uint32_t *>(C),
-                       (int)M, (int)(N / 2), (int64_t)(ldc / 2));
-    if (hipGetLastError() != hipSuccess) return SK_ERR_LAUNCH;
   }
   rc = make_dev_plan(plan, k, ws, ws_bytes, cached_occupancy(k->id, skinny ? 1 : 0), (hipStream_t)stream, &dp, &w,
                      is_static);
   if (rc) return rc;
+  if (plan->fixup == SK_FIXUP_ATOMIC_C && plan->streamk_tiles > 0) {
+    // (behind every check: a call that is refused leaves the caller's C alone)
+    hipLaunchKernelGGL(zero_pairs_kernel, dim3(1024), dim3(256), 0, (hipStream_t)stream, reinterpret_cast<uint32_t *>(C),
+                       (int)M, (int)(N / 2), (int64_t)(ldc / 2));
+    if (hipGetLastError() != hipSuccess) return SK_ERR_LAUNCH;
+  }
   int herr;
   if (skinny) {
     SkinnyArgs a{(const half_t *)A, B, nullptr, (half_t *)C, (int)M, (int)N, (int)K, lda, ldb, ldc, 0, 0, nullptr};
@@ -359,6 +379,11 @@ extern "C" int sk_gemm_f16(const void *A, const void *B, void *C, int64_t M, int
                            int64_t lda, int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws,
                            size_t ws_bytes, void *stream) {
   return gemm_16bit(SK_F16, A, B, C, M, N, K, lda, ldb, ldc, plan, ws, ws_bytes, stream);
+}
+
+extern "C" int sk_static_init(void) {
+  void *ws = nullptr;
+  return static_scratch(&ws);
 }
 
 extern "C" int sk_gemm_f16_static(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K,

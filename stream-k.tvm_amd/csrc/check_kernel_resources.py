@@ -53,6 +53,9 @@ def main(argv):
                 bad.append((no, f"kernel uses {m.group(1)} bytes of scratch memory per lane and is not in scratch_allowed.txt: {kernel}"))
     for no, text in bad[:20]:
         print(f"{path}:{no}: {text}", file=sys.stderr)
+    if bad and "--warn-only" in argv:     # (for experiments: make CHECK_EXTRA=--warn-only)
+        print(f"{len(bad)} problem(s) in {path}: ignored", file=sys.stderr)
+        return
     if bad:
         sys.exit(f"{len(bad)} problem(s) in {path}")
     acc = "; accumulation registers only inside the hand-written blocks" if check_acc else ""

@@ -252,6 +252,12 @@ __device__ __forceinline__ uint4v make_rsrc_words(const void *base, uint32_t num
   const uint64_t b = reinterpret_cast<uint64_t>(base);
   return uint4v{(uint32_t)b, (uint32_t)(b >> 32) & 0xffffu, num_bytes, 0x00020000u};
 }
+// a descriptor whose words the compiler holds in vector registers although they are wave-uniform (values derived
+// from the wave's index): moved to scalar registers, which is where an instruction wants them
+__device__ __forceinline__ uint4v uniform_rsrc(uint4v w) {
+  return uint4v{(uint32_t)__builtin_amdgcn_readfirstlane((int)w[0]), (uint32_t)__builtin_amdgcn_readfirstlane((int)w[1]),
+                (uint32_t)__builtin_amdgcn_readfirstlane((int)w[2]), (uint32_t)__builtin_amdgcn_readfirstlane((int)w[3])};
+}
 __device__ __forceinline__ void dma_load_16(uint4v rsrc, uint32_t lds_base, uint32_t lane_off,
                                             uint32_t uniform_off) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"

@@ -237,9 +237,7 @@ struct TileF16Asm {
     const int rows = max(0, min(WTM, a.M - row0));
     const uint32_t bytes = rows > 0 ? (uint32_t)(((int64_t)(rows - 1) * a.ldc + WTN) * 2) : 0u;
     const uint4v words = make_rsrc_words(a.C + (int64_t)row0 * a.ldc + col0, bytes);
-    // (the descriptor depends on the wave: make the compiler keep it in scalar registers)
-    const uint4v rsrc_c = {(uint32_t)__builtin_amdgcn_readfirstlane((int)words[0]), (uint32_t)__builtin_amdgcn_readfirstlane((int)words[1]),
-                           (uint32_t)__builtin_amdgcn_readfirstlane((int)words[2]), words[3]};
+    const uint4v rsrc_c = uniform_rsrc(words);  // (it depends on the wave's index)
     const uint32_t patch = lds_address(lds()) + 2 * STAGE_BYTES + (uint32_t)wave * FAST_PATCH_BYTES;
     const uint32_t wr = patch + (uint32_t)((lane & 15) * PATCH_STRIDE + (lane >> 4) * 8);
     const uint32_t rd = patch + (uint32_t)((lane >> 4) * PATCH_STRIDE + (lane & 15) * 16);

@@ -85,6 +85,8 @@ def lib():
     L.sk_gemm_f32.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, P(SkPlan), vp, sz, vp]
     L.sk_gemm_f16_static.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, P(SkPlan), vp]
     L.sk_gemm_f16_static.restype = ci
+    L.sk_static_init.argtypes = []
+    L.sk_static_init.restype = ci
     L.sk_gemm_bf16.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, P(SkPlan), vp, sz, vp]
     L.sk_gemm_bf16.restype = ci
     L.sk_gemm_q4_zp.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, ci, P(SkPlan), vp, sz, vp]

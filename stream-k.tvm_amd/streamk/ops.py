@@ -18,10 +18,13 @@ adapters over those operators.  torch is used for device memory, streams and the
 all arithmetic happens in libstreamk.so.
 """
 import ctypes
+import itertools
+import weakref
 
 import torch
 
 from . import _lib
+from . import plan as _plan_mod
 from .plan import make_plan
 
 _workspaces = {}
@@ -101,14 +104,16 @@ def _epilogue(bias, N, dtype, device, activation=None):
 # configuration travels as a string: "" (tuned cache, else the library's heuristic), "k=v;k=v" for
 # make_config keys, or "#n" for a plan object the caller made itself (kept in a registry here).
 # ---------------------------------------------------------------------------------------------
-_plan_registry = {}
+# (weak: a plan object lives as long as its caller keeps it -- the autotuner makes hundreds per shape)
+_plan_registry = weakref.WeakValueDictionary()
+_plan_serial = itertools.count(1)
 _plan_cache = {}
 
 
 def _plan_handle(plan):
     h = getattr(plan, "_sk_handle", None)
     if h is None:
-        h = plan._sk_handle = f"#{len(_plan_registry) + 1}"
+        h = plan._sk_handle = f"#{next(_plan_serial)}"
         _plan_registry[h] = plan
     return h
 
@@ -137,7 +142,8 @@ def _plan_for(config, M, N, K, dtype, layout):
         if plan is None:
             raise ValueError(f"unknown plan handle {config!r}")
         return plan
-    key = (M, N, K, dtype, layout, config)
+    # (a plan depends on the tuned cache it was made from and on the device it was made for)
+    key = (M, N, K, dtype, layout, config, _plan_mod.tuned_generation(), torch.cuda.current_device() if torch.cuda.is_available() else -1)
     plan = _plan_cache.get(key)
     if plan is None:
         plan = make_plan(M, N, K, dtype, layout, _parse_config(config) if config else None)

@@ -53,9 +53,20 @@ def make_config(config=None, **kw):
 _tuned = None
 
 
+_tuned_generation = 0
+
+
 def invalidate_tuned_cache():
-    global _tuned
+    """Forget the loaded tuned cache (the autotuner calls this when it has written an entry).  Plans that other
+    layers made from the old cache are told apart by tuned_generation()."""
+    global _tuned, _tuned_generation
     _tuned = None
+    _tuned_generation += 1
+
+
+def tuned_generation():
+    """Counts the invalidations of the tuned cache: part of the key of every cache of plans made from it."""
+    return _tuned_generation
 
 
 def tuned_config(M, N, K, dtype="float16", layout="nt"):

@@ -309,3 +309,27 @@ def test_autotune_candidates_make_plans():
                 except StreamKError as e:
                     assert e.status == -4, (dtype, M, c, e.status)
             assert valid > 0, (dtype, M)
+
+
+def test_operator_plans_follow_the_tuned_cache(monkeypatch):
+    """The operator layer keeps the plans it made from the tuned cache; an autotune run that writes a new entry
+    invalidates the cache, and the next call of the operator for that shape must run the new plan."""
+    import sys
+    import streamk  # noqa: F401
+    from streamk import ops
+    from streamk import plan as P
+    autotune = sys.modules["streamk.autotune"]   # (the package exports a function of the same name)
+    monkeypatch.setattr(P, "num_cus", lambda: 256)
+    key = "gfx950/float16/nt/512x4096x4096"
+    entries = {key: {"config": dict(bm=128, bn=128, bk=64, schedule="dp")}}
+    monkeypatch.setattr(autotune, "load_cache", lambda path=None: dict(entries))
+    P.invalidate_tuned_cache()
+    p1 = ops._plan_for("", 512, 4096, 4096, "float16", "nt")
+    assert (p1.bm, p1.bn) == (128, 128)
+    assert ops._plan_for("", 512, 4096, 4096, "float16", "nt") is p1
+    entries[key] = {"config": dict(bm=256, bn=256, bk=64, schedule="dp")}
+    P.invalidate_tuned_cache()      # what autotune(..., cache=True) does after writing its entry
+    p2 = ops._plan_for("", 512, 4096, 4096, "float16", "nt")
+    assert (p2.bm, p2.bn) == (256, 256)
+    monkeypatch.undo()
+    P.invalidate_tuned_cache()

@@ -71,3 +71,58 @@ def test_static_workspace_entry_point_matches_sk_gemm_f16():
     assert big.workspace_bytes > 64 * 1024 * 1024 + 262144 + 256
     assert L.sk_gemm_f16_static(A.data_ptr(), A.data_ptr(), C.data_ptr(), 8192, 8192, 8192, 8192, 8192, 8192,
                                 ctypes.byref(big), stream) == -5
+
+
+@pytest.mark.gpu
+def test_static_entry_point_replays_from_a_hip_graph():
+    """sk_gemm_f16_static recorded into a HIP graph (after sk_static_init, so that the capture holds kernel launches
+    only) must give on every replay what the eager call gives, bit for bit: ordered reduce on random data, atomic
+    fix-up on integer data.  Between the replays the program runs eager calls of the other fix-up on the same
+    static array and synchronises, so that each replay meets different leftovers."""
+    import torch
+    import streamk
+    L = streamk.lib()
+    assert L.sk_static_init() == 0
+    rng = np.random.default_rng(77)
+    M, N, K = 520, 776, 2056
+    red = dict(bm=128, bn=128, bk=64, schedule="basic", fixup="reduce", grid=40)
+    atm = dict(red, fixup="atomic")
+
+    def operands(integer):
+        if integer:
+            A = rng.integers(-1, 2, (M, K)).astype(np.float16)
+            B = rng.integers(-1, 2, (N, K)).astype(np.float16)
+        else:
+            A = (rng.random((M, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+            B = (rng.random((N, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+        return torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
+
+    def call(dA, dB, out, plan, stream):
+        return L.sk_gemm_f16_static(dA.data_ptr(), dB.data_ptr(), out.data_ptr(), M, N, K, K, K, N,
+                                    ctypes.byref(plan), ctypes.c_void_p(stream.cuda_stream))
+
+    for cfg, other, integer in ((red, atm, False), (atm, red, True)):
+        dA, dB = operands(integer)
+        plan = streamk.make_plan(M, N, K, "float16", "nt", cfg)
+        other_plan = streamk.make_plan(M, N, K, "float16", "nt", other)
+        assert plan.streamk_tiles > 0 and other_plan.streamk_tiles > 0
+        want = torch.empty(M, N, dtype=torch.float16, device="cuda")
+        assert call(dA, dB, want, plan, torch.cuda.current_stream()) == 0
+        torch.cuda.synchronize()
+        got = torch.empty(M, N, dtype=torch.float16, device="cuda")
+        scratch_out = torch.empty(M, N, dtype=torch.float16, device="cuda")
+        graph = torch.cuda.CUDAGraph()
+        print(f"capture {cfg['fixup']}", flush=True)
+        with torch.cuda.graph(graph):
+            assert call(dA, dB, got, plan, torch.cuda.current_stream()) == 0
+        for replay in range(3):
+            got.fill_(float("nan"))
+            print(f"replay {replay} {cfg['fixup']}", flush=True)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(got, want), (cfg["fixup"], replay)
+            assert call(dA, dB, scratch_out, other_plan, torch.cuda.current_stream()) == 0
+            torch.cuda.synchronize()
+        if integer:
+            ref = dA.cpu().numpy().astype(np.int32) @ dB.cpu().numpy().astype(np.int32).T
+            assert np.array_equal(got.cpu().numpy().astype(np.int32), ref)
