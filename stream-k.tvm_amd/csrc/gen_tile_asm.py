@@ -17,26 +17,32 @@ inside the loop), so the loop is written out with fixed registers:
 
 Three pieces of text per layout:
 
-  SK_TILE_ASM_LOADS*   the 16 direct-to-LDS loads of one 64 KB stage (8 row groups of A, 8 of B per wave).  A segment
-                       starts with the loads of its first two stages; the first stage of the NEXT segment is requested
+  SK_TILE_ASM_LOADS*   the 16 direct-to-LDS loads of one 64 KB stage (8 row groups of A, 8 of B per wave), or
+                       (_EARLY) the half of them the loop does not send itself.  A segment starts with the loads of its
+                       first stage and the early loads of its second; the first stage of the NEXT segment is requested
                        before the epilogue of the current one, so that its latency hides behind the stores of C.
   SK_TILE_ASM_LOOP*    zero the accumulators, wait for the first stage, run the K loop, drain.
   SK_TILE_ASM_STORE*   the epilogue of a tile that needs no edge handling: accumulators -> 16-bit pairs -> a small
                        per-wave patch of LDS behind the stages -> 16-byte stores of whole row pieces.  The stages are
                        not touched, which is what allows the next segment's loads to be in flight.
 
-One iteration of the loop (stage `cur` of the two LDS stages holds its tiles, `nxt` the next iteration's):
-  block 0   64 MFMAs on the K-step-0 fragments.  Riding along: the last six A fragments of K-step 0 (read at the top,
-            each needed eight MFMAs after the previous one), the 16 fragment reads of K-step 1, the lane offsets of
-            the loads to come, one of the two stage flips of the fragment addresses
-  sync      wait for those reads and for this wave's loads into nxt, barrier
-  block 1   64 MFMAs on the K-step-1 fragments.  Riding along: the 16 loads of iteration it + 2 into cur (which
-            every wave has finished reading), the first ten fragment reads of K-step 0 of nxt, the other flips
+One iteration of the 16-bit loop is two blocks of 64 MFMAs, one per K-step of 32, built alike (loop_text has the
+details).  The loads of a stage come in two halves: the row groups that hold blocks 0-3 of the wave tiles (EARLY) and
+those that hold blocks 4-7 (LATE).  The MFMAs of a block run quadrant by quadrant, so the late fragments are needed
+only from the 17th instruction on and are read at the top of their own block; everything a block reads at its top
+was loaded a half-stage later and is overwritten a half-stage later than the rest.  That shifts the two halves of a
+stage by one block against each other, and every block carries eight loads.  Counters on 8192^3 (SQ_BUSY_CU_CYCLES,
+SQ_VMEM_TA_ADDR_FIFO_FULL): with all 16 loads of an iteration in one block, the four waves' 64 KB keep the CU's one
+address unit busy for that whole block, a wave whose load finds the address queue full cannot issue its next MFMA
+either, the waves drift apart and the barrier makes every wave pay the slowest one's delay -- removing the barrier
+(wrong results, timing only) gave +22 % on zero operands, removing the wait for the loads nothing; with eight loads
+per block the queue-full cycles fall to a quarter and the time by 10 % (zero operands) / 3 % (random operands, where
+the clock is set by the power drawn).  Placing the loads of the four waves in different gaps, or earlier in their
+block, or the reads earlier, changed nothing measurable.
 Riders are dealt out ONE GROUP PER MFMA GAP (a gap is the 16 cycles an MFMA occupies the matrix pipe; the wave issues
-about one other instruction per four cycles in it).  Counters: with the four instructions of a load in one gap, as an
-earlier version had them, every load cost ~10 cycles of matrix-pipe time, and the scalar work bunched at the barrier
-and at the loop end another ~90 cycles per iteration; an MFMA that waits for a fragment waits only for the reads it
-needs (the waits are computed from the issue order: LDS reads return in order).
+about one other instruction per four cycles in it): with the four instructions of a load in one gap every load cost
+~10 cycles of matrix-pipe time.  An MFMA that waits for a fragment waits only for the reads it needs (the waits are
+computed from the issue order: LDS reads return in order).
 The loads of iterations past the segment get an out-of-range offset (they fetch nothing and zero a stage nobody
 reads), so the loop has no branch but its own back edge.
 
@@ -53,19 +59,24 @@ A0, B0, A1, B1 = 128, 160, 192, 224     # first registers of the fragment buffer
 VOA, VOB, VOB1 = 120, 121, 122          # v120 / v121 (/ v122, NN: odd row groups of B): load offsets of this iteration
 S_IT, S_KA, S_KB, S_T, S_OOB, S_M0, S_LDS, S_T2 = 80, 81, 82, 83, 84, 85, 86, 87
 
-ROLL = 6    # A fragments of K-step 0 that are read at the top of their own block 0 instead of in the block before
-# (measured at 8192^3, cycles per CU from SQ_BUSY_CU_CYCLES: three gaps per load -- m0, load, offset advance -- against
-# two with the scalar pair sharing a gap: within 0.2 %; the NN loop has 24 fragment reads per K-step and takes two)
-RD0_FIRST, RD0_LAST = 8, 50   # gaps of block 0 over which the K-step-1 fragment reads are spread
+# Row groups of a wave's eight per operand (group x holds rows 8 (wave + 4 x) .. + 7 of the tile's 256): the EARLY ones
+# carry rows of blocks 0-3 of a wave's 128 rows, the LATE ones rows of blocks 4-7
+EARLY_X, LATE_X = (0, 1, 4, 5), (2, 3, 6, 7)
+TOP = 8     # gaps at the top of a block that carry the reads of the late fragments
+LD_LAST, RD_LAST = 61, 53    # last gap of a block that may carry a load / a fragment read of the next K-step
 
 
 def mfma_order():
-    # walk the 8 x 8 blocks so that consecutive instructions share one operand
-    order = []
-    for i in range(8):
-        js = range(8) if i % 2 == 0 else range(7, -1, -1)
-        order += [(i, j) for j in js]
-    return order
+    """the 8 x 8 blocks quadrant by quadrant -- (A 0-3, B 0-3), (A 0-3, B 4-7), (A 4-7, B 4-7), (A 4-7, B 0-3) -- so that
+    the fragments of blocks 4-7 are needed only from the 17th (B) and the 33rd (A) instruction on; consecutive
+    instructions share one operand"""
+    def snake(rows, cols):
+        out = []
+        for n, i in enumerate(rows):
+            out += [(i, j) for j in (cols if n % 2 == 0 else cols[::-1])]
+        return out
+    lo, hi = [0, 1, 2, 3], [4, 5, 6, 7]
+    return snake(lo, lo) + snake(lo[::-1], hi) + snake(hi, hi) + snake(hi[::-1], lo[::-1])
 
 
 class LdsTracker:
@@ -87,34 +98,53 @@ class LdsTracker:
         return f'"s_waitcnt lgkmcnt({min(allowed, 15)})'
 
 
-def load_parts(x, nn, voa, vob, vob1, lds, ka, kb):
+def load_parts(x, nn, voa, vob, vob1, lds, ka, kb, prev=None):
     """load x of a stage: 0..7 row groups of A, 8..15 of B (a wave's groups are 4 KB apart in LDS).  Returns
-    (instructions that go before the m0 write, the m0 write, the load, the advance of the global offset);
-    s[S_T] walks the global offsets of the groups, `lds` is the stage's LDS address for this wave"""
-    pre = []
-    if x == 0:
-        pre.append(f'"s_mov_b32 s{S_T}, {ka}')
-    if x == 8:
-        pre.append(f'"s_mov_b32 s{S_T}, {kb}')
+    (instructions that go before the m0 write, the m0 write, the load); s[S_T] walks the global offsets of the
+    groups -- `prev` is the group the walk comes from (None: x is the first of its operand in this sequence) --,
+    `lds` is the stage's LDS address for this wave"""
+    base, step, first = (ka, "%[gas", 0) if x < 8 else (kb, "%[gbs", 8)
+    if prev is None:
+        skip = x - first
+        pre = [f'"s_mov_b32 s{S_T}, {base}'] if skip == 0 else [f'"s_add_u32 s{S_T}, {base}, {step}{skip}]']
+    else:
+        pre = [f'"s_add_u32 s{S_T}, s{S_T}, {step}{x - prev}]']
+    pre = [t.replace("gas1]", "gas]").replace("gbs1]", "gbs]") for t in pre]
     lds_off = (x * 4096) if x < 8 else (32768 + (x - 8) * 4096)
     m0 = f'"s_add_u32 m0, {lds}, {lds_off}'
     if x < 8:
         ld = f'"buffer_load_dwordx4 {voa}, %[rsa], s{S_T} offen lds'
-        adv = f'"s_add_u32 s{S_T}, s{S_T}, %[gas]'
     else:
         ld = f'"buffer_load_dwordx4 {vob1 if (nn and x % 2 == 1) else vob}, %[rsb], s{S_T} offen lds'
-        adv = f'"s_add_u32 s{S_T}, s{S_T}, %[gbs]'
-    return pre, m0, ld, adv
+    return pre, m0, ld
 
 
-def stage_loads_text(nn):
-    """the 16 loads of one stage, back to back (operands: the stage's LDS address, global offsets and lane offsets)"""
+def load_sequence(xs, nn, voa, vob, vob1, lds, ka, kb):
+    """load_parts for the groups xs (ascending; A before B), with the walk chained through them"""
+    out, prev = [], None
+    for x in xs:
+        if prev is not None and (prev < 8) != (x < 8):
+            prev = None
+        out.append(load_parts(x, nn, voa, vob, vob1, lds, ka, kb, prev))
+        prev = x
+    return out
+
+
+def early_groups(nn):
+    """the loads that must have landed a block ahead of the others: rows of blocks 0-3 (NN: and all of B, whose loads
+    fill whole K-rows)"""
+    return list(EARLY_X) + ([8 + x for x in range(8)] if nn else [8 + x for x in EARLY_X])
+
+
+def late_groups(nn):
+    return list(LATE_X) + ([] if nn else [8 + x for x in LATE_X])
+
+
+def stage_loads_text(nn, xs):
+    """the loads xs of one stage, back to back (operands: the stage's LDS address, global offsets and lane offsets)"""
     L = []
-    for x in range(16):
-        pre, m0, ld, adv = load_parts(x, nn, "%[voa]", "%[vob]", "%[vob1]", "%[lds]", "%[ga]", "%[gb]")
+    for pre, m0, ld in load_sequence(xs, nn, "%[voa]", "%[vob]", "%[vob1]", "%[lds]", "%[ga]", "%[gb]"):
         L += pre + [m0, '"s_nop 0', ld]
-        if x not in (7, 15):
-            L.append(adv)
     return L
 
 
@@ -127,143 +157,137 @@ def offsets_for(nn, ahead):
     return out
 
 
-def loop_entry(L, nn):
-    """accumulators to zero while the first stage is on its way; the loop's state; wait for that stage"""
+def zero_accumulators(L):
     for r in range(256):
         L.append(f'"v_accvgpr_write_b32 a{r}, 0')
-    L.append(f'"s_mov_b32 s{S_IT}, 0')
-    L.append(f'"s_mov_b32 s{S_LDS}, %[lds]')
-    # the loads in the loop start with iteration 2
-    L.append(f'"s_add_u32 s{S_KA}, %[ga0], 256')
-    if nn:
-        L.append(f'"s_lshl_b32 s{S_T2}, %[kbs], 1')
-        L.append(f'"s_add_u32 s{S_KB}, %[gb0], s{S_T2}')
-    else:
-        L.append(f'"s_add_u32 s{S_KB}, %[gb0], 256')
-    L.append('"s_waitcnt vmcnt(16)')     # (the 16 youngest vector memory operations are the loads of the second stage)
-    L.append('"s_barrier')
+
+
+def spread(plan, groups, first, last):
+    """deals `groups` (lists of instruction texts) out over the free gaps among first .. last, in order and evenly"""
+    free = [g for g in range(first, last + 1) if g not in plan]
+    assert len(free) >= len(groups), (len(free), len(groups), first, last)
+    for k, item in enumerate(groups):
+        plan[free[(k * len(free)) // len(groups)]] = item
 
 
 def loop_text(nn):
-    """the lines of the loop for the NT (nn = False) or the NN layout"""
+    """The loop for the NT (nn = False) or the NN layout.  The two blocks of an iteration are built alike; block b
+    (K-step b of iteration `it`, fragment set b, stage cur = it % 2, nxt the other one):
+      top      reads of the LATE fragments (blocks 4-7 of A and B) of set b from cur -- their rows were the last to
+               be loaded and are the last to be overwritten
+      riders   reads of the EARLY fragments of the next K-step into the other set (b = 0: K-step 1 from cur, b = 1:
+               K-step 0 of it + 1 from nxt); eight loads (b = 0: the LATE row groups of it + 1 into nxt, b = 1: the
+               EARLY row groups of it + 2 into cur); address flips and, in block 1, the loop's scalar state
+      end      wait for the reads and for the eight loads issued a block earlier, barrier
+    so every load has between one and two blocks to land, and each block sends the same number of loads."""
     L = []
     e = L.append
     kb_step = "%[kbs]" if nn else "128"
     order = mfma_order()
+    n_early, n_late = len(early_groups(nn)), len(late_groups(nn))
 
     def mf(i, j, ab, bb):
         c = (8 * i + j) * 4
         return f'MF " a[{c}:{c + 3}], v[{bb + 4 * j}:{bb + 4 * j + 3}], v[{ab + 4 * i}:{ab + 4 * i + 3}], a[{c}:{c + 3}]'
 
-    # fragment reads as (tag, text); 16 rows of 128 bytes per block of A (NT: of B too)
+    # fragment reads as (tags, texts); 16 rows of 128 bytes per block of A (NT: of B too)
     def read_a(i, kk):
         ab, addr = (A0, "%[ra0]") if kk == 0 else (A1, "%[ra1]")
-        return (("A", kk, i), f'"ds_read_b128 v[{ab + 4 * i}:{ab + 4 * i + 3}], {addr} offset:{i * 2048}')
+        return ([("A", kk, i)], [f'"ds_read_b128 v[{ab + 4 * i}:{ab + 4 * i + 3}], {addr} offset:{i * 2048}'])
 
     def read_b(j, kk):
         bb = B0 if kk == 0 else B1
         if not nn:
             addr = "%[rb0]" if kk == 0 else "%[rb1]"
-            return [(("B", kk, j), f'"ds_read_b128 v[{bb + 4 * j}:{bb + 4 * j + 3}], {addr} offset:{j * 2048}')]
-        # NN: two halves of four K-rows each
-        return [(("B", kk, j), f'"ds_read_b64_tr_b16 v[{bb + 4 * j + 2 * h}:{bb + 4 * j + 2 * h + 1}], %[rbt{j}] offset:{kk * 16384 + h * 2048}')
-                for h in range(2)]
+            return ([("B", kk, j)], [f'"ds_read_b128 v[{bb + 4 * j}:{bb + 4 * j + 3}], {addr} offset:{j * 2048}'])
+        # NN: two halves of four K-rows each, issued together
+        return ([("B", kk, j)] * 2,
+                [f'"ds_read_b64_tr_b16 v[{bb + 4 * j + 2 * h}:{bb + 4 * j + 2 * h + 1}], %[rbt{j}] offset:{kk * 16384 + h * 2048}'
+                 for h in range(2)])
 
-    def reads_in_need_order(kk):
-        """A_0, B_0 .. B_7 (the first eight MFMAs need them in this order), then A_1 .. A_7 (one per eight MFMAs)"""
-        seq = [read_a(0, kk)]
-        for j in range(8):
-            seq += read_b(j, kk)
-        return seq + [read_a(i, kk) for i in range(1, 8)]
+    def early_reads(kk):    # in the order the first quadrant needs them
+        return [read_a(0, kk)] + [read_b(j, kk) for j in range(4)] + [read_a(i, kk) for i in range(1, 4)]
 
-    loop_entry(L, nn)
-    # the K-step-0 reads that block 1 of an iteration issues for the next one
-    k0_reads = reads_in_need_order(0)
-    n_ahead = len(k0_reads) - ROLL
-    tr = LdsTracker()
-    for tag, text in k0_reads[:n_ahead]:
-        e(text)
-        tr.issue(tag)
-    at_top = list(tr.q)
-    e('"s_nop 7')   # accumulator writes above are long done; cheap insurance before the first MFMA
-    e('"L_sk_loop%=:')
+    def late_reads(kk):     # B 4-7 are needed from the 17th MFMA on, A 4-7 from the 33rd
+        return [read_b(j, kk) for j in range(4, 8)] + [read_a(i, kk) for i in range(4, 8)]
 
-    # ---- block 0
-    tr = LdsTracker(at_top)
-    plan = {}       # gap -> [(tag or None, [texts])]
-    g = 0
-    for tag, text in k0_reads[n_ahead:]:
-        plan.setdefault(g, []).append((tag, [text]))
-        g += 1
-    k1_reads = reads_in_need_order(1)
-    first = max(RD0_FIRST, g)
-    for k, (tag, text) in enumerate(k1_reads):
-        plan.setdefault(first + (k * (RD0_LAST - first)) // (len(k1_reads) - 1), []).append((tag, [text]))
-    off = offsets_for(nn, 2)
-    misc = [['"v_xor_b32 %[ra0], 0x10000, %[ra0]']]             # (behind the reads at the top, which use it)
-    if not nn:
-        misc.append(['"v_xor_b32 %[rb0], 0x10000, %[rb0]'])
-    misc += [off[0:1], off[1:3]] + [[t] for t in off[3:]]        # (compare and select share a gap: nothing between them writes scc)
-    free = [x for x in range(g, 62) if x not in plan]
-    assert len(free) >= len(misc), (len(free), len(misc))
-    for k, texts in enumerate(misc):
-        plan.setdefault(free[(k * len(free)) // len(misc)], []).append((None, texts))
-    for m, (i, j) in enumerate(order):
-        w = tr.wait_for({("A", 0, i), ("B", 0, j)})
-        if w:
-            e(w)
-        e(mf(i, j, A0, B0))
-        for tag, texts in plan.get(m, []):
+    def load_groups(xs):
+        """loads as rider groups: the scalar instructions of a load share a gap, the load has its own"""
+        groups = []
+        for pre, m0, ld in load_sequence(xs, nn, f"v{VOA}", f"v{VOB}", f"v{VOB1}", f"s{S_LDS}", f"s{S_KA}", f"s{S_KB}"):
+            groups += [(None, pre + [m0]), (None, [ld])]
+        return groups
+
+    def block(b, tr, plan, closing):
+        ab, bb = (A0, B0) if b == 0 else (A1, B1)
+        for m, (i, j) in enumerate(order):
+            w = tr.wait_for({("A", b, i), ("B", b, j)})
+            if w:
+                e(w)
+            e(mf(i, j, ab, bb))
+            tags, texts = plan.get(m, (None, []))
             L.extend(texts)
-            if tag:
-                tr.issue(tag)
-    e('"s_waitcnt vmcnt(0) lgkmcnt(0)')
+            for t in tags or []:
+                tr.issue(t)
+        assert all(0 <= g < 64 for g in plan), sorted(plan)
+        L.extend(closing)
+
+    # ---- entry: accumulators to zero while the first stage is on its way; the loop's state: the loads of block 0 are
+    # those of iteration 1, into the second stage
+    zero_accumulators(L)
+    e(f'"s_mov_b32 s{S_IT}, 0')
+    e(f'"s_xor_b32 s{S_LDS}, %[lds], 0x10000')
+    e(f'"s_add_u32 s{S_KA}, %[ga0], 128')
+    e(f'"s_add_u32 s{S_KB}, %[gb0], {kb_step}')
+    L.extend(offsets_for(nn, 1))
+    # (the youngest vector memory operations are the early loads of the second stage; the first stage has landed)
+    e(f'"s_waitcnt vmcnt({n_early})')
     e('"s_barrier')
-    if nn:
-        # one address register per block of B serves both K-steps: they flip between the reads of block 0 and block 1
-        for j in range(8):
-            e(f'"v_xor_b32 %[rbt{j}], 0x10000, %[rbt{j}]')
+    at_top = []
+    for tags, texts in early_reads(0):
+        L.extend(texts)
+        at_top += tags
+    e('"s_nop 7')   # accumulator writes above are long done; cheap insurance before the first MFMA
+    flip = lambda reg: (None, [f'"v_xor_b32 {reg}, 0x10000, {reg}'])
 
-    # ---- block 1
-    tr = LdsTracker()
-    items = []      # (position in [0, 1), tie-break, tag or None, [texts])
-    groups = []
-    for x in range(16):
-        pre, m0, ld, adv = load_parts(x, nn, f"v{VOA}", f"v{VOB}", f"v{VOB1}", f"s{S_LDS}", f"s{S_KA}", f"s{S_KB}")
+    def body():
+        e('"L_sk_loop%=:')
+        # ---- block 0
+        plan = {}
+        for g, item in enumerate(late_reads(0)):
+            plan[g] = item
+        spread(plan, load_groups(late_groups(nn)), TOP, LD_LAST)
+        spread(plan, early_reads(1), TOP, RD_LAST)
+        # the addresses of set 0 move to the other stage behind the reads at the top (block 1 reads the early fragments
+        # of the next iteration with them); NN: one register per block of B serves both K-steps -- those of blocks 0-3
+        # flip between the early reads of block 0 and of block 1, those of blocks 4-7 behind the top reads of block 1
+        spread(plan, [flip("%[ra0]")] + ([] if nn else [flip("%[rb0]")]), TOP, 63)
+        # both ways into the loop: the early fragments of set 0 may still be in flight
+        block(0, LdsTracker(at_top), plan,
+              [f'"s_waitcnt vmcnt({n_late}) lgkmcnt(0)', '"s_barrier'])       # (the early loads, issued a block ago, have landed)
+
+        # ---- block 1
+        plan = {}
+        for g, item in enumerate(late_reads(1)):
+            plan[g] = item
+        state = [(None, [f'"s_add_u32 s{S_KA}, s{S_KA}, 128', f'"s_add_u32 s{S_KB}, s{S_KB}, {kb_step}']),
+                 (None, [f'"s_xor_b32 s{S_LDS}, s{S_LDS}, 0x10000', f'"s_add_u32 s{S_T2}, s{S_IT}, 2']),
+                 (None, [f'"s_cmp_lt_u32 s{S_T2}, %[n]', f'"s_cselect_b32 s{S_OOB}, 0, 0x80000000'])]
+        state += [(None, [t]) for t in offsets_for(nn, 2)[3:]]
         if nn:
-            # two gaps per load: the advance behind load x - 1 shares the gap of the m0 write of load x
-            groups += [([load_parts(x - 1, nn, "", "", "", "", "", "")[3]] if x not in (0, 8) else []) + pre + [m0], [ld]]
-        else:
-            groups += [pre + [m0], [ld]] + ([[adv]] if x not in (7, 15) else [])
-    for k, texts in enumerate(groups):
-        items.append(((k + 0.5) / len(groups), 0, None, texts))
-    ahead = k0_reads[:n_ahead]
-    for k, (tag, text) in enumerate(ahead):
-        items.append((0.05 + 0.9 * (k + 0.5) / len(ahead), 1, tag, [text]))
-    items.append((0.02, 2, None, ['"v_xor_b32 %[ra1], 0x10000, %[ra1]']))
-    if not nn:
-        items.append((0.5, 2, None, ['"v_xor_b32 %[rb1], 0x10000, %[rb1]']))
-    items.sort(key=lambda t: (t[0], t[1]))
-    tail = [[f'"s_add_u32 s{S_KA}, s{S_KA}, 128', f'"s_add_u32 s{S_KB}, s{S_KB}, {kb_step}'],
-            [f'"s_xor_b32 s{S_LDS}, s{S_LDS}, 0x10000', f'"s_add_u32 s{S_IT}, s{S_IT}, 1'],
-            [f'"s_cmp_lt_u32 s{S_IT}, %[n]', '"s_cbranch_scc1 L_sk_loop%=']]
-    ngaps = 64 - len(tail)
-    assert len(items) <= ngaps, (len(items), ngaps)
-    plan = {}
-    for k, it in enumerate(items):
-        plan.setdefault((k * ngaps) // len(items), []).append((it[2], it[3]))
-    for k, texts in enumerate(tail):
-        plan.setdefault(ngaps + k, []).append((None, texts))
-    for m, (i, j) in enumerate(order):
-        w = tr.wait_for({("A", 1, i), ("B", 1, j)})
-        if w:
-            e(w)
-        e(mf(i, j, A1, B1))
-        for tag, texts in plan.get(m, []):
-            L.extend(texts)
-            if tag:
-                tr.issue(tag)
-    assert tr.q == at_top, (tr.q, at_top)            # both ways into the loop leave the same reads in flight
+            state += [flip(f"%[rbt{j}]") for j in range(4)]
+        for g, item in enumerate(state):
+            plan[TOP + g] = item
+        after_state = TOP + len(state)
+        plan[63] = (None, [f'"s_add_u32 s{S_IT}, s{S_IT}, 1'])
+        spread(plan, load_groups(early_groups(nn)), after_state, LD_LAST)
+        spread(plan, early_reads(0), after_state, RD_LAST)
+        spread(plan, [flip("%[ra1]")] + ([flip(f"%[rbt{j}]") for j in range(4, 8)] if nn else [flip("%[rb1]")]), after_state, 62)
+        block(1, LdsTracker(), plan,
+              [f'"s_waitcnt vmcnt({n_early}) lgkmcnt(0)', '"s_barrier',           # (the late loads of iteration it + 1 have landed)
+               f'"s_cmp_lt_u32 s{S_IT}, %[n]', '"s_cbranch_scc1 L_sk_loop%='])
+
+    body()
     for a, b in zip(L, L[1:]):                       # one instruction between an m0 write and the load that uses it
         assert not ("m0" in a and "buffer_load" in b), (a, b)
     # ---- drain: the empty loads of the last two iterations still write LDS; the accumulators must have left
@@ -307,10 +331,17 @@ def loop_text_f8():
         e(f'MF " a[{c}:{c + 3}], v[{B8(j)}:{B8(j) + 7}], v[{A8(i)}:{A8(i) + 7}], a[{c}:{c + 3}] " MOD "')
 
     def dma(x):
-        pre, m0, ld, adv = load_parts(x, False, f"v{VOA}", f"v{VOB}", f"v{VOB1}", f"s{S_LDS}", f"s{S_KA}", f"s{S_KB}")
-        L.extend(pre + [m0, '"s_nop 0', ld, adv])
+        pre, m0, ld = load_parts(x, False, f"v{VOA}", f"v{VOB}", f"v{VOB1}", f"s{S_LDS}", f"s{S_KA}", f"s{S_KB}",
+                                 None if x in (0, 8) else x - 1)
+        L.extend(pre + [m0, '"s_nop 0', ld])
 
-    loop_entry(L, False)
+    zero_accumulators(L)
+    e(f'"s_mov_b32 s{S_IT}, 0')
+    e(f'"s_mov_b32 s{S_LDS}, %[lds]')
+    e(f'"s_add_u32 s{S_KA}, %[ga0], 256')     # the loads in the loop start with iteration 2
+    e(f'"s_add_u32 s{S_KB}, %[gb0], 256')
+    e('"s_waitcnt vmcnt(16)')     # (the 16 youngest vector memory operations are the loads of the second stage)
+    e('"s_barrier')
     tr = LdsTracker()
     for i in range(4):
         for h in range(2):
@@ -445,8 +476,10 @@ def main():
     print("// NT / NN layout, MF = the MFMA mnemonic as a string literal.  SK_TILE_ASM_LOOP_F8(MF, MOD): fp8 operands, MOD =")
     print("// the format modifiers of the MFMA (\"\" for e4m3).  SK_TILE_ASM_STORE_x(CVT): the epilogue that leaves the stages alone.")
     print("#pragma once")
-    emit_macro("SK_TILE_ASM_LOADS", "", stage_loads_text(False))
-    emit_macro("SK_TILE_ASM_LOADS_NN", "", stage_loads_text(True))
+    emit_macro("SK_TILE_ASM_LOADS", "", stage_loads_text(False, range(16)))
+    emit_macro("SK_TILE_ASM_LOADS_NN", "", stage_loads_text(True, range(16)))
+    emit_macro("SK_TILE_ASM_LOADS_EARLY", "", stage_loads_text(False, early_groups(False)))
+    emit_macro("SK_TILE_ASM_LOADS_EARLY_NN", "", stage_loads_text(True, early_groups(True)))
     emit_macro("SK_TILE_ASM_LOOP", "(MF)", loop_text(False))
     emit_macro("SK_TILE_ASM_LOOP_NN", "(MF)", loop_text(True))
     emit_macro("SK_TILE_ASM_LOOP_F8", "(MF, MOD)", loop_text_f8())

@@ -143,25 +143,30 @@ struct TileF16Asm {
     return c;
   }
 
-  // the 16 loads of stage `stage` (iteration k0 + stage of the segment; nothing is fetched if the segment is shorter)
+  // the 16 loads of stage `stage` (iteration k0 + stage of the segment; nothing is fetched if the segment is shorter),
+  // or -- EARLY_ONLY -- just those the loop does not send itself: the row groups that hold blocks 0-3 of the wave tiles
+  // (NN: and all of B); see gen_tile_asm.py
+  template <bool EARLY_ONLY = false>
   static __device__ __forceinline__ void stage_loads(const Ctx &c, int stage, int n) {
     const uint32_t oob = stage < n ? 0u : OOB_OFFSET;
     const uint32_t voa = c.voff_a | oob, vob = c.voff_b | oob, vob1 = c.voff_b1 | oob;
     const uint32_t ga = c.goff_a + (uint32_t)stage * 128, gb = c.goff_b + (uint32_t)stage * c.kstep_b;
     const uint32_t lds_stage = c.lds_wave + (uint32_t)stage * STAGE_BYTES;
-    if constexpr (NN_) {
-      asm volatile(SK_TILE_ASM_LOADS_NN
-                   :
-                   : [rsa] "s"(c.rsrc_a), [rsb] "s"(c.rsrc_b), [voa] "v"(voa), [vob] "v"(vob), [vob1] "v"(vob1), [ga] "s"(ga),
-                     [gb] "s"(gb), [gas] "s"(c.gstep_a), [gbs] "s"(c.gstep_b), [lds] "s"(lds_stage)
-                   : "memory", "m0", "scc", "s83");
+#define SK_ASM_LOAD_OPERANDS                                                                                             \
+  : : [rsa] "s"(c.rsrc_a), [rsb] "s"(c.rsrc_b), [voa] "v"(voa), [vob] "v"(vob), [vob1] "v"(vob1), [ga] "s"(ga),            \
+      [gb] "s"(gb), [gas] "s"(c.gstep_a), [gas2] "s"(2 * c.gstep_a), [gas3] "s"(3 * c.gstep_a), [gbs] "s"(c.gstep_b),     \
+      [gbs2] "s"(2 * c.gstep_b), [gbs3] "s"(3 * c.gstep_b), [lds] "s"(lds_stage)                                          \
+  : "memory", "m0", "scc", "s83"
+    if constexpr (NN_ && EARLY_ONLY) {
+      asm volatile(SK_TILE_ASM_LOADS_EARLY_NN SK_ASM_LOAD_OPERANDS);
+    } else if constexpr (NN_) {
+      asm volatile(SK_TILE_ASM_LOADS_NN SK_ASM_LOAD_OPERANDS);
+    } else if constexpr (EARLY_ONLY) {
+      asm volatile(SK_TILE_ASM_LOADS_EARLY SK_ASM_LOAD_OPERANDS);
     } else {
-      asm volatile(SK_TILE_ASM_LOADS
-                   :
-                   : [rsa] "s"(c.rsrc_a), [rsb] "s"(c.rsrc_b), [voa] "v"(voa), [vob] "v"(vob), [ga] "s"(ga), [gb] "s"(gb),
-                     [gas] "s"(c.gstep_a), [gbs] "s"(c.gstep_b), [lds] "s"(lds_stage)
-                   : "memory", "m0", "scc", "s83");
+      asm volatile(SK_TILE_ASM_LOADS SK_ASM_LOAD_OPERANDS);
     }
+#undef SK_ASM_LOAD_OPERANDS
   }
 
   // Cross-segment prefetch (see run_persistent): the first stage of the NEXT segment is requested as soon as every
@@ -177,15 +182,17 @@ struct TileF16Asm {
                                              bool first_stage_requested = false) {
     Ctx c = make_ctx(a, pm, pn, k0);
     if (!first_stage_requested) stage_loads(c, 0, n);
-    stage_loads(c, 1, n);  // (directly ahead of the loop, whose first wait counts on these being the 16 youngest operations)
+    // (directly ahead of the loop, whose first wait counts on these being the youngest operations; the 16-bit loops
+    // send the late row groups of the second stage themselves)
+    stage_loads<F8 == 0>(c, 1, n);
     const uint32_t iters = (uint32_t)n;
     if constexpr (NN_) {
 #define SK_ASM_NN_OPERANDS                                                                                            \
   : [ra0] "+v"(c.ra0), [ra1] "+v"(c.ra1), [rbt0] "+v"(c.rbt[0]), [rbt1] "+v"(c.rbt[1]), [rbt2] "+v"(c.rbt[2]),          \
     [rbt3] "+v"(c.rbt[3]), [rbt4] "+v"(c.rbt[4]), [rbt5] "+v"(c.rbt[5]), [rbt6] "+v"(c.rbt[6]), [rbt7] "+v"(c.rbt[7])  \
   : [rsa] "s"(c.rsrc_a), [rsb] "s"(c.rsrc_b), [voa] "v"(c.voff_a), [vob] "v"(c.voff_b), [vob1] "v"(c.voff_b1),          \
-    [ga0] "s"(c.goff_a), [gb0] "s"(c.goff_b), [gas] "s"(c.gstep_a), [gbs] "s"(c.gstep_b), [kbs] "s"(c.kstep_b),         \
-    [n] "s"(iters), [lds] "s"(c.lds_wave)                                                                             \
+    [ga0] "s"(c.goff_a), [gb0] "s"(c.goff_b), [gas] "s"(c.gstep_a), [gas2] "s"(2 * c.gstep_a),                          \
+    [gas3] "s"(3 * c.gstep_a), [gbs] "s"(c.gstep_b), [kbs] "s"(c.kstep_b), [n] "s"(iters), [lds] "s"(c.lds_wave)        \
   : "memory", "m0", "scc", SK_TILE_ASM_CLOBBERS
       if constexpr (BF16_) {
         asm volatile(SK_TILE_ASM_LOOP_NN("v_mfma_f32_16x16x32_bf16") SK_ASM_NN_OPERANDS);
@@ -197,7 +204,8 @@ struct TileF16Asm {
 #define SK_ASM_NT_OPERANDS                                                                                          \
   : [ra0] "+v"(c.ra0), [ra1] "+v"(c.ra1), [rb0] "+v"(c.rb0), [rb1] "+v"(c.rb1)                                      \
   : [rsa] "s"(c.rsrc_a), [rsb] "s"(c.rsrc_b), [voa] "v"(c.voff_a), [vob] "v"(c.voff_b), [ga0] "s"(c.goff_a),          \
-    [gb0] "s"(c.goff_b), [gas] "s"(c.gstep_a), [gbs] "s"(c.gstep_b), [n] "s"(iters), [lds] "s"(c.lds_wave)            \
+    [gb0] "s"(c.goff_b), [gas] "s"(c.gstep_a), [gas2] "s"(2 * c.gstep_a), [gas3] "s"(3 * c.gstep_a),                  \
+    [gbs] "s"(c.gstep_b), [gbs2] "s"(2 * c.gstep_b), [gbs3] "s"(3 * c.gstep_b), [n] "s"(iters), [lds] "s"(c.lds_wave)  \
   : "memory", "m0", "scc", SK_TILE_ASM_CLOBBERS
       if constexpr (F8 == 1) {
         asm volatile(SK_TILE_ASM_LOOP_F8("v_mfma_f32_16x16x128_f8f6f4", "") SK_ASM_NT_OPERANDS);
