@@ -235,7 +235,7 @@ struct TileFamily {
   float tau, gamma, o, phi;
 };
 static const TileFamily kFamilies16[] = {
-    {256, 256, 64, 7, 1, 4, 0.999f, 0.20f, 8.4f, 6.0f},   // four waves, K loop in assembly (K % 64 == 0)
+    {256, 256, 64, 7, 1, 4, 0.919f, 0.20f, 6.4f, 6.9f},   // four waves, K loop in assembly (K % 64 == 0)
     {256, 256, 64, 4, 1, 2, 1.080f, 0.20f, 9.3f, 10.0f},  // eight waves, for the other K
     {128, 128, 64, 4, 2, 4, 0.497f, 0.47f, 4.9f, 5.1f},
     {128, 128, 32, 5, 2, 4, 0.218f, 0.89f, 3.8f, 4.5f},   // four stages of 32 (NT only)
@@ -254,7 +254,7 @@ static const TileFamily kFamiliesF8[] = {
     {64, 128, 64, 5, 3, 4, 0.135f, 1.00f, 2.9f, 8.6f},
 };
 static const TileFamily kFamiliesI8[] = {
-    {256, 256, 128, -1, 1, 4, 0.962f, 0.20f, 13.3f, 4.2f},
+    {256, 256, 128, -1, 1, 4, 0.876f, 0.20f, 13.3f, 4.2f},
     {128, 128, 128, -1, 2, 2, 0.531f, 0.52f, 2.3f, 6.4f},
     {128, 256, 128, -1, 1, 2, 0.674f, 0.20f, 6.5f, 6.5f},
     {256, 128, 128, -1, 1, 2, 0.700f, 1.00f, 4.9f, 6.5f},

@@ -1863,6 +1863,48 @@ def test_fp32_reference_shape(sk, oracle):
     sk.workspace_status()
 
 
+def test_reference_run_shapes(sk, oracle):
+    """The shapes the reference's own scripts run: fp16 NT 16 x 16384 x 8192 (streamk.fp16.breakdown/
+    streamk_fp16_nt.py:15, streamk_fp16_block_reduce.py:66) and Q4 16 x 16384 x 16384 (streamk_fp16_ladder_block_reduce_q4
+    .py:73), with the tuned plan, the untuned default and the schedules the reference uses there (Stream-K over every
+    tile, both fix-ups).  fp16: against the fp32 host product of the same fp16 inputs; Q4: against the host product with
+    the dequantised weights on a slice of 1024 weight rows (the full host product takes a minute), and the standalone
+    dequant of all rows bit for bit."""
+    rng = np.random.default_rng(16384)
+    M, N, K = 16, 16384, 8192
+    A, B = _uniform16((M, K), 31), _uniform16((N, K), 32)
+    ref = oracle.matmul_fp32(A, B, trans_b=True)
+    dA, dB = _t(A), _t(B)
+    tuned, untuned = sk.make_plan(M, N, K, "float16", "nt"), sk.make_plan(M, N, K, "float16", "nt", use_tuned=False)
+    for cfg in (dict(plan=tuned), dict(plan=untuned), dict(bm=16, bn=16, bk=512, schedule="dp"),
+                dict(schedule="basic", fixup="reduce"), dict(schedule="basic", fixup="atomic"),
+                dict(bm=16, bn=64, bk=128, schedule="sk2", grid=512, fixup="reduce")):
+        C = sk.streamk_fp16(dA, dB, **cfg)
+        assert _rel(oracle, C, ref) <= 2e-3 <= TOL, cfg
+    del dB
+    N, K = 16384, 16384
+    A = rng.standard_normal((M, K), dtype=np.float32).astype(np.float16)
+    Wq = rng.integers(0, 256, (N, K // 2), dtype=np.uint8)
+    sc = rng.uniform(0.005, 0.02, (N, K // 128)).astype(np.float16)
+    rows = slice(9000, 10024)
+    ref = oracle.q4_gemm_ref(A, Wq[rows], sc[rows], 128, 8)
+    dA, dW, dS = _t(A), _t(Wq), _t(sc)
+    W = sk.dequant_q4(dW[rows], dS[rows]).cpu().numpy()
+    assert np.array_equal(W.view(np.uint16), oracle.dequant_q4(Wq[rows], sc[rows], 128, 8).view(np.uint16))
+    first = None
+    for cfg in (dict(), dict(plan=sk.make_plan(M, N, K, "q4", "nt", use_tuned=False)), dict(schedule="dp"),
+                dict(fixup="reduce", schedule="basic", grid=256),
+                dict(fixup="atomic", schedule="basic", grid=256), dict(bm=16, bn=64, bk=512, schedule="dp")):
+        C = sk.streamk_q4(dA, dW, dS, **cfg)
+        assert _rel(oracle, C[:, rows], ref) <= 2e-3 <= TOL, cfg
+        # every plan multiplies the same decoded weights: outside the checked slice the results agree with each other
+        if first is None:
+            first = C.float()
+        else:
+            assert float((C.float() - first).abs().max()) <= 2e-3 * float(first.abs().max()), cfg
+    sk.workspace_status()
+
+
 def test_linear_layers_replay_in_a_graph(sk):
     """A decode step as a serving loop would capture it: three StreamKLinear layers (fp16, Q4 with bias, Q4 with
     per-group zero points and bias) for a batch of 4 rows in one graph, replayed several times with new inputs
