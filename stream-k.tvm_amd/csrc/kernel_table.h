@@ -240,6 +240,21 @@ struct KernelInfo {
   X(210, 4, 1, 4, 4)                 \
   X(211, 4, 2, 4, 2)
 
+// Up to 16 / 32 / 64 rows of A, fp16 / bfloat16 weights (NT), the weights streaming through LDS in contiguous loads
+// (tile_stream_pairs.h; variant 4):  X(id, MB, WM, WN, RK, DEPTH)
+#define SK_STREAM_PAIRS_F16_KERNELS(X) \
+  X(280, 1, 1, 4, 1, 4)                \
+  X(281, 2, 1, 4, 1, 3)                \
+  X(284, 1, 1, 2, 2, 3)                \
+  X(286, 2, 2, 2, 1, 3)                \
+  X(288, 1, 2, 2, 1, 4)
+#define SK_STREAM_PAIRS_BF16_KERNELS(X) \
+  X(282, 1, 1, 4, 1, 4)                 \
+  X(283, 2, 1, 4, 1, 3)                 \
+  X(285, 1, 1, 2, 2, 3)                 \
+  X(287, 2, 2, 2, 1, 3)                 \
+  X(289, 1, 2, 2, 1, 4)
+
 // bfloat16 twins of the fp16 matrix-vector kernels (dtype SK_BF16, variant 2)
 #define SK_GEMV_BF16_KERNELS(X) \
   X(241, 1, 1, 4, 4, 8192)      \

@@ -1,5 +1,6 @@
 // Small-M kernels in the matrix-vector kernels' form (tile_gemv_rows.h): 2 <= M <= 16, fp16 / bfloat16, NT;
-// and the Q4 kernels for per-group zero points with tiled weights (dtype 9, SK_Q4_ZP_TILED).
+// the Q4 kernels for per-group zero points with tiled weights (dtype 9, SK_Q4_ZP_TILED); and the kernels that stream
+// fp16 / bfloat16 weights through LDS in contiguous loads (tile_stream_pairs.h).
 #include "skinny_launch.h"
 
 namespace sk {
@@ -39,6 +40,22 @@ int gemv_rows_kernel_infos(KernelInfo *out, int max) {
   }
   SK_SKINNY_Q4ZPT_KERNELS(X)
 #undef X
+#define X(id, MB, WM, WN, RK, DEPTH)                                                                                       \
+  if (n < max) {                                                                                               \
+    typedef TileStreamPairs<MB, WM, WN, RK, DEPTH, false> P;                                                               \
+    out[n++] = KernelInfo{id, FAMILY_SKINNY, 0, 0, 4, P::BM, P::BN, P::BKC, P::NT, P::LDS_BYTES, P::CTAS_PER_CU, \
+                          P::TILE_ELEMS, 0, P::MAX_M, 8, "stream_f16_mb" #MB "_wm" #WM "_wn" #WN "_rk" #RK "_d" #DEPTH};                      \
+  }
+  SK_STREAM_PAIRS_F16_KERNELS(X)
+#undef X
+#define X(id, MB, WM, WN, RK, DEPTH)                                                                                       \
+  if (n < max) {                                                                                               \
+    typedef TileStreamPairs<MB, WM, WN, RK, DEPTH, true> P;                                                                \
+    out[n++] = KernelInfo{id, FAMILY_SKINNY, 3, 0, 4, P::BM, P::BN, P::BKC, P::NT, P::LDS_BYTES, P::CTAS_PER_CU, \
+                          P::TILE_ELEMS, 0, P::MAX_M, 8, "stream_bf16_mb" #MB "_wm" #WM "_wn" #WN "_rk" #RK "_d" #DEPTH};                     \
+  }
+  SK_STREAM_PAIRS_BF16_KERNELS(X)
+#undef X
   return n;
 }
 
@@ -71,6 +88,20 @@ int launch_gemv_rows(int id, const SkinnyArgs &a, const DevPlan &p, const Worksp
     return launch_policy<P>(a, p, ws, s, bias);                            \
   }
     SK_SKINNY_Q4ZPT_KERNELS(X)
+#undef X
+#define X(id_, MB, WM, WN, RK, DEPTH)                              \
+  case id_: {                                          \
+    typedef TileStreamPairs<MB, WM, WN, RK, DEPTH, false> P;       \
+    return launch_policy<P>(a, p, ws, s, bias);        \
+  }
+    SK_STREAM_PAIRS_F16_KERNELS(X)
+#undef X
+#define X(id_, MB, WM, WN, RK, DEPTH)                              \
+  case id_: {                                          \
+    typedef TileStreamPairs<MB, WM, WN, RK, DEPTH, true> P;        \
+    return launch_policy<P>(a, p, ws, s, bias);        \
+  }
+    SK_STREAM_PAIRS_BF16_KERNELS(X)
 #undef X
   }
   return (int)hipErrorInvalidValue;
@@ -114,6 +145,24 @@ int occupancy_gemv_rows(int id) {
     return occ;                                                                                          \
   }
     SK_SKINNY_Q4ZPT_KERNELS(X)
+#undef X
+#define X(id_, MB, WM, WN, RK, DEPTH)                                                                                \
+  case id_: {                                                                                            \
+    typedef TileStreamPairs<MB, WM, WN, RK, DEPTH, false> P;                                                         \
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_skinny_kernel<P>, P::NT, 0) != hipSuccess) \
+      return -1;                                                                                         \
+    return occ;                                                                                          \
+  }
+    SK_STREAM_PAIRS_F16_KERNELS(X)
+#undef X
+#define X(id_, MB, WM, WN, RK, DEPTH)                                                                                \
+  case id_: {                                                                                            \
+    typedef TileStreamPairs<MB, WM, WN, RK, DEPTH, true> P;                                                          \
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_skinny_kernel<P>, P::NT, 0) != hipSuccess) \
+      return -1;                                                                                         \
+    return occ;                                                                                          \
+  }
+    SK_STREAM_PAIRS_BF16_KERNELS(X)
 #undef X
   }
   return -1;

@@ -53,8 +53,11 @@ static int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // preference among kernel variants of one tile shape when the caller does not ask for one: the
 // eight-wave direct-to-LDS tile kernels; the most specialised small-M kernel that accepts the shape
 static int variant_rank(const KernelInfo &k) {
-  // (small-M: general 0 < rows-of-A matrix-vector form 3 < single-row 1 < matrix-vector 2)
-  if (k.family == FAMILY_SKINNY) return k.variant == 3 ? 1 : (k.variant == 0 ? 0 : k.variant + 1);
+  // (small-M: general 0 < rows-of-A matrix-vector form 3 < single-row 1 < matrix-vector 2; the kernels that stream
+  // the weights through LDS, variant 4, share tile shapes with general kernels and are taken when asked for by
+  // variant, or by the default rule below)
+  if (k.family == FAMILY_SKINNY)
+    return k.variant == 4 ? -1 : (k.variant == 3 ? 1 : (k.variant == 0 ? 0 : k.variant + 1));
   return k.variant == 7 ? 4 : (k.variant == 4 ? 3 : (k.variant == 1 ? 2 : (k.variant == 2 ? 1 : 0)));
 }
 static bool accepts_shape(const KernelInfo &k, int64_t M, int64_t K) {
@@ -99,6 +102,17 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
     for (int i = 0; i < n; ++i)
       if (t[i].family == FAMILY_TILE && t[i].dtype == SK_Q4 && t[i].bm == want_bm && t[i].bn == want_bn) return &t[i];
     return nullptr;
+  }
+  if ((dtype == SK_F16 || dtype == SK_BF16) && layout == SK_LAYOUT_NT && M >= 5 && M <= 64 && want_variant < 0) {
+    // 5 <= M <= 64 with fp16 / bfloat16 weights: the kernels that stream the weights through LDS in contiguous loads
+    // (tile_stream_pairs.h).  Tiles of 32 weight rows while one wave of them fits the device (N = 8192: one tile per
+    // CU and no fix-up), 64 rows beyond; 64 rows of A exist with 32 weight rows only.
+    const bool narrow = cdiv(N, 32) <= num_cus || M > 32;
+    const int bm = M <= 16 ? 16 : (M <= 32 ? 32 : 64), bn = narrow ? 32 : 64, bk = (bm == 16 && narrow) ? 512 : 256;
+    for (int i = 0; i < n; ++i)
+      if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].variant == 4 && t[i].bm == bm && t[i].bn == bn &&
+          t[i].bk == bk && accepts_shape(t[i], M, K))
+        return &t[i];
   }
   if ((M <= (one_byte ? 64 : 32) && layout == SK_LAYOUT_NT) || q4) {
     // M == 1 with Q4 weights: the matrix-vector kernel with four waves splitting K (data-parallel
@@ -425,6 +439,10 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
     const int64_t waves = (total64 + grid - 1) / grid;
     if (total64 * 10 >= waves * grid * 9) sched = SK_SCHED_DP;
     else sched = total64 >= 2 * (int64_t)grid ? SK_SCHED_SK_ONE_TILE : SK_SCHED_SK_TWO_TILE;
+    // (the kernels that stream the weights through LDS are bound by memory, not by the busiest CU: an uneven last
+    // wave costs them less than the fix-up; 16 x 28672 x 8192: 77.8 us data-parallel against 83.6 us.  With 64 rows of
+    // A it is the other way round: 110 us against 103 us)
+    if (k->family == FAMILY_SKINNY && k->variant == 4 && k->bm == 16 && total64 >= grid) sched = SK_SCHED_DP;
     if (k->family == FAMILY_TILE && sched != SK_SCHED_DP) {
       // Fewer tiles than CUs: the idle CUs are put to work by an aligned split in two or four, never by CTA ranges
       // that start anywhere.  More tiles than CTAs: see

@@ -265,6 +265,18 @@ __device__ __forceinline__ void dma_load_16(uint4v rsrc, uint32_t lds_base, uint
                : "s"(lds_base), "v"(lane_off), "s"(rsrc), "s"(uniform_off)
                : "memory", "m0");
 }
+// Kernels that stream weight rows in long contiguous pieces (tile_stream_pairs.h) start their CTAs together, and the
+// pitch of the rows is a large power of two: walking every tile from K = 0 has all CTAs read the same K offset of
+// their rows at the same moment, which the memory system serves badly (N = K = 8192 fp16, 16 rows of A: 33.3 us;
+// 27.8 us when neighbouring tiles start one iteration apart; 24.6 us with the starts below).  Tile pn starts
+// rot = (3 pn + pn / 16) % n iterations into its segment of n iterations and wraps around; iterations past the
+// segment keep their number (their loads fetch nothing).  The sum of a tile is therefore added up in a K order that
+// depends on the tile, the same on every launch.
+__device__ __forceinline__ int rotation_of(int pn, int n) { return n > 0 ? (3 * pn + (pn >> 4)) % n : 0; }
+__device__ __forceinline__ int rotated_iteration(int t, int rot, int n) {
+  const int r = t + rot;
+  return t >= n ? t : (r >= n ? r - n : r);
+}
 __device__ __forceinline__ uint32_t lds_address(const void *p) {
   return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)p;
 }

@@ -66,9 +66,14 @@ SKINNY_CONFIGS = [
     dict(bm=16, bn=16, bk=512), dict(bm=16, bn=32, bk=256),
     dict(bm=16, bn=32, bk=512, variant=1), dict(bm=16, bn=64, bk=256), dict(bm=32, bn=64, bk=256), dict(bm=64, bn=64, bk=256),
 ]
+# variant 5 of the small-M shapes: the weights stream through LDS in contiguous loads
+STREAM_CONFIGS = [
+    dict(bm=16, bn=64, bk=256, variant=5), dict(bm=32, bn=64, bk=256, variant=5), dict(bm=16, bn=32, bk=512, variant=5),
+    dict(bm=64, bn=32, bk=256, variant=5), dict(bm=32, bn=32, bk=256, variant=5),
+]
 
 
-@pytest.mark.parametrize("cfg", TILE_CONFIGS + SKINNY_CONFIGS, ids=lambda c: f"{c['bm']}x{c['bn']}x{c['bk']}v{c.get('variant', 0)}")
+@pytest.mark.parametrize("cfg", TILE_CONFIGS + SKINNY_CONFIGS + STREAM_CONFIGS, ids=lambda c: f"{c['bm']}x{c['bn']}x{c['bk']}v{c.get('variant', 0)}")
 @pytest.mark.parametrize("sched,fixup,grid", [("dp", "reduce", 8), ("basic", "reduce", 8),
                                              ("basic", "atomic", 8), ("sk2", "reduce", 3),
                                              ("sk2", "atomic", 5)])
@@ -999,6 +1004,59 @@ def test_f16_few_rows_in_the_matrix_vector_form(sk, oracle):
     sk.workspace_status()
 
 
+def test_f16_weights_streamed_through_lds(sk, oracle):
+    """Up to 64 rows of A on the kernels that stream the weights through LDS in contiguous loads (five wave
+    arrangements, fp16 and bfloat16): ragged M and N, K a multiple of 8 only and shorter than one iteration, strided A
+    and W, all schedules and both fix-ups, bias and activation, an output with a row stride; exact on integer data
+    (every tile adds its K-iterations up from a different start), within 2e-3 of the fp32 host product otherwise."""
+    import torch
+    rng = np.random.default_rng(74)
+    ran = 0
+    shapes = {16: (16, 64, 256), 32: (32, 64, 256), 17: (16, 32, 512), 64: (64, 32, 256), 33: (32, 32, 256)}
+    for (M, N, K, pad) in [(16, 1000, 1160, 0), (9, 520, 392, 8), (1, 72, 8, 0), (13, 2048, 8192, 64), (5, 264, 28672, 0),
+                           (64, 4099, 4104, 0), (50, 328, 776, 8), (32, 200, 1032, 0), (27, 8192, 4096, 0)]:
+        A = (rng.random((M, K + pad), dtype=np.float32) * 2 - 1).astype(np.float16)
+        W = (rng.random((N, K + pad), dtype=np.float32) * 2 - 1).astype(np.float16)
+        Ai = rng.integers(-1, 2, (M, K + pad)).astype(np.float16)
+        Wi = rng.integers(-2, 3, (N, K + pad)).astype(np.float16)
+        ref = oracle.matmul_fp32(A[:, :K], W[:, :K], trans_b=True)
+        exact = Ai[:, :K].astype(np.int64) @ Wi[:, :K].astype(np.int64).T
+        assert np.abs(exact).max() < 2048
+        dA, dW, dAi, dWi = _t(A)[:, :K], _t(W)[:, :K], _t(Ai)[:, :K], _t(Wi)[:, :K]
+        for (bm, bn, bk) in shapes.values():
+            if M > bm:
+                with pytest.raises(sk.StreamKError):
+                    sk.make_plan(M, N, K, "float16", "nt", dict(bm=bm, bn=bn, bk=bk, variant=5))
+                continue
+            for sch in (dict(schedule="dp"), dict(schedule="sk2", fixup="reduce", grid=48),
+                        dict(schedule="sk2", fixup="atomic", grid=40), dict(schedule="basic", fixup="reduce", grid=56)):
+                plan = sk.make_plan(M, N, K, "float16", "nt", dict(bm=bm, bn=bn, bk=bk, variant=5, **sch))
+                assert sk.kernel_name(plan.kernel_id).startswith("stream_f16_")
+                C = sk.streamk_fp16(dA, dW, plan=plan)
+                assert _rel(oracle, C, ref) <= 2e-3 <= TOL, (M, N, K, bm, bn, bk, sch)
+                C = sk.streamk_fp16(dAi, dWi, plan=plan)
+                assert np.array_equal(C.cpu().numpy().astype(np.int64), exact), (M, N, K, bm, bn, bk, sch)
+                pb = sk.make_plan(M, N, K, "bfloat16", "nt", dict(bm=bm, bn=bn, bk=bk, variant=5, **sch))
+                assert sk.kernel_name(pb.kernel_id).startswith("stream_bf16_")
+                C = sk.streamk_bf16(dAi.bfloat16(), dWi.bfloat16(), plan=pb)
+                # (the exact sums, rounded once to bfloat16's eight bits)
+                assert torch.equal(C.cpu(), torch.from_numpy(exact).float().bfloat16()), (M, N, K, bm, bn, bk, sch)
+                ran += 1
+    assert ran >= 100
+    # bias and activation, an output with a row stride
+    M, N, K = 48, 1000, 2048
+    Ai = rng.integers(-1, 2, (M, K)).astype(np.float16)
+    Wi = rng.integers(-1, 2, (N, K)).astype(np.float16)
+    bias = rng.integers(-3, 4, N).astype(np.float16)
+    want = np.maximum(Ai.astype(np.int64) @ Wi.astype(np.int64).T + bias.astype(np.int64), 0)
+    for sch in (dict(schedule="dp"), dict(schedule="sk2", fixup="reduce", grid=64), dict(schedule="sk2", fixup="atomic", grid=64)):
+        out = torch.zeros(M, N + 24, dtype=torch.float16, device="cuda")[:, 8:8 + N]
+        C = sk.streamk_fp16(_t(Ai), _t(Wi), out=out, bias=_t(bias), activation="relu", bm=64, bn=32, bk=256, variant=5, **sch)
+        assert np.array_equal(C.cpu().numpy().astype(np.int64), want), sch
+    sk.workspace_status()
+
+
+@pytest.mark.gpu
 def test_device_quantiser_matches_host_and_feeds_the_gemm(sk, oracle):
     """sk_q4_quantize on the device writes the bytes sk_q4_quantize_host and the numpy restatement
     write (special groups included), and a Q4 GEMM on the result agrees with the fp32 product of
@@ -1149,8 +1207,10 @@ def test_bf16_small_m_kernels(sk, oracle):
                     assert torch.equal(C, sk.streamk_bf16(A.cuda(), B.cuda(), plan=plan))
     for M in (1, 2, 16, 32):
         plan = sk.make_plan(M, 4096, 4096, "bfloat16", "nt")
-        # (one row: matrix-vector kernels; two to four rows: their form with four rows of A; else the general kernels)
-        assert (241 <= plan.kernel_id <= 248) if M == 1 else ((210 <= plan.kernel_id <= 211) if M <= 4 else (230 <= plan.kernel_id <= 240)), (M, plan.kernel_id)
+        # (one row: matrix-vector kernels; two to four rows: their form with four rows of A; else the general kernels
+        # or the ones that stream the weights through LDS)
+        assert (241 <= plan.kernel_id <= 248) if M == 1 else ((210 <= plan.kernel_id <= 211) if M <= 4 else
+                                                               (230 <= plan.kernel_id <= 240 or plan.kernel_id in (282, 283, 285, 287, 289))), (M, plan.kernel_id)
         A, W = (torch.rand(M, 4096) * 2 - 1).bfloat16(), (torch.rand(4096, 4096) * 2 - 1).bfloat16()
         ref = oracle.matmul_fp32(A.float().numpy(), W.float().numpy(), trans_b=True)
         assert _rel(oracle, sk.streamk_bf16(A.cuda(), W.cuda()), ref) <= 4e-3, M
