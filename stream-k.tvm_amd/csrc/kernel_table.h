@@ -255,6 +255,12 @@ struct KernelInfo {
   X(287, 2, 2, 2, 1, 3)                 \
   X(289, 1, 2, 2, 1, 4)
 
+// Up to 16 rows of A, Q4 weights (row-major, scalar zero point) streaming through LDS in contiguous loads
+// (tile_stream_q4.h; dtype SK_Q4, variant 4):  X(id, WN, RK, WD, AD)
+#define SK_STREAM_Q4_KERNELS(X) \
+  X(290, 4, 1, 5, 4)            \
+  X(291, 2, 2, 5, 2)
+
 // bfloat16 twins of the fp16 matrix-vector kernels (dtype SK_BF16, variant 2)
 #define SK_GEMV_BF16_KERNELS(X) \
   X(241, 1, 1, 4, 4, 8192)      \

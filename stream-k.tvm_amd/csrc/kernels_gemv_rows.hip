@@ -56,6 +56,14 @@ int gemv_rows_kernel_infos(KernelInfo *out, int max) {
   }
   SK_STREAM_PAIRS_BF16_KERNELS(X)
 #undef X
+#define X(id, WN, RK, WD, AD)                                                                                   \
+  if (n < max) {                                                                                                \
+    typedef TileStreamQ4<WN, RK, WD, AD> P;                                                                     \
+    out[n++] = KernelInfo{id, FAMILY_SKINNY, 2 /* SK_Q4 */, 0, 4, P::BM, P::BN, P::BKC, P::NT, P::LDS_BYTES, P::CTAS_PER_CU, \
+                          P::TILE_ELEMS, 0, P::MAX_M, 256, "stream_q4_wn" #WN "_rk" #RK "_d" #WD};              \
+  }
+  SK_STREAM_Q4_KERNELS(X)
+#undef X
   return n;
 }
 
@@ -102,6 +110,13 @@ int launch_gemv_rows(int id, const SkinnyArgs &a, const DevPlan &p, const Worksp
     return launch_policy<P>(a, p, ws, s, bias);        \
   }
     SK_STREAM_PAIRS_BF16_KERNELS(X)
+#undef X
+#define X(id_, WN, RK, WD, AD)                   \
+  case id_: {                                    \
+    typedef TileStreamQ4<WN, RK, WD, AD> P;      \
+    return launch_policy<P>(a, p, ws, s, bias);  \
+  }
+    SK_STREAM_Q4_KERNELS(X)
 #undef X
   }
   return (int)hipErrorInvalidValue;
@@ -163,6 +178,15 @@ int occupancy_gemv_rows(int id) {
     return occ;                                                                                          \
   }
     SK_STREAM_PAIRS_BF16_KERNELS(X)
+#undef X
+#define X(id_, WN, RK, WD, AD)                                                                           \
+  case id_: {                                                                                            \
+    typedef TileStreamQ4<WN, RK, WD, AD> P;                                                              \
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_skinny_kernel<P>, P::NT, 0) != hipSuccess) \
+      return -1;                                                                                         \
+    return occ;                                                                                          \
+  }
+    SK_STREAM_Q4_KERNELS(X)
 #undef X
   }
   return -1;

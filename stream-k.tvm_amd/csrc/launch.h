@@ -11,6 +11,7 @@
 #include "tile_gemv_q4.h"
 #include "tile_gemv_rows.h"
 #include "tile_stream_pairs.h"
+#include "tile_stream_q4.h"
 #include "tile_skinny.h"
 
 namespace sk {

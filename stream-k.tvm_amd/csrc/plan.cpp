@@ -103,7 +103,10 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
       if (t[i].family == FAMILY_TILE && t[i].dtype == SK_Q4 && t[i].bm == want_bm && t[i].bn == want_bn) return &t[i];
     return nullptr;
   }
-  if ((dtype == SK_F16 || dtype == SK_BF16) && layout == SK_LAYOUT_NT && M >= 5 && M <= 64 && want_variant < 0) {
+  // (2 <= M <= 4: from about 100 MB of weights on; below, the matrix-vector form with four rows of A starts up faster --
+  // 4 x 8192 x 8192: 24.8 us against 32.0 us, 2 x 4096 x 4096: 12.1 us against 11.3 us, weights from HBM)
+  const bool stream_rows = M >= 5 || (M >= 2 && N * K >= (int64_t)48 << 20);
+  if ((dtype == SK_F16 || dtype == SK_BF16) && layout == SK_LAYOUT_NT && stream_rows && M <= 64 && want_variant < 0) {
     // 5 <= M <= 64 with fp16 / bfloat16 weights: the kernels that stream the weights through LDS in contiguous loads
     // (tile_stream_pairs.h).  Tiles of 32 weight rows while one wave of them fits the device (N = 8192: one tile per
     // CU and no fix-up), 64 rows beyond; 64 rows of A exist with 32 weight rows only.
@@ -122,6 +125,25 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
         if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].variant == 2 && t[i].bn == 16 &&
             t[i].bk == 1024 && accepts_shape(t[i], M, K))
           return &t[i];
+    // 2 <= M <= 16 with row-major Q4 weights (scalar zero point), weights from HBM.  Where 64-row tiles give three
+    // fifths of the CUs a tile the general kernel with 64 weight rows and K split over two waves, data-parallel
+    // (16 x 28672 x 8192: 32.8 us; the 32-row kernel below: 48.5; 16 x 11008 x 4096: 10.7 / 14.8; 16 x 16384 x 16384:
+    // 37.6 / 38.1).  Fewer rows and 16 MB of weights or more: the kernel that streams the packed weights through
+    // LDS in contiguous loads, 32 weight rows per tile (tile_stream_q4.h; 16 x 8192 x 8192: 13.4 us against 14.6,
+    // 16 x 4096 x 11008: 15.7 / 17.1; 16 x 4096 x 4096: 8.0 / 7.5, which stays with the kernel below).
+    if (dtype == SK_Q4 && M > 1 && M <= 16 && want_variant < 0) {
+      if (cdiv(N, 64) * 5 >= (int64_t)num_cus * 3) {
+        for (int i = 0; i < n; ++i)
+          if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].variant == 0 && t[i].bm == 16 &&
+              t[i].bn == 64 && t[i].bk == 512 && accepts_shape(t[i], M, K))
+            return &t[i];
+      } else if (N * K >= ((int64_t)32 << 20) && K % 256 == 0) {
+        for (int i = 0; i < n; ++i)
+          if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].variant == 4 && t[i].bn == 32 &&
+              accepts_shape(t[i], M, K))
+            return &t[i];
+      }
+    }
     // 2 <= M <= 16 with Q4 weights: eight waves per CTA (two per SIMD cover each other's waits),
     // 32 weight rows, K split over four waves
     if (((dtype == SK_Q4 && M > 1) || dtype == SK_Q4_ZP || dtype == SK_Q4_ZP_TILED) && M <= 16 && want_variant < 0)
@@ -407,7 +429,11 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
   int sched = cfg ? cfg->schedule : SK_SCHED_AUTO;
   if (!(cfg && cfg->grid > 0)) {
     const int64_t iters = total64 * out->iters_per_tile;
-    if (total64 >= num_cus && total64 <= max_grid) {
+    // (the kernels that stream the weights through LDS are bound by memory: with tiles for three fifths of the CUs
+    // they run data-parallel rather than pay a fix-up -- Q4 16 x 11008 x 4096: 11.5 us against 14.3 us)
+    const bool stream_dp = k->family == FAMILY_SKINNY && (k->variant == 4 || k->dtype == SK_Q4) && k->bm == 16 && k->max_m >= 16 &&
+                           total64 * 5 >= (int64_t)num_cus * 3;
+    if ((total64 >= num_cus || stream_dp) && total64 <= max_grid) {
       grid = (int)total64;  // one tile per CTA, all resident: a single data-parallel wave
     } else if (total64 < num_cus) {
       // fewer tiles than CUs: one CTA per CU, but a split tile keeps at least 4 K-iterations per CTA

@@ -77,6 +77,13 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
                 out.append(dict(bm=bm, bn=bn, bk=bk, variant=1, schedule="dp"))
                 for grid in (cus, 2 * cus):
                     out.append(dict(bm=bm, bn=bn, bk=bk, variant=1, schedule="sk2", grid=grid, fixup="reduce"))
+    if dtype == "q4" and M <= 16 and K % 256 == 0:
+        # row-major Q4 weights streamed through LDS in contiguous loads (variant 5 of these shapes)
+        for (bm, bn, bk) in ((16, 64, 512), (16, 32, 1024)):
+            base = dict(bm=bm, bn=bn, bk=bk, variant=5)
+            out.append(dict(base, schedule="dp"))
+            for sched, fixup in (("sk2", "reduce"), ("basic", "reduce"), ("basic", "atomic")):
+                out.append(dict(base, schedule=sched, grid=cus, fixup=fixup))
     if dtype in ("float16", "bfloat16") and M <= 64:
         for (bm, bn, bk) in _STREAM_F16:
             if bm < M or (bm >= 2 * M and bm > 16):

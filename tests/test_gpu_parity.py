@@ -582,6 +582,50 @@ def test_q4_ragged_shapes_every_kernel(sk, oracle, variant):
     sk.workspace_status()
 
 
+def test_q4_weights_streamed_through_lds(sk, oracle):
+    """Up to 16 rows of A on the kernels that stream row-major Q4 weights through LDS in contiguous loads (64 and 32
+    weight rows per tile): ragged M and N, K a multiple of 256 only (a last iteration hanging over K), zero points
+    0 / 5 / 8 / 15, all schedules and both fix-ups.  The weights these kernels multiply are the fp16-rounded ones of
+    the oracle: exact on integer data with power-of-two scales (any wrong nibble, K order, scale row or rotation
+    shows), within 2e-3 of the oracle on random data; K that is not a multiple of 256 is refused."""
+    import torch
+    rng = np.random.default_rng(58)
+    ran = 0
+    for (M, N, K, zero) in [(16, 1000, 2304, 8), (9, 520, 256, 15), (1, 72, 4096, 0), (13, 2048, 16384, 5), (5, 264, 28672, 8),
+                            (16, 8192, 8192, 8), (2, 4099, 11008, 3)]:
+        A = (rng.random((M, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+        Wq = rng.integers(0, 256, (N, K // 2), dtype=np.uint8)
+        sc = rng.uniform(0.005, 0.02, (N, K // 128)).astype(np.float16)
+        Ai = rng.integers(-2, 3, (M, K)).astype(np.float16)
+        sci = (2.0 ** rng.integers(-3, 1, (N, K // 128))).astype(np.float16)
+        full = N * K <= 1 << 24   # (the host product of the large cases is taken on a slice of the weight rows)
+        rows = slice(None) if full else slice(N - 520, N)
+        ref = oracle.q4_gemm_ref(A, Wq[rows], sc[rows], 128, zero)
+        exact = oracle.q4_gemm_ref(Ai, Wq[rows], sci[rows], 128, zero)
+        assert np.abs(exact).max() < 2 ** 20 and np.array_equal(exact, np.rint(exact * 8) / 8)   # (exact in fp32)
+        dA, dAi, dW, dS, dSi = _t(A), _t(Ai), _t(Wq), _t(sc), _t(sci)
+        for (bn, bk) in ((64, 512), (32, 1024)):
+            for sch in (dict(schedule="dp"), dict(schedule="sk2", fixup="reduce", grid=48),
+                        dict(schedule="sk2", fixup="atomic", grid=40), dict(schedule="basic", fixup="reduce", grid=56)):
+                plan = sk.make_plan(M, N, K, "q4", "nt", dict(bm=16, bn=bn, bk=bk, variant=5, **sch))
+                assert sk.kernel_name(plan.kernel_id).startswith("stream_q4_")
+                C = sk.streamk_q4(dA, dW, dS, zero=zero, plan=plan)
+                assert _rel(oracle, C[:, rows], ref) <= 2e-3 <= TOL, (M, N, K, zero, bn, bk, sch)
+                C = sk.streamk_q4(dAi, dW, dSi, zero=zero, plan=plan)
+                assert np.array_equal(C[:, rows].float().cpu().numpy(), exact.astype(np.float16).astype(np.float32)), (M, N, K, zero, bn, bk, sch)
+                ran += 1
+    assert ran >= 56
+    with pytest.raises(sk.StreamKError):
+        sk.make_plan(16, 1000, 1152, "q4", "nt", dict(bm=16, bn=64, bk=512, variant=5))
+    with pytest.raises(sk.StreamKError):
+        sk.make_plan(17, 1000, 1024, "q4", "nt", dict(bm=16, bn=64, bk=512, variant=5))
+    # what the library picks by itself for 2..16 rows and 16 MB of weights or more
+    assert sk.kernel_name(sk.make_plan(16, 8192, 8192, "q4", "nt", use_tuned=False).kernel_id).startswith("stream_q4_")
+    assert not sk.kernel_name(sk.make_plan(16, 4096, 4096, "q4", "nt", use_tuned=False).kernel_id).startswith("stream_q4_")
+    sk.workspace_status()
+
+
+@pytest.mark.gpu
 def test_q4_tile_kernels_more_than_64_rows(sk, oracle):
     """Q4 weights with more rows of A than the weight-streaming kernels take: the tile kernels that dequantise B
     in registers on its way into the LDS stage (the reference dequantises right before the MMA,
