@@ -23,11 +23,25 @@ __global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_skinny_kernel_bias(
 // nor the workspace.  These kernels run for a few microseconds, most of which is set-up executed from a cold
 // instruction cache: without the plan's argument loads, the range and tile-coordinate arithmetic and the fix-up
 // code the first loads go out earlier.
+// The hardware deals workgroups round-robin to the 8 XCDs.  Policies with XCD_CONTIGUOUS give XCD x a contiguous range
+// of tiles, as the planned launches do (logical_pid), so that each XCD streams one contiguous eighth of the weights;
+// the others take tile = block index (measured per kernel family).
+template <class P, class = void>
+struct xcd_contiguous { static constexpr bool value = false; };
+template <class P>
+struct xcd_contiguous<P, std::void_t<decltype(P::XCD_CONTIGUOUS)>> { static constexpr bool value = P::XCD_CONTIGUOUS; };
+template <class P>
+__device__ __forceinline__ int first_tile_of_block() {
+  const int b = blockIdx.x, grid = gridDim.x, x = b & 7;
+  if constexpr (xcd_contiguous<P>::value) return x * (grid >> 3) + min(x, grid & 7) + (b >> 3);
+  return b;
+}
+
 template <class P>
 __global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_skinny_dp_kernel(typename P::Args a, int total_tiles, int ipt) {
   __shared__ __attribute__((aligned(16))) char smem[P::LDS_BYTES];
   typename P::Acc acc;
-  for (int tile = blockIdx.x; tile < total_tiles; tile += gridDim.x) {
+  for (int tile = first_tile_of_block<P>(); tile < total_tiles; tile += gridDim.x) {
     P::mac(a, acc, 0, tile, 0, ipt, smem);
     P::store_c(a, acc, 0, tile, smem, nullptr);
   }
@@ -39,7 +53,7 @@ __global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_skinny_dp_kernel_bi
   const void *bias = bias_arg;
   asm volatile("" ::"s"(bias));  // fetched with the other arguments, not before the first store
   typename P::Acc acc;
-  for (int tile = blockIdx.x; tile < total_tiles; tile += gridDim.x) {
+  for (int tile = first_tile_of_block<P>(); tile < total_tiles; tile += gridDim.x) {
     P::mac(a, acc, 0, tile, 0, ipt, smem);
     P::store_c(a, acc, 0, tile, smem, bias);
   }
@@ -62,8 +76,9 @@ __global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_skinny_flat_kernel(
   a.lda = K; a.ldw = ldw; a.ldc = N;
   a.zero = zero; a.groups = groups; a.zeros = nullptr;
   typename P::Acc acc;
-  P::mac(a, acc, 0, blockIdx.x, 0, (K + P::BKC - 1) / P::BKC, smem);
-  P::store_c(a, acc, 0, blockIdx.x, smem, nullptr);
+  const int tile = first_tile_of_block<P>();
+  P::mac(a, acc, 0, tile, 0, (K + P::BKC - 1) / P::BKC, smem);
+  P::store_c(a, acc, 0, tile, smem, nullptr);
 }
 
 // NO_FLAT_ARGS: policies whose scalar-argument instance the compiler does not fit into the register budget

@@ -49,6 +49,9 @@ namespace sk {
 // zero points are row-major [N, groups] also where the weights are tiled.)
 template <int NB_, int WN_, int RK_, int DEPTH_, int KMAX_ = 16384, bool TILED_ = false, bool ZP_ = false>
 struct TileGemvQ4 {
+  // data-parallel launches give each XCD a contiguous eighth of the row blocks (skinny_launch.h): N = K = 8192 with
+  // the weights in the Infinity Cache 6.08-6.14 -> 5.81 us, from HBM 8.6-8.8 -> 8.55 us; other shapes unchanged
+  static constexpr bool XCD_CONTIGUOUS = true;
   typedef SkinnyArgs Args;
   static constexpr bool LEAN_ENTRY = false;  // see run_persistent
   static constexpr int NB = NB_, WN = WN_, RK = RK_, DEPTH = DEPTH_, KMAX = KMAX_;
