@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extra] [--no-cpu]
     python bench.py --case MxNxK [--dtype D] [--layout nt|nn] [--config "dict(...)"] [--data rand|zeros|ones]
-                    [--reps R] [--time] [--vendor]       one GEMM case on its own, for a profiler
+                    [--reps R] [--copies C] [--time] [--vendor]       one GEMM case on its own, for a profiler
 
 One "step" is one fp16 GEMM call through the C ABI on inputs already resident in HBM.  The headline
 workload is M = N = K = 8192 (NT layout, U[-1,1) from seed 0), the compute-bound end of the
@@ -12,7 +12,8 @@ carries
   cpu_baseline  the oracle's fp32 host matmul timed on this box's cores on a bounded sample,
   config.metric_parts   the other two parts of the metric in short: Stream-K against the data-parallel schedule at
                 M = 256 / 512 / 1024 (same tile, and the best data-parallel tile), Q4 GEMM at M = 1 / 16 as a
-                fraction of HBM peak with the weights in the Infinity Cache and from HBM,
+                fraction of HBM peak with the weights in the Infinity Cache and from HBM, fp16 with 16 / 64 rows of A
+                with the weights from HBM next to the vendor GEMM,
   extra         the measurements behind them and the rest: M sweep at N = K = 8192, 1024x1024x8192 with all
                 fix-ups, the large dense shapes in both layouts and types, the reference's own run shapes
                 (kernels this short are timed as graph-captured batches).
@@ -99,7 +100,11 @@ def run_case(args):
         A = torch.randn(M, K, generator=g).half().cuda()
         Wq = torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8).cuda()
         sc = (torch.rand(N, K // 128, generator=g) * 0.015 + 0.005).half().cuda()
-        run = lambda: streamk.streamk_q4(A, Wq, sc, plan=plan)  # noqa: E731
+        Wqs, turn = [Wq] + [Wq.clone() for _ in range(args.copies - 1)], [0]
+
+        def run():   # (--copies: the launches rotate over copies of the weights, so that each one reads HBM)
+            turn[0] += 1
+            streamk.streamk_q4(A, Wqs[turn[0] % len(Wqs)], sc, plan=plan)
     elif args.dtype == "int8":
         if args.data == "rand":
             A = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int8).cuda()
@@ -133,7 +138,11 @@ def run_case(args):
             A, B = fill(M, K, dtype=dt, device="cuda"), fill(*bshape, dtype=dt, device="cuda")
         C = torch.empty(M, N, dtype=dt, device="cuda")
         fn = {"float16": streamk.streamk_fp16, "bfloat16": streamk.streamk_bf16}.get(args.dtype, streamk.streamk_fp32)
-        run = lambda: fn(A, B, layout=args.layout, out=C, plan=plan)  # noqa: E731
+        Bs, turn = [B] + [B.clone() for _ in range(args.copies - 1)], [0]
+
+        def run():   # (--copies: the launches rotate over copies of B, so that each one reads HBM)
+            turn[0] += 1
+            fn(A, Bs[turn[0] % len(Bs)], layout=args.layout, out=C, plan=plan)
         Bt = B.T if args.layout == "nt" else B
         vendor = ("torch.matmul", lambda: torch.matmul(A, Bt, out=C))
     for _ in range(args.reps):
@@ -165,6 +174,7 @@ def main():
     ap.add_argument("--layout", default="nt", choices=["nt", "nn"])
     ap.add_argument("--config", default="{}", help="--case: python dict of plan options, e.g. \"dict(bm=256,bn=256,raster=8)\"")
     ap.add_argument("--reps", type=int, default=5)
+    ap.add_argument("--copies", type=int, default=1, help="--case: rotate the launches over this many copies of the weights (fp16 / bfloat16 / q4)")
     ap.add_argument("--data", default="rand", choices=["rand", "zeros", "ones"])
     ap.add_argument("--time", action="store_true", help="--case: print the average time of the launches")
     ap.add_argument("--vendor", action="store_true", help="--case: also run (and with --time, time) the vendor GEMM")
@@ -775,8 +785,12 @@ def main():
                             "matrix; tuned_weights_from_hbm cycles through 20 copies so that every launch reads HBM")
         streamk.workspace_status()
         # the metric's other two parts in short, where the record of a run keeps them
-        parts = {"streamk_vs_data_parallel_N8192_K8192": {}, "q4_gemm_N8192_K8192": {}}
+        parts = {"streamk_vs_data_parallel_N8192_K8192": {}, "q4_gemm_N8192_K8192": {}, "few_rows_fp16_N8192_K8192": {}}
         for row in sweep:
+            if row["M"] in (16, 64):   # (weights from HBM; the vendor GEMM on the same rotation of weights beside it)
+                parts["few_rows_fp16_N8192_K8192"][f"M{row['M']}"] = {
+                    "us_weights_from_hbm": row["auto_weights_from_hbm_us"], "frac_hbm": row["frac_hbm"],
+                    "torch_matmul_us": row["torch_matmul_weights_from_hbm_us"]}
             if row["M"] in (256, 512, 1024):
                 parts["streamk_vs_data_parallel_N8192_K8192"][f"M{row['M']}"] = {
                     "auto_tflops": row["auto"], "auto_tile": row["auto_tile"], "sk_over_dp_same_tile": row["sk_over_dp_same_tile"],

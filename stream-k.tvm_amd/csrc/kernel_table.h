@@ -26,7 +26,8 @@ struct KernelInfo {
                 // 3: as 1 with BK = 32 and four LDS stages (loads three iterations ahead);
                 // 4: as 1 with 16x16x32 MFMAs; 5: as 3 with 16x16x32 MFMAs; 6: as 1 for fp8 operands (32x32x64 MFMAs);
                 // 7: as 4 with four waves per CTA, the K loop in assembly and the accumulators in a[0:255]
-                // small-M kernels -- 0: up to 16*MB rows of A; 1: M == 1; 2: M == 1, matrix-vector on 4x4x4 MFMA
+                // small-M kernels -- 0: up to 16*MB rows of A; 1: M == 1; 2: M == 1, matrix-vector on 4x4x4 MFMA;
+                // 3: the matrix-vector form with up to four rows of A; 4: weights streamed through LDS in contiguous loads
   int bm, bn, bk;  // CTA tile; bk is the K extent of one CTA iteration
   int threads;
   int lds_bytes;
