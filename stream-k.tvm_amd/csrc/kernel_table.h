@@ -256,6 +256,12 @@ struct KernelInfo {
   X(287, 2, 2, 2, 1, 3)                 \
   X(289, 1, 2, 2, 1, 4)
 
+// the same with NB blocks of 16 weight rows per wave, AD slots of A and the unpadded rings (64 x 64 tiles: the 160 KB
+// of LDS exactly):  X(id, MB, WM, WN, RK, DEPTH, NB, AD, BF16)
+#define SK_STREAM_BLOCKS_KERNELS(X)  \
+  X(292, 2, 2, 2, 1, 3, 2, 2, false) \
+  X(293, 2, 2, 2, 1, 3, 2, 2, true)
+
 // Up to 16 rows of A, Q4 weights (row-major, scalar zero point) streaming through LDS in contiguous loads
 // (tile_stream_q4.h; dtype SK_Q4, variant 4):  X(id, WN, RK, WD, AD)
 #define SK_STREAM_Q4_KERNELS(X) \

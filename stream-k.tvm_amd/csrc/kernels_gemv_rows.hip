@@ -56,6 +56,15 @@ int gemv_rows_kernel_infos(KernelInfo *out, int max) {
   }
   SK_STREAM_PAIRS_BF16_KERNELS(X)
 #undef X
+#define X(id, MB, WM, WN, RK, DEPTH, NB, AD, BF)                                                                 \
+  if (n < max) {                                                                                                \
+    typedef TileStreamPairs<MB, WM, WN, RK, DEPTH, BF, NB, AD, false> P;                                        \
+    out[n++] = KernelInfo{id, FAMILY_SKINNY, (BF) ? 3 : 0, 0, 4, P::BM, P::BN, P::BKC, P::NT, P::LDS_BYTES, P::CTAS_PER_CU, \
+                          P::TILE_ELEMS, 0, P::MAX_M, 8, (BF) ? "stream_bf16_mb" #MB "_nb" #NB "_wm" #WM "_wn" #WN "_rk" #RK "_d" #DEPTH \
+                                                              : "stream_f16_mb" #MB "_nb" #NB "_wm" #WM "_wn" #WN "_rk" #RK "_d" #DEPTH}; \
+  }
+  SK_STREAM_BLOCKS_KERNELS(X)
+#undef X
 #define X(id, WN, RK, WD, AD)                                                                                   \
   if (n < max) {                                                                                                \
     typedef TileStreamQ4<WN, RK, WD, AD> P;                                                                     \
@@ -110,6 +119,13 @@ int launch_gemv_rows(int id, const SkinnyArgs &a, const DevPlan &p, const Worksp
     return launch_policy<P>(a, p, ws, s, bias);        \
   }
     SK_STREAM_PAIRS_BF16_KERNELS(X)
+#undef X
+#define X(id_, MB, WM, WN, RK, DEPTH, NB, AD, BF)                         \
+  case id_: {                                                             \
+    typedef TileStreamPairs<MB, WM, WN, RK, DEPTH, BF, NB, AD, false> P;  \
+    return launch_policy<P>(a, p, ws, s, bias);                           \
+  }
+    SK_STREAM_BLOCKS_KERNELS(X)
 #undef X
 #define X(id_, WN, RK, WD, AD)                   \
   case id_: {                                    \
@@ -178,6 +194,15 @@ int occupancy_gemv_rows(int id) {
     return occ;                                                                                          \
   }
     SK_STREAM_PAIRS_BF16_KERNELS(X)
+#undef X
+#define X(id_, MB, WM, WN, RK, DEPTH, NB, AD, BF)                                                        \
+  case id_: {                                                                                            \
+    typedef TileStreamPairs<MB, WM, WN, RK, DEPTH, BF, NB, AD, false> P;                                 \
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_skinny_kernel<P>, P::NT, 0) != hipSuccess) \
+      return -1;                                                                                         \
+    return occ;                                                                                          \
+  }
+    SK_STREAM_BLOCKS_KERNELS(X)
 #undef X
 #define X(id_, WN, RK, WD, AD)                                                                           \
   case id_: {                                                                                            \

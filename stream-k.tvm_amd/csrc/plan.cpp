@@ -110,7 +110,9 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
     // 5 <= M <= 64 with fp16 / bfloat16 weights: the kernels that stream the weights through LDS in contiguous loads
     // (tile_stream_pairs.h).  Tiles of 32 weight rows while one wave of them fits the device (N = 8192: one tile per
     // CU and no fix-up), 64 rows beyond; 64 rows of A exist with 32 weight rows only.
-    const bool narrow = cdiv(N, 32) <= num_cus || M > 32;
+    // (more than 32 rows: 64 weight rows where they give three fifths of the CUs a tile -- A is then as many bytes
+    // per CTA as the weights instead of twice as many; 64 x 16384 x 8192: 49 us against 56 us)
+    const bool narrow = M > 32 ? cdiv(N, 64) * 5 < (int64_t)num_cus * 3 : cdiv(N, 32) <= num_cus;
     const int bm = M <= 16 ? 16 : (M <= 32 ? 32 : 64), bn = narrow ? 32 : 64, bk = (bm == 16 && narrow) ? 512 : 256;
     for (int i = 0; i < n; ++i)
       if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].variant == 4 && t[i].bm == bm && t[i].bn == bn &&
@@ -431,7 +433,8 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
     const int64_t iters = total64 * out->iters_per_tile;
     // (the kernels that stream the weights through LDS are bound by memory: with tiles for three fifths of the CUs
     // they run data-parallel rather than pay a fix-up -- Q4 16 x 11008 x 4096: 11.5 us against 14.3 us)
-    const bool stream_dp = k->family == FAMILY_SKINNY && (k->variant == 4 || k->dtype == SK_Q4) && k->bm == 16 && k->max_m >= 16 &&
+    const bool stream_dp = k->family == FAMILY_SKINNY && (k->variant == 4 || k->dtype == SK_Q4) && k->max_m >= 16 &&
+                           (k->bm == 16 || (k->variant == 4 && k->bm == 64 && k->bn == 64)) &&
                            total64 * 5 >= (int64_t)num_cus * 3;
     if ((total64 >= num_cus || stream_dp) && total64 <= max_grid) {
       grid = (int)total64;  // one tile per CTA, all resident: a single data-parallel wave
@@ -467,8 +470,8 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
     else sched = total64 >= 2 * (int64_t)grid ? SK_SCHED_SK_ONE_TILE : SK_SCHED_SK_TWO_TILE;
     // (the kernels that stream the weights through LDS are bound by memory, not by the busiest CU: an uneven last
     // wave costs them less than the fix-up; 16 x 28672 x 8192: 77.8 us data-parallel against 83.6 us.  With 64 rows of
-    // A it is the other way round: 110 us against 103 us)
-    if (k->family == FAMILY_SKINNY && k->variant == 4 && k->bm == 16 && total64 >= grid) sched = SK_SCHED_DP;
+    // A on 64 x 32 tiles it is the other way round, 110 us against 103 us; on 64 x 64 tiles 91.5 against 92.6)
+    if (k->family == FAMILY_SKINNY && k->variant == 4 && (k->bm == 16 || k->bn == 64) && total64 >= grid) sched = SK_SCHED_DP;
     if (k->family == FAMILY_TILE && sched != SK_SCHED_DP) {
       // Fewer tiles than CUs: the idle CUs are put to work by an aligned split in two or four, never by CTA ranges
       // that start anywhere.  More tiles than CTAs: see

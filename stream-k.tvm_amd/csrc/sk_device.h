@@ -196,8 +196,10 @@ __device__ __forceinline__ int sk_pid_of_iter(const DevPlan &p, int iter) {
 // Returns false if the poll limit ran out.
 // COHERENT = false: one device-scope acquire (L2 invalidate) by the polling wave before the
 // barrier, so that the ordinary loads that follow cannot hit stale lines.
-template <bool COHERENT>
-__device__ __forceinline__ bool wait_partials_ready(int *flags, int npeers, int spin_limit) {
+// WORD: lds_word is a word of LDS of the caller's through which the first wave's verdict reaches the others; without one
+// the device library's block-wide AND does it, which reserves 256 bytes of LDS of its own.
+template <bool COHERENT, bool WORD = false>
+__device__ __forceinline__ bool wait_partials_ready(int *flags, int npeers, int spin_limit, int *lds_word = nullptr) {
   int ok = 1;
   if (threadIdx.x < 64) {
     for (int i = threadIdx.x; i < npeers; i += 64) {
@@ -210,7 +212,18 @@ __device__ __forceinline__ bool wait_partials_ready(int *flags, int npeers, int 
     }
     if (!COHERENT) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
   }
-  return __syncthreads_and(ok) != 0;
+  if constexpr (!WORD) {
+    return __syncthreads_and(ok) != 0;
+  } else {
+    if (threadIdx.x < 64) {
+      const bool all = __builtin_amdgcn_ballot_w64(ok == 0) == 0;
+      if (threadIdx.x == 0) *lds_word = all;
+    }
+    __syncthreads();
+    const bool all = *lds_word != 0;
+    __syncthreads();
+    return all;
+  }
 }
 
 __device__ __forceinline__ void clear_flags_after_use(int *flags, int npeers) {

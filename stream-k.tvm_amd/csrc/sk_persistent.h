@@ -15,6 +15,12 @@
 
 namespace sk {
 
+// policies that lend the persistent loop its one word of LDS (see run_persistent)
+template <class P, class = void>
+struct fixup_word_in_lds { static constexpr bool value = false; };
+template <class P>
+struct fixup_word_in_lds<P, std::void_t<decltype(P::FIXUP_WORD_IN_LDS)>> { static constexpr bool value = P::FIXUP_WORD_IN_LDS; };
+
 // optional members of a policy: COHERENT_REDUCE (partials of the REDUCE fix-up travel with device-scope
 // accesses; default: as COHERENT_PARTIALS says), HALVES (the policy has store_partial_half /
 // add_partial_half / store_c_half, see below) and ATOMIC_C (the policy has atomic_c: its accumulators added to C
@@ -47,7 +53,16 @@ struct has_halves<P, std::void_t<decltype(P::HALVES)>> { static constexpr bool v
 template <class P, bool FIXUP = true, bool BIAS = false>
 __device__ __forceinline__ void run_persistent(const typename P::Args &a, const DevPlan &plan,
                                                const Workspace &ws, char *smem, const void *bias_arg = nullptr) {
-  __shared__ int s_word;
+  // one word through which thread 0 tells the CTA whether it arrived last at a tile.  Policies whose LDS is dead
+  // between two calls of mac and who need all of it (FIXUP_WORD_IN_LDS) lend its first word
+  int *s_word_p;
+  if constexpr (fixup_word_in_lds<P>::value) {
+    s_word_p = reinterpret_cast<int *>(smem);
+  } else {
+    __shared__ int s_word_own;
+    s_word_p = &s_word_own;
+  }
+  int &s_word = *s_word_p;
   // Fetch the bias pointer with the other kernel arguments: left to the compiler it is read from the argument
   // buffer right before the first store, a dependent scalar load (~0.3 us) at the end of every CTA.
   const void *bias = nullptr;
@@ -206,7 +221,8 @@ __device__ __forceinline__ void run_persistent(const typename P::Args &a, const 
         // tile's first CTA: wait for all followers at once, then add their partials in ascending
         // CTA order and store
         const int npeers = sk_pid_of_iter(plan, (tile + 1) * ipt - 1) - pid;
-        if (!wait_partials_ready<reduce_is_coherent<P>::value>(&ws.flags[pid + 1], npeers, plan.spin_limit)) {
+        if (!wait_partials_ready<reduce_is_coherent<P>::value, fixup_word_in_lds<P>::value>(&ws.flags[pid + 1], npeers,
+                                                                                            plan.spin_limit, s_word_p)) {
           if (threadIdx.x == 0) ws.status[WS_STATUS] = -8;  // SK_ERR_TIMEOUT
         } else {
           for (int p = 1; p <= npeers; ++p) P::add_partial(acc, ws.partials + (size_t)(pid + p) * P::TILE_ELEMS);

@@ -30,42 +30,50 @@
 
 namespace sk {
 
-template <int MB_, int WM_, int WN_, int RK_, int DEPTH_, bool BF16_ = false>
+template <int MB_, int WM_, int WN_, int RK_, int DEPTH_, bool BF16_ = false, int NB_ = 1, int AD_ = 3, bool PADDED_ = true>
 struct TileStreamPairs {
   typedef SkinnyArgs Args;
   typedef floatx4 AccV;
   static constexpr bool LEAN_ENTRY = false;  // see run_persistent
   static constexpr bool NO_FLAT_ARGS = false;
   static constexpr bool COHERENT_PARTIALS = true;
-  // three slots of A: its loads are issued one iteration later than the weights' when DEPTH_ is four
-  static constexpr int MB = MB_, WM = WM_, WN = WN_, RK = RK_, WD = DEPTH_, AD = 3, NT = 256;
+  // the rings are dead between two calls of mac (it ends with every load landed and a barrier), and the 64 x 64
+  // instance fills the 160 KB of LDS: the persistent loop's one word of LDS is the first word of the rings
+  static constexpr bool FIXUP_WORD_IN_LDS = true;
+  // AD slots of A (three unless LDS is short): its loads are issued later than the weights' when DEPTH_ is larger
+  static constexpr int MB = MB_, NB = NB_, WM = WM_, WN = WN_, RK = RK_, WD = DEPTH_, AD = AD_, NT = 256;
+  static constexpr bool PADDED = PADDED_;
   static_assert(WM * WN * RK == 4, "four waves");
   static_assert(WM == 1 || WM == 2, "the eight loads of a weight ring are shared out among WM_ waves");
-  static constexpr int BM = 16 * MB * WM, BN = 16 * WN, MAX_M = BM;
+  static constexpr int BM = 16 * MB * WM, BN = 16 * NB * WN, MAX_M = BM;
   static constexpr int BK = 256, BKC = 256 * RK;       // K-values per iteration: of a wave, of the CTA
-  static constexpr int PAIR = 1056;                    // two rows of 512 bytes + 32 bytes of padding
+  // a pair of rows: two rows of 512 bytes; PADDED_: + 32 bytes and neighbouring pieces swapped in the odd row;
+  // else no padding and piece p of row r (of its block of 16) kept at position p ^ r
+  static constexpr int PAIR = PADDED ? 1056 : 1024;
   static constexpr int W_SLOT = 8 * PAIR;              // 16 weight rows of one iteration
   static constexpr int A_PAIRS = 8 * MB * WM;          // pairs of rows of A in the tile
   static constexpr int A_CHUNK = A_PAIRS * PAIR;       // the tile's rows of A, 256 K-values
   static constexpr int A_SLOT = RK * A_CHUNK;          // the tile's rows of A of one iteration
-  static constexpr int LDS_W = WN * RK * WD * W_SLOT, LDS_BYTES = LDS_W + AD * A_SLOT, LDS_TOTAL = LDS_BYTES;
+  static constexpr int RINGS = WN * NB * RK;           // one ring per block of 16 weight rows and K sub-block
+  static constexpr int LDS_W = RINGS * WD * W_SLOT, LDS_BYTES = LDS_W + AD * A_SLOT, LDS_TOTAL = LDS_BYTES;
   static_assert(LDS_BYTES <= 160 * 1024, "the rings must fit the LDS of a CU");
-  static_assert(WD >= AD, "the barrier of an iteration frees the slots read an iteration earlier");
-  static_assert((RK - 1) * WN * WM * 64 * MB * 16 <= LDS_W, "the sums of the K-splitting waves pass through the weights' rings");
+  static_assert(WD >= AD && AD >= 2, "the barrier of an iteration frees the slots read an iteration earlier");
+  static_assert((RK - 1) * WN * WM * 64 * MB * NB * 16 <= LDS_W, "the sums of the K-splitting waves pass through the weights' rings");
   static constexpr int CTAS_PER_CU = (160 * 1024) / (LDS_BYTES + 64) > 0 ? (160 * 1024) / (LDS_BYTES + 64) : 1;
   static constexpr int WAVES_PER_EU = CTAS_PER_CU;
   static constexpr int TILE_ELEMS = BM * BN;
   static constexpr int NTP = WM * WN * 64;             // the rk == 0 waves hold the tile's sums
-  static constexpr int LOADS_W = 8 / WM, LOADS_A = (A_PAIRS * RK) / 4;  // direct-to-LDS loads per wave and iteration
+  static constexpr int NV4 = MB * NB;
+  static constexpr int LOADS_W = NB * 8 / WM, LOADS_A = (A_PAIRS * RK) / 4;  // direct-to-LDS loads per wave and iteration
   static_assert((A_PAIRS * RK) % 4 == 0, "the loads of A are shared out evenly");
   // Loads are issued in the order A(t + AD - 1), W(t + WD - 1) in iteration t, and complete in that order.  Iteration t
   // needs everything up to A(t) and W(t): with WD == AD that leaves the AD - 2 later iterations outstanding, with
   // WD > AD (W(t) is older than A(t)) the weights issued with A(t) and the AD - 2 iterations after them.
   static constexpr int OUTSTANDING = (WD > AD ? LOADS_W : 0) + (AD - 2) * (LOADS_W + LOADS_A);
 
-  // c[i][r] = C[pm*BM + (wm*MB + i)*16 + lane%16][pn*BN + wn*16 + 4*(lane/16) + r]
+  // c[i][j][r] = C[pm*BM + (wm*MB + i)*16 + lane%16][pn*BN + (wn*NB + j)*16 + 4*(lane/16) + r]
   struct Acc {
-    AccV c[MB];
+    AccV c[MB][NB];
   };
 
   template <int N>
@@ -76,29 +84,33 @@ struct TileStreamPairs {
   static __device__ __forceinline__ void mac(const Args &a, Acc &acc, int pm, int pn, int k0, int n, char *smem) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
-    const int wm = wave % WM, ring = wave / WM, wn = ring % WN, rk = ring / WN;
+    const int wm = wave % WM, wn = (wave / WM) % WN, rk = wave / (WM * WN);
 #pragma unroll
-    for (int i = 0; i < MB; ++i) acc.c[i] = AccV{0, 0, 0, 0};
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+      for (int j = 0; j < NB; ++j) acc.c[i][j] = AccV{0, 0, 0, 0};
 
-    // ---- descriptors: the 16 weight rows of (wn) (rows past N read as zero), the tile's rows of A ----
-    const int row0 = pn * BN + wn * 16;
-    const int rows_w = max(0, min(16, a.N - row0));
+    // ---- descriptors: the NB blocks of 16 weight rows of (wn) (rows past N read as zero), the tile's rows of A ----
+    const int row0 = pn * BN + wn * (16 * NB);
+    const int rows_w = max(0, min(16 * NB, a.N - row0));
     const uint32_t ldw_bytes = (uint32_t)a.ldw * 2, lda_bytes = (uint32_t)a.lda * 2;
     const uint4v rsrc_w = uniform_rsrc(
         make_rsrc_words(reinterpret_cast<const char *>(a.W) + (int64_t)row0 * ldw_bytes, (uint32_t)rows_w * ldw_bytes));
     const int a_rows = max(0, min(a.M - pm * BM, BM));
     const uint4v rsrc_a = uniform_rsrc(make_rsrc_words(a.A + (int64_t)pm * BM * a.lda, (uint32_t)a_rows * lda_bytes));
-    // a load: lane l writes position l % 32 of row 2 j + l / 32 of the pair, which holds piece (l % 32) ^ (l / 32)
-    const int odd = lane >> 5, piece = (lane & 31) ^ odd;
-    const uint32_t voff_w = (uint32_t)odd * ldw_bytes + (uint32_t)piece * 16;
-    const uint32_t voff_a = (uint32_t)odd * lda_bytes + (uint32_t)piece * 16;
-    // fragment of lane (i, g) for K-step s of the iteration: row i, piece 4 s + g (kept at position (4 s + g) ^ (i & 1))
+    // a load: lane l writes position l % 32 of row 2 j + l / 32 of pair j (of a block of 16 rows).  PADDED: the
+    // position holds piece (l % 32) ^ (l / 32); else piece (l % 32) ^ (row % 16)
+    const int odd = lane >> 5, piece0 = (lane & 31) ^ odd;
+    auto piece_of = [&](int j) { return PADDED ? piece0 : piece0 ^ ((2 * j) & 15); };
+    // fragment of lane (i, g) for K-step s of the iteration: row i, piece 4 s + g
     const int fi = lane & 15, fg = lane >> 4;
-    const int frag0 = (fi >> 1) * PAIR + (fi & 1) * 512 + ((fg ^ (fi & 1)) * 16);
+    const int frag0 = PADDED ? (fi >> 1) * PAIR + (fi & 1) * 512 + ((fg ^ (fi & 1)) * 16)
+                             : fi * 512 + 16 * ((fi & 12) | (fg ^ (fi & 3)));
     const uint32_t base = lds_address(smem);
-    const uint32_t w_ring = (uint32_t)__builtin_amdgcn_readfirstlane((int)(base + (uint32_t)ring * (WD * W_SLOT)));
+    const int ring0 = (rk * WN + wn) * NB;   // this wave's first ring
+    const uint32_t w_ring = (uint32_t)__builtin_amdgcn_readfirstlane((int)(base + (uint32_t)ring0 * (WD * W_SLOT)));
     const uint32_t a_ring = (uint32_t)__builtin_amdgcn_readfirstlane((int)(base + (uint32_t)LDS_W));
-    const char *w_ptr = smem + ring * (WD * W_SLOT) + frag0;
+    const char *w_ptr = smem + ring0 * (WD * W_SLOT) + frag0;
     const char *a_ptr = smem + LDS_W + rk * A_CHUNK + wm * (8 * MB * PAIR) + frag0;
 
     // iteration t of the segment (t = 0 .. n - 1) covers K-values k_of(t) 256 RK ..; iterations past the segment and
@@ -108,12 +120,16 @@ struct TileStreamPairs {
     auto issue_w = [&](int t, int slot) {
       const int kk = k_of(t) * BKC + rk * BK;
       const uint32_t kbytes = (uint32_t)__builtin_amdgcn_readfirstlane(kk * 2);
-      const uint32_t vw = (t < n && kk + piece * 8 < a.K) ? voff_w : OOB_OFFSET;
 #pragma unroll
-      for (int jj = 0; jj < LOADS_W; ++jj) {
-        const int j = wm * LOADS_W + jj;   // this wave's share of the ring's eight pairs of rows
-        dma_load_16(rsrc_w, w_ring + (uint32_t)(slot * W_SLOT + j * PAIR), vw, kbytes + (uint32_t)(2 * j) * ldw_bytes);
-      }
+      for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int jj = 0; jj < 8 / WM; ++jj) {
+          const int j = wm * (8 / WM) + jj;   // this wave's share of the ring's eight pairs of rows
+          const int pc = piece_of(j);
+          dma_load_16(rsrc_w, w_ring + (uint32_t)((b * WD + slot) * W_SLOT + j * PAIR),
+                      (t < n && kk + pc * 8 < a.K) ? (uint32_t)odd * ldw_bytes + (uint32_t)pc * 16 : OOB_OFFSET,
+                      kbytes + (uint32_t)(16 * b + 2 * j) * ldw_bytes);
+        }
     };
     auto issue_a = [&](int t, int slot) {
 #pragma unroll
@@ -122,8 +138,9 @@ struct TileStreamPairs {
         const int chunk = q / A_PAIRS, pj = q % A_PAIRS;
         const int kk = k_of(t) * BKC + chunk * BK;
         const uint32_t kbytes = (uint32_t)__builtin_amdgcn_readfirstlane(kk * 2);
-        const uint32_t va = (t < n && kk + piece * 8 < a.K) ? voff_a : OOB_OFFSET;
-        dma_load_16(rsrc_a, a_ring + (uint32_t)(slot * A_SLOT + chunk * A_CHUNK + pj * PAIR), va,
+        const int pc = piece_of(pj);
+        dma_load_16(rsrc_a, a_ring + (uint32_t)(slot * A_SLOT + chunk * A_CHUNK + pj * PAIR),
+                    (t < n && kk + pc * 8 < a.K) ? (uint32_t)odd * lda_bytes + (uint32_t)pc * 16 : OOB_OFFSET,
                     kbytes + (uint32_t)(2 * pj) * lda_bytes);
       }
     };
@@ -141,25 +158,32 @@ struct TileStreamPairs {
       issue_a(t + AD - 1, as == 0 ? AD - 1 : as - 1);
       issue_w(t + WD - 1, ws == 0 ? WD - 1 : ws - 1);
       const char *wp = w_ptr + ws * W_SLOT, *ap = a_ptr + as * A_SLOT;
-      half8v fw[8], fa[MB][8];
+      half8v fw[NB][8], fa[MB][8];
 #pragma unroll
       for (int s = 0; s < 8; ++s) {
-        fw[s] = *reinterpret_cast<const half8v *>(wp + s * 64);
+        // PADDED: piece 4 s + g sits 64 s bytes further on; else its position is (4 s + g) ^ i: 64 s XORed in
+        const int so = PADDED ? s * 64 : 0;
+        const int sx = PADDED ? 0 : s * 64;
 #pragma unroll
-        for (int i = 0; i < MB; ++i) fa[i][s] = *reinterpret_cast<const half8v *>(ap + i * 8 * PAIR + s * 64);
+        for (int j = 0; j < NB; ++j)
+          fw[j][s] = *reinterpret_cast<const half8v *>(xor_offset(wp + j * (WD * W_SLOT), frag0, sx) + so);
+#pragma unroll
+        for (int i = 0; i < MB; ++i) fa[i][s] = *reinterpret_cast<const half8v *>(xor_offset(ap + i * 8 * PAIR, frag0, sx) + so);
       }
 #pragma unroll
       for (int s = 0; s < 8; ++s)
 #pragma unroll
-        for (int i = 0; i < MB; ++i) {
-          if constexpr (BF16_) {
-            typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-            acc.c[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, fw[s]), __builtin_bit_cast(bf16x8, fa[i][s]),
-                                                               acc.c[i], 0, 0, 0);
-          } else {
-            acc.c[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fw[s], fa[i][s], acc.c[i], 0, 0, 0);
+        for (int i = 0; i < MB; ++i)
+#pragma unroll
+          for (int j = 0; j < NB; ++j) {
+            if constexpr (BF16_) {
+              typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+              acc.c[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, fw[j][s]), __builtin_bit_cast(bf16x8, fa[i][s]),
+                                                                    acc.c[i][j], 0, 0, 0);
+            } else {
+              acc.c[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fw[j][s], fa[i][s], acc.c[i][j], 0, 0, 0);
+            }
           }
-        }
       // the fragments are in registers before the next barrier hands the slots back to the loads
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       ws = ws + 1 == WD ? 0 : ws + 1;
@@ -174,19 +198,24 @@ struct TileStreamPairs {
       float *red = reinterpret_cast<float *>(smem);
       if (rk > 0) {
 #pragma unroll
-        for (int i = 0; i < MB; ++i)
-          *reinterpret_cast<AccV *>(red + (((wave - WM * WN) * MB + i) * 64 + lane) * 4) = acc.c[i];
+        for (int v = 0; v < NV4; ++v)
+          *reinterpret_cast<AccV *>(red + (((wave - WM * WN) * NV4 + v) * 64 + lane) * 4) = acc.c[v / NB][v % NB];
       }
       __syncthreads();
       if (rk == 0) {
 #pragma unroll
         for (int r = 1; r < RK; ++r)
 #pragma unroll
-          for (int i = 0; i < MB; ++i)
-            acc.c[i] += *reinterpret_cast<const AccV *>(red + ((((r - 1) * WM * WN + wave) * MB + i) * 64 + lane) * 4);
+          for (int v = 0; v < NV4; ++v)
+            acc.c[v / NB][v % NB] += *reinterpret_cast<const AccV *>(red + ((((r - 1) * WM * WN + wave) * NV4 + v) * 64 + lane) * 4);
       }
       __syncthreads();
     }
+  }
+  // p + (x ^ frag-relative bits): the position of a piece inside its row is the low part of the lane's offset frag0
+  // (bits 4..8), which the unpadded layout XORs with 64 s
+  static __device__ __forceinline__ const char *xor_offset(const char *p, int frag0, int sx) {
+    return p - frag0 + (frag0 ^ sx);
   }
 
   // (two copies behind one uniform branch: the epilogue without a bias carries none of its code)
@@ -205,61 +234,64 @@ struct TileStreamPairs {
     const int wm = wave % WM, wn = wave / WM;
     const int lr = lane & 15, lg = lane >> 4;
     const bool vec_ok = (a.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(a.C) & 7) == 0);
-    const int col = pn * BN + wn * 16 + lg * 4;
 #pragma unroll
     for (int i = 0; i < MB; ++i) {
       const int row = pm * BM + (wm * MB + i) * 16 + lr;
-      if (row < a.M && col < a.N) {
-        half4v h;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          float x = acc.c[i][e];
-          if constexpr (BIAS) x = activate(x + bias_at<BF16_>(bias, col + e, a.N), act);
-          if constexpr (BF16_) {
-            const __bf16 b = (__bf16)x;
-            h[e] = __builtin_bit_cast(half_t, b);  // C carries 16-bit patterns
-          } else {
-            h[e] = (half_t)x;
+      for (int j = 0; j < NB; ++j) {
+        const int col = pn * BN + (wn * NB + j) * 16 + lg * 4;
+        if (row < a.M && col < a.N) {
+          half4v h;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            float x = acc.c[i][j][e];
+            if constexpr (BIAS) x = activate(x + bias_at<BF16_>(bias, col + e, a.N), act);
+            if constexpr (BF16_) {
+              const __bf16 b = (__bf16)x;
+              h[e] = __builtin_bit_cast(half_t, b);  // C carries 16-bit patterns
+            } else {
+              h[e] = (half_t)x;
+            }
           }
-        }
-        half_t *dst = a.C + (int64_t)row * a.ldc + col;
-        if (vec_ok && col + 4 <= a.N) {
-          *reinterpret_cast<half4v *>(dst) = h;
-        } else {
-          for (int e = 0; e < 4 && col + e < a.N; ++e) dst[e] = h[e];
+          half_t *dst = a.C + (int64_t)row * a.ldc + col;
+          if (vec_ok && col + 4 <= a.N) {
+            *reinterpret_cast<half4v *>(dst) = h;
+          } else {
+            for (int e = 0; e < 4 && col + e < a.N; ++e) dst[e] = h[e];
+          }
         }
       }
     }
   }
 
   // Partial tiles are a few KB: every access is a coherent (write-through / L2-bypassing) one, as in tile_skinny.h.
-  // Block i of thread t (one of the NTP threads of the rk == 0 waves) is kept at ((i NTP + t) 4; the accumulating
-  // form keeps element e of it at (i 4 + e) NTP + t.
+  // Block v = i NB + j of thread t (one of the NTP threads of the rk == 0 waves) is kept at (v NTP + t) 4; the
+  // accumulating form keeps element e of it at (v 4 + e) NTP + t.
   static __device__ __forceinline__ void store_partial(const Acc &acc, float *dst) {
     if (threadIdx.x >= NTP) return;
 #pragma unroll
-    for (int i = 0; i < MB; ++i) st_coherent(dst + ((size_t)i * NTP + threadIdx.x) * 4, acc.c[i]);
+    for (int v = 0; v < NV4; ++v) st_coherent(dst + ((size_t)v * NTP + threadIdx.x) * 4, acc.c[v / NB][v % NB]);
   }
   static __device__ __forceinline__ void add_partial(Acc &acc, const float *src) {
     if (threadIdx.x >= NTP) return;
 #pragma unroll
-    for (int i = 0; i < MB; ++i) acc.c[i] += ld_coherent(src + ((size_t)i * NTP + threadIdx.x) * 4);
+    for (int v = 0; v < NV4; ++v) acc.c[v / NB][v % NB] += ld_coherent(src + ((size_t)v * NTP + threadIdx.x) * 4);
   }
   static __device__ __forceinline__ void atomic_partial(const Acc &acc, float *dst) {
     if (threadIdx.x >= NTP) return;
 #pragma unroll
-    for (int i = 0; i < MB; ++i)
+    for (int v = 0; v < NV4; ++v)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) atomic_add_f32(dst + (size_t)(i * 4 + e) * NTP + threadIdx.x, acc.c[i][e]);
+      for (int e = 0; e < 4; ++e) atomic_add_f32(dst + (size_t)(v * 4 + e) * NTP + threadIdx.x, acc.c[v / NB][v % NB][e]);
   }
   static __device__ __forceinline__ void take_partial(Acc &acc, float *src) {
     if (threadIdx.x >= NTP) return;
 #pragma unroll
-    for (int i = 0; i < MB; ++i)
+    for (int v = 0; v < NV4; ++v)
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        float *p = src + (size_t)(i * 4 + e) * NTP + threadIdx.x;
-        acc.c[i][e] = ld_coherent_scalar(p);
+        float *p = src + (size_t)(v * 4 + e) * NTP + threadIdx.x;
+        acc.c[v / NB][v % NB][e] = ld_coherent_scalar(p);
         st_coherent(p, 0.f);
       }
   }

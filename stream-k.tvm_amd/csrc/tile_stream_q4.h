@@ -191,7 +191,7 @@ struct TileStreamQ4 : TileStreamPairs<1, 1, WN_, RK_, 3, false> {
       ws = ws + 1 == WD ? 0 : ws + 1;
       as = as + 1 == AD ? 0 : as + 1;
     }
-    acc.c[0] = part[0] + part[1];
+    acc.c[0][0] = part[0] + part[1];
     // the loads still in flight (they fetch nothing) write LDS: let them land before the rings are reused
     wait_loads<0>();
     __syncthreads();
@@ -199,11 +199,11 @@ struct TileStreamQ4 : TileStreamPairs<1, 1, WN_, RK_, 3, false> {
     // ---- sum the partial accumulators of the waves that split K into the first WN waves (through the weights'
     // rings, free by now) ----
     float *red = reinterpret_cast<float *>(smem);
-    if (wave >= WN) *reinterpret_cast<AccV *>(red + ((wave - WN) * 64 + lane) * 4) = acc.c[0];
+    if (wave >= WN) *reinterpret_cast<AccV *>(red + ((wave - WN) * 64 + lane) * 4) = acc.c[0][0];
     __syncthreads();
     if (wave < WN) {
 #pragma unroll
-      for (int r = 1; r < KH * RK; ++r) acc.c[0] += *reinterpret_cast<const AccV *>(red + (((r - 1) * WN + wave) * 64 + lane) * 4);
+      for (int r = 1; r < KH * RK; ++r) acc.c[0][0] += *reinterpret_cast<const AccV *>(red + (((r - 1) * WN + wave) * 64 + lane) * 4);
     }
     __syncthreads();
   }
