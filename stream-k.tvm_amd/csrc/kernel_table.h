@@ -263,10 +263,13 @@ struct KernelInfo {
   X(293, 2, 2, 2, 1, 3, 2, 2, true)
 
 // Up to 16 rows of A, Q4 weights (row-major, scalar zero point) streaming through LDS in contiguous loads
-// (tile_stream_q4.h; dtype SK_Q4, variant 4):  X(id, WN, RK, WD, AD)
+// (tile_stream_q4.h; dtype SK_Q4, variant 4):  X(id, WN, RK, KH, WD, AD)
 #define SK_STREAM_Q4_KERNELS(X) \
-  X(290, 4, 1, 5, 4)            \
-  X(291, 2, 2, 5, 2)
+  X(290, 4, 1, 2, 5, 4)         \
+  X(291, 2, 2, 2, 5, 2)
+// (an instance with eight rings, 128 weight rows and one wave per ring -- X(294, 8, 1, 1, 3, 3): half the bytes of A per
+// byte of weights -- was measured and is not built: 16 x 16384 x 16384 split in two over K 39.7 us against 39.4 for the
+// 64-row instance and 37.5 for the general kernel, 16 x 8192 x 8192 17.8 against 13.8)
 
 // bfloat16 twins of the fp16 matrix-vector kernels (dtype SK_BF16, variant 2)
 #define SK_GEMV_BF16_KERNELS(X) \

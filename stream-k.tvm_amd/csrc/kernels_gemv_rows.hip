@@ -65,11 +65,11 @@ int gemv_rows_kernel_infos(KernelInfo *out, int max) {
   }
   SK_STREAM_BLOCKS_KERNELS(X)
 #undef X
-#define X(id, WN, RK, WD, AD)                                                                                   \
+#define X(id, WN, RK, KH, WD, AD)                                                                                   \
   if (n < max) {                                                                                                \
-    typedef TileStreamQ4<WN, RK, WD, AD> P;                                                                     \
+    typedef TileStreamQ4<WN, RK, KH, WD, AD> P;                                                                     \
     out[n++] = KernelInfo{id, FAMILY_SKINNY, 2 /* SK_Q4 */, 0, 4, P::BM, P::BN, P::BKC, P::NT, P::LDS_BYTES, P::CTAS_PER_CU, \
-                          P::TILE_ELEMS, 0, P::MAX_M, 256, "stream_q4_wn" #WN "_rk" #RK "_d" #WD};              \
+                          P::TILE_ELEMS, 0, P::MAX_M, 256, "stream_q4_wn" #WN "_rk" #RK "_kh" #KH "_d" #WD};              \
   }
   SK_STREAM_Q4_KERNELS(X)
 #undef X
@@ -127,9 +127,9 @@ int launch_gemv_rows(int id, const SkinnyArgs &a, const DevPlan &p, const Worksp
   }
     SK_STREAM_BLOCKS_KERNELS(X)
 #undef X
-#define X(id_, WN, RK, WD, AD)                   \
+#define X(id_, WN, RK, KH, WD, AD)                   \
   case id_: {                                    \
-    typedef TileStreamQ4<WN, RK, WD, AD> P;      \
+    typedef TileStreamQ4<WN, RK, KH, WD, AD> P;      \
     return launch_policy<P>(a, p, ws, s, bias);  \
   }
     SK_STREAM_Q4_KERNELS(X)
@@ -204,9 +204,9 @@ int occupancy_gemv_rows(int id) {
   }
     SK_STREAM_BLOCKS_KERNELS(X)
 #undef X
-#define X(id_, WN, RK, WD, AD)                                                                           \
+#define X(id_, WN, RK, KH, WD, AD)                                                                           \
   case id_: {                                                                                            \
-    typedef TileStreamQ4<WN, RK, WD, AD> P;                                                              \
+    typedef TileStreamQ4<WN, RK, KH, WD, AD> P;                                                              \
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_skinny_kernel<P>, P::NT, 0) != hipSuccess) \
       return -1;                                                                                         \
     return occ;                                                                                          \

@@ -43,7 +43,6 @@ struct TileStreamPairs {
   // AD slots of A (three unless LDS is short): its loads are issued later than the weights' when DEPTH_ is larger
   static constexpr int MB = MB_, NB = NB_, WM = WM_, WN = WN_, RK = RK_, WD = DEPTH_, AD = AD_, NT = 256;
   static constexpr bool PADDED = PADDED_;
-  static_assert(WM * WN * RK == 4, "four waves");
   static_assert(WM == 1 || WM == 2, "the eight loads of a weight ring are shared out among WM_ waves");
   static constexpr int BM = 16 * MB * WM, BN = 16 * NB * WN, MAX_M = BM;
   static constexpr int BK = 256, BKC = 256 * RK;       // K-values per iteration: of a wave, of the CTA
@@ -56,16 +55,13 @@ struct TileStreamPairs {
   static constexpr int A_SLOT = RK * A_CHUNK;          // the tile's rows of A of one iteration
   static constexpr int RINGS = WN * NB * RK;           // one ring per block of 16 weight rows and K sub-block
   static constexpr int LDS_W = RINGS * WD * W_SLOT, LDS_BYTES = LDS_W + AD * A_SLOT, LDS_TOTAL = LDS_BYTES;
-  static_assert(LDS_BYTES <= 160 * 1024, "the rings must fit the LDS of a CU");
   static_assert(WD >= AD && AD >= 2, "the barrier of an iteration frees the slots read an iteration earlier");
-  static_assert((RK - 1) * WN * WM * 64 * MB * NB * 16 <= LDS_W, "the sums of the K-splitting waves pass through the weights' rings");
   static constexpr int CTAS_PER_CU = (160 * 1024) / (LDS_BYTES + 64) > 0 ? (160 * 1024) / (LDS_BYTES + 64) : 1;
   static constexpr int WAVES_PER_EU = CTAS_PER_CU;
   static constexpr int TILE_ELEMS = BM * BN;
   static constexpr int NTP = WM * WN * 64;             // the rk == 0 waves hold the tile's sums
   static constexpr int NV4 = MB * NB;
   static constexpr int LOADS_W = NB * 8 / WM, LOADS_A = (A_PAIRS * RK) / 4;  // direct-to-LDS loads per wave and iteration
-  static_assert((A_PAIRS * RK) % 4 == 0, "the loads of A are shared out evenly");
   // Loads are issued in the order A(t + AD - 1), W(t + WD - 1) in iteration t, and complete in that order.  Iteration t
   // needs everything up to A(t) and W(t): with WD == AD that leaves the AD - 2 later iterations outstanding, with
   // WD > AD (W(t) is older than A(t)) the weights issued with A(t) and the AD - 2 iterations after them.
@@ -82,6 +78,11 @@ struct TileStreamPairs {
   }
 
   static __device__ __forceinline__ void mac(const Args &a, Acc &acc, int pm, int pn, int k0, int n, char *smem) {
+    // (checked here and not in the class: tile_stream_q4.h derives from instances it does not run this loop of)
+    static_assert(WM * WN * RK == 4, "four waves");
+    static_assert(LDS_BYTES <= 160 * 1024, "the rings must fit the LDS of a CU");
+    static_assert((RK - 1) * WN * WM * 64 * MB * NB * 16 <= LDS_W, "the sums of the K-splitting waves pass through the weights' rings");
+    static_assert((A_PAIRS * RK) % 4 == 0, "the loads of A are shared out evenly");
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
     const int wm = wave % WM, wn = (wave / WM) % WN, rk = wave / (WM * WN);

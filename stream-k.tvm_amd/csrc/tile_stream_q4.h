@@ -7,8 +7,9 @@
 // general kernel's loads deliver, and the decode (q4_dequant.h: bit-exact fp16((q - zero) * scale)) and the
 // 16x16x32 MFMAs are the same.
 //
-//  * CTA = eight waves, two per SIMD: WN_ along N x RK_ along K own a ring of weights each (WN_ RK_ = 4), and two
-//    waves share a ring, each taking 256 of the 512 K-values of an iteration (the decode keeps the vector pipeline
+//  * CTA = eight waves, two per SIMD: WN_ along N x RK_ along K rings of weights, KH_ waves per ring (four rings shared
+//    by two waves each, which take 256 of the 512 K-values of an iteration; or eight rings, 128 weight rows, one wave
+//    each) (the decode keeps the vector pipeline
 //    busy: the second wave of a SIMD works while the first waits for LDS or for its MFMAs).  Per iteration and ring:
 //    four loads of weights (16 rows x 256 bytes) shared out between its two waves, one load of scales per wave (16
 //    rows x the wave's 2 groups, four bytes per lane), and the 16 RK_ loads of A (one row of 1024 bytes each) shared
@@ -36,32 +37,36 @@
 
 namespace sk {
 
-template <int WN_, int RK_, int WD_, int AD_>
+template <int WN_, int RK_, int KH_, int WD_, int AD_>
 struct TileStreamQ4 : TileStreamPairs<1, 1, WN_, RK_, 3, false> {
   typedef TileStreamPairs<1, 1, WN_, RK_, 3, false> Base;
   typedef typename Base::Args Args;
   typedef typename Base::Acc Acc;
   typedef typename Base::AccV AccV;
-  static constexpr int KH = 2;                         // waves that share the weights of an iteration, 256 K-values each
-  static constexpr int WN = WN_, RK = RK_, WD = WD_, AD = AD_, NT = 64 * 4 * KH, BM = 16, BN = 16 * WN, MAX_M = 16;
+  static constexpr int KH = KH_;                       // waves that share the weights of an iteration, 512 / KH_ K-values each
+  static constexpr int STEPS = 4 / KH;                 // steps of 128 K-values (one scale group) per wave and iteration
+  static constexpr int RINGS = WN_ * RK_, NWAVES = RINGS * KH;
+  static_assert(KH == 1 || KH == 2, "one or two waves per ring");
+  static constexpr int WN = WN_, RK = RK_, WD = WD_, AD = AD_, NT = 64 * NWAVES, BM = 16, BN = 16 * WN, MAX_M = 16;
   static constexpr int BK = 512, BKC = 512 * RK;       // K-values per iteration: of a weight ring, of the CTA
   static constexpr int W_SLOT = 16 * 256;              // 16 weight rows x 256 bytes
-  static constexpr int S_SLOT = 256;                   // a wave's scales: 16 rows x 2 groups in lanes 0..15 of one load
+  static constexpr int S_SLOT = 256;                   // a wave's scales: 16 rows x STEPS groups in the first lanes of one load
   static constexpr int A_CHUNK = 16 * 1024;            // 16 rows of A x 512 K-values
   static constexpr int A_SLOT = RK * A_CHUNK;
-  static constexpr int LDS_W = 4 * WD * W_SLOT, LDS_S = 4 * KH * WD * S_SLOT;
+  static constexpr int LDS_W = RINGS * WD * W_SLOT, LDS_S = NWAVES * WD * S_SLOT;
   static constexpr int LDS_BYTES = LDS_W + LDS_S + AD * A_SLOT, LDS_TOTAL = LDS_BYTES;
   static_assert(LDS_BYTES <= 160 * 1024, "the rings must fit the LDS of a CU");
-  static_assert(WD > AD && AD >= 2, "weights are requested further ahead than A");
-  static_assert((4 * KH - WN) * 64 * 16 <= LDS_W, "the sums of the K-splitting waves pass through the weights' rings");
+  static_assert(WD >= AD && AD >= 2, "weights are requested at least as far ahead as A");
+  static_assert((NWAVES - WN) * 64 * 16 <= LDS_W, "the sums of the K-splitting waves pass through the weights' rings");
+  static_assert((16 * RK) % NWAVES == 0, "the loads of A are shared out evenly");
   static constexpr int CTAS_PER_CU = 1, WAVES_PER_EU = KH;
   static constexpr int TILE_ELEMS = BM * BN;
   // direct-to-LDS loads per wave and iteration: half of the ring's four loads of weights, the wave's own scales,
   // its share of the iteration's 16 RK rows of A
-  static constexpr int LOADS_W = 4 / KH + 1, LOADS_A = 16 * RK / (4 * KH);
+  static constexpr int LOADS_W = 4 / KH + 1, LOADS_A = 16 * RK / NWAVES;
   // at the top of iteration t everything up to A(t) has to be there: what may still be on its way are the weights
-  // issued behind A(t) and the AD - 2 iterations of loads after them
-  static constexpr int OUTSTANDING = LOADS_W + (AD - 2) * (LOADS_W + LOADS_A);
+  // issued behind A(t) (when they are requested further ahead than A) and the AD - 2 iterations of loads after them
+  static constexpr int OUTSTANDING = (WD > AD ? LOADS_W : 0) + (AD - 2) * (LOADS_W + LOADS_A);
 
   template <int N>
   static __device__ __forceinline__ void wait_loads() {
@@ -78,7 +83,7 @@ struct TileStreamQ4 : TileStreamPairs<1, 1, WN_, RK_, 3, false> {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
     // wave = (kh RK + rk) WN + wn: the waves that end up with the tile's sums come first
-    const int wn = wave % WN, rk = (wave / WN) % RK, kh = wave / (WN * RK);
+    const int wn = wave % WN, rk = (wave / WN) % RK, kh = wave / RINGS;
     const int ring = rk * WN + wn;
     AccV part[2] = {AccV{0, 0, 0, 0}, AccV{0, 0, 0, 0}};
 
@@ -101,8 +106,8 @@ struct TileStreamQ4 : TileStreamPairs<1, 1, WN_, RK_, 3, false> {
       piece_w[jj] = wp0 ^ (4 * (kh * (4 / KH) + jj));
       voff_w[jj] = (uint32_t)wr * ldw_bytes + (uint32_t)piece_w[jj] * 16;
     }
-    // scales: lanes 0..15, one per row, four bytes (the two groups of the wave's 256 K-values)
-    const uint32_t voff_s = lane < 16 ? (uint32_t)lane * lds_bytes : OOB_OFFSET;
+    // scales: STEPS / 2 lanes per row, four bytes each (the groups of the wave's 128 STEPS K-values)
+    const uint32_t voff_s = lane < 8 * STEPS ? (uint32_t)(lane / (STEPS / 2)) * lds_bytes + (uint32_t)(lane % (STEPS / 2)) * 4 : OOB_OFFSET;
     // fragments: wave kh takes the steps s = 2 kh, 2 kh + 1 of the iteration; lane (i, g) reads piece 4 s + g of
     // weight row i, found at position (4 s + g) ^ i, and for word q of it the eight values of A row i from K offset
     // 32 (4 s + g) + 8 q: piece 16 s + 4 g + q, at position piece ^ i
@@ -111,14 +116,14 @@ struct TileStreamQ4 : TileStreamPairs<1, 1, WN_, RK_, 3, false> {
     const uint32_t w_ring = (uint32_t)__builtin_amdgcn_readfirstlane((int)(base + (uint32_t)ring * (WD * W_SLOT)));
     const uint32_t s_ring = (uint32_t)__builtin_amdgcn_readfirstlane((int)(base + (uint32_t)(LDS_W + wave * (WD * S_SLOT))));
     const uint32_t a_ring = (uint32_t)__builtin_amdgcn_readfirstlane((int)(base + (uint32_t)(LDS_W + LDS_S)));
-    const char *w_rd[2], *a_rd[4];
+    const char *w_rd[STEPS], *a_rd[4];
 #pragma unroll
-    for (int ss = 0; ss < 2; ++ss)
-      w_rd[ss] = smem + ring * (WD * W_SLOT) + fi * 256 + 64 * ((2 * kh + ss) ^ (fi >> 2)) + 16 * (fg ^ (fi & 3));
+    for (int ss = 0; ss < STEPS; ++ss)
+      w_rd[ss] = smem + ring * (WD * W_SLOT) + fi * 256 + 64 * ((STEPS * kh + ss) ^ (fi >> 2)) + 16 * (fg ^ (fi & 3));
 #pragma unroll
     for (int q = 0; q < 4; ++q)
-      a_rd[q] = smem + LDS_W + LDS_S + rk * A_CHUNK + fi * 1024 + 512 * kh + 16 * ((4 * fg + q) ^ fi);
-    const char *s_rd = smem + LDS_W + wave * (WD * S_SLOT) + fi * 4;
+      a_rd[q] = smem + LDS_W + LDS_S + rk * A_CHUNK + fi * 1024 + 256 * STEPS * kh + 16 * ((4 * fg + q) ^ fi);
+    const char *s_rd = smem + LDS_W + wave * (WD * S_SLOT) + fi * (2 * STEPS);
     const Q4Consts qc = q4_consts(a.zero);
 
     // iteration t of the segment (t = 0 .. n - 1) covers K-values k_of(t) 512 RK ..; iterations past the segment and
@@ -135,7 +140,7 @@ struct TileStreamQ4 : TileStreamPairs<1, 1, WN_, RK_, 3, false> {
                     (t < n && kk + piece_w[jj] * 32 < a.K) ? voff_w[jj] : OOB_OFFSET, kbytes + (uint32_t)(4 * j) * ldw_bytes);
       }
       dma_load_4(rsrc_s, s_ring + (uint32_t)(slot * S_SLOT), t < n ? voff_s : OOB_OFFSET,
-                 (uint32_t)__builtin_amdgcn_readfirstlane((kk / 128 + 2 * kh) * 2));
+                 (uint32_t)__builtin_amdgcn_readfirstlane((kk / 128 + STEPS * kh) * 2));
     };
     auto issue_a = [&](int t, int slot) {
 #pragma unroll
@@ -163,16 +168,17 @@ struct TileStreamQ4 : TileStreamPairs<1, 1, WN_, RK_, 3, false> {
       issue_a(t + AD - 1, as == 0 ? AD - 1 : as - 1);
       issue_w(t + WD - 1, ws == 0 ? WD - 1 : ws - 1);
       const int wofs = ws * W_SLOT, aofs = as * A_SLOT;
-      uint4v wf[2];
+      uint4v wf[STEPS];
 #pragma unroll
-      for (int ss = 0; ss < 2; ++ss) wf[ss] = *reinterpret_cast<const uint4v *>(w_rd[ss] + wofs);
+      for (int ss = 0; ss < STEPS; ++ss) wf[ss] = *reinterpret_cast<const uint4v *>(w_rd[ss] + wofs);
       union {
-        uint32_t u;
-        half_t h[2];
+        uint32_t u[STEPS / 2];
+        half_t h[STEPS];
       } sc;
-      sc.u = *reinterpret_cast<const uint32_t *>(s_rd + ws * S_SLOT);
 #pragma unroll
-      for (int ss = 0; ss < 2; ++ss) {
+      for (int d = 0; d < STEPS / 2; ++d) sc.u[d] = *reinterpret_cast<const uint32_t *>(s_rd + ws * S_SLOT + 4 * d);
+#pragma unroll
+      for (int ss = 0; ss < STEPS; ++ss) {
         const half2v sc2 = half2v{sc.h[ss], sc.h[ss]};
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
@@ -198,14 +204,16 @@ struct TileStreamQ4 : TileStreamPairs<1, 1, WN_, RK_, 3, false> {
 
     // ---- sum the partial accumulators of the waves that split K into the first WN waves (through the weights'
     // rings, free by now) ----
-    float *red = reinterpret_cast<float *>(smem);
-    if (wave >= WN) *reinterpret_cast<AccV *>(red + ((wave - WN) * 64 + lane) * 4) = acc.c[0][0];
-    __syncthreads();
-    if (wave < WN) {
+    if constexpr (NWAVES > WN) {
+      float *red = reinterpret_cast<float *>(smem);
+      if (wave >= WN) *reinterpret_cast<AccV *>(red + ((wave - WN) * 64 + lane) * 4) = acc.c[0][0];
+      __syncthreads();
+      if (wave < WN) {
 #pragma unroll
-      for (int r = 1; r < KH * RK; ++r) acc.c[0][0] += *reinterpret_cast<const AccV *>(red + (((r - 1) * WN + wave) * 64 + lane) * 4);
+        for (int r = 1; r < KH * RK; ++r) acc.c[0][0] += *reinterpret_cast<const AccV *>(red + (((r - 1) * WN + wave) * 64 + lane) * 4);
+      }
+      __syncthreads();
     }
-    __syncthreads();
   }
 };
 
