@@ -191,6 +191,10 @@ int sk_workspace_status(void *ws, void *stream);
  * Replaces tl_mod(A, B, C) of streamk_fp16.py:382-387.  C need not be zeroed by the caller
  * (the reference requires it, streamk_fp16.py:385).
  * Requirements: K, lda, ldb multiples of 8 and 16-byte aligned A, B (vector loads).
+ * Results are the same bits on every launch of a plan with the data-parallel, fixed-split or any schedule with
+ * the REDUCE fix-up.  The order in which a tile's K-iterations are summed is the kernel's: the kernels that take
+ * 5 to 64 rows of A (2 to 4 on large weights) start each tile at a different K offset and wrap around, so two
+ * tiles of one launch do not add their products in the same order.
  */
 int sk_gemm_f16(const void *A, const void *B, void *C, int64_t M, int64_t N, int64_t K, int64_t lda,
                 int64_t ldb, int64_t ldc, const sk_plan *plan, void *ws, size_t ws_bytes,

@@ -191,6 +191,23 @@ def test_untuned_plans_keep_cta_ranges_aligned(sk):
     assert (sk.kernel_name(p.kernel_id), p.schedule, p.grid) == ("tile_f16_nt_asm_256x256x64", DP, 256)
     p = sk.make_plan(1024, 8192, 8192, "float16", "nt", cus=256, use_tuned=False)
     assert (sk.kernel_name(p.kernel_id), p.schedule, p.grid) == ("tile_f16_nt_asm_256x256x64", SPLITK, 256)
+    # few rows of A: the kernels that stream the weights through LDS, a tile per CU and no fix-up where N allows it
+    for (M, N, K, dtype, want, grid) in [(16, 8192, 8192, "float16", "stream_f16_mb1_wm1_wn2_rk2_d3", 256),
+                                         (5, 8192, 8192, "bfloat16", "stream_bf16_mb1_wm1_wn2_rk2_d3", 256),
+                                         (16, 16384, 8192, "float16", "stream_f16_mb1_wm1_wn4_rk1_d4", 256),
+                                         (16, 28672, 8192, "float16", "stream_f16_mb1_wm1_wn4_rk1_d4", 256),
+                                         (16, 11008, 4096, "float16", "stream_f16_mb1_wm1_wn4_rk1_d4", 172),
+                                         (32, 8192, 8192, "float16", "stream_f16_mb1_wm2_wn2_rk1_d4", 256),
+                                         (64, 8192, 8192, "float16", "stream_f16_mb2_wm2_wn2_rk1_d3", 256),
+                                         (64, 16384, 8192, "float16", "stream_f16_mb2_nb2_wm2_wn2_rk1_d3", 256),
+                                         (64, 11008, 4096, "bfloat16", "stream_bf16_mb2_nb2_wm2_wn2_rk1_d3", 172),
+                                         (4, 8192, 8192, "float16", "stream_f16_mb1_wm1_wn2_rk2_d3", 256),
+                                         (4, 4096, 4096, "float16", "gemv_rows_f16_m4_wn1_rk4", 256),
+                                         (16, 8192, 8192, "q4", "stream_q4_wn2_rk2_kh2_d5", 256),
+                                         (16, 28672, 8192, "q4", "skinny_q4_mb1_wn4_rk2_row1_0", 448),
+                                         (16, 4096, 4096, "q4", "skinny_q4_mb1_wn2_rk4_row1_0", 128)]:
+        p = sk.make_plan(M, N, K, dtype, "nt", cus=256, use_tuned=False)
+        assert (sk.kernel_name(p.kernel_id), p.schedule, p.grid) == (want, DP, grid), (M, N, K, dtype, sk.kernel_name(p.kernel_id), p.grid)
     # a caller's tile or schedule is not overridden
     p = sk.make_plan(1024, 8192, 8192, "float16", "nt", cus=256, use_tuned=False, bm=128, bn=128)
     assert (p.bm, p.bn) == (128, 128)
