@@ -105,9 +105,11 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
   }
   // (2 <= M <= 4: from about 100 MB of weights on; below, the matrix-vector form with four rows of A starts up faster --
   // 4 x 8192 x 8192: 24.8 us against 32.0 us, 2 x 4096 x 4096: 12.1 us against 11.3 us, weights from HBM)
-  const bool stream_rows = M >= 5 || (M >= 2 && N * K >= (int64_t)48 << 20);
+  // (one row: from 128 MB on -- 1 x 8192 x 8192 24.4 us against 28.9 us for the matrix-vector kernel, 1 x 28672 x 8192
+  // 76.4 / 76.6, 1 x 11008 x 4096 19.8 / 17.6)
+  const bool stream_rows = M >= 5 || (M >= 2 && N * K >= (int64_t)48 << 20) || N * K >= (int64_t)64 << 20;
   if ((dtype == SK_F16 || dtype == SK_BF16) && layout == SK_LAYOUT_NT && stream_rows && M <= 64 && want_variant < 0) {
-    // 5 <= M <= 64 with fp16 / bfloat16 weights: the kernels that stream the weights through LDS in contiguous loads
+    // 5 <= M <= 64 (fewer rows on large weights, above) with fp16 / bfloat16 weights: the kernels that stream the weights through LDS in contiguous loads
     // (tile_stream_pairs.h).  Tiles of 32 weight rows while one wave of them fits the device (N = 8192: one tile per
     // CU and no fix-up), 64 rows beyond; 64 rows of A exist with 32 weight rows only.
     // (more than 32 rows: 64 weight rows where they give three fifths of the CUs a tile -- A is then as many bytes
