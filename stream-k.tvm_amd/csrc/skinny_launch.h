@@ -37,12 +37,29 @@ __device__ __forceinline__ int first_tile_of_block() {
   return b;
 }
 
+// policies with mac_again: what a CTA's later tiles skip because its first tile left it in LDS (the row of A)
+template <class P, class = void>
+struct has_mac_again { static constexpr bool value = false; };
+template <class P>
+struct has_mac_again<P, std::void_t<decltype(&P::mac_again)>> { static constexpr bool value = true; };
+template <class P>
+__device__ __forceinline__ void mac_of_tile(const typename P::Args &a, typename P::Acc &acc, int tile, int ipt, char *smem, bool first) {
+  if constexpr (has_mac_again<P>::value) {
+    if (!first) {
+      P::mac_again(a, acc, 0, tile, 0, ipt, smem);
+      return;
+    }
+  }
+  P::mac(a, acc, 0, tile, 0, ipt, smem);
+}
+
 template <class P>
 __global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_skinny_dp_kernel(typename P::Args a, int total_tiles, int ipt) {
   __shared__ __attribute__((aligned(16))) char smem[P::LDS_BYTES];
   typename P::Acc acc;
-  for (int tile = first_tile_of_block<P>(); tile < total_tiles; tile += gridDim.x) {
-    P::mac(a, acc, 0, tile, 0, ipt, smem);
+  const int tile0 = first_tile_of_block<P>();
+  for (int tile = tile0; tile < total_tiles; tile += gridDim.x) {
+    mac_of_tile<P>(a, acc, tile, ipt, smem, tile == tile0);
     P::store_c(a, acc, 0, tile, smem, nullptr);
   }
 }
@@ -53,8 +70,9 @@ __global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_skinny_dp_kernel_bi
   const void *bias = bias_arg;
   asm volatile("" ::"s"(bias));  // fetched with the other arguments, not before the first store
   typename P::Acc acc;
-  for (int tile = first_tile_of_block<P>(); tile < total_tiles; tile += gridDim.x) {
-    P::mac(a, acc, 0, tile, 0, ipt, smem);
+  const int tile0 = first_tile_of_block<P>();
+  for (int tile = tile0; tile < total_tiles; tile += gridDim.x) {
+    mac_of_tile<P>(a, acc, tile, ipt, smem, tile == tile0);
     P::store_c(a, acc, 0, tile, smem, bias);
   }
 }
