@@ -432,6 +432,9 @@ def main():
                 key = {(bm, bn): t for t, (bm, bn) in tiles.items()}.get((pa.bm, pa.bn))
                 row["auto_tile"], row["auto_kernel"] = [pa.bm, pa.bn, pa.bk], streamk.kernel_name(pa.kernel_id)
                 row["auto_streamk_tiles"], row["auto_grid"] = pa.streamk_tiles, pa.grid
+                # (reduce16: the tuned entry exchanges its half tiles rounded to 16 bits; the sk_* rows beside it use
+                # the fp32 REDUCE)
+                row["auto_fixup"] = {v: k for k, v in streamk._lib.FIXUPS.items()}.get(pa.fixup, pa.fixup) if pa.streamk_tiles else "none"
                 if key is None:
                     pd = streamk.make_plan(m, N, K, "float16", "nt", bm=pa.bm, bn=pa.bn, bk=pa.bk, schedule="dp", raster=8)
                     ms = time_graph(lambda: streamk.streamk_fp16(a, B, out=c, plan=pd))
@@ -793,8 +796,10 @@ def main():
                     "torch_matmul_us": row["torch_matmul_weights_from_hbm_us"]}
             if row["M"] in (256, 512, 1024):
                 parts["streamk_vs_data_parallel_N8192_K8192"][f"M{row['M']}"] = {
-                    "auto_tflops": row["auto"], "auto_tile": row["auto_tile"], "sk_over_dp_same_tile": row["sk_over_dp_same_tile"],
-                    "auto_over_best_dp": row["auto_over_best_dp"]}
+                    "auto_tflops": row["auto"], "auto_tile": row["auto_tile"], "auto_fixup": row["auto_fixup"],
+                    "sk_over_dp_same_tile": row["sk_over_dp_same_tile"], "auto_over_best_dp": row["auto_over_best_dp"],
+                    "fp32_reduce_over_best_dp": round(max(row.get("sk_" + t, 0.0) for t in ("128", "128x256", "256")) /
+                                                      max(v for k, v in row.items() if k.startswith("dp_")), 3)}
         for row in q4:
             parts["q4_gemm_N8192_K8192"][f"M{row['M']}"] = {
                 "us_weights_in_infinity_cache": row["tuned"]["us"], "frac_hbm_weights_in_infinity_cache": row["tuned"]["frac_hbm"],

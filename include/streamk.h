@@ -74,6 +74,15 @@ typedef enum sk_fixup {
                               is less accurate than the other two, and like ATOMIC not reproducible.  fp16 and
                               bfloat16 tile kernels with 16x16 accumulator blocks only (256x256, 128x128,
                               128x256, 256x128); N and ldc even, C 4-byte aligned; no bias / activation */
+  ,
+  SK_FIXUP_REDUCE16 = 4    /* SK_FIXUP_REDUCE with the exchanged partial sums rounded to C's 16-bit type, as the
+                              reference's fix-up rounds them (streamk_fp16.py:248-255), and added in fp32 by the
+                              CTA that finishes the tile: half the bytes through memory, which is what the
+                              exchange costs (1024 x 8192 x 8192 on 256 x 256 tiles cut in two: 105 -> 97 us).
+                              Still the same bits on every launch.  Only for plans whose every Stream-K tile
+                              is cut into two or four equal segments on the fp16 / bfloat16 256 x 256 assembly-
+                              loop kernel (the fixed split in two or four, `basic` with a grid of two or four
+                              CTAs per tile); anything else is refused.  Never chosen by SK_FIXUP_AUTO */
 } sk_fixup;
 
 typedef enum sk_dtype {

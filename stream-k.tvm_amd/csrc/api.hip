@@ -134,6 +134,9 @@ __global__ void zero_pairs_kernel(uint32_t *C, int M, int pairs, int64_t ld) {
   }
 }
 
+// the ordered reduce, with fp32 or 16-bit partial tiles
+static inline bool is_reduce(int fixup) { return fixup == SK_FIXUP_REDUCE || fixup == SK_FIXUP_REDUCE16; }
+
 int check_plan(const sk_plan *plan, int64_t M, int64_t N, int64_t K, int dtype, int layout) {
   if (!plan) return SK_ERR_NULL;
   if (plan->M != M || plan->N != N || plan->K != K || plan->dtype != dtype || plan->layout != layout)
@@ -150,13 +153,13 @@ int make_dev_plan(const sk_plan *plan, const KernelInfo *k, void *ws, size_t ws_
   const DeviceInfo d = device_info();
   if (!d.ok) return SK_ERR_DEVICE;
   // every CTA of the Stream-K wave may wait on another one: they must all be resident
-  if (plan->streamk_tiles > 0 && plan->fixup == SK_FIXUP_REDUCE &&
+  if (plan->streamk_tiles > 0 && is_reduce(plan->fixup) &&
       (occupancy <= 0 || plan->grid > d.cus * occupancy))
     return SK_ERR_CONFIG;
   if (plan->workspace_bytes > 0 && is_static) {
     char *base = static_cast<char *>(ws);
     // (REDUCE: one flag per CTA, and a second one for the two-round exchange of tiles cut into four)
-    const int nflags = plan->fixup == SK_FIXUP_REDUCE ? 2 * plan->grid : plan->streamk_tiles;
+    const int nflags = is_reduce(plan->fixup) ? 2 * plan->grid : plan->streamk_tiles;
     const size_t units = (ws_bytes - (size_t)WS_PART_OFF) / 256;
     hipLaunchKernelGGL(prepare_static_kernel, dim3(1024), dim3(256), 0, stream, reinterpret_cast<int *>(base),
                        reinterpret_cast<int *>(base + 256), nflags, reinterpret_cast<uint4v *>(base + WS_PART_OFF),
@@ -174,7 +177,7 @@ int make_dev_plan(const sk_plan *plan, const KernelInfo *k, void *ws, size_t ws_
       if (plan->fixup == SK_FIXUP_ATOMIC) {
         wide_clean = it->second.maybe_dirty;
         it->second.maybe_dirty = false;
-      } else if (plan->fixup == SK_FIXUP_REDUCE && plan->streamk_tiles > 0) {
+      } else if (is_reduce(plan->fixup) && plan->streamk_tiles > 0) {
         it->second.maybe_dirty = true;
       }
     }
@@ -212,10 +215,17 @@ int make_dev_plan(const sk_plan *plan, const KernelInfo *k, void *ws, size_t ws_
   dp->raster_tail = plan->num_block_m % raster ? plan->num_block_m % raster : raster;
   // every Stream-K tile cut into exactly two equal CTA segments: both CTAs of a pair finish half a tile
   dp->halves = 0;
-  if (plan->fixup == SK_FIXUP_REDUCE && plan->streamk_tiles > 0 && plan->streamk_partial_tiles == 0) {
+  if (is_reduce(plan->fixup) && plan->streamk_tiles > 0 && plan->streamk_partial_tiles == 0) {
     if (2 * plan->streamk_full_tiles == plan->iters_per_tile) dp->halves = 1;
     // four equal segments: two rounds of the same exchange (the second round's flags follow the first `grid` ones)
     if (4 * plan->streamk_full_tiles == plan->iters_per_tile && 2 * (int64_t)plan->grid <= WS_MAX_FLAGS) dp->halves = 2;
+  }
+  dp->partials16 = 0;
+  if (plan->fixup == SK_FIXUP_REDUCE16) {
+    // (a plan that sk_make_plan would not have made: refuse it rather than run another fix-up than it names)
+    if (!(dp->halves > 0 && k->family == FAMILY_TILE && k->variant == 7 && (plan->dtype == SK_F16 || plan->dtype == SK_BF16)))
+      return SK_ERR_CONFIG;
+    dp->partials16 = 1;
   }
   dp->by_ipt = FastDiv::make(plan->iters_per_tile);
   dp->by_tiles_n = FastDiv::make(plan->num_block_n);

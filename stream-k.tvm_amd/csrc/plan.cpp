@@ -516,7 +516,15 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
   out->dp_waves = (int32_t)cdiv(out->blocking_tiles, grid);
   int fixup = cfg ? cfg->fixup : SK_FIXUP_AUTO;
   if (fixup == SK_FIXUP_AUTO) fixup = SK_FIXUP_REDUCE;
-  if (fixup != SK_FIXUP_ATOMIC && fixup != SK_FIXUP_REDUCE && fixup != SK_FIXUP_ATOMIC_C) return SK_ERR_CONFIG;
+  if (fixup != SK_FIXUP_ATOMIC && fixup != SK_FIXUP_REDUCE && fixup != SK_FIXUP_ATOMIC_C && fixup != SK_FIXUP_REDUCE16)
+    return SK_ERR_CONFIG;
+  // partial sums exchanged in 16 bits: the assembly-loop kernels for fp16 / bfloat16, every Stream-K tile cut into two
+  // or four equal segments (what the device side's exchange of half tiles handles)
+  if (fixup == SK_FIXUP_REDUCE16 &&
+      !(k->family == FAMILY_TILE && k->variant == 7 && (dtype == SK_F16 || dtype == SK_BF16) && sk_tiles > 0 &&
+        out->streamk_partial_tiles == 0 &&
+        (2 * out->streamk_full_tiles == out->iters_per_tile || 4 * out->streamk_full_tiles == out->iters_per_tile)))
+    return SK_ERR_CONFIG;
   // packed 16-bit atomics into C: the 16-bit tile kernels with 16x16 accumulator blocks
   if (fixup == SK_FIXUP_ATOMIC_C &&
       !(k->family == FAMILY_TILE && (k->variant == 4 || k->variant == 5 || k->variant == 7) &&
@@ -544,7 +552,7 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
   // changes which tiles a CTA takes -- never reach the fix-up: no workspace)
   const bool whole_tiles = out->streamk_partial_tiles == 0 && out->streamk_full_tiles % out->iters_per_tile == 0;
   if (sk_tiles > 0 && fixup != SK_FIXUP_ATOMIC_C && !whole_tiles) {
-    const int64_t nflags = fixup == SK_FIXUP_REDUCE ? grid : sk_tiles;
+    const int64_t nflags = (fixup == SK_FIXUP_REDUCE || fixup == SK_FIXUP_REDUCE16) ? grid : sk_tiles;
     if (nflags > WS_MAX_FLAGS) return SK_ERR_CONFIG;
     ws = WS_PART_OFF + nflags * (int64_t)k->partial_elems * 4;
   }

@@ -58,6 +58,7 @@ struct DevPlan {
   int xcd_remap;              // 1: spread logical CTA ids so each XCD owns a contiguous range
   int raster_tail;            // tile rows in the last raster group (tiles_m % raster, or raster)
   int halves;                 // REDUCE plan whose every Stream-K tile is cut into two (1) or four (2) equal CTA segments
+  int partials16;             // such a plan exchanges its half tiles rounded to C's 16-bit type (SK_FIXUP_REDUCE16)
   int perm_s, perm_g;         // perm_s > 1: Stream-K tile v stands at position (v % perm_s) * perm_g + v / perm_s
   FastDiv by_ipt, by_tiles_n, by_width, by_raster, by_tail, by_full1, by_full, by_perm;
 };

@@ -21,6 +21,32 @@ struct fixup_word_in_lds { static constexpr bool value = false; };
 template <class P>
 struct fixup_word_in_lds<P, std::void_t<decltype(P::FIXUP_WORD_IN_LDS)>> { static constexpr bool value = P::FIXUP_WORD_IN_LDS; };
 
+// policies whose half tiles can travel rounded to 16 bits (store_partial_half16 / add_partial_half16)
+template <class P, class = void>
+struct has_halves16 { static constexpr bool value = false; };
+template <class P>
+struct has_halves16<P, std::void_t<decltype(P::HALVES16)>> { static constexpr bool value = P::HALVES16; };
+template <class P>
+__device__ __forceinline__ void park_half(const DevPlan &plan, const typename P::Acc &acc, float *dst, int h) {
+  if constexpr (has_halves16<P>::value) {
+    if (plan.partials16) {
+      P::store_partial_half16(acc, dst, h);
+      return;
+    }
+  }
+  P::store_partial_half(acc, dst, h);
+}
+template <class P>
+__device__ __forceinline__ void take_half(const DevPlan &plan, typename P::Acc &acc, const float *src, int h) {
+  if constexpr (has_halves16<P>::value) {
+    if (plan.partials16) {
+      P::add_partial_half16(acc, src, h);
+      return;
+    }
+  }
+  P::add_partial_half(acc, src, h);
+}
+
 // optional members of a policy: COHERENT_REDUCE (partials of the REDUCE fix-up travel with device-scope
 // accesses; default: as COHERENT_PARTIALS says), HALVES (the policy has store_partial_half /
 // add_partial_half / store_c_half, see below) and ATOMIC_C (the policy has atomic_c: its accumulators added to C
@@ -176,21 +202,21 @@ __device__ __forceinline__ void run_persistent(const typename P::Args &a, const 
             const int half = q & 1, peer1 = base + (q ^ 1);
             const int units = (int)(((size_t)(pid + 1) * P::TILE_ELEMS * 4 + 255) >> 8);
             bool ok = true;
-            P::store_partial_half(acc, ws.partials + (size_t)pid * P::TILE_ELEMS, 1 - half);
+            park_half<P>(plan, acc, ws.partials + (size_t)pid * P::TILE_ELEMS, 1 - half);
             signal_partial_ready<true>(&ws.flags[pid], ws.status + WS_DIRTY, units);
             if (wait_partials_ready<true>(&ws.flags[peer1], 1, plan.spin_limit)) {
-              P::add_partial_half(acc, ws.partials + (size_t)peer1 * P::TILE_ELEMS, half);
+              take_half<P>(plan, acc, ws.partials + (size_t)peer1 * P::TILE_ELEMS, half);
               clear_flags_after_use(&ws.flags[peer1], 1);
             } else {
               ok = false;
             }
             if (q >= 2) {
-              P::store_partial_half(acc, ws.partials + (size_t)pid * P::TILE_ELEMS, half);
+              park_half<P>(plan, acc, ws.partials + (size_t)pid * P::TILE_ELEMS, half);
               signal_partial_ready<true>(&ws.flags[plan.grid + pid], ws.status + WS_DIRTY, units);
             } else {
               const int peer2 = pid + 2;
               if (wait_partials_ready<true>(&ws.flags[plan.grid + peer2], 1, plan.spin_limit)) {
-                P::add_partial_half(acc, ws.partials + (size_t)peer2 * P::TILE_ELEMS, half);
+                take_half<P>(plan, acc, ws.partials + (size_t)peer2 * P::TILE_ELEMS, half);
                 clear_flags_after_use(&ws.flags[plan.grid + peer2], 1);
               } else {
                 ok = false;
@@ -201,13 +227,13 @@ __device__ __forceinline__ void run_persistent(const typename P::Args &a, const 
             continue;
           }
           const int half = k0 != 0 ? 1 : 0, peer = k0 != 0 ? pid - 1 : pid + 1;
-          P::store_partial_half(acc, ws.partials + (size_t)pid * P::TILE_ELEMS, 1 - half);
+          park_half<P>(plan, acc, ws.partials + (size_t)pid * P::TILE_ELEMS, 1 - half);
           signal_partial_ready<true>(&ws.flags[pid], ws.status + WS_DIRTY,
                                      (int)(((size_t)(pid + 1) * P::TILE_ELEMS * 4 + 255) >> 8));
           if (!wait_partials_ready<true>(&ws.flags[peer], 1, plan.spin_limit)) {
             if (threadIdx.x == 0) ws.status[WS_STATUS] = -8;  // SK_ERR_TIMEOUT
           } else {
-            P::add_partial_half(acc, ws.partials + (size_t)peer * P::TILE_ELEMS, half);
+            take_half<P>(plan, acc, ws.partials + (size_t)peer * P::TILE_ELEMS, half);
             clear_flags_after_use(&ws.flags[peer], 1);
           }
           P::store_c_half(a, acc, pm, pn, smem, bias, half);

@@ -462,6 +462,66 @@ struct TileF16Asm {
       });
     });
   }
+  // The same exchange with the partial sums rounded to C's 16-bit type (SK_FIXUP_REDUCE16: half the bytes through
+  // memory; fp16 / bfloat16 kernels).  Groups v and v + 1 of thread t travel as eight 16-bit values at
+  // (v / 2 * NT + t) * 16; the receiver widens them and adds in fp32.
+  static constexpr bool HALVES16 = MODE_ <= 1;
+  static __device__ __forceinline__ uint32_t pack16(float lo, float hi) {
+    uint32_t r;
+    if constexpr (BF16_)
+      asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(lo), "v"(hi));
+    else
+      asm("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(r) : "v"(lo), "v"(hi));
+    return r;
+  }
+  static __device__ __forceinline__ float widen16(uint32_t w, int hi) {
+    if constexpr (BF16_) return __builtin_bit_cast(float, hi ? (w & 0xffff0000u) : (w << 16));
+    const half2v h = __builtin_bit_cast(half2v, w);
+    return (float)h[hi];
+  }
+  template <int V0, int V1>
+  static __device__ __forceinline__ void store_groups16(float *dst) {
+    static_assert((V0 | V1) % 2 == 0, "pairs of groups");
+    const BufferRsrc r = make_rsrc(dst, TILE_ELEMS * 2);
+    const uint32_t off = (uint32_t)pin_here((int)threadIdx.x) * 16;
+    static_for<V0 / 2, V1 / 2>([&](auto g) {
+      constexpr int v = decltype(g)::value;
+      const floatx4 a0 = agpr_read4<(2 * v) * 4>(), a1 = agpr_read4<(2 * v + 1) * 4>();
+      const uint4v w = {pack16(a0[0], a0[1]), pack16(a0[2], a0[3]), pack16(a1[0], a1[1]), pack16(a1[2], a1[3])};
+      st_coherent16(r, off, (uint32_t)v * NT * 16, w);
+    });
+  }
+  template <int V0, int V1>
+  static __device__ __forceinline__ void add_groups16(const float *src) {
+    const BufferRsrc r = make_rsrc(src, TILE_ELEMS * 2);
+    const uint32_t off = (uint32_t)pin_here((int)threadIdx.x) * 16;
+    constexpr int BATCH = 16;   // loads in flight per lane (see add_groups)
+    static_assert((V1 - V0) / 2 % BATCH == 0 && V0 % 2 == 0, "whole batches of pairs of groups");
+    static_for<0, (V1 - V0) / 2 / BATCH>([&](auto b) {
+      constexpr int base = V0 / 2 + decltype(b)::value * BATCH;
+      uint4v raw[BATCH];
+      static_for<0, BATCH>([&](auto i) {
+        constexpr int v = base + decltype(i)::value;
+        raw[decltype(i)::value] = ld_coherent16(r, off, (uint32_t)v * NT * 16);
+      });
+      static_for<0, BATCH>([&](auto i) {
+        constexpr int v = base + decltype(i)::value;
+        const uint4v w = raw[decltype(i)::value];
+        const floatx4 p0 = {widen16(w[0], 0), widen16(w[0], 1), widen16(w[1], 0), widen16(w[1], 1)};
+        const floatx4 p1 = {widen16(w[2], 0), widen16(w[2], 1), widen16(w[3], 0), widen16(w[3], 1)};
+        agpr_write4<(2 * v) * 4>(agpr_read4<(2 * v) * 4>() + p0);
+        agpr_write4<(2 * v + 1) * 4>(agpr_read4<(2 * v + 1) * 4>() + p1);
+      });
+    });
+  }
+  static __device__ __forceinline__ void store_partial_half16(const Acc &, float *dst, int h) {
+    if (h == 0) store_groups16<0, NV4 / 2>(dst);
+    else store_groups16<NV4 / 2, NV4>(dst);
+  }
+  static __device__ __forceinline__ void add_partial_half16(Acc &, const float *src, int h) {
+    if (h == 0) add_groups16<0, NV4 / 2>(src);
+    else add_groups16<NV4 / 2, NV4>(src);
+  }
   static __device__ __forceinline__ void store_partial(const Acc &, float *dst) { store_groups<0, NV4>(dst); }
   static __device__ __forceinline__ void add_partial(Acc &, const float *src) { add_groups<0, NV4>(src); }
   static __device__ __forceinline__ void store_partial_half(const Acc &, float *dst, int h) {

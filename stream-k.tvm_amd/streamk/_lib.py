@@ -11,7 +11,7 @@ LIB_PATH = os.path.join(_HERE, "libstreamk.so")
 SK_F16, SK_F32, SK_Q4, SK_BF16, SK_Q4_TILED, SK_F8E4M3, SK_I8, SK_Q4_ZP, SK_F8E5M2, SK_Q4_ZP_TILED = 0, 1, 2, 3, 4, 5, 6, 7, 8, 9
 LAYOUT_NT, LAYOUT_NN = 0, 1
 SCHEDULES = {"auto": 0, "dp": 1, "sk2": 2, "sk1": 3, "basic": 4, "splitk": 5}
-FIXUPS = {"auto": 0, "atomic": 1, "reduce": 2, "atomic_c": 3}
+FIXUPS = {"auto": 0, "atomic": 1, "reduce": 2, "atomic_c": 3, "reduce16": 4}
 
 
 class SkConfig(ctypes.Structure):

@@ -54,10 +54,11 @@ def save_cache(cache, path=None):
         json.dump(cache, f, indent=1, sort_keys=True)
 
 
-def candidate_configs(M, N, K, dtype="float16", cus=None):
+def candidate_configs(M, N, K, dtype="float16", cus=None, reduce16=True):
     """The search space.  The reference multiplies out warp/chunk/stage lists
     (autotune/streamk_fp16_autotune.py:38-53); here the axes are tile shape, kernel variant,
-    schedule, grid and fix-up."""
+    schedule, grid and fix-up.  reduce16=False leaves out the candidates that exchange partial sums rounded to 16
+    bits (fixup 'reduce16': within the 1e-2 every candidate is held to, but not the fp32 sums of the other fix-ups)."""
     cus = cus or _plan.num_cus()
     out = []
     f8 = dtype in ("float8_e4m3", "float8_e5m2", "int8")  # one-byte operands
@@ -117,6 +118,10 @@ def candidate_configs(M, N, K, dtype="float16", cus=None):
                 if -(-M // bm) * -(-N // bn) < cus:
                     out.extend(dict(base, schedule="splitk", fixup=fixup) for fixup in ("reduce", "atomic"))
                     out.append(dict(base, schedule="splitk", split=2, fixup="reduce"))
+                    # the exchange of half tiles with the partial sums rounded to 16 bits (assembly-loop kernel)
+                    if variant == 8 and reduce16:
+                        out.append(dict(base, schedule="splitk", fixup="reduce16"))
+                        out.append(dict(base, schedule="splitk", split=2, fixup="reduce16"))
     if dtype in ("float8_e4m3", "float8_e5m2", "int8"):
         # (bk 0: the tile's default, two stages of 128 K-values; 64: four stages of 64)
         tiles = [(256, 256, 0), (256, 128, 0), (128, 256, 0), (128, 128, 0), (64, 128, 0), (128, 128, 64), (64, 128, 64)]
@@ -169,7 +174,7 @@ def _time_ms(fn, warmup, rep, graph, min_ms=None):
 
 
 def autotune(M, N, K, dtype="float16", layout="nt", *, configs=None, warmup=5, rep=20, check=True,
-             cache=True, cache_path=None, verbose=False, weights=None):
+             cache=True, cache_path=None, verbose=False, weights=None, reduce16=True):
     """Searches `configs` (default: candidate_configs) for the fastest plan.
 
     weights="hbm" times every candidate on a rotation of copies of the weight operand (more than
@@ -180,7 +185,7 @@ def autotune(M, N, K, dtype="float16", layout="nt", *, configs=None, warmup=5, r
     Returns (best_latency_ms, best_config, ref_latency_ms); ref is torch.matmul on the same GPU, the
     reference's comparator (streamk_fp16.py:396) -- None for Q4.  Every candidate is checked against
     the first valid one (max-abs-rel 1e-2) unless check=False, mirroring `skip_check` of the
-    reference's jit decorator."""
+    reference's jit decorator.  reduce16=False keeps the candidates with 16-bit partial sums out of the search."""
     dev = "cuda"
     g = torch.Generator(device="cpu").manual_seed(0)
     A = (torch.rand(M, K, generator=g) * 2 - 1).half().to(dev)
@@ -237,7 +242,7 @@ def autotune(M, N, K, dtype="float16", layout="nt", *, configs=None, warmup=5, r
         as_b = (lambda b: b.T) if layout == "nt" else (lambda b: b)
         ref_ms = _time_ms(lambda: torch.matmul(A, as_b(rotate(Bs)), out=C), warmup, rep, small)
     small = 2.0 * M * N * K < 5e11  # microsecond kernels: time graph-captured batches
-    configs = configs if configs is not None else candidate_configs(M, N, K, dtype)
+    configs = configs if configs is not None else candidate_configs(M, N, K, dtype, reduce16=reduce16)
     best, golden, results = None, None, []
     for cfg in configs:
         try:

@@ -24,7 +24,7 @@ def num_cus():
 
 def make_config(config=None, **kw):
     """dict / kwargs -> SkConfig.  Keys: bm, bn, bk, grid, schedule ('auto'|'dp'|'sk2'|'sk1'|
-    'basic'|'splitk'), split, fixup ('auto'|'atomic'|'reduce'|'atomic_c'), raster, spin_limit, variant, interleave."""
+    'basic'|'splitk'), split, fixup ('auto'|'atomic'|'reduce'|'atomic_c'|'reduce16'), raster, spin_limit, variant, interleave."""
     d = dict(config or {})
     d.update(kw)
     c = SkConfig()

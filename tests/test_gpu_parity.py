@@ -470,6 +470,55 @@ def test_fixed_split_k(sk, oracle):
     sk.workspace_status()
 
 
+def test_reduce_fixup_with_16_bit_partials(sk, oracle):
+    """SK_FIXUP_REDUCE16: the halves of a split tile travel rounded to C's 16-bit type and are added in fp32 by the CTA
+    that finishes them.  Tiles cut in two and in four, fp16 and bfloat16, ragged shapes: within 2e-3 (bfloat16: 8e-3)
+    of the fp32 host product, the same bits on every launch, exact on small-integer data (every partial sum is
+    representable in 16 bits), equal to the fp32 REDUCE wherever no partial sum needs rounding; refused for any plan
+    that is not an equal split in two or four on the 256 x 256 assembly-loop kernel."""
+    import torch
+    g = torch.Generator(device="cpu").manual_seed(7)
+    for (M, N, K, split) in [(1024, 8192, 8192, 2), (512, 8192, 8192, 4), (256, 512, 1024, 2), (200, 500, 2048, 4), (300, 1000, 512, 2)]:
+        for name, dt, fn, tol in (("float16", torch.float16, sk.streamk_fp16, 2e-3), ("bfloat16", torch.bfloat16, sk.streamk_bf16, 8e-3)):
+            A = (torch.rand(M, K, generator=g) * 2 - 1).to(dt)
+            B = (torch.rand(N, K, generator=g) * 2 - 1).to(dt)
+            Ai = torch.randint(-1, 2, (M, K), generator=g).to(dt)
+            Bi = torch.randint(-1, 2, (N, K), generator=g).to(dt)
+            Ai[:, 150:] = 0   # |sums| <= 150: exact in fp16 and in bfloat16's eight bits
+            ref = oracle.matmul_fp32(A.float().numpy(), B.float().numpy(), trans_b=True)
+            exact = (Ai.double() @ Bi.double().T).numpy()
+            cfg = dict(bm=256, bn=256, bk=64, variant=8, schedule="splitk", split=split)
+            p16 = sk.make_plan(M, N, K, name, "nt", dict(cfg, fixup="reduce16"))
+            p32 = sk.make_plan(M, N, K, name, "nt", dict(cfg, fixup="reduce"))
+            assert p16.workspace_bytes == p32.workspace_bytes and p16.grid == p32.grid
+            C = fn(A.cuda(), B.cuda(), plan=p16)
+            assert _rel(oracle, C, ref) <= tol <= TOL, (M, N, K, split, name)
+            assert torch.equal(C, fn(A.cuda(), B.cuda(), plan=p16)), (M, N, K, split, name)
+            Ci = fn(Ai.cuda(), Bi.cuda(), plan=p16)
+            assert np.array_equal(Ci.double().cpu().numpy(), exact), (M, N, K, split, name)
+            assert torch.equal(Ci, fn(Ai.cuda(), Bi.cuda(), plan=p32)), (M, N, K, split, name)
+    # `basic` / `sk2` with two CTAs per tile are the same equal split; with bias and activation
+    M, N, K = 512, 1024, 4096
+    Ai = torch.randint(-1, 2, (M, K), generator=g).half()
+    Bi = torch.randint(-1, 2, (N, K), generator=g).half()
+    Ai[:, 150:] = 0
+    bias = torch.randint(-3, 4, (N,), generator=g).half()
+    want = np.maximum((Ai.double() @ Bi.double().T).numpy() + bias.double().numpy(), 0)
+    for sch in (dict(schedule="basic", grid=16), dict(schedule="sk2", grid=16), dict(schedule="basic", grid=32)):
+        C = sk.streamk_fp16(Ai.cuda(), Bi.cuda(), bias=bias.cuda(), activation="relu", bm=256, bn=256, bk=64, variant=8,
+                            fixup="reduce16", **sch)
+        assert np.array_equal(C.double().cpu().numpy(), want), sch
+    for cfg in (dict(bm=128, bn=128, bk=64, schedule="splitk", split=2), dict(bm=256, bn=256, bk=64, variant=5, schedule="splitk", split=2),
+                dict(bm=256, bn=256, bk=64, variant=8, schedule="dp"), dict(bm=256, bn=256, bk=64, variant=8, schedule="basic", grid=24),
+                dict(bm=256, bn=256, bk=64, variant=8, schedule="splitk", split=8)):
+        with pytest.raises(sk.StreamKError):
+            sk.make_plan(M, N, K, "float16", "nt", dict(cfg, fixup="reduce16"))
+    with pytest.raises(sk.StreamKError):
+        sk.make_plan(M, N, K, "int8", "nt", dict(bm=256, bn=256, schedule="splitk", split=2, fixup="reduce16"))
+    sk.workspace_status()
+
+
+@pytest.mark.gpu
 def test_reduce_fixup_is_bitwise_reproducible(sk):
     """The ordered reduce must give identical bits run to run (10 runs, two shapes); the schedule
     splits every tile."""
