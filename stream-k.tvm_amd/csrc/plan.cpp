@@ -115,7 +115,10 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
     // (more than 32 rows: 64 weight rows where they give three fifths of the CUs a tile -- A is then as many bytes
     // per CTA as the weights instead of twice as many; 64 x 16384 x 8192: 49 us against 56 us)
     const bool narrow = M > 32 ? cdiv(N, 64) * 5 < (int64_t)num_cus * 3 : cdiv(N, 32) <= num_cus;
-    const int bm = M <= 16 ? 16 : (M <= 32 ? 32 : 64), bn = narrow ? 32 : 64, bk = (bm == 16 && narrow) ? 512 : 256;
+    int bm = M <= 16 ? 16 : (M <= 32 ? 32 : 64), bn = narrow ? 32 : 64, bk = (bm == 16 && narrow) ? 512 : 256;
+    // (up to 16 rows and no more than a tile of 16 weight rows per CU: K split over all four waves -- N = 4096 then
+    // has a tile per CU; 16 x 4096 x 11008: 18.6 us against 21.4 us on 32-row tiles with a fix-up)
+    if (bm == 16 && cdiv(N, 16) <= num_cus) bn = 16, bk = 1024;
     for (int i = 0; i < n; ++i)
       if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].variant == 4 && t[i].bm == bm && t[i].bn == bn &&
           t[i].bk == bk && accepts_shape(t[i], M, K))
@@ -433,11 +436,12 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
   int sched = cfg ? cfg->schedule : SK_SCHED_AUTO;
   if (!(cfg && cfg->grid > 0)) {
     const int64_t iters = total64 * out->iters_per_tile;
-    // (the kernels that stream the weights through LDS are bound by memory: with tiles for three fifths of the CUs
-    // they run data-parallel rather than pay a fix-up -- Q4 16 x 11008 x 4096: 11.5 us against 14.3 us)
+    // (the kernels that stream the weights through LDS are bound by memory: with tiles for three fifths of the CUs --
+    // fp16 / bfloat16: two fifths -- they run data-parallel rather than pay a fix-up; Q4 16 x 11008 x 4096: 11.5 us
+    // against 14.3 us, fp16 16 x 2048 x 8192 on 128 tiles: 11.5 against 14.1)
     const bool stream_dp = k->family == FAMILY_SKINNY && (k->variant == 4 || k->dtype == SK_Q4) && k->max_m >= 16 &&
                            (k->bm == 16 || (k->variant == 4 && k->bm == 64 && k->bn == 64)) &&
-                           total64 * 5 >= (int64_t)num_cus * 3;
+                           total64 * 5 >= (int64_t)num_cus * (k->variant == 4 && k->dtype != SK_Q4 ? 2 : 3);
     if ((total64 >= num_cus || stream_dp) && total64 <= max_grid) {
       grid = (int)total64;  // one tile per CTA, all resident: a single data-parallel wave
     } else if (total64 < num_cus) {

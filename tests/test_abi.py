@@ -197,6 +197,8 @@ def test_untuned_plans_keep_cta_ranges_aligned(sk):
                                          (16, 16384, 8192, "float16", "stream_f16_mb1_wm1_wn4_rk1_d4", 256),
                                          (16, 28672, 8192, "float16", "stream_f16_mb1_wm1_wn4_rk1_d4", 256),
                                          (16, 11008, 4096, "float16", "stream_f16_mb1_wm1_wn4_rk1_d4", 172),
+                                         (16, 4096, 11008, "float16", "stream_f16_mb1_nb1_wm1_wn1_rk4_d3", 256),
+                                         (8, 2048, 8192, "bfloat16", "stream_bf16_mb1_nb1_wm1_wn1_rk4_d3", 128),
                                          (32, 8192, 8192, "float16", "stream_f16_mb1_wm2_wn2_rk1_d4", 256),
                                          (64, 8192, 8192, "float16", "stream_f16_mb2_wm2_wn2_rk1_d3", 256),
                                          (64, 16384, 8192, "float16", "stream_f16_mb2_nb2_wm2_wn2_rk1_d3", 256),

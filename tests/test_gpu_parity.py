@@ -70,6 +70,7 @@ SKINNY_CONFIGS = [
 STREAM_CONFIGS = [
     dict(bm=16, bn=64, bk=256, variant=5), dict(bm=32, bn=64, bk=256, variant=5), dict(bm=16, bn=32, bk=512, variant=5),
     dict(bm=64, bn=32, bk=256, variant=5), dict(bm=32, bn=32, bk=256, variant=5), dict(bm=64, bn=64, bk=256, variant=5),
+    dict(bm=16, bn=16, bk=1024, variant=5),
 ]
 
 
@@ -1100,14 +1101,15 @@ def test_f16_few_rows_in_the_matrix_vector_form(sk, oracle):
 
 
 def test_f16_weights_streamed_through_lds(sk, oracle):
-    """Up to 64 rows of A on the kernels that stream the weights through LDS in contiguous loads (six tile
+    """Up to 64 rows of A on the kernels that stream the weights through LDS in contiguous loads (seven tile
     shapes, fp16 and bfloat16): ragged M and N, K a multiple of 8 only and shorter than one iteration, strided A
     and W, all schedules and both fix-ups, bias and activation, an output with a row stride; exact on integer data
     (every tile adds its K-iterations up from a different start), within 2e-3 of the fp32 host product otherwise."""
     import torch
     rng = np.random.default_rng(74)
     ran = 0
-    shapes = {16: (16, 64, 256), 32: (32, 64, 256), 17: (16, 32, 512), 64: (64, 32, 256), 33: (32, 32, 256), 65: (64, 64, 256)}
+    shapes = {16: (16, 64, 256), 32: (32, 64, 256), 17: (16, 32, 512), 64: (64, 32, 256), 33: (32, 32, 256), 65: (64, 64, 256),
+              18: (16, 16, 1024)}
     for (M, N, K, pad) in [(16, 1000, 1160, 0), (9, 520, 392, 8), (1, 72, 8, 0), (13, 2048, 8192, 64), (5, 264, 28672, 0),
                            (64, 4099, 4104, 0), (50, 328, 776, 8), (32, 200, 1032, 0), (27, 8192, 4096, 0)]:
         A = (rng.random((M, K + pad), dtype=np.float32) * 2 - 1).astype(np.float16)
@@ -1305,7 +1307,7 @@ def test_bf16_small_m_kernels(sk, oracle):
         # (one row: matrix-vector kernels; two to four rows: their form with four rows of A; else the general kernels
         # or the ones that stream the weights through LDS)
         assert (241 <= plan.kernel_id <= 248) if M == 1 else ((210 <= plan.kernel_id <= 211) if M <= 4 else
-                                                               (230 <= plan.kernel_id <= 240 or plan.kernel_id in (282, 283, 285, 287, 289, 293))), (M, plan.kernel_id)
+                                                               (230 <= plan.kernel_id <= 240 or plan.kernel_id in (282, 283, 285, 287, 289, 293, 297))), (M, plan.kernel_id)
         A, W = (torch.rand(M, 4096) * 2 - 1).bfloat16(), (torch.rand(4096, 4096) * 2 - 1).bfloat16()
         ref = oracle.matmul_fp32(A.float().numpy(), W.float().numpy(), trans_b=True)
         assert _rel(oracle, sk.streamk_bf16(A.cuda(), W.cuda()), ref) <= 4e-3, M
