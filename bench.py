@@ -13,7 +13,8 @@ carries
   config.metric_parts   the other two parts of the metric in short: Stream-K against the data-parallel schedule at
                 M = 256 / 512 / 1024 (same tile, and the best data-parallel tile), Q4 GEMM at M = 1 / 16 as a
                 fraction of HBM peak with the weights in the Infinity Cache and from HBM, fp16 with 16 / 64 rows of A
-                with the weights from HBM next to the vendor GEMM,
+                with the weights from HBM next to the vendor GEMM, and the 16 cells M = 1 / 16 / 64 / 256 over four
+                projection shapes (N, K) of a 7B / 70B decoder against `torch.matmul` in the same run,
   extra         the measurements behind them and the rest: M sweep at N = K = 8192, 1024x1024x8192 with all
                 fix-ups, the large dense shapes in both layouts and types, the reference's own run shapes
                 (kernels this short are timed as graph-captured batches).
@@ -766,6 +767,36 @@ def main():
         del wqs, wd
         extra["reference_run_shapes"] = ref_rows
 
+        # the small-M sweep of the metric's third configuration: M in {1, 16, 64, 256} over four (N, K) pairs, inputs
+        # normal(0, 0.02), the plan the library makes by itself (tuned cache included) next to the vendor GEMM; up to
+        # 64 rows with the launches rotating over copies of the weights (> 512 MB in all), so that they come from HBM
+        cells = []
+        for (n3, k3) in ((4096, 4096), (11008, 4096), (4096, 11008), (28672, 8192)):
+            g3 = torch.Generator(device="cpu").manual_seed(n3 + k3)
+            w0 = (torch.randn(n3, k3, generator=g3) * 0.02).half().cuda()
+            wc = [w0] + [w0.clone() for _ in range(int(512e6 / (n3 * k3 * 2)) + 1)]
+            for m3 in (1, 16, 64, 256):
+                a3 = (torch.randn(m3, k3, generator=g3) * 0.02).half().cuda()
+                c3 = torch.empty(m3, n3, dtype=torch.float16, device="cuda")
+                p3 = streamk.make_plan(m3, n3, k3, "float16", "nt")
+                ws3 = wc if m3 <= 64 else wc[:1]
+                turn = [0]
+
+                def ours3():
+                    turn[0] += 1
+                    streamk.streamk_fp16(a3, ws3[turn[0] % len(ws3)], out=c3, plan=p3)
+
+                def vendor3():
+                    turn[0] += 1
+                    torch.matmul(a3, ws3[turn[0] % len(ws3)].T, out=c3)
+                t_o, t_v = time_graph(ours3, launches=10), time_graph(vendor3, launches=10)
+                nbytes = 2.0 * (m3 * k3 + n3 * k3 + m3 * n3)
+                cells.append({"M": m3, "N": n3, "K": k3, "us": round(t_o * 1e3, 2), "torch_matmul_us": round(t_v * 1e3, 2),
+                              "ratio": round(t_o / t_v, 3), "gbs": round(nbytes / t_o / 1e6, 1),
+                              "kernel": streamk.kernel_name(p3.kernel_id)})
+            del wc, w0
+        extra["small_m_sweep"] = cells
+
         # bfloat16 at the headline shape, both layouts, against the vendor GEMM in interleaved rounds
         bf = []
         ab, bb = A.bfloat16(), B.bfloat16()
@@ -804,6 +835,10 @@ def main():
             parts["q4_gemm_N8192_K8192"][f"M{row['M']}"] = {
                 "us_weights_in_infinity_cache": row["tuned"]["us"], "frac_hbm_weights_in_infinity_cache": row["tuned"]["frac_hbm"],
                 "us_weights_from_hbm": row["tuned_weights_from_hbm"]["us"], "frac_hbm_weights_from_hbm": row["tuned_weights_from_hbm"]["frac_hbm"]}
+        parts["small_m_sweep_16_cells"] = {
+            "cells_at_or_below_torch_matmul": sum(1 for c in cells if c["ratio"] <= 1.0),
+            "geomean_time_over_torch_matmul": round(float(np.exp(np.mean([np.log(c["ratio"]) for c in cells]))), 3),
+            "worst": max(cells, key=lambda c: c["ratio"])}
         out["config"]["metric_parts"] = parts
         out["extra"] = extra
 
