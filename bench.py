@@ -764,7 +764,28 @@ def main():
                          "us": round(ms * 1e3, 1), "gbs": round(nbytes / ms / 1e6, 1),
                          "frac_hbm": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4),
                          "torch_matmul_on_fp16_weights_us": round(ms_t * 1e3, 1)})
-        del wqs, wd
+        del wd
+        # one row of A on the same weights and on 28672 x 8192: the Q4 matrix-vector kernels where the planner runs
+        # several 16-row tiles per CTA (the later tiles' first loads are requested while the tile before is summed)
+        q4_rows = []
+        for (n1, k1) in ((16384, 16384), (28672, 8192)):
+            a1 = torch.randn(1, k1, generator=g).half().cuda()
+            c1 = torch.empty(1, n1, dtype=torch.float16, device="cuda")
+            # (the 28672 x 8192 operands are views of the same random bytes and scales)
+            w1 = [(wq_.view(-1)[: n1 * k1 // 2].view(n1, k1 // 2), sc_.view(-1)[: n1 * (k1 // 128)].view(n1, k1 // 128))
+                  for (wq_, sc_) in wqs]
+            p1 = streamk.make_plan(1, n1, k1, "q4", "nt")
+
+            def q4_m1():
+                turn[0] += 1
+                w, s_ = w1[turn[0] % 4]
+                streamk.streamk_q4(a1, w, s_, out=c1, plan=p1)
+            nbytes = 2 * k1 + n1 * k1 // 2 + 2 * n1 * (k1 // 128) + 2 * n1
+            ms = time_graph(q4_m1, launches=8)
+            q4_rows.append({"shape": [1, n1, k1], "kernel": streamk.kernel_name(p1.kernel_id), "grid": p1.grid, "us": round(ms * 1e3, 1),
+                            "gbs": round(nbytes / ms / 1e6, 1), "frac_hbm": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)})
+        extra["q4_one_row_large_weights_from_hbm"] = q4_rows
+        del wqs, w1
         extra["reference_run_shapes"] = ref_rows
 
         # the small-M sweep of the metric's third configuration: M in {1, 16, 64, 256} over four (N, K) pairs, inputs

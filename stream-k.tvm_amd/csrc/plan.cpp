@@ -126,12 +126,21 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
   }
   if ((M <= (one_byte ? 64 : 32) && layout == SK_LAYOUT_NT) || q4) {
     // M == 1 with Q4 weights: the matrix-vector kernel with four waves splitting K (data-parallel
-    // over 16-row tiles), the fastest instance at LLM-sized N and K
-    if (q4 && M == 1 && want_variant < 0)
-      for (int i = 0; i < n; ++i)
-        if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].variant == 2 && t[i].bn == 16 &&
-            t[i].bk == 1024 && accepts_shape(t[i], M, K))
-          return &t[i];
+    // over 16-row tiles), the fastest instance at LLM-sized N and K.  Weights from HBM: from K = 14336 on eight waves
+    // (1 x 16384 x 16384: 25.9 us against 28.7 us, 1 x 4096 x 14336: 7.9 / 9.0; 1 x 4096 x 11008: 8.2 / 7.4).  With more
+    // 16-row tiles than CTAs of four waves stay resident (three per CU): K up to 6144 split over two waves, four
+    // CTAs per CU (1 x 14336 x 4096: 7.7 us in one round against 10.8 us in two; 1 x 32000 x 4096: 14.6 / 16.2,
+    // 1 x 65536 x 4096: 25.7 / 27.9), K from 8192 on over eight (1 x 28672 x 8192: 25.5 / 27.1).
+    if (q4 && M == 1 && want_variant < 0) {
+      int bk = 1024;
+      if (K >= 14336) bk = 2048;
+      else if (cdiv(N, 16) > (int64_t)num_cus * 3) bk = K <= 6144 ? 512 : (K >= 8192 ? 2048 : 1024);
+      for (int pass = 0; pass < 2; ++pass, bk = 1024)
+        for (int i = 0; i < n; ++i)
+          if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].variant == 2 && t[i].bn == 16 &&
+              t[i].bk == bk && accepts_shape(t[i], M, K))
+            return &t[i];
+    }
     // 2 <= M <= 16 with row-major Q4 weights (scalar zero point), weights from HBM.  Where 64-row tiles give three
     // fifths of the CUs a tile the general kernel with 64 weight rows and K split over two waves, data-parallel
     // (16 x 28672 x 8192: 32.8 us; the 32-row kernel below: 48.5; 16 x 11008 x 4096: 10.7 / 14.8; 16 x 16384 x 16384:
@@ -442,8 +451,14 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
     const bool stream_dp = k->family == FAMILY_SKINNY && (k->variant == 4 || k->dtype == SK_Q4) && k->max_m >= 16 &&
                            (k->bm == 16 || (k->variant == 4 && k->bm == 64 && k->bn == 64)) &&
                            total64 * 5 >= (int64_t)num_cus * (k->variant == 4 && k->dtype != SK_Q4 ? 2 : 3);
+    const bool q4_gemv = k->family == FAMILY_SKINNY && k->variant == 2 && k->max_m == 1 &&
+                         (k->dtype == SK_Q4 || k->dtype == SK_Q4_ZP || k->dtype == SK_Q4_TILED || k->dtype == SK_Q4_ZP_TILED);
     if ((total64 >= num_cus || stream_dp) && total64 <= max_grid) {
       grid = (int)total64;  // one tile per CTA, all resident: a single data-parallel wave
+    } else if (q4_gemv && total64 > max_grid) {
+      // more tiles than resident CTAs: as few CTAs as finish in the same number of rounds, so that every CTA walks
+      // (nearly) the same number of tiles -- a CTA's later tiles find their first loads in flight (mac_tiles)
+      grid = (int)cdiv(total64, cdiv(total64, max_grid));
     } else if (total64 < num_cus) {
       // fewer tiles than CUs: one CTA per CU, but a split tile keeps at least 4 K-iterations per CTA
       // and there are never fewer CTAs than tiles
@@ -478,6 +493,11 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
     // wave costs them less than the fix-up; 16 x 28672 x 8192: 77.8 us data-parallel against 83.6 us.  With 64 rows of
     // A on 64 x 32 tiles it is the other way round, 110 us against 103 us; on 64 x 64 tiles 91.5 against 92.6)
     if (k->family == FAMILY_SKINNY && k->variant == 4 && (k->bm == 16 || k->bn == 64) && total64 >= grid) sched = SK_SCHED_DP;
+    // (the same for the Q4 matrix-vector kernels: 1 x 28672 x 8192 on 1792 tiles 28.0 us data-parallel against 31.2 us,
+    // 1 x 14336 x 4096 with K split over four waves 10.8 against 16.1)
+    if (k->family == FAMILY_SKINNY && k->variant == 2 && k->max_m == 1 && total64 >= grid &&
+        (k->dtype == SK_Q4 || k->dtype == SK_Q4_ZP || k->dtype == SK_Q4_TILED || k->dtype == SK_Q4_ZP_TILED))
+      sched = SK_SCHED_DP;
     if (k->family == FAMILY_TILE && sched != SK_SCHED_DP) {
       // Fewer tiles than CUs: the idle CUs are put to work by an aligned split in two or four, never by CTA ranges
       // that start anywhere.  More tiles than CTAs: see

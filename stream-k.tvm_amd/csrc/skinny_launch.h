@@ -53,11 +53,22 @@ __device__ __forceinline__ void mac_of_tile(const typename P::Args &a, typename 
   P::mac(a, acc, 0, tile, 0, ipt, smem);
 }
 
+// policies with mac_tiles: the whole data-parallel loop of a CTA, stores included (a tile's first loads are requested
+// while the tile before is still being summed)
+template <class P, class = void>
+struct has_mac_tiles { static constexpr bool value = false; };
+template <class P>
+struct has_mac_tiles<P, std::void_t<decltype(&P::mac_tiles)>> { static constexpr bool value = true; };
+
 template <class P>
 __global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_skinny_dp_kernel(typename P::Args a, int total_tiles, int ipt) {
   __shared__ __attribute__((aligned(16))) char smem[P::LDS_BYTES];
-  typename P::Acc acc;
   const int tile0 = first_tile_of_block<P>();
+  if constexpr (has_mac_tiles<P>::value) {
+    P::mac_tiles(a, tile0, gridDim.x, total_tiles, ipt, smem, nullptr);
+    return;
+  }
+  typename P::Acc acc;
   for (int tile = tile0; tile < total_tiles; tile += gridDim.x) {
     mac_of_tile<P>(a, acc, tile, ipt, smem, tile == tile0);
     P::store_c(a, acc, 0, tile, smem, nullptr);
@@ -69,8 +80,12 @@ __global__ __launch_bounds__(P::NT, P::WAVES_PER_EU) void sk_skinny_dp_kernel_bi
   __shared__ __attribute__((aligned(16))) char smem[P::LDS_BYTES];
   const void *bias = bias_arg;
   asm volatile("" ::"s"(bias));  // fetched with the other arguments, not before the first store
-  typename P::Acc acc;
   const int tile0 = first_tile_of_block<P>();
+  if constexpr (has_mac_tiles<P>::value) {
+    P::mac_tiles(a, tile0, gridDim.x, total_tiles, ipt, smem, bias);
+    return;
+  }
+  typename P::Acc acc;
   for (int tile = tile0; tile < total_tiles; tile += gridDim.x) {
     mac_of_tile<P>(a, acc, tile, ipt, smem, tile == tile0);
     P::store_c(a, acc, 0, tile, smem, bias);

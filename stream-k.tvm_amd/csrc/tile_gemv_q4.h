@@ -85,18 +85,48 @@ struct TileGemvQ4 {
     float y[NB];
   };
 
+  // What one tile leaves in registers for the next tile of the same CTA: the weights of the next tile's first DEPTH
+  // iterations and the first pieces of its scales (and zero points), requested during the last round of the tile
+  // before, so that the memory round trip of a tile's start overlaps the end of the one before.
+  struct Carry {
+    uint4v wreg[DEPTH][NB][2];
+    ScaleStager<BN, SC_ROW, NT> scales, zero_points;
+  };
+
   static __device__ __forceinline__ void mac(const Args &a, Acc &acc, int pm, int pn, int k0, int n, char *smem) {
-    mac_impl<false>(a, acc, pm, pn, k0, n, smem);
+    Carry cy;
+    mac_impl<false, false, false>(a, acc, pm, pn, k0, n, smem, cy, -1);
   }
   // The same for a CTA whose previous call had the same k0 and n (the tiles of a data-parallel launch that a CTA
   // takes one after the other): the row of A and its correction sums are in LDS already and are neither loaded
   // nor staged again -- a fifth of a tile's time at K = 8192.
   static __device__ __forceinline__ void mac_again(const Args &a, Acc &acc, int pm, int pn, int k0, int n, char *smem) {
-    mac_impl<true>(a, acc, pm, pn, k0, n, smem);
+    Carry cy;
+    mac_impl<true, false, false>(a, acc, pm, pn, k0, n, smem, cy, -1);
   }
-  template <bool A_RESIDENT>
+  // All tiles of a CTA in a data-parallel launch (tile0, tile0 + stride, ... below total), K from 0 over ipt
+  // iterations each, C stored as store_c does: every tile but the first finds its first loads in flight.
+  static __device__ __forceinline__ void mac_tiles(const Args &a, int tile0, int stride, int total, int ipt, char *smem,
+                                                   const void *bias) {
+    if (tile0 >= total) return;
+    Carry cy;
+    Acc acc;
+    int next = tile0 + stride < total ? tile0 + stride : -1;
+    mac_impl<false, false, true>(a, acc, 0, tile0, 0, ipt, smem, cy, next);
+    store_c(a, acc, 0, tile0, smem, bias);
+    while (next >= 0) {
+      const int tile = next;
+      next = tile + stride < total ? tile + stride : -1;
+      mac_impl<true, true, true>(a, acc, 0, tile, 0, ipt, smem, cy, next);
+      store_c(a, acc, 0, tile, smem, bias);
+    }
+  }
+  // PRELOADED: cy holds this tile's first DEPTH iterations of weights and the first pieces of its scales (the
+  // previous call was given this tile as next_pn, same k0 and n).  CHAIN with next_pn >= 0: the last round requests
+  // those of tile next_pn instead of reading past the segment.
+  template <bool A_RESIDENT, bool PRELOADED, bool CHAIN>
   static __device__ __forceinline__ void mac_impl(const Args &a, Acc &acc, int /*pm*/, int pn, int k0, int n,
-                                                  char *smem) {
+                                                  char *smem, Carry &cy, int next_pn) {
     char *ldsA = smem;
     float *ldsCorr = reinterpret_cast<float *>(smem + LDS_A);
     half_t *ldsS = reinterpret_cast<half_t *>(smem + LDS_A + LDS_CORR);
@@ -122,10 +152,17 @@ struct TileGemvQ4 {
     for (int j = 0; j < NB; ++j)
       voff_w[j] = TILED_ ? (uint32_t)(wn * NB + j) * block_bytes + (uint32_t)lane * 16
                          : (uint32_t)((wn * NB + j) * 16 + row) * ldw + (uint32_t)(klane / 2);
-    uint4v wreg[DEPTH][NB][2];
+    auto &wreg = cy.wreg;
+    // the next tile's rows (an empty range without one: its loads return zeros without touching memory)
+    const int rows_next = next_pn >= 0 ? min(BN, a.N - next_pn * BN) : 0;
+    const char *base_cur = reinterpret_cast<const char *>(a.W) + (int64_t)pn * (TILED_ ? (BN / 16) * block_bytes : BN * ldw);
+    const char *base_next =
+        reinterpret_cast<const char *>(a.W) + (int64_t)max(next_pn, 0) * (TILED_ ? (BN / 16) * block_bytes : BN * ldw);
+    const uint32_t bytes_cur = TILED_ ? (uint32_t)((rows_w + 15) / 16) * block_bytes : rows_w * ldw;
+    const uint32_t bytes_next = TILED_ ? (uint32_t)((rows_next + 15) / 16) * block_bytes : rows_next * ldw;
     // loads of iterations past the segment or past K get an out-of-range offset: they return
     // zeros without touching memory, and every round of the main loop has the same loads in flight
-    auto issue_loads = [&](int slot, int rel_it) {
+    auto issue_from = [&](const BufferRsrc &rsrc, int slot, int rel_it) {
       const int kbase = (k0 + rel_it) * BKC;
       const int klimit = rel_it < n ? a.K - kbase : 0;
 #pragma unroll
@@ -133,11 +170,12 @@ struct TileGemvQ4 {
 #pragma unroll
         for (int c = 0; c < 2; ++c)
           wreg[slot][j][c] =
-              TILED_ ? buffer_load_16(rsrc_w, rk * BK + c * 128 < klimit ? voff_w[j] : OOB_OFFSET,
+              TILED_ ? buffer_load_16(rsrc, rk * BK + c * 128 < klimit ? voff_w[j] : OOB_OFFSET,
                                       (uint32_t)((kbase + rk * BK) / QGROUP + c) * 1024)
-                     : buffer_load_16(rsrc_w, klane + c * 128 < klimit ? voff_w[j] : OOB_OFFSET,
+                     : buffer_load_16(rsrc, klane + c * 128 < klimit ? voff_w[j] : OOB_OFFSET,
                                       (uint32_t)(kbase / 2) + c * 64);
     };
+    auto issue_loads = [&](int slot, int rel_it) { issue_from(rsrc_w, slot, rel_it); };
 
     // ---- all global loads of the prologue go out back to back, in the order they are consumed:
     // A (first two rounds of the CTA), the first round of scale pieces, then DEPTH iterations of
@@ -163,15 +201,16 @@ struct TileGemvQ4 {
     // 8-aligned group below and ldsS[r][sc_shift + i] is group k0*SC_PER_ITER + i
     const int g_first = k0 * SC_PER_ITER, g0 = g_first & ~7;
     const int sc_shift = g_first - g0;
-    ScaleStager<BN, SC_ROW, NT> scales;
-    scales.begin(ldsS, a.scales + (int64_t)pn * BN * a.groups, rows_w, a.groups, g0,
-                 (sc_shift + n * SC_PER_ITER + 7) >> 3);
-    ScaleStager<BN, SC_ROW, NT> zero_points;
-    if constexpr (ZP_)
-      zero_points.begin(ldsS + BN * SC_ROW, a.zeros + (int64_t)pn * BN * a.groups, rows_w, a.groups, g0,
-                        (sc_shift + n * SC_PER_ITER + 7) >> 3);
+    auto &scales = cy.scales;
+    auto &zero_points = cy.zero_points;
+    const int sc_chunks = (sc_shift + n * SC_PER_ITER + 7) >> 3;
+    if constexpr (!PRELOADED) {
+      scales.begin(ldsS, a.scales + (int64_t)pn * BN * a.groups, rows_w, a.groups, g0, sc_chunks);
+      if constexpr (ZP_)
+        zero_points.begin(ldsS + BN * SC_ROW, a.zeros + (int64_t)pn * BN * a.groups, rows_w, a.groups, g0, sc_chunks);
 #pragma unroll
-    for (int d = 0; d < DEPTH; ++d) issue_loads(d, d);
+      for (int d = 0; d < DEPTH; ++d) issue_loads(d, d);
+    }
     // nothing of what follows is to be scheduled ahead of these loads
     __builtin_amdgcn_sched_barrier(0);
 
@@ -235,6 +274,17 @@ struct TileGemvQ4 {
 
     // ---- main loop: rounds of DEPTH iterations without an exit inside a round ----
     for (int it0 = 0; it0 < n; it0 += DEPTH) {
+      // the last round asks for the next tile's start instead of iterations past the segment: its scales first,
+      // then slot by slot the weights of its iterations 0 .. DEPTH-1
+      const bool last_round = CHAIN && it0 + DEPTH >= n;
+      // (one descriptor per round, chosen with scalar selects: the loop body has a single path)
+      const BufferRsrc rsrc_it = CHAIN ? make_rsrc(last_round ? base_next : base_cur, last_round ? bytes_next : bytes_cur) : rsrc_w;
+      if (last_round && next_pn >= 0) {
+        scales.begin(ldsS, a.scales + (int64_t)next_pn * BN * a.groups, rows_next, a.groups, g0, sc_chunks);
+        if constexpr (ZP_)
+          zero_points.begin(ldsS + BN * SC_ROW, a.zeros + (int64_t)next_pn * BN * a.groups, rows_next, a.groups, g0,
+                            sc_chunks);
+      }
 #pragma unroll
       for (int d = 0; d < DEPTH; ++d) {
         const int it = it0 + d;
@@ -290,7 +340,7 @@ struct TileGemvQ4 {
             acc.y[j] = __builtin_fmaf(sum32, (float)s2[c] * live, acc.y[j]);
           }
         }
-        issue_loads(d, it + DEPTH);
+        issue_from(rsrc_it, d, last_round ? d : it + DEPTH);
       }
     }
 

@@ -949,6 +949,58 @@ def test_q4_matrix_vector_exact_on_integer_data(sk):
     sk.workspace_status()
 
 
+def test_q4_matrix_vector_tiles_chained_in_one_cta(sk, oracle):
+    """Data-parallel launches of the Q4 matrix-vector kernels with fewer CTAs than tiles: a CTA requests the first
+    loads and scales of its next tile during the last round of the tile before.  Whatever the grid, every element
+    of C must equal, bit for bit, what the launch with one tile per CTA gives -- on a ragged N (last tile partial),
+    K with a tail iteration, K shorter than the prefetch depth, with a bias, with per-group zero points and with
+    tiled weights -- and the oracle's product."""
+    import torch
+    rng = np.random.default_rng(73)
+    ran = 0
+    for (N, K) in [(1000, 1152), (264, 28672), (2056, 4096), (520, 384), (4096, 8192)]:
+        A = (rng.random((1, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+        Wq = rng.integers(0, 256, (N, K // 2), dtype=np.uint8)
+        sc = rng.uniform(0.005, 0.02, (N, K // 128)).astype(np.float16)
+        zp = rng.integers(0, 16, (N, K // 128)).astype(np.float16)
+        bias = (rng.random(N, dtype=np.float32) * 2 - 1).astype(np.float16)
+        dA, dW, dS, dZ, dB = _t(A), _t(Wq), _t(sc), _t(zp), _t(bias)
+        dT = sk.tile_q4(dW)
+        ref = oracle.q4_gemm_ref(A, Wq, sc, 128, 8)
+        refz = oracle.q4_zp_gemm_ref(A, Wq, sc, zp)
+        for (bm, bn, bk) in Q4_TILES + [(16, 16, 2048)]:
+            for name, kw in (("q4", dict()), ("q4_zp", dict(zeros=dZ)), ("q4_tiled", dict(tiled=True)),
+                             ("q4_zp_tiled", dict(zeros=dZ, tiled=True))):
+                cfg = dict(bm=bm, bn=bn, bk=bk, variant=3, schedule="dp")
+                try:
+                    one = sk.make_plan(1, N, K, name, "nt", cfg)
+                except sk.StreamKError:
+                    continue  # no such instance for this format, or K beyond what it stages
+                if not sk.kernel_name(one.kernel_id).startswith("gemv_q4"):
+                    continue
+                w = dT if "tiled" in name else dW
+                want = sk.streamk_q4(dA, w, dS, plan=one, **kw)
+                assert _rel(oracle, want, refz if "zp" in name else ref) <= 2e-3, (N, K, name, cfg)
+                want_b = sk.streamk_q4(dA, w, dS, plan=one, bias=dB, **kw)
+                for grid in (1, 3, 7, 64):
+                    if grid >= one.grid:
+                        continue
+                    plan = sk.make_plan(1, N, K, name, "nt", dict(cfg, grid=grid))
+                    assert plan.grid == grid and plan.kernel_id == one.kernel_id
+                    C = torch.full_like(want, float("nan"))
+                    sk.streamk_q4(dA, w, dS, out=C, plan=plan, **kw)
+                    assert torch.equal(C, want), (N, K, name, cfg, grid)
+                    assert torch.equal(sk.streamk_q4(dA, w, dS, plan=plan, bias=dB, **kw), want_b), (N, K, name, cfg, grid, "bias")
+                    ran += 1
+    assert ran >= 150, ran
+    # the planner's own choice for more 16-row tiles than CTAs stay resident: every CTA walks the same number of tiles
+    plan = sk.make_plan(1, 28672, 8192, "q4", "nt", use_tuned=False)
+    assert sk.kernel_name(plan.kernel_id) == "gemv_q4_nb1_wn1_rk8_k16384" and plan.grid == 256
+    plan = sk.make_plan(1, 32000, 4096, "q4", "nt", use_tuned=False)
+    assert sk.kernel_name(plan.kernel_id) == "gemv_q4_nb1_wn1_rk2_k16384" and plan.grid == 1000
+    sk.workspace_status()
+
+
 def test_q4_matrix_vector_deviation_from_rounded_weights_is_bounded(sk, oracle):
     """The M = 1 matrix-vector kernels multiply the unrounded (q - zero) * scale instead of the fp16-rounded
     weights the other kernels (and sk_dequant_q4) form.  Per output that moves the result by at most
