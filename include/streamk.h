@@ -311,10 +311,12 @@ int sk_gemm_f32(const void *A, const void *B, void *C, int64_t M, int64_t N, int
  * Replaces tl_mod(A, QLB, C) of streamk_fp16_ladder_block_reduce_q4.py:597-599; the weights stay in
  * the natural byte order above (no LadderPermutate / LOP3Permutate step, :568-595).
  * Requirements: K multiple of 128, group == 128, 0 <= zero <= 15.
- * For M == 1 the matrix-vector kernels multiply the nibbles undecoded and apply zero point and
- * scale to fp32 group sums, i.e. they use the unrounded (q - zero) * scale: at least as close to
- * the exact product as the rounded-weight form (within 2^-11 relative per weight of it).
- * sk_dequant_q4 and the M > 1 kernels produce the rounded weights bit for bit.
+ * Up to 16 rows of A (the matrix-vector kernels for M == 1; the 16-row kernels with a scalar zero point)
+ * the nibbles are multiplied undecoded and zero point and scale are applied to fp32 group sums, i.e.
+ * these kernels use the unrounded (q - zero) * scale: at least as close to the exact product as the
+ * rounded-weight form (within 2^-11 relative per weight of it).
+ * sk_dequant_q4, the kernels for more than 16 rows and the per-group zero-point kernels for M > 1
+ * produce the rounded weights bit for bit.
  * Up to 64 rows of A the plan is a weight-streaming kernel; for more rows (plan dtype SK_Q4) it is a tile kernel
  * that moves the nibbles through LDS and dequantises them, bit for bit as above, on their way into the fp16
  * stage of the 16x16x32 MFMA loop (256x256, 256x128 or 128x128 tiles; every schedule and fix-up).

@@ -127,6 +127,14 @@ struct TileSkinny {
   static constexpr bool LEAN_ENTRY = false;  // see run_persistent
   static constexpr int MB = MB_, NB = NB_, WN = WN_, RK = RK_, DEPTH = DEPTH_;
   static constexpr bool Q4 = Q4_;
+  // Up to 16 rows of A with a scalar zero point: the nibbles go into the MFMA undecoded (1024 + q from bits 0..3
+  // of a half, 64 + q from bits 4..7: one shift and four v_and_or_b32 per word), the sum over each 128-wide scale
+  // group starts from -sum a_k (offset_k + zero) -- four MFMAs per group on a constant fragment, shared by the
+  // wave's row blocks -- and the group's scale multiplies the fp32 group sum.  (q - zero) * scale is then never
+  // rounded to fp16: the result is at least as close to the exact product as the one from rounded weights, as in
+  // the matrix-vector kernels (tile_gemv_q4.h).  8 vector instructions per MFMA instead of 15.
+  // (not the instance of four waves along N without a K split, whose registers it does not fit)
+  static constexpr bool UNDECODED = Q4_ && !ZP_ && !ROW1_ && MB_ == 1 && F8_ == 0 && !(NB_ == 1 && WN_ == 4 && RK_ == 1);
   // the Q4 instances of one row block per wave without K split: their scalar-argument form spills (skinny_launch.h)
   static constexpr bool NO_FLAT_ARGS = Q4_ && NB_ == 1 && WN_ == 4 && RK_ == 1 && !ROW1_;
   static constexpr int BM = 16 * MB, BN = 16 * NB * WN;
@@ -261,6 +269,15 @@ struct TileSkinny {
     };
 
     const Q4Consts qc = q4_consts(a.zero);
+    // UNDECODED: the magic of the nibbles at bits 4..7 (fp16 64.0: 64 + q) and minus the offsets of a word's eight
+    // elements in the order the decode leaves them (0,4 | 1,5 | 2,6 | 3,7: bits 0..3, bits 4..7, 0..3, 4..7)
+    uint32_t magic_hi = 0x54005400u;
+    asm volatile("" : "+v"(magic_hi));
+    half8v neg_offsets;
+    {
+      const half_t lo = (half_t)(float)(-(1024 + a.zero)), hi = (half_t)(float)(-(64 + a.zero));
+      neg_offsets = half8v{lo, lo, hi, hi, lo, lo, hi, hi};
+    }
 
     // ---- prologue: DEPTH iterations of loads in flight ----
 #pragma unroll
@@ -308,6 +325,40 @@ struct TileSkinny {
             }
           }
         }
+        if constexpr (UNDECODED) {
+          // load c of the iteration is one scale group: chunks 4c .. 4c+3
+#pragma unroll
+          for (int c = 0; c < WLOADS; ++c) {
+            half8v fa4[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) fa4[q] = *reinterpret_cast<const half8v *>(abuf + a_rd[0] + c * 128 + q * 8);
+            floatx4 base = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int q = 0; q < 4; ++q) base = __builtin_amdgcn_mfma_f32_16x16x32_f16(neg_offsets, fa4[q], base, 0, 0, 0);
+#pragma unroll
+            for (int j = 0; j < NB; ++j) {
+              floatx4 p = base;
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                union {
+                  uint32_t u[4];
+                  half8v v;
+                } r;
+                const uint32_t w = wreg[d][j][c][q], t = w >> 8;
+                r.u[0] = and_or(w, qc.mask_lo, qc.magic);
+                r.u[1] = and_or(w, qc.mask_hi, magic_hi);
+                r.u[2] = and_or(t, qc.mask_lo, qc.magic);
+                r.u[3] = and_or(t, qc.mask_hi, magic_hi);
+                p = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.v, fa4[q], p, 0, 0, 0);
+              }
+              // result register r of the lane is weight row 4 * (lane / 16) + r of the block
+              const half_t *sp = ldsS + ((wn * NB + j) * 16 + lg * 4) * SC_ROW + sc_shift + min(it, n - 1) * SC_PER_ITER + rk * 2 + c;
+#pragma unroll
+              for (int r4 = 0; r4 < 4; ++r4)
+                acc.c[0][j][r4] = __builtin_fmaf(p[r4], (float)sp[r4 * SC_ROW], acc.c[0][j][r4]);
+            }
+          }
+        } else
 #pragma unroll
         for (int ch = 0; ch < NCH; ++ch) {
           half8v fa[MB];

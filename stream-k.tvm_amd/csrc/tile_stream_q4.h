@@ -4,8 +4,9 @@
 // The general small-M kernel (tile_skinny.h) loads 16 bytes of weight row l % 16 per lane: one load instruction
 // touches 16 rows, 64 bytes of each.  Here a load instruction reads four rows of 256 contiguous bytes (512 K-values)
 // directly into LDS, and lane (i, g) reads its 16 bytes of row i back out of LDS: the registers then hold what the
-// general kernel's loads deliver, and the decode (q4_dequant.h: bit-exact fp16((q - zero) * scale)) and the
-// 16x16x32 MFMAs are the same.
+// general kernel's loads deliver, and the arithmetic is that kernel's for up to 16 rows (tile_skinny.h, UNDECODED):
+// the nibbles enter the 16x16x32 MFMA as 1024 + q / 64 + q, every 128-wide scale group's sum starts from
+// -sum a_k (offset_k + zero) (four MFMAs on a constant fragment) and is multiplied by the group's scale in fp32.
 //
 //  * CTA = eight waves, two per SIMD: WN_ along N x RK_ along K rings of weights, KH_ waves per ring (four rings shared
 //    by two waves each, which take 256 of the 512 K-values of an iteration; or eight rings, 128 weight rows, one wave
@@ -17,16 +18,17 @@
 //  * No padding: lane l of a load fetches the 16-byte piece (l % 16) ^ (row % 16) of its row for position l % 16
 //    (A: piece l ^ row of the row's 64), so the sixteen lanes that read the same piece of sixteen rows find it on
 //    sixteen different bank groups.
-//  * A arrives in natural element order; the decode delivers the eight values of a word in the order 0,4,1,5,2,6,3,7,
-//    so each 16-byte fragment of A is put into that order with four byte permutes after it is read.
+//  * A arrives in natural element order; the extraction delivers the eight values of a word in the order
+//    0,4,1,5,2,6,3,7, so each 16-byte fragment of A is put into that order with four byte permutes after it is read.
 //  * Rings of WD_ slots for weights and scales (per wave), AD_ slots for A; loads are issued in the order
 //    A(t + AD_ - 1), W(t + WD_ - 1) and complete in that order, one wait and one barrier per iteration.
 //  * Tiles walk K from different offsets (rotation_of, sk_device.h).
 //
 // Where the time goes (16 x 16384 x 16384, 134 MB of weights, one 64-row tile per CU): A is as many bytes per CTA as
 // the weights (16 rows of fp16 against 64 rows of nibbles) and travels from the L2 into LDS beside them; with the
-// decode and the permutes taken out the kernel runs 24 us with the weights in the Infinity Cache and 32 us from
-// HBM, with them 35 / 38 us (155 vector instructions per wave and iteration for 8 MFMAs).
+// bit-exact decode it had first (fp16((q - zero) * scale) per weight, 155 vector instructions per wave and iteration
+// for 8 MFMAs) and the permutes taken out the kernel ran 24 us with the weights in the Infinity Cache and 32 us
+// from HBM, with them 35 / 41 us; with the nibbles undecoded 31.7 / 37.8 us.
 //
 // Epilogue, partial tiles and fix-ups are those of tile_stream_pairs.h (one block of 16 rows of A per wave).
 // Replaces the reference's decode-then-MMA step for its own run shape, 16 x 16384 x 16384
@@ -123,8 +125,14 @@ struct TileStreamQ4 : TileStreamPairs<1, 1, WN_, RK_, 3, false> {
 #pragma unroll
     for (int q = 0; q < 4; ++q)
       a_rd[q] = smem + LDS_W + LDS_S + rk * A_CHUNK + fi * 1024 + 256 * STEPS * kh + 16 * ((4 * fg + q) ^ fi);
-    const char *s_rd = smem + LDS_W + wave * (WD * S_SLOT) + fi * (2 * STEPS);
+    const char *s_rd4 = smem + LDS_W + wave * (WD * S_SLOT) + fg * (4 * 2 * STEPS);
     const Q4Consts qc = q4_consts(a.zero);
+    // the magic of the nibbles at bits 4..7 of a half (fp16 64.0: 64 + q) and minus the offsets of a word's eight
+    // elements in the order the extraction leaves them (0,4 | 1,5 | 2,6 | 3,7: bits 0..3, bits 4..7, 0..3, 4..7)
+    uint32_t magic_hi = 0x54005400u;
+    asm volatile("" : "+v"(magic_hi));
+    const half_t off_lo = (half_t)(float)(-(1024 + a.zero)), off_hi = (half_t)(float)(-(64 + a.zero));
+    const half8v neg_offsets = half8v{off_lo, off_lo, off_hi, off_hi, off_lo, off_lo, off_hi, off_hi};
 
     // iteration t of the segment (t = 0 .. n - 1) covers K-values k_of(t) 512 RK ..; iterations past the segment and
     // pieces past K fetch nothing (out-of-range offset: zeros arrive and the wait counts stay exact)
@@ -171,15 +179,17 @@ struct TileStreamQ4 : TileStreamPairs<1, 1, WN_, RK_, 3, false> {
       uint4v wf[STEPS];
 #pragma unroll
       for (int ss = 0; ss < STEPS; ++ss) wf[ss] = *reinterpret_cast<const uint4v *>(w_rd[ss] + wofs);
-      union {
-        uint32_t u[STEPS / 2];
-        half_t h[STEPS];
-      } sc;
+      // the scales of the four weight rows this lane holds sums of (result register r: row 4 (lane / 16) + r)
+      half_t sc[4][STEPS];
 #pragma unroll
-      for (int d = 0; d < STEPS / 2; ++d) sc.u[d] = *reinterpret_cast<const uint32_t *>(s_rd + ws * S_SLOT + 4 * d);
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int ss = 0; ss < STEPS; ++ss) sc[r][ss] = *reinterpret_cast<const half_t *>(s_rd4 + ws * S_SLOT + (r * STEPS + ss) * 2);
 #pragma unroll
       for (int ss = 0; ss < STEPS; ++ss) {
-        const half2v sc2 = half2v{sc.h[ss], sc.h[ss]};
+        // one step is one scale group: its sum starts from -sum a_k (offset_k + zero), four MFMAs on a constant
+        // fragment; the nibbles follow undecoded (1024 + q, 64 + q); the scale multiplies the fp32 group sum
+        half8v fa[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const uint4v v = *reinterpret_cast<const uint4v *>(a_rd[q] + aofs + 256 * ss);
@@ -188,9 +198,26 @@ struct TileStreamQ4 : TileStreamPairs<1, 1, WN_, RK_, 3, false> {
           p[1] = __builtin_amdgcn_perm(v[2], v[0], 0x07060302u);
           p[2] = __builtin_amdgcn_perm(v[3], v[1], 0x05040100u);
           p[3] = __builtin_amdgcn_perm(v[3], v[1], 0x07060302u);
-          const half8v fw = dequant_word_q4(wf[ss][q], qc, sc2);
-          part[q & 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fw, __builtin_bit_cast(half8v, p), part[q & 1], 0, 0, 0);
+          fa[q] = __builtin_bit_cast(half8v, p);
         }
+        AccV sum[2] = {AccV{0, 0, 0, 0}, AccV{0, 0, 0, 0}};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) sum[q & 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(neg_offsets, fa[q], sum[q & 1], 0, 0, 0);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          union {
+            uint32_t u[4];
+            half8v v;
+          } raw;
+          const uint32_t w = wf[ss][q], t8 = w >> 8;
+          raw.u[0] = and_or(w, qc.mask_lo, qc.magic);
+          raw.u[1] = and_or(w, qc.mask_hi, magic_hi);
+          raw.u[2] = and_or(t8, qc.mask_lo, qc.magic);
+          raw.u[3] = and_or(t8, qc.mask_hi, magic_hi);
+          sum[q & 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(raw.v, fa[q], sum[q & 1], 0, 0, 0);
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) part[0][r] = __builtin_fmaf(sum[0][r] + sum[1][r], (float)sc[r][ss], part[0][r]);
       }
       // the fragments are in registers before the next barrier hands the slots back to the loads
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");

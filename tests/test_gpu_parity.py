@@ -791,7 +791,11 @@ def test_q4_per_group_zero_points(sk, oracle):
                 assert gemv == (M == 1 and (bm, bn, bk) in ((16, 32, 512), (16, 64, 256), (16, 16, 1024))), (M, bm, bn, bk)
                 if sch.get("fixup") != "atomic" and not gemv:
                     same = sk.make_plan(M, N, K, "q4", "nt", dict(bm=bm, bn=bn, bk=bk, variant=1, **sch))
-                    assert torch.equal(sk.streamk_q4(dA, dW, dS, zeros=z7, plan=plan), sk.streamk_q4(dA, dW, dS, zero=7, plan=same))
+                    Cz, Cs = sk.streamk_q4(dA, dW, dS, zeros=z7, plan=plan), sk.streamk_q4(dA, dW, dS, zero=7, plan=same)
+                    if bm > 16:
+                        assert torch.equal(Cz, Cs)
+                    else:  # up to 16 rows the scalar-zero kernels multiply the nibbles undecoded and scale fp32 group sums
+                        assert _rel(oracle, Cz, Cs.double().cpu().numpy()) <= 1e-3
                 if gemv and (bm, bn, bk) != (16, 32, 512):   # the general kernel of the tile (bit-exact rounded weights) stays selectable
                     general = sk.make_plan(M, N, K, "q4_zp", "nt", dict(bm=bm, bn=bn, bk=bk, variant=1, **sch))
                     assert sk.kernel_name(general.kernel_id).startswith("skinny_q4zp")
@@ -1002,8 +1006,8 @@ def test_q4_matrix_vector_tiles_chained_in_one_cta(sk, oracle):
 
 
 def test_q4_matrix_vector_deviation_from_rounded_weights_is_bounded(sk, oracle):
-    """The M = 1 matrix-vector kernels multiply the unrounded (q - zero) * scale instead of the fp16-rounded
-    weights the other kernels (and sk_dequant_q4) form.  Per output that moves the result by at most
+    """The M = 1 matrix-vector kernels and the 16-row kernels with a scalar zero point multiply the unrounded
+    (q - zero) * scale instead of the fp16-rounded weights the other kernels (and sk_dequant_q4) form.  Per output that moves the result by at most
     sum_k |a_k| |w_exact - w_rounded| <= 2^-11 sum_k |a_k w_k|, plus the rounding of C to fp16 (2^-11 |c|) and fp32
     accumulation noise; and the result is the fp16 rounding of the exact (unrounded-weight) product up to that
     noise.  Checked at N = K = 8192 on the benchmark's data for every matrix-vector instance, beside the
@@ -1023,7 +1027,9 @@ def test_q4_matrix_vector_deviation_from_rounded_weights_is_bounded(sk, oracle):
     dA, dW, dS = _t(A), _t(Wq), _t(sc)
     ran = 0
     for (bm, bn, bk) in Q4_TILES[:8]:
-        for variant, rounded in ((3, False), (2, True), (1, True)):
+        # (the single-row instances form the rounded weights; the 16-row instances multiply the nibbles undecoded
+        # like the matrix-vector kernels)
+        for variant, rounded in ((3, False), (2, True), (1, (bm, bn, bk) == (16, 64, 256))):  # (that one instance decodes)
             try:
                 plan = sk.make_plan(1, N, K, "q4", "nt", dict(bm=bm, bn=bn, bk=bk, variant=variant, schedule="dp"))
             except sk.StreamKError:
@@ -1034,6 +1040,18 @@ def test_q4_matrix_vector_deviation_from_rounded_weights_is_bounded(sk, oracle):
             assert np.all(np.abs(y - target) <= 2.0 ** -11 * np.abs(target) + 2.0 ** -24 + noise), (bm, bn, bk, variant)
             ran += 1
     assert ran >= 12
+    # sixteen rows of A on the 16-row kernels (general and streamed through LDS): every row meets the same bounds
+    A16 = rng.standard_normal((16, K), dtype=np.float32).astype(np.float16)
+    a16 = A16.astype(np.float64)
+    y_rounded16, y_exact16 = a16 @ w_rounded.T, a16 @ w_exact.T
+    mass16 = np.abs(a16) @ np.abs(w_exact).T
+    for cfg in (dict(bm=16, bn=64, bk=512, variant=1), dict(bm=16, bn=32, bk=1024, variant=1), dict(bm=16, bn=16, bk=1024, variant=1),
+                dict(bm=16, bn=64, bk=512, variant=5), dict(bm=16, bn=32, bk=1024, variant=5)):
+        for sch in (dict(schedule="dp"), dict(schedule="basic", fixup="reduce", grid=200)):
+            plan = sk.make_plan(16, N, K, "q4", "nt", dict(cfg, **sch))
+            y = sk.streamk_q4(_t(A16), dW, dS, plan=plan).double().cpu().numpy()
+            assert np.all(np.abs(y - y_rounded16) <= 2.0 ** -11 * mass16 + 2.0 ** -11 * np.abs(y_rounded16) + 2e-5 * mass16), (cfg, sch)
+            assert np.all(np.abs(y - y_exact16) <= 2.0 ** -11 * np.abs(y_exact16) + 2.0 ** -24 + 2e-5 * mass16), (cfg, sch)
     # the same bound for the matrix-vector kernels with one zero point per group and row
     zp = rng.integers(0, 16, (N, K // 128)).astype(np.float16)
     w_rounded = oracle.dequant_q4_zp_np(Wq, sc, zp).astype(np.float64)
