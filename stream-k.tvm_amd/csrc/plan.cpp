@@ -145,15 +145,15 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
     // fifths of the CUs a tile the general kernel with 64 weight rows and K split over two waves, data-parallel
     // (16 x 28672 x 8192: 32.8 us; the 32-row kernel below: 48.5; 16 x 11008 x 4096: 10.7 / 14.8; 16 x 16384 x 16384:
     // 37.6 / 38.1).  Fewer rows and 16 MB of weights or more: the kernel that streams the packed weights through
-    // LDS in contiguous loads, 32 weight rows per tile (tile_stream_q4.h; 16 x 8192 x 8192: 13.4 us against 14.6,
-    // 16 x 4096 x 11008: 15.7 / 17.1; 16 x 4096 x 4096: 8.0 / 7.5, which stays with the kernel below).
+    // LDS in contiguous loads, 32 weight rows per tile (tile_stream_q4.h; 16 x 8192 x 8192: 12.2 us against 14.2,
+    // 16 x 4096 x 11008: 13.3 / 15.3; 16 x 4096 x 4096: 6.9 / 7.3).
     if (dtype == SK_Q4 && M > 1 && M <= 16 && want_variant < 0) {
       if (cdiv(N, 64) * 5 >= (int64_t)num_cus * 3) {
         for (int i = 0; i < n; ++i)
           if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].variant == 0 && t[i].bm == 16 &&
               t[i].bn == 64 && t[i].bk == 512 && accepts_shape(t[i], M, K))
             return &t[i];
-      } else if (N * K >= ((int64_t)32 << 20) && K % 256 == 0) {
+      } else if (N * K >= ((int64_t)16 << 20) && K % 256 == 0) {
         for (int i = 0; i < n; ++i)
           if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].variant == 4 && t[i].bn == 32 &&
               accepts_shape(t[i], M, K))

@@ -205,9 +205,9 @@ def test_untuned_plans_keep_cta_ranges_aligned(sk):
                                          (64, 11008, 4096, "bfloat16", "stream_bf16_mb2_nb2_wm2_wn2_rk1_d3", 172),
                                          (4, 8192, 8192, "float16", "stream_f16_mb1_wm1_wn2_rk2_d3", 256),
                                          (4, 4096, 4096, "float16", "gemv_rows_f16_m4_wn1_rk4", 256),
-                                         (16, 8192, 8192, "q4", "stream_q4_wn2_rk2_kh2_d5", 256),
+                                         (16, 8192, 8192, "q4", "stream_q4_wn2_rk2_kh2_d3", 256),
                                          (16, 28672, 8192, "q4", "skinny_q4_mb1_wn4_rk2_row1_0", 448),
-                                         (16, 4096, 4096, "q4", "skinny_q4_mb1_wn2_rk4_row1_0", 128)]:
+                                         (16, 4096, 4096, "q4", "stream_q4_wn2_rk2_kh2_d3", 128)]:
         p = sk.make_plan(M, N, K, dtype, "nt", cus=256, use_tuned=False)
         assert (sk.kernel_name(p.kernel_id), p.schedule, p.grid) == (want, DP, grid), (M, N, K, dtype, sk.kernel_name(p.kernel_id), p.grid)
     # a caller's tile or schedule is not overridden

@@ -637,9 +637,9 @@ def test_q4_ragged_shapes_every_kernel(sk, oracle, variant):
 def test_q4_weights_streamed_through_lds(sk, oracle):
     """Up to 16 rows of A on the kernels that stream row-major Q4 weights through LDS in contiguous loads (64 and 32
     weight rows per tile): ragged M and N, K a multiple of 256 only (a last iteration hanging over K), zero points
-    0 / 5 / 8 / 15, all schedules and both fix-ups.  The weights these kernels multiply are the fp16-rounded ones of
-    the oracle: exact on integer data with power-of-two scales (any wrong nibble, K order, scale row or rotation
-    shows), within 2e-3 of the oracle on random data; K that is not a multiple of 256 is refused."""
+    0 / 5 / 8 / 15, all schedules and both fix-ups.  Exact on integer data with power-of-two scales (any wrong nibble,
+    K order, scale row or rotation shows), within 2e-3 of the oracle on random data (these kernels multiply the
+    unrounded (q - zero) * scale, the oracle the fp16-rounded weights); K that is not a multiple of 256 is refused."""
     import torch
     rng = np.random.default_rng(58)
     ran = 0
@@ -673,7 +673,8 @@ def test_q4_weights_streamed_through_lds(sk, oracle):
         sk.make_plan(17, 1000, 1024, "q4", "nt", dict(bm=16, bn=64, bk=512, variant=5))
     # what the library picks by itself for 2..16 rows and 16 MB of weights or more
     assert sk.kernel_name(sk.make_plan(16, 8192, 8192, "q4", "nt", use_tuned=False).kernel_id).startswith("stream_q4_")
-    assert not sk.kernel_name(sk.make_plan(16, 4096, 4096, "q4", "nt", use_tuned=False).kernel_id).startswith("stream_q4_")
+    assert sk.kernel_name(sk.make_plan(16, 4096, 4096, "q4", "nt", use_tuned=False).kernel_id).startswith("stream_q4_")
+    assert not sk.kernel_name(sk.make_plan(16, 2048, 4096, "q4", "nt", use_tuned=False).kernel_id).startswith("stream_q4_")
     sk.workspace_status()
 
 
