@@ -16,7 +16,8 @@ carries
                 with the weights from HBM next to the vendor GEMM, and the 16 cells M = 1 / 16 / 64 / 256 over four
                 projection shapes (N, K) of a 7B / 70B decoder against `torch.matmul` in the same run,
   extra         the measurements behind them and the rest: M sweep at N = K = 8192, 1024x1024x8192 with all
-                fix-ups, the large dense shapes in both layouts and types, the reference's own run shapes
+                fix-ups, the large dense shapes in both layouts and types, the reference's own run shapes, one row of
+                A on 16384 x 16384 and 28672 x 8192 Q4 weights from HBM
                 (kernels this short are timed as graph-captured batches).
 The oracle is used here as the timed CPU baseline and as a result check only.
 """
