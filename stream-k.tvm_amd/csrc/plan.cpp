@@ -103,11 +103,13 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
       if (t[i].family == FAMILY_TILE && t[i].dtype == SK_Q4 && t[i].bm == want_bm && t[i].bn == want_bn) return &t[i];
     return nullptr;
   }
-  // (2 <= M <= 4: from about 100 MB of weights on; below, the matrix-vector form with four rows of A starts up faster --
-  // 4 x 8192 x 8192: 24.8 us against 32.0 us, 2 x 4096 x 4096: 12.1 us against 11.3 us, weights from HBM)
-  // (one row: from 128 MB on -- 1 x 8192 x 8192 24.4 us against 28.9 us for the matrix-vector kernel, 1 x 28672 x 8192
-  // 76.4 / 76.6, 1 x 11008 x 4096 19.8 / 17.6)
-  const bool stream_rows = M >= 5 || (M >= 2 && N * K >= (int64_t)48 << 20) || N * K >= (int64_t)64 << 20;
+  // (2 <= M <= 4 as well: the matrix-vector form with four rows of A (variant 3) is behind at every size measured,
+  // weights from HBM -- 2 x 4096 x 4096 11.3 us against 8.7 us on 16 x 16 tiles, 4 x 11008 x 4096 23.0 / 17.5,
+  // 4 x 4096 x 11008 26.9 / 17.4, 4 x 8192 x 8192 32.0 / 24.8 -- and stays as an explicit choice)
+  // (one row: from 40 MB on -- 1 x 8192 x 8192 24.4 us against 28.9 us for the matrix-vector kernel, 1 x 14336 x 4096
+  // 22.3 / 27.3, 1 x 4096 x 11008 17.3 / 19.9, 1 x 5120 x 5120 11.7 / 13.8, 1 x 11008 x 4096 17.5 / 17.2; 1 x 4096 x 4096
+  // 8.6 / 8.1 stays with the matrix-vector kernel)
+  const bool stream_rows = M >= 2 || N * K >= (int64_t)20 << 20;
   if ((dtype == SK_F16 || dtype == SK_BF16) && layout == SK_LAYOUT_NT && stream_rows && M <= 64 && want_variant < 0) {
     // 5 <= M <= 64 (fewer rows on large weights, above) with fp16 / bfloat16 weights: the kernels that stream the weights through LDS in contiguous loads
     // (tile_stream_pairs.h).  Tiles of 32 weight rows while one wave of them fits the device (N = 8192: one tile per
@@ -447,9 +449,10 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
     const int64_t iters = total64 * out->iters_per_tile;
     // (the kernels that stream the weights through LDS are bound by memory: with tiles for three fifths of the CUs --
     // fp16 / bfloat16: two fifths -- they run data-parallel rather than pay a fix-up; Q4 16 x 11008 x 4096: 11.5 us
-    // against 14.3 us, fp16 16 x 2048 x 8192 on 128 tiles: 11.5 against 14.1)
+    // against 14.3 us, fp16 16 x 2048 x 8192 on 128 tiles: 11.5 against 14.1, 32 x 11008 x 4096 on 172 tiles of 32 x 64:
+    // 19.2 against 22.7; not the 64 x 32 tiles, where the split wins)
     const bool stream_dp = k->family == FAMILY_SKINNY && (k->variant == 4 || k->dtype == SK_Q4) && k->max_m >= 16 &&
-                           (k->bm == 16 || (k->variant == 4 && k->bm == 64 && k->bn == 64)) &&
+                           (k->bm == 16 || (k->variant == 4 && k->dtype != SK_Q4 && !(k->bm == 64 && k->bn == 32))) &&
                            total64 * 5 >= (int64_t)num_cus * (k->variant == 4 && k->dtype != SK_Q4 ? 2 : 3);
     const bool q4_gemv = k->family == FAMILY_SKINNY && k->variant == 2 && k->max_m == 1 &&
                          (k->dtype == SK_Q4 || k->dtype == SK_Q4_ZP || k->dtype == SK_Q4_TILED || k->dtype == SK_Q4_ZP_TILED);

@@ -1160,8 +1160,12 @@ def test_f16_few_rows_in_the_matrix_vector_form(sk, oracle):
     Wi = rng.integers(-1, 2, (N, K)).astype(np.float16)
     bias = rng.integers(-3, 4, N).astype(np.float16)
     want = np.maximum(Ai.astype(np.int64) @ Wi.astype(np.int64).T + bias.astype(np.int64), 0)
-    assert sk.kernel_name(sk.make_plan(M, N, K, "float16", "nt", use_tuned=False).kernel_id) == "gemv_rows_f16_m4_wn1_rk4"
-    for sch in (dict(), dict(schedule="sk2", fixup="reduce", grid=64), dict(schedule="sk2", fixup="atomic", grid=64)):
+    # (the planner itself takes the kernels that stream the weights through LDS from two rows on; this form stays an
+    # explicit choice)
+    assert sk.kernel_name(sk.make_plan(M, N, K, "float16", "nt", use_tuned=False).kernel_id).startswith("stream_f16_")
+    rows = dict(bm=16, bn=16, bk=512, variant=4)
+    assert sk.kernel_name(sk.make_plan(M, N, K, "float16", "nt", rows).kernel_id) == "gemv_rows_f16_m4_wn1_rk4"
+    for sch in (dict(), rows, dict(rows, schedule="sk2", fixup="reduce", grid=64), dict(rows, schedule="sk2", fixup="atomic", grid=64)):
         out = torch.zeros(M, N + 24, dtype=torch.float16, device="cuda")[:, 8:8 + N]
         C = sk.streamk_fp16(_t(Ai), _t(Wi), out=out, bias=_t(bias), activation="relu", **sch)
         assert np.array_equal(C.cpu().numpy().astype(np.int64), want), sch
@@ -1375,10 +1379,10 @@ def test_bf16_small_m_kernels(sk, oracle):
                     assert torch.equal(C, sk.streamk_bf16(A.cuda(), B.cuda(), plan=plan))
     for M in (1, 2, 16, 32):
         plan = sk.make_plan(M, 4096, 4096, "bfloat16", "nt")
-        # (one row: matrix-vector kernels; two to four rows: their form with four rows of A; else the general kernels
-        # or the ones that stream the weights through LDS)
-        assert (241 <= plan.kernel_id <= 248) if M == 1 else ((210 <= plan.kernel_id <= 211) if M <= 4 else
-                                                               (230 <= plan.kernel_id <= 240 or plan.kernel_id in (282, 283, 285, 287, 289, 293, 297))), (M, plan.kernel_id)
+        # (one row of 4096 x 4096: matrix-vector kernels; more rows: the general kernels or the ones that stream the
+        # weights through LDS)
+        assert (241 <= plan.kernel_id <= 248) if M == 1 else (230 <= plan.kernel_id <= 240 or
+                                                               plan.kernel_id in (282, 283, 285, 287, 289, 293, 297)), (M, plan.kernel_id)
         A, W = (torch.rand(M, 4096) * 2 - 1).bfloat16(), (torch.rand(4096, 4096) * 2 - 1).bfloat16()
         ref = oracle.matmul_fp32(A.float().numpy(), W.float().numpy(), trans_b=True)
         assert _rel(oracle, sk.streamk_bf16(A.cuda(), W.cuda()), ref) <= 4e-3, M
