@@ -1003,6 +1003,18 @@ def test_q4_matrix_vector_tiles_chained_in_one_cta(sk, oracle):
     assert sk.kernel_name(plan.kernel_id) == "gemv_q4_nb1_wn1_rk8_k16384" and plan.grid == 256
     plan = sk.make_plan(1, 32000, 4096, "q4", "nt", use_tuned=False)
     assert sk.kernel_name(plan.kernel_id) == "gemv_q4_nb1_wn1_rk2_k16384" and plan.grid == 1000
+    # such plans against the oracle, N ragged (the host product is taken on the first and the last rows of the weights)
+    for (N, K) in [(20010, 4096), (28672 + 8, 8192), (16400, 1536)]:
+        A = (rng.random((1, K), dtype=np.float32) * 2 - 1).astype(np.float16)
+        Wq = rng.integers(0, 256, (N, K // 2), dtype=np.uint8)
+        sc = rng.uniform(0.005, 0.02, (N, K // 128)).astype(np.float16)
+        plan = sk.make_plan(1, N, K, "q4", "nt", use_tuned=False)
+        assert plan.grid < plan.total_tiles and sk.kernel_name(plan.kernel_id).startswith("gemv_q4"), (N, K, plan.grid)
+        C = torch.full((1, N), float("nan"), dtype=torch.float16, device="cuda")
+        sk.streamk_q4(_t(A), _t(Wq), _t(sc), out=C, plan=plan)
+        assert not bool(torch.isnan(C).any())
+        for rows in (slice(0, 600), slice(N // 2 - 300, N // 2 + 300), slice(N - 600, N)):
+            assert _rel(oracle, C[:, rows], oracle.q4_gemm_ref(A, Wq[rows], sc[rows], 128, 8)) <= 2e-3, (N, K, rows)
     sk.workspace_status()
 
 
