@@ -267,11 +267,12 @@ struct KernelInfo {
 // Up to 16 rows of A, Q4 weights (row-major, scalar zero point) streaming through LDS in contiguous loads
 // (tile_stream_q4.h; dtype SK_Q4, variant 4):  X(id, WN, RK, KH, WD, AD)
 #define SK_STREAM_Q4_KERNELS(X) \
-  X(290, 4, 1, 2, 5, 4)         \
-  X(291, 2, 2, 2, 3, 3)
+  X(290, 4, 1, 4, 4, 4)         \
+  X(291, 2, 2, 4, 3, 3)
 // (the 32-row instance asks for A two iterations ahead, three slots of each ring: with five slots of weights and two
 // of A -- A requested one iteration ahead -- 16 x 8192 x 8192 took 13.2 us from HBM against 12.2, 11.6 / 10.7 with the
-// weights in the Infinity Cache)
+// weights in the Infinity Cache; four waves per ring instead of two: 10.7 -> 10.2, the 64-row instance 31.7 -> 28.9 us
+// at 16 x 16384 x 16384, 37.7 -> 36.2 from HBM)
 // (an instance with eight rings, 128 weight rows and one wave per ring -- X(294, 8, 1, 1, 3, 3): half the bytes of A per
 // byte of weights -- was measured and is not built: 16 x 16384 x 16384 split in two over K 39.7 us against 39.4 for the
 // 64-row instance and 37.5 for the general kernel, 16 x 8192 x 8192 17.8 against 13.8)

@@ -8,13 +8,13 @@
 // the nibbles enter the 16x16x32 MFMA as 1024 + q / 64 + q, every 128-wide scale group's sum starts from
 // -sum a_k (offset_k + zero) (four MFMAs on a constant fragment) and is multiplied by the group's scale in fp32.
 //
-//  * CTA = eight waves, two per SIMD: WN_ along N x RK_ along K rings of weights, KH_ waves per ring (four rings shared
-//    by two waves each, which take 256 of the 512 K-values of an iteration; or eight rings, 128 weight rows, one wave
-//    each) (the decode keeps the vector pipeline
-//    busy: the second wave of a SIMD works while the first waits for LDS or for its MFMAs).  Per iteration and ring:
-//    four loads of weights (16 rows x 256 bytes) shared out between its two waves, one load of scales per wave (16
-//    rows x the wave's 2 groups, four bytes per lane), and the 16 RK_ loads of A (one row of 1024 bytes each) shared
-//    out among all eight waves, all direct to LDS.
+//  * CTA = WN_ along N x RK_ along K rings of weights, KH_ waves per ring, which share out the 512 K-values of an
+//    iteration in steps of 128 (one scale group): four rings of four waves each in the instances built, sixteen waves,
+//    four per SIMD (one wave's waits for LDS and for its MFMAs are covered by the three others: with two waves per
+//    ring 16 x 8192 x 8192 took 10.7 us against 10.2 with the weights in the Infinity Cache, 16 x 4096 x 11008 13.3
+//    against 12.2).  Per iteration and ring: four loads of weights (16 rows x 256 bytes) shared out between its
+//    waves, one load of scales per wave (16 rows x the pair of groups its step is in, four bytes per lane), and the
+//    16 RK_ loads of A (one row of 1024 bytes each) shared out among all waves, all direct to LDS.
 //  * No padding: lane l of a load fetches the 16-byte piece (l % 16) ^ (row % 16) of its row for position l % 16
 //    (A: piece l ^ row of the row's 64), so the sixteen lanes that read the same piece of sixteen rows find it on
 //    sixteen different bank groups.
@@ -48,7 +48,8 @@ struct TileStreamQ4 : TileStreamPairs<1, 1, WN_, RK_, 3, false> {
   static constexpr int KH = KH_;                       // waves that share the weights of an iteration, 512 / KH_ K-values each
   static constexpr int STEPS = 4 / KH;                 // steps of 128 K-values (one scale group) per wave and iteration
   static constexpr int RINGS = WN_ * RK_, NWAVES = RINGS * KH;
-  static_assert(KH == 1 || KH == 2, "one or two waves per ring");
+  static_assert(KH == 1 || KH == 2 || KH == 4, "one, two or four waves per ring");
+  static constexpr int SG = STEPS < 2 ? 2 : STEPS;     // scale groups a wave's load of scales brings per row (a load moves four bytes per lane)
   static constexpr int WN = WN_, RK = RK_, WD = WD_, AD = AD_, NT = 64 * NWAVES, BM = 16, BN = 16 * WN, MAX_M = 16;
   static constexpr int BK = 512, BKC = 512 * RK;       // K-values per iteration: of a weight ring, of the CTA
   static constexpr int W_SLOT = 16 * 256;              // 16 weight rows x 256 bytes
@@ -109,7 +110,7 @@ struct TileStreamQ4 : TileStreamPairs<1, 1, WN_, RK_, 3, false> {
       voff_w[jj] = (uint32_t)wr * ldw_bytes + (uint32_t)piece_w[jj] * 16;
     }
     // scales: STEPS / 2 lanes per row, four bytes each (the groups of the wave's 128 STEPS K-values)
-    const uint32_t voff_s = lane < 8 * STEPS ? (uint32_t)(lane / (STEPS / 2)) * lds_bytes + (uint32_t)(lane % (STEPS / 2)) * 4 : OOB_OFFSET;
+    const uint32_t voff_s = lane < 8 * SG ? (uint32_t)(lane / (SG / 2)) * lds_bytes + (uint32_t)(lane % (SG / 2)) * 4 : OOB_OFFSET;
     // fragments: wave kh takes the steps s = 2 kh, 2 kh + 1 of the iteration; lane (i, g) reads piece 4 s + g of
     // weight row i, found at position (4 s + g) ^ i, and for word q of it the eight values of A row i from K offset
     // 32 (4 s + g) + 8 q: piece 16 s + 4 g + q, at position piece ^ i
@@ -125,7 +126,7 @@ struct TileStreamQ4 : TileStreamPairs<1, 1, WN_, RK_, 3, false> {
 #pragma unroll
     for (int q = 0; q < 4; ++q)
       a_rd[q] = smem + LDS_W + LDS_S + rk * A_CHUNK + fi * 1024 + 256 * STEPS * kh + 16 * ((4 * fg + q) ^ fi);
-    const char *s_rd4 = smem + LDS_W + wave * (WD * S_SLOT) + fg * (4 * 2 * STEPS);
+    const char *s_rd4 = smem + LDS_W + wave * (WD * S_SLOT) + fg * (4 * 2 * SG) + ((STEPS * kh) % SG) * 2;
     const Q4Consts qc = q4_consts(a.zero);
     // the magic of the nibbles at bits 4..7 of a half (fp16 64.0: 64 + q) and minus the offsets of a word's eight
     // elements in the order the extraction leaves them (0,4 | 1,5 | 2,6 | 3,7: bits 0..3, bits 4..7, 0..3, 4..7)
@@ -148,7 +149,7 @@ struct TileStreamQ4 : TileStreamPairs<1, 1, WN_, RK_, 3, false> {
                     (t < n && kk + piece_w[jj] * 32 < a.K) ? voff_w[jj] : OOB_OFFSET, kbytes + (uint32_t)(4 * j) * ldw_bytes);
       }
       dma_load_4(rsrc_s, s_ring + (uint32_t)(slot * S_SLOT), t < n ? voff_s : OOB_OFFSET,
-                 (uint32_t)__builtin_amdgcn_readfirstlane((kk / 128 + STEPS * kh) * 2));
+                 (uint32_t)__builtin_amdgcn_readfirstlane((kk / 128 + (STEPS * kh) / SG * SG) * 2));
     };
     auto issue_a = [&](int t, int slot) {
 #pragma unroll
@@ -184,7 +185,7 @@ struct TileStreamQ4 : TileStreamPairs<1, 1, WN_, RK_, 3, false> {
 #pragma unroll
       for (int r = 0; r < 4; ++r)
 #pragma unroll
-        for (int ss = 0; ss < STEPS; ++ss) sc[r][ss] = *reinterpret_cast<const half_t *>(s_rd4 + ws * S_SLOT + (r * STEPS + ss) * 2);
+        for (int ss = 0; ss < STEPS; ++ss) sc[r][ss] = *reinterpret_cast<const half_t *>(s_rd4 + ws * S_SLOT + (r * SG + ss) * 2);
 #pragma unroll
       for (int ss = 0; ss < STEPS; ++ss) {
         // one step is one scale group: its sum starts from -sum a_k (offset_k + zero), four MFMAs on a constant

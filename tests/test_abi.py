@@ -208,9 +208,9 @@ def test_untuned_plans_keep_cta_ranges_aligned(sk):
                                          (2, 11008, 4096, "float16", "stream_f16_mb1_wm1_wn4_rk1_d4", 172),
                                          (32, 11008, 4096, "float16", "stream_f16_mb2_wm1_wn4_rk1_d3", 172),
                                          (3, 4096, 4160, "float16", "stream_f16_mb1_nb1_wm1_wn1_rk4_d3", 256),
-                                         (16, 8192, 8192, "q4", "stream_q4_wn2_rk2_kh2_d3", 256),
+                                         (16, 8192, 8192, "q4", "stream_q4_wn2_rk2_kh4_d3", 256),
                                          (16, 28672, 8192, "q4", "skinny_q4_mb1_wn4_rk2_row1_0", 448),
-                                         (16, 4096, 4096, "q4", "stream_q4_wn2_rk2_kh2_d3", 128)]:
+                                         (16, 4096, 4096, "q4", "stream_q4_wn2_rk2_kh4_d3", 128)]:
         p = sk.make_plan(M, N, K, dtype, "nt", cus=256, use_tuned=False)
         assert (sk.kernel_name(p.kernel_id), p.schedule, p.grid) == (want, DP, grid), (M, N, K, dtype, sk.kernel_name(p.kernel_id), p.grid)
     # a caller's tile or schedule is not overridden
