@@ -257,7 +257,8 @@ struct KernelInfo {
   X(289, 1, 2, 2, 1, 4)
 
 // the same with NB blocks of 16 weight rows per wave, AD slots of A and the unpadded rings (64 x 64 tiles: the 160 KB
-// of LDS exactly; 16 x 16 tiles with K split over the four waves: the same):  X(id, MB, WM, WN, RK, DEPTH, NB, AD, BF16)
+// of LDS exactly; 16 x 16 tiles with K split over the four waves: the same), and two waves sharing the K-steps of each
+// of those four (eight waves per CTA):  X(id, MB, WM, WN, RK, DEPTH, NB, AD, BF16)
 #define SK_STREAM_BLOCKS_KERNELS(X)  \
   X(292, 2, 2, 2, 1, 3, 2, 2, false) \
   X(293, 2, 2, 2, 1, 3, 2, 2, true)  \

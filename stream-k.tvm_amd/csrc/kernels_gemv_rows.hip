@@ -58,7 +58,7 @@ int gemv_rows_kernel_infos(KernelInfo *out, int max) {
 #undef X
 #define X(id, MB, WM, WN, RK, DEPTH, NB, AD, BF)                                                                 \
   if (n < max) {                                                                                                \
-    typedef TileStreamPairs<MB, WM, WN, RK, DEPTH, BF, NB, AD, false> P;                                        \
+    typedef TileStreamPairs<MB, WM, WN, RK, DEPTH, BF, NB, AD, false, 2> P;                                        \
     out[n++] = KernelInfo{id, FAMILY_SKINNY, (BF) ? 3 : 0, 0, 4, P::BM, P::BN, P::BKC, P::NT, P::LDS_BYTES, P::CTAS_PER_CU, \
                           P::TILE_ELEMS, 0, P::MAX_M, 8, (BF) ? "stream_bf16_mb" #MB "_nb" #NB "_wm" #WM "_wn" #WN "_rk" #RK "_d" #DEPTH \
                                                               : "stream_f16_mb" #MB "_nb" #NB "_wm" #WM "_wn" #WN "_rk" #RK "_d" #DEPTH}; \
@@ -122,7 +122,7 @@ int launch_gemv_rows(int id, const SkinnyArgs &a, const DevPlan &p, const Worksp
 #undef X
 #define X(id_, MB, WM, WN, RK, DEPTH, NB, AD, BF)                         \
   case id_: {                                                             \
-    typedef TileStreamPairs<MB, WM, WN, RK, DEPTH, BF, NB, AD, false> P;  \
+    typedef TileStreamPairs<MB, WM, WN, RK, DEPTH, BF, NB, AD, false, 2> P;  \
     return launch_policy<P>(a, p, ws, s, bias);                           \
   }
     SK_STREAM_BLOCKS_KERNELS(X)
@@ -197,7 +197,7 @@ int occupancy_gemv_rows(int id) {
 #undef X
 #define X(id_, MB, WM, WN, RK, DEPTH, NB, AD, BF)                                                        \
   case id_: {                                                                                            \
-    typedef TileStreamPairs<MB, WM, WN, RK, DEPTH, BF, NB, AD, false> P;                                 \
+    typedef TileStreamPairs<MB, WM, WN, RK, DEPTH, BF, NB, AD, false, 2> P;                                 \
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, sk_skinny_kernel<P>, P::NT, 0) != hipSuccess) \
       return -1;                                                                                         \
     return occ;                                                                                          \

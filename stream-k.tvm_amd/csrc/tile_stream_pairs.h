@@ -6,7 +6,7 @@
 // instruction reads two rows of 512 contiguous bytes (the first 32 lanes one row, the others the next) directly into
 // LDS, and the fragments come back out of LDS in the MFMA's order (16 x 16384 x 16384: 134 us -> 87 us, 6.2 TB/s):
 //
-//  * CTA = four waves, WM_ along M x WN_ along N x RK_ along K: wave (wm, wn, rk) owns MB_ blocks of 16 rows of A,
+//  * CTA = four waves (times KH_, below), WM_ along M x WN_ along N x RK_ along K: wave (wm, wn, rk) owns MB_ blocks of 16 rows of A,
 //    16 weight rows and the K sub-block rk of every iteration; the RK_ sums are added through LDS when the segment
 //    ends (the reference's "block reduction", streamk_fp16_block_reduce.py:45,235-306).  An iteration is 256
 //    K-values per wave.  The 16 weight rows x 512 bytes of (wn, rk) are fetched once, by eight loads shared out
@@ -22,6 +22,10 @@
 //    and two of A are in flight.  Per iteration one wait for the wave's own loads (vmcnt, in order), one barrier
 //    (everybody's loads of the iteration have landed, and the slots refilled next have been read by everybody), the
 //    loads that refill them, 8 + 8 MB_ fragment reads and 8 MB_ MFMAs.
+//  * KH_ = 2 (the 64 x 64 and the 16 x 16 instances): two waves share the eight 32-wide K-steps of every (wm, wn, rk)
+//    and its loads, eight waves per CTA, their sums added through LDS with the RK_ ones (64 x 28672 x 8192 from HBM
+//    90.8 -> 86.4 us, 16 x 4096 x 4096 9.7 -> 9.2; the other instances gain nothing or lose: 64 x 32 tiles at
+//    64 x 8192 x 8192 28.8 -> 33.8 us).
 //  * Tiles walk K from different offsets (rotation_of, sk_device.h).
 //
 // Replaces the reference's inner MAC for its own run shape, 16 x 16384 x 8192 (streamk_fp16_nt.py:15, :196-240).
@@ -30,7 +34,8 @@
 
 namespace sk {
 
-template <int MB_, int WM_, int WN_, int RK_, int DEPTH_, bool BF16_ = false, int NB_ = 1, int AD_ = 3, bool PADDED_ = true>
+template <int MB_, int WM_, int WN_, int RK_, int DEPTH_, bool BF16_ = false, int NB_ = 1, int AD_ = 3, bool PADDED_ = true,
+          int KH_ = 1>
 struct TileStreamPairs {
   typedef SkinnyArgs Args;
   typedef floatx4 AccV;
@@ -41,7 +46,10 @@ struct TileStreamPairs {
   // instance fills the 160 KB of LDS: the persistent loop's one word of LDS is the first word of the rings
   static constexpr bool FIXUP_WORD_IN_LDS = true;
   // AD slots of A (three unless LDS is short): its loads are issued later than the weights' when DEPTH_ is larger
-  static constexpr int MB = MB_, NB = NB_, WM = WM_, WN = WN_, RK = RK_, WD = DEPTH_, AD = AD_, NT = 256;
+  // KH_ waves share the eight 32-wide K-steps of a (wm, wn, rk) wave's iteration (and its loads) between them
+  static constexpr int MB = MB_, NB = NB_, WM = WM_, WN = WN_, RK = RK_, WD = DEPTH_, AD = AD_, KH = KH_, NT = 256 * KH_;
+  static constexpr int NWAVES = 4 * KH, STEPS = 8 / KH;
+  static_assert(KH == 1 || KH == 2 || KH == 4, "one, two or four waves per K sub-block");
   static constexpr bool PADDED = PADDED_;
   static_assert(WM == 1 || WM == 2, "the eight loads of a weight ring are shared out among WM_ waves");
   static constexpr int BM = 16 * MB * WM, BN = 16 * NB * WN, MAX_M = BM;
@@ -57,11 +65,11 @@ struct TileStreamPairs {
   static constexpr int LDS_W = RINGS * WD * W_SLOT, LDS_BYTES = LDS_W + AD * A_SLOT, LDS_TOTAL = LDS_BYTES;
   static_assert(WD >= AD && AD >= 2, "the barrier of an iteration frees the slots read an iteration earlier");
   static constexpr int CTAS_PER_CU = (160 * 1024) / (LDS_BYTES + 64) > 0 ? (160 * 1024) / (LDS_BYTES + 64) : 1;
-  static constexpr int WAVES_PER_EU = CTAS_PER_CU;
+  static constexpr int WAVES_PER_EU = CTAS_PER_CU * KH;
   static constexpr int TILE_ELEMS = BM * BN;
   static constexpr int NTP = WM * WN * 64;             // the rk == 0 waves hold the tile's sums
   static constexpr int NV4 = MB * NB;
-  static constexpr int LOADS_W = NB * 8 / WM, LOADS_A = (A_PAIRS * RK) / 4;  // direct-to-LDS loads per wave and iteration
+  static constexpr int LOADS_W = NB * 8 / (WM * KH), LOADS_A = (A_PAIRS * RK) / NWAVES;  // direct-to-LDS loads per wave and iteration
   // Loads are issued in the order A(t + AD - 1), W(t + WD - 1) in iteration t, and complete in that order.  Iteration t
   // needs everything up to A(t) and W(t): with WD == AD that leaves the AD - 2 later iterations outstanding, with
   // WD > AD (W(t) is older than A(t)) the weights issued with A(t) and the AD - 2 iterations after them.
@@ -81,11 +89,12 @@ struct TileStreamPairs {
     // (checked here and not in the class: tile_stream_q4.h derives from instances it does not run this loop of)
     static_assert(WM * WN * RK == 4, "four waves");
     static_assert(LDS_BYTES <= 160 * 1024, "the rings must fit the LDS of a CU");
-    static_assert((RK - 1) * WN * WM * 64 * MB * NB * 16 <= LDS_W, "the sums of the K-splitting waves pass through the weights' rings");
-    static_assert((A_PAIRS * RK) % 4 == 0, "the loads of A are shared out evenly");
+    static_assert((RK * KH - 1) * WN * WM * 64 * MB * NB * 16 <= LDS_W, "the sums of the K-splitting waves pass through the weights' rings");
+    static_assert((A_PAIRS * RK) % NWAVES == 0 && 8 % (WM * KH) == 0, "the loads are shared out evenly");
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
-    const int wm = wave % WM, wn = (wave / WM) % WN, rk = wave / (WM * WN);
+    // wave = ((kh RK + rk) WN + wn) WM + wm: the waves that end up with the tile's sums come first
+    const int wm = wave % WM, wn = (wave / WM) % WN, rk = (wave / (WM * WN)) % RK, kh = wave / (WM * WN * RK);
 #pragma unroll
     for (int i = 0; i < MB; ++i)
 #pragma unroll
@@ -124,8 +133,8 @@ struct TileStreamPairs {
 #pragma unroll
       for (int b = 0; b < NB; ++b)
 #pragma unroll
-        for (int jj = 0; jj < 8 / WM; ++jj) {
-          const int j = wm * (8 / WM) + jj;   // this wave's share of the ring's eight pairs of rows
+        for (int jj = 0; jj < 8 / (WM * KH); ++jj) {
+          const int j = (kh * WM + wm) * (8 / (WM * KH)) + jj;   // this wave's share of the ring's eight pairs of rows
           const int pc = piece_of(j);
           dma_load_16(rsrc_w, w_ring + (uint32_t)((b * WD + slot) * W_SLOT + j * PAIR),
                       (t < n && kk + pc * 8 < a.K) ? (uint32_t)odd * ldw_bytes + (uint32_t)pc * 16 : OOB_OFFSET,
@@ -159,20 +168,21 @@ struct TileStreamPairs {
       issue_a(t + AD - 1, as == 0 ? AD - 1 : as - 1);
       issue_w(t + WD - 1, ws == 0 ? WD - 1 : ws - 1);
       const char *wp = w_ptr + ws * W_SLOT, *ap = a_ptr + as * A_SLOT;
-      half8v fw[NB][8], fa[MB][8];
+      half8v fw[NB][8], fa[MB][8];   // (this wave's steps kh STEPS .. kh STEPS + STEPS - 1 only)
 #pragma unroll
-      for (int s = 0; s < 8; ++s) {
+      for (int s8 = 0; s8 < STEPS; ++s8) {
+        const int s = KH == 1 ? s8 : kh * STEPS + s8;
         // PADDED: piece 4 s + g sits 64 s bytes further on; else its position is (4 s + g) ^ i: 64 s XORed in
         const int so = PADDED ? s * 64 : 0;
         const int sx = PADDED ? 0 : s * 64;
 #pragma unroll
         for (int j = 0; j < NB; ++j)
-          fw[j][s] = *reinterpret_cast<const half8v *>(xor_offset(wp + j * (WD * W_SLOT), frag0, sx) + so);
+          fw[j][s8] = *reinterpret_cast<const half8v *>(xor_offset(wp + j * (WD * W_SLOT), frag0, sx) + so);
 #pragma unroll
-        for (int i = 0; i < MB; ++i) fa[i][s] = *reinterpret_cast<const half8v *>(xor_offset(ap + i * 8 * PAIR, frag0, sx) + so);
+        for (int i = 0; i < MB; ++i) fa[i][s8] = *reinterpret_cast<const half8v *>(xor_offset(ap + i * 8 * PAIR, frag0, sx) + so);
       }
 #pragma unroll
-      for (int s = 0; s < 8; ++s)
+      for (int s = 0; s < STEPS; ++s)
 #pragma unroll
         for (int i = 0; i < MB; ++i)
 #pragma unroll
@@ -195,17 +205,17 @@ struct TileStreamPairs {
     __syncthreads();
 
     // ---- sum the RK partial accumulators into the rk == 0 waves (through the weights' rings, free by now) ----
-    if constexpr (RK > 1) {
+    if constexpr (RK * KH > 1) {
       float *red = reinterpret_cast<float *>(smem);
-      if (rk > 0) {
+      if (wave >= WM * WN) {
 #pragma unroll
         for (int v = 0; v < NV4; ++v)
           *reinterpret_cast<AccV *>(red + (((wave - WM * WN) * NV4 + v) * 64 + lane) * 4) = acc.c[v / NB][v % NB];
       }
       __syncthreads();
-      if (rk == 0) {
+      if (wave < WM * WN) {
 #pragma unroll
-        for (int r = 1; r < RK; ++r)
+        for (int r = 1; r < RK * KH; ++r)
 #pragma unroll
           for (int v = 0; v < NV4; ++v)
             acc.c[v / NB][v % NB] += *reinterpret_cast<const AccV *>(red + ((((r - 1) * WM * WN + wave) * NV4 + v) * 64 + lane) * 4);
