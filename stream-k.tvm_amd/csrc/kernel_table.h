@@ -274,6 +274,9 @@ struct KernelInfo {
 // of A -- A requested one iteration ahead -- 16 x 8192 x 8192 took 13.2 us from HBM against 12.2, 11.6 / 10.7 with the
 // weights in the Infinity Cache; four waves per ring instead of two: 10.7 -> 10.2, the 64-row instance 31.7 -> 28.9 us
 // at 16 x 16384 x 16384, 37.7 -> 36.2 from HBM)
+// (an instance of 32 weight rows with 512 instead of 1024 K-values per iteration, eight waves and six slots of A
+// -- X(294, 2, 1, 4, 4, 6), weights issued before A -- was measured and is not built: 16 x 8192 x 8192 13.6 us from HBM
+// against 12.1, 12.6 / 10.2 with the weights in the Infinity Cache)
 // (an instance with eight rings, 128 weight rows and one wave per ring -- X(294, 8, 1, 1, 3, 3): half the bytes of A per
 // byte of weights -- was measured and is not built: 16 x 16384 x 16384 split in two over K 39.7 us against 39.4 for the
 // 64-row instance and 37.5 for the general kernel, 16 x 8192 x 8192 17.8 against 13.8)
