@@ -201,9 +201,9 @@ struct TileStreamQ4 : TileStreamPairs<1, 1, WN_, RK_, 3, false> {
           p[3] = __builtin_amdgcn_perm(v[3], v[1], 0x07060302u);
           fa[q] = __builtin_bit_cast(half8v, p);
         }
-        AccV sum[2] = {AccV{0, 0, 0, 0}, AccV{0, 0, 0, 0}};
+        AccV sum = AccV{0, 0, 0, 0};   // (one chain: the other waves of the SIMD cover the wait between dependent MFMAs)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) sum[q & 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(neg_offsets, fa[q], sum[q & 1], 0, 0, 0);
+        for (int q = 0; q < 4; ++q) sum = __builtin_amdgcn_mfma_f32_16x16x32_f16(neg_offsets, fa[q], sum, 0, 0, 0);
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           union {
@@ -215,10 +215,10 @@ struct TileStreamQ4 : TileStreamPairs<1, 1, WN_, RK_, 3, false> {
           raw.u[1] = and_or(w, qc.mask_hi, magic_hi);
           raw.u[2] = and_or(t8, qc.mask_lo, qc.magic);
           raw.u[3] = and_or(t8, qc.mask_hi, magic_hi);
-          sum[q & 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(raw.v, fa[q], sum[q & 1], 0, 0, 0);
+          sum = __builtin_amdgcn_mfma_f32_16x16x32_f16(raw.v, fa[q], sum, 0, 0, 0);
         }
 #pragma unroll
-        for (int r = 0; r < 4; ++r) part[0][r] = __builtin_fmaf(sum[0][r] + sum[1][r], (float)sc[r][ss], part[0][r]);
+        for (int r = 0; r < 4; ++r) part[0][r] = __builtin_fmaf(sum[r], (float)sc[r][ss], part[0][r]);
       }
       // the fragments are in registers before the next barrier hands the slots back to the loads
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
