@@ -197,7 +197,7 @@ __device__ __forceinline__ int sk_pid_of_iter(const DevPlan &p, int iter) {
 // Returns false if the poll limit ran out.
 // COHERENT = false: one device-scope acquire (L2 invalidate) by the polling wave before the
 // barrier, so that the ordinary loads that follow cannot hit stale lines.
-// WORD: lds_word is a word of LDS of the caller's through which the first wave's verdict reaches the others; without one
+// WORD: lds_word is a word of LDS of the caller's through which the first wave's result reaches the others; without one
 // the device library's block-wide AND does it, which reserves 256 bytes of LDS of its own.
 template <bool COHERENT, bool WORD = false>
 __device__ __forceinline__ bool wait_partials_ready(int *flags, int npeers, int spin_limit, int *lds_word = nullptr) {

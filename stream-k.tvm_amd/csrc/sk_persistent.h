@@ -192,10 +192,10 @@ __device__ __forceinline__ void run_persistent(const typename P::Args &a, const 
         // the sum of two terms does not depend on their order.
         if constexpr (has_halves<P>::value) {
           if (plan.halves == 2) {
-            // Four equal segments per tile, CTAs base .. base + 3.  Round 1: the pairs (0, 1) and (2, 3) exchange
+            // Four equal segments per tile, CTAs base .. base + 3.  First exchange: the pairs (0, 1) and (2, 3) swap
             // halves as above; CTAs 0 and 2 then hold the pair's sum of half 0, CTAs 1 and 3 that of half 1.
-            // Round 2: CTA 2 hands its half to CTA 0 and CTA 3 its half to CTA 1 (parked in the other half of
-            // their slots, which nobody reads in round 1; flags of their own, grid entries further on), and CTAs 0
+            // Second exchange: CTA 2 hands its half to CTA 0 and CTA 3 its half to CTA 1 (parked in the other half of
+            // their slots, which nobody reads in the first; flags of their own, grid entries further on), and CTAs 0
             // and 1 finish half of C each.  Every flag has one reader, who clears it; the order of the sums is
             // fixed.  Two half-tile exchanges in a row instead of one CTA adding three partial tiles.
             const int q = plan.by_full.div(k0), base = pid - q;
