@@ -258,12 +258,15 @@ struct KernelInfo {
 
 // the same with NB blocks of 16 weight rows per wave, AD slots of A and the unpadded rings (64 x 64 tiles: the 160 KB
 // of LDS exactly; 16 x 16 tiles with K split over the four waves: the same), and two waves sharing the K-steps of each
-// of those four (eight waves per CTA):  X(id, MB, WM, WN, RK, DEPTH, NB, AD, BF16)
+// of those four (eight waves per CTA); 96 x 32 tiles (three blocks of rows per wave, four slots of weights and two of
+// A: the 160 KB as well) for 65 to 96 rows where N gives every CU a tile:  X(id, MB, WM, WN, RK, DEPTH, NB, AD, BF16)
 #define SK_STREAM_BLOCKS_KERNELS(X)  \
   X(292, 2, 2, 2, 1, 3, 2, 2, false) \
   X(293, 2, 2, 2, 1, 3, 2, 2, true)  \
   X(296, 1, 1, 1, 4, 3, 1, 2, false) \
-  X(297, 1, 1, 1, 4, 3, 1, 2, true)
+  X(297, 1, 1, 1, 4, 3, 1, 2, true)  \
+  X(298, 3, 2, 2, 1, 4, 1, 2, false) \
+  X(299, 3, 2, 2, 1, 4, 1, 2, true)
 
 // Up to 16 rows of A, Q4 weights (row-major, scalar zero point) streaming through LDS in contiguous loads
 // (tile_stream_q4.h; dtype SK_Q4, variant 4):  X(id, WN, RK, KH, WD, AD)

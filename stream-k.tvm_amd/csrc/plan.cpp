@@ -66,6 +66,12 @@ static bool accepts_shape(const KernelInfo &k, int64_t M, int64_t K) {
          (k.family != FAMILY_TILE || k.variant != 7 || K % k.k_align == 0);
 }
 
+// 65 to 96 rows of fp16 / bfloat16 (NT) whose 96 x 32 tiles fill the device in one round: see pick_kernel
+static bool rows_65_to_96_stream(int64_t M, int64_t N, int dtype, int layout, int num_cus) {
+  return (dtype == SK_F16 || dtype == SK_BF16) && layout == SK_LAYOUT_NT && M > 64 && M <= 96 && cdiv(N, 32) <= num_cus &&
+         cdiv(N, 32) * 5 >= (int64_t)num_cus * 4;
+}
+
 static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype, int layout,
                                      const sk_config *cfg, int num_cus) {
   int n;
@@ -126,6 +132,14 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
           t[i].bk == bk && accepts_shape(t[i], M, K))
         return &t[i];
   }
+  // 65 to 96 rows of fp16 / bfloat16 where 96 x 32 tiles fill the device in one round (N = 8192 on 256 CUs): the
+  // streaming kernel with three blocks of rows per wave -- A is three times the bytes of the weights per CTA, but the
+  // weights still arrive in contiguous loads; 80 x 8192 x 8192 from HBM 38.5 us against 44.1 us on the tile kernels.
+  // Other widths lose to them (96 x 11008 x 4096: 38.8 / 32.2, 80 x 4096 x 11008: 44.7 / 37.9).
+  if (want_variant < 0 && rows_65_to_96_stream(M, N, dtype, layout, num_cus))
+    for (int i = 0; i < n; ++i)
+      if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].variant == 4 && t[i].bm == 96 && accepts_shape(t[i], M, K))
+        return &t[i];
   if ((M <= (one_byte ? 64 : 32) && layout == SK_LAYOUT_NT) || q4) {
     // M == 1 with Q4 weights: the matrix-vector kernel with four waves splitting K (data-parallel
     // over 16-row tiles), the fastest instance at LLM-sized N and K.  Weights from HBM: from K = 14336 on eight waves
@@ -408,6 +422,7 @@ extern "C" int sk_make_plan(int64_t M, int64_t N, int64_t K, int dtype, int layo
   // weight-streaming kernels take: the cost model chooses kernel and split
   sk_config modelled;
   if ((dtype == SK_F16 || dtype == SK_BF16 || dtype == SK_F8E4M3 || dtype == SK_F8E5M2 || dtype == SK_I8) && M > 64 &&
+      !rows_65_to_96_stream(M, N, dtype, layout, num_cus) &&
       (!cfg || (cfg->bm == 0 && cfg->bn == 0 && cfg->bk == 0 && cfg->reserved[0] == 0 &&
                 cfg->schedule == SK_SCHED_AUTO && cfg->grid == 0))) {
     int split = 1, model_sched = SK_SCHED_AUTO;

@@ -27,7 +27,8 @@ _TILES_F16 = [(256, 256, 64), (128, 128, 64), (128, 256, 64), (256, 128, 64), (6
 _SKINNY_F16 = [(16, 64, 128), (32, 64, 128), (64, 64, 128), (16, 16, 512), (16, 32, 256), (16, 16, 128),
                (16, 16, 1024), (16, 32, 512), (16, 16, 256), (16, 64, 256), (32, 64, 256), (64, 64, 256)]
 # fp16 / bfloat16 weights streamed through LDS in contiguous loads (variant 5 of these shapes)
-_STREAM_F16 = [(16, 16, 1024), (16, 32, 512), (16, 64, 256), (32, 32, 256), (32, 64, 256), (64, 32, 256), (64, 64, 256)]
+_STREAM_F16 = [(16, 16, 1024), (16, 32, 512), (16, 64, 256), (32, 32, 256), (32, 64, 256), (64, 32, 256), (64, 64, 256),
+               (96, 32, 256)]
 _SKINNY_F8 = [(16, 64, 256), (32, 64, 256), (16, 16, 1024), (16, 32, 512), (16, 32, 1024), (16, 64, 512), (32, 64, 512),
               (64, 64, 256), (64, 64, 512)]
 _SKINNY_Q4 = [(16, 64, 256), (32, 64, 256), (64, 64, 256), (16, 16, 1024), (16, 32, 512), (16, 16, 256),
@@ -85,7 +86,7 @@ def candidate_configs(M, N, K, dtype="float16", cus=None, reduce16=True):
             out.append(dict(base, schedule="dp"))
             for sched, fixup in (("sk2", "reduce"), ("basic", "reduce"), ("basic", "atomic")):
                 out.append(dict(base, schedule=sched, grid=cus, fixup=fixup))
-    if dtype in ("float16", "bfloat16") and M <= 64:
+    if dtype in ("float16", "bfloat16") and M <= 96:
         for (bm, bn, bk) in _STREAM_F16:
             if bm < M or (bm >= 2 * M and bm > 16):
                 continue

@@ -207,6 +207,8 @@ def test_untuned_plans_keep_cta_ranges_aligned(sk):
                                          (4, 4096, 4096, "float16", "stream_f16_mb1_nb1_wm1_wn1_rk4_d3", 256),
                                          (2, 11008, 4096, "float16", "stream_f16_mb1_wm1_wn4_rk1_d4", 172),
                                          (32, 11008, 4096, "float16", "stream_f16_mb2_wm1_wn4_rk1_d3", 172),
+                                         (80, 8192, 8192, "float16", "stream_f16_mb3_nb1_wm2_wn2_rk1_d4", 256),
+                                         (96, 7168, 4096, "bfloat16", "stream_bf16_mb3_nb1_wm2_wn2_rk1_d4", 224),
                                          (3, 4096, 4160, "float16", "stream_f16_mb1_nb1_wm1_wn1_rk4_d3", 256),
                                          (16, 8192, 8192, "q4", "stream_q4_wn2_rk2_kh4_d3", 256),
                                          (16, 28672, 8192, "q4", "skinny_q4_mb1_wn4_rk2_row1_0", 448),

@@ -70,7 +70,7 @@ SKINNY_CONFIGS = [
 STREAM_CONFIGS = [
     dict(bm=16, bn=64, bk=256, variant=5), dict(bm=32, bn=64, bk=256, variant=5), dict(bm=16, bn=32, bk=512, variant=5),
     dict(bm=64, bn=32, bk=256, variant=5), dict(bm=32, bn=32, bk=256, variant=5), dict(bm=64, bn=64, bk=256, variant=5),
-    dict(bm=16, bn=16, bk=1024, variant=5),
+    dict(bm=16, bn=16, bk=1024, variant=5), dict(bm=96, bn=32, bk=256, variant=5),
 ]
 
 
@@ -83,7 +83,7 @@ def test_fixture_ragged_f16(sk, oracle, golden_dir, cfg, sched, fixup, grid):
     small grids force tiles to be split over several CTAs."""
     g = np.load(os.path.join(golden_dir, "gemm_f16_nt_200x136x328.npz"))
     A, B, ref = g["A"], g["B"], g["C"]
-    if cfg["bm"] <= 64 and cfg["bn"] <= 64 and cfg["bk"] != 64:  # small-M kernels take M <= bm
+    if cfg["bm"] <= 96 and cfg["bn"] <= 64 and cfg["bk"] != 64:  # small-M kernels take M <= bm
         A, ref = A[:cfg["bm"] - 3], ref[:cfg["bm"] - 3]
     C = sk.streamk_fp16(_t(A), _t(B), schedule=sched, fixup=fixup, grid=grid, **cfg)
     sk.workspace_status()
@@ -1188,7 +1188,7 @@ def test_f16_few_rows_in_the_matrix_vector_form(sk, oracle):
 
 
 def test_f16_weights_streamed_through_lds(sk, oracle):
-    """Up to 64 rows of A on the kernels that stream the weights through LDS in contiguous loads (seven tile
+    """Up to 96 rows of A on the kernels that stream the weights through LDS in contiguous loads (eight tile
     shapes, fp16 and bfloat16): ragged M and N, K a multiple of 8 only and shorter than one iteration, strided A
     and W, all schedules and both fix-ups, bias and activation, an output with a row stride; exact on integer data
     (every tile adds its K-iterations up from a different start), within 2e-3 of the fp32 host product otherwise."""
@@ -1196,9 +1196,10 @@ def test_f16_weights_streamed_through_lds(sk, oracle):
     rng = np.random.default_rng(74)
     ran = 0
     shapes = {16: (16, 64, 256), 32: (32, 64, 256), 17: (16, 32, 512), 64: (64, 32, 256), 33: (32, 32, 256), 65: (64, 64, 256),
-              18: (16, 16, 1024)}
+              18: (16, 16, 1024), 96: (96, 32, 256)}
     for (M, N, K, pad) in [(16, 1000, 1160, 0), (9, 520, 392, 8), (1, 72, 8, 0), (13, 2048, 8192, 64), (5, 264, 28672, 0),
-                           (64, 4099, 4104, 0), (50, 328, 776, 8), (32, 200, 1032, 0), (27, 8192, 4096, 0)]:
+                           (64, 4099, 4104, 0), (50, 328, 776, 8), (32, 200, 1032, 0), (27, 8192, 4096, 0), (96, 1000, 1160, 8),
+                           (81, 8192, 2048, 0)]:
         A = (rng.random((M, K + pad), dtype=np.float32) * 2 - 1).astype(np.float16)
         W = (rng.random((N, K + pad), dtype=np.float32) * 2 - 1).astype(np.float16)
         Ai = rng.integers(-1, 2, (M, K + pad)).astype(np.float16)

@@ -14,8 +14,9 @@ pytestmark = pytest.mark.gpu
 ROWS = [1, 2, 3, 4, 5, 8, 9, 15, 16, 17, 31, 32, 33, 48, 63, 64, 65, 100, 200]
 COLS = [16, 48, 100, 250, 512, 1000, 1024, 2048, 2050, 4096, 5120, 8192, 11008]
 DEPTHS = [256, 512, 768, 1024, 1280, 2048, 4096, 4352, 5120, 8192]
-# tiles of the kernels that stream fp16 / bfloat16 weights through LDS (up to 64 rows of A)
-STREAM_TILES = [(16, 16, 1024), (16, 32, 512), (16, 64, 256), (32, 32, 256), (32, 64, 256), (64, 32, 256), (64, 64, 256)]
+# tiles of the kernels that stream fp16 / bfloat16 weights through LDS (up to 96 rows of A)
+STREAM_TILES = [(16, 16, 1024), (16, 32, 512), (16, 64, 256), (32, 32, 256), (32, 64, 256), (64, 32, 256), (64, 64, 256),
+                (96, 32, 256)]
 
 
 @pytest.fixture(scope="module")
@@ -61,7 +62,7 @@ def test_random_16_bit_shapes_plans_and_epilogues(sk, oracle, seed):
         C = cbuf[:, :N]
         bias = torch.from_numpy(rng.standard_normal(N, dtype=np.float32)).to(tdt).cuda() if rnd.random() < 0.4 else None
         act = rnd.choice([None, None, "relu", "silu", "gelu_tanh"])
-        cfg = _draw_config(rnd, M) if M <= 64 and rnd.random() < 0.6 else None
+        cfg = _draw_config(rnd, M) if M <= 96 and rnd.random() < 0.6 else None
         case = (seed, it, name, M, N, K, pad_a, pad_c, bias is not None, act, cfg)
         try:
             plan = sk.make_plan(M, N, K, name, "nt", cfg) if cfg else sk.make_plan(M, N, K, name, "nt", use_tuned=rnd.random() < 0.5)
