@@ -69,7 +69,7 @@ static bool accepts_shape(const KernelInfo &k, int64_t M, int64_t K) {
 // 65 to 96 rows of fp16 / bfloat16 (NT) whose 96 x 32 tiles fill the device in one round: see pick_kernel
 static bool rows_65_to_96_stream(int64_t M, int64_t N, int dtype, int layout, int num_cus) {
   return (dtype == SK_F16 || dtype == SK_BF16) && layout == SK_LAYOUT_NT && M > 64 && M <= 96 && cdiv(N, 32) <= num_cus &&
-         cdiv(N, 32) * 5 >= (int64_t)num_cus * 4;
+         cdiv(N, 32) * 5 >= (int64_t)num_cus * 3;
 }
 
 static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype, int layout,
@@ -135,7 +135,8 @@ static const KernelInfo *pick_kernel(int64_t M, int64_t N, int64_t K, int dtype,
   // 65 to 96 rows of fp16 / bfloat16 where 96 x 32 tiles fill the device in one round (N = 8192 on 256 CUs): the
   // streaming kernel with three blocks of rows per wave -- A is three times the bytes of the weights per CTA, but the
   // weights still arrive in contiguous loads; 80 x 8192 x 8192 from HBM 38.5 us against 44.1 us on the tile kernels.
-  // Other widths lose to them (96 x 11008 x 4096: 38.8 / 32.2, 80 x 4096 x 11008: 44.7 / 37.9).
+  // From three fifths of the CUs on (80 x 6144 x 4096: 19.6 / 27.1, 80 x 5120 x 5120: 24.0 / 33.5); other widths lose
+  // to the tile kernels (96 x 11008 x 4096: 38.8 / 32.2, 80 x 4096 x 11008: 44.7 / 37.9, 80 x 16384 x 8192: 74.7 / 67.7).
   if (want_variant < 0 && rows_65_to_96_stream(M, N, dtype, layout, num_cus))
     for (int i = 0; i < n; ++i)
       if (t[i].family == FAMILY_SKINNY && t[i].dtype == dtype && t[i].variant == 4 && t[i].bm == 96 && accepts_shape(t[i], M, K))
